@@ -1,0 +1,75 @@
+"""Build libboat_amd.so for gfx950: HIP kernels (hipcc) + the C host side (gcc), one shared library.
+
+    python -m boat_amd.build            # compile everything into boat_amd/lib/libboat_amd.so
+
+hipcc cross-compiles for gfx950 without a GPU, so this runs anywhere ROCm is installed.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+CSRC = ROOT / "boat_amd" / "csrc"
+OBJ = ROOT / "boat_amd" / "lib" / "obj"
+LIB = ROOT / "boat_amd" / "lib" / "libboat_amd.so"
+ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+HIPCC = str(ROCM / "bin" / "hipcc")
+
+HIP_SOURCES = sorted((CSRC / "hip").glob("*.hip"))
+C_SOURCES = sorted((CSRC / "host").glob("*.c"))
+
+# -ffp-contract=off: a*b+c stays two roundings, like the reference's scalar C loops.
+# packed-fp32 ops are switched off for every device compile.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{ROOT / 'include'}", f"-I{CSRC / 'hip'}",
+]
+C_FLAGS = [
+    "-O2", "-std=c11", "-fPIC", "-Wall", "-Wextra", "-fvisibility=hidden", "-D_GNU_SOURCE",
+    f"-I{ROOT / 'include'}", f"-I{CSRC / 'host'}",
+]
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{proc.stdout}\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+
+
+def _compile_hip(src: Path) -> Path:
+    out = OBJ / (src.stem + ".o")
+    _run([HIPCC, *HIP_FLAGS, "-c", str(src), "-o", str(out)])
+    return out
+
+
+def _compile_c(src: Path) -> Path:
+    out = OBJ / (src.stem + ".o")
+    _run(["gcc", *C_FLAGS, "-c", str(src), "-o", str(out)])
+    return out
+
+
+def build_all(jobs: int = 8, verbose: bool = True) -> Path:
+    """Compile every source and link boat_amd/lib/libboat_amd.so; returns its path."""
+    OBJ.mkdir(parents=True, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        hip_objs = list(pool.map(_compile_hip, HIP_SOURCES))
+        c_objs = list(pool.map(_compile_c, C_SOURCES))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB),
+          *map(str, hip_objs), *map(str, c_objs), "-lm", f"-Wl,-rpath,{ROCM / 'lib'}"])
+    if verbose:
+        print(f"built {LIB} ({LIB.stat().st_size // 1024} KiB) from {len(hip_objs)} HIP + {len(c_objs)} C sources")
+    return LIB
+
+
+if __name__ == "__main__":
+    build_all()

@@ -1,0 +1,245 @@
+"""ctypes binding of Boat's C API (the subset on the training hot path).
+
+`BoatAPI(path)` loads any shared library that exports Boat's symbols with Boat's
+signatures -- libboat_amd.so (the default, GPU) or a build of the reference itself
+-- so the same test code can drive both and compare results.
+
+The binding is deliberately thin: tensors, variables, layers and optimizers are
+opaque pointers exactly as in the C headers; only numpy <-> tensor copies are added.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+import numpy as np
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libboat_amd.so"
+
+# include/boat/tensor.h:22-55
+DTYPE_FLOAT64, DTYPE_FLOAT32 = 0, 1
+DTYPE_INT64, DTYPE_INT32, DTYPE_UINT8 = 5, 6, 7
+DEVICE_CPU, DEVICE_HIP = 0, 1
+
+_NP = {DTYPE_FLOAT64: np.float64, DTYPE_FLOAT32: np.float32, DTYPE_INT64: np.int64,
+       DTYPE_INT32: np.int32, DTYPE_UINT8: np.uint8}
+_DT = {np.dtype(v): k for k, v in _NP.items()}
+
+P = C.c_void_p
+
+
+class AttentionConfig(C.Structure):  # include/boat/layers/attention.h:21-30
+    _fields_ = [("hidden_size", C.c_size_t), ("num_heads", C.c_size_t), ("head_size", C.c_size_t),
+                ("dropout_prob", C.c_float), ("causal_mask", C.c_bool), ("use_bias", C.c_bool),
+                ("use_rotary", C.c_bool), ("rotary_theta", C.c_float)]
+
+
+class LayerNormConfig(C.Structure):  # include/boat/layers/norm.h:21-26
+    _fields_ = [("normalized_shape", C.c_size_t), ("eps", C.c_float),
+                ("elementwise_affine", C.c_bool), ("use_bias", C.c_bool)]
+
+
+_SIGS = {
+    # tensor
+    "boat_tensor_create": (P, [C.POINTER(C.c_int64), C.c_size_t, C.c_int, C.c_int]),
+    "boat_tensor_create_like": (P, [P]),
+    "boat_tensor_free": (None, [P]),
+    "boat_tensor_ref": (None, [P]),
+    "boat_tensor_unref": (None, [P]),
+    "boat_tensor_shape": (C.POINTER(C.c_int64), [P]),
+    "boat_tensor_ndim": (C.c_size_t, [P]),
+    "boat_tensor_dtype": (C.c_int, [P]),
+    "boat_tensor_device": (C.c_int, [P]),
+    "boat_tensor_nbytes": (C.c_size_t, [P]),
+    "boat_tensor_nelements": (C.c_size_t, [P]),
+    "boat_tensor_data": (P, [P]),
+    "boat_tensor_const_data": (P, [P]),
+    "boat_tensor_reshape": (P, [P, C.POINTER(C.c_int64), C.c_size_t]),
+    # ops
+    "boat_add": (P, [P, P]), "boat_sub": (P, [P, P]), "boat_mul": (P, [P, P]), "boat_div": (P, [P, P]),
+    "boat_add_": (None, [P, P]),
+    "boat_mul_scalar": (P, [P, C.c_double]),
+    "boat_matmul": (P, [P, P]),
+    "boat_transpose": (P, [P, C.c_int, C.c_int]),
+    "boat_relu": (P, [P]),
+    "boat_softmax": (P, [P, C.c_int]), "boat_log_softmax": (P, [P, C.c_int]),
+    "boat_sum": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_bool]),
+    # autodiff
+    "boat_variable_create": (P, [P, C.c_bool]),
+    "boat_variable_free": (None, [P]),
+    "boat_variable_data": (P, [P]),
+    "boat_variable_grad": (P, [P]),
+    "boat_variable_requires_grad": (C.c_bool, [P]),
+    "boat_variable_zero_grad": (None, [P]),
+    "boat_variable_backward": (None, [P, P]),
+    "boat_variable_backward_full": (None, [P]),
+    "boat_var_add": (P, [P, P]), "boat_var_sub": (P, [P, P]), "boat_var_mul": (P, [P, P]), "boat_var_div": (P, [P, P]),
+    "boat_var_matmul": (P, [P, P]), "boat_var_dot": (P, [P, P]),
+    "boat_var_relu": (P, [P]), "boat_var_sigmoid": (P, [P]), "boat_var_tanh": (P, [P]),
+    "boat_var_softmax": (P, [P, C.c_int]), "boat_var_log_softmax": (P, [P, C.c_int]),
+    "boat_var_sum": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_bool]),
+    "boat_var_dense": (P, [P, P]),
+    "boat_var_attention": (P, [P, P, P, P, P]),
+    "boat_autodiff_clear_computation_graph": (None, []),
+    # dense
+    "boat_dense_layer_create": (P, [C.c_size_t, C.c_size_t, C.c_bool]),
+    "boat_dense_layer_free": (None, [P]),
+    "boat_dense_layer_forward": (P, [P, P]),
+    "boat_dense_layer_backward": (P, [P, P]),
+    "boat_dense_layer_update": (None, [P, C.c_float]),
+    "boat_dense_layer_get_weight": (P, [P]), "boat_dense_layer_get_bias": (P, [P]),
+    "boat_dense_layer_get_grad_weight": (P, [P]), "boat_dense_layer_get_grad_bias": (P, [P]),
+    # relu / softmax hooks
+    "boat_relu_layer_create": (P, []), "boat_relu_layer_free": (None, [P]),
+    "boat_relu_layer_forward": (P, [P, P]), "boat_relu_layer_backward": (P, [P, P]),
+    "boat_softmax_layer_create": (P, [C.c_int]), "boat_softmax_layer_free": (None, [P]),
+    "boat_softmax_layer_forward": (P, [P, P]), "boat_softmax_layer_backward": (P, [P, P]),
+    # layernorm
+    "boat_layernorm_create": (P, [C.POINTER(LayerNormConfig)]),
+    "boat_layernorm_free": (None, [P]),
+    "boat_layernorm_forward": (P, [P, P]),
+    "boat_layernorm_backward": (P, [P, P]),
+    "boat_layernorm_set_weight": (None, [P, P]), "boat_layernorm_set_bias": (None, [P, P]),
+    "boat_norm_layer_create": (P, [C.c_size_t, C.c_float, C.c_bool]),
+    "boat_norm_layer_free": (None, [P]),
+    "boat_norm_layer_forward": (P, [P, P]), "boat_norm_layer_backward": (P, [P, P]),
+    # attention
+    "boat_attention_create": (P, [C.POINTER(AttentionConfig)]),
+    "boat_attention_free": (None, [P]),
+    "boat_attention_forward": (P, [P, P, P, P, P]),
+    "boat_attention_backward": (C.c_bool, [P, P, C.POINTER(P), C.POINTER(P), C.POINTER(P)]),
+    "boat_attention_update": (None, [P, C.c_float]),
+    # optimizer
+    "boat_adam_optimizer_create": (P, [C.c_float, C.c_float, C.c_float, C.c_float]),
+    "boat_optimizer_add_parameter": (None, [P, P, P]),
+    "boat_optimizer_step": (None, [P]),
+    "boat_optimizer_zero_grad": (None, [P]),
+    "boat_optimizer_free": (None, [P]),
+    "boat_optimizer_get_learning_rate": (C.c_float, [P]),
+    "boat_optimizer_set_learning_rate": (None, [P, C.c_float]),
+    # model
+    "boat_model_create": (P, []), "boat_model_free": (None, [P]),
+    "boat_model_add_layer": (None, [P, P]), "boat_model_layer_count": (C.c_size_t, [P]),
+    "boat_model_forward": (P, [P, P]), "boat_model_backward": (P, [P, P]),
+    "boat_model_update": (None, [P, C.c_float]),
+}
+for _n in "qkvo":
+    for _k in ("weight", "bias", "grad_weight", "grad_bias"):
+        _SIGS[f"boat_attention_get_{_k}_{_n}"] = (P, [P])
+
+# symbols only libboat_amd.so has
+_EXT_SIGS = {
+    "boat_gelu": (P, [P]),
+    "boat_tensor_to_device": (P, [P, C.c_int]),
+    "boat_tensor_clone": (P, [P]),
+    "boat_hip_synchronize": (None, []),
+    "boat_hip_variable_ensure_grad": (P, [P]),
+    "boat_hip_var_gelu": (P, [P]),
+    "boat_hip_var_layernorm": (P, [P, P]),
+    "boat_hip_layernorm_get_weight": (P, [P]), "boat_hip_layernorm_get_bias": (P, [P]),
+    "boat_hip_layernorm_get_grad_weight": (P, [P]), "boat_hip_layernorm_get_grad_bias": (P, [P]),
+    "boat_hip_softmax_cross_entropy": (P, [P, P, C.POINTER(P)]),
+    "boat_hip_mse_loss": (P, [P, P, C.POINTER(P)]),
+    "boat_hip_layer_from_dense": (P, [P]), "boat_hip_layer_from_norm": (P, [P]),
+    "boat_hip_layer_relu": (P, []), "boat_hip_layer_gelu": (P, []),
+    "boat_hip_optimizer_add_dense": (None, [P, P]),
+    "boat_hip_optimizer_add_attention": (None, [P, P]),
+    "boat_hip_optimizer_add_layernorm": (None, [P, P]),
+    "boat_layernorm_update": (None, [P, C.c_float]),
+    "boat_get_last_error_message": (C.c_char_p, []),
+    "boat_memory_get_stats": (None, []),
+}
+
+
+class BoatAPI:
+    """Loaded Boat library with typed entry points as attributes (api.boat_tensor_create(...))."""
+
+    def __init__(self, path: str | Path | None = None):
+        path = Path(path) if path is not None else LIB_PATH
+        if not path.exists():
+            raise FileNotFoundError(
+                f"{path} not found: build it first (python -m boat_amd.build); there is no host fallback")
+        self.path = path
+        self.lib = C.CDLL(str(path), mode=C.RTLD_LOCAL)
+        self.is_amd = hasattr(self.lib, "boat_hip_synchronize")
+        for name, (res, args) in _SIGS.items():
+            self._bind(name, res, args)
+        if self.is_amd:
+            for name, (res, args) in _EXT_SIGS.items():
+                self._bind(name, res, args)
+
+    def _bind(self, name, res, args):
+        fn = getattr(self.lib, name)
+        fn.restype = res
+        fn.argtypes = args
+        setattr(self, name, fn)
+
+    # ---- numpy helpers ----
+    def tensor(self, array, device: int = DEVICE_CPU):
+        """New tensor holding a copy of `array` (written through boat_tensor_data, as Boat's tests do)."""
+        a = np.ascontiguousarray(array)
+        shape = (C.c_int64 * max(a.ndim, 1))(*a.shape)
+        t = self.boat_tensor_create(shape, a.ndim, _DT[a.dtype], DEVICE_CPU)
+        if not t:
+            raise RuntimeError("boat_tensor_create failed")
+        if a.size:
+            C.memmove(self.boat_tensor_data(t), a.ctypes.data, a.nbytes)
+        if device != DEVICE_CPU:
+            d = self.boat_tensor_to_device(t, device)
+            self.boat_tensor_free(t)
+            return d
+        return t
+
+    def zeros(self, shape, dtype=DTYPE_FLOAT32, device: int = DEVICE_CPU):
+        shape = tuple(shape)
+        arr = (C.c_int64 * max(len(shape), 1))(*shape)
+        t = self.boat_tensor_create(arr, len(shape), dtype, device)
+        if not t:
+            raise RuntimeError("boat_tensor_create failed")
+        return t
+
+    def shape(self, t):
+        n = self.boat_tensor_ndim(t)
+        s = self.boat_tensor_shape(t)
+        return tuple(int(s[i]) for i in range(n))
+
+    def numpy(self, t):
+        """Copy of the tensor's current contents (downloads from the GPU when needed)."""
+        if not t:
+            raise ValueError("NULL tensor")
+        if self.is_amd and self.boat_tensor_device(t) == DEVICE_HIP:
+            h = self.boat_tensor_to_device(t, DEVICE_CPU)
+            try:
+                return self.numpy(h)
+            finally:
+                self.boat_tensor_free(h)
+        shape = self.shape(t)
+        dt = _NP[self.boat_tensor_dtype(t)]
+        n = self.boat_tensor_nelements(t)
+        out = np.empty(n, dtype=dt)
+        if n:
+            C.memmove(out.ctypes.data, self.boat_tensor_const_data(t), out.nbytes)
+        return out.reshape(shape)
+
+    def write(self, t, array):
+        """Overwrite a tensor in place through its data pointer (how Boat's tests inject weights)."""
+        a = np.ascontiguousarray(array, dtype=_NP[self.boat_tensor_dtype(t)])
+        if a.size != self.boat_tensor_nelements(t):
+            raise ValueError("size mismatch")
+        if a.size:
+            C.memmove(self.boat_tensor_data(t), a.ctypes.data, a.nbytes)
+
+    def sync(self):
+        if self.is_amd:
+            self.boat_hip_synchronize()
+
+
+_default: BoatAPI | None = None
+
+
+def default_api() -> BoatAPI:
+    """The GPU library, loaded once; raises if it has not been built."""
+    global _default
+    if _default is None:
+        _default = BoatAPI()
+    return _default

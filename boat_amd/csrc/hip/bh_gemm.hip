@@ -1,0 +1,488 @@
+// bh_gemm.hip - fp32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// Replaces boat_matmul (src/ops/linear.c:12-170) together with the materialised
+// boat_transpose calls (src/ops/linear.c:238-406) that the reference's backward passes
+// wrap around it:
+//   dense forward   Y  = X.W (+ b)      src/layers/dense.c:150-185
+//   dense backward  dX = dY.W^T         src/layers/dense.c:219-228
+//                   dW += X^T.dY        src/layers/dense.c:230-261
+//   attention projections and their backward, src/layers/attention.c:247-308, 1186-1285
+// Transposed operands are read in place: an operand is either "k-contiguous" (the
+// contraction index is the fast index in memory) or "row-contiguous" (the output index is
+// the fast one); each has its own LDS layout and fragment read, so no transpose is ever
+// written to memory.
+//
+// Tiling (wave64, gfx950):
+//   macro tile BM x BN per workgroup, k-tile BK=16, LDS double buffered, next k-tile
+//   prefetched into registers while the current one feeds the MFMAs (one barrier per k-tile)
+//   each wavefront owns a (32*TM) x (32*TN) block = TM*TN accumulators of 16 VGPRs
+//   A-fragment for MFMA step s comes from one ds_read_b128 / ds_read_b64:
+//     k-contiguous operand   [rows][BK+4] : lane (r, half) reads k = kb+4*half .. +3 of row r;
+//                                            element s feeds step s (any k order is a valid sum)
+//     row-contiguous operand [BK][rows+4] : lane (r, half) reads rows T*r .. T*r+T-1 of k-row
+//                                            kb+4*half+s; element t feeds tile t, i.e. tile t
+//                                            owns the interleaved rows {base + T*i + t}
+//   workgroup -> tile map is XCD-aware: consecutive tiles of a group land on the same XCD
+//   (same L2), and tiles are walked in groups of 8 tile-rows.
+// Small or unaligned problems take a bounds-checked LDS-tiled fallback kernel; problems with a
+// small output and a long contraction (weight gradients) are split along K into a workspace and
+// folded by a second kernel (deterministic, no atomics).
+#include "bh_common.h"
+
+namespace bh {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kBK = 16;
+constexpr int kPad = 4;
+
+template <int T> struct FragT;             // T consecutive floats from LDS
+template <> struct FragT<1> { float v[1]; __device__ __forceinline__ void load(const float* p) { v[0] = p[0]; } };
+template <> struct FragT<2> { float v[2]; __device__ __forceinline__ void load(const float* p) { float2 t = *reinterpret_cast<const float2*>(p); v[0] = t.x; v[1] = t.y; } };
+template <> struct FragT<4> { float v[4]; __device__ __forceinline__ void load(const float* p) { float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; } };
+
+template <int BM_, int BN_, int WGM_, int WGN_>
+struct GemmCfg {
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
+    static constexpr int NT = WGM * WGN * 64;
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
+    static constexpr int TM = WM / 32, TN = WN / 32;
+};
+
+// LDS floats for one operand tile of R rows
+template <bool KC, int R> struct TileShape {
+    static constexpr int ld = KC ? (kBK + kPad) : (R + kPad);
+    static constexpr int floats = KC ? R * ld : kBK * ld;
+};
+
+struct GemmArgs {
+    const float* a; const float* b; float* c; const float* bias;
+    int64_t m, n, k;
+    int64_t lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;   // per batch
+    int accumulate;
+    int k_splits;        // >1: write partials to c (workspace [split][batch][m][n], ldc == n)
+    int64_t k_per_split; // multiple of kBK
+    int tiles_m, tiles_n;
+};
+
+// Global -> registers for one operand tile.  KC: tile is [R rows][kBK], row r at base + r*ld.
+// !KC: tile is [kBK k-rows][R], k-row kk at base + kk*ld.
+template <bool KC, int R, int NT>
+struct TileLoader {
+    static constexpr int F4 = R * kBK / 4;
+    static constexpr int PER = (F4 + NT - 1) / NT;
+    float4 reg[PER];
+
+    __device__ __forceinline__ void load(const float* __restrict__ base, int64_t ld, int64_t row0, int64_t row_lim,
+                                         int64_t k0, int64_t k_lim, int tid) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * NT;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (F4 % NT == 0 || idx < F4) {
+                if (KC) {
+                    const int r = idx / (kBK / 4), kq = idx % (kBK / 4);
+                    const int64_t gr = row0 + r, gk = k0 + kq * 4;
+                    if (gr < row_lim && gk < k_lim) v = *reinterpret_cast<const float4*>(base + gr * ld + gk);
+                } else {
+                    const int kk = idx / (R / 4), c4 = idx % (R / 4);
+                    const int64_t gk = k0 + kk, gr = row0 + c4 * 4;
+                    if (gk < k_lim && gr < row_lim) v = *reinterpret_cast<const float4*>(base + gk * ld + gr);
+                }
+            }
+            reg[i] = v;
+        }
+    }
+    __device__ __forceinline__ void store(float* lds, int tid) const {
+        constexpr int ld = TileShape<KC, R>::ld;
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * NT;
+            if (F4 % NT == 0 || idx < F4) {
+                if (KC) {
+                    const int r = idx / (kBK / 4), kq = idx % (kBK / 4);
+                    *reinterpret_cast<float4*>(lds + r * ld + kq * 4) = reg[i];
+                } else {
+                    const int kk = idx / (R / 4), c4 = idx % (R / 4);
+                    *reinterpret_cast<float4*>(lds + kk * ld + c4 * 4) = reg[i];
+                }
+            }
+        }
+    }
+};
+
+// Fragments of one operand for one k-group (8 k values = 4 MFMA steps), T tiles.
+template <bool KC, int R, int T>
+struct Frags {
+    float v[4][T];   // [step][tile]
+    __device__ __forceinline__ void load(const float* lds, int wave_off, int kb, int r, int half) {
+        constexpr int ld = TileShape<KC, R>::ld;
+        if (KC) {
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                float4 q = *reinterpret_cast<const float4*>(lds + (wave_off + t * 32 + r) * ld + kb + 4 * half);
+                v[0][t] = q.x; v[1][t] = q.y; v[2][t] = q.z; v[3][t] = q.w;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                FragT<T> f;
+                f.load(lds + (kb + 4 * half + s) * ld + wave_off + T * r);
+#pragma unroll
+                for (int t = 0; t < T; t++) v[s][t] = f.v[t];
+            }
+        }
+    }
+};
+
+template <typename Cfg, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
+    constexpr int A_FLOATS = TileShape<A_KC, BM>::floats, B_FLOATS = TileShape<B_KC, BN>::floats;
+    extern __shared__ __align__(16) float smem[];
+    constexpr int STAGE = A_FLOATS + B_FLOATS;   // stage `cur` holds A at smem+cur*STAGE, B right after it
+
+    // ---- workgroup -> (tile_m, tile_n): XCD-aware, grouped ----
+    const int total = g.tiles_m * g.tiles_n;
+    int pid = blockIdx.x;
+    if (total % kNumXcd == 0) pid = (pid % kNumXcd) * (total / kNumXcd) + pid / kNumXcd;
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * g.tiles_n;
+    const int group_id = pid / per_group;
+    const int first_m = group_id * GROUP;
+    const int gsz = min(g.tiles_m - first_m, GROUP);
+    const int tile_m = first_m + (pid % per_group) % gsz;
+    const int tile_n = (pid % per_group) / gsz;
+
+    const int batch = blockIdx.y;
+    const int split = blockIdx.z;
+    const int64_t k_begin = (int64_t)split * g.k_per_split;
+    int64_t k_end = g.k_splits > 1 ? k_begin + g.k_per_split : g.k;
+    if (k_end > g.k) k_end = g.k;
+
+    const float* A = g.a + (int64_t)batch * g.stride_a;
+    const float* B = g.b + (int64_t)batch * g.stride_b;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave / Cfg::WGN, wn = wave % Cfg::WGN;
+    const int r = lane & 31, half = lane >> 5;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    TileLoader<A_KC, BM, NT> la;
+    TileLoader<B_KC, BN, NT> lb;
+
+    const int64_t kt_count = (k_end - k_begin + kBK - 1) / kBK;
+    if (kt_count > 0) {
+        la.load(A, g.lda, m0, g.m, k_begin, k_end, tid);
+        lb.load(B, g.ldb, n0, g.n, k_begin, k_end, tid);
+        la.store(smem, tid);
+        lb.store(smem + A_FLOATS, tid);
+    }
+    __syncthreads();
+
+    int cur = 0;
+    for (int64_t kt = 0; kt < kt_count; kt++) {
+        const bool more = kt + 1 < kt_count;
+        if (more) {
+            const int64_t k0 = k_begin + (kt + 1) * kBK;
+            la.load(A, g.lda, m0, g.m, k0, k_end, tid);
+            lb.load(B, g.ldb, n0, g.n, k0, k_end, tid);
+        }
+        const float* sa = smem + cur * STAGE;
+        const float* sb = sa + A_FLOATS;
+#pragma unroll
+        for (int kb = 0; kb < kBK; kb += 8) {
+            Frags<A_KC, BM, TM> fa;
+            Frags<B_KC, BN, TN> fb;
+            fa.load(sa, wm * Cfg::WM, kb, r, half);
+            fb.load(sb, wn * Cfg::WN, kb, r, half);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            la.store(smem + (cur ^ 1) * STAGE, tid);
+            lb.store(smem + (cur ^ 1) * STAGE + A_FLOATS, tid);
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // ---- epilogue ----
+    float* C = g.c + (int64_t)batch * g.stride_c;
+    if (g.k_splits > 1) C += (int64_t)split * gridDim.y * g.stride_c;
+    const bool add_c = g.accumulate && g.k_splits <= 1;
+    const float* bias = g.k_splits <= 1 ? g.bias : nullptr;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int ri = (e >> 2) * 8 + half * 4 + (e & 3);    // row inside the 32x32 tile
+            const int64_t row = m0 + wm * Cfg::WM + (A_KC ? i * 32 + ri : TM * ri + i);
+            if (row >= g.m) continue;
+            float* crow = C + row * g.ldc;
+            if (B_KC) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int64_t col = n0 + wn * Cfg::WN + j * 32 + r;
+                    if (col < g.n) {
+                        float v = acc[i][j][e];
+                        if (bias) v += bias[col];
+                        if (add_c) v += crow[col];
+                        crow[col] = v;
+                    }
+                }
+            } else {
+                const int64_t col0 = n0 + wn * Cfg::WN + TN * r;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int64_t col = col0 + j;
+                    if (col < g.n) {
+                        float v = acc[i][j][e];
+                        if (bias) v += bias[col];
+                        if (add_c) v += crow[col];
+                        crow[col] = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- fold split-K partials: c (+)= sum_s ws[s] (+ bias) ----
+__global__ __launch_bounds__(256) void splitk_fold_kernel(const float* __restrict__ ws, float* __restrict__ c,
+                                                          const float* __restrict__ bias, int64_t m, int64_t n, int64_t ldc,
+                                                          int splits, int64_t batch_count, int64_t stride_c, int accumulate) {
+    const int64_t per = m * n;
+    const int64_t total = per * batch_count;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t bt = i / per, rem = i % per, row = rem / n, col = rem % n;
+        float acc = 0.f;
+        for (int s = 0; s < splits; s++) acc += ws[((int64_t)s * batch_count + bt) * per + rem];
+        float* dst = c + bt * stride_c + row * ldc + col;
+        if (bias) acc += bias[col];
+        *dst = accumulate ? *dst + acc : acc;
+    }
+}
+
+// ---- fallback: bounds-checked 32x32 LDS tiles, any shape / alignment ----
+__global__ __launch_bounds__(256) void gemm_fallback_kernel(GemmArgs g, int trans_a, int trans_b) {
+    __shared__ float ta[32][33];
+    __shared__ float tb[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+    const int64_t m0 = (int64_t)blockIdx.y * 32, n0 = (int64_t)blockIdx.x * 32;
+    const float* A = g.a + (int64_t)blockIdx.z * g.stride_a;
+    const float* B = g.b + (int64_t)blockIdx.z * g.stride_b;
+    float* C = g.c + (int64_t)blockIdx.z * g.stride_c;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t k0 = 0; k0 < g.k; k0 += 32) {
+        for (int p = 0; p < 4; p++) {
+            const int rr = ty + p * 8;
+            // ta[rr][tx] = A(m0+rr, k0+tx) ; tb[rr][tx] = B(k0+rr, n0+tx)
+            const int64_t am = m0 + rr, ak = k0 + tx;
+            ta[rr][tx] = (am < g.m && ak < g.k) ? (trans_a ? A[ak * g.lda + am] : A[am * g.lda + ak]) : 0.f;
+            const int64_t bk = k0 + rr, bn = n0 + tx;
+            tb[rr][tx] = (bk < g.k && bn < g.n) ? (trans_b ? B[bn * g.ldb + bk] : B[bk * g.ldb + bn]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int kk = 0; kk < 32; kk++) {
+            const float bv = tb[kk][tx];
+#pragma unroll
+            for (int p = 0; p < 4; p++) acc[p] += ta[ty + p * 8][kk] * bv;
+        }
+        __syncthreads();
+    }
+    for (int p = 0; p < 4; p++) {
+        const int64_t row = m0 + ty + p * 8, col = n0 + tx;
+        if (row < g.m && col < g.n) {
+            float v = acc[p];
+            if (g.bias) v += g.bias[col];
+            if (g.accumulate) v += C[row * g.ldc + col];
+            C[row * g.ldc + col] = v;
+        }
+    }
+}
+
+// ---- out-of-place transpose of the last two dims (for boat_transpose callers) ----
+__global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict__ a, float* __restrict__ out, int64_t rows,
+                                                        int64_t cols) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const float* ab = a + (int64_t)blockIdx.z * rows * cols;
+    float* ob = out + (int64_t)blockIdx.z * rows * cols;
+    const int64_t r0 = (int64_t)blockIdx.y * 32, c0 = (int64_t)blockIdx.x * 32;
+    for (int p = 0; p < 4; p++) {
+        const int64_t rr = r0 + ty + p * 8, cc = c0 + tx;
+        if (rr < rows && cc < cols) tile[ty + p * 8][tx] = ab[rr * cols + cc];
+    }
+    __syncthreads();
+    for (int p = 0; p < 4; p++) {
+        const int64_t cc = c0 + ty + p * 8, rr = r0 + tx;
+        if (rr < rows && cc < cols) ob[cc * rows + rr] = tile[tx][ty + p * 8];
+    }
+}
+
+using CfgBig = GemmCfg<256, 256, 2, 4>;   // 8 waves, 128x64 per wave
+using CfgMid = GemmCfg<128, 128, 2, 2>;   // 4 waves, 64x64 per wave
+
+template <typename Cfg, bool A_KC, bool B_KC>
+static int launch_mfma(const GemmArgs& g, int64_t batch) {
+    constexpr size_t lds = 2 * sizeof(float) * (TileShape<A_KC, Cfg::BM>::floats + TileShape<B_KC, Cfg::BN>::floats);
+    static bool attr_set = false;
+    if (!attr_set) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)(g.k_splits > 1 ? g.k_splits : 1));
+    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC>), grid, dim3(Cfg::NT), lds, stream(), g);
+    return BH_LAUNCH_CHECK("gemm_mfma_kernel");
+}
+
+template <typename Cfg>
+static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc) {
+    if (a_kc && b_kc) return launch_mfma<Cfg, true, true>(g, batch);
+    if (a_kc && !b_kc) return launch_mfma<Cfg, true, false>(g, batch);
+    if (!a_kc && b_kc) return launch_mfma<Cfg, false, true>(g, batch);
+    return launch_mfma<Cfg, false, false>(g, batch);
+}
+
+static int g_force_cfg = -1;   // test hook: 0 = fallback, 1 = mid, 2 = big, -1 = heuristic
+
+}  // namespace bh
+
+using namespace bh;
+
+extern "C" {
+
+// test/benchmark hook: pin the kernel choice (-1 restores the heuristic)
+int bh_gemm_force_config(int cfg) {
+    g_force_cfg = cfg;
+    return BH_OK;
+}
+
+int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const float* a, int64_t lda, const float* b,
+            int64_t ldb, float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && batch >= 0, "negative dimension");
+    if (m == 0 || n == 0 || batch == 0) return BH_OK;
+    BH_CHECK_ARG(a && b && c, "null pointer");
+    BH_CHECK_ARG(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "leading dimension too small");
+    BH_CHECK_ARG(batch <= 65535, "batch too large");
+
+    GemmArgs g;
+    g.a = a; g.b = b; g.c = c; g.bias = bias;
+    g.m = m; g.n = n; g.k = k;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+    g.stride_a = (trans_a ? k : m) * lda;
+    g.stride_b = (trans_b ? n : k) * ldb;
+    g.stride_c = m * ldc;
+    g.accumulate = accumulate;
+    g.k_splits = 1;
+    g.k_per_split = k;
+
+    const bool a_kc = !trans_a, b_kc = trans_b != 0;
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    // float4 global loads need: 16 B aligned bases, leading dimensions and the contiguous extent % 4
+    bool vec_ok = al16(a) && al16(b) && (lda % 4 == 0) && (ldb % 4 == 0) && k > 0;
+    vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
+    int cfg;   // 0 fallback, 1 mid, 2 big
+    if (!vec_ok || m * n < 64 * 64) {
+        cfg = 0;
+    } else {
+        const int64_t big_tiles = ceil_div(m, 256) * ceil_div(n, 256);
+        cfg = big_tiles >= 256 ? 2 : 1;
+    }
+    if (g_force_cfg >= 0 && (vec_ok || g_force_cfg == 0)) cfg = g_force_cfg;
+
+    if (cfg == 0) {
+        if (k == 0 && !accumulate && !bias) {   // empty contraction: zeros (linear.c zero-fills its output)
+            for (int64_t bt = 0; bt < batch; bt++)
+                for (int64_t r = 0; r < m; r++) bh_memset_zero(c + bt * g.stride_c + r * ldc, sizeof(float) * (size_t)n);
+            return BH_OK;
+        }
+        dim3 grid((unsigned)ceil_div(n, 32), (unsigned)ceil_div(m, 32), (unsigned)batch);
+        BH_CHECK_ARG(grid.y <= 65535, "m too large for the fallback kernel");
+        hipLaunchKernelGGL(gemm_fallback_kernel, grid, dim3(256), 0, stream(), g, trans_a, trans_b);
+        return BH_LAUNCH_CHECK("gemm_fallback_kernel");
+    }
+
+    const int bm = cfg == 2 ? 256 : 128, bn = bm;
+    g.tiles_m = (int)ceil_div(m, bm);
+    g.tiles_n = (int)ceil_div(n, bn);
+    // split K when the output alone cannot fill the chip
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * batch;
+    float* ws = nullptr;
+    if (tiles < 256 && k >= 1024) {
+        int64_t splits = ceil_div(512, tiles);
+        if (splits > k / 256) splits = k / 256;
+        if (splits > 32) splits = 32;
+        if (splits > 1) {
+            g.k_per_split = ceil_div(ceil_div(k, splits), kBK) * kBK;
+            g.k_splits = (int)ceil_div(k, g.k_per_split);
+        }
+    }
+    GemmArgs run = g;
+    if (g.k_splits > 1) {
+        ws = (float*)bh_malloc(sizeof(float) * (size_t)(g.k_splits * batch * m * n));
+        if (!ws) return BH_ENOMEM;
+        run.c = ws;
+        run.ldc = n;
+        run.stride_c = m * n;
+    }
+    int rc = cfg == 2 ? launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc);
+    if (rc == BH_OK && g.k_splits > 1) {
+        int64_t blocks = ceil_div(m * n * batch, 256);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), ws, c, bias, m, n, ldc,
+                           g.k_splits, batch, g.stride_c, accumulate);
+        rc = BH_LAUNCH_CHECK("splitk_fold_kernel");
+    }
+    if (ws) bh_free(ws);
+    return rc;
+}
+
+int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, int64_t cols) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(batch >= 0 && rows >= 0 && cols >= 0, "negative dimension");
+    if (batch * rows * cols == 0) return BH_OK;
+    BH_CHECK_ARG(a && out && batch <= 65535, "bad argument");
+    dim3 grid((unsigned)ceil_div(cols, 32), (unsigned)ceil_div(rows, 32), (unsigned)batch);
+    BH_CHECK_ARG(grid.y <= 65535, "too many rows");
+    hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, stream(), a, out, rows, cols);
+    return BH_LAUNCH_CHECK("transpose_kernel");
+}
+
+int bh_dense_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t m,
+                      int64_t k, int64_t n, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(m >= 0 && k >= 0 && n >= 0, "negative dimension");
+    BH_CHECK_ARG(x && w && dy, "null pointer");
+    int rc = BH_OK;
+    // dX[m,k] = dY[m,n] . W[k,n]^T
+    if (dx) rc = bh_gemm(0, 1, m, k, n, dy, n, w, n, dx, k, nullptr, 0, 1);
+    // dW[k,n] (+)= X[m,k]^T . dY[m,n]
+    if (rc == BH_OK && gw) rc = bh_gemm(1, 0, k, n, m, x, k, dy, n, gw, n, nullptr, accumulate, 1);
+    if (rc == BH_OK && gb) rc = bh_colsum(dy, gb, m, n, accumulate);
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,439 @@
+// bh_layernorm.hip - LayerNorm forward (emits mean, rstd) and single-pass backward.
+//
+// Forward follows boat_layernorm_forward, src/layers/norm.c:184-209 (per-row mean, then
+// two-pass biased variance) and :283-305 (rstd = 1/sqrtf(var+eps); y = (x-mean)*rstd*gamma+beta),
+// and additionally writes mean/rstd, which the reference computes and frees (:313-314).
+//
+// Backward has no counterpart in the reference (boat_layernorm_backward is a stub,
+// src/layers/norm.c:397-402).  It implements
+//   xhat = (x-mean)*rstd ; g = dy*gamma
+//   dx = rstd*(g - mean_h(g) - xhat*mean_h(g*xhat)) ; dgamma = sum_rows dy*xhat ; dbeta = sum_rows dy
+// in one read of x and dy: each thread owns fixed columns, keeps its slice of the row in
+// registers, reduces the two row sums with wavefront shuffles (+ one LDS exchange when a row
+// spans 4 wavefronts), and accumulates dgamma/dbeta for its columns over all rows of its
+// block.  Per-block partials are folded by a second small kernel (two-stage reduction, no
+// atomics, deterministic).
+#include "bh_common.h"
+
+namespace bh {
+
+constexpr int kLnBlock = 256;
+
+__device__ __forceinline__ float4 ld4(const float* p, int64_t i4) { return reinterpret_cast<const float4*>(p)[i4]; }
+__device__ __forceinline__ void st4(float* p, int64_t i4, float4 v) { reinterpret_cast<float4*>(p)[i4] = v; }
+
+// Sum of two values over the TPR threads that share a row.
+template <int TPR>
+__device__ __forceinline__ void row_sum2(float& a, float& b, float* lds, int group) {
+    a = wave_sum(a);
+    b = wave_sum(b);
+    if (TPR > 64) {
+        constexpr int W = TPR / 64;
+        const int lane = threadIdx.x & 63, w = (threadIdx.x >> 6) % W;
+        float* slot = lds + group * W * 2;
+        __syncthreads();
+        if (lane == 0) {
+            slot[w * 2] = a;
+            slot[w * 2 + 1] = b;
+        }
+        __syncthreads();
+        float ta = 0.f, tb = 0.f;
+#pragma unroll
+        for (int i = 0; i < W; i++) {
+            ta += slot[i * 2];
+            tb += slot[i * 2 + 1];
+        }
+        a = ta;
+        b = tb;
+    }
+}
+
+// ---------------------------------------------------------------- forward
+template <int TPR, int VPT>
+__global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                          const float* __restrict__ beta, float* __restrict__ y,
+                                                          float* __restrict__ mean, float* __restrict__ rstd,
+                                                          int64_t rows, int hidden, float eps, int64_t rows_per_group) {
+    constexpr int GROUPS = kLnBlock / TPR;
+    __shared__ float lds[GROUPS * (TPR / 64) * 2 + 2];
+    const int group = threadIdx.x / TPR, t = threadIdx.x % TPR;
+    const int h4 = hidden >> 2;
+    const int64_t g_id = (int64_t)blockIdx.x * GROUPS + group;
+    const int64_t r0 = g_id * rows_per_group;
+    int64_t r1 = r0 + rows_per_group;
+    if (r1 > rows) r1 = rows;
+
+    float4 gm[VPT], bt[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int c4 = t + i * TPR;
+        gm[i] = (gamma && c4 < h4) ? ld4(gamma, c4) : make_float4(1, 1, 1, 1);
+        bt[i] = (beta && c4 < h4) ? ld4(beta, c4) : make_float4(0, 0, 0, 0);
+    }
+    // rows_per_group is the same for every group, so the loop trip count (and every
+    // barrier inside row_sum2) is uniform across the block; out-of-range rows are masked.
+    for (int64_t it = 0; it < rows_per_group; it++) {
+        const int64_t r = r0 + it;
+        const bool live = r < r1;
+        float4 xv[VPT];
+        float s = 0.f, dummy = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c4 = t + i * TPR;
+            xv[i] = (live && c4 < h4) ? ld4(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
+            s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+        }
+        row_sum2<TPR>(s, dummy, lds, group);
+        const float mu = s / (float)hidden;
+        float q = 0.f;
+        dummy = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c4 = t + i * TPR;
+            if (c4 < h4) {
+                float dx0 = xv[i].x - mu, dx1 = xv[i].y - mu, dx2 = xv[i].z - mu, dx3 = xv[i].w - mu;
+                q += (dx0 * dx0 + dx1 * dx1) + (dx2 * dx2 + dx3 * dx3);
+            }
+        }
+        row_sum2<TPR>(q, dummy, lds, group);
+        const float var = q / (float)hidden;
+        const float rs = 1.0f / sqrtf(var + eps);
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                const int c4 = t + i * TPR;
+                if (c4 < h4) {
+                    float4 o;
+                    o.x = (xv[i].x - mu) * rs;
+                    o.y = (xv[i].y - mu) * rs;
+                    o.z = (xv[i].z - mu) * rs;
+                    o.w = (xv[i].w - mu) * rs;
+                    if (gamma) { o.x *= gm[i].x; o.y *= gm[i].y; o.z *= gm[i].z; o.w *= gm[i].w; }
+                    if (beta) { o.x += bt[i].x; o.y += bt[i].y; o.z += bt[i].z; o.w += bt[i].w; }
+                    st4(y + r * hidden, c4, o);
+                }
+            }
+            if (t == 0) {
+                if (mean) mean[r] = mu;
+                if (rstd) rstd[r] = rs;
+            }
+        }
+    }
+}
+
+// any hidden size: one block per row, three passes over the row (served from cache)
+__global__ __launch_bounds__(kLnBlock) void ln_fwd_generic_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                                  const float* __restrict__ beta, float* __restrict__ y,
+                                                                  float* __restrict__ mean, float* __restrict__ rstd,
+                                                                  int64_t rows, int64_t hidden, float eps) {
+    __shared__ float red[kLnBlock / 64];
+    const int64_t r = blockIdx.x;
+    const float* xr = x + r * hidden;
+    float s = 0.f;
+    for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) s += xr[c];
+    const float mu = block_sum<kLnBlock / 64>(s, red) / (float)hidden;
+    float q = 0.f;
+    for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
+        float d = xr[c] - mu;
+        q += d * d;
+    }
+    const float var = block_sum<kLnBlock / 64>(q, red) / (float)hidden;
+    const float rs = 1.0f / sqrtf(var + eps);
+    for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
+        float o = (xr[c] - mu) * rs;
+        if (gamma) o *= gamma[c];
+        if (beta) o += beta[c];
+        y[r * hidden + c] = o;
+    }
+    if (threadIdx.x == 0) {
+        if (mean) mean[r] = mu;
+        if (rstd) rstd[r] = rs;
+    }
+}
+
+// --------------------------------------------------------------- backward
+// partial layout: [num_blocks][2][hidden]  (dgamma slice, then dbeta slice)
+template <int TPR, int VPT>
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                          const float* __restrict__ dy, const float* __restrict__ mean,
+                                                          const float* __restrict__ rstd, float* __restrict__ dx,
+                                                          float* __restrict__ partial, int64_t rows, int hidden,
+                                                          int64_t rows_per_group) {
+    constexpr int GROUPS = kLnBlock / TPR;
+    extern __shared__ float dyn_lds[];           // GROUPS>1: [GROUPS][2][hidden] for the cross-group fold
+    __shared__ float lds[GROUPS * (TPR / 64) * 2 + 2];
+    const int group = threadIdx.x / TPR, t = threadIdx.x % TPR;
+    const int h4 = hidden >> 2;
+    const int64_t g_id = (int64_t)blockIdx.x * GROUPS + group;
+    const int64_t r0 = g_id * rows_per_group;
+    int64_t r1 = r0 + rows_per_group;
+    if (r1 > rows) r1 = rows;
+
+    float4 gm[VPT], dg[VPT], db[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int c4 = t + i * TPR;
+        gm[i] = (gamma && c4 < h4) ? ld4(gamma, c4) : make_float4(1, 1, 1, 1);
+        dg[i] = make_float4(0, 0, 0, 0);
+        db[i] = make_float4(0, 0, 0, 0);
+    }
+    const float inv_h = 1.0f / (float)hidden;
+    for (int64_t it = 0; it < rows_per_group; it++) {
+        const int64_t r = r0 + it;
+        const bool live = r < r1;
+        const float mu = live ? mean[r] : 0.f;
+        const float rs = live ? rstd[r] : 0.f;
+        float4 xh[VPT], g[VPT];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c4 = t + i * TPR;
+            const bool on = live && c4 < h4;
+            float4 xv = on ? ld4(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
+            float4 gy = on ? ld4(dy + r * hidden, c4) : make_float4(0, 0, 0, 0);
+            xh[i].x = (xv.x - mu) * rs; xh[i].y = (xv.y - mu) * rs; xh[i].z = (xv.z - mu) * rs; xh[i].w = (xv.w - mu) * rs;
+            g[i].x = gy.x * gm[i].x; g[i].y = gy.y * gm[i].y; g[i].z = gy.z * gm[i].z; g[i].w = gy.w * gm[i].w;
+            s1 += (g[i].x + g[i].y) + (g[i].z + g[i].w);
+            s2 += (g[i].x * xh[i].x + g[i].y * xh[i].y) + (g[i].z * xh[i].z + g[i].w * xh[i].w);
+            dg[i].x += gy.x * xh[i].x; dg[i].y += gy.y * xh[i].y; dg[i].z += gy.z * xh[i].z; dg[i].w += gy.w * xh[i].w;
+            db[i].x += gy.x; db[i].y += gy.y; db[i].z += gy.z; db[i].w += gy.w;
+        }
+        row_sum2<TPR>(s1, s2, lds, group);
+        s1 *= inv_h;
+        s2 *= inv_h;
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                const int c4 = t + i * TPR;
+                if (c4 < h4) {
+                    float4 o;
+                    o.x = rs * (g[i].x - s1 - xh[i].x * s2);
+                    o.y = rs * (g[i].y - s1 - xh[i].y * s2);
+                    o.z = rs * (g[i].z - s1 - xh[i].z * s2);
+                    o.w = rs * (g[i].w - s1 - xh[i].w * s2);
+                    st4(dx + r * hidden, c4, o);
+                }
+            }
+        }
+    }
+    float* out = partial + (int64_t)blockIdx.x * 2 * hidden;
+    if (GROUPS == 1) {
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c4 = t + i * TPR;
+            if (c4 < h4) {
+                st4(out, c4, dg[i]);
+                st4(out + hidden, c4, db[i]);
+            }
+        }
+    } else {
+        // fold the GROUPS row-groups of this block through LDS, then write one partial
+        float* mine = dyn_lds + (size_t)group * 2 * hidden;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c4 = t + i * TPR;
+            if (c4 < h4) {
+                st4(mine, c4, dg[i]);
+                st4(mine + hidden, c4, db[i]);
+            }
+        }
+        __syncthreads();
+        for (int c = threadIdx.x; c < 2 * hidden; c += kLnBlock) {
+            float acc = 0.f;
+#pragma unroll
+            for (int gidx = 0; gidx < GROUPS; gidx++) acc += dyn_lds[(size_t)gidx * 2 * hidden + c];
+            out[c] = acc;
+        }
+    }
+}
+
+// generic backward: one block per row, partial per row-chunk accumulated by columns
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_generic_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                                     const float* __restrict__ dy, const float* __restrict__ mean,
+                                                                     const float* __restrict__ rstd, float* __restrict__ dx,
+                                                                     int64_t rows, int64_t hidden) {
+    __shared__ float red[kLnBlock / 64];
+    const int64_t r = blockIdx.x;
+    const float mu = mean[r], rs = rstd[r];
+    float s1 = 0.f, s2 = 0.f;
+    for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
+        float xh = (x[r * hidden + c] - mu) * rs;
+        float g = dy[r * hidden + c] * (gamma ? gamma[c] : 1.0f);
+        s1 += g;
+        s2 += g * xh;
+    }
+    s1 = block_sum<kLnBlock / 64>(s1, red) / (float)hidden;
+    s2 = block_sum<kLnBlock / 64>(s2, red) / (float)hidden;
+    for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
+        float xh = (x[r * hidden + c] - mu) * rs;
+        float g = dy[r * hidden + c] * (gamma ? gamma[c] : 1.0f);
+        dx[r * hidden + c] = rs * (g - s1 - xh * s2);
+    }
+}
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_param_generic_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                                        const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                                        float* __restrict__ partial, int64_t rows, int64_t hidden,
+                                                                        int64_t rows_per_block) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= hidden) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    int64_t r1 = r0 + rows_per_block;
+    if (r1 > rows) r1 = rows;
+    float dg = 0.f, db = 0.f;
+    for (int64_t r = r0; r < r1; r++) {
+        float gy = dy[r * hidden + c];
+        dg += gy * ((x[r * hidden + c] - mean[r]) * rstd[r]);
+        db += gy;
+    }
+    partial[((int64_t)blockIdx.y * 2) * hidden + c] = dg;
+    partial[((int64_t)blockIdx.y * 2 + 1) * hidden + c] = db;
+}
+
+// fold partial[nblk][2][hidden] into dgamma / dbeta
+__global__ __launch_bounds__(kLnBlock) void ln_param_fold_kernel(const float* __restrict__ partial, float* __restrict__ dgamma,
+                                                                 float* __restrict__ dbeta, int64_t nblk, int64_t hidden,
+                                                                 int accumulate) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // over 2*hidden
+    if (c >= 2 * hidden) return;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int64_t k = 0;
+    for (; k + 3 < nblk; k += 4) {
+        a0 += partial[(k * 2) * hidden + c];
+        a1 += partial[((k + 1) * 2) * hidden + c];
+        a2 += partial[((k + 2) * 2) * hidden + c];
+        a3 += partial[((k + 3) * 2) * hidden + c];
+    }
+    for (; k < nblk; k++) a0 += partial[(k * 2) * hidden + c];
+    const float acc = (a0 + a1) + (a2 + a3);
+    float* dst = c < hidden ? (dgamma ? dgamma + c : nullptr) : (dbeta ? dbeta + (c - hidden) : nullptr);
+    if (dst) *dst = accumulate ? *dst + acc : acc;
+}
+
+struct LnPlan {
+    bool vector;     // register-resident float4 path
+    int tpr, vpt;
+};
+
+static LnPlan plan_for(int64_t hidden, const void* p0, const void* p1, const void* p2) {
+    LnPlan p{false, 0, 0};
+    const bool al = ((reinterpret_cast<uintptr_t>(p0) | reinterpret_cast<uintptr_t>(p1) | reinterpret_cast<uintptr_t>(p2)) & 15) == 0;
+    if (!al || (hidden & 3) || hidden <= 0) return p;
+    const int64_t h4 = hidden >> 2;
+    if (h4 <= 64 * 8) {
+        p.tpr = 64;
+    } else if (h4 <= 256 * 8) {
+        p.tpr = 256;
+    } else {
+        return p;
+    }
+    const int64_t need = ceil_div(h4, p.tpr);
+    p.vpt = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
+    p.vector = true;
+    return p;
+}
+
+}  // namespace bh
+
+using namespace bh;
+
+#define BH_LN_DISPATCH(KERNEL, plan, grid, shmem, ...)                                                         \
+    do {                                                                                                       \
+        if ((plan).tpr == 64) {                                                                                \
+            switch ((plan).vpt) {                                                                              \
+                case 1: hipLaunchKernelGGL((KERNEL<64, 1>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                case 2: hipLaunchKernelGGL((KERNEL<64, 2>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                case 4: hipLaunchKernelGGL((KERNEL<64, 4>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                default: hipLaunchKernelGGL((KERNEL<64, 8>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+            }                                                                                                  \
+        } else {                                                                                               \
+            switch ((plan).vpt) {                                                                              \
+                case 4: hipLaunchKernelGGL((KERNEL<256, 4>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                default: hipLaunchKernelGGL((KERNEL<256, 8>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+            }                                                                                                  \
+        }                                                                                                      \
+    } while (0)
+
+extern "C" {
+
+int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, float* y, float* mean, float* rstd,
+                         int64_t rows, int64_t hidden, float eps) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && hidden > 0, "bad shape");
+    if (rows == 0) return BH_OK;
+    BH_CHECK_ARG(x && y, "null pointer");
+    BH_CHECK_ARG(hidden < (int64_t(1) << 30), "hidden too large");
+    LnPlan plan = plan_for(hidden, x, y, gamma ? (const void*)gamma : (const void*)x);
+    if (plan.vector && beta && (reinterpret_cast<uintptr_t>(beta) & 15)) plan.vector = false;
+    if (!plan.vector) {
+        hipLaunchKernelGGL(ln_fwd_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, beta, y,
+                           mean, rstd, rows, hidden, eps);
+        return BH_LAUNCH_CHECK("bh_layernorm_forward");
+    }
+    const int groups = kLnBlock / plan.tpr;
+    int64_t blocks = ceil_div(rows, groups);
+    const int64_t cap = 256 * 8;
+    if (blocks > cap) blocks = cap;
+    const int64_t rpg = ceil_div(rows, blocks * groups);
+    blocks = ceil_div(rows, rpg * groups);
+    BH_LN_DISPATCH(ln_fwd_kernel, plan, dim3((unsigned)blocks), 0, x, gamma, beta, y, mean, rstd, rows, (int)hidden, eps, rpg);
+    return BH_LAUNCH_CHECK("bh_layernorm_forward");
+}
+
+int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
+                          float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && hidden > 0, "bad shape");
+    BH_CHECK_ARG(hidden < (int64_t(1) << 30), "hidden too large");
+    if (rows == 0) {
+        if (!accumulate) {
+            if (dgamma) bh_memset_zero(dgamma, sizeof(float) * (size_t)hidden);
+            if (dbeta) bh_memset_zero(dbeta, sizeof(float) * (size_t)hidden);
+        }
+        return BH_OK;
+    }
+    BH_CHECK_ARG(x && dy && mean && rstd && dx, "null pointer");
+    LnPlan plan = plan_for(hidden, x, dy, dx);
+    if (plan.vector && gamma && (reinterpret_cast<uintptr_t>(gamma) & 15)) plan.vector = false;
+    const int groups = plan.vector ? kLnBlock / plan.tpr : 1;
+    const size_t shmem = (plan.vector && groups > 1) ? sizeof(float) * (size_t)groups * 2 * (size_t)hidden : 0;
+    if (shmem > 64 * 1024) plan.vector = false;
+
+    int rc;
+    if (plan.vector) {
+        int64_t blocks = ceil_div(rows, groups);
+        const int64_t cap = 256 * 4;     // 4 blocks per CU keeps the per-block partials at a few % of the traffic
+        if (blocks > cap) blocks = cap;
+        const int64_t rpg = ceil_div(rows, blocks * groups);
+        blocks = ceil_div(rows, rpg * groups);
+        float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(blocks * 2 * hidden));
+        if (!partial) return BH_ENOMEM;
+        BH_LN_DISPATCH(ln_bwd_kernel, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
+                       (int)hidden, rpg);
+        if (dgamma || dbeta)
+            hipLaunchKernelGGL(ln_param_fold_kernel, dim3((unsigned)ceil_div(2 * hidden, kLnBlock)), dim3(kLnBlock), 0,
+                               stream(), partial, dgamma, dbeta, blocks, hidden, accumulate);
+        bh_free(partial);
+        rc = BH_LAUNCH_CHECK("bh_layernorm_backward");
+    } else {
+        hipLaunchKernelGGL(ln_bwd_dx_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, dy, mean,
+                           rstd, dx, rows, hidden);
+        rc = BH_LAUNCH_CHECK("bh_layernorm_backward dx");
+        if (rc == BH_OK && (dgamma || dbeta)) {
+            int64_t chunks = ceil_div(rows, 64);
+            if (chunks > 256) chunks = 256;
+            const int64_t rpb = ceil_div(rows, chunks);
+            chunks = ceil_div(rows, rpb);
+            float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * 2 * hidden));
+            if (!partial) return BH_ENOMEM;
+            hipLaunchKernelGGL(ln_bwd_param_generic_kernel, dim3((unsigned)ceil_div(hidden, kLnBlock), (unsigned)chunks),
+                               dim3(kLnBlock), 0, stream(), x, dy, mean, rstd, partial, rows, hidden, rpb);
+            hipLaunchKernelGGL(ln_param_fold_kernel, dim3((unsigned)ceil_div(2 * hidden, kLnBlock)), dim3(kLnBlock), 0,
+                               stream(), partial, dgamma, dbeta, chunks, hidden, accumulate);
+            bh_free(partial);
+            rc = BH_LAUNCH_CHECK("bh_layernorm_backward params");
+        }
+    }
+    return rc;
+}
+
+}  // extern "C"

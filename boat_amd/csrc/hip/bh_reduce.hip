@@ -1,0 +1,265 @@
+// bh_reduce.hip - reductions and row softmax family.
+//
+//   full sum                      src/ops/arithmetic.c:611-691 (boat_sum)
+//   column sum (bias gradient)    src/layers/dense.c:286-291, src/layers/attention.c:1257-1268
+//   softmax / log-softmax, last axis, forward and backward
+//                                 src/autodiff.c:1701-1883, 1885-2068
+//   fused softmax + cross-entropy gradient replacing the tape chain
+//   log_softmax -> mul(onehot) -> sum -> mul(-1/B) of examples/mnist/mnist_autodiff.c:397-522
+//
+// The reference adds left to right in fp32; these kernels add in wavefront trees, so
+// results agree to rounding (a few ulp), not bit for bit.
+#include "bh_common.h"
+
+#include <float.h>
+
+namespace bh {
+
+constexpr int kRBlock = 256;
+
+// ---- full sum: per-block partials, then one block folds them (double accumulator) ----
+__global__ __launch_bounds__(kRBlock) void sum_partial_kernel(const float* x, float* partial, int64_t n) {
+    __shared__ float red[kRBlock / 64];
+    float acc = 0.f;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) acc += x[i];
+    float t = block_sum<kRBlock / 64>(acc, red);
+    if (threadIdx.x == 0) partial[blockIdx.x] = t;
+}
+__global__ __launch_bounds__(kRBlock) void sum_final_kernel(const float* partial, float* out, int n, float scale) {
+    __shared__ double red[kRBlock / 64];
+    double acc = 0.0;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) acc += (double)partial[i];
+    acc = wave_sum_f64(acc);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int i = 0; i < kRBlock / 64; i++) t += red[i];
+        out[0] = (float)t * scale;
+    }
+}
+
+// ---- column sum: partial[rb][c] over row chunks, then fold the chunks ----
+__global__ __launch_bounds__(kRBlock) void colsum_partial_kernel(const float* __restrict__ x, float* __restrict__ partial,
+                                                                 int64_t rows, int64_t cols, int64_t rows_per_block) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    int64_t r1 = r0 + rows_per_block;
+    if (r1 > rows) r1 = rows;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int64_t r = r0;
+    for (; r + 3 < r1; r += 4) {
+        a0 += x[r * cols + c];
+        a1 += x[(r + 1) * cols + c];
+        a2 += x[(r + 2) * cols + c];
+        a3 += x[(r + 3) * cols + c];
+    }
+    for (; r < r1; r++) a0 += x[r * cols + c];
+    partial[(int64_t)blockIdx.y * cols + c] = (a0 + a1) + (a2 + a3);
+}
+__global__ __launch_bounds__(kRBlock) void colsum_final_kernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                               int64_t chunks, int64_t cols, int accumulate) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float acc = 0.f;
+    for (int64_t k = 0; k < chunks; k++) acc += partial[k * cols + c];
+    out[c] = accumulate ? out[c] + acc : acc;
+}
+
+// ---- row kernels: one wavefront per row, 4 rows per block ----
+// MODE 0 softmax fwd, 1 softmax bwd, 2 log-softmax fwd, 3 log-softmax bwd
+template <int MODE>
+__global__ __launch_bounds__(kRBlock) void row_softmax_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                              float* __restrict__ out, int64_t rows, int64_t cols) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kRBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* ar = a + row * cols;
+    const float* br = b ? b + row * cols : nullptr;
+    float* orow = out + row * cols;
+    if (MODE == 0 || MODE == 2) {
+        float mx = -FLT_MAX;
+        for (int64_t i = lane; i < cols; i += 64) mx = fmaxf(mx, ar[i]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int64_t i = lane; i < cols; i += 64) sum += expf(ar[i] - mx);
+        sum = wave_sum(sum);
+        if (MODE == 0) {
+            const float inv = 1.0f / sum;
+            for (int64_t i = lane; i < cols; i += 64) {
+                float e = expf(ar[i] - mx);
+                orow[i] = sum != 0.0f ? e * inv : e;
+            }
+        } else {
+            const float lse = logf(fmaxf(sum, FLT_MIN));
+            for (int64_t i = lane; i < cols; i += 64) orow[i] = ar[i] - mx - lse;
+        }
+    } else if (MODE == 1) {   // a = y, b = dy : dx = y*(dy - sum(y*dy))
+        float t = 0.f;
+        for (int64_t i = lane; i < cols; i += 64) t += ar[i] * br[i];
+        t = wave_sum(t);
+        for (int64_t i = lane; i < cols; i += 64) orow[i] = ar[i] * (br[i] - t);
+    } else {                  // a = y (log-probs), b = dy : dx = dy - exp(y)*sum(dy)
+        float g = 0.f;
+        for (int64_t i = lane; i < cols; i += 64) g += br[i];
+        g = wave_sum(g);
+        for (int64_t i = lane; i < cols; i += 64) orow[i] = br[i] - expf(ar[i]) * g;
+    }
+}
+
+// fused softmax + cross-entropy gradient; row_ll receives log_softmax(z)[label] per row
+__global__ __launch_bounds__(kRBlock) void softmax_ce_kernel(const float* __restrict__ z, const int32_t* __restrict__ labels,
+                                                             float* __restrict__ dz, float* __restrict__ row_ll,
+                                                             int64_t rows, int64_t cols, float f) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kRBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* zr = z + row * cols;
+    float mx = -FLT_MAX;
+    for (int64_t i = lane; i < cols; i += 64) mx = fmaxf(mx, zr[i]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int64_t i = lane; i < cols; i += 64) sum += expf(zr[i] - mx);
+    sum = wave_sum(sum);
+    const float lse = logf(fmaxf(sum, FLT_MIN));
+    const int32_t label = labels[row];
+    const bool valid = label >= 0 && label < cols;
+    // backward of the tape chain: d(ls)_j = f*onehot_j, dz_j = d(ls)_j - exp(ls_j) * sum_j d(ls)_j
+    const float g = valid ? f : 0.0f;
+    for (int64_t i = lane; i < cols; i += 64) {
+        const float ls = zr[i] - mx - lse;
+        const float dls = (valid && i == label) ? f : 0.0f;
+        if (dz) dz[row * cols + i] = dls - expf(ls) * g;
+        if (valid && i == label && row_ll) row_ll[row] = ls;
+    }
+    if (!valid && lane == 0 && row_ll) row_ll[row] = 0.0f;
+}
+
+}  // namespace bh
+
+using namespace bh;
+
+extern "C" {
+
+int bh_sum_all(const float* x, float* out1, int64_t n) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(n >= 0 && out1 && (x || n == 0), "bad argument");
+    int blocks = (int)ceil_div(n > 0 ? n : 1, (int64_t)kRBlock * 8);
+    if (blocks > 1024) blocks = 1024;
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);
+    if (!partial) return BH_ENOMEM;
+    hipLaunchKernelGGL(sum_partial_kernel, dim3(blocks), dim3(kRBlock), 0, stream(), x, partial, n);
+    hipLaunchKernelGGL(sum_final_kernel, dim3(1), dim3(kRBlock), 0, stream(), partial, out1, blocks, 1.0f);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK("bh_sum_all");
+}
+
+int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n);  // defined below
+
+int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && cols >= 0 && (out || cols == 0) && (x || rows * cols == 0), "bad argument");
+    if (cols == 0) return BH_OK;
+    const int col_blocks = (int)ceil_div(cols, kRBlock);
+    // enough row chunks to put ~2k blocks on the chip, at least 32 rows each
+    int64_t chunks = ceil_div(2048, col_blocks);
+    if (chunks > ceil_div(rows, 32)) chunks = ceil_div(rows, 32);
+    if (chunks < 1) chunks = 1;
+    const int64_t rpb = ceil_div(rows > 0 ? rows : 1, chunks);
+    chunks = ceil_div(rows > 0 ? rows : 1, rpb);
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * cols));
+    if (!partial) return BH_ENOMEM;
+    hipLaunchKernelGGL(colsum_partial_kernel, dim3(col_blocks, (unsigned)chunks), dim3(kRBlock), 0, stream(), x, partial,
+                       rows, cols, rpb);
+    hipLaunchKernelGGL(colsum_final_kernel, dim3(col_blocks), dim3(kRBlock), 0, stream(), partial, out, chunks, cols,
+                       accumulate);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK("bh_colsum");
+}
+
+#define BH_ROW_LAUNCH(MODE, a, b, out, name)                                                                   \
+    do {                                                                                                       \
+        BH_REQUIRE_INIT();                                                                                     \
+        BH_CHECK_ARG(rows >= 0 && cols >= 0, "negative shape");                                                \
+        if (rows * cols == 0) return BH_OK;                                                                    \
+        BH_CHECK_ARG((a) && (out), "null pointer");                                                            \
+        hipLaunchKernelGGL((row_softmax_kernel<MODE>), dim3((unsigned)ceil_div(rows, kRBlock / 64)), dim3(kRBlock), \
+                           0, stream(), a, b, out, rows, cols);                                                \
+        return BH_LAUNCH_CHECK(name);                                                                          \
+    } while (0)
+
+int bh_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols) {
+    BH_ROW_LAUNCH(0, x, (const float*)nullptr, y, "bh_softmax_forward");
+}
+int bh_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols) {
+    BH_CHECK_ARG(dy || rows * cols == 0, "null dy");
+    BH_ROW_LAUNCH(1, y, dy, dx, "bh_softmax_backward");
+}
+int bh_log_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols) {
+    BH_ROW_LAUNCH(2, x, (const float*)nullptr, y, "bh_log_softmax_forward");
+}
+int bh_log_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols) {
+    BH_CHECK_ARG(dy || rows * cols == 0, "null dy");
+    BH_ROW_LAUNCH(3, y, dy, dx, "bh_log_softmax_backward");
+}
+
+int bh_softmax_ce_grad(const float* logits, const int32_t* labels, float* dlogits, float* loss_out, int64_t rows,
+                       int64_t cols) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows > 0 && cols > 0 && logits && labels, "bad argument");
+    float* row_ll = nullptr;
+    if (loss_out) {
+        row_ll = (float*)bh_malloc(sizeof(float) * (size_t)rows);
+        if (!row_ll) return BH_ENOMEM;
+    }
+    const float f = -1.0f / (float)(size_t)rows;
+    hipLaunchKernelGGL(softmax_ce_kernel, dim3((unsigned)ceil_div(rows, kRBlock / 64)), dim3(kRBlock), 0, stream(),
+                       logits, labels, dlogits, row_ll, rows, cols, f);
+    if (loss_out) {
+        int blocks = (int)ceil_div(rows, (int64_t)kRBlock * 8);
+        if (blocks > 1024) blocks = 1024;
+        float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);
+        if (!partial) {
+            bh_free(row_ll);
+            return BH_ENOMEM;
+        }
+        hipLaunchKernelGGL(sum_partial_kernel, dim3(blocks), dim3(kRBlock), 0, stream(), row_ll, partial, rows);
+        hipLaunchKernelGGL(sum_final_kernel, dim3(1), dim3(kRBlock), 0, stream(), partial, loss_out, blocks, f);
+        bh_free(partial);
+        bh_free(row_ll);
+    }
+    return BH_LAUNCH_CHECK("bh_softmax_ce_grad");
+}
+
+}  // extern "C"
+
+// ---- mean squared error value (src/loss/mse.c:70-78) ----
+namespace bh {
+__global__ __launch_bounds__(kRBlock) void sse_partial_kernel(const float* p, const float* t, float* partial, int64_t n) {
+    __shared__ float red[kRBlock / 64];
+    float acc = 0.f;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float d = p[i] - t[i];
+        acc += d * d;
+    }
+    float s = block_sum<kRBlock / 64>(acc, red);
+    if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
+}  // namespace bh
+
+extern "C" int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(n > 0 && pred && target && loss_out, "bad argument");
+    int blocks = (int)ceil_div(n, (int64_t)kRBlock * 8);
+    if (blocks > 1024) blocks = 1024;
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);
+    if (!partial) return BH_ENOMEM;
+    hipLaunchKernelGGL(bh::sse_partial_kernel, dim3(blocks), dim3(bh::kRBlock), 0, bh::stream(), pred, target, partial, n);
+    hipLaunchKernelGGL(bh::sum_final_kernel, dim3(1), dim3(bh::kRBlock), 0, bh::stream(), partial, loss_out, blocks,
+                       1.0f / (float)(size_t)n);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK("bh_mse_loss");
+}

@@ -1,0 +1,249 @@
+// bh_sdpa.hip - scaled dot-product attention on [bh, s, d] blocks, forward and backward.
+//
+// Forward follows scaled_dot_product_attention_impl, src/layers/attention.c:997-1073:
+//   score = (q.k) * scale ; causal: score[j>i] = -1e9 ; row softmax (max-subtract, expf, /sum) ; out = A.v
+// but keeps the row log-sum-exp (max + logf(sum)) instead of the [bh,s,s] matrix A the
+// reference caches (:1049-1059).  Backward follows attention_backward, :1417-1520:
+//   dV = A^T.dO ; dA = dO.V^T ; dS = A*(dA - rowsum(dA*A)) * scale ; dQ = dS.K ; dK = dS^T.Q
+// with A recomputed as exp(score - lse).  The row term rowsum(dA*A) is evaluated as
+// rowsum(dO*O), which is the same number (A.V = O) without needing A.
+//
+// Two implementations behind one entry point:
+//   * general kernels (any s, d): one workgroup per query row (forward, dQ) or per key row
+//     (dK, dV); scores of one row live in LDS.
+//   * MFMA kernels for d == 64 and s % 64 == 0 (the shapes of the attention benchmarks).
+#include "bh_common.h"
+
+#include <float.h>
+
+namespace bh {
+
+constexpr int kSBlock = 256;
+constexpr int kMaxRowFloats = 12288;   // general path: one score row (or two) must fit in LDS
+
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float t = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) t = fmaxf(t, red[i]);
+    return t;
+}
+
+// ---- general forward: block per (head-block, query row) ----
+__global__ __launch_bounds__(kSBlock) void sdpa_fwd_row_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                               const float* __restrict__ v, float scale, int causal,
+                                                               float* __restrict__ out, float* __restrict__ lse,
+                                                               float* __restrict__ attn, int64_t s, int64_t d) {
+    extern __shared__ float row[];                 // s scores, then d floats of q
+    __shared__ float red[kSBlock / 64];
+    float* qrow = row + s;
+    const int64_t i = blockIdx.x, h = blockIdx.y;
+    const float* qh = q + h * s * d;
+    const float* kh = k + h * s * d;
+    const float* vh = v + h * s * d;
+    for (int64_t t = threadIdx.x; t < d; t += kSBlock) qrow[t] = qh[i * d + t];
+    __syncthreads();
+    float mx = -FLT_MAX;
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) {
+        float sum = 0.f;
+        for (int64_t t = 0; t < d; t++) sum += qrow[t] * kh[j * d + t];
+        float sc = sum * scale;
+        if (causal && j > i) sc = -1e9f;
+        row[j] = sc;
+        mx = fmaxf(mx, sc);
+    }
+    mx = block_max<kSBlock / 64>(mx, red);
+    float sum = 0.f;
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) {
+        float e = expf(row[j] - mx);
+        row[j] = e;
+        sum += e;
+    }
+    sum = block_sum<kSBlock / 64>(sum, red);
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) {
+        float p = sum != 0.0f ? row[j] / sum : row[j];
+        row[j] = p;
+        if (attn) attn[(h * s + i) * s + j] = p;
+    }
+    if (threadIdx.x == 0 && lse) lse[h * s + i] = mx + logf(sum);
+    __syncthreads();
+    for (int64_t t = threadIdx.x; t < d; t += kSBlock) {
+        float acc = 0.f;
+        for (int64_t j = 0; j < s; j++) acc += row[j] * vh[j * d + t];
+        out[(h * s + i) * d + t] = acc;
+    }
+}
+
+// delta[i] = sum_d dO[i,d] * O[i,d], one wavefront per row
+__global__ __launch_bounds__(kSBlock) void sdpa_delta_kernel(const float* __restrict__ o, const float* __restrict__ d_out,
+                                                             float* __restrict__ delta, int64_t rows, int64_t d) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * (kSBlock / 64) + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    float acc = 0.f;
+    for (int64_t t = lane; t < d; t += 64) acc += o[r * d + t] * d_out[r * d + t];
+    acc = wave_sum(acc);
+    if (lane == 0) delta[r] = acc;
+}
+
+// ---- general backward, dQ: block per (head-block, query row) ----
+__global__ __launch_bounds__(kSBlock) void sdpa_bwd_dq_row_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                                  const float* __restrict__ v, const float* __restrict__ lse,
+                                                                  const float* __restrict__ delta, const float* __restrict__ d_out,
+                                                                  float scale, int causal, float* __restrict__ dq, int64_t s,
+                                                                  int64_t d) {
+    extern __shared__ float row[];                 // s floats of dS, then q row, then dO row
+    float* qrow = row + s;
+    float* grow = qrow + d;
+    const int64_t i = blockIdx.x, h = blockIdx.y;
+    const float* kh = k + h * s * d;
+    const float* vh = v + h * s * d;
+    for (int64_t t = threadIdx.x; t < d; t += kSBlock) {
+        qrow[t] = q[(h * s + i) * d + t];
+        grow[t] = d_out[(h * s + i) * d + t];
+    }
+    __syncthreads();
+    const float l = lse[h * s + i], dl = delta[h * s + i];
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) {
+        float sc = 0.f, dp = 0.f;
+        for (int64_t t = 0; t < d; t++) {
+            sc += qrow[t] * kh[j * d + t];
+            dp += grow[t] * vh[j * d + t];
+        }
+        sc *= scale;
+        if (causal && j > i) sc = -1e9f;
+        const float p = expf(sc - l);
+        row[j] = p * (dp - dl) * scale;
+    }
+    __syncthreads();
+    for (int64_t t = threadIdx.x; t < d; t += kSBlock) {
+        float acc = 0.f;
+        for (int64_t j = 0; j < s; j++) acc += row[j] * kh[j * d + t];
+        dq[(h * s + i) * d + t] = acc;
+    }
+}
+
+// ---- general backward, dK and dV: block per (head-block, key row) ----
+__global__ __launch_bounds__(kSBlock) void sdpa_bwd_dkv_row_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                                   const float* __restrict__ v, const float* __restrict__ lse,
+                                                                   const float* __restrict__ delta, const float* __restrict__ d_out,
+                                                                   float scale, int causal, float* __restrict__ dk,
+                                                                   float* __restrict__ dv, int64_t s, int64_t d) {
+    extern __shared__ float col[];                 // s floats of P, s floats of dS, k row, v row
+    float* ds = col + s;
+    float* krow = ds + s;
+    float* vrow = krow + d;
+    const int64_t j = blockIdx.x, h = blockIdx.y;
+    const float* qh = q + h * s * d;
+    const float* gh = d_out + h * s * d;
+    for (int64_t t = threadIdx.x; t < d; t += kSBlock) {
+        krow[t] = k[(h * s + j) * d + t];
+        vrow[t] = v[(h * s + j) * d + t];
+    }
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < s; i += kSBlock) {
+        float sc = 0.f, dp = 0.f;
+        for (int64_t t = 0; t < d; t++) {
+            sc += qh[i * d + t] * krow[t];
+            dp += gh[i * d + t] * vrow[t];
+        }
+        sc *= scale;
+        if (causal && j > i) sc = -1e9f;
+        const float p = expf(sc - lse[h * s + i]);
+        col[i] = p;
+        ds[i] = p * (dp - delta[h * s + i]) * scale;
+    }
+    __syncthreads();
+    for (int64_t t = threadIdx.x; t < d; t += kSBlock) {
+        float av = 0.f, ak = 0.f;
+        for (int64_t i = 0; i < s; i++) {
+            av += col[i] * gh[i * d + t];
+            ak += ds[i] * qh[i * d + t];
+        }
+        dv[(h * s + j) * d + t] = av;
+        dk[(h * s + j) * d + t] = ak;
+    }
+}
+
+}  // namespace bh
+
+using namespace bh;
+
+namespace bh {
+// MFMA path (defined in bh_sdpa_mfma.hip); returns BH_EINVAL-free "not applicable" as 1
+int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
+                      int64_t bh_count, int64_t s, int64_t d);
+int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
+                       const float* d_out, float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count,
+                       int64_t s, int64_t d);
+static int g_sdpa_force_general = 0;
+}  // namespace bh
+
+extern "C" {
+
+// test hook: 1 forces the general kernels even where the MFMA path applies
+int bh_sdpa_force_general(int on) {
+    g_sdpa_force_general = on;
+    return BH_OK;
+}
+
+int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
+                    float* attn_out, int64_t bh_count, int64_t s, int64_t d) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
+    if (bh_count == 0 || s == 0) return BH_OK;
+    BH_CHECK_ARG(q && k && v && out, "null pointer");
+    BH_CHECK_ARG(bh_count <= 65535, "too many head blocks");
+    if (!g_sdpa_force_general && !attn_out && lse) {
+        int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, bh_count, s, d);
+        if (rc <= 0) return rc;   // 0 done, <0 error, 1 shape not covered
+    }
+    BH_CHECK_ARG(s + d <= kMaxRowFloats, "sequence too long for the general attention kernel");
+    const size_t shmem = sizeof(float) * (size_t)(s + d);
+    hipLaunchKernelGGL(sdpa_fwd_row_kernel, dim3((unsigned)s, (unsigned)bh_count), dim3(kSBlock), shmem, stream(), q, k, v,
+                       scale, causal, out, lse, attn_out, s, d);
+    return BH_LAUNCH_CHECK("sdpa_fwd_row_kernel");
+}
+
+int bh_sdpa_backward(const float* q, const float* k, const float* v, const float* out, const float* lse, const float* d_out,
+                     float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count, int64_t s, int64_t d) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
+    if (bh_count == 0 || s == 0) return BH_OK;
+    BH_CHECK_ARG(q && k && v && out && lse && d_out && dq && dk && dv, "null pointer");
+    BH_CHECK_ARG(bh_count <= 65535, "too many head blocks");
+    const int64_t rows = bh_count * s;
+    float* delta = (float*)bh_malloc(sizeof(float) * (size_t)rows);
+    if (!delta) return BH_ENOMEM;
+    hipLaunchKernelGGL(sdpa_delta_kernel, dim3((unsigned)ceil_div(rows, kSBlock / 64)), dim3(kSBlock), 0, stream(), out,
+                       d_out, delta, rows, d);
+    int rc = BH_LAUNCH_CHECK("sdpa_delta_kernel");
+    if (rc == BH_OK) {
+        int done = 1;
+        if (!g_sdpa_force_general)
+            done = sdpa_backward_mfma(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);
+        if (done < 0) rc = done;
+        if (done == 1) {
+            if (2 * s + 2 * d > kMaxRowFloats) {
+                bh_free(delta);
+                return set_error(BH_EINVAL, "bh_sdpa_backward: sequence too long for the general attention kernel");
+            }
+            hipLaunchKernelGGL(sdpa_bwd_dq_row_kernel, dim3((unsigned)s, (unsigned)bh_count), dim3(kSBlock),
+                               sizeof(float) * (size_t)(s + 2 * d), stream(), q, k, v, lse, delta, d_out, scale, causal, dq, s,
+                               d);
+            hipLaunchKernelGGL(sdpa_bwd_dkv_row_kernel, dim3((unsigned)s, (unsigned)bh_count), dim3(kSBlock),
+                               sizeof(float) * (size_t)(2 * s + 2 * d), stream(), q, k, v, lse, delta, d_out, scale, causal,
+                               dk, dv, s, d);
+            rc = BH_LAUNCH_CHECK("sdpa_bwd_row_kernels");
+        }
+    }
+    bh_free(delta);
+    return rc;
+}
+
+}  // extern "C"

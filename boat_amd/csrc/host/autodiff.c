@@ -1,0 +1,571 @@
+/* autodiff.c - tape recording and the backward driver.
+ *
+ * API and per-op gradient arithmetic follow src/autodiff.c of the reference: variables
+ * (:138-297), op recording (:2070-2150, :2283-2347, :2388-2456; layer ops record only when
+ * their FIRST input requires grad, generic ops when ANY input does), the per-op backward
+ * rules (:1002-2068, :2458-2672) and gradient accumulation into input->grad with boat_add_.
+ *
+ * The driver differs on purpose.  The reference recurses depth-first from every op into each
+ * non-leaf input (:431-450), which propagates a non-leaf's gradient once per consumer and so
+ * double-counts fan-out (z = y + y, y = a*b gives dz/da = 4b).  Here every op reachable from
+ * the root is visited exactly once, in reverse recording order, after all of its consumers:
+ * identical to the reference on chains and leaf fan-out, and the true gradient elsewhere.
+ *
+ * Lifetime: an op is owned by its output variable and holds references on its inputs, so a
+ * variable the caller has freed stays alive while a later result still needs it, and the whole
+ * tape of a step is released when its last result is freed.
+ */
+#include "boat_internal.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+typedef enum {
+    OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_RELU, OP_SIGMOID, OP_TANH, OP_MATMUL, OP_DOT, OP_SUM, OP_MEAN,
+    OP_SOFTMAX, OP_LOG_SOFTMAX, OP_FLATTEN, OP_DENSE, OP_ATTENTION, OP_GELU, OP_LAYERNORM
+} op_type_t;
+
+typedef struct boat_op {
+    op_type_t type;
+    boat_variable_t* inputs[3];
+    size_t num_inputs;
+    boat_variable_t* output;     /* weak: the output owns the op */
+    void* layer;                 /* dense / attention / layernorm */
+    boat_tensor_t* saved[3];     /* per-op saved tensors (layernorm: input, mean, rstd) */
+    uint64_t seq;                /* recording order == a topological order */
+    uint64_t mark;               /* visit epoch of the backward that last collected it */
+} boat_op_t;
+
+struct boat_variable_t {
+    boat_tensor_t* data;
+    boat_tensor_t* grad;
+    bool requires_grad;
+    bool persistent_grad;        /* grad buffer survives zero_grad (boat_hip_variable_ensure_grad) */
+    boat_op_t* producer;
+    size_t refs;
+    struct boat_variable_t *prev, *next;   /* live-variable list of the library */
+};
+
+struct boat_autodiff_context_t {
+    bool grad_enabled;
+};
+
+static _Thread_local boat_autodiff_context_t* g_current = NULL;
+static boat_variable_t* g_live = NULL;
+static uint64_t g_seq = 0, g_epoch = 0;
+
+/* ------------------------------------------------------------- variables */
+
+static void variable_unref(boat_variable_t* v);
+
+static void op_free(boat_op_t* op) {
+    if (!op) return;
+    for (size_t i = 0; i < 3; i++) boat_tensor_free(op->saved[i]);
+    for (size_t i = 0; i < op->num_inputs; i++) variable_unref(op->inputs[i]);
+    free(op);
+}
+
+static void variable_unref(boat_variable_t* v) {
+    if (!v || --v->refs > 0) return;
+    if (v->prev) v->prev->next = v->next; else g_live = v->next;
+    if (v->next) v->next->prev = v->prev;
+    boat_op_t* op = v->producer;
+    v->producer = NULL;
+    boat_tensor_free(v->grad);
+    boat_tensor_free(v->data);
+    free(v);
+    op_free(op);
+}
+
+boat_variable_t* boat_variable_create(boat_tensor_t* tensor, bool requires_grad) {
+    if (!tensor) return NULL;
+    boat_variable_t* v = (boat_variable_t*)calloc(1, sizeof(*v));
+    if (!v) return NULL;
+    v->data = tensor;
+    boat_tensor_ref(tensor);
+    v->requires_grad = requires_grad;
+    v->refs = 1;
+    v->next = g_live;
+    if (g_live) g_live->prev = v;
+    g_live = v;
+    if (!g_current) g_current = boat_autodiff_context_create();   /* lazily, as autodiff.c:167-190 */
+    return v;
+}
+
+boat_variable_t* boat_variable_create_with_shape(const int64_t* shape, size_t ndim, boat_dtype_t dtype, bool requires_grad) {
+    boat_tensor_t* t = boat_tensor_create(shape, ndim, dtype, BOAT_DEVICE_CPU);
+    if (!t) return NULL;
+    boat_variable_t* v = boat_variable_create(t, requires_grad);
+    boat_tensor_unref(t);
+    return v;
+}
+
+void boat_variable_free(const boat_variable_t* variable) { variable_unref((boat_variable_t*)variable); }
+boat_tensor_t* boat_variable_data(const boat_variable_t* v) { return v ? v->data : NULL; }
+boat_tensor_t* boat_variable_grad(const boat_variable_t* v) { return v ? v->grad : NULL; }
+bool boat_variable_requires_grad(const boat_variable_t* v) { return v ? v->requires_grad : false; }
+void boat_variable_set_requires_grad(boat_variable_t* v, bool requires_grad) {
+    if (v) v->requires_grad = requires_grad;
+}
+
+bool boat_variable_reset_data(boat_variable_t* v, boat_tensor_t* new_tensor) {
+    if (!v || !new_tensor) return false;
+    if (v->producer) {
+        fprintf(stderr, "Warning: Cannot reset data for variable with computation graph node\n");
+        return false;
+    }
+    boat_tensor_ref(new_tensor);
+    boat_tensor_unref(v->data);
+    v->data = new_tensor;
+    if (v->grad && !v->persistent_grad) {
+        boat_tensor_unref(v->grad);
+        v->grad = NULL;
+    }
+    return true;
+}
+
+void boat_variable_zero_grad(boat_variable_t* v) {
+    if (!v || !v->grad) return;
+    if (v->persistent_grad) {
+        float* g = bt_dev_write(v->grad);
+        if (g) boat_hip_ok(bh_memset_zero(g, v->grad->nbytes), "boat_variable_zero_grad");
+    } else {
+        boat_tensor_unref(v->grad);   /* the reference drops the tensor (autodiff.c:285-292) */
+        v->grad = NULL;
+    }
+}
+
+boat_tensor_t* boat_hip_variable_ensure_grad(boat_variable_t* v) {
+    if (!v) return NULL;
+    if (!v->grad) v->grad = boat_tensor_create_like(v->data);
+    v->persistent_grad = v->grad != NULL;
+    return v->grad;
+}
+
+void boat_variable_retain_grad(const boat_variable_t* v, bool retain) {
+    (void)v;
+    (void)retain;   /* every variable keeps its gradient, as in the reference */
+}
+
+/* --------------------------------------------------------------- context */
+
+boat_autodiff_context_t* boat_autodiff_context_create(void) {
+    boat_autodiff_context_t* c = (boat_autodiff_context_t*)calloc(1, sizeof(*c));
+    if (c) c->grad_enabled = true;
+    return c;
+}
+void boat_autodiff_context_free(const boat_autodiff_context_t* c) {
+    if (c == g_current) g_current = NULL;
+    free((void*)c);
+}
+void boat_autodiff_context_enable_grad(boat_autodiff_context_t* c) { if (c) c->grad_enabled = true; }
+void boat_autodiff_context_disable_grad(boat_autodiff_context_t* c) { if (c) c->grad_enabled = false; }
+bool boat_autodiff_context_grad_enabled(const boat_autodiff_context_t* c) { return c ? c->grad_enabled : false; }
+void boat_autodiff_set_current_context(const boat_autodiff_context_t* c) { g_current = (boat_autodiff_context_t*)c; }
+boat_autodiff_context_t* boat_autodiff_get_current_context(void) { return g_current; }
+
+/* Drops every recorded op: all live variables become leaves, intermediates that only the tape
+ * kept alive are released; layers and their parameters are never touched. */
+void boat_autodiff_clear_computation_graph(void) {
+    /* detach first, free afterwards: freeing an op can free variables further down the list */
+    size_t n = 0, cap = 64;
+    boat_op_t** ops = (boat_op_t**)malloc(cap * sizeof(*ops));
+    if (!ops) return;
+    for (boat_variable_t* v = g_live; v; v = v->next) {
+        if (!v->producer) continue;
+        if (n == cap) {
+            boat_op_t** grown = (boat_op_t**)realloc(ops, 2 * cap * sizeof(*ops));
+            if (!grown) break;
+            ops = grown;
+            cap *= 2;
+        }
+        ops[n++] = v->producer;
+        v->producer = NULL;
+    }
+    for (size_t i = 0; i < n; i++) op_free(ops[i]);
+    free(ops);
+}
+
+/* ------------------------------------------------------------- recording */
+
+static bool recording(void) { return !g_current || g_current->grad_enabled; }
+
+static boat_variable_t* record(op_type_t type, boat_variable_t* const* inputs, size_t n, boat_tensor_t* out_tensor,
+                               bool requires_grad, void* layer) {
+    if (!out_tensor) return NULL;
+    boat_variable_t* out = boat_variable_create(out_tensor, requires_grad);
+    boat_tensor_unref(out_tensor);   /* the variable holds the reference now */
+    if (!out) return NULL;
+    if (requires_grad && recording()) {
+        boat_op_t* op = (boat_op_t*)calloc(1, sizeof(*op));
+        if (!op) {
+            boat_variable_free(out);
+            return NULL;
+        }
+        op->type = type;
+        op->num_inputs = n;
+        for (size_t i = 0; i < n; i++) {
+            op->inputs[i] = inputs[i];
+            inputs[i]->refs++;
+        }
+        op->output = out;
+        op->layer = layer;
+        op->seq = ++g_seq;
+        out->producer = op;
+    }
+    return out;
+}
+
+static boat_variable_t* binary(op_type_t type, const boat_variable_t* a, const boat_variable_t* b,
+                               boat_tensor_t* (*fwd)(const boat_tensor_t*, const boat_tensor_t*)) {
+    if (!a || !b) return NULL;
+    boat_variable_t* in[2] = {(boat_variable_t*)a, (boat_variable_t*)b};
+    return record(type, in, 2, fwd(a->data, b->data), a->requires_grad || b->requires_grad, NULL);
+}
+static boat_variable_t* unary(op_type_t type, const boat_variable_t* a, boat_tensor_t* out) {
+    if (!a) {
+        boat_tensor_free(out);
+        return NULL;
+    }
+    boat_variable_t* in[1] = {(boat_variable_t*)a};
+    return record(type, in, 1, out, a->requires_grad, NULL);
+}
+
+boat_variable_t* boat_var_add(const boat_variable_t* a, const boat_variable_t* b) { return binary(OP_ADD, a, b, boat_add); }
+boat_variable_t* boat_var_sub(const boat_variable_t* a, const boat_variable_t* b) { return binary(OP_SUB, a, b, boat_sub); }
+boat_variable_t* boat_var_mul(const boat_variable_t* a, const boat_variable_t* b) { return binary(OP_MUL, a, b, boat_mul); }
+boat_variable_t* boat_var_div(const boat_variable_t* a, const boat_variable_t* b) { return binary(OP_DIV, a, b, boat_div); }
+boat_variable_t* boat_var_matmul(const boat_variable_t* a, const boat_variable_t* b) { return binary(OP_MATMUL, a, b, boat_matmul); }
+boat_variable_t* boat_var_dot(const boat_variable_t* a, const boat_variable_t* b) { return binary(OP_DOT, a, b, boat_dot); }
+boat_variable_t* boat_var_relu(const boat_variable_t* a) { return a ? unary(OP_RELU, a, boat_relu(a->data)) : NULL; }
+boat_variable_t* boat_var_sigmoid(const boat_variable_t* a) { return a ? unary(OP_SIGMOID, a, boat_sigmoid(a->data)) : NULL; }
+boat_variable_t* boat_var_tanh(const boat_variable_t* a) { return a ? unary(OP_TANH, a, boat_tanh(a->data)) : NULL; }
+boat_variable_t* boat_hip_var_gelu(const boat_variable_t* a) { return a ? unary(OP_GELU, a, boat_gelu(a->data)) : NULL; }
+/* the axis argument is ignored by the reference, which always works on the last axis (autodiff.c:530-548) */
+boat_variable_t* boat_var_softmax(const boat_variable_t* a, int axis) {
+    (void)axis;
+    return a ? unary(OP_SOFTMAX, a, boat_softmax(a->data, -1)) : NULL;
+}
+boat_variable_t* boat_var_log_softmax(const boat_variable_t* a, int axis) {
+    (void)axis;
+    return a ? unary(OP_LOG_SOFTMAX, a, boat_log_softmax(a->data, -1)) : NULL;
+}
+boat_variable_t* boat_var_sum(const boat_variable_t* a, const int64_t* dims, size_t n_dims, bool keepdim) {
+    (void)dims; (void)n_dims; (void)keepdim;   /* full reduction only (autodiff.c:937-940) */
+    return a ? unary(OP_SUM, a, boat_sum(a->data, NULL, 0, false)) : NULL;
+}
+/* mean keeps the input's shape with the mean in element 0 and zeros elsewhere (autodiff.c:947-985) */
+boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim) {
+    (void)dims; (void)n_dims; (void)keepdim;
+    if (!a || a->data->nelements == 0 || !bt_is_f32(a->data)) return NULL;
+    boat_tensor_t* m = boat_mean(a->data, NULL, 0, false);
+    boat_tensor_t* out = m ? boat_tensor_create_like(a->data) : NULL;
+    float* po = out ? bt_dev_rw(out) : NULL;
+    if (!po || !boat_hip_ok(bh_memcpy_d2d(po, bt_dev_read(m), sizeof(float)), "boat_var_mean")) {
+        boat_tensor_free(m);
+        boat_tensor_free(out);
+        return NULL;
+    }
+    boat_tensor_free(m);
+    return unary(OP_MEAN, a, out);
+}
+boat_variable_t* boat_var_flatten(const boat_variable_t* a) {
+    if (!a) return NULL;
+    const boat_tensor_t* t = a->data;
+    if (t->ndim < 2) {
+        fprintf(stderr, "Error: Flatten expects at least 2D input tensor\n");
+        return NULL;
+    }
+    int64_t rest = 1;
+    for (size_t i = 1; i < t->ndim; i++) rest *= t->shape[i];
+    const int64_t shape[] = {t->shape[0], rest};
+    return unary(OP_FLATTEN, a, boat_tensor_reshape(t, shape, 2));
+}
+
+boat_variable_t* boat_var_dense(const boat_variable_t* input, const struct boat_dense_layer_t* layer) {
+    if (!input || !layer) return NULL;
+    boat_variable_t* in[1] = {(boat_variable_t*)input};
+    return record(OP_DENSE, in, 1, boat_dense_layer_forward((boat_dense_layer_t*)layer, input->data), input->requires_grad, (void*)layer);
+}
+
+boat_variable_t* boat_var_attention(const boat_variable_t* q, const boat_variable_t* k, const boat_variable_t* v,
+                                    const struct boat_attention_t* attention, const boat_tensor_t* mask) {
+    if (!q || !k || !v || !attention) return NULL;
+    boat_variable_t* in[3] = {(boat_variable_t*)q, (boat_variable_t*)k, (boat_variable_t*)v};
+    return record(OP_ATTENTION, in, 3, boat_attention_forward((boat_attention_t*)attention, q->data, k->data, v->data, mask),
+                  q->requires_grad || k->requires_grad || v->requires_grad, (void*)attention);
+}
+
+boat_variable_t* boat_hip_var_layernorm(const boat_variable_t* a, boat_layernorm_t* norm) {
+    if (!a || !norm) return NULL;
+    boat_tensor_t* y = boat_layernorm_forward(norm, a->data);
+    if (!y) return NULL;
+    boat_variable_t* in[1] = {(boat_variable_t*)a};
+    boat_variable_t* out = record(OP_LAYERNORM, in, 1, y, a->requires_grad, norm);
+    if (out && out->producer) {
+        /* the layer may run again before this op's backward: keep this call's statistics */
+        boat_op_t* op = out->producer;
+        op->saved[0] = a->data;
+        op->saved[1] = norm->cache_mean;
+        op->saved[2] = norm->cache_rstd;
+        for (int i = 0; i < 3; i++) boat_tensor_ref(op->saved[i]);
+    }
+    return out;
+}
+
+/* -------------------------------------------------------------- backward */
+
+/* v->grad += g ; takes ownership of g when `own` (it may become the gradient tensor itself,
+ * as the reference does with freshly computed gradients, autodiff.c:1128-1135) */
+static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
+    if (!g) return;
+    if (!v->grad) {
+        if (own && g->ref_count == 1 && !g->is_view && g->nelements == v->data->nelements) {
+            v->grad = g;
+            return;
+        }
+        v->grad = boat_tensor_create_like(v->data);
+    }
+    if (v->grad) boat_add_(v->grad, g);
+    if (own) boat_tensor_unref(g);
+}
+
+static boat_tensor_t* ones_like(const boat_tensor_t* t) {
+    boat_tensor_t* o = bt_new_like_uninit(t);
+    float* p = o ? bt_dev_write(o) : NULL;
+    if (!p || !boat_hip_ok(bh_fill(p, 1.0f, (int64_t)o->nelements), "ones_like")) {
+        boat_tensor_free(o);
+        return NULL;
+    }
+    return o;
+}
+
+static boat_tensor_t* activation_grad(int act, const boat_tensor_t* saved, const boat_tensor_t* dy) {
+    if (saved->nelements != dy->nelements) return NULL;
+    boat_tensor_t* dx = bt_new_like_uninit(saved);
+    const float* ps = bt_dev_read(saved);
+    const float* pg = bt_dev_read(dy);
+    float* pd = dx ? bt_dev_write(dx) : NULL;
+    if (!ps || !pg || !pd || !boat_hip_ok(bh_activation_backward(act, ps, pg, pd, (int64_t)saved->nelements, 0), "activation backward")) {
+        boat_tensor_free(dx);
+        return NULL;
+    }
+    return dx;
+}
+
+static boat_tensor_t* row_softmax_grad(bool log_form, const boat_tensor_t* y, const boat_tensor_t* dy) {
+    if (y->nelements != dy->nelements || y->nelements == 0) return NULL;
+    const int64_t cols = y->ndim > 0 ? y->shape[y->ndim - 1] : 1;
+    const int64_t rows = (int64_t)y->nelements / cols;
+    boat_tensor_t* dx = bt_new_like_uninit(y);
+    const float* py = bt_dev_read(y);
+    const float* pg = bt_dev_read(dy);
+    float* pd = dx ? bt_dev_write(dx) : NULL;
+    int rc = (!py || !pg || !pd) ? BH_EDEVICE
+                                 : log_form ? bh_log_softmax_backward(py, pg, pd, rows, cols) : bh_softmax_backward(py, pg, pd, rows, cols);
+    if (!boat_hip_ok(rc, "softmax backward")) {
+        boat_tensor_free(dx);
+        return NULL;
+    }
+    return dx;
+}
+
+/* first element of a (scalar) gradient tensor, read back to the host: the reference reads
+ * grad_output[0] as float for sum/dot (autodiff.c:1228, 1536) */
+static bool scalar_of(const boat_tensor_t* t, float* out) {
+    if (!t || t->nelements < 1) return false;
+    const float* p = bt_dev_read(t);
+    return p && boat_hip_ok(bh_memcpy_d2h(out, p, sizeof(float)), "scalar readback");
+}
+
+static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
+    boat_variable_t* a = op->inputs[0];
+    boat_variable_t* b = op->num_inputs > 1 ? op->inputs[1] : NULL;
+    switch (op->type) {
+        case OP_ADD:   /* autodiff.c:1002-1061 */
+            if (a->requires_grad) accumulate(a, (boat_tensor_t*)dy, false);
+            if (b->requires_grad) accumulate(b, (boat_tensor_t*)dy, false);
+            break;
+        case OP_SUB:   /* :1063-1113 */
+            if (a->requires_grad) accumulate(a, (boat_tensor_t*)dy, false);
+            if (b->requires_grad) accumulate(b, boat_mul_scalar(dy, -1.0), true);
+            break;
+        case OP_MUL:   /* :1115-1147 */
+            if (a->requires_grad) accumulate(a, boat_mul(dy, b->data), true);
+            if (b->requires_grad) accumulate(b, boat_mul(dy, a->data), true);
+            break;
+        case OP_DIV:   /* :1149-1203 */
+            if (a->requires_grad) accumulate(a, boat_div(dy, b->data), true);
+            if (b->requires_grad && bt_same_shape(a->data, b->data) && bt_same_shape(a->data, dy)) {
+                boat_tensor_t* g = bt_new_like_uninit(b->data);
+                float* pg = g ? bt_dev_write(g) : NULL;
+                if (pg && boat_hip_ok(bh_div_backward_b(bt_dev_read(a->data), bt_dev_read(b->data), bt_dev_read(dy), pg,
+                                                        (int64_t)g->nelements), "div backward"))
+                    accumulate(b, g, true);
+                else
+                    boat_tensor_free(g);
+            } else if (b->requires_grad) {   /* broadcast operands: the reference's op-by-op form */
+                boat_tensor_t* bsq = boat_mul(b->data, b->data);
+                boat_tensor_t* adb = bsq ? boat_div(a->data, bsq) : NULL;
+                boat_tensor_t* neg = boat_mul_scalar(dy, -1.0);
+                boat_tensor_t* g = (adb && neg) ? boat_mul(neg, adb) : NULL;
+                boat_tensor_free(bsq);
+                boat_tensor_free(adb);
+                boat_tensor_free(neg);
+                accumulate(b, g, true);
+            }
+            break;
+        case OP_DOT: {   /* :1205-1242 */
+            float s;
+            if (!scalar_of(dy, &s)) break;
+            if (a->requires_grad) accumulate(a, boat_mul_scalar(b->data, s), true);
+            if (b->requires_grad) accumulate(b, boat_mul_scalar(a->data, s), true);
+            break;
+        }
+        case OP_RELU:      /* :1244-1296, mask from the op input */
+            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_RELU, a->data, dy), true);
+            break;
+        case OP_GELU:
+            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_GELU, a->data, dy), true);
+            break;
+        case OP_SIGMOID:   /* :1298-1353, from the saved output */
+            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_SIGMOID, op->output->data, dy), true);
+            break;
+        case OP_TANH:      /* :1355-1452 */
+            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_TANH, op->output->data, dy), true);
+            break;
+        case OP_MATMUL: {  /* :1454-1496, 2-D operands */
+            const boat_tensor_t *A = a->data, *B = b->data;
+            if (A->ndim != 2 || B->ndim != 2 || dy->ndim != 2) break;
+            const int64_t m = A->shape[0], k = A->shape[1], n = B->shape[1];
+            if (a->requires_grad) {   /* dA = dY . B^T */
+                boat_tensor_t* g = bt_new_like_uninit(A);
+                float* pg = g ? bt_dev_write(g) : NULL;
+                if (pg && boat_hip_ok(bh_gemm(0, 1, m, k, n, bt_dev_read(dy), n, bt_dev_read(B), n, pg, k, NULL, 0, 1), "matmul backward"))
+                    accumulate(a, g, true);
+                else
+                    boat_tensor_free(g);
+            }
+            if (b->requires_grad) {   /* dB = A^T . dY */
+                boat_tensor_t* g = bt_new_like_uninit(B);
+                float* pg = g ? bt_dev_write(g) : NULL;
+                if (pg && boat_hip_ok(bh_gemm(1, 0, k, n, m, bt_dev_read(A), k, bt_dev_read(dy), n, pg, n, NULL, 0, 1), "matmul backward"))
+                    accumulate(b, g, true);
+                else
+                    boat_tensor_free(g);
+            }
+            break;
+        }
+        case OP_SUM: {     /* :1498-1548: ones * (float)dy[0] */
+            float s;
+            if (!a->requires_grad || !scalar_of(dy, &s)) break;
+            boat_tensor_t* ones = ones_like(a->data);
+            boat_tensor_t* g = ones ? boat_mul_scalar(ones, s) : NULL;
+            boat_tensor_free(ones);
+            accumulate(a, g, true);
+            break;
+        }
+        case OP_MEAN: {    /* :1550-1618: (ones * 1/n) * dy */
+            if (!a->requires_grad) break;
+            boat_tensor_t* ones = ones_like(a->data);
+            boat_tensor_t* scaled = ones ? boat_mul_scalar(ones, 1.0f / a->data->nelements) : NULL;
+            boat_tensor_t* g = scaled ? boat_mul(scaled, dy) : NULL;
+            boat_tensor_free(ones);
+            boat_tensor_free(scaled);
+            accumulate(a, g, true);
+            break;
+        }
+        case OP_SOFTMAX:       /* :1885-1973 */
+            if (a->requires_grad) accumulate(a, row_softmax_grad(false, op->output->data, dy), true);
+            break;
+        case OP_LOG_SOFTMAX:   /* :1975-2068 */
+            if (a->requires_grad) accumulate(a, row_softmax_grad(true, op->output->data, dy), true);
+            break;
+        case OP_FLATTEN:       /* :2563-2590 */
+            if (a->requires_grad) accumulate(a, boat_tensor_reshape(dy, a->data->shape, a->data->ndim), true);
+            break;
+        case OP_DENSE: {       /* :2640-2672 */
+            boat_tensor_t* dx = boat_dense_layer_backward((boat_dense_layer_t*)op->layer, dy);
+            if (dx && a->requires_grad) accumulate(a, dx, true);
+            else boat_tensor_free(dx);
+            break;
+        }
+        case OP_LAYERNORM: {
+            boat_tensor_t* dx = boat_layernorm_backward_impl((boat_layernorm_t*)op->layer, op->saved[0], op->saved[1], op->saved[2], dy);
+            if (dx && a->requires_grad) accumulate(a, dx, true);
+            else boat_tensor_free(dx);
+            break;
+        }
+        case OP_ATTENTION: {   /* :2458-2532 */
+            boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
+            if (!boat_attention_backward((boat_attention_t*)op->layer, dy, &gq, &gk, &gv)) break;
+            boat_variable_t* in[3] = {op->inputs[0], op->inputs[1], op->inputs[2]};
+            boat_tensor_t* g[3] = {gq, gk, gv};
+            for (int i = 0; i < 3; i++) {
+                if (in[i]->requires_grad) accumulate(in[i], g[i], true);
+                else boat_tensor_free(g[i]);
+            }
+            break;
+        }
+    }
+}
+
+static int by_seq_desc(const void* x, const void* y) {
+    const boat_op_t* a = *(boat_op_t* const*)x;
+    const boat_op_t* b = *(boat_op_t* const*)y;
+    return a->seq < b->seq ? 1 : a->seq > b->seq ? -1 : 0;
+}
+
+void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_output) {
+    if (!variable || !variable->requires_grad) return;
+    boat_tensor_t* seed = grad_output;
+    if (!seed) {
+        if (!bt_is_f32(variable->data)) return;
+        seed = ones_like(variable->data);   /* autodiff.c:313-338 */
+        if (!seed) return;
+    }
+    if (!variable->producer) {
+        accumulate(variable, seed, false);  /* leaf: grad += dY (autodiff.c:346-361) */
+        if (!grad_output) boat_tensor_unref(seed);
+        return;
+    }
+    /* collect the ops reachable from the root, each once */
+    const uint64_t epoch = ++g_epoch;
+    size_t n = 0, cap = 64, head = 0;
+    boat_op_t** ops = (boat_op_t**)malloc(cap * sizeof(*ops));
+    if (!ops) {
+        if (!grad_output) boat_tensor_unref(seed);
+        return;
+    }
+    variable->producer->mark = epoch;
+    ops[n++] = variable->producer;
+    while (head < n) {
+        boat_op_t* op = ops[head++];
+        for (size_t i = 0; i < op->num_inputs; i++) {
+            boat_variable_t* in = op->inputs[i];
+            if (!in || !in->requires_grad || !in->producer || in->producer->mark == epoch) continue;
+            in->producer->mark = epoch;
+            if (n == cap) {
+                boat_op_t** grown = (boat_op_t**)realloc(ops, 2 * cap * sizeof(*ops));
+                if (!grown) break;
+                ops = grown;
+                cap *= 2;
+            }
+            ops[n++] = in->producer;
+        }
+    }
+    qsort(ops, n, sizeof(*ops), by_seq_desc);
+    /* reverse recording order: every consumer of a variable runs before its producer */
+    for (size_t i = 0; i < n; i++) {
+        boat_op_t* op = ops[i];
+        const boat_tensor_t* dy = op == variable->producer ? seed : op->output->grad;
+        if (dy) backward_op(op, dy);
+    }
+    free(ops);
+    if (!grad_output) boat_tensor_unref(seed);
+}
+
+void boat_variable_backward_full(const boat_variable_t* variable) {
+    if (!variable || !variable->requires_grad) return;
+    boat_variable_backward((boat_variable_t*)variable, NULL);
+}

@@ -1,0 +1,86 @@
+/* boat_internal.h - private structures of the host side of libboat_amd (C11). */
+#ifndef BOAT_INTERNAL_H
+#define BOAT_INTERNAL_H
+
+#include "boat_api.h"
+#include "boat_hip.h"
+
+/* Payload shared by a tensor and its views (the reference shares the raw `data`
+ * pointer between a view and its parent, src/core/tensor.c:253-300). */
+typedef struct boat_storage {
+    void* host;            /* host mirror (malloc), NULL until first host access */
+    bh_buffer_t* dev;      /* device buffer, NULL until first device access */
+    size_t nbytes;
+    bool host_valid;       /* host mirror holds the current values */
+    bool dev_valid;        /* device buffer holds the current values */
+    size_t refs;
+} boat_storage_t;
+
+struct boat_tensor_t {
+    int64_t* shape;
+    size_t ndim;
+    boat_dtype_t dtype;
+    boat_device_t device;
+    boat_storage_t* st;
+    size_t nbytes;
+    size_t nelements;
+    bool is_contiguous;
+    size_t ref_count;
+    bool is_view;
+};
+
+/* device pointer for reading: uploads the host mirror first if it is the newer copy */
+const float* bt_dev_read(const boat_tensor_t* t);
+/* device pointer for a full overwrite: nothing is uploaded, the device copy becomes the current one */
+float* bt_dev_write(boat_tensor_t* t);
+/* device pointer for read-modify-write */
+float* bt_dev_rw(boat_tensor_t* t);
+/* new fp32 tensor with the shape/device of `like`, contents unspecified (to be fully written by a kernel) */
+boat_tensor_t* bt_new_like_uninit(const boat_tensor_t* like);
+boat_tensor_t* bt_new_uninit(const int64_t* shape, size_t ndim, boat_device_t device);
+bool bt_same_shape(const boat_tensor_t* a, const boat_tensor_t* b);
+bool bt_is_f32(const boat_tensor_t* t);
+
+void boat_fail(boat_error_t code, const char* fmt, ...);
+/* turns a bh_* return code into a Boat error; returns true when rc == 0 */
+bool boat_hip_ok(int rc, const char* what);
+
+/* layer internals shared between layers.c, autodiff.c and optimizer.c */
+struct boat_dense_layer_t {
+    size_t input_features, output_features;
+    boat_tensor_t* weight;
+    boat_tensor_t* bias;
+    bool use_bias;
+    boat_tensor_t* grad_weight;
+    boat_tensor_t* grad_bias;
+    boat_tensor_t* cache_input;
+};
+
+struct boat_layernorm_t {
+    boat_layernorm_config_t config;
+    boat_tensor_t* weight;
+    boat_tensor_t* bias;
+    boat_tensor_t* grad_weight;
+    boat_tensor_t* grad_bias;
+    boat_tensor_t* cache_input;
+    boat_tensor_t* cache_mean;   /* [rows] */
+    boat_tensor_t* cache_rstd;   /* [rows]; the reference's field is named cache_variance and never written */
+};
+
+struct boat_attention_t {
+    boat_attention_config_t config;
+    boat_tensor_t *weight_q, *weight_k, *weight_v, *weight_o;
+    boat_tensor_t *bias_q, *bias_k, *bias_v, *bias_o;
+    boat_tensor_t *grad_weight_q, *grad_weight_k, *grad_weight_v, *grad_weight_o;
+    boat_tensor_t *grad_bias_q, *grad_bias_k, *grad_bias_v, *grad_bias_o;
+    boat_tensor_t *cache_query, *cache_key, *cache_value;
+    boat_tensor_t *cache_q_proj, *cache_k_proj, *cache_v_proj;
+    boat_tensor_t* cache_lse;                /* [B*nh, S] row log-sum-exp, replaces the [B,nh,S,S] weights cache */
+    boat_tensor_t* cache_attention_output;   /* [B,S,H] before the output projection */
+};
+
+/* layernorm backward used by both the layer hook and the tape */
+boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
+                                            const boat_tensor_t* rstd, const boat_tensor_t* grad_output);
+
+#endif

@@ -1,0 +1,460 @@
+/* core.c - errors, memory seam and reference-counted tensors with a host mirror and a device copy.
+ *
+ * Mirrors the behaviour of src/core/tensor.c:65-300 (zero-filled creation, ref/unref, views that
+ * share their parent's payload), src/core/memory.c:46-247 (header-tracked allocation with
+ * statistics; here the `device` argument selects real HBM) and src/core/error.c:1-79.
+ */
+#include "boat_internal.h"
+
+#include <stdarg.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ errors */
+
+static _Thread_local boat_error_t g_last_error = BOAT_SUCCESS;
+static _Thread_local char g_last_message[512] = "";
+
+void boat_fail(boat_error_t code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_message, sizeof(g_last_message), fmt, ap);
+    va_end(ap);
+    g_last_error = code;
+    /* the reference reports failures on stderr and returns NULL/false (dense.c:203-217) */
+    fprintf(stderr, "Error: %s\n", g_last_message);
+}
+
+bool boat_hip_ok(int rc, const char* what) {
+    if (rc == BH_OK) return true;
+    boat_fail(rc == BH_ENOMEM ? BOAT_ERROR_OUT_OF_MEMORY : rc == BH_EINVAL ? BOAT_ERROR_INVALID_ARGUMENT : BOAT_ERROR_DEVICE,
+              "%s: %s", what, bh_last_error());
+    return false;
+}
+
+void boat_init(void) {
+    if (bh_init() != BH_OK) boat_fail(BOAT_ERROR_DEVICE, "boat_init: %s", bh_last_error());
+}
+void boat_cleanup(void) { bh_shutdown(); }
+
+const char* boat_error_string(boat_error_t error) {
+    switch (error) {
+        case BOAT_SUCCESS: return "Success";
+        case BOAT_ERROR_INVALID_ARGUMENT: return "Invalid argument";
+        case BOAT_ERROR_OUT_OF_MEMORY: return "Out of memory";
+        case BOAT_ERROR_INVALID_OPERATION: return "Invalid operation";
+        case BOAT_ERROR_DEVICE: return "Device error";
+        case BOAT_ERROR_FILE_IO: return "File I/O error";
+        case BOAT_ERROR_FORMAT: return "Format error";
+        case BOAT_ERROR_NOT_IMPLEMENTED: return "Not implemented";
+        default: return "Unknown error";
+    }
+}
+boat_error_t boat_get_last_error(void) { return g_last_error; }
+const char* boat_get_last_error_message(void) { return g_last_message; }
+void boat_set_error(boat_error_t error, const char* message) {
+    g_last_error = error;
+    snprintf(g_last_message, sizeof(g_last_message), "%s", message ? message : "");
+}
+void boat_clear_error(void) {
+    g_last_error = BOAT_SUCCESS;
+    g_last_message[0] = 0;
+}
+bool boat_has_error(void) { return g_last_error != BOAT_SUCCESS; }
+void boat_hip_synchronize(void) { boat_hip_ok(bh_synchronize(), "boat_hip_synchronize"); }
+
+/* ------------------------------------------------------------------ memory */
+
+#define BOAT_MEM_MAGIC 0xB0A7A11Cu
+typedef struct {
+    uint32_t magic;
+    uint32_t device;
+    size_t size;
+} mem_header_t;
+
+static boat_memory_stats_t g_stats;
+
+static void stats_alloc(size_t size) {
+    g_stats.allocated_bytes += size;
+    g_stats.allocated_blocks++;
+    size_t live = g_stats.allocated_bytes - g_stats.freed_bytes;
+    if (live > g_stats.peak_allocated_bytes) g_stats.peak_allocated_bytes = live;
+}
+static void stats_free(size_t size) {
+    g_stats.freed_bytes += size;
+    g_stats.freed_blocks++;
+}
+
+/* device blocks handed out through the memory seam, so boat_memory_free can tell them apart */
+static struct { void* ptr; size_t size; }* g_dev_blocks = NULL;
+static size_t g_dev_count = 0, g_dev_cap = 0;
+
+static void* device_block_alloc(size_t size) {
+    void* p = bh_malloc(size);
+    if (!p) {
+        boat_fail(BOAT_ERROR_OUT_OF_MEMORY, "device allocation of %zu bytes failed: %s", size, bh_last_error());
+        return NULL;
+    }
+    if (g_dev_count == g_dev_cap) {
+        size_t cap = g_dev_cap ? g_dev_cap * 2 : 16;
+        void* grown = realloc(g_dev_blocks, cap * sizeof(*g_dev_blocks));
+        if (!grown) {
+            bh_free(p);
+            return NULL;
+        }
+        g_dev_blocks = grown;
+        g_dev_cap = cap;
+    }
+    g_dev_blocks[g_dev_count].ptr = p;
+    g_dev_blocks[g_dev_count].size = size;
+    g_dev_count++;
+    stats_alloc(size);
+    return p;
+}
+static bool device_block_free(void* ptr) {
+    for (size_t i = 0; i < g_dev_count; i++) {
+        if (g_dev_blocks[i].ptr == ptr) {
+            stats_free(g_dev_blocks[i].size);
+            bh_free(ptr);
+            g_dev_blocks[i] = g_dev_blocks[--g_dev_count];
+            return true;
+        }
+    }
+    return false;
+}
+
+void* boat_memory_allocate(size_t size, boat_device_t device, const char* file, int line) {
+    (void)file;
+    (void)line;
+    if (device == BOAT_DEVICE_HIP) return device_block_alloc(size);
+    mem_header_t* h = (mem_header_t*)malloc(sizeof(mem_header_t) + size);
+    if (!h) return NULL;
+    h->magic = BOAT_MEM_MAGIC;
+    h->device = (uint32_t)device;
+    h->size = size;
+    stats_alloc(size);
+    return h + 1;
+}
+void* boat_memory_allocate_zero(size_t size, boat_device_t device, const char* file, int line) {
+    void* p = boat_memory_allocate(size, device, file, line);
+    if (p) boat_memory_set(p, 0, size, device);
+    return p;
+}
+void boat_memory_free(void* ptr) {
+    if (!ptr) return;
+    if (device_block_free(ptr)) return;
+    mem_header_t* h = (mem_header_t*)ptr - 1;
+    if (h->magic != BOAT_MEM_MAGIC) {
+        boat_fail(BOAT_ERROR_INVALID_ARGUMENT, "boat_memory_free: pointer %p was not allocated by boat_memory_allocate", ptr);
+        return;
+    }
+    h->magic = 0;
+    stats_free(h->size);
+    free(h);
+}
+void* boat_memory_allocate_device(size_t size, boat_device_t device, const char* file, int line) {
+    return boat_memory_allocate(size, device, file, line);
+}
+void boat_memory_free_device(void* ptr, boat_device_t device) {
+    (void)device;
+    boat_memory_free(ptr);
+}
+void boat_memory_copy(void* dest, const void* src, size_t size, boat_device_t dest_device, boat_device_t src_device) {
+    if (!dest || !src || size == 0) return;
+    const bool dd = dest_device == BOAT_DEVICE_HIP, sd = src_device == BOAT_DEVICE_HIP;
+    if (!dd && !sd) memcpy(dest, src, size);
+    else if (dd && !sd) boat_hip_ok(bh_memcpy_h2d(dest, src, size), "boat_memory_copy");
+    else if (!dd && sd) boat_hip_ok(bh_memcpy_d2h(dest, src, size), "boat_memory_copy");
+    else boat_hip_ok(bh_memcpy_d2d(dest, src, size), "boat_memory_copy");
+}
+void boat_memory_set(void* dest, int value, size_t size, boat_device_t device) {
+    if (!dest || size == 0) return;
+    if (device != BOAT_DEVICE_HIP) {
+        memset(dest, value, size);
+        return;
+    }
+    if (value == 0) {
+        boat_hip_ok(bh_memset_zero(dest, size), "boat_memory_set");
+    } else {
+        void* tmp = malloc(size);
+        if (!tmp) return;
+        memset(tmp, value, size);
+        boat_hip_ok(bh_memcpy_h2d(dest, tmp, size), "boat_memory_set");
+        free(tmp);
+    }
+}
+boat_memory_stats_t boat_memory_get_stats(void) { return g_stats; }
+void boat_memory_reset_stats(void) { memset(&g_stats, 0, sizeof(g_stats)); }
+void boat_memory_print_stats(FILE* stream) {
+    if (!stream) stream = stdout;
+    fprintf(stream, "Memory: allocated %zu B in %zu blocks, freed %zu B in %zu blocks, peak %zu B; device in use %zu B, cached %zu B\n",
+            g_stats.allocated_bytes, g_stats.allocated_blocks, g_stats.freed_bytes, g_stats.freed_blocks,
+            g_stats.peak_allocated_bytes, bh_bytes_in_use(), bh_bytes_cached());
+}
+
+/* ------------------------------------------------------------------ tensor */
+
+size_t boat_dtype_size(boat_dtype_t dtype) {
+    switch (dtype) {
+        case BOAT_DTYPE_FLOAT64: return 8;
+        case BOAT_DTYPE_FLOAT32: return 4;
+        case BOAT_DTYPE_FLOAT16: return 2;
+        case BOAT_DTYPE_FLOAT8: return 1;
+        case BOAT_DTYPE_FLOAT4: return 1;
+        case BOAT_DTYPE_INT64: return 8;
+        case BOAT_DTYPE_INT32: return 4;
+        case BOAT_DTYPE_UINT8: return 1;
+        case BOAT_DTYPE_BITS2: return 1;
+        case BOAT_DTYPE_BITS1: return 1;
+        case BOAT_DTYPE_BOOL: return sizeof(bool);
+        default: return 0;
+    }
+}
+const char* boat_dtype_name(boat_dtype_t dtype) {
+    static const char* names[] = {"float64", "float32", "float16", "float8", "float4", "int64",
+                                  "int32", "uint8", "bits2", "bits1", "bool"};
+    return (int)dtype >= 0 && dtype < BOAT_DTYPE_COUNT ? names[dtype] : "unknown";
+}
+
+static boat_tensor_t* tensor_alloc(const int64_t* shape, size_t ndim, boat_dtype_t dtype, boat_device_t device,
+                                   boat_storage_t* share) {
+    if (ndim > BOAT_MAX_DIMS || (ndim > 0 && !shape)) return NULL;
+    if ((int)dtype < 0 || dtype >= BOAT_DTYPE_COUNT) return NULL;
+    size_t n = 1;
+    for (size_t i = 0; i < ndim; i++) {
+        if (shape[i] < 0) return NULL;
+        n *= (size_t)shape[i];
+    }
+    boat_tensor_t* t = (boat_tensor_t*)calloc(1, sizeof(*t));
+    if (!t) return NULL;
+    t->shape = (int64_t*)malloc(sizeof(int64_t) * (ndim ? ndim : 1));
+    if (!t->shape) {
+        free(t);
+        return NULL;
+    }
+    if (ndim) memcpy(t->shape, shape, sizeof(int64_t) * ndim);
+    t->ndim = ndim;
+    t->dtype = dtype;
+    t->device = device;
+    t->nelements = n;
+    t->nbytes = n * boat_dtype_size(dtype);
+    t->is_contiguous = true;
+    t->ref_count = 1;
+    if (share) {
+        t->st = share;
+        share->refs++;
+        t->is_view = true;
+    } else {
+        boat_storage_t* st = (boat_storage_t*)calloc(1, sizeof(*st));
+        if (!st) {
+            free(t->shape);
+            free(t);
+            return NULL;
+        }
+        st->nbytes = t->nbytes;
+        st->refs = 1;
+        t->st = st;   /* neither copy valid yet == logically all zeros (tensor.c:132 zero-fills) */
+        stats_alloc(t->nbytes);
+    }
+    return t;
+}
+
+static void storage_unref(boat_storage_t* st) {
+    if (--st->refs > 0) return;
+    free(st->host);
+    if (st->dev) bh_buffer_unref(st->dev);
+    stats_free(st->nbytes);
+    free(st);
+}
+
+boat_tensor_t* boat_tensor_create(const int64_t* shape, size_t ndim, boat_dtype_t dtype, boat_device_t device) {
+    if ((int)device < 0 || device >= BOAT_DEVICE_COUNT) return NULL;
+    return tensor_alloc(shape, ndim, dtype, device, NULL);
+}
+boat_tensor_t* boat_tensor_create_like(const boat_tensor_t* other) {
+    if (!other) return NULL;
+    return boat_tensor_create(other->shape, other->ndim, other->dtype, other->device);
+}
+boat_tensor_t* bt_new_uninit(const int64_t* shape, size_t ndim, boat_device_t device) {
+    return boat_tensor_create(shape, ndim, BOAT_DTYPE_FLOAT32, device);
+}
+boat_tensor_t* bt_new_like_uninit(const boat_tensor_t* like) {
+    return like ? boat_tensor_create(like->shape, like->ndim, BOAT_DTYPE_FLOAT32, like->device) : NULL;
+}
+
+static bool storage_host_ready(boat_storage_t* st) {
+    if (!st->host) {
+        st->host = calloc(1, st->nbytes ? st->nbytes : 1);
+        if (!st->host) return false;
+        if (!st->dev_valid) st->host_valid = true;   /* zero state */
+    }
+    if (!st->host_valid) {
+        if (st->dev_valid) {
+            if (!boat_hip_ok(bh_memcpy_d2h(st->host, bh_buffer_ptr(st->dev), st->nbytes), "tensor download")) return false;
+        } else {
+            memset(st->host, 0, st->nbytes);
+        }
+        st->host_valid = true;
+    }
+    return true;
+}
+
+static bool storage_dev_ready(boat_storage_t* st, bool need_contents) {
+    if (!st->dev) {
+        const bool zero = need_contents && !st->host_valid;
+        st->dev = bh_buffer_create(st->nbytes ? st->nbytes : 4, zero);
+        if (!st->dev) {
+            boat_fail(BOAT_ERROR_OUT_OF_MEMORY, "device allocation of %zu bytes failed: %s", st->nbytes, bh_last_error());
+            return false;
+        }
+        if (zero) st->dev_valid = true;
+    }
+    if (need_contents && !st->dev_valid) {
+        if (st->host_valid) {
+            if (!boat_hip_ok(bh_memcpy_h2d(bh_buffer_ptr(st->dev), st->host, st->nbytes), "tensor upload")) return false;
+        } else {
+            if (!boat_hip_ok(bh_memset_zero(bh_buffer_ptr(st->dev), st->nbytes), "tensor zero fill")) return false;
+        }
+        st->dev_valid = true;
+    }
+    return true;
+}
+
+const float* bt_dev_read(const boat_tensor_t* t) {
+    if (!t || !storage_dev_ready(t->st, true)) return NULL;
+    return (const float*)bh_buffer_ptr(t->st->dev);
+}
+float* bt_dev_write(boat_tensor_t* t) {
+    if (!t) return NULL;
+    /* a view covers its whole parent payload (reshape only), so a full overwrite is still full */
+    if (!storage_dev_ready(t->st, false)) return NULL;
+    t->st->dev_valid = true;
+    t->st->host_valid = false;
+    return (float*)bh_buffer_ptr(t->st->dev);
+}
+float* bt_dev_rw(boat_tensor_t* t) {
+    if (!t || !storage_dev_ready(t->st, true)) return NULL;
+    t->st->host_valid = false;
+    return (float*)bh_buffer_ptr(t->st->dev);
+}
+
+boat_tensor_t* boat_tensor_from_data(const int64_t* shape, size_t ndim, boat_dtype_t dtype, const void* data) {
+    boat_tensor_t* t = boat_tensor_create(shape, ndim, dtype, BOAT_DEVICE_CPU);
+    if (!t) return NULL;
+    if (data) {
+        void* dst = boat_tensor_data(t);
+        if (!dst) {
+            boat_tensor_free(t);
+            return NULL;
+        }
+        memcpy(dst, data, t->nbytes);
+    }
+    return t;
+}
+
+void boat_tensor_free(boat_tensor_t* tensor) {
+    if (!tensor) return;
+    if (--tensor->ref_count == 0) {
+        storage_unref(tensor->st);
+        free(tensor->shape);
+        free(tensor);
+    }
+}
+void boat_tensor_ref(boat_tensor_t* tensor) {
+    if (tensor) tensor->ref_count++;
+}
+void boat_tensor_unref(boat_tensor_t* tensor) { boat_tensor_free(tensor); }
+
+const int64_t* boat_tensor_shape(const boat_tensor_t* t) { return t ? t->shape : NULL; }
+size_t boat_tensor_ndim(const boat_tensor_t* t) { return t ? t->ndim : 0; }
+boat_dtype_t boat_tensor_dtype(const boat_tensor_t* t) { return t ? t->dtype : BOAT_DTYPE_FLOAT32; }
+boat_device_t boat_tensor_device(const boat_tensor_t* t) { return t ? t->device : BOAT_DEVICE_CPU; }
+size_t boat_tensor_nbytes(const boat_tensor_t* t) { return t ? t->nbytes : 0; }
+size_t boat_tensor_nelements(const boat_tensor_t* t) { return t ? t->nelements : 0; }
+bool boat_tensor_is_contiguous(const boat_tensor_t* t) { return t ? t->is_contiguous : false; }
+
+void* boat_tensor_data(const boat_tensor_t* tensor) {
+    if (!tensor) return NULL;
+    boat_storage_t* st = tensor->st;
+    if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_rw((boat_tensor_t*)tensor);
+    if (!storage_host_ready(st)) return NULL;
+    st->dev_valid = false;   /* the caller may write through the pointer */
+    return st->host;
+}
+const void* boat_tensor_const_data(const boat_tensor_t* tensor) {
+    if (!tensor) return NULL;
+    if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_read(tensor);
+    if (!storage_host_ready(tensor->st)) return NULL;
+    return tensor->st->host;
+}
+
+boat_tensor_t* boat_tensor_reshape(const boat_tensor_t* tensor, const int64_t* new_shape, size_t new_ndim) {
+    if (!tensor || !new_shape) return NULL;
+    size_t n = 1;
+    for (size_t i = 0; i < new_ndim; i++) n *= (size_t)new_shape[i];
+    if (n != tensor->nelements) {
+        fprintf(stderr, "Error: Reshape element count mismatch: %zu != %zu\n", n, tensor->nelements);
+        return NULL;
+    }
+    boat_tensor_t* v = tensor_alloc(new_shape, new_ndim, tensor->dtype, tensor->device, tensor->st);
+    if (v) v->is_contiguous = false;   /* the reference marks reshaped views so (tensor.c:289) */
+    return v;
+}
+
+boat_tensor_t* boat_tensor_clone(const boat_tensor_t* tensor) {
+    if (!tensor) return NULL;
+    boat_tensor_t* c = boat_tensor_create_like(tensor);
+    if (!c) return NULL;
+    boat_storage_t* st = tensor->st;
+    if (st->dev_valid) {
+        float* dst = bt_dev_write(c);
+        if (!dst || !boat_hip_ok(bh_memcpy_d2d(dst, bh_buffer_ptr(st->dev), tensor->nbytes), "boat_tensor_clone")) {
+            boat_tensor_free(c);
+            return NULL;
+        }
+    } else if (st->host_valid) {
+        void* dst = boat_tensor_data(c);
+        if (!dst) {
+            boat_tensor_free(c);
+            return NULL;
+        }
+        memcpy(dst, st->host, tensor->nbytes);
+    }
+    return c;
+}
+
+boat_tensor_t* boat_tensor_to_device(const boat_tensor_t* tensor, boat_device_t dev) {
+    if (!tensor || (int)dev < 0 || dev >= BOAT_DEVICE_COUNT) return NULL;
+    boat_tensor_t* out = boat_tensor_create(tensor->shape, tensor->ndim, tensor->dtype, dev);
+    if (!out) return NULL;
+    boat_storage_t* src = tensor->st;
+    if (!src->dev_valid && !src->host_valid) return out;   /* zeros */
+    if (dev == BOAT_DEVICE_HIP) {
+        float* dst = bt_dev_write(out);
+        bool ok = dst != NULL;
+        if (ok && src->dev_valid) ok = boat_hip_ok(bh_memcpy_d2d(dst, bh_buffer_ptr(src->dev), tensor->nbytes), "boat_tensor_to_device");
+        else if (ok) ok = boat_hip_ok(bh_memcpy_h2d(dst, src->host, tensor->nbytes), "boat_tensor_to_device");
+        if (!ok) {
+            boat_tensor_free(out);
+            return NULL;
+        }
+    } else {
+        void* dst = boat_tensor_data(out);
+        bool ok = dst != NULL;
+        if (ok && src->host_valid) memcpy(dst, src->host, tensor->nbytes);
+        else if (ok) ok = boat_hip_ok(bh_memcpy_d2h(dst, bh_buffer_ptr(src->dev), tensor->nbytes), "boat_tensor_to_device");
+        if (!ok) {
+            boat_tensor_free(out);
+            return NULL;
+        }
+    }
+    return out;
+}
+
+bool bt_same_shape(const boat_tensor_t* a, const boat_tensor_t* b) {
+    if (!a || !b || a->ndim != b->ndim) return false;
+    for (size_t i = 0; i < a->ndim; i++)
+        if (a->shape[i] != b->shape[i]) return false;
+    return true;
+}
+bool bt_is_f32(const boat_tensor_t* t) { return t && t->dtype == BOAT_DTYPE_FLOAT32; }

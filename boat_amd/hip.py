@@ -1,0 +1,158 @@
+"""ctypes binding of the device layer's C-ABI (include/boat_hip.h) plus a tiny device-array helper.
+
+Everything here runs on the GPU through libboat_amd.so; importing the module loads the
+library and fails loudly if it has not been built.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from .capi import LIB_PATH
+
+P = C.c_void_p
+F = C.c_float
+I = C.c_int
+L = C.c_int64
+Z = C.c_size_t
+
+if not LIB_PATH.exists():
+    raise FileNotFoundError(f"{LIB_PATH} not found: build it first (python -m boat_amd.build); there is no host fallback")
+lib = C.CDLL(str(LIB_PATH), mode=C.RTLD_LOCAL)
+
+_SIGS = {
+    "bh_init": (I, []), "bh_shutdown": (I, []), "bh_synchronize": (I, []),
+    "bh_last_error": (C.c_char_p, []), "bh_device_name": (C.c_char_p, []), "bh_device_cu_count": (I, []),
+    "bh_stream": (P, []),
+    "bh_malloc": (P, [Z]), "bh_free": (None, [P]), "bh_cache_release": (I, []),
+    "bh_bytes_in_use": (Z, []), "bh_bytes_cached": (Z, []),
+    "bh_buffer_create": (P, [Z, I]), "bh_buffer_ref": (None, [P]), "bh_buffer_unref": (None, [P]),
+    "bh_buffer_ptr": (P, [P]), "bh_buffer_nbytes": (Z, [P]), "bh_buffer_refcount": (I, [P]),
+    "bh_memcpy_h2d": (I, [P, P, Z]), "bh_memcpy_d2h": (I, [P, P, Z]), "bh_memcpy_d2d": (I, [P, P, Z]),
+    "bh_memset_zero": (I, [P, Z]),
+    "bh_event_create": (P, []), "bh_event_destroy": (None, [P]), "bh_event_record": (I, [P]),
+    "bh_event_elapsed_ms": (F, [P, P]),
+    "bh_fill": (I, [P, F, L]),
+    "bh_add_inplace": (I, [P, P, L]),
+    "bh_binary": (I, [I, P, P, P, L]),
+    "bh_binary_broadcast": (I, [I, P, C.POINTER(L), P, C.POINTER(L), P, C.POINTER(L), I]),
+    "bh_scalar_op": (I, [I, P, F, P, L]),
+    "bh_div_backward_b": (I, [P, P, P, P, L]),
+    "bh_activation_forward": (I, [I, P, P, L]),
+    "bh_activation_backward": (I, [I, P, P, P, L, I]),
+    "bh_bias_add_rows": (I, [P, P, L, L]),
+    "bh_mse_grad": (I, [P, P, P, L]), "bh_mse_loss": (I, [P, P, P, L]),
+    "bh_sgd_update": (I, [P, P, F, L, I]),
+    "bh_sum_all": (I, [P, P, L]),
+    "bh_colsum": (I, [P, P, L, L, I]),
+    "bh_softmax_forward": (I, [P, P, L, L]), "bh_softmax_backward": (I, [P, P, P, L, L]),
+    "bh_log_softmax_forward": (I, [P, P, L, L]), "bh_log_softmax_backward": (I, [P, P, P, L, L]),
+    "bh_softmax_ce_grad": (I, [P, P, P, P, L, L]),
+    "bh_layernorm_forward": (I, [P, P, P, P, P, P, L, L, F]),
+    "bh_layernorm_backward": (I, [P, P, P, P, P, P, P, P, L, L, I]),
+    "bh_gemm": (I, [I, I, L, L, L, P, L, P, L, P, L, P, I, L]),
+    "bh_gemm_force_config": (I, [I]),
+    "bh_transpose_last2": (I, [P, P, L, L, L]),
+    "bh_dense_backward": (I, [P, P, P, P, P, P, L, L, L, I]),
+    "bh_sdpa_forward": (I, [P, P, P, F, I, P, P, P, L, L, L]),
+    "bh_sdpa_backward": (I, [P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
+    "bh_sdpa_force_general": (I, [I]),
+    "bh_adam_update": (I, [P, P, P, P, L, F, F, F, F, L]),
+    "bh_adam_update_multi": (I, [C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(L), I, F, F, F, F, L]),
+}
+for _name, (_res, _args) in _SIGS.items():
+    _fn = getattr(lib, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args
+    globals()[_name] = _fn
+
+ACT_RELU, ACT_SIGMOID, ACT_TANH, ACT_GELU = 0, 1, 2, 3
+
+
+class HipError(RuntimeError):
+    pass
+
+
+def check(rc: int, what: str = "") -> None:
+    if rc != 0:
+        raise HipError(f"{what or 'device call'} failed ({rc}): {lib.bh_last_error().decode()}")
+
+
+class DeviceArray:
+    """A dense row-major array in HBM (fp32 unless told otherwise); freed when collected."""
+
+    def __init__(self, shape, dtype=np.float32, zero: bool = False):
+        self.shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        self.ptr = lib.bh_malloc(max(self.nbytes, 4))
+        if not self.ptr:
+            raise HipError(f"bh_malloc({self.nbytes}) failed: {lib.bh_last_error().decode()}")
+        if zero:
+            check(lib.bh_memset_zero(self.ptr, self.nbytes), "memset")
+
+    @classmethod
+    def from_numpy(cls, a) -> "DeviceArray":
+        a = np.ascontiguousarray(a)
+        d = cls(a.shape, a.dtype)
+        if a.nbytes:
+            check(lib.bh_memcpy_h2d(d.ptr, a.ctypes.data, a.nbytes), "h2d")
+        return d
+
+    def numpy(self) -> np.ndarray:
+        out = np.empty(self.shape, dtype=self.dtype)
+        if self.nbytes:
+            check(lib.bh_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes), "d2h")
+        return out
+
+    def __del__(self):
+        try:
+            if getattr(self, "ptr", None):
+                lib.bh_free(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+def to_device(a) -> DeviceArray:
+    return DeviceArray.from_numpy(a)
+
+
+def empty(shape, dtype=np.float32) -> DeviceArray:
+    return DeviceArray(shape, dtype)
+
+
+def zeros(shape, dtype=np.float32) -> DeviceArray:
+    return DeviceArray(shape, dtype, zero=True)
+
+
+def synchronize() -> None:
+    check(lib.bh_synchronize(), "synchronize")
+
+
+class Timer:
+    """Times work enqueued on the library stream with HIP events."""
+
+    def __init__(self):
+        self.start = lib.bh_event_create()
+        self.stop = lib.bh_event_create()
+        if not self.start or not self.stop:
+            raise HipError("event creation failed")
+
+    def __enter__(self):
+        check(lib.bh_event_record(self.start), "event record")
+        return self
+
+    def __exit__(self, *exc):
+        check(lib.bh_event_record(self.stop), "event record")
+        self.ms = float(lib.bh_event_elapsed_ms(self.start, self.stop))
+        return False
+
+    def __del__(self):
+        try:
+            lib.bh_event_destroy(self.start)
+            lib.bh_event_destroy(self.stop)
+        except Exception:
+            pass

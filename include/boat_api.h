@@ -1,0 +1,334 @@
+/* boat_api.h - the part of Boat's public C API that lies on the training hot path, as exported
+ * by libboat_amd.so.  Names, argument meaning, ownership and error conventions are those of the
+ * reference headers cited beside each group, so a program written against them links unchanged;
+ * all arithmetic behind them runs on the GPU through boat_hip.h (there is no host fallback).
+ *
+ * Host/device coherence.  A tensor created with BOAT_DEVICE_CPU keeps a host mirror and a device
+ * copy with ownership flags: kernels upload a dirty host mirror before use, and
+ * boat_tensor_data()/boat_tensor_const_data() wait for the stream and download a dirty device copy
+ * before returning the host pointer (boat_tensor_data() also hands ownership to the host, since the
+ * caller may write).  A host pointer is therefore valid until the next Boat call that takes the
+ * tensor; fetch it again afterwards.  A tensor created with BOAT_DEVICE_CUDA (the reference's only
+ * GPU slot, value 1; alias BOAT_DEVICE_HIP) lives in HBM only and boat_tensor_data() returns the
+ * device pointer.
+ *
+ * Only fp32 tensors take part in arithmetic, as on the reference's hot path.
+ */
+#ifndef BOAT_API_H
+#define BOAT_API_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BOAT_API __attribute__((visibility("default")))
+
+/* ---- include/boat/tensor.h:18-110 ---- */
+typedef struct boat_tensor_t boat_tensor_t;
+
+typedef enum {
+    BOAT_DTYPE_FLOAT64, BOAT_DTYPE_FLOAT32, BOAT_DTYPE_FLOAT16, BOAT_DTYPE_FLOAT8, BOAT_DTYPE_FLOAT4,
+    BOAT_DTYPE_INT64, BOAT_DTYPE_INT32, BOAT_DTYPE_UINT8, BOAT_DTYPE_BITS2, BOAT_DTYPE_BITS1,
+    BOAT_DTYPE_BOOL, BOAT_DTYPE_COUNT
+} boat_dtype_t;
+
+enum boat_device_enum { BOAT_DEVICE_CPU, BOAT_DEVICE_CUDA, BOAT_DEVICE_COUNT };
+typedef enum boat_device_enum boat_device_t;
+#define BOAT_DEVICE_HIP BOAT_DEVICE_CUDA   /* same ABI value: the one GPU slot of tensor.h:50-55 */
+#define BOAT_MAX_DIMS 8
+
+BOAT_API boat_tensor_t* boat_tensor_create(const int64_t* shape, size_t ndim, boat_dtype_t dtype, boat_device_t device);
+BOAT_API boat_tensor_t* boat_tensor_create_like(const boat_tensor_t* other);
+BOAT_API boat_tensor_t* boat_tensor_from_data(const int64_t* shape, size_t ndim, boat_dtype_t dtype, const void* data);
+BOAT_API void boat_tensor_free(boat_tensor_t* tensor);
+BOAT_API void boat_tensor_ref(boat_tensor_t* tensor);
+BOAT_API void boat_tensor_unref(boat_tensor_t* tensor);
+BOAT_API const int64_t* boat_tensor_shape(const boat_tensor_t* tensor);
+BOAT_API size_t boat_tensor_ndim(const boat_tensor_t* tensor);
+BOAT_API boat_dtype_t boat_tensor_dtype(const boat_tensor_t* tensor);
+BOAT_API boat_device_t boat_tensor_device(const boat_tensor_t* tensor);
+BOAT_API size_t boat_tensor_nbytes(const boat_tensor_t* tensor);
+BOAT_API size_t boat_tensor_nelements(const boat_tensor_t* tensor);
+BOAT_API bool boat_tensor_is_contiguous(const boat_tensor_t* tensor);
+BOAT_API void* boat_tensor_data(const boat_tensor_t* tensor);
+BOAT_API const void* boat_tensor_const_data(const boat_tensor_t* tensor);
+BOAT_API boat_tensor_t* boat_tensor_reshape(const boat_tensor_t* tensor, const int64_t* new_shape, size_t new_ndim);
+BOAT_API boat_tensor_t* boat_tensor_to_device(const boat_tensor_t* tensor, boat_device_t dev);   /* declared only in the reference (tensor.h:92) */
+BOAT_API boat_tensor_t* boat_tensor_clone(const boat_tensor_t* tensor);
+BOAT_API size_t boat_dtype_size(boat_dtype_t dtype);
+BOAT_API const char* boat_dtype_name(boat_dtype_t dtype);
+
+/* ---- include/boat/memory.h:17-55 ---- */
+typedef struct {
+    size_t allocated_bytes;
+    size_t allocated_blocks;
+    size_t peak_allocated_bytes;
+    size_t freed_bytes;
+    size_t freed_blocks;
+} boat_memory_stats_t;
+
+BOAT_API void* boat_memory_allocate(size_t size, boat_device_t device, const char* file, int line);
+BOAT_API void* boat_memory_allocate_zero(size_t size, boat_device_t device, const char* file, int line);
+BOAT_API void boat_memory_free(void* ptr);
+BOAT_API void* boat_memory_allocate_device(size_t size, boat_device_t device, const char* file, int line);
+BOAT_API void boat_memory_free_device(void* ptr, boat_device_t device);
+BOAT_API void boat_memory_copy(void* dest, const void* src, size_t size, boat_device_t dest_device, boat_device_t src_device);
+BOAT_API void boat_memory_set(void* dest, int value, size_t size, boat_device_t device);
+BOAT_API boat_memory_stats_t boat_memory_get_stats(void);
+BOAT_API void boat_memory_reset_stats(void);
+BOAT_API void boat_memory_print_stats(FILE* stream);
+
+/* ---- include/boat.h:64-94 (error reporting; declared there, mostly undefined in the reference) ---- */
+typedef enum {
+    BOAT_SUCCESS = 0, BOAT_ERROR_INVALID_ARGUMENT, BOAT_ERROR_OUT_OF_MEMORY, BOAT_ERROR_INVALID_OPERATION,
+    BOAT_ERROR_DEVICE, BOAT_ERROR_FILE_IO, BOAT_ERROR_FORMAT, BOAT_ERROR_NOT_IMPLEMENTED, BOAT_ERROR_UNKNOWN
+} boat_error_t;
+BOAT_API void boat_init(void);
+BOAT_API void boat_cleanup(void);
+BOAT_API const char* boat_error_string(boat_error_t error);
+BOAT_API boat_error_t boat_get_last_error(void);
+BOAT_API const char* boat_get_last_error_message(void);
+BOAT_API void boat_set_error(boat_error_t error, const char* message);
+BOAT_API void boat_clear_error(void);
+BOAT_API bool boat_has_error(void);
+
+/* ---- include/boat/ops.h:15-60 (the ops the backward pass is built from) ---- */
+BOAT_API boat_tensor_t* boat_add(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_sub(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_mul(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_div(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API void boat_add_(boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API void boat_sub_(boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API void boat_mul_(boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API void boat_div_(boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_add_scalar(const boat_tensor_t* a, double scalar);
+BOAT_API boat_tensor_t* boat_sub_scalar(const boat_tensor_t* a, double scalar);
+BOAT_API boat_tensor_t* boat_mul_scalar(const boat_tensor_t* a, double scalar);
+BOAT_API boat_tensor_t* boat_div_scalar(const boat_tensor_t* a, double scalar);
+BOAT_API boat_tensor_t* boat_matmul(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_dot(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1);
+BOAT_API boat_tensor_t* boat_relu(const boat_tensor_t* a);
+BOAT_API boat_tensor_t* boat_sigmoid(const boat_tensor_t* a);
+BOAT_API boat_tensor_t* boat_tanh(const boat_tensor_t* a);
+BOAT_API boat_tensor_t* boat_softmax(const boat_tensor_t* a, int axis);
+BOAT_API boat_tensor_t* boat_log_softmax(const boat_tensor_t* a, int axis);
+BOAT_API boat_tensor_t* boat_gelu(const boat_tensor_t* a);                          /* stub in the reference (src/ops/activation.c:298-302) */
+BOAT_API boat_tensor_t* boat_sum(const boat_tensor_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
+BOAT_API boat_tensor_t* boat_mean(const boat_tensor_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
+
+/* ---- include/boat/autodiff.h:15-98 ---- */
+typedef struct boat_variable_t boat_variable_t;
+typedef struct boat_autodiff_context_t boat_autodiff_context_t;
+struct boat_dense_layer_t;
+struct boat_attention_t;
+
+BOAT_API boat_variable_t* boat_variable_create(boat_tensor_t* tensor, bool requires_grad);
+BOAT_API boat_variable_t* boat_variable_create_with_shape(const int64_t* shape, size_t ndim, boat_dtype_t dtype, bool requires_grad);
+BOAT_API void boat_variable_free(const boat_variable_t* variable);
+BOAT_API boat_tensor_t* boat_variable_data(const boat_variable_t* variable);
+BOAT_API boat_tensor_t* boat_variable_grad(const boat_variable_t* variable);
+BOAT_API bool boat_variable_requires_grad(const boat_variable_t* variable);
+BOAT_API void boat_variable_set_requires_grad(boat_variable_t* variable, bool requires_grad);
+BOAT_API bool boat_variable_reset_data(boat_variable_t* variable, boat_tensor_t* new_tensor);
+BOAT_API void boat_variable_zero_grad(boat_variable_t* variable);
+BOAT_API void boat_variable_retain_grad(const boat_variable_t* variable, bool retain);
+BOAT_API void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_output);
+BOAT_API void boat_variable_backward_full(const boat_variable_t* variable);
+BOAT_API boat_variable_t* boat_var_add(const boat_variable_t* a, const boat_variable_t* b);
+BOAT_API boat_variable_t* boat_var_sub(const boat_variable_t* a, const boat_variable_t* b);
+BOAT_API boat_variable_t* boat_var_mul(const boat_variable_t* a, const boat_variable_t* b);
+BOAT_API boat_variable_t* boat_var_div(const boat_variable_t* a, const boat_variable_t* b);
+BOAT_API boat_variable_t* boat_var_matmul(const boat_variable_t* a, const boat_variable_t* b);
+BOAT_API boat_variable_t* boat_var_dot(const boat_variable_t* a, const boat_variable_t* b);
+BOAT_API boat_variable_t* boat_var_flatten(const boat_variable_t* input);
+BOAT_API boat_variable_t* boat_var_dense(const boat_variable_t* input, const struct boat_dense_layer_t* layer);
+BOAT_API boat_variable_t* boat_var_attention(const boat_variable_t* query, const boat_variable_t* key, const boat_variable_t* value,
+                                             const struct boat_attention_t* attention, const boat_tensor_t* attention_mask);
+BOAT_API boat_variable_t* boat_var_relu(const boat_variable_t* a);
+BOAT_API boat_variable_t* boat_var_sigmoid(const boat_variable_t* a);
+BOAT_API boat_variable_t* boat_var_tanh(const boat_variable_t* a);
+BOAT_API boat_variable_t* boat_var_softmax(const boat_variable_t* a, int axis);
+BOAT_API boat_variable_t* boat_var_log_softmax(const boat_variable_t* a, int axis);
+BOAT_API boat_variable_t* boat_var_sum(const boat_variable_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
+BOAT_API boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim);
+BOAT_API boat_autodiff_context_t* boat_autodiff_context_create(void);
+BOAT_API void boat_autodiff_context_free(const boat_autodiff_context_t* context);
+BOAT_API void boat_autodiff_context_enable_grad(boat_autodiff_context_t* context);
+BOAT_API void boat_autodiff_context_disable_grad(boat_autodiff_context_t* context);
+BOAT_API bool boat_autodiff_context_grad_enabled(const boat_autodiff_context_t* context);
+BOAT_API void boat_autodiff_set_current_context(const boat_autodiff_context_t* context);
+BOAT_API boat_autodiff_context_t* boat_autodiff_get_current_context(void);
+BOAT_API void boat_autodiff_clear_computation_graph(void);
+
+/* ---- include/boat/layers.h:23-35 (dense) ---- */
+typedef struct boat_dense_layer_t boat_dense_layer_t;
+BOAT_API boat_dense_layer_t* boat_dense_layer_create(size_t input_features, size_t output_features, bool use_bias);
+BOAT_API void boat_dense_layer_free(boat_dense_layer_t* layer);
+BOAT_API boat_tensor_t* boat_dense_layer_forward(boat_dense_layer_t* layer, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_dense_layer_backward(boat_dense_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_dense_layer_update(boat_dense_layer_t* layer, float learning_rate);
+BOAT_API void boat_dense_layer_set_weight(boat_dense_layer_t* layer, boat_tensor_t* weight);
+BOAT_API void boat_dense_layer_set_bias(boat_dense_layer_t* layer, boat_tensor_t* bias);
+BOAT_API boat_tensor_t* boat_dense_layer_get_weight(const boat_dense_layer_t* layer);
+BOAT_API boat_tensor_t* boat_dense_layer_get_bias(const boat_dense_layer_t* layer);
+BOAT_API boat_tensor_t* boat_dense_layer_get_grad_weight(const boat_dense_layer_t* layer);
+BOAT_API boat_tensor_t* boat_dense_layer_get_grad_bias(const boat_dense_layer_t* layer);
+
+/* ---- include/boat/layers.h:95-107 (activation layers) ---- */
+typedef struct boat_relu_layer_t boat_relu_layer_t;
+BOAT_API boat_relu_layer_t* boat_relu_layer_create(void);
+BOAT_API void boat_relu_layer_free(boat_relu_layer_t* layer);
+BOAT_API boat_tensor_t* boat_relu_layer_forward(const boat_relu_layer_t* layer, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_relu_layer_backward(boat_relu_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_relu_layer_update(boat_relu_layer_t* layer, float learning_rate);
+typedef struct boat_softmax_layer_t boat_softmax_layer_t;
+BOAT_API boat_softmax_layer_t* boat_softmax_layer_create(int axis);
+BOAT_API void boat_softmax_layer_free(boat_softmax_layer_t* layer);
+BOAT_API boat_tensor_t* boat_softmax_layer_forward(const boat_softmax_layer_t* layer, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_softmax_layer_backward(boat_softmax_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_softmax_layer_update(boat_softmax_layer_t* layer, float learning_rate);
+
+/* ---- include/boat/layers/norm.h:15-76, include/boat/layers.h:75-79 ---- */
+typedef struct boat_layernorm_t boat_layernorm_t;
+typedef boat_layernorm_t boat_norm_layer_t;
+typedef struct {
+    size_t normalized_shape;
+    float eps;
+    bool elementwise_affine;
+    bool use_bias;
+} boat_layernorm_config_t;
+BOAT_API boat_layernorm_t* boat_layernorm_create(const boat_layernorm_config_t* config);
+BOAT_API void boat_layernorm_free(boat_layernorm_t* norm);
+BOAT_API boat_tensor_t* boat_layernorm_forward(boat_layernorm_t* norm, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_layernorm_backward(boat_layernorm_t* norm, const boat_tensor_t* grad_output);   /* stub in the reference (norm.c:397-402) */
+BOAT_API void boat_layernorm_update(boat_layernorm_t* norm, float learning_rate);                          /* stub in the reference (norm.c:411-415) */
+BOAT_API void boat_layernorm_set_weight(boat_layernorm_t* norm, boat_tensor_t* weight);
+BOAT_API void boat_layernorm_set_bias(boat_layernorm_t* norm, boat_tensor_t* bias);
+BOAT_API boat_tensor_t* boat_layer_norm_grad(const boat_tensor_t* grad_output, const boat_tensor_t* input, const boat_tensor_t* output,
+                                             const int64_t* normalized_shape, size_t normalized_shape_len, float eps);  /* stub in the reference (norm.c:450-463) */
+BOAT_API boat_norm_layer_t* boat_norm_layer_create(size_t normalized_shape, float eps, bool elementwise_affine);
+BOAT_API void boat_norm_layer_free(boat_norm_layer_t* layer);
+BOAT_API boat_tensor_t* boat_norm_layer_forward(boat_norm_layer_t* layer, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_norm_layer_backward(boat_norm_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_norm_layer_update(boat_norm_layer_t* layer, float learning_rate);
+
+/* ---- include/boat/layers/attention.h:17-107, include/boat/layers.h:82-92 ---- */
+typedef struct boat_attention_t boat_attention_t;
+typedef struct {
+    size_t hidden_size;
+    size_t num_heads;
+    size_t head_size;
+    float dropout_prob;
+    bool causal_mask;
+    bool use_bias;
+    bool use_rotary;
+    float rotary_theta;
+} boat_attention_config_t;
+BOAT_API boat_attention_t* boat_attention_create(const boat_attention_config_t* config);
+BOAT_API void boat_attention_free(boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_forward(boat_attention_t* attention, const boat_tensor_t* query, const boat_tensor_t* key,
+                                               const boat_tensor_t* value, const boat_tensor_t* attention_mask);
+BOAT_API bool boat_attention_backward(boat_attention_t* attention, const boat_tensor_t* grad_output,
+                                      boat_tensor_t** grad_query, boat_tensor_t** grad_key, boat_tensor_t** grad_value);
+BOAT_API void boat_attention_update(boat_attention_t* attention, float learning_rate);
+BOAT_API void boat_attention_set_causal(boat_attention_t* attention, bool causal);
+BOAT_API boat_tensor_t* boat_attention_get_weight_q(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_weight_k(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_weight_v(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_weight_o(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_bias_q(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_bias_k(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_bias_v(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_bias_o(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_weight_q(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_weight_k(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_weight_v(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_weight_o(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_bias_q(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_bias_k(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_bias_v(const boat_attention_t* attention);
+BOAT_API boat_tensor_t* boat_attention_get_grad_bias_o(const boat_attention_t* attention);
+typedef struct boat_attention_layer_t boat_attention_layer_t;
+BOAT_API boat_attention_layer_t* boat_attention_layer_create(size_t hidden_size, size_t num_heads, float dropout_prob, bool causal_mask);
+BOAT_API void boat_attention_layer_free(boat_attention_layer_t* layer);
+BOAT_API boat_tensor_t* boat_attention_layer_forward(boat_attention_layer_t* layer, const boat_tensor_t* query, const boat_tensor_t* key,
+                                                     const boat_tensor_t* value, const boat_tensor_t* attention_mask);
+BOAT_API boat_tensor_t* boat_attention_layer_backward(boat_attention_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_attention_layer_update(boat_attention_layer_t* layer, float learning_rate);
+
+/* ---- include/boat/optimizers.h:15-44 ---- */
+typedef enum { BOAT_OPTIMIZER_SGD, BOAT_OPTIMIZER_ADAM, BOAT_OPTIMIZER_RMSPROP, BOAT_OPTIMIZER_ADAGRAD } boat_optimizer_type_t;
+typedef struct boat_optimizer_t boat_optimizer_t;
+BOAT_API boat_optimizer_t* boat_adam_optimizer_create(float learning_rate, float beta1, float beta2, float epsilon);
+BOAT_API void boat_optimizer_step(boat_optimizer_t* optimizer);
+BOAT_API void boat_optimizer_zero_grad(boat_optimizer_t* optimizer);
+BOAT_API void boat_optimizer_free(boat_optimizer_t* optimizer);
+BOAT_API void boat_optimizer_add_parameter(boat_optimizer_t* optimizer, boat_tensor_t* param, boat_tensor_t* grad);
+BOAT_API float boat_optimizer_get_learning_rate(const boat_optimizer_t* optimizer);
+BOAT_API void boat_optimizer_set_learning_rate(boat_optimizer_t* optimizer, float learning_rate);
+
+/* ---- include/boat/model.h:17-65 ---- */
+typedef struct boat_model_t boat_model_t;
+typedef struct boat_layer_ops_t boat_layer_ops_t;
+typedef struct boat_layer_t {
+    void* data;
+    const boat_layer_ops_t* ops;
+} boat_layer_t;
+struct boat_layer_ops_t {
+    boat_tensor_t* (*forward)(const boat_layer_t* layer, const boat_tensor_t* input);
+    boat_tensor_t* (*backward)(const boat_layer_t* layer, const boat_tensor_t* grad_output);
+    void (*update)(const boat_layer_t* layer, float learning_rate);
+    void (*free)(const boat_layer_t* layer);
+};
+BOAT_API boat_model_t* boat_model_create(void);
+BOAT_API void boat_model_free(boat_model_t* model);
+BOAT_API void boat_model_add_layer(boat_model_t* model, boat_layer_t* layer);
+BOAT_API size_t boat_model_layer_count(const boat_model_t* model);
+BOAT_API boat_tensor_t* boat_model_forward(const boat_model_t* model, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_model_backward(const boat_model_t* model, const boat_tensor_t* grad_output);  /* stub in the reference (model.c:354-359) */
+BOAT_API void boat_model_update(const boat_model_t* model, float learning_rate);                          /* stub in the reference (model.c:361-365) */
+typedef boat_model_t boat_sequential_model_t;
+BOAT_API boat_sequential_model_t* boat_sequential_create(void);
+BOAT_API void boat_sequential_add(boat_sequential_model_t* model, boat_layer_t* layer);
+
+/* ---- additions with no counterpart in the reference (named boat_hip_*) ---- */
+/* wait for all queued GPU work */
+BOAT_API void boat_hip_synchronize(void);
+/* gradient tensor of a variable, created zero-filled if absent and kept across boat_variable_zero_grad
+ * (which then zero-fills in place), so it can be registered with an optimizer before the first backward */
+BOAT_API boat_tensor_t* boat_hip_variable_ensure_grad(boat_variable_t* variable);
+/* GELU with gradient tracking (exact erf form) */
+BOAT_API boat_variable_t* boat_hip_var_gelu(const boat_variable_t* a);
+/* LayerNorm with gradient tracking; dgamma/dbeta accumulate in the layer */
+BOAT_API boat_variable_t* boat_hip_var_layernorm(const boat_variable_t* a, boat_layernorm_t* norm);
+BOAT_API boat_tensor_t* boat_hip_layernorm_get_weight(const boat_layernorm_t* norm);
+BOAT_API boat_tensor_t* boat_hip_layernorm_get_bias(const boat_layernorm_t* norm);
+BOAT_API boat_tensor_t* boat_hip_layernorm_get_grad_weight(const boat_layernorm_t* norm);
+BOAT_API boat_tensor_t* boat_hip_layernorm_get_grad_bias(const boat_layernorm_t* norm);
+/* fused loss + gradient of the tape chain log_softmax -> mul(onehot) -> sum -> mul(-1/B)
+ * (examples/mnist/mnist_autodiff.c:397-522): labels is an INT32 or UINT8 tensor of class indices;
+ * returns the [1] loss tensor and, through *dlogits, (softmax(z)-onehot)/B */
+BOAT_API boat_tensor_t* boat_hip_softmax_cross_entropy(const boat_tensor_t* logits, const boat_tensor_t* labels, boat_tensor_t** dlogits);
+/* mean squared error (src/loss/mse.c:70-78) and its gradient 2(o-t)/n (tests/test_attention_training.c:28-41) */
+BOAT_API boat_tensor_t* boat_hip_mse_loss(const boat_tensor_t* pred, const boat_tensor_t* target, boat_tensor_t** grad);
+/* ready-made vtables for boat_model_add_layer (the reference ships none; callers write these wrappers,
+ * tests/test_model_graph_integration.c:8-77).  The returned boat_layer_t is freed by ops->free. */
+BOAT_API boat_layer_t* boat_hip_layer_from_dense(boat_dense_layer_t* layer);
+BOAT_API boat_layer_t* boat_hip_layer_from_norm(boat_norm_layer_t* layer);
+BOAT_API boat_layer_t* boat_hip_layer_relu(void);
+BOAT_API boat_layer_t* boat_hip_layer_gelu(void);
+/* register every trainable tensor of a layer with an optimizer */
+BOAT_API void boat_hip_optimizer_add_dense(boat_optimizer_t* opt, boat_dense_layer_t* layer);
+BOAT_API void boat_hip_optimizer_add_attention(boat_optimizer_t* opt, boat_attention_t* attention);
+BOAT_API void boat_hip_optimizer_add_layernorm(boat_optimizer_t* opt, boat_layernorm_t* norm);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

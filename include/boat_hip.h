@@ -1,0 +1,153 @@
+/* boat_hip.h - C-ABI of the MI355X (gfx950) device layer under Boat's training hot path.
+ *
+ * One process, one GPU, one HIP stream.  Every entry point takes plain pointers and
+ * sizes; device pointers come from bh_malloc()/bh_buffer_ptr().  Kernels are enqueued
+ * on the library's single stream and return without waiting; bh_synchronize() or any
+ * device-to-host copy waits.  All tensors are dense, row-major, contiguous fp32.
+ *
+ * Return value: 0 on success, a negative BH_E* code otherwise; bh_last_error() gives the
+ * message of the most recent failure.  No entry point falls back to host arithmetic.
+ *
+ * Each kernel entry point names the reference routine (file:line under the Boat tree)
+ * whose arithmetic it replaces.
+ */
+#ifndef BOAT_HIP_H
+#define BOAT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BH_OK          0
+#define BH_EINVAL     -1   /* bad argument / shape the kernel cannot take */
+#define BH_EDEVICE    -2   /* HIP runtime failure */
+#define BH_ENOMEM     -3
+
+/* ---- runtime: replaces the device seam src/core/memory.c:46-74,174-186,230-247 ---- */
+int         bh_init(void);                       /* idempotent; picks device 0, creates the stream */
+int         bh_shutdown(void);
+int         bh_synchronize(void);
+const char* bh_last_error(void);
+const char* bh_device_name(void);
+int         bh_device_cu_count(void);
+void*       bh_stream(void);                     /* the hipStream_t, for callers that time or profile */
+
+/* raw device memory from a size-bucketed cache (stream-ordered reuse, no hipFree per call) */
+void*  bh_malloc(size_t nbytes);
+void   bh_free(void* dptr);
+int    bh_cache_release(void);                   /* hand cached blocks back to the driver */
+size_t bh_bytes_in_use(void);
+size_t bh_bytes_cached(void);
+
+/* reference-counted device buffer: the device twin of boat_tensor_t's ref/unref (src/core/tensor.c:164-191) */
+typedef struct bh_buffer bh_buffer_t;
+bh_buffer_t* bh_buffer_create(size_t nbytes, int zero_fill);
+void         bh_buffer_ref(bh_buffer_t* b);
+void         bh_buffer_unref(bh_buffer_t* b);
+void*        bh_buffer_ptr(const bh_buffer_t* b);
+size_t       bh_buffer_nbytes(const bh_buffer_t* b);
+int          bh_buffer_refcount(const bh_buffer_t* b);
+
+int bh_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes);
+int bh_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes);   /* waits for the stream */
+int bh_memcpy_d2d(void* dst_dev, const void* src_dev, size_t nbytes);
+int bh_memset_zero(void* dst_dev, size_t nbytes);
+
+/* events on the library stream, for timing */
+typedef struct bh_event bh_event_t;
+bh_event_t* bh_event_create(void);
+void        bh_event_destroy(bh_event_t* e);
+int         bh_event_record(bh_event_t* e);
+float       bh_event_elapsed_ms(bh_event_t* start, bh_event_t* stop);    /* synchronises on stop */
+
+/* ---- elementwise (src/ops/arithmetic.c:157-285,362-484; src/autodiff.c:1002-1452) ---- */
+int bh_fill(float* x, float value, int64_t n);
+int bh_add_inplace(float* a, const float* b, int64_t n);                              /* boat_add_ */
+int bh_binary(int op, const float* a, const float* b, float* out, int64_t n);         /* 0 add 1 sub 2 mul 3 div */
+/* broadcasting binary op, numpy rules, shapes right-aligned to ndim<=8 (arithmetic.c:78-104,199-203) */
+int bh_binary_broadcast(int op, const float* a, const int64_t* a_shape,
+                        const float* b, const int64_t* b_shape,
+                        float* out, const int64_t* out_shape, int ndim);
+int bh_scalar_op(int op, const float* a, float s, float* out, int64_t n);             /* boat_*_scalar */
+/* d(a/b)/db = (dy*-1) * (a/(b*b))  (src/autodiff.c:1172-1201) */
+int bh_div_backward_b(const float* a, const float* b, const float* dy, float* db, int64_t n);
+
+#define BH_ACT_RELU    0
+#define BH_ACT_SIGMOID 1
+#define BH_ACT_TANH    2
+#define BH_ACT_GELU    3   /* exact erf form; the reference's boat_gelu is a stub (src/ops/activation.c:298-302) */
+int bh_activation_forward(int act, const float* x, float* y, int64_t n);             /* autodiff.c:808-909 */
+/* saved = op input for RELU/GELU, op output for SIGMOID/TANH (autodiff.c:1244-1452).
+ * accumulate!=0 adds into dx instead of assigning. */
+int bh_activation_backward(int act, const float* saved, const float* dy, float* dx, int64_t n, int accumulate);
+
+int bh_bias_add_rows(float* y, const float* bias, int64_t rows, int64_t cols);        /* dense.c:180-184 */
+int bh_mse_grad(const float* pred, const float* target, float* grad, int64_t n);      /* tests/test_attention_training.c:28-41 */
+int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n);  /* src/loss/mse.c:70-78 */
+int bh_sgd_update(float* p, float* g, float lr, int64_t n, int zero_grad);            /* dense.c:297-329 */
+
+/* ---- reductions / softmax (src/ops/arithmetic.c:611-691; src/autodiff.c:1701-2068; dense.c:286-291) ---- */
+int bh_sum_all(const float* x, float* out1, int64_t n);
+int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumulate); /* db (+)= sum_rows dY */
+int bh_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);
+int bh_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols);
+int bh_log_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);
+int bh_log_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols);
+/* fused replacement of the chain log_softmax -> mul(onehot) -> sum -> mul(-1/B) and its backward
+ * (examples/mnist/mnist_autodiff.c:397-522): loss_out[0] = -(1/B) sum onehot*log_softmax(z),
+ * dlogits = (softmax(z) - onehot)/B.  labels are class indices. */
+int bh_softmax_ce_grad(const float* logits, const int32_t* labels, float* dlogits, float* loss_out,
+                       int64_t rows, int64_t cols);
+
+/* ---- LayerNorm (forward: src/layers/norm.c:184-317; backward: stub there, :397-402) ---- */
+int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, float* y,
+                         float* mean, float* rstd, int64_t rows, int64_t hidden, float eps);
+/* dx (assigned), dgamma/dbeta (assigned unless accumulate).  gamma may be NULL (no affine). */
+int bh_layernorm_backward(const float* x, const float* gamma, const float* dy,
+                          const float* mean, const float* rstd,
+                          float* dx, float* dgamma, float* dbeta,
+                          int64_t rows, int64_t hidden, int accumulate);
+
+/* ---- GEMM on fp32 MFMA (src/ops/linear.c:12-170 with the transposes of :238-406 folded in) ----
+ * C[M,N] (+)= op(A) . op(B) (+ bias[N]), row-major.
+ *   trans_a == 0: A is [M,K] with leading dimension lda;  trans_a != 0: A is stored [K,M]
+ *   trans_b == 0: B is [K,N] with leading dimension ldb;  trans_b != 0: B is stored [N,K]
+ * dense forward  Y  = X.W + b   : trans_a=0 trans_b=0          (dense.c:150-185)
+ * dense backward dX = dY.W^T    : trans_a=0 trans_b=1          (dense.c:219-228)
+ *                dW += X^T.dY   : trans_a=1 trans_b=0, accumulate=1 (dense.c:230-261)
+ * batch > 1 strides all three operands by their full matrix size (linear.c:116-130). */
+int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+            const float* a, int64_t lda, const float* b, int64_t ldb,
+            float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch);
+int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, int64_t cols); /* linear.c:238-406 */
+/* dense layer backward in one call: dx = dy.W^T, gw += x^T.dy, gb += colsum(dy)  (dense.c:190-295) */
+int bh_dense_backward(const float* x, const float* w, const float* dy,
+                      float* dx, float* gw, float* gb, int64_t m, int64_t k, int64_t n,
+                      int accumulate);
+
+/* ---- scaled dot-product attention on [bh, s, d] blocks (src/layers/attention.c:882-1079,1388-1534) ----
+ * forward keeps O and the row log-sum-exp instead of the reference's [bh,s,s] softmax matrix;
+ * backward recomputes P = exp(scale*QK^T - lse).  attn_out (may be NULL) receives the softmax
+ * matrix when a caller wants the reference's cache. */
+int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale, int causal,
+                    float* out, float* lse, float* attn_out, int64_t bh, int64_t s, int64_t d);
+int bh_sdpa_backward(const float* q, const float* k, const float* v, const float* out, const float* lse,
+                     const float* d_out, float scale, int causal,
+                     float* dq, float* dk, float* dv, int64_t bh, int64_t s, int64_t d);
+
+/* ---- Adam (src/optimizers/adam.c:180-240) ----
+ * timestep is the pre-increment value the reference passes to powf(beta, (float)(t+1)). */
+int bh_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
+                   float lr, float beta1, float beta2, float eps, int64_t timestep);
+/* one launch over a table of tensors (host arrays of device pointers and element counts) */
+int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m, float* const* v,
+                         const int64_t* n, int count,
+                         float lr, float beta1, float beta2, float eps, int64_t timestep);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,300 @@
+"""Training-path scenarios written once against Boat's C API and run against any library that
+exports it: the compiled reference (to pin the oracle and to write golden vectors) and
+libboat_amd.so (the GPU path under test).  Each function takes a BoatAPI and numpy inputs and
+returns numpy outputs, so results from two libraries can be compared directly.
+
+The call sequences follow the reference's own callers and tests:
+  tests/unit/test_autodiff.c:116-456, tests/test_dense_forward.c, tests/unit/test_optimizer_adam.c,
+  tests/unit/test_attention_gradient_check.c, tests/test_attention_training.c:115-179,
+  examples/mnist/mnist_autodiff.c:397-522,2437-2488.
+"""
+import contextlib
+import ctypes as C
+import os
+import tempfile
+
+import numpy as np
+
+from boat_amd.capi import AttentionConfig, LayerNormConfig
+
+
+@contextlib.contextmanager
+def scratch_cwd():
+    """The reference's attention backward appends to a debug file in the current directory
+    (src/layers/attention.c:478); run it from a throw-away directory."""
+    old = os.getcwd()
+    with tempfile.TemporaryDirectory() as tmp:
+        os.chdir(tmp)
+        try:
+            yield
+        finally:
+            os.chdir(old)
+
+
+def _var(api, arr, requires_grad):
+    t = api.tensor(np.asarray(arr, np.float32))
+    v = api.boat_variable_create(t, requires_grad)
+    api.boat_tensor_unref(t)
+    return v
+
+
+def _grad(api, v):
+    g = api.boat_variable_grad(v)
+    return None if not g else api.numpy(g)
+
+
+BINARY = {"add": "boat_var_add", "sub": "boat_var_sub", "mul": "boat_var_mul", "div": "boat_var_div"}
+UNARY = {"relu": "boat_var_relu", "sigmoid": "boat_var_sigmoid", "tanh": "boat_var_tanh"}
+
+
+def binary_grads(api, op, a, b, dy=None):
+    """c = a (op) b; backward with dy (or ones).  Returns c, da, db."""
+    va, vb = _var(api, a, True), _var(api, b, True)
+    vc = getattr(api, BINARY[op])(va, vb)
+    c = api.numpy(api.boat_variable_data(vc))
+    if dy is None:
+        api.boat_variable_backward_full(vc)
+    else:
+        tdy = api.tensor(np.asarray(dy, np.float32))
+        api.boat_variable_backward(vc, tdy)
+        api.boat_tensor_unref(tdy)
+    out = c, _grad(api, va), _grad(api, vb)
+    return out
+
+
+def unary_grads(api, op, x, dy=None, axis=-1):
+    """y = f(x); backward with dy (or ones).  Returns y, dx."""
+    vx = _var(api, x, True)
+    if op in UNARY:
+        vy = getattr(api, UNARY[op])(vx)
+    elif op == "softmax":
+        vy = api.boat_var_softmax(vx, axis)
+    elif op == "log_softmax":
+        vy = api.boat_var_log_softmax(vx, axis)
+    elif op == "sum":
+        vy = api.boat_var_sum(vx, None, 0, False)
+    else:
+        raise ValueError(op)
+    y = api.numpy(api.boat_variable_data(vy))
+    if dy is None:
+        api.boat_variable_backward_full(vy)
+    else:
+        tdy = api.tensor(np.asarray(dy, np.float32))
+        api.boat_variable_backward(vy, tdy)
+        api.boat_tensor_unref(tdy)
+    return y, _grad(api, vx)
+
+
+def dot_grads(api, a, b):
+    va, vb = _var(api, a, True), _var(api, b, True)
+    vc = api.boat_var_dot(va, vb)
+    c = api.numpy(api.boat_variable_data(vc))
+    api.boat_variable_backward_full(vc)
+    return c, _grad(api, va), _grad(api, vb)
+
+
+def matmul_grads(api, a, b, dy):
+    va, vb = _var(api, a, True), _var(api, b, True)
+    vc = api.boat_var_matmul(va, vb)
+    c = api.numpy(api.boat_variable_data(vc))
+    tdy = api.tensor(np.asarray(dy, np.float32))
+    api.boat_variable_backward(vc, tdy)
+    api.boat_tensor_unref(tdy)
+    return c, _grad(api, va), _grad(api, vb)
+
+
+def matmul(api, a, b):
+    ta, tb = api.tensor(np.asarray(a, np.float32)), api.tensor(np.asarray(b, np.float32))
+    tc = api.boat_matmul(ta, tb)
+    out = api.numpy(tc)
+    for t in (ta, tb, tc):
+        api.boat_tensor_unref(t)
+    return out
+
+
+def transpose(api, a, d0, d1):
+    ta = api.tensor(np.asarray(a, np.float32))
+    tt = api.boat_transpose(ta, d0, d1)
+    out = api.numpy(tt)
+    api.boat_tensor_unref(ta)
+    api.boat_tensor_unref(tt)
+    return out
+
+
+def fanout(api, a, b):
+    """z = y + y with y = a*b: the reference's recursive backward double-counts (returns da, db)."""
+    va, vb = _var(api, a, True), _var(api, b, True)
+    vy = api.boat_var_mul(va, vb)
+    vz = api.boat_var_add(vy, vy)
+    api.boat_variable_backward_full(vz)
+    return _grad(api, va), _grad(api, vb)
+
+
+def _make_dense(api, w, b):
+    layer = api.boat_dense_layer_create(w.shape[0], w.shape[1], b is not None)
+    api.write(api.boat_dense_layer_get_weight(layer), w)      # in place, never set_weight (dangling optimizer pointers)
+    if b is not None:
+        api.write(api.boat_dense_layer_get_bias(layer), b)
+    return layer
+
+
+def dense_forward(api, x, w, b):
+    layer = _make_dense(api, np.asarray(w, np.float32), None if b is None else np.asarray(b, np.float32))
+    tx = api.tensor(np.asarray(x, np.float32))
+    ty = api.boat_dense_layer_forward(layer, tx)
+    y = api.numpy(ty)
+    api.boat_tensor_unref(ty)
+    api.boat_tensor_unref(tx)
+    api.boat_dense_layer_free(layer)
+    return y
+
+
+def dense_backward_twice(api, w, b, x1, dy1, x2, dy2):
+    """forward/backward called twice on one layer: grads accumulate (dense.c:255-291).
+    Returns [(dx, grad_weight, grad_bias) after call 1, after call 2]."""
+    layer = _make_dense(api, np.asarray(w, np.float32), None if b is None else np.asarray(b, np.float32))
+    out = []
+    for x, dy in ((x1, dy1), (x2, dy2)):
+        tx, tdy = api.tensor(np.asarray(x, np.float32)), api.tensor(np.asarray(dy, np.float32))
+        ty = api.boat_dense_layer_forward(layer, tx)
+        tdx = api.boat_dense_layer_backward(layer, tdy)
+        gb = api.boat_dense_layer_get_grad_bias(layer)
+        out.append((api.numpy(tdx), api.numpy(api.boat_dense_layer_get_grad_weight(layer)),
+                    None if not gb else api.numpy(gb)))
+        for t in (ty, tdx, tx, tdy):
+            api.boat_tensor_unref(t)
+    api.boat_dense_layer_free(layer)
+    return out
+
+
+def mlp_ce_adam(api, x, labels, w1, b1, w2, b2, steps=1, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8):
+    """The config-1 training step: dense -> relu -> dense -> log_softmax -> mul(onehot) -> sum -> mul(-1/B),
+    boat_variable_backward_full, boat_optimizer_step, boat_optimizer_zero_grad; `steps` times.
+    Returns a list per step of dict(loss, gw1, gb1, gw2, gb2, w1, b1, w2, b2)."""
+    x = np.asarray(x, np.float32)
+    B = x.shape[0]
+    classes = w2.shape[1]
+    l1 = _make_dense(api, np.asarray(w1, np.float32), np.asarray(b1, np.float32))
+    l2 = _make_dense(api, np.asarray(w2, np.float32), np.asarray(b2, np.float32))
+    opt = api.boat_adam_optimizer_create(lr, beta1, beta2, eps)
+    for layer in (l1, l2):
+        api.boat_optimizer_add_parameter(opt, api.boat_dense_layer_get_weight(layer), api.boat_dense_layer_get_grad_weight(layer))
+        api.boat_optimizer_add_parameter(opt, api.boat_dense_layer_get_bias(layer), api.boat_dense_layer_get_grad_bias(layer))
+    onehot = np.zeros((B, classes), np.float32)
+    onehot[np.arange(B), np.asarray(labels)] = 1.0
+    history = []
+    for _ in range(steps):
+        vx = _var(api, x, True)                       # requires_grad so the dense ops record (autodiff.c:2287)
+        h = api.boat_var_dense(vx, l1)
+        r = api.boat_var_relu(h)
+        z = api.boat_var_dense(r, l2)
+        ls = api.boat_var_log_softmax(z, 1)
+        voh = _var(api, onehot, False)
+        m = api.boat_var_mul(voh, ls)
+        s = api.boat_var_sum(m, None, 0, False)
+        vf = _var(api, np.array([-1.0 / B], np.float32), False)
+        loss = api.boat_var_mul(vf, s)
+        loss_value = float(api.numpy(api.boat_variable_data(loss))[0])
+        api.boat_variable_backward_full(loss)
+        rec = {"loss": loss_value}
+        for name, layer in (("1", l1), ("2", l2)):
+            rec["gw" + name] = api.numpy(api.boat_dense_layer_get_grad_weight(layer))
+            rec["gb" + name] = api.numpy(api.boat_dense_layer_get_grad_bias(layer))
+        api.boat_optimizer_step(opt)
+        api.boat_optimizer_zero_grad(opt)
+        for name, layer in (("1", l1), ("2", l2)):
+            rec["w" + name] = api.numpy(api.boat_dense_layer_get_weight(layer))
+            rec["b" + name] = api.numpy(api.boat_dense_layer_get_bias(layer))
+        history.append(rec)
+        # variables are left to the library that owns them: the reference cannot release a recorded tape
+        if api.is_amd:
+            for v in (loss, vf, s, m, voh, ls, z, r, h, vx):
+                api.boat_variable_free(v)
+    api.boat_optimizer_free(opt)
+    if api.is_amd:
+        api.boat_dense_layer_free(l1)
+        api.boat_dense_layer_free(l2)
+    return history
+
+
+def adam_trajectory(api, params, grads_per_step, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, lr_change=None):
+    """Several tensors registered with one optimizer; grads rewritten in place before each step.
+    lr_change = (step_index, new_lr).  Returns params after every step: list of lists of arrays."""
+    tp = [api.tensor(np.asarray(p, np.float32)) for p in params]
+    tg = [api.zeros(np.asarray(p).shape) for p in params]
+    opt = api.boat_adam_optimizer_create(lr, beta1, beta2, eps)
+    for p, g in zip(tp, tg):
+        api.boat_optimizer_add_parameter(opt, p, g)
+    out = []
+    for step, grads in enumerate(grads_per_step):
+        if lr_change and lr_change[0] == step:
+            api.boat_optimizer_set_learning_rate(opt, lr_change[1])
+        for g, arr in zip(tg, grads):
+            api.write(g, arr)
+        api.boat_optimizer_step(opt)
+        out.append([api.numpy(p) for p in tp])
+    api.boat_optimizer_zero_grad(opt)
+    zeroed = [api.numpy(g) for g in tg]
+    api.boat_optimizer_free(opt)
+    for t in tp + tg:
+        api.boat_tensor_unref(t)
+    return out, zeroed
+
+
+def layernorm_forward(api, x, gamma, beta, eps):
+    x = np.asarray(x, np.float32)
+    cfg = LayerNormConfig(x.shape[-1], eps, gamma is not None, beta is not None)
+    norm = api.boat_layernorm_create(C.byref(cfg))
+    if gamma is not None:
+        tg = api.tensor(np.asarray(gamma, np.float32))
+        api.boat_layernorm_set_weight(norm, tg)
+        api.boat_tensor_unref(tg)
+    if beta is not None:
+        tb = api.tensor(np.asarray(beta, np.float32))
+        api.boat_layernorm_set_bias(norm, tb)
+        api.boat_tensor_unref(tb)
+    tx = api.tensor(x)
+    ty = api.boat_layernorm_forward(norm, tx)
+    y = api.numpy(ty)
+    api.boat_tensor_unref(ty)
+    api.boat_tensor_unref(tx)
+    api.boat_layernorm_free(norm)
+    return y
+
+
+def attention(api, xq, xk, xv, weights, biases, heads, causal, d_out_list):
+    """boat_attention_forward once, then boat_attention_backward for each dY in d_out_list
+    (parameter grads are overwritten per call).  weights/biases: dicts q,k,v,o (biases None = no bias).
+    Returns out and, per backward call, dict(dq, dk, dv, gw{q,k,v,o}, gb{q,k,v,o})."""
+    xq = np.asarray(xq, np.float32)
+    hidden = xq.shape[-1]
+    cfg = AttentionConfig(hidden, heads, hidden // heads, 0.0, bool(causal), biases is not None, False, 10000.0)
+    att = api.boat_attention_create(C.byref(cfg))
+    for n in "qkvo":
+        api.write(getattr(api, f"boat_attention_get_weight_{n}")(att), weights[n])
+        if biases is not None:
+            api.write(getattr(api, f"boat_attention_get_bias_{n}")(att), biases[n])
+    tq, tk, tv = (api.tensor(np.asarray(a, np.float32)) for a in (xq, xk, xv))
+    results = []
+    with scratch_cwd():
+        tout = api.boat_attention_forward(att, tq, tk, tv, None)
+        out = api.numpy(tout)
+        for d_out in d_out_list:
+            tdy = api.tensor(np.asarray(d_out, np.float32))
+            gq, gk, gv = C.c_void_p(), C.c_void_p(), C.c_void_p()
+            ok = api.boat_attention_backward(att, tdy, C.byref(gq), C.byref(gk), C.byref(gv))
+            assert ok, "boat_attention_backward failed"
+            rec = {"dq": api.numpy(gq), "dk": api.numpy(gk), "dv": api.numpy(gv)}
+            for n in "qkvo":
+                rec["gw" + n] = api.numpy(getattr(api, f"boat_attention_get_grad_weight_{n}")(att))
+                gb = getattr(api, f"boat_attention_get_grad_bias_{n}")(att)
+                rec["gb" + n] = api.numpy(gb) if (biases is not None and gb) else None
+            results.append(rec)
+            for t in (gq, gk, gv, tdy):
+                api.boat_tensor_unref(t)
+    api.boat_tensor_unref(tout)
+    if api.is_amd:
+        api.boat_attention_free(att)
+        for t in (tq, tk, tv):
+            api.boat_tensor_unref(t)
+    return out, results

@@ -1,0 +1,297 @@
+"""Pins the oracle: every routine of oracle/boat_oracle.c must reproduce the compiled reference
+(oracle/_ref/libboat_ref.so, built from the reference's own C sources) BIT FOR BIT on seeded
+inputs, and the reference's own known-answer tests must hold for both.
+
+Runs on the CPU.  Skipped when the reference library was not built (no reference tree); the
+committed golden vectors (test_golden.py) then keep the same pins.
+"""
+import numpy as np
+import pytest
+
+import boat_cases as bc
+
+
+def same(a, b):
+    return a is not None and b is not None and a.shape == b.shape and np.array_equal(a, b)
+
+
+# ---- known answers the reference's own tests assert (tests/unit/test_autodiff.c:116-374) ----
+
+def test_known_answers_reference_unit_tests(ref, oracle):
+    c, da, db = bc.binary_grads(ref, "mul", [2, 3], [4, 5])
+    assert c.tolist() == [8, 15] and da.tolist() == [4, 5] and db.tolist() == [2, 3]
+    o_da, o_db = oracle.mul_backward([2, 3], [4, 5], [1, 1])
+    assert same(o_da, da) and same(o_db, db)
+
+    c, da, db = bc.binary_grads(ref, "div", [6, 12], [2, 3])
+    assert c.tolist() == [3, 4]
+    assert da.tolist() == [0.5, np.float32(1 / 3)] and db.tolist() == [-1.5, np.float32(-12 / 9)]
+    o_da, o_db = oracle.div_backward([6, 12], [2, 3], [1, 1])
+    assert same(o_da, da) and same(o_db, db)
+
+    y, dx = bc.unary_grads(ref, "relu", [-1, 0, 2])
+    assert y.tolist() == [0, 0, 2] and dx.tolist() == [0, 0, 1]          # gradient at exactly 0 is 0
+    assert same(oracle.relu_backward([-1, 0, 2], [1, 1, 1]), dx)
+
+    c, da, db = bc.dot_grads(ref, [1, 2, 3], [4, 5, 6])
+    assert c.tolist() == [32] and da.tolist() == [4, 5, 6] and db.tolist() == [1, 2, 3]
+
+    c, da, db = bc.binary_grads(ref, "add", [1, 2], [3, 4])
+    assert da.tolist() == [1, 1] and db.tolist() == [1, 1]
+    c, da, db = bc.binary_grads(ref, "sub", [1, 2], [3, 4])
+    assert da.tolist() == [1, 1] and db.tolist() == [-1, -1]
+
+
+def test_known_answer_dense_forward(ref, oracle):
+    # tests/test_dense_forward.c:79-91
+    x = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    w = np.array([[0.1, 0.2], [0.3, 0.4], [0.5, 0.6]], np.float32)
+    b = np.array([0.1, 0.2], np.float32)
+    y_ref = bc.dense_forward(ref, x, w, b)
+    assert np.allclose(y_ref, x.astype(np.float64) @ w.astype(np.float64) + b, rtol=1e-6)
+    assert same(oracle.dense_forward(x, w, b), y_ref)
+
+
+# ---- seeded bit-exact comparisons ----
+
+@pytest.mark.parametrize("shape_a,shape_b", [((7, 5), (5, 9)), ((2, 3, 5, 4), (2, 3, 4, 6)), ((3, 8, 2), (3, 2, 5))])
+def test_matmul_bit_exact(ref, oracle, rng, shape_a, shape_b):
+    a = rng.standard_normal(shape_a).astype(np.float32)
+    b = rng.standard_normal(shape_b).astype(np.float32)
+    assert same(oracle.matmul(a, b), bc.matmul(ref, a, b))
+
+
+def test_transpose_bit_exact(ref, oracle, rng):
+    a = rng.standard_normal((6, 11)).astype(np.float32)
+    assert same(oracle.transpose_last2(a), bc.transpose(ref, a, 0, 1))
+    a4 = rng.standard_normal((2, 3, 5, 4)).astype(np.float32)
+    assert same(oracle.transpose_last2(a4), bc.transpose(ref, a4, 2, 3))
+
+
+@pytest.mark.parametrize("op", ["mul", "div"])
+def test_binary_grads_bit_exact(ref, oracle, rng, op):
+    a = rng.standard_normal((5, 7)).astype(np.float32)
+    b = (rng.standard_normal((5, 7)) + 3.0).astype(np.float32)
+    dy = rng.standard_normal((5, 7)).astype(np.float32)
+    _, da, db = bc.binary_grads(ref, op, a, b, dy)
+    o_da, o_db = (oracle.mul_backward if op == "mul" else oracle.div_backward)(a, b, dy)
+    assert same(o_da, da) and same(o_db, db)
+
+
+@pytest.mark.parametrize("op", ["relu", "sigmoid", "tanh"])
+def test_activation_bit_exact(ref, oracle, rng, op):
+    x = rng.standard_normal((5, 7)).astype(np.float32)
+    x[0, :3] = [0.0, -0.0, 1e-30]
+    dy = rng.standard_normal((5, 7)).astype(np.float32)
+    y, dx = bc.unary_grads(ref, op, x, dy)
+    o_y = getattr(oracle, op + "_forward")(x)
+    assert same(o_y, y)
+    saved = x if op == "relu" else y
+    assert same(getattr(oracle, op + "_backward")(saved, dy), dx)
+
+
+@pytest.mark.parametrize("shape", [(6, 10), (3, 33), (2, 4, 5)])
+@pytest.mark.parametrize("op", ["softmax", "log_softmax"])
+def test_softmax_family_bit_exact(ref, oracle, rng, op, shape):
+    x = (3 * rng.standard_normal(shape)).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    y, dx = bc.unary_grads(ref, op, x, dy)
+    assert same(getattr(oracle, op + "_forward")(x), y)
+    assert same(getattr(oracle, op + "_backward")(y, dy), dx)
+    # the invariant the reference's tests check (test_autodiff.c:393-397,437-441)
+    p = y if op == "softmax" else np.exp(y)
+    assert np.allclose(p.sum(-1), 1.0, atol=1e-5)
+
+
+def test_sum_bit_exact(ref, oracle, rng):
+    x = rng.standard_normal(1000).astype(np.float32)
+    y, dx = bc.unary_grads(ref, "sum", x)
+    assert y[0] == np.float32(oracle.sum(x)) and np.all(dx == 1.0)
+
+
+def test_dense_backward_accumulates_bit_exact(ref, oracle, rng):
+    m, k, n = 9, 13, 6
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    x1, x2 = (rng.standard_normal((m, k)).astype(np.float32) for _ in range(2))
+    dy1, dy2 = (rng.standard_normal((m, n)).astype(np.float32) for _ in range(2))
+    (dx1, gw1, gb1), (dx2, gw2, gb2) = bc.dense_backward_twice(ref, w, b, x1, dy1, x2, dy2)
+    o_dx1, o_gw1, o_gb1 = oracle.dense_backward(x1, w, dy1)
+    o_dx2, o_gw2, o_gb2 = oracle.dense_backward(x2, w, dy2, o_gw1, o_gb1)
+    assert same(o_dx1, dx1) and same(o_gw1, gw1) and same(o_gb1, gb1)
+    assert same(o_dx2, dx2) and same(o_gw2, gw2) and same(o_gb2, gb2)
+    # grads really accumulate (+=) across calls
+    assert not np.array_equal(gw1, gw2)
+    assert np.allclose(gb2, dy1.sum(0) + dy2.sum(0), rtol=1e-5, atol=1e-5)
+
+
+def oracle_mlp_steps(oracle, x, labels, w1, b1, w2, b2, steps, lr, beta1, beta2, eps):
+    """The config-1 step restated with oracle primitives."""
+    B, classes = x.shape[0], w2.shape[1]
+    onehot = np.zeros((B, classes), np.float32)
+    onehot[np.arange(B), labels] = 1.0
+    params = [w1.copy(), b1.copy(), w2.copy(), b2.copy()]
+    m = [np.zeros_like(p) for p in params]
+    v = [np.zeros_like(p) for p in params]
+    hist = []
+    for t in range(steps):
+        w1_, b1_, w2_, b2_ = params
+        h = oracle.dense_forward(x, w1_, b1_)
+        r = oracle.relu_forward(h)
+        z = oracle.dense_forward(r, w2_, b2_)
+        loss, dz = oracle.ce_chain(z, onehot)
+        dr, gw2, gb2 = oracle.dense_backward(r, w2_, dz)
+        dh = oracle.relu_backward(h, dr)
+        _, gw1, gb1 = oracle.dense_backward(x, w1_, dh)
+        grads = [gw1, gb1, gw2, gb2]
+        for i in range(4):
+            p, mm, vv = oracle.adam_update(params[i], grads[i], m[i], v[i], lr, beta1, beta2, eps, t)
+            params[i], m[i], v[i] = p.reshape(params[i].shape), mm.reshape(params[i].shape), vv.reshape(params[i].shape)
+        hist.append(dict(loss=loss, gw1=gw1, gb1=gb1, gw2=gw2, gb2=gb2,
+                         w1=params[0].copy(), b1=params[1].copy(), w2=params[2].copy(), b2=params[3].copy()))
+    return hist
+
+
+@pytest.mark.parametrize("dims,batch,steps", [((20, 16, 10), 8, 3), ((784, 128, 10), 64, 1)])
+def test_mlp_ce_adam_steps_bit_exact(ref, oracle, dims, batch, steps):
+    rng = np.random.default_rng(1234 + dims[0])
+    d_in, d_h, d_out = dims
+    x = rng.random((batch, d_in), dtype=np.float32)
+    labels = rng.integers(0, d_out, batch)
+    lim1, lim2 = np.sqrt(6.0 / (d_in + d_h)), np.sqrt(6.0 / (d_h + d_out))
+    w1 = rng.uniform(-lim1, lim1, (d_in, d_h)).astype(np.float32)
+    w2 = rng.uniform(-lim2, lim2, (d_h, d_out)).astype(np.float32)
+    b1, b2 = np.zeros(d_h, np.float32), np.zeros(d_out, np.float32)
+    hp = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    got = bc.mlp_ce_adam(ref, x, labels, w1, b1, w2, b2, steps=steps, **hp)
+    want = oracle_mlp_steps(oracle, x, labels, w1, b1, w2, b2, steps, **hp)
+    for g, w in zip(got, want):
+        assert np.float32(g["loss"]) == np.float32(w["loss"])
+        for key in ("gw1", "gb1", "gw2", "gb2", "w1", "b1", "w2", "b2"):
+            assert same(w[key], g[key]), key
+    # sanity: the fused identity dlogits = (softmax - onehot)/B holds to rounding
+    assert abs(got[0]["loss"] - np.log(d_out)) < 1.0
+
+
+def test_adam_trajectory_bit_exact(ref, oracle, rng):
+    shapes = [(4, 3), (7,), (1,)]
+    params = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    grads = [[(rng.standard_normal(s) * 10 ** rng.uniform(-4, 1)).astype(np.float32) for s in shapes] for _ in range(10)]
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8)
+    got, zeroed = bc.adam_trajectory(ref, params, grads, lr_change=(5, 3e-3), **hp)
+    p = [a.copy() for a in params]
+    m = [np.zeros_like(a) for a in params]
+    v = [np.zeros_like(a) for a in params]
+    for t, gstep in enumerate(grads):
+        lr = 3e-3 if t >= 5 else 1e-2
+        for i in range(3):
+            pi, mi, vi = oracle.adam_update(p[i], gstep[i], m[i], v[i], lr, 0.9, 0.999, 1e-8, t)
+            p[i], m[i], v[i] = pi, mi, vi
+            assert same(p[i].reshape(shapes[i]), got[t][i]), (t, i)
+    assert all(np.all(z == 0) for z in zeroed)
+
+
+def test_adam_first_step_closed_form(ref, oracle):
+    # from m = v = 0: p -= lr*g/(|g|+eps)  =>  p=5, g=2, lr=.01 -> 4.99 (tests/unit/test_optimizer_adam.c:96-108)
+    got, _ = bc.adam_trajectory(ref, [np.array([5.0], np.float32)], [[np.array([2.0], np.float32)]], lr=0.01)
+    assert abs(float(got[0][0][0]) - 4.99) < 1e-6
+    p, m, v = oracle.adam_update(np.array([5.0]), np.array([2.0]), np.zeros(1), np.zeros(1), 0.01, 0.9, 0.999, 1e-8, 0)
+    assert same(p, got[0][0])
+    # zero gradient leaves the parameter alone (:203-205)
+    got, _ = bc.adam_trajectory(ref, [np.array([1.5], np.float32)], [[np.array([0.0], np.float32)]], lr=0.01)
+    assert float(got[0][0][0]) == 1.5
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 48), (7, 64), (4, 768)])
+def test_layernorm_forward_bit_exact(ref, oracle, rng, shape):
+    x = rng.standard_normal(shape).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(shape[-1])).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(shape[-1])).astype(np.float32)
+    y = bc.layernorm_forward(ref, x, gamma, beta, 1e-5)
+    o_y, mean, rstd = oracle.layernorm_forward(x, gamma, beta, 1e-5)
+    assert same(o_y, y)
+    # closed form in float64
+    xd = x.astype(np.float64)
+    mu = xd.mean(-1, keepdims=True)
+    var = xd.var(-1, keepdims=True)
+    assert np.allclose(y, (xd - mu) / np.sqrt(var + 1e-5) * gamma + beta, atol=1e-5)
+    assert np.allclose(mean, mu.ravel(), atol=1e-6) and np.allclose(rstd, 1 / np.sqrt(var.ravel() + 1e-5), rtol=1e-5)
+
+
+def test_layernorm_pattern_input(ref, oracle):
+    # tests/test_layernorm_simple.c: pattern (i % 10) * 0.1, H = 768, eps 1e-5
+    x = ((np.arange(2 * 3 * 768) % 10) * 0.1).astype(np.float32).reshape(2, 3, 768)
+    y = bc.layernorm_forward(ref, x, np.ones(768, np.float32), np.zeros(768, np.float32), 1e-5)
+    o_y, _, _ = oracle.layernorm_forward(x, np.ones(768, np.float32), np.zeros(768, np.float32), 1e-5)
+    assert same(o_y, y)
+    assert np.allclose(y.mean(-1), 0, atol=1e-5) and np.allclose(y.var(-1), 1, atol=1e-3)
+
+
+ATT_CASES = [
+    dict(B=2, S=4, H=32, heads=4, causal=False, bias=True),    # tests/unit/test_attention_gradient_check.c config
+    dict(B=2, S=4, H=32, heads=4, causal=True, bias=True),
+    dict(B=1, S=16, H=64, heads=4, causal=False, bias=False),
+    dict(B=1, S=16, H=64, heads=4, causal=True, bias=True),
+]
+
+
+def make_attention_inputs(case, seed):
+    rng = np.random.default_rng(seed)
+    B, S, H = case["B"], case["S"], case["H"]
+    xs = [rng.standard_normal((B, S, H)).astype(np.float32) for _ in range(3)]
+    w = {n: (rng.standard_normal((H, H)) / np.sqrt(H)).astype(np.float32) for n in "qkvo"}
+    b = {n: (0.1 * rng.standard_normal(H)).astype(np.float32) for n in "qkvo"} if case["bias"] else None
+    dys = [rng.standard_normal((B, S, H)).astype(np.float32) for _ in range(2)]
+    return xs, w, b, dys
+
+
+@pytest.mark.parametrize("case", ATT_CASES, ids=lambda c: f"B{c['B']}S{c['S']}H{c['H']}{'c' if c['causal'] else ''}{'b' if c['bias'] else ''}")
+def test_attention_layer_bit_exact(ref, oracle, case):
+    xs, w, b, dys = make_attention_inputs(case, 99)
+    out, results = bc.attention(ref, *xs, w, b, case["heads"], case["causal"], dys)
+    o_out, cache = oracle.attention_forward(*xs, w, b, case["heads"], case["causal"])
+    assert same(o_out, out)
+    for dy, rec in zip(dys, results):          # second call: parameter grads overwritten, not accumulated
+        g = oracle.attention_backward(*xs, w, b is not None, cache, dy, case["heads"])
+        assert same(g["d_query"], rec["dq"]) and same(g["d_key"], rec["dk"]) and same(g["d_value"], rec["dv"])
+        for n in "qkvo":
+            assert same(g["gw" + n], rec["gw" + n]), n
+            if b is not None:
+                assert same(g["gb" + n], rec["gb" + n]), n
+
+
+def test_sdpa_core_via_identity_projections(ref, oracle):
+    """With W = I and no bias the layer is bare SDPA on the reshaped [B*nh, S, hd] blocks: pins the
+    head split (plain reshape, no transpose), the scale on the scores and the double row-dot."""
+    B, S, H, heads = 1, 8, 16, 2
+    rng = np.random.default_rng(5)
+    xs = [rng.standard_normal((B, S, H)).astype(np.float32) for _ in range(3)]
+    eye = {n: np.eye(H, dtype=np.float32) for n in "qkvo"}
+    dy = rng.standard_normal((B, S, H)).astype(np.float32)
+    out, (rec,) = bc.attention(ref, *xs, eye, None, heads, False, [dy])
+    hd = H // heads
+    q, k, v = (x.reshape(B * heads, S, hd) for x in xs)       # the reference's reshape, not a head transpose
+    scale = np.float32(1.0) / np.sqrt(np.float32(hd))
+    o, lse, attn = oracle.sdpa_forward(q, k, v, scale)
+    assert same(o.reshape(B, S, H), out)
+    dq, dk, dv = oracle.sdpa_backward(q, k, v, attn, dy.reshape(B * heads, S, hd), scale)
+    assert same(dq.reshape(B, S, H), rec["dq"]) and same(dk.reshape(B, S, H), rec["dk"]) and same(dv.reshape(B, S, H), rec["dv"])
+    # textbook SDPA backward in float64 on each contiguous block
+    qd, kd, vd, gd = (a.astype(np.float64) for a in (q, k, v, dy.reshape(B * heads, S, hd)))
+    sc = np.einsum("bid,bjd->bij", qd, kd) / np.sqrt(hd)
+    p = np.exp(sc - sc.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    dp = np.einsum("bid,bjd->bij", gd, vd)
+    ds = p * (dp - (dp * p).sum(-1, keepdims=True)) / np.sqrt(hd)
+    assert np.allclose(dq, np.einsum("bij,bjd->bid", ds, kd), atol=1e-5)
+    assert np.allclose(dk, np.einsum("bij,bid->bjd", ds, qd), atol=1e-5)
+    assert np.allclose(dv, np.einsum("bij,bid->bjd", p, gd), atol=1e-5)
+    assert np.allclose(lse, np.log(np.exp(sc).sum(-1)), atol=1e-5)
+
+
+def test_fanout_divergence_is_documented(ref):
+    """z = y + y, y = a*b: the reference's depth-first recursion visits y once per consumer and
+    reports dz/da = 4b; the true gradient is 2b.  Recorded as a known reference behaviour."""
+    a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
+    da, db = bc.fanout(ref, a, b)
+    assert np.array_equal(da, 4 * b) and np.array_equal(db, 4 * a)

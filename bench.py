@@ -1,0 +1,318 @@
+#!/usr/bin/env python3
+"""Benchmark of the training hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+A step is one dense-layer backward at BASELINE config 2 (the GEMM-bound configuration the
+metric is quoted on): X[8192x4096] ~N(0,1), W[4096x4096] ~N(0,0.02), dY[8192x4096] ~N(0,1);
+dX = dY.W^T, dW += X^T.dY, db += colsum(dY) -- the three launches bh_dense_backward makes,
+issued here one by one so that HIP events on the library stream can time the GEMM launches
+inside the timed region.  Inputs are resident in HBM before timing starts.
+
+Prints ONE JSON line: the step time in ms (value), the roofline of the dominant kernel
+(fp32 MFMA GEMM: algorithmic 2*M*K*N flops per launch / measured average launch duration,
+against the 157.3 TFLOP/s fp32-MFMA peak), the CPU baseline (the compiled reference's
+boat_dense_layer_backward, or the oracle port when the reference library is absent, timed on
+one host core on a bounded sample and scaled by flops), and -- under "extra" -- the other
+configurations of the path with their own roofline fractions.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
+PEAK_FP32_MFMA_TFLOPS = 157.3
+METRIC = "backward+Adam step ms; GB/s & TFLOP/s as % of MI355X roofline (1 GPU)"
+
+# HBM bytes per GEMM launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a copy
+# kernel of known size; see profiles/.  None until measured.
+GEMM_TRAFFIC_BYTES = None
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def time_steps(hip, fn, steps, warmup):
+    """ms per step of fn(), timed with HIP events on the library stream, device idle on both sides."""
+    for _ in range(warmup):
+        fn()
+    hip.synchronize()
+    t = hip.Timer()
+    with t:
+        for _ in range(steps):
+            fn()
+    hip.synchronize()
+    return t.ms / steps
+
+
+def bench_dense_backward(hip, steps, warmup):
+    M, K, N = 8192, 4096, 4096
+    rng = np.random.default_rng(20250102)
+    X = hip.to_device(rng.standard_normal((M, K), dtype=np.float32))
+    W = hip.to_device((0.02 * rng.standard_normal((K, N), dtype=np.float32)).astype(np.float32))
+    dY = hip.to_device(rng.standard_normal((M, N), dtype=np.float32))
+    dX, dW, dB = hip.empty((M, K)), hip.zeros((K, N)), hip.zeros(N)
+
+    ev = [hip.bh_event_create() for _ in range(3 * steps)]
+
+    def step(i=None):
+        if i is not None:
+            hip.check(hip.bh_event_record(ev[3 * i]))
+        hip.check(hip.bh_gemm(0, 1, M, K, N, dY.ptr, N, W.ptr, N, dX.ptr, K, None, 0, 1), "dX = dY.W^T")
+        if i is not None:
+            hip.check(hip.bh_event_record(ev[3 * i + 1]))
+        hip.check(hip.bh_gemm(1, 0, K, N, M, X.ptr, K, dY.ptr, N, dW.ptr, N, None, 1, 1), "dW += X^T.dY")
+        if i is not None:
+            hip.check(hip.bh_event_record(ev[3 * i + 2]))
+        hip.check(hip.bh_colsum(dY.ptr, dB.ptr, M, N, 1), "db += colsum(dY)")
+
+    for _ in range(warmup):
+        step()
+    hip.synchronize()
+    t0 = time.perf_counter()
+    timer = hip.Timer()
+    with timer:
+        for i in range(steps):
+            step(i)
+    hip.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms_per_step = timer.ms / steps
+    gemm_ms = 0.0
+    for i in range(steps):
+        gemm_ms += hip.bh_event_elapsed_ms(ev[3 * i], ev[3 * i + 1]) + hip.bh_event_elapsed_ms(ev[3 * i + 1], ev[3 * i + 2])
+    for e in ev:
+        hip.bh_event_destroy(e)
+    gemm_launch_ms = gemm_ms / (2 * steps)
+    flops_per_launch = 2.0 * M * K * N
+    achieved = flops_per_launch / (gemm_launch_ms * 1e-3) / 1e12
+    # quick correctness guard on the timed buffers (one tile against float64)
+    got = dX.numpy()[:32, :32]
+    want = dY.numpy()[:32].astype(np.float64) @ W.numpy()[:32].astype(np.float64).T
+    assert np.linalg.norm(got - want) <= 1e-3 * np.linalg.norm(want), "dense backward result check failed"
+    return {
+        "ms_per_step": ms_per_step,
+        "wall_ms_per_step": wall_ms,
+        "roofline": {
+            "bound": "mfma", "kernel": "gemm_mfma_kernel (fp32 v_mfma_f32_32x32x2_f32, 256x256 tile)",
+            "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+            "avg_launch_ms": round(gemm_launch_ms, 4), "flops_per_launch": flops_per_launch,
+            "traffic": GEMM_TRAFFIC_BYTES,
+        },
+        "step_tflops": round(2 * flops_per_launch / (ms_per_step * 1e-3) / 1e12, 2),
+    }
+
+
+def bench_extra(hip, steps, warmup):
+    """The other configurations of the path, each with its own roofline."""
+    out = {}
+    rng = np.random.default_rng(20250103)
+
+    # config 5b: flat fused Adam over 268,435,456 parameters (28 B/param)
+    n = 268435456
+    p, g, m, v = (hip.empty(n) for _ in range(4))
+    chunk = 1 << 24
+    noise_p = (0.02 * rng.standard_normal(chunk, dtype=np.float32)).astype(np.float32)
+    noise_g = (1e-3 * rng.standard_normal(chunk, dtype=np.float32)).astype(np.float32)
+    for off in range(0, n, chunk):   # N(0,.02) params, N(0,1e-3) grads, tiled from one 16M-element draw
+        hip.check(hip.bh_memcpy_h2d(p.ptr + 4 * off, noise_p.ctypes.data, 4 * chunk))
+        hip.check(hip.bh_memcpy_h2d(g.ptr + 4 * off, noise_g.ctypes.data, 4 * chunk))
+    hip.check(hip.bh_memset_zero(m.ptr, 4 * n))
+    hip.check(hip.bh_memset_zero(v.ptr, 4 * n))
+    step = [0]
+
+    def adam():
+        hip.check(hip.bh_adam_update(p.ptr, g.ptr, m.ptr, v.ptr, n, 1e-3, 0.9, 0.999, 1e-8, step[0]))
+        step[0] += 1
+
+    ms = time_steps(hip, adam, steps, warmup)
+    gbs = 28.0 * n / (ms * 1e-3) / 1e9
+    out["adam_flat_268M"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4),
+                             "bytes": 28 * n}
+    del p, g, m, v
+
+    # config 3: LayerNorm backward and GELU backward, 16384 x 4096
+    R, H = 16384, 4096
+    x = hip.to_device(rng.standard_normal((R, H), dtype=np.float32))
+    dy = hip.to_device(rng.standard_normal((R, H), dtype=np.float32))
+    gamma = hip.to_device((1 + 0.1 * rng.standard_normal(H)).astype(np.float32))
+    beta = hip.to_device((0.1 * rng.standard_normal(H)).astype(np.float32))
+    y, mean, rstd = hip.empty((R, H)), hip.empty(R), hip.empty(R)
+    hip.check(hip.bh_layernorm_forward(x.ptr, gamma.ptr, beta.ptr, y.ptr, mean.ptr, rstd.ptr, R, H, 1e-5))
+    dx, dg, db = hip.empty((R, H)), hip.zeros(H), hip.zeros(H)
+    ms = time_steps(hip, lambda: hip.check(hip.bh_layernorm_backward(x.ptr, gamma.ptr, dy.ptr, mean.ptr, rstd.ptr, dx.ptr, dg.ptr,
+                                                                      db.ptr, R, H, 0)), steps, warmup)
+    nbytes = 3 * 4 * R * H + 4 * (3 * H + 2 * R)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out["layernorm_bwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
+                                       "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    ms = time_steps(hip, lambda: hip.check(hip.bh_activation_backward(hip.ACT_GELU, x.ptr, dy.ptr, dx.ptr, R * H, 0)), steps, warmup)
+    nbytes = 3 * 4 * R * H
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out["gelu_bwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
+                                  "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    del x, dy, y, dx
+
+    # config 4: attention core backward, B8 h16 S1024 D64 (credited flops: dV, dP, dQ, dK contractions)
+    bh_, S, D = 8 * 16, 1024, 64
+    q, k, vv, go = (hip.to_device(rng.standard_normal((bh_, S, D), dtype=np.float32)) for _ in range(4))
+    o, lse = hip.empty((bh_, S, D)), hip.empty((bh_, S))
+    scale = 1.0 / 8.0
+    hip.check(hip.bh_sdpa_forward(q.ptr, k.ptr, vv.ptr, scale, 0, o.ptr, lse.ptr, None, bh_, S, D))
+    dq, dk, dv = hip.empty((bh_, S, D)), hip.empty((bh_, S, D)), hip.empty((bh_, S, D))
+    sd_steps = max(2, min(steps, 5))
+    ms = time_steps(hip, lambda: hip.check(hip.bh_sdpa_backward(q.ptr, k.ptr, vv.ptr, o.ptr, lse.ptr, go.ptr, scale, 0, dq.ptr, dk.ptr,
+                                                                dv.ptr, bh_, S, D)), sd_steps, 1)
+    flops = 4 * 2.0 * bh_ * S * S * D
+    tf = flops / (ms * 1e-3) / 1e12
+    out["sdpa_bwd_B8h16S1024D64"] = {"ms": round(ms, 4), "bound": "mfma", "achieved_TFLOPs": round(tf, 2),
+                                     "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "credited_flops": flops}
+    return out
+
+
+def bench_mlp_step(steps, warmup):
+    """Config 1 through Boat's C API: forward + boat_variable_backward_full + boat_optimizer_step, wall ms."""
+    from boat_amd.capi import default_api
+    api = default_api()
+    rng = np.random.default_rng(20250101)
+    B, d_in, d_h, d_out = 64, 784, 128, 10
+    x = rng.random((B, d_in), dtype=np.float32)
+    labels = rng.integers(0, d_out, B)
+    onehot = np.zeros((B, d_out), np.float32)
+    onehot[np.arange(B), labels] = 1
+    l1 = api.boat_dense_layer_create(d_in, d_h, True)
+    l2 = api.boat_dense_layer_create(d_h, d_out, True)
+    for layer, (fi, fo) in ((l1, (d_in, d_h)), (l2, (d_h, d_out))):
+        lim = np.sqrt(6.0 / (fi + fo))
+        api.write(api.boat_dense_layer_get_weight(layer), rng.uniform(-lim, lim, (fi, fo)).astype(np.float32))
+    opt = api.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
+    api.boat_hip_optimizer_add_dense(opt, l1)
+    api.boat_hip_optimizer_add_dense(opt, l2)
+    tx, toh = api.tensor(x), api.tensor(onehot)
+    tf = api.tensor(np.array([-1.0 / B], np.float32))
+
+    def step():
+        vx = api.boat_variable_create(tx, True)
+        voh = api.boat_variable_create(toh, False)
+        vf = api.boat_variable_create(tf, False)
+        h = api.boat_var_dense(vx, l1)
+        r = api.boat_var_relu(h)
+        z = api.boat_var_dense(r, l2)
+        ls = api.boat_var_log_softmax(z, 1)
+        mm = api.boat_var_mul(voh, ls)
+        s = api.boat_var_sum(mm, None, 0, False)
+        loss = api.boat_var_mul(vf, s)
+        api.boat_variable_backward_full(loss)
+        api.boat_optimizer_step(opt)
+        api.boat_optimizer_zero_grad(opt)
+        for var in (loss, s, mm, ls, z, r, h, vf, voh, vx):
+            api.boat_variable_free(var)
+
+    for _ in range(warmup):
+        step()
+    api.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.sync()
+    return {"ms": round((time.perf_counter() - t0) * 1e3 / steps, 4), "bound": "launch latency",
+            "note": "MLP 784-128-10 B64 fwd+bwd+Adam through boat_var_* / boat_variable_backward_full / boat_optimizer_step, wall clock"}
+
+
+def cpu_baseline():
+    """Dense-layer backward of the reference on ONE host core, bounded sample, scaled by flops to config 2."""
+    sys.path.insert(0, str(ROOT / "tests"))
+    import oracle_lib
+    m = k = n = 1024
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    w = (0.02 * rng.standard_normal((k, n), dtype=np.float32)).astype(np.float32)
+    dy = rng.standard_normal((m, n), dtype=np.float32)
+    full_flops = 2 * 2.0 * 8192 * 4096 * 4096
+    sample_flops = 2 * 2.0 * m * k * n
+    ref = oracle_lib.load_reference()
+    if ref is not None:
+        import boat_cases as bc
+        layer = ref.boat_dense_layer_create(k, n, True)
+        ref.write(ref.boat_dense_layer_get_weight(layer), w)
+        tx, tdy = ref.tensor(x), ref.tensor(dy)
+        ty = ref.boat_dense_layer_forward(layer, tx)          # caches the input; not timed
+        t0 = time.perf_counter()
+        tdx = ref.boat_dense_layer_backward(layer, tdy)
+        sec = time.perf_counter() - t0
+        assert tdx, "reference backward failed"
+        kind, what = "reference", "boat_dense_layer_backward of the compiled reference (oracle/_ref)"
+    else:
+        oracle = oracle_lib.load()
+        t0 = time.perf_counter()
+        oracle.dense_backward(x, w, dy)
+        sec = time.perf_counter() - t0
+        kind, what = "port", "oracle dense_backward (loop-order restatement of src/layers/dense.c:190-295)"
+    return {
+        "value": round(sec * 1e3 * full_flops / sample_flops, 1), "unit": "ms", "cores": 1, "kind": kind,
+        "host_cores_total": os.cpu_count(),
+        "sample": f"{what} at M=K=N={m} ({sample_flops / 1e9:.2f} GFLOP) took {sec:.2f} s = "
+                  f"{sample_flops / sec / 1e9:.2f} GFLOP/s; value is that time scaled by flops to the "
+                  f"{full_flops / 1e9:.2f} GFLOP workload (extrapolated)",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build (the path has no inter-GPU work)",
+              file=sys.stderr)
+        sys.exit(2)
+    from boat_amd import hip
+    hip.check(hip.bh_init(), "bh_init")
+
+    main_res = bench_dense_backward(hip, args.steps, args.warmup)
+    line = {
+        "metric": METRIC,
+        "value": round(main_res["ms_per_step"], 4),
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_res["ms_per_step"], 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "dense layer backward (BASELINE config 2): X[8192x4096], W[4096x4096], dY[8192x4096] -> dX, dW, db; "
+                               "549.76 GFLOP per step", "M": 8192, "K": 4096, "N": 4096,
+                   "device": hip.bh_device_name().decode().strip(), "compute_units": hip.bh_device_cu_count()},
+        "roofline": main_res["roofline"],
+        "step_tflops": main_res["step_tflops"],
+        "wall_ms_per_step": round(main_res["wall_ms_per_step"], 4),
+    }
+    if not args.no_extra:
+        extra = bench_extra(hip, args.steps, args.warmup)
+        extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20), args.warmup)
+        line["extra"] = extra
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

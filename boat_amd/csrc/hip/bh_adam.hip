@@ -33,28 +33,36 @@ __device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, 
     p -= s.lr * m_hat / (sqrtf(v_hat) + s.eps);
 }
 
-__device__ __forceinline__ void adam_span(float* __restrict__ p, const float* __restrict__ g, float* __restrict__ m,
-                                          float* __restrict__ v, int64_t n, const AdamScalars& s, int64_t first,
-                                          int64_t stride) {
-    // n4 float4 groups, then a scalar tail
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// One float4 group per lane: lane `idx` of the tensor's own grid updates elements 4*idx..4*idx+3;
+// the first (n % 4) lanes also take one tail element.  No loop: the grid covers the tensor, so the
+// resident workgroups sweep p, g, m and v as four contiguous moving windows, and every access is
+// non-temporal (each byte is touched once per step).
+__device__ __forceinline__ void adam_group(float* __restrict__ p, const float* __restrict__ g, float* __restrict__ m,
+                                           float* __restrict__ v, int64_t n, const AdamScalars& s, int64_t idx) {
     const int64_t n4 = n >> 2;
-    float4* p4 = reinterpret_cast<float4*>(p);
-    const float4* g4 = reinterpret_cast<const float4*>(g);
-    float4* m4 = reinterpret_cast<float4*>(m);
-    float4* v4 = reinterpret_cast<float4*>(v);
-    for (int64_t i = first; i < n4; i += stride) {
-        float4 pp = p4[i], gg = g4[i], mm = m4[i], vv = v4[i];
-        adam_one(pp.x, gg.x, mm.x, vv.x, s);
-        adam_one(pp.y, gg.y, mm.y, vv.y, s);
-        adam_one(pp.z, gg.z, mm.z, vv.z, s);
-        adam_one(pp.w, gg.w, mm.w, vv.w, s);
-        p4[i] = pp;
-        m4[i] = mm;
-        v4[i] = vv;
+    if (idx < n4) {
+        f32x4 pp = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(p) + idx);
+        f32x4 gg = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(g) + idx);
+        f32x4 mm = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(m) + idx);
+        f32x4 vv = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(v) + idx);
+        float px = pp.x, py = pp.y, pz = pp.z, pw = pp.w;
+        float mx = mm.x, my = mm.y, mz = mm.z, mw = mm.w;
+        float vx = vv.x, vy = vv.y, vz = vv.z, vw = vv.w;
+        adam_one(px, gg.x, mx, vx, s);
+        adam_one(py, gg.y, my, vy, s);
+        adam_one(pz, gg.z, mz, vz, s);
+        adam_one(pw, gg.w, mw, vw, s);
+        pp = (f32x4){px, py, pz, pw};
+        mm = (f32x4){mx, my, mz, mw};
+        vv = (f32x4){vx, vy, vz, vw};
+        __builtin_nontemporal_store(pp, reinterpret_cast<f32x4*>(p) + idx);
+        __builtin_nontemporal_store(mm, reinterpret_cast<f32x4*>(m) + idx);
+        __builtin_nontemporal_store(vv, reinterpret_cast<f32x4*>(v) + idx);
     }
-    const int64_t tail = n & 3;
-    if (first < tail) {
-        const int64_t i = (n4 << 2) + first;
+    if (idx < (n & 3)) {
+        const int64_t i = (n4 << 2) + idx;
         float pp = p[i], mm = m[i], vv = v[i];
         adam_one(pp, g[i], mm, vv, s);
         p[i] = pp;
@@ -65,13 +73,13 @@ __device__ __forceinline__ void adam_span(float* __restrict__ p, const float* __
 
 __global__ __launch_bounds__(kAdamBlock) void adam_flat_kernel(float* p, const float* g, float* m, float* v,
                                                                int64_t n, AdamScalars s) {
-    adam_span(p, g, m, v, n, s, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
+    adam_group(p, g, m, v, n, s, (int64_t)blockIdx.x * kAdamBlock + threadIdx.x);
 }
 
 __global__ __launch_bounds__(kAdamBlock) void adam_flat_scalar_kernel(float* p, const float* g, float* m, float* v,
                                                                       int64_t n, AdamScalars s) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int64_t i = (int64_t)blockIdx.x * kAdamBlock + threadIdx.x;
+    if (i < n) {
         float pp = p[i], mm = m[i], vv = v[i];
         adam_one(pp, g[i], mm, vv, s);
         p[i] = pp;
@@ -99,8 +107,7 @@ __global__ __launch_bounds__(kAdamBlock) void adam_multi_kernel(AdamTable t, Ada
         int mid = (lo + hi) >> 1;
         if ((int)blockIdx.x >= t.first_block[mid]) lo = mid; else hi = mid;
     }
-    const int nb = t.first_block[lo + 1] - t.first_block[lo];
-    const int lb = (int)blockIdx.x - t.first_block[lo];
+    const int64_t idx = (int64_t)((int)blockIdx.x - t.first_block[lo]) * kAdamBlock + threadIdx.x;
     float* p = t.p[lo];
     const float* g = t.g[lo];
     float* m = t.m[lo];
@@ -108,11 +115,12 @@ __global__ __launch_bounds__(kAdamBlock) void adam_multi_kernel(AdamTable t, Ada
     const int64_t n = t.n[lo];
     const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
                        reinterpret_cast<uintptr_t>(v)) & 15) == 0;
-    const int64_t first = (int64_t)lb * blockDim.x + threadIdx.x, stride = (int64_t)nb * blockDim.x;
     if (vec) {
-        adam_span(p, g, m, v, n, s, first, stride);
+        adam_group(p, g, m, v, n, s, idx);
     } else {
-        for (int64_t i = first; i < n; i += stride) {
+        // unaligned tensor: this block's lanes walk the tensor with the stride of the blocks it was given
+        const int64_t stride = (int64_t)(t.first_block[lo + 1] - t.first_block[lo]) * kAdamBlock;
+        for (int64_t i = idx; i < n; i += stride) {
             float pp = p[i], mm = m[i], vv = v[i];
             adam_one(pp, g[i], mm, vv, s);
             p[i] = pp;
@@ -136,11 +144,10 @@ static AdamScalars make_scalars(float lr, float beta1, float beta2, float eps, i
     return s;
 }
 
-static int blocks_for(int64_t n) {
+// workgroups that cover n elements with one float4 group per lane
+static int64_t blocks_for(int64_t n) {
     int64_t b = ceil_div(ceil_div(n, 4), kAdamBlock);
-    if (b > 256 * 16) b = 256 * 16;
-    if (b < 1) b = 1;
-    return (int)b;
+    return b < 1 ? 1 : b;
 }
 
 }  // namespace bh
@@ -158,11 +165,12 @@ int bh_adam_update(float* p, const float* g, float* m, float* v, int64_t n, floa
     AdamScalars s = make_scalars(lr, beta1, beta2, eps, timestep);
     const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
                        reinterpret_cast<uintptr_t>(v)) & 15) == 0;
+    const int64_t blocks = vec ? blocks_for(n) : blocks_for(n * 4);
+    BH_CHECK_ARG(blocks <= 0x7fffffff, "tensor too large");
     if (vec)
-        hipLaunchKernelGGL(adam_flat_kernel, dim3(blocks_for(n)), dim3(kAdamBlock), 0, stream(), p, g, m, v, n, s);
+        hipLaunchKernelGGL(adam_flat_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), p, g, m, v, n, s);
     else
-        hipLaunchKernelGGL(adam_flat_scalar_kernel, dim3(blocks_for(n * 4)), dim3(kAdamBlock), 0, stream(), p, g, m, v,
-                           n, s);
+        hipLaunchKernelGGL(adam_flat_scalar_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), p, g, m, v, n, s);
     return BH_LAUNCH_CHECK("bh_adam_update");
 }
 
@@ -176,7 +184,7 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
     while (done < count) {
         AdamTable t;
         t.count = 0;
-        int blocks = 0;
+        int64_t blocks = 0;
         while (done < count && t.count < kAdamMaxTensors) {
             const int i = done++;
             BH_CHECK_ARG(n[i] >= 0, "negative element count");
@@ -188,12 +196,13 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
             t.m[k] = m[i];
             t.v[k] = v[i];
             t.n[k] = n[i];
-            t.first_block[k] = blocks;
+            t.first_block[k] = (int)blocks;
             blocks += blocks_for(n[i]);
+            BH_CHECK_ARG(blocks <= 0x7fffffff, "tensors too large for one launch");
         }
         if (t.count == 0) continue;
-        t.first_block[t.count] = blocks;
-        hipLaunchKernelGGL(adam_multi_kernel, dim3(blocks), dim3(kAdamBlock), 0, stream(), t, s);
+        t.first_block[t.count] = (int)blocks;
+        hipLaunchKernelGGL(adam_multi_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), t, s);
         int rc = BH_LAUNCH_CHECK("bh_adam_update_multi");
         if (rc) return rc;
     }

@@ -65,4 +65,38 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
+// Column sums of a small row-major matrix of per-workgroup partials: out[c] (+)= sum_r partial[r][c].
+// 1024 lanes per workgroup = 64 columns x 16 row-lanes, so a column's rows are summed by 16 lanes in
+// parallel (4 loads in flight each) and folded through LDS.  Columns [0, split) go to out_a, the rest
+// to out_b (either may be NULL).  Launch with grid = ceil(ncols / 64), block = 1024.
+constexpr int kFoldCols = 64;
+constexpr int kFoldLanes = 16;
+static __global__ __launch_bounds__(kFoldCols * kFoldLanes) void fold_rows_kernel(
+    const float* __restrict__ partial, int64_t nrows, int64_t ncols, float* __restrict__ out_a,
+    float* __restrict__ out_b, int64_t split, int accumulate) {
+    __shared__ float red[kFoldLanes][kFoldCols + 1];
+    const int tx = threadIdx.x % kFoldCols, ty = threadIdx.x / kFoldCols;
+    const int64_t c = (int64_t)blockIdx.x * kFoldCols + tx;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (c < ncols) {
+        int64_t r = ty;
+        for (; r + 3 * kFoldLanes < nrows; r += 4 * kFoldLanes) {
+            a0 += partial[r * ncols + c];
+            a1 += partial[(r + kFoldLanes) * ncols + c];
+            a2 += partial[(r + 2 * kFoldLanes) * ncols + c];
+            a3 += partial[(r + 3 * kFoldLanes) * ncols + c];
+        }
+        for (; r < nrows; r += kFoldLanes) a0 += partial[r * ncols + c];
+    }
+    red[ty][tx] = (a0 + a1) + (a2 + a3);
+    __syncthreads();
+    if (ty == 0 && c < ncols) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < kFoldLanes; i++) acc += red[i][tx];
+        float* dst = c < split ? (out_a ? out_a + c : nullptr) : (out_b ? out_b + (c - split) : nullptr);
+        if (dst) *dst = accumulate ? *dst + acc : acc;
+    }
+}
+
 }  // namespace bh

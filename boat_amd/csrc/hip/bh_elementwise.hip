@@ -28,33 +28,35 @@ static inline int grid_for(int64_t work_items) {
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // out[i] = f(in0[i], in1[i], in2[i], out[i]); NIN inputs are read, out is read when RO.
+// One float4 per lane per input, one workgroup per 256 float4: the grid is as large as the data, so
+// the resident workgroups sweep memory as one contiguous moving window (measured faster on MI355X
+// than a persistent grid-stride loop), and the accesses are marked non-temporal (streamed once).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 template <int NIN, bool RO, typename F>
 __global__ __launch_bounds__(kBlock) void ew_vec4(F f, float* __restrict__ out, const float* __restrict__ in0,
                                                   const float* __restrict__ in1, const float* __restrict__ in2,
                                                   int64_t n) {
     const int64_t n4 = n >> 2;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const float4* a4 = reinterpret_cast<const float4*>(in0);
-    const float4* b4 = reinterpret_cast<const float4*>(in1);
-    const float4* c4 = reinterpret_cast<const float4*>(in2);
-    float4* o4 = reinterpret_cast<float4*>(out);
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-        float4 a = NIN > 0 ? a4[i] : make_float4(0, 0, 0, 0);
-        float4 b = NIN > 1 ? b4[i] : make_float4(0, 0, 0, 0);
-        float4 c = NIN > 2 ? c4[i] : make_float4(0, 0, 0, 0);
-        float4 o = RO ? o4[i] : make_float4(0, 0, 0, 0);
-        float4 r;
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n4) {
+        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        f32x4 a = NIN > 0 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(in0) + i) : zero;
+        f32x4 b = NIN > 1 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(in1) + i) : zero;
+        f32x4 c = NIN > 2 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(in2) + i) : zero;
+        f32x4 o = RO ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(out) + i) : zero;
+        f32x4 r;
         r.x = f(a.x, b.x, c.x, o.x);
         r.y = f(a.y, b.y, c.y, o.y);
         r.z = f(a.z, b.z, c.z, o.z);
         r.w = f(a.w, b.w, c.w, o.w);
-        o4[i] = r;
+        __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(out) + i);
     }
     // tail (n % 4 elements), first lanes of block 0
     const int64_t tail = n & 3;
     if (blockIdx.x == 0 && threadIdx.x < tail) {
-        const int64_t i = (n4 << 2) + threadIdx.x;
-        out[i] = f(NIN > 0 ? in0[i] : 0.f, NIN > 1 ? in1[i] : 0.f, NIN > 2 ? in2[i] : 0.f, RO ? out[i] : 0.f);
+        const int64_t j = (n4 << 2) + threadIdx.x;
+        out[j] = f(NIN > 0 ? in0[j] : 0.f, NIN > 1 ? in1[j] : 0.f, NIN > 2 ? in2[j] : 0.f, RO ? out[j] : 0.f);
     }
 }
 
@@ -73,8 +75,10 @@ static int launch_ew(const char* name, F f, float* out, const float* in0, const 
     const bool vec = aligned16(out) && (NIN < 1 || aligned16(in0)) && (NIN < 2 || aligned16(in1)) &&
                      (NIN < 3 || aligned16(in2));
     if (vec) {
-        hipLaunchKernelGGL((ew_vec4<NIN, RO, F>), dim3(grid_for((n + 3) >> 2)), dim3(kBlock), 0, stream(), f, out,
-                           in0, in1, in2, n);
+        const int64_t blocks = ceil_div((n >> 2) > 0 ? (n >> 2) : 1, kBlock);
+        if (blocks > 0x7fffffff) return set_error(BH_EINVAL, "%s: tensor too large", name);
+        hipLaunchKernelGGL((ew_vec4<NIN, RO, F>), dim3((unsigned)blocks), dim3(kBlock), 0, stream(), f, out, in0, in1,
+                           in2, n);
     } else {
         hipLaunchKernelGGL((ew_scalar<NIN, RO, F>), dim3(grid_for(n)), dim3(kBlock), 0, stream(), f, out, in0, in1,
                            in2, n);

@@ -21,6 +21,16 @@ constexpr int kLnBlock = 256;
 
 __device__ __forceinline__ float4 ld4(const float* p, int64_t i4) { return reinterpret_cast<const float4*>(p)[i4]; }
 __device__ __forceinline__ void st4(float* p, int64_t i4, float4 v) { reinterpret_cast<float4*>(p)[i4] = v; }
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4_stream(const float* p, int64_t i4) {
+    f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p) + i4);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st4_stream(float* p, int64_t i4, float4 v) {
+    f32x4 o = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(p) + i4);
+}
+
 
 // Sum of two values over the TPR threads that share a row.
 template <int TPR>
@@ -59,9 +69,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
     const int group = threadIdx.x / TPR, t = threadIdx.x % TPR;
     const int h4 = hidden >> 2;
     const int64_t g_id = (int64_t)blockIdx.x * GROUPS + group;
-    const int64_t r0 = g_id * rows_per_group;
-    int64_t r1 = r0 + rows_per_group;
-    if (r1 > rows) r1 = rows;
+    const int64_t total_groups = (int64_t)gridDim.x * GROUPS;
 
     float4 gm[VPT], bt[VPT];
 #pragma unroll
@@ -70,17 +78,18 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
         gm[i] = (gamma && c4 < h4) ? ld4(gamma, c4) : make_float4(1, 1, 1, 1);
         bt[i] = (beta && c4 < h4) ? ld4(beta, c4) : make_float4(0, 0, 0, 0);
     }
-    // rows_per_group is the same for every group, so the loop trip count (and every
-    // barrier inside row_sum2) is uniform across the block; out-of-range rows are masked.
+    // Group g takes rows g, g+G, g+2G, ...: the resident workgroups read neighbouring rows (one moving
+    // window).  rows_per_group is the same for every group, so the loop trip count (and every barrier
+    // inside row_sum2) is uniform across the block; out-of-range rows are masked.
     for (int64_t it = 0; it < rows_per_group; it++) {
-        const int64_t r = r0 + it;
-        const bool live = r < r1;
+        const int64_t r = it * total_groups + g_id;
+        const bool live = r < rows;
         float4 xv[VPT];
         float s = 0.f, dummy = 0.f;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
             const int c4 = t + i * TPR;
-            xv[i] = (live && c4 < h4) ? ld4(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
+            xv[i] = (live && c4 < h4) ? ld4_stream(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
             s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
         }
         row_sum2<TPR>(s, dummy, lds, group);
@@ -110,7 +119,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
                     o.w = (xv[i].w - mu) * rs;
                     if (gamma) { o.x *= gm[i].x; o.y *= gm[i].y; o.z *= gm[i].z; o.w *= gm[i].w; }
                     if (beta) { o.x += bt[i].x; o.y += bt[i].y; o.z += bt[i].z; o.w += bt[i].w; }
-                    st4(y + r * hidden, c4, o);
+                    st4_stream(y + r * hidden, c4, o);
                 }
             }
             if (t == 0) {
@@ -153,23 +162,27 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_generic_kernel(const float* _
 
 // --------------------------------------------------------------- backward
 // partial layout: [num_blocks][2][hidden]  (dgamma slice, then dbeta slice)
+//
+// Row -> workgroup map: group g of G takes rows g, g+G, g+2G, ... so that at any moment the resident
+// workgroups read neighbouring rows (one contiguous moving window over x and dy) instead of G far-apart
+// chunks.  The loop is software-pipelined: the loads of the next row are issued before the current
+// row's reduction barrier and dx stores, so memory requests stay in flight across the barrier.
+// x, dy and dx are streamed once each and marked non-temporal.
 template <int TPR, int VPT>
 __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                           const float* __restrict__ dy, const float* __restrict__ mean,
                                                           const float* __restrict__ rstd, float* __restrict__ dx,
                                                           float* __restrict__ partial, int64_t rows, int hidden,
-                                                          int64_t rows_per_group) {
+                                                          int64_t iters) {
     constexpr int GROUPS = kLnBlock / TPR;
     extern __shared__ float dyn_lds[];           // GROUPS>1: [GROUPS][2][hidden] for the cross-group fold
     __shared__ float lds[GROUPS * (TPR / 64) * 2 + 2];
     const int group = threadIdx.x / TPR, t = threadIdx.x % TPR;
     const int h4 = hidden >> 2;
+    const int64_t total_groups = (int64_t)gridDim.x * GROUPS;
     const int64_t g_id = (int64_t)blockIdx.x * GROUPS + group;
-    const int64_t r0 = g_id * rows_per_group;
-    int64_t r1 = r0 + rows_per_group;
-    if (r1 > rows) r1 = rows;
 
-    float4 gm[VPT], dg[VPT], db[VPT];
+    float4 gm[VPT], dg[VPT], db[VPT], xv[VPT], gy[VPT];
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int c4 = t + i * TPR;
@@ -178,40 +191,60 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
         db[i] = make_float4(0, 0, 0, 0);
     }
     const float inv_h = 1.0f / (float)hidden;
-    for (int64_t it = 0; it < rows_per_group; it++) {
-        const int64_t r = r0 + it;
-        const bool live = r < r1;
-        const float mu = live ? mean[r] : 0.f;
-        const float rs = live ? rstd[r] : 0.f;
+    // prologue: first row of this group
+    int64_t row = g_id;
+    bool live = row < rows;
+    float mu = live ? mean[row] : 0.f, rs = live ? rstd[row] : 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int c4 = t + i * TPR;
+        const bool on = live && c4 < h4;
+        xv[i] = on ? ld4_stream(x + row * hidden, c4) : make_float4(0, 0, 0, 0);
+        gy[i] = on ? ld4_stream(dy + row * hidden, c4) : make_float4(0, 0, 0, 0);
+    }
+    // `iters` is the same for every group, so the barriers below are reached uniformly; rows past the
+    // end are masked (they contribute zeros and store nothing).
+    for (int64_t it = 0; it < iters; it++) {
         float4 xh[VPT], g[VPT];
         float s1 = 0.f, s2 = 0.f;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
-            const int c4 = t + i * TPR;
-            const bool on = live && c4 < h4;
-            float4 xv = on ? ld4(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
-            float4 gy = on ? ld4(dy + r * hidden, c4) : make_float4(0, 0, 0, 0);
-            xh[i].x = (xv.x - mu) * rs; xh[i].y = (xv.y - mu) * rs; xh[i].z = (xv.z - mu) * rs; xh[i].w = (xv.w - mu) * rs;
-            g[i].x = gy.x * gm[i].x; g[i].y = gy.y * gm[i].y; g[i].z = gy.z * gm[i].z; g[i].w = gy.w * gm[i].w;
+            xh[i].x = (xv[i].x - mu) * rs; xh[i].y = (xv[i].y - mu) * rs; xh[i].z = (xv[i].z - mu) * rs; xh[i].w = (xv[i].w - mu) * rs;
+            g[i].x = gy[i].x * gm[i].x; g[i].y = gy[i].y * gm[i].y; g[i].z = gy[i].z * gm[i].z; g[i].w = gy[i].w * gm[i].w;
             s1 += (g[i].x + g[i].y) + (g[i].z + g[i].w);
             s2 += (g[i].x * xh[i].x + g[i].y * xh[i].y) + (g[i].z * xh[i].z + g[i].w * xh[i].w);
-            dg[i].x += gy.x * xh[i].x; dg[i].y += gy.y * xh[i].y; dg[i].z += gy.z * xh[i].z; dg[i].w += gy.w * xh[i].w;
-            db[i].x += gy.x; db[i].y += gy.y; db[i].z += gy.z; db[i].w += gy.w;
+            dg[i].x += gy[i].x * xh[i].x; dg[i].y += gy[i].y * xh[i].y; dg[i].z += gy[i].z * xh[i].z; dg[i].w += gy[i].w * xh[i].w;
+            db[i].x += gy[i].x; db[i].y += gy[i].y; db[i].z += gy[i].z; db[i].w += gy[i].w;
+        }
+        const int64_t cur_row = row;
+        const bool cur_live = live;
+        const float cur_rs = rs;
+        // issue the next row's loads before the barrier
+        row = (it + 1) * total_groups + g_id;
+        live = (it + 1 < iters) && row < rows;
+        mu = live ? mean[row] : 0.f;
+        rs = live ? rstd[row] : 0.f;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int c4 = t + i * TPR;
+            const bool on = live && c4 < h4;
+            xv[i] = on ? ld4_stream(x + row * hidden, c4) : make_float4(0, 0, 0, 0);
+            gy[i] = on ? ld4_stream(dy + row * hidden, c4) : make_float4(0, 0, 0, 0);
         }
         row_sum2<TPR>(s1, s2, lds, group);
         s1 *= inv_h;
         s2 *= inv_h;
-        if (live) {
+        if (cur_live) {
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
                 const int c4 = t + i * TPR;
                 if (c4 < h4) {
                     float4 o;
-                    o.x = rs * (g[i].x - s1 - xh[i].x * s2);
-                    o.y = rs * (g[i].y - s1 - xh[i].y * s2);
-                    o.z = rs * (g[i].z - s1 - xh[i].z * s2);
-                    o.w = rs * (g[i].w - s1 - xh[i].w * s2);
-                    st4(dx + r * hidden, c4, o);
+                    o.x = cur_rs * (g[i].x - s1 - xh[i].x * s2);
+                    o.y = cur_rs * (g[i].y - s1 - xh[i].y * s2);
+                    o.z = cur_rs * (g[i].z - s1 - xh[i].z * s2);
+                    o.w = cur_rs * (g[i].w - s1 - xh[i].w * s2);
+                    st4_stream(dx + cur_row * hidden, c4, o);
                 }
             }
         }
@@ -289,25 +322,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_param_generic_kernel(const fl
     partial[((int64_t)blockIdx.y * 2 + 1) * hidden + c] = db;
 }
 
-// fold partial[nblk][2][hidden] into dgamma / dbeta
-__global__ __launch_bounds__(kLnBlock) void ln_param_fold_kernel(const float* __restrict__ partial, float* __restrict__ dgamma,
-                                                                 float* __restrict__ dbeta, int64_t nblk, int64_t hidden,
-                                                                 int accumulate) {
-    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // over 2*hidden
-    if (c >= 2 * hidden) return;
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int64_t k = 0;
-    for (; k + 3 < nblk; k += 4) {
-        a0 += partial[(k * 2) * hidden + c];
-        a1 += partial[((k + 1) * 2) * hidden + c];
-        a2 += partial[((k + 2) * 2) * hidden + c];
-        a3 += partial[((k + 3) * 2) * hidden + c];
-    }
-    for (; k < nblk; k++) a0 += partial[(k * 2) * hidden + c];
-    const float acc = (a0 + a1) + (a2 + a3);
-    float* dst = c < hidden ? (dgamma ? dgamma + c : nullptr) : (dbeta ? dbeta + (c - hidden) : nullptr);
-    if (dst) *dst = accumulate ? *dst + acc : acc;
-}
+static int g_ln_bwd_blocks = 512;    // cap on backward workgroups (2 per CU)
 
 struct LnPlan {
     bool vector;     // register-resident float4 path
@@ -355,6 +370,13 @@ using namespace bh;
 
 extern "C" {
 
+// tuning hook for benchmarks: cap on backward workgroups
+int bh_layernorm_tune(int bwd_blocks, int reserved) {
+    (void)reserved;
+    if (bwd_blocks > 0) g_ln_bwd_blocks = bwd_blocks;
+    return BH_OK;
+}
+
 int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, float* y, float* mean, float* rstd,
                          int64_t rows, int64_t hidden, float eps) {
     BH_REQUIRE_INIT();
@@ -374,7 +396,6 @@ int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, 
     const int64_t cap = 256 * 8;
     if (blocks > cap) blocks = cap;
     const int64_t rpg = ceil_div(rows, blocks * groups);
-    blocks = ceil_div(rows, rpg * groups);
     BH_LN_DISPATCH(ln_fwd_kernel, plan, dim3((unsigned)blocks), 0, x, gamma, beta, y, mean, rstd, rows, (int)hidden, eps, rpg);
     return BH_LAUNCH_CHECK("bh_layernorm_forward");
 }
@@ -401,17 +422,16 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, c
     int rc;
     if (plan.vector) {
         int64_t blocks = ceil_div(rows, groups);
-        const int64_t cap = 256 * 4;     // 4 blocks per CU keeps the per-block partials at a few % of the traffic
+        const int64_t cap = g_ln_bwd_blocks;   // per-block dgamma/dbeta partials cost 2*hidden floats each way
         if (blocks > cap) blocks = cap;
-        const int64_t rpg = ceil_div(rows, blocks * groups);
-        blocks = ceil_div(rows, rpg * groups);
+        const int64_t iters = ceil_div(rows, blocks * groups);
         float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(blocks * 2 * hidden));
         if (!partial) return BH_ENOMEM;
         BH_LN_DISPATCH(ln_bwd_kernel, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
-                       (int)hidden, rpg);
+                       (int)hidden, iters);
         if (dgamma || dbeta)
-            hipLaunchKernelGGL(ln_param_fold_kernel, dim3((unsigned)ceil_div(2 * hidden, kLnBlock)), dim3(kLnBlock), 0,
-                               stream(), partial, dgamma, dbeta, blocks, hidden, accumulate);
+            hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
+                               stream(), partial, blocks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
         bh_free(partial);
         rc = BH_LAUNCH_CHECK("bh_layernorm_backward");
     } else {
@@ -427,8 +447,8 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, c
             if (!partial) return BH_ENOMEM;
             hipLaunchKernelGGL(ln_bwd_param_generic_kernel, dim3((unsigned)ceil_div(hidden, kLnBlock), (unsigned)chunks),
                                dim3(kLnBlock), 0, stream(), x, dy, mean, rstd, partial, rows, hidden, rpb);
-            hipLaunchKernelGGL(ln_param_fold_kernel, dim3((unsigned)ceil_div(2 * hidden, kLnBlock)), dim3(kLnBlock), 0,
-                               stream(), partial, dgamma, dbeta, chunks, hidden, accumulate);
+            hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
+                               stream(), partial, chunks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
             bh_free(partial);
             rc = BH_LAUNCH_CHECK("bh_layernorm_backward params");
         }

@@ -40,32 +40,23 @@ __global__ __launch_bounds__(kRBlock) void sum_final_kernel(const float* partial
     }
 }
 
-// ---- column sum: partial[rb][c] over row chunks, then fold the chunks ----
+// ---- column sum: partial[rb][c] over row chunks, then fold_rows_kernel folds the chunks ----
+// Row chunk y of Y takes rows y, y+Y, y+2Y, ...: the resident workgroups read neighbouring rows.
 __global__ __launch_bounds__(kRBlock) void colsum_partial_kernel(const float* __restrict__ x, float* __restrict__ partial,
-                                                                 int64_t rows, int64_t cols, int64_t rows_per_block) {
+                                                                 int64_t rows, int64_t cols) {
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= cols) return;
-    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
-    int64_t r1 = r0 + rows_per_block;
-    if (r1 > rows) r1 = rows;
+    const int64_t step = gridDim.y;
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int64_t r = r0;
-    for (; r + 3 < r1; r += 4) {
+    int64_t r = blockIdx.y;
+    for (; r + 3 * step < rows; r += 4 * step) {
         a0 += x[r * cols + c];
-        a1 += x[(r + 1) * cols + c];
-        a2 += x[(r + 2) * cols + c];
-        a3 += x[(r + 3) * cols + c];
+        a1 += x[(r + step) * cols + c];
+        a2 += x[(r + 2 * step) * cols + c];
+        a3 += x[(r + 3 * step) * cols + c];
     }
-    for (; r < r1; r++) a0 += x[r * cols + c];
+    for (; r < rows; r += step) a0 += x[r * cols + c];
     partial[(int64_t)blockIdx.y * cols + c] = (a0 + a1) + (a2 + a3);
-}
-__global__ __launch_bounds__(kRBlock) void colsum_final_kernel(const float* __restrict__ partial, float* __restrict__ out,
-                                                               int64_t chunks, int64_t cols, int accumulate) {
-    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= cols) return;
-    float acc = 0.f;
-    for (int64_t k = 0; k < chunks; k++) acc += partial[k * cols + c];
-    out[c] = accumulate ? out[c] + acc : acc;
 }
 
 // ---- row kernels: one wavefront per row, 4 rows per block ----
@@ -167,14 +158,12 @@ int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumu
     int64_t chunks = ceil_div(2048, col_blocks);
     if (chunks > ceil_div(rows, 32)) chunks = ceil_div(rows, 32);
     if (chunks < 1) chunks = 1;
-    const int64_t rpb = ceil_div(rows > 0 ? rows : 1, chunks);
-    chunks = ceil_div(rows > 0 ? rows : 1, rpb);
     float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * cols));
     if (!partial) return BH_ENOMEM;
     hipLaunchKernelGGL(colsum_partial_kernel, dim3(col_blocks, (unsigned)chunks), dim3(kRBlock), 0, stream(), x, partial,
-                       rows, cols, rpb);
-    hipLaunchKernelGGL(colsum_final_kernel, dim3(col_blocks), dim3(kRBlock), 0, stream(), partial, out, chunks, cols,
-                       accumulate);
+                       rows, cols);
+    hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(cols, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0, stream(),
+                       partial, chunks, cols, out, (float*)nullptr, cols, accumulate);
     bh_free(partial);
     return BH_LAUNCH_CHECK("bh_colsum");
 }

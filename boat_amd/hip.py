@@ -156,3 +156,7 @@ class Timer:
             lib.bh_event_destroy(self.stop)
         except Exception:
             pass
+
+lib.bh_layernorm_tune.restype = I
+lib.bh_layernorm_tune.argtypes = [I, I]
+bh_layernorm_tune = lib.bh_layernorm_tune

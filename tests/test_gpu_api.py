@@ -1,0 +1,343 @@
+"""The training path driven through Boat's own C API on libboat_amd.so (GPU) and compared with the
+oracle on the same seeded inputs -- the same scenarios that pin the oracle to the compiled
+reference in test_oracle_vs_reference.py, so the chain GPU == oracle == reference closes.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import boat_cases as bc
+from oracle_lib import max_rel, rel_fro
+from test_oracle_vs_reference import ATT_CASES, make_attention_inputs, oracle_mlp_steps
+
+pytestmark = pytest.mark.gpu
+
+TOL_EW, TOL_RED, TOL_GEMM = 1e-5, 1e-4, 1e-3
+
+
+def test_known_answers_of_the_reference_unit_tests(boat):
+    # tests/unit/test_autodiff.c:116-374
+    c, da, db = bc.binary_grads(boat, "mul", [2, 3], [4, 5])
+    assert c.tolist() == [8, 15] and da.tolist() == [4, 5] and db.tolist() == [2, 3]
+    c, da, db = bc.binary_grads(boat, "div", [6, 12], [2, 3])
+    assert da.tolist() == [0.5, np.float32(1 / 3)] and db.tolist() == [-1.5, np.float32(-12 / 9)]
+    y, dx = bc.unary_grads(boat, "relu", [-1, 0, 2])
+    assert y.tolist() == [0, 0, 2] and dx.tolist() == [0, 0, 1]
+    c, da, db = bc.dot_grads(boat, [1, 2, 3], [4, 5, 6])
+    assert c.tolist() == [32] and da.tolist() == [4, 5, 6] and db.tolist() == [1, 2, 3]
+    c, da, db = bc.binary_grads(boat, "add", [1, 2], [3, 4])
+    assert c.tolist() == [4, 6] and da.tolist() == [1, 1] and db.tolist() == [1, 1]
+    c, da, db = bc.binary_grads(boat, "sub", [1, 2], [3, 4])
+    assert da.tolist() == [1, 1] and db.tolist() == [-1, -1]
+    # tests/test_dense_forward.c:79-91
+    x = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    w = np.array([[0.1, 0.2], [0.3, 0.4], [0.5, 0.6]], np.float32)
+    y = bc.dense_forward(boat, x, w, np.array([0.1, 0.2], np.float32))
+    assert np.allclose(y, [[2.3, 3.0], [5.0, 6.6]], rtol=1e-6)
+
+
+def test_variable_semantics(boat):
+    t = boat.tensor(np.ones((2, 2), np.float32))
+    v = boat.boat_variable_create(t, True)
+    assert not boat.boat_variable_grad(v)                      # no gradient before backward (test_autodiff.c:20)
+    boat.boat_variable_backward_full(v)
+    assert np.all(boat.numpy(boat.boat_variable_grad(v)) == 1)
+    boat.boat_variable_backward_full(v)                        # leaf gradients accumulate across calls
+    assert np.all(boat.numpy(boat.boat_variable_grad(v)) == 2)
+    boat.boat_variable_zero_grad(v)
+    assert not boat.boat_variable_grad(v)                      # zero_grad drops the tensor (autodiff.c:285-292)
+    g = boat.boat_hip_variable_ensure_grad(v)                  # persistent gradient buffer for optimizers
+    boat.boat_variable_backward_full(v)
+    boat.boat_variable_zero_grad(v)
+    assert boat.boat_variable_grad(v) == g and not boat.numpy(g).any()
+    nv = boat.boat_variable_create(t, False)
+    boat.boat_variable_backward_full(nv)                       # silently ignored without requires_grad
+    assert not boat.boat_variable_grad(nv)
+    boat.boat_variable_free(v)
+    boat.boat_variable_free(nv)
+    boat.boat_tensor_unref(t)
+
+
+@pytest.mark.parametrize("op", ["mul", "div", "add", "sub"])
+def test_binary_grads(boat, oracle, rng, op):
+    a = rng.standard_normal((5, 7)).astype(np.float32)
+    b = (rng.standard_normal((5, 7)) + 3).astype(np.float32)
+    dy = rng.standard_normal((5, 7)).astype(np.float32)
+    _, da, db = bc.binary_grads(boat, op, a, b, dy)
+    if op == "mul":
+        wa, wb = oracle.mul_backward(a, b, dy)
+    elif op == "div":
+        wa, wb = oracle.div_backward(a, b, dy)
+    else:
+        wa, wb = dy, (dy if op == "add" else dy * np.float32(-1))
+    assert np.array_equal(da, wa) and np.array_equal(db, wb)
+
+
+@pytest.mark.parametrize("op", ["relu", "sigmoid", "tanh", "softmax", "log_softmax"])
+def test_unary_grads(boat, oracle, rng, op):
+    x = (2 * rng.standard_normal((6, 10))).astype(np.float32)
+    dy = rng.standard_normal((6, 10)).astype(np.float32)
+    y, dx = bc.unary_grads(boat, op, x, dy)
+    wy = getattr(oracle, op + "_forward")(x)
+    wdx = getattr(oracle, op + "_backward")(x if op == "relu" else wy, dy)
+    assert np.max(np.abs(y - wy)) <= TOL_RED * max(1, np.abs(wy).max())
+    assert np.max(np.abs(dx - wdx)) <= TOL_RED * max(1, np.abs(wdx).max())
+
+
+def test_sum_and_matmul_grads(boat, oracle, rng):
+    x = rng.standard_normal(1000).astype(np.float32)
+    y, dx = bc.unary_grads(boat, "sum", x)
+    assert abs(y[0] - oracle.sum(x)) <= TOL_RED * np.abs(x).sum() and np.all(dx == 1)
+    a = rng.standard_normal((9, 12)).astype(np.float32)
+    b = rng.standard_normal((12, 7)).astype(np.float32)
+    dy = rng.standard_normal((9, 7)).astype(np.float32)
+    c, da, db = bc.matmul_grads(boat, a, b, dy)
+    assert rel_fro(c, oracle.matmul(a, b)) <= TOL_GEMM
+    assert rel_fro(da, oracle.matmul(dy, oracle.transpose_last2(b))) <= TOL_GEMM
+    assert rel_fro(db, oracle.matmul(oracle.transpose_last2(a), dy)) <= TOL_GEMM
+
+
+def test_matmul_layouts_and_transpose(boat, oracle, rng):
+    a = rng.standard_normal((2, 3, 5, 4)).astype(np.float32)
+    b = rng.standard_normal((2, 3, 4, 6)).astype(np.float32)
+    assert rel_fro(bc.matmul(boat, a, b), oracle.matmul(a, b)) <= TOL_GEMM
+    assert np.array_equal(bc.transpose(boat, a, 2, 3), oracle.transpose_last2(a))
+    m = rng.standard_normal((6, 11)).astype(np.float32)
+    assert np.array_equal(bc.transpose(boat, m, 0, 1), m.T)
+
+
+def test_fanout_gives_the_true_gradient(boat):
+    """z = y + y, y = a*b.  The reference reports 4b (its recursion revisits y); each op is visited once here."""
+    a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
+    da, db = bc.fanout(boat, a, b)
+    assert np.array_equal(da, 2 * b) and np.array_equal(db, 2 * a)
+
+
+def test_dense_backward_accumulates(boat, oracle, rng):
+    m, k, n = 9, 13, 6
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    x1, x2 = (rng.standard_normal((m, k)).astype(np.float32) for _ in range(2))
+    dy1, dy2 = (rng.standard_normal((m, n)).astype(np.float32) for _ in range(2))
+    (dx1, gw1, gb1), (dx2, gw2, gb2) = bc.dense_backward_twice(boat, w, b, x1, dy1, x2, dy2)
+    o1 = oracle.dense_backward(x1, w, dy1)
+    o2 = oracle.dense_backward(x2, w, dy2, o1[1], o1[2])
+    for got, want in zip((dx1, gw1, gb1, dx2, gw2, gb2), o1 + o2):
+        assert rel_fro(got, want) <= TOL_GEMM
+
+
+def test_dense_error_paths(boat):
+    layer = boat.boat_dense_layer_create(4, 3, True)
+    bad = boat.tensor(np.zeros((2, 3), np.float32))
+    assert not boat.boat_dense_layer_backward(layer, bad)              # no forward yet (dense.c:191)
+    x = boat.tensor(np.zeros((2, 4), np.float32))
+    y = boat.boat_dense_layer_forward(layer, x)
+    wrong = boat.tensor(np.zeros((5, 3), np.float32))
+    assert not boat.boat_dense_layer_backward(layer, wrong)            # batch mismatch (dense.c:212-217)
+    assert not boat.boat_dense_layer_forward(layer, bad)               # wrong feature count
+    assert not boat.boat_adam_optimizer_create(0.0, 0.9, 0.999, 1e-8)  # adam.c:45-53
+    assert not boat.boat_adam_optimizer_create(0.1, 1.0, 0.999, 1e-8)
+    assert not boat.boat_adam_optimizer_create(0.1, 0.9, 0.0, 1e-8)
+    for t in (bad, x, y, wrong):
+        boat.boat_tensor_unref(t)
+    boat.boat_dense_layer_free(layer)
+
+
+@pytest.mark.parametrize("dims,batch,steps", [((20, 16, 10), 8, 3), ((784, 128, 10), 64, 2)])
+def test_mlp_ce_adam_training_steps(boat, oracle, dims, batch, steps):
+    """Config 1: MLP 784->128->10, batch 64, forward + boat_variable_backward_full + Adam."""
+    rng = np.random.default_rng(1234 + dims[0])
+    d_in, d_h, d_out = dims
+    x = rng.random((batch, d_in), dtype=np.float32)
+    labels = rng.integers(0, d_out, batch)
+    lim1, lim2 = np.sqrt(6.0 / (d_in + d_h)), np.sqrt(6.0 / (d_h + d_out))
+    w1 = rng.uniform(-lim1, lim1, (d_in, d_h)).astype(np.float32)
+    w2 = rng.uniform(-lim2, lim2, (d_h, d_out)).astype(np.float32)
+    b1, b2 = np.zeros(d_h, np.float32), np.zeros(d_out, np.float32)
+    hp = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    got = bc.mlp_ce_adam(boat, x, labels, w1, b1, w2, b2, steps=steps, **hp)
+    want = oracle_mlp_steps(oracle, x, labels, w1, b1, w2, b2, steps, **hp)
+    g, w = got[0], want[0]
+    assert abs(g["loss"] - w["loss"]) <= TOL_RED * abs(w["loss"])
+    for key in ("gw1", "gw2"):
+        assert rel_fro(g[key], w[key]) <= TOL_GEMM, key
+    for key in ("gb1", "gb2"):
+        assert np.max(np.abs(g[key] - w[key])) <= TOL_RED * max(1e-3, np.abs(w[key]).max()), key
+    # Updated parameters.  The first Adam step moves every weight by ~lr*sign(g), so weights whose gradient is
+    # pure rounding noise may flip; compare where the gradient is resolved and bound the rest by 2*lr.
+    for t in range(steps):
+        for key, gkey in (("w1", "gw1"), ("b1", "gb1"), ("w2", "gw2"), ("b2", "gb2")):
+            diff = np.abs(got[t][key] - want[t][key])
+            assert diff.max() <= 2.1e-3 * (t + 1), (t, key)
+            resolved = np.abs(want[0][gkey]) > 1e-4 * np.abs(want[0][gkey]).max()
+            if t == 0:
+                assert np.max(diff[resolved]) <= 1e-5 * max(1.0, np.abs(want[t][key]).max()), (t, key)
+
+
+def test_adam_trajectory_bit_exact(boat, oracle, rng):
+    shapes = [(4, 3), (7,), (1,)]
+    params = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    grads = [[(rng.standard_normal(s) * 10 ** rng.uniform(-4, 1)).astype(np.float32) for s in shapes] for _ in range(10)]
+    got, zeroed = bc.adam_trajectory(boat, params, grads, lr=1e-2, lr_change=(5, 3e-3))
+    p = [a.copy() for a in params]
+    m = [np.zeros_like(a) for a in params]
+    v = [np.zeros_like(a) for a in params]
+    for t, gstep in enumerate(grads):
+        lr = 3e-3 if t >= 5 else 1e-2
+        for i in range(3):
+            p[i], m[i], v[i] = oracle.adam_update(p[i], gstep[i], m[i], v[i], lr, 0.9, 0.999, 1e-8, t)
+            assert np.array_equal(p[i].reshape(shapes[i]), got[t][i]), (t, i)
+    assert all(not z.any() for z in zeroed)
+    got, _ = bc.adam_trajectory(boat, [np.array([5.0], np.float32)], [[np.array([2.0], np.float32)]], lr=0.01)
+    assert abs(float(got[0][0][0]) - 4.99) < 1e-6
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 48), (7, 64), (4, 768), (3, 2, 1024), (2, 3, 4, 16)])
+def test_layernorm_forward(boat, oracle, rng, shape):
+    x = rng.standard_normal(shape).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(shape[-1])).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(shape[-1])).astype(np.float32)
+    y = bc.layernorm_forward(boat, x, gamma, beta, 1e-5)
+    rows = shape[0] * shape[1] if len(shape) >= 3 else shape[0]      # rows the reference's loops visit (norm.c:279-281)
+    flat = x.reshape(-1, shape[-1])
+    want = np.zeros_like(flat)
+    want[:rows] = oracle.layernorm_forward(flat[:rows], gamma, beta, 1e-5)[0]
+    assert np.max(np.abs(y.reshape(want.shape) - want)) <= TOL_RED * np.abs(want).max()
+
+
+def test_layernorm_backward_hook(boat, oracle, rng):
+    """boat_layernorm_backward is a stub in the reference: checked against the float64 closed form."""
+    from boat_amd.capi import LayerNormConfig
+    x = rng.standard_normal((3, 5, 64)).astype(np.float32)
+    dy = rng.standard_normal((3, 5, 64)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    cfg = LayerNormConfig(64, 1e-5, True, True)
+    norm = boat.boat_layernorm_create(C.byref(cfg))
+    assert not boat.boat_layernorm_backward(norm, boat.tensor(dy))        # before forward: NULL
+    boat.write(boat.boat_hip_layernorm_get_weight(norm), gamma)
+    tx, tdy = boat.tensor(x), boat.tensor(dy)
+    ty = boat.boat_layernorm_forward(norm, tx)
+    _, mean, rstd = oracle.layernorm_forward(x, gamma, None, 1e-5)
+    wdx, wdg, wdb = oracle.layernorm_backward_f64(x, gamma, dy, mean, rstd)
+    for call in (1, 2):                                                   # parameter grads accumulate
+        tdx = boat.boat_layernorm_backward(norm, tdy)
+        assert np.max(np.abs(boat.numpy(tdx) - wdx)) <= TOL_RED * np.abs(wdx).max()
+        assert np.max(np.abs(boat.numpy(boat.boat_hip_layernorm_get_grad_weight(norm)) - call * wdg)) <= call * TOL_RED * np.abs(wdg).max()
+        assert np.max(np.abs(boat.numpy(boat.boat_hip_layernorm_get_grad_bias(norm)) - call * wdb)) <= call * TOL_RED * np.abs(wdb).max()
+        boat.boat_tensor_unref(tdx)
+    boat.boat_layernorm_free(norm)
+
+
+@pytest.mark.parametrize("case", ATT_CASES, ids=lambda c: f"B{c['B']}S{c['S']}H{c['H']}{'c' if c['causal'] else ''}{'b' if c['bias'] else ''}")
+def test_attention_layer(boat, oracle, case):
+    xs, w, b, dys = make_attention_inputs(case, 99)
+    out, results = bc.attention(boat, *xs, w, b, case["heads"], case["causal"], dys)
+    o_out, cache = oracle.attention_forward(*xs, w, b, case["heads"], case["causal"])
+    assert rel_fro(out, o_out) <= TOL_GEMM
+    for dy, rec in zip(dys, results):
+        g = oracle.attention_backward(*xs, w, b is not None, cache, dy, case["heads"])
+        for got, want in ((rec["dq"], g["d_query"]), (rec["dk"], g["d_key"]), (rec["dv"], g["d_value"])):
+            assert rel_fro(got, want) <= TOL_GEMM
+        for n in "qkvo":
+            assert rel_fro(rec["gw" + n], g["gw" + n]) <= TOL_GEMM, n
+            if b is not None:
+                assert rel_fro(rec["gb" + n], g["gb" + n]) <= TOL_GEMM, n
+
+
+def test_attention_through_the_tape_self_attention(boat, oracle):
+    """boat_var_attention(x, x, x): the three input gradients land in the same leaf (autodiff.c:2458-2532)."""
+    case = dict(B=2, S=8, H=32, heads=4, causal=False, bias=True)
+    xs, w, b, dys = make_attention_inputs(case, 7)
+    x = xs[0]
+    from boat_amd.capi import AttentionConfig
+    cfg = AttentionConfig(32, 4, 8, 0.0, False, True, False, 10000.0)
+    att = boat.boat_attention_create(C.byref(cfg))
+    for n in "qkvo":
+        boat.write(getattr(boat, f"boat_attention_get_weight_{n}")(att), w[n])
+        boat.write(getattr(boat, f"boat_attention_get_bias_{n}")(att), b[n])
+    tx = boat.tensor(x)
+    vx = boat.boat_variable_create(tx, True)
+    vy = boat.boat_var_attention(vx, vx, vx, att, None)
+    tdy = boat.tensor(dys[0])
+    boat.boat_variable_backward(vy, tdy)
+    _, cache = oracle.attention_forward(x, x, x, w, b, 4, False)
+    g = oracle.attention_backward(x, x, x, w, True, cache, dys[0], 4)
+    want = g["d_query"] + g["d_key"] + g["d_value"]
+    assert rel_fro(boat.numpy(boat.boat_variable_grad(vx)), want) <= TOL_GEMM
+    boat.boat_variable_free(vy)
+    boat.boat_variable_free(vx)
+    boat.boat_attention_free(att)
+
+
+def test_model_backward_over_layer_vtables(boat, oracle, rng):
+    """boat_model_backward is a stub in the reference; here it walks layers[n-1..0] through ops->backward."""
+    m, d_in, d_h, d_out = 16, 24, 32, 8
+    x = rng.standard_normal((m, d_in)).astype(np.float32)
+    dy = rng.standard_normal((m, d_out)).astype(np.float32)
+    w1 = rng.standard_normal((d_in, d_h)).astype(np.float32) * 0.2
+    w2 = rng.standard_normal((d_h, d_out)).astype(np.float32) * 0.2
+    l1 = boat.boat_dense_layer_create(d_in, d_h, True)
+    l2 = boat.boat_dense_layer_create(d_h, d_out, True)
+    boat.write(boat.boat_dense_layer_get_weight(l1), w1)
+    boat.write(boat.boat_dense_layer_get_weight(l2), w2)
+    model = boat.boat_model_create()
+    for layer in (boat.boat_hip_layer_from_dense(l1), boat.boat_hip_layer_relu(), boat.boat_hip_layer_from_dense(l2)):
+        boat.boat_model_add_layer(model, layer)
+    assert boat.boat_model_layer_count(model) == 3
+    tx, tdy = boat.tensor(x), boat.tensor(dy)
+    ty = boat.boat_model_forward(model, tx)
+    tdx = boat.boat_model_backward(model, tdy)
+    h = oracle.dense_forward(x, w1, np.zeros(d_h, np.float32))
+    r = oracle.relu_forward(h)
+    assert rel_fro(boat.numpy(ty), oracle.dense_forward(r, w2, np.zeros(d_out, np.float32))) <= TOL_GEMM
+    dr, gw2, _ = oracle.dense_backward(r, w2, dy)
+    dh = oracle.relu_backward(h, dr)
+    dx, gw1, _ = oracle.dense_backward(x, w1, dh)
+    assert rel_fro(boat.numpy(tdx), dx) <= TOL_GEMM
+    assert rel_fro(boat.numpy(boat.boat_dense_layer_get_grad_weight(l1)), gw1) <= TOL_GEMM
+    assert rel_fro(boat.numpy(boat.boat_dense_layer_get_grad_weight(l2)), gw2) <= TOL_GEMM
+    boat.boat_model_update(model, 0.1)                                   # SGD step, gradients cleared (dense.c:297-329)
+    assert rel_fro(boat.numpy(boat.boat_dense_layer_get_weight(l2)), w2 - np.float32(0.1) * gw2) <= TOL_GEMM
+    assert not boat.numpy(boat.boat_dense_layer_get_grad_weight(l2)).any()
+    boat.boat_model_free(model)
+
+
+def test_relu_and_softmax_layer_hooks_pass_gradients_through(boat):
+    # src/layers/relu.c:58-72, src/layers/softmax.c:43-58
+    relu = boat.boat_relu_layer_create()
+    g = boat.tensor(np.array([[-1.0, 2.0]], np.float32))
+    back = boat.boat_relu_layer_backward(relu, g)
+    assert back == g
+    boat.boat_tensor_unref(back)
+    sm = boat.boat_softmax_layer_create(-1)
+    back = boat.boat_softmax_layer_backward(sm, g)
+    assert back == g
+    boat.boat_tensor_unref(back)
+    y = boat.boat_relu_layer_forward(relu, g)
+    assert boat.numpy(y).tolist() == [[0.0, 2.0]]
+    boat.boat_relu_layer_free(relu)
+    boat.boat_softmax_layer_free(sm)
+
+
+def test_device_tensors_and_fused_losses(boat, oracle, rng):
+    from boat_amd.capi import DEVICE_HIP
+    a = rng.standard_normal((4, 6)).astype(np.float32)
+    ta = boat.tensor(a, device=DEVICE_HIP)                               # lives in HBM only
+    assert boat.boat_tensor_device(ta) == DEVICE_HIP
+    tb = boat.boat_mul_scalar(ta, 2.0)
+    assert boat.boat_tensor_device(tb) == DEVICE_HIP and np.array_equal(boat.numpy(tb), a * 2)
+    cpu = boat.tensor(a)
+    assert not boat.boat_add(ta, cpu)                                    # mixed devices refused (arithmetic.c:136-143)
+    z = (2 * rng.standard_normal((8, 10))).astype(np.float32)
+    labels = rng.integers(0, 10, 8).astype(np.int32)
+    onehot = np.zeros((8, 10), np.float32)
+    onehot[np.arange(8), labels] = 1
+    dz = C.c_void_p()
+    tl = boat.boat_hip_softmax_cross_entropy(boat.tensor(z), boat.tensor(labels), C.byref(dz))
+    wl, wdz = oracle.ce_chain(z, onehot)
+    assert abs(boat.numpy(tl)[0] - wl) <= TOL_RED * abs(wl) and np.max(np.abs(boat.numpy(dz) - wdz)) <= 1e-7
+    p, t = rng.standard_normal((3, 5)).astype(np.float32), rng.standard_normal((3, 5)).astype(np.float32)
+    gm = C.c_void_p()
+    tl = boat.boat_hip_mse_loss(boat.tensor(p), boat.tensor(t), C.byref(gm))
+    assert abs(boat.numpy(tl)[0] - oracle.mse_loss(p, t)) <= TOL_RED and np.array_equal(boat.numpy(gm), oracle.mse_grad(p, t))

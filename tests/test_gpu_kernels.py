@@ -1,0 +1,412 @@
+"""Parity of every HIP kernel, called through the C-ABI of include/boat_hip.h, with the CPU oracle on the
+same seeded inputs.  Tolerances are the ones the path states:
+  elementwise / activation / Adam   max relative error <= 1e-5   (Adam and the exp-free ops are checked bit for bit)
+  reductions / LayerNorm            <= 1e-4
+  GEMM / attention gradients        <= 1e-3 relative Frobenius norm
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle_lib import max_rel, rel_fro
+
+pytestmark = pytest.mark.gpu
+
+TOL_EW = 1e-5
+TOL_RED = 1e-4
+TOL_GEMM = 1e-3
+
+
+_KEEP = []
+
+
+def dev(hip, a):
+    """Upload and keep the device array alive until the test ends: a temporary used only for its .ptr
+    would be returned to the allocator cache (and reused by the next upload) before the kernel is launched."""
+    d = hip.to_device(np.ascontiguousarray(a, dtype=np.float32))
+    _KEEP.append(d)
+    return d
+
+
+@pytest.fixture(autouse=True)
+def _release_device_arrays():
+    yield
+    _KEEP.clear()
+
+
+# ------------------------------------------------------------------ runtime
+
+def test_runtime_buffers_and_cache(hip):
+    assert b"gfx950" in hip.bh_device_name()
+    assert hip.bh_device_cu_count() >= 200
+    b = hip.bh_buffer_create(4096, 1)
+    assert b and hip.bh_buffer_refcount(b) == 1 and hip.bh_buffer_nbytes(b) == 4096
+    hip.bh_buffer_ref(b)
+    assert hip.bh_buffer_refcount(b) == 2
+    host = np.empty(1024, np.float32)
+    hip.check(hip.bh_memcpy_d2h(host.ctypes.data, hip.bh_buffer_ptr(b), 4096))
+    assert not host.any()
+    hip.bh_buffer_unref(b)
+    hip.bh_buffer_unref(b)
+    # a freed block is reused for the next request of the same size
+    p1 = hip.bh_malloc(1 << 20)
+    hip.bh_free(p1)
+    p2 = hip.bh_malloc(1 << 20)
+    assert p1 == p2
+    hip.bh_free(p2)
+    # error path: bad arguments are refused, nothing runs
+    assert hip.bh_gemm(0, 0, 4, 4, 4, None, 4, None, 4, None, 4, None, 0, 1) == -1
+    assert b"null pointer" in hip.bh_last_error()
+
+
+# -------------------------------------------------------------- elementwise
+
+@pytest.mark.parametrize("n", [1, 3, 4, 1023, 4096, 100003])
+def test_elementwise_bit_exact(hip, oracle, rng, n):
+    a = rng.standard_normal(n).astype(np.float32)
+    b = (rng.standard_normal(n) + 3).astype(np.float32)
+    dy = rng.standard_normal(n).astype(np.float32)
+    da, db, ddy = dev(hip, a), dev(hip, b), dev(hip, dy)
+    out = hip.empty(n)
+    for op, fn in enumerate([np.add, np.subtract, np.multiply, np.divide]):
+        hip.check(hip.bh_binary(op, da.ptr, db.ptr, out.ptr, n))
+        assert np.array_equal(out.numpy(), fn(a, b))
+    hip.check(hip.bh_scalar_op(2, da.ptr, -0.015625, out.ptr, n))
+    assert np.array_equal(out.numpy(), oracle.mul_scalar(a, -0.015625))
+    acc = dev(hip, b)
+    hip.check(hip.bh_add_inplace(acc.ptr, da.ptr, n))
+    assert np.array_equal(acc.numpy(), b + a)
+    hip.check(hip.bh_div_backward_b(da.ptr, db.ptr, ddy.ptr, out.ptr, n))
+    assert np.array_equal(out.numpy(), oracle.div_backward(a, b, dy)[1])
+    hip.check(hip.bh_fill(out.ptr, 1.0, n))
+    assert np.all(out.numpy() == 1.0)
+
+
+def test_elementwise_unaligned_pointers(hip, rng):
+    n = 1001
+    a = rng.standard_normal(n + 1).astype(np.float32)
+    da = dev(hip, a)
+    out = hip.empty(n + 1)
+    hip.check(hip.bh_memset_zero(out.ptr, 4 * (n + 1)))
+    hip.check(hip.bh_scalar_op(2, da.ptr + 4, 2.0, out.ptr + 4, n))      # 4-byte aligned only
+    got = out.numpy()
+    assert got[0] == 0 and np.array_equal(got[1:], a[1:] * 2)
+
+
+def test_broadcast_binary(hip, rng):
+    a = rng.standard_normal((3, 1, 5)).astype(np.float32)
+    b = rng.standard_normal((4, 1)).astype(np.float32)
+    want = a * b
+    da, db, out = dev(hip, a), dev(hip, b), hip.empty(want.shape)
+    L3 = C.c_int64 * 3
+    hip.check(hip.bh_binary_broadcast(2, da.ptr, L3(3, 1, 5), db.ptr, L3(1, 4, 1), out.ptr, L3(3, 4, 5), 3))
+    assert np.array_equal(out.numpy(), want)
+
+
+@pytest.mark.parametrize("n", [5, 4096, 70001])
+def test_activations(hip, oracle, rng, n):
+    x = rng.standard_normal(n).astype(np.float32) * 2
+    x[:3] = [0.0, -0.0, 1e-30][: min(3, n)]
+    dy = rng.standard_normal(n).astype(np.float32)
+    dx_, ddy, y, g = dev(hip, x), dev(hip, dy), hip.empty(n), hip.empty(n)
+    # relu: exp-free, bit exact
+    hip.check(hip.bh_activation_forward(hip.ACT_RELU, dx_.ptr, y.ptr, n))
+    assert np.array_equal(y.numpy(), oracle.relu_forward(x))
+    hip.check(hip.bh_activation_backward(hip.ACT_RELU, dx_.ptr, ddy.ptr, g.ptr, n, 0))
+    assert np.array_equal(g.numpy(), oracle.relu_backward(x, dy))
+    for act, name in ((hip.ACT_SIGMOID, "sigmoid"), (hip.ACT_TANH, "tanh")):
+        hip.check(hip.bh_activation_forward(act, dx_.ptr, y.ptr, n))
+        want = getattr(oracle, name + "_forward")(x)
+        # The reference's tanh, (e^x - e^-x)/(e^x + e^-x), cancels for small |x|: there its own result carries
+        # expf's last-bit noise amplified by 1/|x|, so the relative bound is taken against max(|y|, 0.05).
+        assert max_rel(y.numpy(), want, floor=0.05 if name == "tanh" else 1e-6) <= TOL_EW
+        dc = dev(hip, want)
+        hip.check(hip.bh_activation_backward(act, dc.ptr, ddy.ptr, g.ptr, n, 0))
+        assert np.array_equal(g.numpy(), getattr(oracle, name + "_backward")(want, dy))   # from the same saved output
+    # gelu (no reference implementation): double-precision closed form
+    hip.check(hip.bh_activation_forward(hip.ACT_GELU, dx_.ptr, y.ptr, n))
+    assert np.max(np.abs(y.numpy() - oracle.gelu_forward_f64(x))) <= 1e-6
+    hip.check(hip.bh_activation_backward(hip.ACT_GELU, dx_.ptr, ddy.ptr, g.ptr, n, 0))
+    want = oracle.gelu_backward_f64(x, dy)
+    assert np.max(np.abs(g.numpy() - want)) <= 1e-5 * max(1.0, np.abs(want).max())
+    # accumulate form adds into dx
+    hip.check(hip.bh_activation_backward(hip.ACT_GELU, dx_.ptr, ddy.ptr, g.ptr, n, 1))
+    assert np.allclose(g.numpy(), 2 * want, rtol=1e-5, atol=1e-6)
+
+
+def test_bias_mse_sgd(hip, oracle, rng):
+    rows, cols = 37, 53
+    y = rng.standard_normal((rows, cols)).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    dy_, db = dev(hip, y), dev(hip, b)
+    hip.check(hip.bh_bias_add_rows(dy_.ptr, db.ptr, rows, cols))
+    assert np.array_equal(dy_.numpy(), y + b)
+    t = rng.standard_normal((rows, cols)).astype(np.float32)
+    dp, dt, g, loss = dev(hip, y), dev(hip, t), hip.empty((rows, cols)), hip.empty(1)
+    hip.check(hip.bh_mse_grad(dp.ptr, dt.ptr, g.ptr, rows * cols))
+    assert np.array_equal(g.numpy(), oracle.mse_grad(y, t))
+    hip.check(hip.bh_mse_loss(dp.ptr, dt.ptr, loss.ptr, rows * cols))
+    assert abs(loss.numpy()[0] - oracle.mse_loss(y, t)) <= TOL_RED * oracle.mse_loss(y, t)
+    p, gr = dev(hip, y), dev(hip, t)
+    hip.check(hip.bh_sgd_update(p.ptr, gr.ptr, 0.1, rows * cols, 1))
+    assert np.array_equal(p.numpy(), y - np.float32(0.1) * t) and not gr.numpy().any()
+
+
+# --------------------------------------------------------------------- adam
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 1 << 20, (1 << 20) + 3])
+def test_adam_bit_exact_over_steps(hip, oracle, rng, n):
+    p = (0.02 * rng.standard_normal(n)).astype(np.float32)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    dp, dm, dv = dev(hip, p), dev(hip, m), dev(hip, v)
+    for t in range(3):
+        g = (1e-3 * rng.standard_normal(n)).astype(np.float32)
+        dg = dev(hip, g)
+        hip.check(hip.bh_adam_update(dp.ptr, dg.ptr, dm.ptr, dv.ptr, n, 1e-3, 0.9, 0.999, 1e-8, t))
+        p, m, v = oracle.adam_update(p, g, m, v, 1e-3, 0.9, 0.999, 1e-8, t)
+        assert np.array_equal(dp.numpy(), p) and np.array_equal(dm.numpy(), m) and np.array_equal(dv.numpy(), v)
+
+
+def test_adam_multi_tensor_bit_exact(hip, oracle, rng):
+    sizes = [12, 1, 4099, 128 * 784, 10] + [33] * 60          # more tensors than one launch table holds
+    ps = [rng.standard_normal(s).astype(np.float32) for s in sizes]
+    gs = [(rng.standard_normal(s) * 0.1).astype(np.float32) for s in sizes]
+    ms = [np.abs(rng.standard_normal(s)).astype(np.float32) * 0.01 for s in sizes]
+    vs = [np.abs(rng.standard_normal(s)).astype(np.float32) * 0.001 for s in sizes]
+    d = [[dev(hip, a) for a in group] for group in (ps, gs, ms, vs)]
+    PA = C.c_void_p * len(sizes)
+    tabs = [PA(*[x.ptr for x in group]) for group in d]
+    ns = (C.c_int64 * len(sizes))(*sizes)
+    hip.check(hip.bh_adam_update_multi(*tabs, ns, len(sizes), 3e-4, 0.9, 0.999, 1e-8, 41))
+    for i in range(len(sizes)):
+        p, m, v = oracle.adam_update(ps[i], gs[i], ms[i], vs[i], 3e-4, 0.9, 0.999, 1e-8, 41)
+        assert np.array_equal(d[0][i].numpy(), p), i
+        assert np.array_equal(d[2][i].numpy(), m) and np.array_equal(d[3][i].numpy(), v)
+
+
+def test_adam_zero_gradient_is_a_no_op(hip):
+    p = hip.to_device(np.full(1000, 1.5, np.float32))
+    g, m, v = hip.zeros(1000), hip.zeros(1000), hip.zeros(1000)
+    hip.check(hip.bh_adam_update(p.ptr, g.ptr, m.ptr, v.ptr, 1000, 0.01, 0.9, 0.999, 1e-8, 0))
+    assert np.all(p.numpy() == 1.5)
+
+
+# ------------------------------------------------------- reductions, softmax
+
+@pytest.mark.parametrize("n", [1, 63, 100000])
+def test_sum_all(hip, oracle, rng, n):
+    x = rng.standard_normal(n).astype(np.float32)
+    out = hip.empty(1)
+    hip.check(hip.bh_sum_all(dev(hip, x).ptr, out.ptr, n))
+    assert abs(out.numpy()[0] - x.astype(np.float64).sum()) <= TOL_RED * max(1.0, np.abs(x).sum())
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (64, 10), (8, 128), (1000, 37), (4096, 512)])
+def test_colsum(hip, rng, rows, cols):
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    base = rng.standard_normal(cols).astype(np.float32)
+    out = dev(hip, base)
+    hip.check(hip.bh_colsum(dev(hip, x).ptr, out.ptr, rows, cols, 0))
+    want = x.astype(np.float64).sum(0)
+    assert np.max(np.abs(out.numpy() - want)) <= TOL_RED * np.abs(x).sum(0).max()
+    hip.check(hip.bh_colsum(dev(hip, x).ptr, out.ptr, rows, cols, 1))
+    assert np.max(np.abs(out.numpy() - 2 * want)) <= 2 * TOL_RED * np.abs(x).sum(0).max()
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 10), (3, 33), (5, 1), (7, 1000)])
+def test_softmax_family(hip, oracle, rng, rows, cols):
+    x = (3 * rng.standard_normal((rows, cols))).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    dx_, ddy, y, g = dev(hip, x), dev(hip, dy), hip.empty((rows, cols)), hip.empty((rows, cols))
+    for fwd, bwd, name in ((hip.bh_softmax_forward, hip.bh_softmax_backward, "softmax"),
+                           (hip.bh_log_softmax_forward, hip.bh_log_softmax_backward, "log_softmax")):
+        hip.check(fwd(dx_.ptr, y.ptr, rows, cols))
+        want = getattr(oracle, name + "_forward")(x)
+        assert np.max(np.abs(y.numpy() - want)) <= TOL_RED * max(1.0, np.abs(want).max())
+        dwant = dev(hip, want)
+        hip.check(bwd(dwant.ptr, ddy.ptr, g.ptr, rows, cols))
+        gw = getattr(oracle, name + "_backward")(want, dy)
+        assert np.max(np.abs(g.numpy() - gw)) <= TOL_RED * max(1.0, np.abs(gw).max())
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 10), (8, 10), (5, 130)])
+def test_fused_softmax_ce_matches_tape_chain(hip, oracle, rng, rows, cols):
+    z = (2 * rng.standard_normal((rows, cols))).astype(np.float32)
+    labels = rng.integers(0, cols, rows).astype(np.int32)
+    onehot = np.zeros((rows, cols), np.float32)
+    onehot[np.arange(rows), labels] = 1
+    loss_want, dz_want = oracle.ce_chain(z, onehot)
+    dz, loss = hip.empty((rows, cols)), hip.empty(1)
+    dlabels = hip.to_device(labels)
+    hip.check(hip.bh_softmax_ce_grad(dev(hip, z).ptr, dlabels.ptr, dz.ptr, loss.ptr, rows, cols))
+    assert abs(loss.numpy()[0] - loss_want) <= TOL_RED * abs(loss_want)
+    assert np.max(np.abs(dz.numpy() - dz_want)) <= TOL_EW * np.abs(dz_want).max() + 1e-9
+    # closed form: (softmax - onehot)/B
+    p = np.exp(z.astype(np.float64) - z.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    assert np.allclose(dz.numpy(), (p - onehot) / rows, atol=1e-7)
+
+
+# ---------------------------------------------------------------- layernorm
+
+LN_SHAPES = [(1, 4), (7, 64), (10, 48), (33, 768), (64, 1024), (17, 4096), (5, 8192), (6, 50), (3, 9000)]
+
+
+@pytest.mark.parametrize("rows,hidden", LN_SHAPES)
+def test_layernorm_forward(hip, oracle, rng, rows, hidden):
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    y, mean, rstd = hip.empty((rows, hidden)), hip.empty(rows), hip.empty(rows)
+    hip.check(hip.bh_layernorm_forward(dev(hip, x).ptr, dev(hip, gamma).ptr, dev(hip, beta).ptr, y.ptr, mean.ptr, rstd.ptr,
+                                       rows, hidden, 1e-5))
+    wy, wm, wr = oracle.layernorm_forward(x, gamma, beta, 1e-5)
+    assert np.max(np.abs(y.numpy() - wy)) <= TOL_RED * np.abs(wy).max()
+    assert np.max(np.abs(mean.numpy() - wm)) <= 1e-6 and max_rel(rstd.numpy(), wr) <= TOL_RED
+    # no affine
+    hip.check(hip.bh_layernorm_forward(dev(hip, x).ptr, None, None, y.ptr, None, None, rows, hidden, 1e-5))
+    wy, _, _ = oracle.layernorm_forward(x, None, None, 1e-5)
+    assert np.max(np.abs(y.numpy() - wy)) <= TOL_RED * np.abs(wy).max()
+
+
+@pytest.mark.parametrize("rows,hidden", LN_SHAPES + [(1000, 1024), (300, 4096)])
+def test_layernorm_backward(hip, oracle, rng, rows, hidden):
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    dy = rng.standard_normal((rows, hidden)).astype(np.float32)
+    _, mean, rstd = oracle.layernorm_forward(x, gamma, None, 1e-5)
+    dx, dg, db = hip.empty((rows, hidden)), hip.zeros(hidden), hip.zeros(hidden)
+    args = (dev(hip, x).ptr, dev(hip, gamma).ptr, dev(hip, dy).ptr, dev(hip, mean).ptr, dev(hip, rstd).ptr)
+    hip.check(hip.bh_layernorm_backward(*args, dx.ptr, dg.ptr, db.ptr, rows, hidden, 0))
+    wdx, wdg, wdb = oracle.layernorm_backward_f64(x, gamma, dy, mean, rstd)
+    assert np.max(np.abs(dx.numpy() - wdx)) <= TOL_RED * np.abs(wdx).max()
+    assert np.max(np.abs(dg.numpy() - wdg)) <= TOL_RED * max(1.0, np.abs(wdg).max())
+    assert np.max(np.abs(db.numpy() - wdb)) <= TOL_RED * max(1.0, np.abs(wdb).max())
+    # accumulate into the parameter gradients
+    hip.check(hip.bh_layernorm_backward(*args, dx.ptr, dg.ptr, db.ptr, rows, hidden, 1))
+    assert np.max(np.abs(dg.numpy() - 2 * wdg)) <= 2 * TOL_RED * max(1.0, np.abs(wdg).max())
+    assert np.max(np.abs(db.numpy() - 2 * wdb)) <= 2 * TOL_RED * max(1.0, np.abs(wdb).max())
+
+
+# --------------------------------------------------------------------- gemm
+
+def gemm_case(hip, rng, ta, tb, m, n, k, accumulate=False, bias=False, batch=1, force=None):
+    a = rng.standard_normal((batch, k, m) if ta else (batch, m, k)).astype(np.float32)
+    b = rng.standard_normal((batch, n, k) if tb else (batch, k, n)).astype(np.float32)
+    c0 = rng.standard_normal((batch, m, n)).astype(np.float32)
+    bv = rng.standard_normal(n).astype(np.float32) if bias else None
+    A = a.transpose(0, 2, 1) if ta else a
+    B = b.transpose(0, 2, 1) if tb else b
+    want = np.matmul(A.astype(np.float64), B.astype(np.float64))
+    if bias:
+        want = want + bv
+    if accumulate:
+        want = want + c0
+    dc = dev(hip, c0)
+    if force is not None:
+        hip.bh_gemm_force_config(force)
+    try:
+        hip.check(hip.bh_gemm(int(ta), int(tb), m, n, k, dev(hip, a).ptr, a.shape[2], dev(hip, b).ptr, b.shape[2], dc.ptr, n,
+                              dev(hip, bv).ptr if bias else None, int(accumulate), batch))
+    finally:
+        hip.bh_gemm_force_config(-1)
+    got = dc.numpy()
+    assert rel_fro(got, want) <= TOL_GEMM, (ta, tb, m, n, k, rel_fro(got, want))
+    return got, want
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 784), (64, 784, 128), (784, 128, 64), (64, 10, 128), (128, 10, 64),
+                                   (64, 128, 10), (1, 1, 1), (33, 17, 5), (256, 256, 64), (384, 640, 200),
+                                   (512, 512, 512), (300, 260, 1028)])
+def test_gemm_heuristic_path(hip, rng, ta, tb, m, n, k):
+    gemm_case(hip, rng, ta, tb, m, n, k)
+
+
+@pytest.mark.parametrize("force", [1, 2])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 16), (256, 512, 64), (128, 128, 8), (260, 132, 36), (512, 768, 100), (1024, 1024, 256)])
+def test_gemm_mfma_tiles(hip, rng, force, ta, tb, m, n, k):
+    gemm_case(hip, rng, ta, tb, m, n, k, force=force)
+
+
+def test_gemm_epilogues_and_batch(hip, rng):
+    gemm_case(hip, rng, 0, 0, 256, 384, 128, bias=True)
+    gemm_case(hip, rng, 1, 0, 384, 256, 128, accumulate=True)
+    gemm_case(hip, rng, 0, 1, 130, 70, 64, accumulate=True, bias=True)
+    gemm_case(hip, rng, 0, 0, 128, 128, 64, batch=6)
+    gemm_case(hip, rng, 0, 0, 5, 4, 6, batch=6)                      # the [2,3,5,4].[2,3,4,6] layout case
+    gemm_case(hip, rng, 1, 0, 256, 256, 4096, accumulate=True)       # split-K with accumulation
+    gemm_case(hip, rng, 1, 0, 128, 384, 2048, bias=True)             # split-K with bias
+
+
+def test_gemm_matches_reference_loop_order_within_tolerance(hip, oracle, rng):
+    a = rng.standard_normal((96, 200)).astype(np.float32)
+    b = rng.standard_normal((200, 160)).astype(np.float32)
+    c = hip.empty((96, 160))
+    hip.check(hip.bh_gemm(0, 0, 96, 160, 200, dev(hip, a).ptr, 200, dev(hip, b).ptr, 160, c.ptr, 160, None, 0, 1))
+    assert rel_fro(c.numpy(), oracle.matmul(a, b)) <= TOL_GEMM
+
+
+@pytest.mark.parametrize("m,k,n", [(9, 13, 6), (64, 784, 128), (64, 128, 10), (512, 256, 384)])
+def test_dense_backward_entry_point(hip, oracle, rng, m, k, n):
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    dy = rng.standard_normal((m, n)).astype(np.float32)
+    gw0 = rng.standard_normal((k, n)).astype(np.float32)
+    gb0 = rng.standard_normal(n).astype(np.float32)
+    dx, gw, gb = hip.empty((m, k)), dev(hip, gw0), dev(hip, gb0)
+    hip.check(hip.bh_dense_backward(dev(hip, x).ptr, dev(hip, w).ptr, dev(hip, dy).ptr, dx.ptr, gw.ptr, gb.ptr, m, k, n, 1))
+    wdx, wgw, wgb = oracle.dense_backward(x, w, dy, gw0, gb0)
+    assert rel_fro(dx.numpy(), wdx) <= TOL_GEMM and rel_fro(gw.numpy(), wgw) <= TOL_GEMM
+    assert np.max(np.abs(gb.numpy() - wgb)) <= TOL_RED * max(1.0, np.abs(wgb).max())
+    # invariant: db == column sum of dY
+    hip.check(hip.bh_dense_backward(dev(hip, x).ptr, dev(hip, w).ptr, dev(hip, dy).ptr, dx.ptr, gw.ptr, gb.ptr, m, k, n, 0))
+    assert np.allclose(gb.numpy(), dy.sum(0), rtol=1e-4, atol=1e-4)
+
+
+def test_transpose(hip, oracle, rng):
+    a = rng.standard_normal((3, 45, 70)).astype(np.float32)
+    out = hip.empty((3, 70, 45))
+    hip.check(hip.bh_transpose_last2(dev(hip, a).ptr, out.ptr, 3, 45, 70))
+    assert np.array_equal(out.numpy(), oracle.transpose_last2(a))
+
+
+# ---------------------------------------------------------------- attention
+
+SDPA_SHAPES = [(8, 4, 8), (4, 16, 16), (2, 8, 8), (3, 33, 20), (2, 64, 64), (4, 128, 64), (2, 256, 64), (3, 100, 64)]
+
+
+@pytest.mark.parametrize("causal", [0, 1])
+@pytest.mark.parametrize("bh,s,d", SDPA_SHAPES)
+@pytest.mark.parametrize("general", [0, 1])
+def test_sdpa_forward_backward(hip, oracle, rng, bh, s, d, causal, general):
+    q, k, v, go = (rng.standard_normal((bh, s, d)).astype(np.float32) for _ in range(4))
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(d)))
+    wo, wlse, wattn = oracle.sdpa_forward(q, k, v, scale, causal)
+    wdq, wdk, wdv = oracle.sdpa_backward(q, k, v, wattn, go, scale)
+    dq_, dk_, dv_ = dev(hip, q), dev(hip, k), dev(hip, v)
+    out, lse = hip.empty((bh, s, d)), hip.empty((bh, s))
+    hip.bh_sdpa_force_general(general)
+    try:
+        hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, causal, out.ptr, lse.ptr, None, bh, s, d))
+        assert rel_fro(out.numpy(), wo) <= TOL_GEMM
+        assert np.max(np.abs(lse.numpy() - wlse)) <= 1e-4
+        gq, gk, gv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
+        hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, out.ptr, lse.ptr, dev(hip, go).ptr, scale, causal,
+                                       gq.ptr, gk.ptr, gv.ptr, bh, s, d))
+    finally:
+        hip.bh_sdpa_force_general(0)
+    assert rel_fro(gq.numpy(), wdq) <= TOL_GEMM and rel_fro(gk.numpy(), wdk) <= TOL_GEMM and rel_fro(gv.numpy(), wdv) <= TOL_GEMM
+
+
+def test_sdpa_attention_matrix_output(hip, oracle, rng):
+    bh, s, d = 3, 12, 8
+    q, k, v = (rng.standard_normal((bh, s, d)).astype(np.float32) for _ in range(3))
+    out, lse, attn = hip.empty((bh, s, d)), hip.empty((bh, s)), hip.empty((bh, s, s))
+    hip.check(hip.bh_sdpa_forward(dev(hip, q).ptr, dev(hip, k).ptr, dev(hip, v).ptr, 0.35, 0, out.ptr, lse.ptr, attn.ptr, bh, s, d))
+    _, _, wattn = oracle.sdpa_forward(q, k, v, 0.35)
+    assert np.max(np.abs(attn.numpy() - wattn)) <= 1e-6
+    assert np.allclose(attn.numpy().sum(-1), 1.0, atol=1e-5)

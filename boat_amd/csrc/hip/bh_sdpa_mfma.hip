@@ -1,7 +1,474 @@
-// placeholder until the MFMA attention kernels land: reports "shape not covered"
+// bh_sdpa_mfma.hip - attention core on the fp32 matrix cores for head_dim 64 (seq % 128 == 0).
+//
+// Same mathematics as the reference's scaled_dot_product_attention_impl / attention_backward
+// (src/layers/attention.c:997-1073, 1417-1520) on one [s, 64] block per (batch, head):
+//   forward   P = softmax(scale * Q.K^T)  (causal: keys after the query are masked), O = P.V,
+//             lse = rowmax + log(rowsum)
+//   backward  P = exp(scale*Q.K^T - lse) recomputed; dV = P^T.dO; dP = dO.V^T;
+//             dS = P*(dP - delta)*scale with delta = rowsum(dO*O); dQ = dS.K; dK = dS^T.Q
+// The [s, s] matrices never exist in memory.
+//
+// Every contraction is a chain of v_mfma_f32_32x32x2_f32.  Operand roles are chosen so that a product
+// leaves the accumulator already in the register layout the next product needs as an input:
+//   forward: S^T = K.Q^T puts "query = lane, key = register", which is exactly the B operand of
+//            O^T = V^T.P^T; all per-query state (running max, sum, the O^T accumulator) lives in the
+//            query's own lane, so the online-softmax rescale is a per-lane multiply.
+//   backward: S = Q.K^T and dP = dO.V^T put "key = lane, query = register", the A operand of
+//            dV += P^T.dO and dK += dS^T.Q; only dQ = dS.K needs dS with "query = lane", which is one
+//            32x32 transpose per wavefront through LDS.  dK/dV accumulate in registers over the loop
+//            on query tiles.  The dQ contributions of a workgroup's four wavefronts are exchanged
+//            through LDS, summed, and written as one partial per (key tile, query tile); a second
+//            kernel sums the s/128 partials.  No atomics anywhere, so dQ is deterministic.
+// Any order of the contraction index is a valid sum, so the index order inside a chain is whatever the
+// register layout gives; operands fetched from LDS use 16-byte reads along head_dim (row stride 68
+// floats, conflict free) or 8-byte reads that hand one lane two interleaved output columns.
 #include "bh_common.h"
+
 namespace bh {
-int sdpa_forward_mfma(const float*, const float*, const float*, float, int, float*, float*, int64_t, int64_t, int64_t) { return 1; }
-int sdpa_backward_mfma(const float*, const float*, const float*, const float*, const float*, const float*, float, int,
-                       float*, float*, float*, int64_t, int64_t, int64_t) { return 1; }
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kD = 64;         // head_dim
+constexpr int kLd = 68;        // LDS row stride in floats (64 + 4 pad)
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
+
+__device__ __forceinline__ floatx16 zero16() {
+    floatx16 z;
+#pragma unroll
+    for (int e = 0; e < 16; e++) z[e] = 0.f;
+    return z;
 }
+// row index inside a 32x32 accumulator tile held by register e of a lane in half `half`
+__device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + half * 4 + (e & 3); }
+
+// ------------------------------------------------------------------ forward
+// grid (s/128, bh); 4 wavefronts, each owns 32 queries; key/value tiles of 64 rows double-buffered in LDS.
+template <bool CAUSAL>
+__global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                            const float* __restrict__ v, float* __restrict__ out,
+                                                            float* __restrict__ lse, int s, float scale_log2e) {
+    extern __shared__ __align__(16) float smem[];
+    constexpr int KT = 64;                       // keys per tile
+    constexpr int TILE = KT * kLd;               // floats per K or V tile in LDS
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int64_t head = blockIdx.y;
+    const float* qh = q + head * s * kD;
+    const float* kh = k + head * s * kD;
+    const float* vh = v + head * s * kD;
+    const int q0 = blockIdx.x * 128 + w * 32;    // first query of this wavefront
+    const int my_q = q0 + r;
+
+    // this lane's query row, pre-scaled so that scores come out in log2 units: step (g, e) <-> d = 8g + 4*half + e
+    float qreg[32];
+#pragma unroll
+    for (int g = 0; g < 8; g++) {
+        const float4 t = *reinterpret_cast<const float4*>(qh + (int64_t)my_q * kD + 8 * g + 4 * half);
+        qreg[4 * g + 0] = t.x * scale_log2e;
+        qreg[4 * g + 1] = t.y * scale_log2e;
+        qreg[4 * g + 2] = t.z * scale_log2e;
+        qreg[4 * g + 3] = t.w * scale_log2e;
+    }
+    floatx16 acc_o[2] = {zero16(), zero16()};    // O^T: [d tile][...]; d = 2*row + tile, query = lane
+    float m_run = -INFINITY, l_run = 0.f;
+
+    int n_tiles = s / KT;
+    if (CAUSAL) {
+        const int last = (blockIdx.x * 128 + 127) / KT + 1;   // tiles that hold a key <= the last query of the workgroup
+        if (last < n_tiles) n_tiles = last;
+    }
+    // global -> register staging: 1024 float4 per tile and operand, 4 per lane (macros, not lambdas:
+    // the staging registers must stay registers)
+    float4 kst0, kst1, kst2, kst3, vst0, vst1, vst2, vst3;
+#define FWD_LD(i, K, V)                                                                                   \
+    {                                                                                                     \
+        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+        K = *reinterpret_cast<const float4*>(kh + (int64_t)(jt_ld * KT + row) * kD + c4 * 4);             \
+        V = *reinterpret_cast<const float4*>(vh + (int64_t)(jt_ld * KT + row) * kD + c4 * 4);             \
+    }
+#define FWD_ST(i, K, V)                                                                                   \
+    {                                                                                                     \
+        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+        *reinterpret_cast<float4*>(st_base + row * kLd + c4 * 4) = K;                                     \
+        *reinterpret_cast<float4*>(st_base + TILE + row * kLd + c4 * 4) = V;                              \
+    }
+#define FWD_STAGE_LOAD(JT) { const int jt_ld = (JT); FWD_LD(0, kst0, vst0) FWD_LD(1, kst1, vst1) FWD_LD(2, kst2, vst2) FWD_LD(3, kst3, vst3) }
+#define FWD_STAGE_STORE(BUF) { float* st_base = smem + (BUF) * 2 * TILE; FWD_ST(0, kst0, vst0) FWD_ST(1, kst1, vst1) FWD_ST(2, kst2, vst2) FWD_ST(3, kst3, vst3) }
+    FWD_STAGE_LOAD(0)
+    FWD_STAGE_STORE(0)
+    __syncthreads();
+
+    for (int jt = 0; jt < n_tiles; jt++) {
+        const int cur = jt & 1;
+        const bool more = jt + 1 < n_tiles;
+        if (more) FWD_STAGE_LOAD(jt + 1)
+        const float* ks = smem + cur * 2 * TILE;
+        const float* vs = ks + TILE;
+        // a wavefront whose queries all precede this tile's keys has nothing to add
+        if (!CAUSAL || jt * KT <= q0 + 31) {
+            floatx16 acc_s[2] = {zero16(), zero16()};   // S^T: key = row (tile*32 + acc_row), query = lane
+#pragma unroll
+            for (int g = 0; g < 8; g++) {
+                const float4 a0 = *reinterpret_cast<const float4*>(ks + r * kLd + 8 * g + 4 * half);
+                const float4 a1 = *reinterpret_cast<const float4*>(ks + (32 + r) * kLd + 8 * g + 4 * half);
+                acc_s[0] = MFMA(a0.x, qreg[4 * g + 0], acc_s[0]);
+                acc_s[1] = MFMA(a1.x, qreg[4 * g + 0], acc_s[1]);
+                acc_s[0] = MFMA(a0.y, qreg[4 * g + 1], acc_s[0]);
+                acc_s[1] = MFMA(a1.y, qreg[4 * g + 1], acc_s[1]);
+                acc_s[0] = MFMA(a0.z, qreg[4 * g + 2], acc_s[0]);
+                acc_s[1] = MFMA(a1.z, qreg[4 * g + 2], acc_s[1]);
+                acc_s[0] = MFMA(a0.w, qreg[4 * g + 3], acc_s[0]);
+                acc_s[1] = MFMA(a1.w, qreg[4 * g + 3], acc_s[1]);
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    if (CAUSAL) {
+                        const int key = jt * KT + t * 32 + acc_row(e, half);
+                        if (key > my_q) acc_s[t][e] = -INFINITY;
+                    }
+                    mx = fmaxf(mx, acc_s[t][e]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);      // finite: key 0 is never masked and tiles are visited in order
+            const float alpha = exp2f(m_run - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const float p = exp2f(acc_s[t][e] - m_new);
+                    acc_s[t][e] = p;
+                    psum += p;
+                }
+            psum += __shfl_xor(psum, 32, 64);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc_o[t][e] *= alpha;
+            // O^T += V^T . P^T : step e of key tile t uses key row t*32 + acc_row(e, half)
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int key = t * 32 + acc_row(e, half);
+                    const float2 a = *reinterpret_cast<const float2*>(vs + key * kLd + 2 * r);
+                    acc_o[0] = MFMA(a.x, acc_s[t][e], acc_o[0]);
+                    acc_o[1] = MFMA(a.y, acc_s[t][e], acc_o[1]);
+                }
+        }
+        if (more) FWD_STAGE_STORE(cur ^ 1)
+        __syncthreads();
+    }
+#undef FWD_LD
+#undef FWD_ST
+#undef FWD_STAGE_LOAD
+#undef FWD_STAGE_STORE
+
+    // O = O^T / l, transposed through LDS so that rows are written whole
+    const float inv_l = 1.0f / l_run;
+    float* os = smem + w * 32 * kLd;             // 32 x 68 floats per wavefront, tiles are no longer needed
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) os[r * kLd + 2 * acc_row(e, half) + t] = acc_o[t][e] * inv_l;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float* oh = out + head * s * kD;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int row = it * 4 + (lane >> 4), c4 = lane & 15;
+        const float4 val = *reinterpret_cast<const float4*>(os + row * kLd + c4 * 4);
+        *reinterpret_cast<float4*>(oh + (int64_t)(q0 + row) * kD + c4 * 4) = val;
+    }
+    if (half == 0) lse[head * s + my_q] = (m_run + log2f(l_run)) * kLn2;
+}
+
+// ----------------------------------------------------------------- backward
+// grid (s/128, bh); 4 wavefronts, each owns 32 keys (dK, dV rows) and loops over query tiles of 32.
+// LDS: per wavefront its K and V rows and a 32x33 transpose pad; per workgroup two buffers of the
+// current Q and dO tiles plus their lse/delta.
+struct BwdSmem {
+    static constexpr int KV = 4 * 32 * kLd;             // K (or V) rows of the four wavefronts
+    static constexpr int QT = 32 * kLd;                 // one Q (or dO) tile
+    static constexpr int TP = 4 * 32 * 33;              // transpose pads
+    static constexpr int OFF_K = 0;
+    static constexpr int OFF_V = OFF_K + KV;
+    static constexpr int OFF_Q = OFF_V + KV;            // [2][QT]
+    static constexpr int OFF_DO = OFF_Q + 2 * QT;       // [2][QT]
+    static constexpr int OFF_T = OFF_DO + 2 * QT;
+    static constexpr int OFF_STAT = OFF_T + TP;         // [2][2][32]: lse*log2e, delta
+    static constexpr int OFF_DQ = OFF_STAT + 2 * 2 * 32; // [4][32][kLd] dQ tiles of the four wavefronts
+    static constexpr int TOTAL = OFF_DQ + 4 * 32 * kLd;
+};
+
+template <bool CAUSAL>
+__global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                            const float* __restrict__ v, const float* __restrict__ lse,
+                                                            const float* __restrict__ delta, const float* __restrict__ d_out,
+                                                            float* __restrict__ dq_partial, float* __restrict__ dk,
+                                                            float* __restrict__ dv, int s, float scale) {
+    extern __shared__ __align__(16) float smem[];
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int64_t head = blockIdx.y;
+    const float* qh = q + head * s * kD;
+    const float* kh = k + head * s * kD;
+    const float* vh = v + head * s * kD;
+    const float* gh = d_out + head * s * kD;
+    const float* lh = lse + head * s;
+    const float* dh = delta + head * s;
+    // partial dQ of this key tile: [key tile][bh][s][64]
+    float* dqh = dq_partial + ((int64_t)blockIdx.x * gridDim.y + head) * s * kD;
+    float* dq_mine = smem + BwdSmem::OFF_DQ + w * 32 * kLd;
+    const int kv_wg = blockIdx.x * 128;          // first key of the workgroup
+    const int kv0 = kv_wg + w * 32;              // first key of this wavefront
+    const float c1 = scale * kLog2e;
+
+    float* ks = smem + BwdSmem::OFF_K + w * 32 * kLd;
+    float* vs = smem + BwdSmem::OFF_V + w * 32 * kLd;
+    float* tp = smem + BwdSmem::OFF_T + w * 32 * 33;
+    // this wavefront's K and V rows -> LDS (each lane: 8 float4 per operand)
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int idx = lane + i * 64, row = idx >> 4, c4 = idx & 15;
+        *reinterpret_cast<float4*>(ks + row * kLd + c4 * 4) =
+            *reinterpret_cast<const float4*>(kh + (int64_t)(kv0 + row) * kD + c4 * 4);
+        *reinterpret_cast<float4*>(vs + row * kLd + c4 * 4) =
+            *reinterpret_cast<const float4*>(vh + (int64_t)(kv0 + row) * kD + c4 * 4);
+    }
+
+    floatx16 acc_dk[2] = {zero16(), zero16()};   // [d tile]: key = acc_row, d = 2*lane + tile
+    floatx16 acc_dv[2] = {zero16(), zero16()};
+
+    const int n_qt = s / 32;
+    const int first_qt = CAUSAL ? kv_wg / 32 : 0;   // earlier query tiles see none of this workgroup's keys
+    // their partial dQ rows are zero
+    for (int i = tid; i < first_qt * 32 * (kD / 4); i += 256)
+        reinterpret_cast<float4*>(dqh)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    // staging: a Q tile and a dO tile are 512 float4 each, 2 per lane and operand
+    float4 qst0, qst1, gst0, gst1;
+    float stat = 0.f;
+#define BWD_LD(i, Q, G)                                                                                   \
+    {                                                                                                     \
+        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+        Q = *reinterpret_cast<const float4*>(qh + (int64_t)(qt_ld * 32 + row) * kD + c4 * 4);             \
+        G = *reinterpret_cast<const float4*>(gh + (int64_t)(qt_ld * 32 + row) * kD + c4 * 4);             \
+    }
+#define BWD_ST(i, Q, G)                                                                                   \
+    {                                                                                                     \
+        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+        *reinterpret_cast<float4*>(q_base + row * kLd + c4 * 4) = Q;                                      \
+        *reinterpret_cast<float4*>(g_base + row * kLd + c4 * 4) = G;                                      \
+    }
+#define BWD_STAGE_LOAD(QT)                                                 \
+    {                                                                      \
+        const int qt_ld = (QT);                                            \
+        BWD_LD(0, qst0, gst0) BWD_LD(1, qst1, gst1)                        \
+        if (tid < 32) stat = lh[qt_ld * 32 + tid] * kLog2e;                \
+        else if (tid < 64) stat = dh[qt_ld * 32 + tid - 32];               \
+    }
+#define BWD_STAGE_STORE(BUF)                                               \
+    {                                                                      \
+        float* q_base = smem + BwdSmem::OFF_Q + (BUF) * BwdSmem::QT;       \
+        float* g_base = smem + BwdSmem::OFF_DO + (BUF) * BwdSmem::QT;      \
+        BWD_ST(0, qst0, gst0) BWD_ST(1, qst1, gst1)                        \
+        if (tid < 64) smem[BwdSmem::OFF_STAT + (BUF) * 64 + tid] = stat;   \
+    }
+    if (first_qt < n_qt) {
+        BWD_STAGE_LOAD(first_qt)
+        BWD_STAGE_STORE(0)
+    }
+    __syncthreads();
+
+    for (int qt = first_qt; qt < n_qt; qt++) {
+        const int cur = (qt - first_qt) & 1;
+        const bool more = qt + 1 < n_qt;
+        if (more) BWD_STAGE_LOAD(qt + 1)
+        const float* qs = smem + BwdSmem::OFF_Q + cur * BwdSmem::QT;
+        const float* gs = smem + BwdSmem::OFF_DO + cur * BwdSmem::QT;
+        const float* st = smem + BwdSmem::OFF_STAT + cur * 64;
+        const int q0 = qt * 32;
+        if (!CAUSAL || q0 + 31 >= kv0) {
+            // S = Q.K^T and dP = dO.V^T : query = row (acc_row), key = lane
+            floatx16 acc_s = zero16(), acc_dp = zero16();
+#pragma unroll
+            for (int g = 0; g < 8; g++) {
+                const int off = r * kLd + 8 * g + 4 * half;
+                const float4 aq = *reinterpret_cast<const float4*>(qs + off);
+                const float4 bk = *reinterpret_cast<const float4*>(ks + off);
+                const float4 ag = *reinterpret_cast<const float4*>(gs + off);
+                const float4 bv = *reinterpret_cast<const float4*>(vs + off);
+                acc_s = MFMA(aq.x, bk.x, acc_s);
+                acc_dp = MFMA(ag.x, bv.x, acc_dp);
+                acc_s = MFMA(aq.y, bk.y, acc_s);
+                acc_dp = MFMA(ag.y, bv.y, acc_dp);
+                acc_s = MFMA(aq.z, bk.z, acc_s);
+                acc_dp = MFMA(ag.z, bv.z, acc_dp);
+                acc_s = MFMA(aq.w, bk.w, acc_s);
+                acc_dp = MFMA(ag.w, bv.w, acc_dp);
+            }
+            // P and dS in place
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = acc_row(e, half);
+                float p = exp2f(acc_s[e] * c1 - st[row]);
+                if (CAUSAL && kv0 + r > q0 + row) p = 0.f;
+                acc_s[e] = p;
+                acc_dp[e] = p * (acc_dp[e] - st[32 + row]) * scale;
+            }
+            // dV += P^T.dO ; dK += dS^T.Q : step e contracts query row acc_row(e, half)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = acc_row(e, half);
+                const float2 bg = *reinterpret_cast<const float2*>(gs + row * kLd + 2 * r);
+                const float2 bq = *reinterpret_cast<const float2*>(qs + row * kLd + 2 * r);
+                acc_dv[0] = MFMA(acc_s[e], bg.x, acc_dv[0]);
+                acc_dv[1] = MFMA(acc_s[e], bg.y, acc_dv[1]);
+                acc_dk[0] = MFMA(acc_dp[e], bq.x, acc_dk[0]);
+                acc_dk[1] = MFMA(acc_dp[e], bq.y, acc_dk[1]);
+            }
+            // dS -> "query = lane" through the wavefront's pad
+#pragma unroll
+            for (int e = 0; e < 16; e++) tp[acc_row(e, half) * 33 + r] = acc_dp[e];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // dQ = dS.K : step e contracts key row acc_row(e, half)
+            floatx16 acc_dq[2] = {zero16(), zero16()};
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int key = acc_row(e, half);
+                const float a = tp[r * 33 + key];
+                const float2 bk = *reinterpret_cast<const float2*>(ks + key * kLd + 2 * r);
+                acc_dq[0] = MFMA(a, bk.x, acc_dq[0]);
+                acc_dq[1] = MFMA(a, bk.y, acc_dq[1]);
+            }
+            __builtin_amdgcn_wave_barrier();   // the pad is rewritten next iteration
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                *reinterpret_cast<float2*>(dq_mine + acc_row(e, half) * kLd + 2 * r) = make_float2(acc_dq[0][e], acc_dq[1][e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                *reinterpret_cast<float2*>(dq_mine + acc_row(e, half) * kLd + 2 * r) = make_float2(0.f, 0.f);
+        }
+        __syncthreads();
+        // sum of the four wavefronts' tiles -> this key tile's partial dQ (whole rows)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int idx = tid + i * 256, row = idx >> 4, c4 = idx & 15;
+            const float* src = smem + BwdSmem::OFF_DQ + row * kLd + c4 * 4;
+            const float4 t0 = *reinterpret_cast<const float4*>(src);
+            const float4 t1 = *reinterpret_cast<const float4*>(src + 32 * kLd);
+            const float4 t2 = *reinterpret_cast<const float4*>(src + 2 * 32 * kLd);
+            const float4 t3 = *reinterpret_cast<const float4*>(src + 3 * 32 * kLd);
+            float4 o;
+            o.x = (t0.x + t1.x) + (t2.x + t3.x);
+            o.y = (t0.y + t1.y) + (t2.y + t3.y);
+            o.z = (t0.z + t1.z) + (t2.z + t3.z);
+            o.w = (t0.w + t1.w) + (t2.w + t3.w);
+            *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + row) * kD + c4 * 4) = o;
+        }
+        if (more) BWD_STAGE_STORE(cur ^ 1)
+        __syncthreads();
+    }
+#undef BWD_LD
+#undef BWD_ST
+#undef BWD_STAGE_LOAD
+#undef BWD_STAGE_STORE
+
+    float* dkh = dk + head * s * kD;
+    float* dvh = dv + head * s * kD;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        const int64_t row = kv0 + acc_row(e, half);
+        *reinterpret_cast<float2*>(dkh + row * kD + 2 * r) = make_float2(acc_dk[0][e], acc_dk[1][e]);
+        *reinterpret_cast<float2*>(dvh + row * kD + 2 * r) = make_float2(acc_dv[0][e], acc_dv[1][e]);
+    }
+}
+
+// dq = sum over key tiles of the partials: out[i] = sum_t partial[t][i], float4 per lane, streamed
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void dq_partial_sum_kernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                             int64_t n4, int tiles) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    f32x4 acc = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partial) + i);
+    for (int t = 1; t < tiles; t++) acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partial) + (int64_t)t * n4 + i);
+    __builtin_nontemporal_store(acc, reinterpret_cast<f32x4*>(out) + i);
+}
+
+static bool mfma_shape(int64_t s, int64_t d) { return d == kD && s >= 128 && s % 128 == 0 && s <= (1 << 24); }
+
+int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
+                      int64_t bh_count, int64_t s, int64_t d) {
+    if (!mfma_shape(s, d)) return 1;
+    const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (!al(q) || !al(k) || !al(v) || !al(out)) return 1;
+    constexpr size_t lds = sizeof(float) * 2 * 2 * 64 * kLd;
+    static bool attr = false;
+    if (!attr) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc == BH_OK)
+            rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr = true;
+    }
+    dim3 grid((unsigned)(s / 128), (unsigned)bh_count);
+    if (causal)
+        hipLaunchKernelGGL(sdpa_fwd_mfma_kernel<true>, grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, scale * kLog2e);
+    else
+        hipLaunchKernelGGL(sdpa_fwd_mfma_kernel<false>, grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, scale * kLog2e);
+    return BH_LAUNCH_CHECK("sdpa_fwd_mfma_kernel");
+}
+
+int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
+                       const float* d_out, float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count,
+                       int64_t s, int64_t d) {
+    if (!mfma_shape(s, d)) return 1;
+    const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (!al(q) || !al(k) || !al(v) || !al(d_out) || !al(dq) || !al(dk) || !al(dv)) return 1;
+    constexpr size_t lds = sizeof(float) * BwdSmem::TOTAL;
+    static bool attr = false;
+    if (!attr) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc == BH_OK)
+            rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr = true;
+    }
+    const int tiles = (int)(s / 128);
+    const int64_t n = bh_count * s * d;
+    float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one key tile: dq itself
+    if (!partial) return BH_ENOMEM;
+    dim3 grid((unsigned)tiles, (unsigned)bh_count);
+    if (causal)
+        hipLaunchKernelGGL(sdpa_bwd_mfma_kernel<true>, grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk,
+                           dv, (int)s, scale);
+    else
+        hipLaunchKernelGGL(sdpa_bwd_mfma_kernel<false>, grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk,
+                           dv, (int)s, scale);
+    int rc = BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
+    if (tiles > 1) {
+        if (rc == BH_OK) {
+            const int64_t n4 = n / 4;
+            hipLaunchKernelGGL(dq_partial_sum_kernel, dim3((unsigned)ceil_div(n4, 256)), dim3(256), 0, stream(), partial, dq, n4, tiles);
+            rc = BH_LAUNCH_CHECK("dq_partial_sum_kernel");
+        }
+        bh_free(partial);
+    }
+    return rc;
+}
+
+}  // namespace bh

@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/*.npz: inputs and expected outputs of the training hot path.
+
+Reference-derived vectors come from the COMPILED REFERENCE (oracle/_ref/libboat_ref.so, built by
+oracle/Makefile from the reference's own C sources) driven through its public C API by
+tests/boat_cases.py -- the reference is C, so nothing of it is imported.  Two fixtures have no
+reference counterpart (the reference ships stubs): LayerNorm backward and GELU; their vectors
+come from an independent library, torch autograd in float64 on the CPU.
+
+Run from the repository root in a container that has the reference tree:
+    make -C oracle ref && python tests/golden/make_golden.py
+Fixtures are plain numpy archives (np.load with allow_pickle=False reads them).
+"""
+import sys
+from pathlib import Path
+
+import numpy as np
+
+HERE = Path(__file__).resolve().parent
+ROOT = HERE.parent.parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+import boat_cases as bc  # noqa: E402
+import oracle_lib  # noqa: E402
+from test_oracle_vs_reference import ATT_CASES, make_attention_inputs  # noqa: E402
+
+
+def save(name, **arrays):
+    path = HERE / f"{name}.npz"
+    np.savez_compressed(path, **{k: np.asarray(v) for k, v in arrays.items() if v is not None})
+    print(f"{path.name}: {path.stat().st_size / 1024:.1f} KiB, {len(arrays)} arrays")
+
+
+def main():
+    ref = oracle_lib.load_reference()
+    if ref is None:
+        sys.exit("oracle/_ref/libboat_ref.so is missing: run `make -C oracle ref` where the reference tree is present")
+    rng = np.random.default_rng(20250611)
+
+    # elementwise and activation gradients, [5,7], relu input contains exact zeros
+    el = {}
+    a = rng.standard_normal((5, 7)).astype(np.float32)
+    b = (rng.standard_normal((5, 7)) + 3).astype(np.float32)
+    dy = rng.standard_normal((5, 7)).astype(np.float32)
+    el.update(a=a, b=b, dy=dy)
+    for op in ("add", "sub", "mul", "div"):
+        c, da, db = bc.binary_grads(ref, op, a, b, dy)
+        el.update({f"{op}_out": c, f"{op}_da": da, f"{op}_db": db})
+    x = rng.standard_normal((5, 7)).astype(np.float32)
+    x[0, :3] = [0.0, -0.0, 1e-30]
+    el["x"] = x
+    for op in ("relu", "sigmoid", "tanh"):
+        y, dx = bc.unary_grads(ref, op, x, dy)
+        el.update({f"{op}_y": y, f"{op}_dx": dx})
+    s, ds = bc.unary_grads(ref, "sum", x)
+    el.update(sum_y=s, sum_dx=ds)
+    save("elementwise", **el)
+
+    sm = {}
+    for tag, shape in (("a", (6, 10)), ("b", (3, 33))):
+        x = (3 * rng.standard_normal(shape)).astype(np.float32)
+        dy = rng.standard_normal(shape).astype(np.float32)
+        sm.update({f"{tag}_x": x, f"{tag}_dy": dy})
+        for op in ("softmax", "log_softmax"):
+            y, dx = bc.unary_grads(ref, op, x, dy)
+            sm.update({f"{tag}_{op}_y": y, f"{tag}_{op}_dx": dx})
+    save("softmax", **sm)
+
+    a4 = rng.standard_normal((2, 3, 5, 4)).astype(np.float32)
+    b4 = rng.standard_normal((2, 3, 4, 6)).astype(np.float32)
+    a2 = rng.standard_normal((7, 5)).astype(np.float32)
+    b2 = rng.standard_normal((5, 9)).astype(np.float32)
+    dy2 = rng.standard_normal((7, 9)).astype(np.float32)
+    c2, da2, db2 = bc.matmul_grads(ref, a2, b2, dy2)
+    save("matmul", a4=a4, b4=b4, c4=bc.matmul(ref, a4, b4), a4_t23=bc.transpose(ref, a4, 2, 3),
+         a2=a2, b2=b2, dy2=dy2, c2=c2, da2=da2, db2=db2, a2_t01=bc.transpose(ref, a2, 0, 1))
+
+    m, k, n = 9, 13, 6
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    x1, x2 = (rng.standard_normal((m, k)).astype(np.float32) for _ in range(2))
+    dy1, dy2 = (rng.standard_normal((m, n)).astype(np.float32) for _ in range(2))
+    (dx1, gw1, gb1), (dx2, gw2, gb2) = bc.dense_backward_twice(ref, w, bias, x1, dy1, x2, dy2)
+    save("dense_bwd_accum", w=w, b=bias, x1=x1, x2=x2, dy1=dy1, dy2=dy2, y1=bc.dense_forward(ref, x1, w, bias),
+         dx1=dx1, gw1=gw1, gb1=gb1, dx2=dx2, gw2=gw2, gb2=gb2)
+
+    # config-1 chain: small MLP with full tensors over 3 Adam steps
+    d_in, d_h, d_out, batch = 20, 16, 10, 8
+    x = rng.random((batch, d_in), dtype=np.float32)
+    labels = rng.integers(0, d_out, batch)
+    w1 = rng.uniform(-0.4, 0.4, (d_in, d_h)).astype(np.float32)
+    w2 = rng.uniform(-0.4, 0.4, (d_h, d_out)).astype(np.float32)
+    b1, b2 = np.zeros(d_h, np.float32), np.zeros(d_out, np.float32)
+    hist = bc.mlp_ce_adam(ref, x, labels, w1, b1, w2, b2, steps=3)
+    arrays = dict(x=x, labels=labels, w1=w1, b1=b1, w2=w2, b2=b2)
+    for t, rec in enumerate(hist):
+        for key, val in rec.items():
+            arrays[f"s{t}_{key}"] = np.float32(val) if key == "loss" else val
+    save("mlp_small_3steps", **arrays)
+
+    # config 1 at its real size (784-128-10, batch 64, one step): inputs are regenerated from the seed,
+    # the large tensors are pinned by a few rows plus float64 checksums
+    seed = 20250101
+    r1 = np.random.default_rng(seed)
+    d_in, d_h, d_out, batch = 784, 128, 10, 64
+    x = r1.random((batch, d_in), dtype=np.float32)
+    labels = r1.integers(0, d_out, batch)
+    lim1, lim2 = np.sqrt(6.0 / (d_in + d_h)), np.sqrt(6.0 / (d_h + d_out))
+    w1 = r1.uniform(-lim1, lim1, (d_in, d_h)).astype(np.float32)
+    w2 = r1.uniform(-lim2, lim2, (d_h, d_out)).astype(np.float32)
+    b1, b2 = np.zeros(d_h, np.float32), np.zeros(d_out, np.float32)
+    rec = bc.mlp_ce_adam(ref, x, labels, w1, b1, w2, b2, steps=1)[0]
+
+    def chk(arr):
+        arr = np.asarray(arr, np.float64)
+        return np.array([arr.sum(), np.abs(arr).sum(), (arr * arr).sum()])
+
+    save("mlp_config1_step", seed=seed, labels=labels, input_checksums=np.stack([chk(x), chk(w1), chk(w2)]),
+         loss=np.float32(rec["loss"]), gb1=rec["gb1"], gb2=rec["gb2"], gw2=rec["gw2"], b1=rec["b1"], b2=rec["b2"], w2=rec["w2"],
+         gw1_rows=rec["gw1"][:4], w1_rows=rec["w1"][:4], gw1_chk=chk(rec["gw1"]), w1_chk=chk(rec["w1"]))
+
+    for i, case in enumerate(ATT_CASES):
+        xs, w, b, dys = make_attention_inputs(case, 99)
+        out, results = bc.attention(ref, *xs, w, b, case["heads"], case["causal"], dys)
+        arrays = dict(xq=xs[0], xk=xs[1], xv=xs[2], dy0=dys[0], dy1=dys[1], out=out,
+                      meta=np.array([case["B"], case["S"], case["H"], case["heads"], int(case["causal"]), int(case["bias"])]))
+        for nme in "qkvo":
+            arrays["w" + nme] = w[nme]
+            if b is not None:
+                arrays["b" + nme] = b[nme]
+        for t, rec in enumerate(results):
+            for key, val in rec.items():
+                if val is not None:
+                    arrays[f"c{t}_{key}"] = val
+        save(f"attention_case{i}", **arrays)
+
+    # bare SDPA through identity projections (head split = plain reshape, scale on the scores, double row-dot)
+    B, S, H, heads = 1, 8, 16, 2
+    xs = [rng.standard_normal((B, S, H)).astype(np.float32) for _ in range(3)]
+    eye = {nme: np.eye(H, dtype=np.float32) for nme in "qkvo"}
+    dy = rng.standard_normal((B, S, H)).astype(np.float32)
+    out, (rec,) = bc.attention(ref, *xs, eye, None, heads, False, [dy])
+    save("sdpa_core", xq=xs[0], xk=xs[1], xv=xs[2], dy=dy, out=out, dq=rec["dq"], dk=rec["dk"], dv=rec["dv"],
+         meta=np.array([B, S, H, heads]))
+
+    ln = {}
+    for tag, shape in (("a", (2, 5, 48)), ("b", (7, 64))):
+        x = rng.standard_normal(shape).astype(np.float32)
+        gamma = (1 + 0.1 * rng.standard_normal(shape[-1])).astype(np.float32)
+        beta = (0.1 * rng.standard_normal(shape[-1])).astype(np.float32)
+        ln.update({f"{tag}_x": x, f"{tag}_gamma": gamma, f"{tag}_beta": beta,
+                   f"{tag}_y": bc.layernorm_forward(ref, x, gamma, beta, 1e-5)})
+    save("layernorm_fwd", **ln)
+
+    shapes = [(4, 3), (7,), (1,)]
+    params = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    grads = [[(rng.standard_normal(s) * 10 ** rng.uniform(-4, 1)).astype(np.float32) for s in shapes] for _ in range(10)]
+    traj, _ = bc.adam_trajectory(ref, params, grads, lr=1e-2, lr_change=(5, 3e-3))
+    arrays = {}
+    for i in range(3):
+        arrays[f"p{i}"] = params[i]
+        arrays[f"g{i}"] = np.stack([g[i] for g in grads])
+        arrays[f"traj{i}"] = np.stack([t[i] for t in traj])
+    save("adam_traj", **arrays)
+
+    a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
+    da, db = bc.fanout(ref, a, b)
+    save("fanout_divergence", a=a, b=b, ref_da=da, ref_db=db)
+
+    # ---- not the reference: float64 autograd of an independent library ----
+    import torch
+    torch.manual_seed(0)
+    x = torch.randn(9, 64, dtype=torch.float64, requires_grad=True)
+    gamma = (1 + 0.1 * torch.randn(64, dtype=torch.float64)).requires_grad_()
+    beta = (0.1 * torch.randn(64, dtype=torch.float64)).requires_grad_()
+    dy = torch.randn(9, 64, dtype=torch.float64)
+    y = torch.nn.functional.layer_norm(x, (64,), gamma, beta, 1e-5)
+    y.backward(dy)
+    save("ln_bwd_ref64", x=x.detach().numpy(), gamma=gamma.detach().numpy(), beta=beta.detach().numpy(), dy=dy.numpy(),
+         y=y.detach().numpy(), dx=x.grad.numpy(), dgamma=gamma.grad.numpy(), dbeta=beta.grad.numpy())
+    x = (2 * torch.randn(9, 64, dtype=torch.float64)).requires_grad_()
+    y = torch.nn.functional.gelu(x, approximate="none")
+    y.backward(dy)
+    save("gelu_ref64", x=x.detach().numpy(), dy=dy.numpy(), y=y.detach().numpy(), dx=x.grad.numpy())
+
+
+if __name__ == "__main__":
+    main()

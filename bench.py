@@ -169,6 +169,13 @@ def bench_extra(hip, steps, warmup):
     gbs = nbytes / (ms * 1e-3) / 1e9
     out["gelu_bwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
                                   "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    # streaming copy of known size (read 256 MiB, write 256 MiB): the practical HBM ceiling on this part and the
+    # calibration kernel for the FETCH_SIZE / WRITE_SIZE counters
+    ms = time_steps(hip, lambda: hip.check(hip.bh_scalar_op(2, x.ptr, 1.0, dx.ptr, R * H)), steps, warmup)
+    nbytes = 2 * 4 * R * H
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out["stream_copy_256MiB"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
+                                 "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
     del x, dy, y, dx
 
     # config 4: attention core backward, B8 h16 S1024 D64 (credited flops: dV, dP, dQ, dK contractions)
@@ -235,6 +242,87 @@ def bench_mlp_step(steps, warmup):
     api.sync()
     return {"ms": round((time.perf_counter() - t0) * 1e3 / steps, 4), "bound": "launch latency",
             "note": "MLP 784-128-10 B64 fwd+bwd+Adam through boat_var_* / boat_variable_backward_full / boat_optimizer_step, wall clock"}
+
+
+def bench_block_step(steps, warmup):
+    """Config 5a through Boat's C API: pre-LN encoder block d_model 1024, 16 heads, FFN 4096 (GELU), seq 512, batch 16;
+    forward + boat_variable_backward + fused Adam over the block's 12,596,224 parameters (16 tensors), wall ms."""
+    from boat_amd.capi import AttentionConfig, LayerNormConfig, default_api
+    api = default_api()
+    rng = np.random.default_rng(20250105)
+    B, S, H, heads, ffn = 16, 512, 1024, 16, 4096
+    T = B * S
+
+    def normal(shape, std):
+        return (std * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
+
+    ln = []
+    for _ in range(2):
+        cfg = LayerNormConfig(H, 1e-5, True, True)
+        ln.append(api.boat_layernorm_create(C.byref(cfg)))          # gamma = 1, beta = 0
+    cfg = AttentionConfig(H, heads, H // heads, 0.0, False, True, False, 10000.0)
+    att = api.boat_attention_create(C.byref(cfg))
+    for n in "qkvo":
+        api.write(getattr(api, f"boat_attention_get_weight_{n}")(att), normal((H, H), 0.02))
+    d1 = api.boat_dense_layer_create(H, ffn, True)
+    d2 = api.boat_dense_layer_create(ffn, H, True)
+    api.write(api.boat_dense_layer_get_weight(d1), normal((H, ffn), 0.02))
+    api.write(api.boat_dense_layer_get_weight(d2), normal((ffn, H), 0.02))
+    opt = api.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
+    api.boat_hip_optimizer_add_layernorm(opt, ln[0])
+    api.boat_hip_optimizer_add_attention(opt, att)
+    api.boat_hip_optimizer_add_layernorm(opt, ln[1])
+    api.boat_hip_optimizer_add_dense(opt, d1)
+    api.boat_hip_optimizer_add_dense(opt, d2)
+    tx = api.tensor(normal((B, S, H), 1.0))
+    tt = api.tensor(normal((B, S, H), 1.0))
+    shape2 = (C.c_int64 * 2)(T, H)
+    shape3 = (C.c_int64 * 3)(B, S, H)
+    losses = []
+
+    def step(keep_loss=False):
+        vx = api.boat_variable_create(tx, True)
+        h1 = api.boat_hip_var_layernorm(vx, ln[0])
+        a = api.boat_var_attention(h1, h1, h1, att, None)
+        x1 = api.boat_var_add(vx, a)
+        h2 = api.boat_hip_var_layernorm(x1, ln[1])
+        h2f = api.boat_hip_var_reshape(h2, shape2, 2)
+        f1 = api.boat_var_dense(h2f, d1)
+        g1 = api.boat_hip_var_gelu(f1)
+        f2 = api.boat_var_dense(g1, d2)
+        f2r = api.boat_hip_var_reshape(f2, shape3, 3)
+        y = api.boat_var_add(x1, f2r)
+        grad = C.c_void_p()
+        tloss = api.boat_hip_mse_loss(api.boat_variable_data(y), tt, C.byref(grad))
+        assert tloss and grad, "block forward failed"
+        api.boat_variable_backward(y, grad)
+        api.boat_optimizer_step(opt)
+        api.boat_optimizer_zero_grad(opt)
+        if keep_loss:
+            losses.append(float(api.numpy(tloss)[0]))
+        api.boat_tensor_unref(tloss)
+        api.boat_tensor_unref(grad)
+        for v in (y, f2r, f2, g1, f1, h2f, h2, x1, a, h1, vx):
+            api.boat_variable_free(v)
+
+    step(keep_loss=True)
+    for _ in range(max(warmup - 1, 1)):
+        step()
+    api.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.sync()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    step(keep_loss=True)
+    assert np.isfinite(losses).all() and losses[1] < losses[0], f"block training does not reduce the loss: {losses}"
+    flops = 2.0 * T * (4 * H * H + 2 * H * ffn) * 3 + 3 * 2 * 2.0 * (B * heads) * S * S * (H // heads)   # linear fwd+bwd, attention core fwd+bwd
+    n_params = 4 * (H * H + H) + 4 * H + 2 * H * ffn + ffn + H
+    return {"ms": round(ms, 4), "bound": "mixed", "achieved_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 2),
+            "frac_of_fp32_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4), "flops": flops,
+            "adam_params": n_params, "loss_first_last": [round(l, 6) for l in losses],
+            "note": "pre-LN block d1024 h16 ffn4096 S512 B16: forward + boat_variable_backward + boat_optimizer_step + zero_grad "
+                    "through the C API, wall clock"}
 
 
 def cpu_baseline():
@@ -308,6 +396,7 @@ def main():
     if not args.no_extra:
         extra = bench_extra(hip, args.steps, args.warmup)
         extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20), args.warmup)
+        extra["transformer_block_step"] = bench_block_step(max(2, min(args.steps, 10)), min(args.warmup, 2))
         line["extra"] = extra
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()

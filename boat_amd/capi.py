@@ -136,6 +136,7 @@ _EXT_SIGS = {
     "boat_hip_variable_ensure_grad": (P, [P]),
     "boat_hip_var_gelu": (P, [P]),
     "boat_hip_var_layernorm": (P, [P, P]),
+    "boat_hip_var_reshape": (P, [P, C.POINTER(C.c_int64), C.c_size_t]),
     "boat_hip_layernorm_get_weight": (P, [P]), "boat_hip_layernorm_get_bias": (P, [P]),
     "boat_hip_layernorm_get_grad_weight": (P, [P]), "boat_hip_layernorm_get_grad_bias": (P, [P]),
     "boat_hip_softmax_cross_entropy": (P, [P, P, C.POINTER(P)]),

@@ -282,6 +282,12 @@ boat_variable_t* boat_var_flatten(const boat_variable_t* a) {
     return unary(OP_FLATTEN, a, boat_tensor_reshape(t, shape, 2));
 }
 
+/* any shape with the same element count; the gradient is reshaped back (the same rule as flatten) */
+boat_variable_t* boat_hip_var_reshape(const boat_variable_t* a, const int64_t* shape, size_t ndim) {
+    if (!a || !shape || ndim == 0 || ndim > BOAT_MAX_DIMS) return NULL;
+    return unary(OP_FLATTEN, a, boat_tensor_reshape(a->data, shape, ndim));
+}
+
 boat_variable_t* boat_var_dense(const boat_variable_t* input, const struct boat_dense_layer_t* layer) {
     if (!input || !layer) return NULL;
     boat_variable_t* in[1] = {(boat_variable_t*)input};

@@ -305,6 +305,9 @@ BOAT_API void boat_hip_synchronize(void);
 BOAT_API boat_tensor_t* boat_hip_variable_ensure_grad(boat_variable_t* variable);
 /* GELU with gradient tracking (exact erf form) */
 BOAT_API boat_variable_t* boat_hip_var_gelu(const boat_variable_t* a);
+/* reshape with gradient tracking (boat_var_flatten generalised to any target shape of equal size), e.g.
+ * [batch, seq, hidden] <-> [batch*seq, hidden] between attention (3-D) and dense (2-D) */
+BOAT_API boat_variable_t* boat_hip_var_reshape(const boat_variable_t* a, const int64_t* shape, size_t ndim);
 /* LayerNorm with gradient tracking; dgamma/dbeta accumulate in the layer */
 BOAT_API boat_variable_t* boat_hip_var_layernorm(const boat_variable_t* a, boat_layernorm_t* norm);
 BOAT_API boat_tensor_t* boat_hip_layernorm_get_weight(const boat_layernorm_t* norm);

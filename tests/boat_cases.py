@@ -298,3 +298,93 @@ def attention(api, xq, xk, xv, weights, biases, heads, causal, d_out_list):
         for t in (tq, tk, tv):
             api.boat_tensor_unref(t)
     return out, results
+
+
+BLOCK_PARAM_ORDER = ("ln1_g", "ln1_b", "wq", "wk", "wv", "wo", "bq", "bk", "bv", "bo", "ln2_g", "ln2_b", "w1", "b1", "w2", "b2")
+
+
+def transformer_block_steps(api, x, target, params, heads, steps=1, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8):
+    """Pre-LN encoder block training steps through the tape (libboat_amd only: LayerNorm backward and GELU are
+    stubs in the reference):
+        x1 = x + Attention(LN1(x)) ; y = x1 + Dense2(GELU(Dense1(LN2(x1)))) ; loss = MSE(y, target)
+    then boat_variable_backward(y, dLoss/dy), boat_optimizer_step over the 16 parameter tensors, zero_grad.
+    x, target: [B, S, H]; params: dict keyed by BLOCK_PARAM_ORDER ([in, out] weights).
+    Returns per step dict(loss, y, dx, g_<name>..., p_<name>...)."""
+    x = np.asarray(x, np.float32)
+    B, S, H = x.shape
+    ffn = params["w1"].shape[1]
+    ln = []
+    for tag in ("ln1", "ln2"):
+        cfg = LayerNormConfig(H, 1e-5, True, True)
+        norm = api.boat_layernorm_create(C.byref(cfg))
+        api.write(api.boat_hip_layernorm_get_weight(norm), params[tag + "_g"])
+        api.write(api.boat_hip_layernorm_get_bias(norm), params[tag + "_b"])
+        ln.append(norm)
+    cfg = AttentionConfig(H, heads, H // heads, 0.0, False, True, False, 10000.0)
+    att = api.boat_attention_create(C.byref(cfg))
+    for n in "qkvo":
+        api.write(getattr(api, f"boat_attention_get_weight_{n}")(att), params["w" + n])
+        api.write(getattr(api, f"boat_attention_get_bias_{n}")(att), params["b" + n])
+    d1 = _make_dense(api, np.asarray(params["w1"], np.float32), np.asarray(params["b1"], np.float32))
+    d2 = _make_dense(api, np.asarray(params["w2"], np.float32), np.asarray(params["b2"], np.float32))
+    opt = api.boat_adam_optimizer_create(lr, beta1, beta2, eps)
+    api.boat_hip_optimizer_add_layernorm(opt, ln[0])
+    api.boat_hip_optimizer_add_attention(opt, att)
+    api.boat_hip_optimizer_add_layernorm(opt, ln[1])
+    api.boat_hip_optimizer_add_dense(opt, d1)
+    api.boat_hip_optimizer_add_dense(opt, d2)
+
+    def tensors():
+        out = {"ln1_g": (api.boat_hip_layernorm_get_weight(ln[0]), api.boat_hip_layernorm_get_grad_weight(ln[0])),
+               "ln1_b": (api.boat_hip_layernorm_get_bias(ln[0]), api.boat_hip_layernorm_get_grad_bias(ln[0])),
+               "ln2_g": (api.boat_hip_layernorm_get_weight(ln[1]), api.boat_hip_layernorm_get_grad_weight(ln[1])),
+               "ln2_b": (api.boat_hip_layernorm_get_bias(ln[1]), api.boat_hip_layernorm_get_grad_bias(ln[1])),
+               "w1": (api.boat_dense_layer_get_weight(d1), api.boat_dense_layer_get_grad_weight(d1)),
+               "b1": (api.boat_dense_layer_get_bias(d1), api.boat_dense_layer_get_grad_bias(d1)),
+               "w2": (api.boat_dense_layer_get_weight(d2), api.boat_dense_layer_get_grad_weight(d2)),
+               "b2": (api.boat_dense_layer_get_bias(d2), api.boat_dense_layer_get_grad_bias(d2))}
+        for n in "qkvo":
+            out["w" + n] = (getattr(api, f"boat_attention_get_weight_{n}")(att), getattr(api, f"boat_attention_get_grad_weight_{n}")(att))
+            out["b" + n] = (getattr(api, f"boat_attention_get_bias_{n}")(att), getattr(api, f"boat_attention_get_grad_bias_{n}")(att))
+        return out
+
+    tt = api.tensor(np.asarray(target, np.float32))
+    shape2 = (C.c_int64 * 2)(B * S, H)
+    shape3 = (C.c_int64 * 3)(B, S, H)
+    history = []
+    for _ in range(steps):
+        vx = _var(api, x, True)
+        h1 = api.boat_hip_var_layernorm(vx, ln[0])
+        a = api.boat_var_attention(h1, h1, h1, att, None)
+        x1 = api.boat_var_add(vx, a)
+        h2 = api.boat_hip_var_layernorm(x1, ln[1])
+        h2f = api.boat_hip_var_reshape(h2, shape2, 2)
+        f1 = api.boat_var_dense(h2f, d1)
+        g1 = api.boat_hip_var_gelu(f1)
+        f2 = api.boat_var_dense(g1, d2)
+        f2r = api.boat_hip_var_reshape(f2, shape3, 3)
+        y = api.boat_var_add(x1, f2r)
+        grad = C.c_void_p()
+        tloss = api.boat_hip_mse_loss(api.boat_variable_data(y), tt, C.byref(grad))
+        rec = {"loss": float(api.numpy(tloss)[0]), "y": api.numpy(api.boat_variable_data(y))}
+        api.boat_variable_backward(y, grad)
+        rec["dx"] = _grad(api, vx)
+        for name, (p, g) in tensors().items():
+            rec["g_" + name] = api.numpy(g)
+        api.boat_optimizer_step(opt)
+        api.boat_optimizer_zero_grad(opt)
+        for name, (p, g) in tensors().items():
+            rec["p_" + name] = api.numpy(p)
+        history.append(rec)
+        api.boat_tensor_unref(tloss)
+        api.boat_tensor_unref(grad)
+        for v in (y, f2r, f2, g1, f1, h2f, h2, x1, a, h1, vx):
+            api.boat_variable_free(v)
+    api.boat_optimizer_free(opt)
+    api.boat_tensor_unref(tt)
+    api.boat_dense_layer_free(d1)
+    api.boat_dense_layer_free(d2)
+    api.boat_attention_free(att)
+    for norm in ln:
+        api.boat_layernorm_free(norm)
+    return history

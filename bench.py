@@ -35,9 +35,10 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 PEAK_FP32_MFMA_TFLOPS = 157.3
 METRIC = "backward+Adam step ms; GB/s & TFLOP/s as % of MI355X roofline (1 GPU)"
 
-# HBM bytes per GEMM launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a copy
-# kernel of known size; see profiles/.  None until measured.
-GEMM_TRAFFIC_BYTES = None
+# HBM bytes per GEMM launch (average of the dX and dW launches of a step) measured with rocprofv3 --pmc:
+# FETCH_SIZE 409,880 KiB x 2.000 + WRITE_SIZE 98,304 KiB x 1.000, the factors being what the same counters read for
+# a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).
+GEMM_TRAFFIC_BYTES = int((2.0 * 409880.2 + 98304.0) * 1024)
 
 
 def parse_args():
@@ -47,6 +48,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--legs", default="all",
+                    help="comma list of dense,adam,ln_gelu,sdpa,mlp,block (default all); for profiling one workload at a time. "
+                         "Without the dense leg the line carries no value/roofline.")
     return ap.parse_args()
 
 
@@ -121,12 +125,10 @@ def bench_dense_backward(hip, steps, warmup):
     }
 
 
-def bench_extra(hip, steps, warmup):
-    """The other configurations of the path, each with its own roofline."""
+def bench_adam(hip, steps, warmup):
+    """Config 5b: flat fused Adam over 268,435,456 parameters (28 B/param)."""
     out = {}
     rng = np.random.default_rng(20250103)
-
-    # config 5b: flat fused Adam over 268,435,456 parameters (28 B/param)
     n = 268435456
     p, g, m, v = (hip.empty(n) for _ in range(4))
     chunk = 1 << 24
@@ -148,8 +150,13 @@ def bench_extra(hip, steps, warmup):
     out["adam_flat_268M"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4),
                              "bytes": 28 * n}
     del p, g, m, v
+    return out
 
-    # config 3: LayerNorm backward and GELU backward, 16384 x 4096
+
+def bench_ln_gelu(hip, steps, warmup):
+    """Config 3: LayerNorm backward and GELU backward, 16384 x 4096, plus a streaming copy of known size."""
+    out = {}
+    rng = np.random.default_rng(20250104)
     R, H = 16384, 4096
     x = hip.to_device(rng.standard_normal((R, H), dtype=np.float32))
     dy = hip.to_device(rng.standard_normal((R, H), dtype=np.float32))
@@ -177,8 +184,13 @@ def bench_extra(hip, steps, warmup):
     out["stream_copy_256MiB"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
                                  "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
     del x, dy, y, dx
+    return out
 
-    # config 4: attention core backward, B8 h16 S1024 D64 (credited flops: dV, dP, dQ, dK contractions)
+
+def bench_sdpa(hip, steps, warmup):
+    """Config 4: attention core backward, B8 h16 S1024 D64 (credited flops: dV, dP, dQ, dK contractions)."""
+    out = {}
+    rng = np.random.default_rng(20250106)
     bh_, S, D = 8 * 16, 1024, 64
     q, k, vv, go = (hip.to_device(rng.standard_normal((bh_, S, D), dtype=np.float32)) for _ in range(4))
     o, lse = hip.empty((bh_, S, D)), hip.empty((bh_, S))
@@ -369,36 +381,43 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build (the path has no inter-GPU work)",
               file=sys.stderr)
         sys.exit(2)
+    all_legs = ["dense", "adam", "ln_gelu", "sdpa", "mlp", "block"]
+    legs = all_legs if args.legs == "all" else [l.strip() for l in args.legs.split(",") if l.strip()]
+    unknown = [l for l in legs if l not in all_legs]
+    if unknown:
+        sys.exit(f"unknown leg(s) {unknown}; choose from {all_legs}")
+    if args.no_extra:
+        legs = [l for l in legs if l == "dense"]
     from boat_amd import hip
     hip.check(hip.bh_init(), "bh_init")
 
-    main_res = bench_dense_backward(hip, args.steps, args.warmup)
     line = {
-        "metric": METRIC,
-        "value": round(main_res["ms_per_step"], 4),
-        "unit": "ms",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(main_res["ms_per_step"], 4),
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
+        "metric": METRIC, "value": None, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "dense layer backward (BASELINE config 2): X[8192x4096], W[4096x4096], dY[8192x4096] -> dX, dW, db; "
                                "549.76 GFLOP per step", "M": 8192, "K": 4096, "N": 4096,
                    "device": hip.bh_device_name().decode().strip(), "compute_units": hip.bh_device_cu_count()},
-        "roofline": main_res["roofline"],
-        "step_tflops": main_res["step_tflops"],
-        "wall_ms_per_step": round(main_res["wall_ms_per_step"], 4),
     }
-    if not args.no_extra:
-        extra = bench_extra(hip, args.steps, args.warmup)
+    if "dense" in legs:
+        main_res = bench_dense_backward(hip, args.steps, args.warmup)
+        line.update({"value": round(main_res["ms_per_step"], 4), "ms_per_step": round(main_res["ms_per_step"], 4),
+                     "roofline": main_res["roofline"], "step_tflops": main_res["step_tflops"],
+                     "wall_ms_per_step": round(main_res["wall_ms_per_step"], 4)})
+    extra = {}
+    if "adam" in legs:
+        extra.update(bench_adam(hip, args.steps, args.warmup))
+    if "ln_gelu" in legs:
+        extra.update(bench_ln_gelu(hip, args.steps, args.warmup))
+    if "sdpa" in legs:
+        extra.update(bench_sdpa(hip, args.steps, args.warmup))
+    if "mlp" in legs:
         extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20), args.warmup)
+    if "block" in legs:
         extra["transformer_block_step"] = bench_block_step(max(2, min(args.steps, 10)), min(args.warmup, 2))
+    if extra:
         line["extra"] = extra
-    if not args.no_cpu:
+    if not args.no_cpu and "dense" in legs:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
 

@@ -152,6 +152,9 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
  * -1 = heuristic (default).  bh_sdpa_force_general: 1 = always use the general attention kernels. */
 int bh_gemm_force_config(int cfg);
 int bh_sdpa_force_general(int on);
+/* bh_layernorm_tune: cap on the workgroups of the LayerNorm backward (each writes one dgamma/dbeta partial);
+ * 0 keeps the current value.  The second argument is reserved. */
+int bh_layernorm_tune(int bwd_blocks, int reserved);
 
 #ifdef __cplusplus
 }

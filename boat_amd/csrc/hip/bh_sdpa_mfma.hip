@@ -16,9 +16,10 @@
 //   backward: S = Q.K^T and dP = dO.V^T put "key = lane, query = register", the A operand of
 //            dV += P^T.dO and dK += dS^T.Q; only dQ = dS.K needs dS with "query = lane", which is one
 //            32x32 transpose per wavefront through LDS.  dK/dV accumulate in registers over the loop
-//            on query tiles.  The dQ contributions of a workgroup's four wavefronts are exchanged
-//            through LDS, summed, and written as one partial per (key tile, query tile); a second
-//            kernel sums the s/128 partials.  No atomics anywhere, so dQ is deterministic.
+//            on query tiles.  dQ of a query tile contracts over the workgroup's 128 keys: the four
+//            wavefronts publish dS in LDS and each computes a 16-column slice, written as one partial
+//            per (key tile, query tile); a second kernel sums the s/128 partials.  No atomics
+//            anywhere, so dQ is deterministic.
 // Any order of the contraction index is a valid sum, so the index order inside a chain is whatever the
 // register layout gives; operands fetched from LDS use 16-byte reads along head_dim (row stride 68
 // floats, conflict free) or 8-byte reads that hand one lane two interleaved output columns.
@@ -193,30 +194,39 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
 
 // ----------------------------------------------------------------- backward
 // grid (s/128, bh); 4 wavefronts, each owns 32 keys (dK, dV rows) and loops over query tiles of 32.
-// LDS: per wavefront its K and V rows and a 32x33 transpose pad; per workgroup two buffers of the
-// current Q and dO tiles plus their lse/delta.
+// Two workgroups fit a CU (69 KB of LDS, <= 256 registers per lane), so a SIMD always has a second
+// wavefront to run while one waits at a barrier or on LDS.
+// LDS per workgroup: the 128 K rows, one Q tile and one dO tile (refilled through registers between the
+// two barriers of an iteration), a [32 queries][128 keys] dS tile, and the tile's lse/delta.
+// V never enters LDS: a lane keeps the 32 values of V it feeds to dP = dO.V^T in registers for the
+// whole kernel.
+// dQ = dS.K of a query tile contracts over all 128 keys of the workgroup, so the four wavefronts first
+// publish their dS blocks in LDS and then each computes a [32 queries][16 head-dim columns] slice with
+// v_mfma_f32_16x16x4_f32 and stores it straight to the key tile's partial dQ: no cross-wavefront sum.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
+
 struct BwdSmem {
-    static constexpr int KV = 4 * 32 * kLd;             // K (or V) rows of the four wavefronts
+    static constexpr int K = 128 * kLd;                 // K rows of the workgroup
     static constexpr int QT = 32 * kLd;                 // one Q (or dO) tile
-    static constexpr int TP = 4 * 32 * 33;              // transpose pads
+    static constexpr int kDsLd = 132;                   // dS row stride: 128 keys + 4 pad
     static constexpr int OFF_K = 0;
-    static constexpr int OFF_V = OFF_K + KV;
-    static constexpr int OFF_Q = OFF_V + KV;            // [2][QT]
-    static constexpr int OFF_DO = OFF_Q + 2 * QT;       // [2][QT]
-    static constexpr int OFF_T = OFF_DO + 2 * QT;
-    static constexpr int OFF_STAT = OFF_T + TP;         // [2][2][32]: lse*log2e, delta
-    static constexpr int OFF_DQ = OFF_STAT + 2 * 2 * 32; // [4][32][kLd] dQ tiles of the four wavefronts
-    static constexpr int TOTAL = OFF_DQ + 4 * 32 * kLd;
+    static constexpr int OFF_Q = OFF_K + K;
+    static constexpr int OFF_DO = OFF_Q + QT;
+    static constexpr int OFF_DS = OFF_DO + QT;          // [32][kDsLd]
+    static constexpr int OFF_STAT = OFF_DS + 32 * kDsLd; // [2][32]: lse*log2e, delta
+    static constexpr int TOTAL = OFF_STAT + 64;
 };
 
 template <bool CAUSAL>
-__global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
-                                                            const float* __restrict__ v, const float* __restrict__ lse,
-                                                            const float* __restrict__ delta, const float* __restrict__ d_out,
-                                                            float* __restrict__ dq_partial, float* __restrict__ dk,
-                                                            float* __restrict__ dv, int s, float scale) {
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                               const float* __restrict__ v, const float* __restrict__ lse,
+                                                               const float* __restrict__ delta, const float* __restrict__ d_out,
+                                                               float* __restrict__ dq_partial, float* __restrict__ dk,
+                                                               float* __restrict__ dv, int s, float scale) {
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
     const int64_t head = blockIdx.y;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
@@ -226,23 +236,28 @@ __global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restr
     const float* dh = delta + head * s;
     // partial dQ of this key tile: [key tile][bh][s][64]
     float* dqh = dq_partial + ((int64_t)blockIdx.x * gridDim.y + head) * s * kD;
-    float* dq_mine = smem + BwdSmem::OFF_DQ + w * 32 * kLd;
     const int kv_wg = blockIdx.x * 128;          // first key of the workgroup
     const int kv0 = kv_wg + w * 32;              // first key of this wavefront
     const float c1 = scale * kLog2e;
 
-    float* ks = smem + BwdSmem::OFF_K + w * 32 * kLd;
-    float* vs = smem + BwdSmem::OFF_V + w * 32 * kLd;
-    float* tp = smem + BwdSmem::OFF_T + w * 32 * 33;
-    // this wavefront's K and V rows -> LDS (each lane: 8 float4 per operand)
+    float* kall = smem + BwdSmem::OFF_K;         // all 128 K rows
+    float* ks = kall + w * 32 * kLd;             // this wavefront's 32
+    float* qs = smem + BwdSmem::OFF_Q;
+    float* gs = smem + BwdSmem::OFF_DO;
+    float* dsb = smem + BwdSmem::OFF_DS;
+    float* st = smem + BwdSmem::OFF_STAT;
+    // this wavefront's K rows -> LDS (each lane: 8 float4)
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const int idx = lane + i * 64, row = idx >> 4, c4 = idx & 15;
         *reinterpret_cast<float4*>(ks + row * kLd + c4 * 4) =
             *reinterpret_cast<const float4*>(kh + (int64_t)(kv0 + row) * kD + c4 * 4);
-        *reinterpret_cast<float4*>(vs + row * kLd + c4 * 4) =
-            *reinterpret_cast<const float4*>(vh + (int64_t)(kv0 + row) * kD + c4 * 4);
     }
+    // this lane's slice of V: key kv0 + r, head-dim 8g + 4*half .. +3 for g = 0..7
+    float4 vreg[8];
+#pragma unroll
+    for (int g = 0; g < 8; g++)
+        vreg[g] = *reinterpret_cast<const float4*>(vh + (int64_t)(kv0 + r) * kD + 8 * g + 4 * half);
 
     floatx16 acc_dk[2] = {zero16(), zero16()};   // [d tile]: key = acc_row, d = 2*lane + tile
     floatx16 acc_dv[2] = {zero16(), zero16()};
@@ -264,8 +279,8 @@ __global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restr
 #define BWD_ST(i, Q, G)                                                                                   \
     {                                                                                                     \
         const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
-        *reinterpret_cast<float4*>(q_base + row * kLd + c4 * 4) = Q;                                      \
-        *reinterpret_cast<float4*>(g_base + row * kLd + c4 * 4) = G;                                      \
+        *reinterpret_cast<float4*>(qs + row * kLd + c4 * 4) = Q;                                          \
+        *reinterpret_cast<float4*>(gs + row * kLd + c4 * 4) = G;                                          \
     }
 #define BWD_STAGE_LOAD(QT)                                                 \
     {                                                                      \
@@ -274,26 +289,20 @@ __global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restr
         if (tid < 32) stat = lh[qt_ld * 32 + tid] * kLog2e;                \
         else if (tid < 64) stat = dh[qt_ld * 32 + tid - 32];               \
     }
-#define BWD_STAGE_STORE(BUF)                                               \
+#define BWD_STAGE_STORE()                                                  \
     {                                                                      \
-        float* q_base = smem + BwdSmem::OFF_Q + (BUF) * BwdSmem::QT;       \
-        float* g_base = smem + BwdSmem::OFF_DO + (BUF) * BwdSmem::QT;      \
         BWD_ST(0, qst0, gst0) BWD_ST(1, qst1, gst1)                        \
-        if (tid < 64) smem[BwdSmem::OFF_STAT + (BUF) * 64 + tid] = stat;   \
+        if (tid < 64) st[tid] = stat;                                      \
     }
     if (first_qt < n_qt) {
         BWD_STAGE_LOAD(first_qt)
-        BWD_STAGE_STORE(0)
+        BWD_STAGE_STORE()
     }
     __syncthreads();
 
     for (int qt = first_qt; qt < n_qt; qt++) {
-        const int cur = (qt - first_qt) & 1;
         const bool more = qt + 1 < n_qt;
         if (more) BWD_STAGE_LOAD(qt + 1)
-        const float* qs = smem + BwdSmem::OFF_Q + cur * BwdSmem::QT;
-        const float* gs = smem + BwdSmem::OFF_DO + cur * BwdSmem::QT;
-        const float* st = smem + BwdSmem::OFF_STAT + cur * 64;
         const int q0 = qt * 32;
         if (!CAUSAL || q0 + 31 >= kv0) {
             // S = Q.K^T and dP = dO.V^T : query = row (acc_row), key = lane
@@ -304,7 +313,7 @@ __global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restr
                 const float4 aq = *reinterpret_cast<const float4*>(qs + off);
                 const float4 bk = *reinterpret_cast<const float4*>(ks + off);
                 const float4 ag = *reinterpret_cast<const float4*>(gs + off);
-                const float4 bv = *reinterpret_cast<const float4*>(vs + off);
+                const float4 bv = vreg[g];
                 acc_s = MFMA(aq.x, bk.x, acc_s);
                 acc_dp = MFMA(ag.x, bv.x, acc_dp);
                 acc_s = MFMA(aq.y, bk.y, acc_s);
@@ -334,50 +343,41 @@ __global__ __launch_bounds__(256) void sdpa_bwd_mfma_kernel(const float* __restr
                 acc_dk[0] = MFMA(acc_dp[e], bq.x, acc_dk[0]);
                 acc_dk[1] = MFMA(acc_dp[e], bq.y, acc_dk[1]);
             }
-            // dS -> "query = lane" through the wavefront's pad
+            // publish dS[query][key] for the dQ product
 #pragma unroll
-            for (int e = 0; e < 16; e++) tp[acc_row(e, half) * 33 + r] = acc_dp[e];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            // dQ = dS.K : step e contracts key row acc_row(e, half)
-            floatx16 acc_dq[2] = {zero16(), zero16()};
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int key = acc_row(e, half);
-                const float a = tp[r * 33 + key];
-                const float2 bk = *reinterpret_cast<const float2*>(ks + key * kLd + 2 * r);
-                acc_dq[0] = MFMA(a, bk.x, acc_dq[0]);
-                acc_dq[1] = MFMA(a, bk.y, acc_dq[1]);
-            }
-            __builtin_amdgcn_wave_barrier();   // the pad is rewritten next iteration
-#pragma unroll
-            for (int e = 0; e < 16; e++)
-                *reinterpret_cast<float2*>(dq_mine + acc_row(e, half) * kLd + 2 * r) = make_float2(acc_dq[0][e], acc_dq[1][e]);
+            for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * BwdSmem::kDsLd + w * 32 + r] = acc_dp[e];
         } else {
 #pragma unroll
-            for (int e = 0; e < 16; e++)
-                *reinterpret_cast<float2*>(dq_mine + acc_row(e, half) * kLd + 2 * r) = make_float2(0.f, 0.f);
+            for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * BwdSmem::kDsLd + w * 32 + r] = 0.f;
         }
-        __syncthreads();
-        // sum of the four wavefronts' tiles -> this key tile's partial dQ (whole rows)
+        __syncthreads();   // dS complete; every wavefront is done with the Q and dO tiles
+        if (more) BWD_STAGE_STORE()
+        // dQ[32 queries][16w .. 16w+15] = dS[32][128 keys] . K[128][16w ..]; lane (i16, kk) reads four
+        // consecutive keys of its dS row at once and feeds them to four successive products (the order
+        // of the contraction index is free as long as both operands use the same one)
+        floatx4 acc_dq0 = {0.f, 0.f, 0.f, 0.f}, acc_dq1 = {0.f, 0.f, 0.f, 0.f};
+        const int g_lim = CAUSAL ? min(8, (q0 + 32 - kv_wg + 15) / 16) : 8;   // keys past the tile's last query are masked
+        for (int g = 0; g < g_lim; g++) {
+            const float4 a0 = *reinterpret_cast<const float4*>(dsb + i16 * BwdSmem::kDsLd + 16 * g + 4 * kk);
+            const float4 a1 = *reinterpret_cast<const float4*>(dsb + (16 + i16) * BwdSmem::kDsLd + 16 * g + 4 * kk);
+            const float* kb = kall + (16 * g + 4 * kk) * kLd + 16 * w + i16;
+            const float b0 = kb[0], b1 = kb[kLd], b2 = kb[2 * kLd], b3 = kb[3 * kLd];
+            acc_dq0 = MFMA16(a0.x, b0, acc_dq0);
+            acc_dq1 = MFMA16(a1.x, b0, acc_dq1);
+            acc_dq0 = MFMA16(a0.y, b1, acc_dq0);
+            acc_dq1 = MFMA16(a1.y, b1, acc_dq1);
+            acc_dq0 = MFMA16(a0.z, b2, acc_dq0);
+            acc_dq1 = MFMA16(a1.z, b2, acc_dq1);
+            acc_dq0 = MFMA16(a0.w, b3, acc_dq0);
+            acc_dq1 = MFMA16(a1.w, b3, acc_dq1);
+        }
+        // accumulator register e of lane (i16, kk) is query row 4*kk + e of the 16-row tile, column i16
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int idx = tid + i * 256, row = idx >> 4, c4 = idx & 15;
-            const float* src = smem + BwdSmem::OFF_DQ + row * kLd + c4 * 4;
-            const float4 t0 = *reinterpret_cast<const float4*>(src);
-            const float4 t1 = *reinterpret_cast<const float4*>(src + 32 * kLd);
-            const float4 t2 = *reinterpret_cast<const float4*>(src + 2 * 32 * kLd);
-            const float4 t3 = *reinterpret_cast<const float4*>(src + 3 * 32 * kLd);
-            float4 o;
-            o.x = (t0.x + t1.x) + (t2.x + t3.x);
-            o.y = (t0.y + t1.y) + (t2.y + t3.y);
-            o.z = (t0.z + t1.z) + (t2.z + t3.z);
-            o.w = (t0.w + t1.w) + (t2.w + t3.w);
-            *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + row) * kD + c4 * 4) = o;
+        for (int e = 0; e < 4; e++) {
+            dqh[(int64_t)(q0 + 4 * kk + e) * kD + 16 * w + i16] = acc_dq0[e];
+            dqh[(int64_t)(q0 + 16 + 4 * kk + e) * kD + 16 * w + i16] = acc_dq1[e];
         }
-        if (more) BWD_STAGE_STORE(cur ^ 1)
-        __syncthreads();
+        __syncthreads();   // dS tile free again; the next Q and dO tiles are in place
     }
 #undef BWD_LD
 #undef BWD_ST

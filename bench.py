@@ -197,9 +197,8 @@ def bench_sdpa(hip, steps, warmup):
     scale = 1.0 / 8.0
     hip.check(hip.bh_sdpa_forward(q.ptr, k.ptr, vv.ptr, scale, 0, o.ptr, lse.ptr, None, bh_, S, D))
     dq, dk, dv = hip.empty((bh_, S, D)), hip.empty((bh_, S, D)), hip.empty((bh_, S, D))
-    sd_steps = max(2, min(steps, 5))
     ms = time_steps(hip, lambda: hip.check(hip.bh_sdpa_backward(q.ptr, k.ptr, vv.ptr, o.ptr, lse.ptr, go.ptr, scale, 0, dq.ptr, dk.ptr,
-                                                                dv.ptr, bh_, S, D)), sd_steps, 1)
+                                                                dv.ptr, bh_, S, D)), steps, warmup)
     flops = 4 * 2.0 * bh_ * S * S * D
     tf = flops / (ms * 1e-3) / 1e12
     out["sdpa_bwd_B8h16S1024D64"] = {"ms": round(ms, 4), "bound": "mfma", "achieved_TFLOPs": round(tf, 2),

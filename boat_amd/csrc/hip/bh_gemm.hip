@@ -13,7 +13,7 @@
 // written to memory.
 //
 // Tiling (wave64, gfx950):
-//   macro tile BM x BN per workgroup, k-tile BK=16, LDS double buffered, next k-tile
+//   macro tile BM x BN per workgroup (256x256, 256x128, 128x256 or 128x128), k-tile BK=16, LDS double buffered, next k-tile
 //   prefetched into registers while the current one feeds the MFMAs (one barrier per k-tile)
 //   each wavefront owns a (32*TM) x (32*TN) block = TM*TN accumulators of 16 VGPRs
 //   A-fragment for MFMA step s comes from one ds_read_b128 / ds_read_b64:
@@ -340,6 +340,8 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict_
 
 using CfgBig = GemmCfg<256, 256, 2, 4>;   // 8 waves, 128x64 per wave
 using CfgMid = GemmCfg<128, 128, 2, 2>;   // 4 waves, 64x64 per wave
+using CfgTall = GemmCfg<256, 128, 4, 2>;  // 8 waves, 64x64 per wave
+using CfgWide = GemmCfg<128, 256, 2, 4>;  // 8 waves, 64x64 per wave
 
 template <typename Cfg, bool A_KC, bool B_KC>
 static int launch_mfma(const GemmArgs& g, int64_t batch) {
@@ -365,7 +367,7 @@ static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool 
     return launch_mfma<Cfg, false, false>(g, batch);
 }
 
-static int g_force_cfg = -1;   // test hook: 0 = fallback, 1 = mid, 2 = big, -1 = heuristic
+static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, -1 = heuristic
 
 }  // namespace bh
 
@@ -404,14 +406,20 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     // float4 global loads need: 16 B aligned bases, leading dimensions and the contiguous extent % 4
     bool vec_ok = al16(a) && al16(b) && (lda % 4 == 0) && (ldb % 4 == 0) && k > 0;
     vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
-    int cfg;   // 0 fallback, 1 mid, 2 big
+    int cfg;   // 0 fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
+        // measured on MI355X: the 256x256 tile wins once it fills the chip twice over with a long contraction;
+        // below that the 8-wavefront 128x256 / 256x128 tiles (same operand reuse per wavefront, twice the
+        // workgroups) beat both it and the 128x128 tile; narrow outputs keep the small tile
         const int64_t big_tiles = ceil_div(m, 256) * ceil_div(n, 256);
-        cfg = big_tiles >= 256 ? 2 : 1;
+        if (big_tiles >= 512 && k >= 2048) cfg = 2;
+        else if (n >= 192 && m >= 96) cfg = 4;
+        else if (m >= 192 && n >= 96) cfg = 3;
+        else cfg = 1;
     }
-    if (g_force_cfg >= 0 && (vec_ok || g_force_cfg == 0)) cfg = g_force_cfg;
+    if (g_force_cfg >= 0 && g_force_cfg <= 4 && (vec_ok || g_force_cfg == 0)) cfg = g_force_cfg;
 
     if (cfg == 0) {
         if (k == 0 && !accumulate && !bias) {   // empty contraction: zeros (linear.c zero-fills its output)
@@ -425,7 +433,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         return BH_LAUNCH_CHECK("gemm_fallback_kernel");
     }
 
-    const int bm = cfg == 2 ? 256 : 128, bn = bm;
+    const int bm = (cfg == 2 || cfg == 3) ? 256 : 128, bn = (cfg == 2 || cfg == 4) ? 256 : 128;
     g.tiles_m = (int)ceil_div(m, bm);
     g.tiles_n = (int)ceil_div(n, bn);
     // split K when the output alone cannot fill the chip
@@ -448,7 +456,13 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         run.ldc = n;
         run.stride_c = m * n;
     }
-    int rc = cfg == 2 ? launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc);
+    int rc;
+    switch (cfg) {
+        case 2: rc = launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc); break;
+        case 3: rc = launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc); break;
+        case 4: rc = launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc); break;
+        default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc); break;
+    }
     if (rc == BH_OK && g.k_splits > 1) {
         int64_t blocks = ceil_div(m * n * batch, 256);
         if (blocks > 4096) blocks = 4096;

@@ -330,6 +330,18 @@ static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
             v->grad = g;
             return;
         }
+        if (bt_is_f32(g) && bt_is_f32(v->data) && g->nelements == v->data->nelements && g->nelements > 0) {
+            /* first contribution: one copy instead of zero-fill + add (0 + g == g bit for bit) */
+            boat_tensor_t* fresh = bt_new_like_uninit(v->data);
+            const float* src = fresh ? bt_dev_read(g) : NULL;
+            float* dst = src ? bt_dev_write(fresh) : NULL;
+            if (dst && boat_hip_ok(bh_memcpy_d2d(dst, src, g->nbytes), "gradient copy")) {
+                v->grad = fresh;
+                if (own) boat_tensor_unref(g);
+                return;
+            }
+            boat_tensor_free(fresh);
+        }
         v->grad = boat_tensor_create_like(v->data);
     }
     if (v->grad) boat_add_(v->grad, g);

@@ -148,7 +148,7 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
                          float lr, float beta1, float beta2, float eps, int64_t timestep);
 
 /* ---- test hooks (no arithmetic of their own) ----
- * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128 MFMA tile, 2 = 256x256 MFMA tile,
+ * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256 MFMA tile,
  * -1 = heuristic (default).  bh_sdpa_force_general: 1 = always use the general attention kernels. */
 int bh_gemm_force_config(int cfg);
 int bh_sdpa_force_general(int on);

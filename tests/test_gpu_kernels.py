@@ -325,7 +325,7 @@ def test_gemm_heuristic_path(hip, rng, ta, tb, m, n, k):
     gemm_case(hip, rng, ta, tb, m, n, k)
 
 
-@pytest.mark.parametrize("force", [1, 2])
+@pytest.mark.parametrize("force", [1, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 16), (256, 512, 64), (128, 128, 8), (260, 132, 36), (512, 768, 100), (1024, 1024, 256)])
 def test_gemm_mfma_tiles(hip, rng, force, ta, tb, m, n, k):

@@ -439,9 +439,12 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     // split K when the output alone cannot fill the chip
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * batch;
     float* ws = nullptr;
-    if (tiles < 256 && k >= 1024) {
+    // (a handful of tiles with a contraction of a few hundred is latency bound per k-tile: split it finer)
+    const bool few_tiles = tiles <= 8 && k >= 256;
+    if ((tiles < 256 && k >= 1024) || few_tiles) {
+        const int64_t min_k = few_tiles && k < 2048 ? 128 : 256;
         int64_t splits = ceil_div(512, tiles);
-        if (splits > k / 256) splits = k / 256;
+        if (splits > k / min_k) splits = k / min_k;
         if (splits > 32) splits = 32;
         if (splits > 1) {
             g.k_per_split = ceil_div(ceil_div(k, splits), kBK) * kBK;

@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
-                    const float p = exp2f(acc_s[t][e] - m_new);
+                    const float p = __builtin_amdgcn_exp2f(acc_s[t][e] - m_new);
                     acc_s[t][e] = p;
                     psum += p;
                 }
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int row = acc_row(e, half);
-                float p = exp2f(acc_s[e] * c1 - st[row]);
+                float p = __builtin_amdgcn_exp2f(acc_s[e] * c1 - st[row]);
                 if (CAUSAL && kv0 + r > q0 + row) p = 0.f;
                 acc_s[e] = p;
                 acc_dp[e] = p * (acc_dp[e] - st[32 + row]) * scale;

@@ -111,6 +111,8 @@ _SIGS = {
     "boat_attention_update": (None, [P, C.c_float]),
     # optimizer
     "boat_adam_optimizer_create": (P, [C.c_float, C.c_float, C.c_float, C.c_float]),
+    "boat_rmsprop_optimizer_create": (P, [C.c_float, C.c_float, C.c_float]),
+    "boat_adagrad_optimizer_create": (P, [C.c_float, C.c_float]),
     "boat_optimizer_add_parameter": (None, [P, P, P]),
     "boat_optimizer_step": (None, [P]),
     "boat_optimizer_zero_grad": (None, [P]),

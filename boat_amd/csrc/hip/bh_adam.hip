@@ -10,6 +10,11 @@
 // result is bit-identical to the scalar C loop, not merely within tolerance.
 //
 // Traffic per element: read p,g,m,v + write p,m,v = 28 bytes, one pass, float4 lanes.
+//
+// RMSprop (src/optimizers/rmsprop.c:181-211) and Adagrad (src/optimizers/adagrad.c:167-197) use the same
+// launch shapes with one state tensor instead of two (20 bytes per element):
+//   RMSprop  s = alpha*s + (1-alpha)*g*g ; p -= lr*g/(sqrtf(s)+eps)
+//   Adagrad  s += g*g                    ; p -= lr*g/(sqrtf(s)+eps)
 #include "bh_common.h"
 
 #include <math.h>
@@ -33,7 +38,46 @@ __device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, 
     p -= s.lr * m_hat / (sqrtf(v_hat) + s.eps);
 }
 
+struct SqScalars {
+    float lr, alpha, one_minus_alpha, eps;
+    int rule;   // 0 = RMSprop, 1 = Adagrad
+};
+
+__device__ __forceinline__ void sq_one(float& p, float g, float& sq, const SqScalars& s) {
+    if (s.rule == 0) sq = s.alpha * sq + s.one_minus_alpha * g * g;
+    else sq += g * g;
+    p -= s.lr * g / (sqrtf(sq) + s.eps);
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// same lane map as adam_group, one state tensor
+__device__ __forceinline__ void sq_group(float* __restrict__ p, const float* __restrict__ g, float* __restrict__ sq,
+                                         int64_t n, const SqScalars& s, int64_t idx) {
+    const int64_t n4 = n >> 2;
+    if (idx < n4) {
+        f32x4 pp = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(p) + idx);
+        f32x4 gg = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(g) + idx);
+        f32x4 ss = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(sq) + idx);
+        float px = pp.x, py = pp.y, pz = pp.z, pw = pp.w;
+        float sx = ss.x, sy = ss.y, sz = ss.z, sw = ss.w;
+        sq_one(px, gg.x, sx, s);
+        sq_one(py, gg.y, sy, s);
+        sq_one(pz, gg.z, sz, s);
+        sq_one(pw, gg.w, sw, s);
+        pp = (f32x4){px, py, pz, pw};
+        ss = (f32x4){sx, sy, sz, sw};
+        __builtin_nontemporal_store(pp, reinterpret_cast<f32x4*>(p) + idx);
+        __builtin_nontemporal_store(ss, reinterpret_cast<f32x4*>(sq) + idx);
+    }
+    if (idx < (n & 3)) {
+        const int64_t i = (n4 << 2) + idx;
+        float pp = p[i], ss = sq[i];
+        sq_one(pp, g[i], ss, s);
+        p[i] = pp;
+        sq[i] = ss;
+    }
+}
 
 // One float4 group per lane: lane `idx` of the tensor's own grid updates elements 4*idx..4*idx+3;
 // the first (n % 4) lanes also take one tail element.  No loop: the grid covers the tensor, so the
@@ -130,6 +174,31 @@ __global__ __launch_bounds__(kAdamBlock) void adam_multi_kernel(AdamTable t, Ada
     }
 }
 
+__global__ __launch_bounds__(kAdamBlock) void sq_multi_kernel(AdamTable t, SqScalars s) {
+    int lo = 0, hi = t.count;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if ((int)blockIdx.x >= t.first_block[mid]) lo = mid; else hi = mid;
+    }
+    const int64_t idx = (int64_t)((int)blockIdx.x - t.first_block[lo]) * kAdamBlock + threadIdx.x;
+    float* p = t.p[lo];
+    const float* g = t.g[lo];
+    float* sq = t.m[lo];
+    const int64_t n = t.n[lo];
+    const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(sq)) & 15) == 0;
+    if (vec) {
+        sq_group(p, g, sq, n, s, idx);
+    } else {
+        const int64_t stride = (int64_t)(t.first_block[lo + 1] - t.first_block[lo]) * kAdamBlock;
+        for (int64_t i = idx; i < n; i += stride) {
+            float pp = p[i], ss = sq[i];
+            sq_one(pp, g[i], ss, s);
+            p[i] = pp;
+            sq[i] = ss;
+        }
+    }
+}
+
 static AdamScalars make_scalars(float lr, float beta1, float beta2, float eps, int64_t timestep) {
     AdamScalars s;
     s.lr = lr;
@@ -207,6 +276,64 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
         if (rc) return rc;
     }
     return BH_OK;
+}
+
+// rule 0: RMSprop (alpha used), rule 1: Adagrad (alpha ignored)
+static int sq_update_multi(int rule, float* const* p, const float* const* g, float* const* sq, const int64_t* n, int count,
+                           float lr, float alpha, float eps) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(count >= 0, "negative count");
+    BH_CHECK_ARG(count == 0 || (p && g && sq && n), "null table");
+    SqScalars s;
+    s.lr = lr;
+    s.alpha = alpha;
+    s.one_minus_alpha = 1.0f - alpha;
+    s.eps = eps;
+    s.rule = rule;
+    int done = 0;
+    while (done < count) {
+        AdamTable t;
+        t.count = 0;
+        int64_t blocks = 0;
+        while (done < count && t.count < kAdamMaxTensors) {
+            const int i = done++;
+            BH_CHECK_ARG(n[i] >= 0, "negative element count");
+            if (n[i] == 0) continue;
+            BH_CHECK_ARG(p[i] && g[i] && sq[i], "null tensor pointer");
+            const int k = t.count++;
+            t.p[k] = p[i];
+            t.g[k] = g[i];
+            t.m[k] = sq[i];
+            t.v[k] = nullptr;
+            t.n[k] = n[i];
+            t.first_block[k] = (int)blocks;
+            blocks += blocks_for(n[i]);
+            BH_CHECK_ARG(blocks <= 0x7fffffff, "tensors too large for one launch");
+        }
+        if (t.count == 0) continue;
+        t.first_block[t.count] = (int)blocks;
+        hipLaunchKernelGGL(sq_multi_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), t, s);
+        int rc = BH_LAUNCH_CHECK("bh_sq_update_multi");
+        if (rc) return rc;
+    }
+    return BH_OK;
+}
+
+int bh_rmsprop_update_multi(float* const* p, const float* const* g, float* const* sq, const int64_t* n, int count, float lr,
+                            float alpha, float eps) {
+    return sq_update_multi(0, p, g, sq, n, count, lr, alpha, eps);
+}
+int bh_adagrad_update_multi(float* const* p, const float* const* g, float* const* sum, const int64_t* n, int count, float lr,
+                            float eps) {
+    return sq_update_multi(1, p, g, sum, n, count, lr, 0.0f, eps);
+}
+int bh_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps) {
+    const float* gg = g;
+    return sq_update_multi(0, &p, &gg, &sq, &n, 1, lr, alpha, eps);
+}
+int bh_adagrad_update(float* p, const float* g, float* sum, int64_t n, float lr, float eps) {
+    const float* gg = g;
+    return sq_update_multi(1, &p, &gg, &sum, &n, 1, lr, 0.0f, eps);
 }
 
 }  // extern "C"

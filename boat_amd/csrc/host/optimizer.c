@@ -1,7 +1,7 @@
-/* optimizer.c - Adam behind boat_optimizer_* with one fused multi-tensor launch per step.
+/* optimizer.c - Adam, RMSprop and Adagrad behind boat_optimizer_* with one fused multi-tensor launch per step.
  *
- * Same state machine as src/optimizers/adam.c:15-308 and the type dispatch of
- * src/optimizers/optimizer_common.c:108-235: the state's first field is the optimizer type;
+ * Same state machines as src/optimizers/adam.c:15-308, rmsprop.c:15-300, adagrad.c:15-290 and the type
+ * dispatch of src/optimizers/optimizer_common.c:108-235: the state's first field is the optimizer type;
  * parameters are registered as borrowed (param, grad) tensor pairs that must outlive the
  * optimizer; m and v are created zero at registration; `step` updates every registered tensor
  * with the bias correction of the CURRENT timestep and increments it once afterwards; `step`
@@ -14,7 +14,7 @@
 
 typedef struct {
     boat_optimizer_type_t type;   /* must stay first: the dispatcher reads it (optimizer_common.c:108-114) */
-    float learning_rate, beta1, beta2, epsilon;
+    float learning_rate, beta1, beta2, epsilon;   /* beta1 doubles as RMSprop's alpha */
     int64_t timestep;
     boat_tensor_t** params;
     boat_tensor_t** grads;
@@ -43,6 +43,40 @@ boat_optimizer_t* boat_adam_optimizer_create(float learning_rate, float beta1, f
     return (boat_optimizer_t*)s;
 }
 
+/* rmsprop.c:33-57: lr > 0, alpha in (0,1), eps > 0 */
+boat_optimizer_t* boat_rmsprop_optimizer_create(float learning_rate, float alpha, float epsilon) {
+    if (learning_rate <= 0.0f || alpha <= 0.0f || alpha >= 1.0f || epsilon <= 0.0f) return NULL;
+    adam_state_t* s = (adam_state_t*)calloc(1, sizeof(*s));
+    if (!s) return NULL;
+    s->type = BOAT_OPTIMIZER_RMSPROP;
+    s->learning_rate = learning_rate;
+    s->beta1 = alpha;
+    s->epsilon = epsilon;
+    return (boat_optimizer_t*)s;
+}
+
+/* adagrad.c:41-50: lr > 0, eps > 0 */
+boat_optimizer_t* boat_adagrad_optimizer_create(float learning_rate, float epsilon) {
+    if (learning_rate <= 0.0f || epsilon <= 0.0f) return NULL;
+    adam_state_t* s = (adam_state_t*)calloc(1, sizeof(*s));
+    if (!s) return NULL;
+    s->type = BOAT_OPTIMIZER_ADAGRAD;
+    s->learning_rate = learning_rate;
+    s->epsilon = epsilon;
+    return (boat_optimizer_t*)s;
+}
+
+/* declared by the reference and defined as a stub that returns NULL (optimizer_common.c:62-67) */
+boat_optimizer_t* boat_sgd_optimizer_create(float learning_rate, float momentum) {
+    (void)learning_rate;
+    (void)momentum;
+    return NULL;
+}
+
+static bool known_type(const adam_state_t* s) {
+    return s->type == BOAT_OPTIMIZER_ADAM || s->type == BOAT_OPTIMIZER_RMSPROP || s->type == BOAT_OPTIMIZER_ADAGRAD;
+}
+
 static bool adam_grow(adam_state_t* s) {
     const size_t cap = s->capacity ? s->capacity * 2 : 16;
 #define GROW(field, type)                                              \
@@ -68,7 +102,7 @@ static bool adam_grow(adam_state_t* s) {
 void boat_optimizer_add_parameter(boat_optimizer_t* optimizer, boat_tensor_t* param, boat_tensor_t* grad) {
     if (!optimizer) return;
     adam_state_t* s = (adam_state_t*)optimizer;
-    if (s->type != BOAT_OPTIMIZER_ADAM) return;
+    if (!known_type(s)) return;
     if (!param || !grad) return;   /* silently ignored, as adam.c:99-101 */
     if (!bt_is_f32(param) || !bt_is_f32(grad) || param->nelements != grad->nelements) {
         boat_fail(BOAT_ERROR_INVALID_ARGUMENT, "boat_optimizer_add_parameter: param and grad must be float32 tensors of equal size");
@@ -79,26 +113,37 @@ void boat_optimizer_add_parameter(boat_optimizer_t* optimizer, boat_tensor_t* pa
     s->params[i] = param;
     s->grads[i] = grad;
     s->m[i] = boat_tensor_create(param->shape, param->ndim, param->dtype, param->device);   /* zero moments */
-    s->v[i] = boat_tensor_create(param->shape, param->ndim, param->dtype, param->device);
+    /* Adam's second moment; RMSprop and Adagrad keep one state tensor (square_avg / sum_square_grad) in m */
+    s->v[i] = s->type == BOAT_OPTIMIZER_ADAM ? boat_tensor_create(param->shape, param->ndim, param->dtype, param->device) : NULL;
     s->num_params++;
 }
 
 static void adam_step(adam_state_t* s) {
+    const bool two = s->type == BOAT_OPTIMIZER_ADAM;
     int count = 0;
     for (size_t i = 0; i < s->num_params; i++) {
-        if (!s->params[i] || !s->grads[i] || !s->m[i] || !s->v[i]) continue;
+        if (!s->params[i] || !s->grads[i] || !s->m[i] || (two && !s->v[i])) continue;
         if (s->params[i]->nelements == 0) continue;
         const float* g = bt_dev_read(s->grads[i]);
         float* p = bt_dev_rw(s->params[i]);
         float* m = bt_dev_rw(s->m[i]);
-        float* v = bt_dev_rw(s->v[i]);
-        if (!g || !p || !m || !v) return;
+        float* v = two ? bt_dev_rw(s->v[i]) : NULL;
+        if (!g || !p || !m || (two && !v)) return;
         s->tp[count] = p;
         s->tg[count] = g;
         s->tm[count] = m;
         s->tv[count] = v;
         s->tn[count] = (int64_t)s->params[i]->nelements;
         count++;
+    }
+    if (s->type == BOAT_OPTIMIZER_RMSPROP) {
+        boat_hip_ok(bh_rmsprop_update_multi(s->tp, s->tg, s->tm, s->tn, count, s->learning_rate, s->beta1, s->epsilon),
+                    "boat_optimizer_step");
+        return;
+    }
+    if (s->type == BOAT_OPTIMIZER_ADAGRAD) {
+        boat_hip_ok(bh_adagrad_update_multi(s->tp, s->tg, s->tm, s->tn, count, s->learning_rate, s->epsilon), "boat_optimizer_step");
+        return;
     }
     boat_hip_ok(bh_adam_update_multi(s->tp, s->tg, s->tm, s->tv, s->tn, count, s->learning_rate, s->beta1, s->beta2,
                                      s->epsilon, s->timestep),
@@ -109,13 +154,13 @@ static void adam_step(adam_state_t* s) {
 void boat_optimizer_step(boat_optimizer_t* optimizer) {
     if (!optimizer) return;
     adam_state_t* s = (adam_state_t*)optimizer;
-    if (s->type == BOAT_OPTIMIZER_ADAM) adam_step(s);
+    if (known_type(s)) adam_step(s);
 }
 
 void boat_optimizer_zero_grad(boat_optimizer_t* optimizer) {
     if (!optimizer) return;
     adam_state_t* s = (adam_state_t*)optimizer;
-    if (s->type != BOAT_OPTIMIZER_ADAM) return;
+    if (!known_type(s)) return;
     for (size_t i = 0; i < s->num_params; i++) {
         boat_tensor_t* g = s->grads[i];
         if (!g || g->nelements == 0) continue;

@@ -265,7 +265,10 @@ BOAT_API void boat_attention_layer_update(boat_attention_layer_t* layer, float l
 /* ---- include/boat/optimizers.h:15-44 ---- */
 typedef enum { BOAT_OPTIMIZER_SGD, BOAT_OPTIMIZER_ADAM, BOAT_OPTIMIZER_RMSPROP, BOAT_OPTIMIZER_ADAGRAD } boat_optimizer_type_t;
 typedef struct boat_optimizer_t boat_optimizer_t;
+BOAT_API boat_optimizer_t* boat_sgd_optimizer_create(float learning_rate, float momentum);    /* returns NULL, as the reference's stub (optimizer_common.c:62-67) */
 BOAT_API boat_optimizer_t* boat_adam_optimizer_create(float learning_rate, float beta1, float beta2, float epsilon);
+BOAT_API boat_optimizer_t* boat_rmsprop_optimizer_create(float learning_rate, float alpha, float epsilon);
+BOAT_API boat_optimizer_t* boat_adagrad_optimizer_create(float learning_rate, float epsilon);
 BOAT_API void boat_optimizer_step(boat_optimizer_t* optimizer);
 BOAT_API void boat_optimizer_zero_grad(boat_optimizer_t* optimizer);
 BOAT_API void boat_optimizer_free(boat_optimizer_t* optimizer);

@@ -147,6 +147,15 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
                          const int64_t* n, int count,
                          float lr, float beta1, float beta2, float eps, int64_t timestep);
 
+/* ---- RMSprop (src/optimizers/rmsprop.c:181-211) and Adagrad (src/optimizers/adagrad.c:167-197) ----
+ * one state tensor each: sq = alpha*sq + (1-alpha)*g*g, resp. sum += g*g; then p -= lr*g/(sqrtf(state)+eps) */
+int bh_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps);
+int bh_adagrad_update(float* p, const float* g, float* sum, int64_t n, float lr, float eps);
+int bh_rmsprop_update_multi(float* const* p, const float* const* g, float* const* sq, const int64_t* n, int count,
+                            float lr, float alpha, float eps);
+int bh_adagrad_update_multi(float* const* p, const float* const* g, float* const* sum, const int64_t* n, int count,
+                            float lr, float eps);
+
 /* ---- test hooks (no arithmetic of their own) ----
  * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256 MFMA tile,
  * -1 = heuristic (default).  bh_sdpa_force_general: 1 = always use the general attention kernels. */

@@ -433,6 +433,24 @@ void bo_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
     }
 }
 
+/* src/optimizers/rmsprop.c:197-210 */
+void bo_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps) {
+    for (int64_t i = 0; i < n; i++) {
+        float gi = g[i];
+        sq[i] = alpha * sq[i] + (1.0f - alpha) * gi * gi;
+        p[i] -= lr * gi / (sqrtf(sq[i]) + eps);
+    }
+}
+
+/* src/optimizers/adagrad.c:183-196 */
+void bo_adagrad_update(float* p, const float* g, float* sum, int64_t n, float lr, float eps) {
+    for (int64_t i = 0; i < n; i++) {
+        float gi = g[i];
+        sum[i] += gi * gi;
+        p[i] -= lr * gi / (sqrtf(sum[i]) + eps);
+    }
+}
+
 /* -------------------------------------------------------------------- loss */
 
 /* src/loss/mse.c:70-78 */

@@ -109,6 +109,10 @@ void bo_layernorm_forward(const float* x, const float* gamma, const float* beta,
 void bo_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
                     float lr, float beta1, float beta2, float eps, int64_t timestep);
 
+/* src/optimizers/rmsprop.c:181-211 and src/optimizers/adagrad.c:167-197: one tensor, one step. */
+void bo_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps);
+void bo_adagrad_update(float* p, const float* g, float* sum, int64_t n, float lr, float eps);
+
 /* src/loss/mse.c:37-88 (value) -- mean over all elements, fp32 running sum. */
 float bo_mse_loss(const float* pred, const float* target, int64_t n);
 

@@ -217,12 +217,19 @@ def mlp_ce_adam(api, x, labels, w1, b1, w2, b2, steps=1, lr=1e-3, beta1=0.9, bet
     return history
 
 
-def adam_trajectory(api, params, grads_per_step, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, lr_change=None):
+def adam_trajectory(api, params, grads_per_step, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, lr_change=None, kind="adam"):
     """Several tensors registered with one optimizer; grads rewritten in place before each step.
-    lr_change = (step_index, new_lr).  Returns params after every step: list of lists of arrays."""
+    lr_change = (step_index, new_lr).  kind: "adam", "rmsprop" (beta1 is its alpha) or "adagrad".
+    Returns params after every step: list of lists of arrays."""
     tp = [api.tensor(np.asarray(p, np.float32)) for p in params]
     tg = [api.zeros(np.asarray(p).shape) for p in params]
-    opt = api.boat_adam_optimizer_create(lr, beta1, beta2, eps)
+    if kind == "adam":
+        opt = api.boat_adam_optimizer_create(lr, beta1, beta2, eps)
+    elif kind == "rmsprop":
+        opt = api.boat_rmsprop_optimizer_create(lr, beta1, eps)
+    else:
+        opt = api.boat_adagrad_optimizer_create(lr, eps)
+    assert opt, f"{kind} optimizer creation failed"
     for p, g in zip(tp, tg):
         api.boat_optimizer_add_parameter(opt, p, g)
     out = []

@@ -26,7 +26,12 @@ import oracle_lib  # noqa: E402
 from test_oracle_vs_reference import ATT_CASES, make_attention_inputs  # noqa: E402
 
 
+ONLY = set(sys.argv[1:])   # fixture names to (re)write; none given = all
+
+
 def save(name, **arrays):
+    if ONLY and name not in ONLY:
+        return
     path = HERE / f"{name}.npz"
     np.savez_compressed(path, **{k: np.asarray(v) for k, v in arrays.items() if v is not None})
     print(f"{path.name}: {path.stat().st_size / 1024:.1f} KiB, {len(arrays)} arrays")
@@ -163,6 +168,18 @@ def main():
         arrays[f"g{i}"] = np.stack([g[i] for g in grads])
         arrays[f"traj{i}"] = np.stack([t[i] for t in traj])
     save("adam_traj", **arrays)
+
+    r2 = np.random.default_rng(20250612)   # its own stream, so the fixtures above never change
+    for kind in ("rmsprop", "adagrad"):
+        params = [r2.standard_normal(s).astype(np.float32) for s in shapes]
+        grads = [[(r2.standard_normal(s) * 10 ** r2.uniform(-4, 1)).astype(np.float32) for s in shapes] for _ in range(10)]
+        traj, _ = bc.adam_trajectory(ref, params, grads, lr=1e-2, beta1=0.99, eps=1e-8, lr_change=(5, 3e-3), kind=kind)
+        arrays = {}
+        for i in range(3):
+            arrays[f"p{i}"] = params[i]
+            arrays[f"g{i}"] = np.stack([g[i] for g in grads])
+            arrays[f"traj{i}"] = np.stack([t[i] for t in traj])
+        save(f"{kind}_traj", **arrays)
 
     a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
     da, db = bc.fanout(ref, a, b)

@@ -225,6 +225,17 @@ class Oracle:
                                 C.c_float(eps), L(t))
         return p, m, v
 
+    def rmsprop_update(self, p, g, sq, lr, alpha, eps):
+        """In place on copies; returns (p, sq)."""
+        p, sq, g = f32(p).copy(), f32(sq).copy(), f32(g)
+        self.lib.bo_rmsprop_update(fp(p), fp(g), fp(sq), L(p.size), C.c_float(lr), C.c_float(alpha), C.c_float(eps))
+        return p, sq
+
+    def adagrad_update(self, p, g, acc, lr, eps):
+        p, acc, g = f32(p).copy(), f32(acc).copy(), f32(g)
+        self.lib.bo_adagrad_update(fp(p), fp(g), fp(acc), L(p.size), C.c_float(lr), C.c_float(eps))
+        return p, acc
+
     def mse_loss(self, pred, target):
         pred, target = f32(pred), f32(target)
         return float(self.lib.bo_mse_loss(fp(pred), fp(target), L(pred.size)))

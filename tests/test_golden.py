@@ -179,6 +179,18 @@ def test_oracle_adam_golden(oracle):
             assert same(p.reshape(g[f"p{i}"].shape), g[f"traj{i}"][t]), (i, t)
 
 
+@pytest.mark.parametrize("kind", ["rmsprop", "adagrad"])
+def test_oracle_rmsprop_adagrad_golden(oracle, kind):
+    from test_oracle_vs_reference import oracle_sq_trajectory
+    g = load(f"{kind}_traj")
+    params = [g[f"p{i}"] for i in range(3)]
+    grads = [[g[f"g{i}"][t] for i in range(3)] for t in range(10)]
+    want = oracle_sq_trajectory(oracle, kind, params, grads, 1e-2, 0.99, 1e-8, lr_change=(5, 3e-3))
+    for t in range(10):
+        for i in range(3):
+            assert same(want[t][i], g[f"traj{i}"][t]), (t, i)
+
+
 def test_oracle_f64_closed_forms_against_library_vectors(oracle):
     """LayerNorm backward and GELU: no reference implementation; the oracle's float64 closed forms
     against float64 autograd vectors of an independent library."""
@@ -317,6 +329,21 @@ def test_gpu_adam_golden_bit_exact(boat):
         for i in range(3):
             assert same(traj[t][i], g[f"traj{i}"][t]), (t, i)
     assert all(not z.any() for z in zeroed)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["rmsprop", "adagrad"])
+def test_gpu_rmsprop_adagrad_golden_bit_exact(boat, kind):
+    g = load(f"{kind}_traj")
+    params = [g[f"p{i}"] for i in range(3)]
+    grads = [[g[f"g{i}"][t] for i in range(3)] for t in range(10)]
+    traj, zeroed = bc.adam_trajectory(boat, params, grads, lr=1e-2, beta1=0.99, eps=1e-8, lr_change=(5, 3e-3), kind=kind)
+    for t in range(10):
+        for i in range(3):
+            assert same(traj[t][i], g[f"traj{i}"][t]), (t, i)
+    assert all(not z.any() for z in zeroed)
+    assert not boat.boat_rmsprop_optimizer_create(0.0, 0.9, 1e-8) and not boat.boat_rmsprop_optimizer_create(0.1, 1.0, 1e-8)
+    assert not boat.boat_adagrad_optimizer_create(0.1, 0.0)
 
 
 @pytest.mark.gpu

@@ -186,6 +186,24 @@ def test_adam_multi_tensor_bit_exact(hip, oracle, rng):
         assert np.array_equal(d[2][i].numpy(), m) and np.array_equal(d[3][i].numpy(), v)
 
 
+@pytest.mark.parametrize("n", [1, 7, 4096, (1 << 20) + 3])
+def test_rmsprop_adagrad_bit_exact_over_steps(hip, oracle, rng, n):
+    for kind in ("rmsprop", "adagrad"):
+        p = rng.standard_normal(n).astype(np.float32)
+        st = np.zeros(n, np.float32)
+        dp, dst = dev(hip, p), dev(hip, st)
+        for step in range(3):
+            g = (rng.standard_normal(n) * 10 ** rng.uniform(-3, 0)).astype(np.float32)
+            dg = dev(hip, g)
+            if kind == "rmsprop":
+                hip.check(hip.bh_rmsprop_update(dp.ptr, dg.ptr, dst.ptr, n, 1e-2, 0.99, 1e-8))
+                p, st = oracle.rmsprop_update(p, g, st, 1e-2, 0.99, 1e-8)
+            else:
+                hip.check(hip.bh_adagrad_update(dp.ptr, dg.ptr, dst.ptr, n, 1e-2, 1e-8))
+                p, st = oracle.adagrad_update(p, g, st, 1e-2, 1e-8)
+            assert np.array_equal(dp.numpy(), p) and np.array_equal(dst.numpy(), st), (kind, step)
+
+
 def test_adam_zero_gradient_is_a_no_op(hip):
     p = hip.to_device(np.full(1000, 1.5, np.float32))
     g, m, v = hip.zeros(1000), hip.zeros(1000), hip.zeros(1000)

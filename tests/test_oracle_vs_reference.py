@@ -191,6 +191,46 @@ def test_adam_trajectory_bit_exact(ref, oracle, rng):
     assert all(np.all(z == 0) for z in zeroed)
 
 
+def oracle_sq_trajectory(oracle, kind, params, grads, lr, alpha, eps, lr_change=None):
+    """RMSprop / Adagrad trajectories restated with the oracle: list over steps of lists of arrays."""
+    p = [np.asarray(a, np.float32).copy() for a in params]
+    st = [np.zeros_like(a) for a in p]
+    out = []
+    for t, gstep in enumerate(grads):
+        if lr_change and t >= lr_change[0]:
+            lr = lr_change[1]
+        for i in range(len(p)):
+            if kind == "rmsprop":
+                pi, si = oracle.rmsprop_update(p[i], gstep[i], st[i], lr, alpha, eps)
+            else:
+                pi, si = oracle.adagrad_update(p[i], gstep[i], st[i], lr, eps)
+            p[i], st[i] = pi.reshape(p[i].shape), si.reshape(p[i].shape)
+        out.append([a.copy() for a in p])
+    return out
+
+
+@pytest.mark.parametrize("kind", ["rmsprop", "adagrad"])
+def test_rmsprop_adagrad_trajectory_bit_exact(ref, oracle, rng, kind, capfd):
+    # tests/unit/test_optimizer_rmsprop.c / test_optimizer_adagrad.c only assert "the parameter moved";
+    # here whole trajectories of three tensors over ten steps, with a learning-rate change, must agree exactly
+    shapes = [(4, 3), (7,), (1,)]
+    params = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    grads = [[(rng.standard_normal(s) * 10 ** rng.uniform(-4, 1)).astype(np.float32) for s in shapes] for _ in range(10)]
+    got, zeroed = bc.adam_trajectory(ref, params, grads, lr=1e-2, beta1=0.99, eps=1e-8, lr_change=(5, 3e-3), kind=kind)
+    want = oracle_sq_trajectory(oracle, kind, params, grads, 1e-2, 0.99, 1e-8, lr_change=(5, 3e-3))
+    for t in range(10):
+        for i in range(3):
+            assert same(want[t][i], got[t][i]), (t, i)
+    assert all(np.all(z == 0) for z in zeroed)
+    # closed form of the first step from zero state: RMSprop dp = -lr*g/(sqrt((1-a))*|g| + eps); Adagrad dp = -lr*g/(|g| + eps)
+    g0, p0 = np.float64(grads[0][1]), np.float64(params[1])
+    den = np.sqrt(1 - 0.99) * np.abs(g0) + 1e-8 if kind == "rmsprop" else np.abs(g0) + 1e-8
+    assert np.allclose(got[0][1], p0 - 1e-2 * g0 / den, rtol=1e-5, atol=1e-7)
+    # creation validation (rmsprop.c:33-57, adagrad.c:41-50)
+    assert not ref.boat_rmsprop_optimizer_create(0.0, 0.9, 1e-8) and not ref.boat_rmsprop_optimizer_create(0.1, 1.0, 1e-8)
+    assert not ref.boat_adagrad_optimizer_create(0.1, 0.0) and not ref.boat_adagrad_optimizer_create(-1.0, 1e-8)
+
+
 def test_adam_first_step_closed_form(ref, oracle):
     # from m = v = 0: p -= lr*g/(|g|+eps)  =>  p=5, g=2, lr=.01 -> 4.99 (tests/unit/test_optimizer_adam.c:96-108)
     got, _ = bc.adam_trajectory(ref, [np.array([5.0], np.float32)], [[np.array([2.0], np.float32)]], lr=0.01)

@@ -89,6 +89,19 @@ _SIGS = {
     "boat_dense_layer_update": (None, [P, C.c_float]),
     "boat_dense_layer_get_weight": (P, [P]), "boat_dense_layer_get_bias": (P, [P]),
     "boat_dense_layer_get_grad_weight": (P, [P]), "boat_dense_layer_get_grad_bias": (P, [P]),
+    # conv / pool / flatten
+    "boat_conv_layer_create": (P, [C.c_size_t] * 5), "boat_conv_layer_free": (None, [P]),
+    "boat_conv_layer_forward": (P, [P, P]), "boat_conv_layer_backward": (P, [P, P]),
+    "boat_conv_layer_update": (None, [P, C.c_float]),
+    "boat_conv_layer_set_weight": (None, [P, P]), "boat_conv_layer_set_bias": (None, [P, P]),
+    "boat_pool_layer_update": (None, [P, C.c_float]), "boat_flatten_layer_update": (None, [P, C.c_float]),
+    "boat_conv_layer_get_weight": (P, [P]), "boat_conv_layer_get_bias": (P, [P]),
+    "boat_conv_layer_get_grad_weight": (P, [P]), "boat_conv_layer_get_grad_bias": (P, [P]),
+    "boat_pool_layer_create": (P, [C.c_size_t] * 3), "boat_pool_layer_free": (None, [P]),
+    "boat_pool_layer_forward": (P, [P, P]), "boat_pool_layer_backward": (P, [P, P]),
+    "boat_flatten_layer_create": (P, []), "boat_flatten_layer_free": (None, [P]),
+    "boat_flatten_layer_forward": (P, [P, P]), "boat_flatten_layer_backward": (P, [P, P]),
+    "boat_var_conv": (P, [P, P]), "boat_var_pool": (P, [P, P]), "boat_var_flatten": (P, [P]),
     # relu / softmax hooks
     "boat_relu_layer_create": (P, []), "boat_relu_layer_free": (None, [P]),
     "boat_relu_layer_forward": (P, [P, P]), "boat_relu_layer_backward": (P, [P, P]),
@@ -146,6 +159,8 @@ _EXT_SIGS = {
     "boat_hip_layer_from_dense": (P, [P]), "boat_hip_layer_from_norm": (P, [P]),
     "boat_hip_layer_relu": (P, []), "boat_hip_layer_gelu": (P, []),
     "boat_hip_optimizer_add_dense": (None, [P, P]),
+    "boat_hip_optimizer_add_conv": (None, [P, P]),
+    "boat_hip_conv_reference_input_grad": (None, [C.c_int]),
     "boat_hip_optimizer_add_attention": (None, [P, P]),
     "boat_hip_optimizer_add_layernorm": (None, [P, P]),
     "boat_layernorm_update": (None, [P, C.c_float]),

@@ -22,7 +22,7 @@
 
 typedef enum {
     OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_RELU, OP_SIGMOID, OP_TANH, OP_MATMUL, OP_DOT, OP_SUM, OP_MEAN,
-    OP_SOFTMAX, OP_LOG_SOFTMAX, OP_FLATTEN, OP_DENSE, OP_ATTENTION, OP_GELU, OP_LAYERNORM
+    OP_SOFTMAX, OP_LOG_SOFTMAX, OP_FLATTEN, OP_DENSE, OP_ATTENTION, OP_GELU, OP_LAYERNORM, OP_CONV, OP_POOL
 } op_type_t;
 
 typedef struct boat_op {
@@ -294,6 +294,19 @@ boat_variable_t* boat_var_dense(const boat_variable_t* input, const struct boat_
     return record(OP_DENSE, in, 1, boat_dense_layer_forward((boat_dense_layer_t*)layer, input->data), input->requires_grad, (void*)layer);
 }
 
+/* like dense, these record only when their input requires grad (autodiff.c:2155, 2221) */
+boat_variable_t* boat_var_conv(const boat_variable_t* input, const struct boat_conv_layer_t* layer) {
+    if (!input || !layer) return NULL;
+    boat_variable_t* in[1] = {(boat_variable_t*)input};
+    return record(OP_CONV, in, 1, boat_conv_layer_forward((boat_conv_layer_t*)layer, input->data), input->requires_grad, (void*)layer);
+}
+
+boat_variable_t* boat_var_pool(const boat_variable_t* input, const struct boat_pool_layer_t* layer) {
+    if (!input || !layer) return NULL;
+    boat_variable_t* in[1] = {(boat_variable_t*)input};
+    return record(OP_POOL, in, 1, boat_pool_layer_forward((boat_pool_layer_t*)layer, input->data), input->requires_grad, (void*)layer);
+}
+
 boat_variable_t* boat_var_attention(const boat_variable_t* q, const boat_variable_t* k, const boat_variable_t* v,
                                     const struct boat_attention_t* attention, const boat_tensor_t* mask) {
     if (!q || !k || !v || !attention) return NULL;
@@ -504,6 +517,18 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
             break;
         case OP_DENSE: {       /* :2640-2672 */
             boat_tensor_t* dx = boat_dense_layer_backward((boat_dense_layer_t*)op->layer, dy);
+            if (dx && a->requires_grad) accumulate(a, dx, true);
+            else boat_tensor_free(dx);
+            break;
+        }
+        case OP_CONV: {        /* :2349-2386 */
+            boat_tensor_t* dx = boat_conv_layer_backward((boat_conv_layer_t*)op->layer, dy);
+            if (dx && a->requires_grad) accumulate(a, dx, true);
+            else boat_tensor_free(dx);
+            break;
+        }
+        case OP_POOL: {        /* :2590-2630 */
+            boat_tensor_t* dx = boat_pool_layer_backward((boat_pool_layer_t*)op->layer, dy);
             if (dx && a->requires_grad) accumulate(a, dx, true);
             else boat_tensor_free(dx);
             break;

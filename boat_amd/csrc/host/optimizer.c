@@ -203,6 +203,12 @@ void boat_hip_optimizer_add_dense(boat_optimizer_t* opt, boat_dense_layer_t* lay
     if (layer->use_bias) boat_optimizer_add_parameter(opt, layer->bias, layer->grad_bias);
 }
 
+void boat_hip_optimizer_add_conv(boat_optimizer_t* opt, boat_conv_layer_t* layer) {
+    if (!opt || !layer) return;
+    boat_optimizer_add_parameter(opt, boat_conv_layer_get_weight(layer), boat_conv_layer_get_grad_weight(layer));
+    boat_optimizer_add_parameter(opt, boat_conv_layer_get_bias(layer), boat_conv_layer_get_grad_bias(layer));
+}
+
 void boat_hip_optimizer_add_layernorm(boat_optimizer_t* opt, boat_layernorm_t* norm) {
     if (!opt || !norm) return;
     if (norm->weight) boat_optimizer_add_parameter(opt, norm->weight, norm->grad_weight);

@@ -59,6 +59,10 @@ _SIGS = {
     "bh_sdpa_backward": (I, [P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_force_general": (I, [I]),
     "bh_adam_update": (I, [P, P, P, P, L, F, F, F, F, L]),
+    "bh_conv2d_forward": (I, [P, P, P, P] + [L] * 8),
+    "bh_conv2d_backward": (I, [P, P, P, P, P, P] + [L] * 8 + [I, I]),
+    "bh_maxpool2d_forward": (I, [P, P, P] + [L] * 6),
+    "bh_maxpool2d_backward": (I, [P, P, P] + [L] * 6),
     "bh_rmsprop_update": (I, [P, P, P, L, F, F, F]),
     "bh_adagrad_update": (I, [P, P, P, L, F, F]),
     "bh_adam_update_multi": (I, [C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(L), I, F, F, F, F, L]),

@@ -127,6 +127,8 @@ typedef struct boat_variable_t boat_variable_t;
 typedef struct boat_autodiff_context_t boat_autodiff_context_t;
 struct boat_dense_layer_t;
 struct boat_attention_t;
+struct boat_conv_layer_t;
+struct boat_pool_layer_t;
 
 BOAT_API boat_variable_t* boat_variable_create(boat_tensor_t* tensor, bool requires_grad);
 BOAT_API boat_variable_t* boat_variable_create_with_shape(const int64_t* shape, size_t ndim, boat_dtype_t dtype, bool requires_grad);
@@ -148,6 +150,8 @@ BOAT_API boat_variable_t* boat_var_matmul(const boat_variable_t* a, const boat_v
 BOAT_API boat_variable_t* boat_var_dot(const boat_variable_t* a, const boat_variable_t* b);
 BOAT_API boat_variable_t* boat_var_flatten(const boat_variable_t* input);
 BOAT_API boat_variable_t* boat_var_dense(const boat_variable_t* input, const struct boat_dense_layer_t* layer);
+BOAT_API boat_variable_t* boat_var_conv(const boat_variable_t* input, const struct boat_conv_layer_t* layer);
+BOAT_API boat_variable_t* boat_var_pool(const boat_variable_t* input, const struct boat_pool_layer_t* layer);
 BOAT_API boat_variable_t* boat_var_attention(const boat_variable_t* query, const boat_variable_t* key, const boat_variable_t* value,
                                              const struct boat_attention_t* attention, const boat_tensor_t* attention_mask);
 BOAT_API boat_variable_t* boat_var_relu(const boat_variable_t* a);
@@ -179,6 +183,34 @@ BOAT_API boat_tensor_t* boat_dense_layer_get_weight(const boat_dense_layer_t* la
 BOAT_API boat_tensor_t* boat_dense_layer_get_bias(const boat_dense_layer_t* layer);
 BOAT_API boat_tensor_t* boat_dense_layer_get_grad_weight(const boat_dense_layer_t* layer);
 BOAT_API boat_tensor_t* boat_dense_layer_get_grad_bias(const boat_dense_layer_t* layer);
+
+/* ---- include/boat/layers.h:38-51 (2-D convolution), :68-72 (max pooling), :128-132 (flatten) ---- */
+typedef struct boat_conv_layer_t boat_conv_layer_t;
+BOAT_API boat_conv_layer_t* boat_conv_layer_create(size_t in_channels, size_t out_channels, size_t kernel_size, size_t stride, size_t padding);
+BOAT_API void boat_conv_layer_free(boat_conv_layer_t* layer);
+BOAT_API boat_tensor_t* boat_conv_layer_forward(boat_conv_layer_t* layer, const boat_tensor_t* input);
+/* grad_weight/grad_bias are overwritten in place (the reference replaces the tensors, src/layers/conv.c:523-532);
+ * the returned input gradient is the true one (the reference mirrors the kernel taps, conv.c:86-88) */
+BOAT_API boat_tensor_t* boat_conv_layer_backward(boat_conv_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_conv_layer_update(boat_conv_layer_t* layer, float learning_rate);
+BOAT_API void boat_conv_layer_set_weight(boat_conv_layer_t* layer, boat_tensor_t* weight);
+BOAT_API void boat_conv_layer_set_bias(boat_conv_layer_t* layer, boat_tensor_t* bias);
+BOAT_API boat_tensor_t* boat_conv_layer_get_weight(const boat_conv_layer_t* layer);
+BOAT_API boat_tensor_t* boat_conv_layer_get_bias(const boat_conv_layer_t* layer);
+BOAT_API boat_tensor_t* boat_conv_layer_get_grad_weight(const boat_conv_layer_t* layer);
+BOAT_API boat_tensor_t* boat_conv_layer_get_grad_bias(const boat_conv_layer_t* layer);
+typedef struct boat_pool_layer_t boat_pool_layer_t;
+BOAT_API boat_pool_layer_t* boat_pool_layer_create(size_t pool_size, size_t stride, size_t padding);
+BOAT_API void boat_pool_layer_free(boat_pool_layer_t* layer);
+BOAT_API boat_tensor_t* boat_pool_layer_forward(boat_pool_layer_t* layer, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_pool_layer_backward(boat_pool_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_pool_layer_update(boat_pool_layer_t* layer, float learning_rate);
+typedef struct boat_flatten_layer_t boat_flatten_layer_t;
+BOAT_API boat_flatten_layer_t* boat_flatten_layer_create(void);
+BOAT_API void boat_flatten_layer_free(boat_flatten_layer_t* layer);
+BOAT_API boat_tensor_t* boat_flatten_layer_forward(boat_flatten_layer_t* layer, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_flatten_layer_backward(const boat_flatten_layer_t* layer, const boat_tensor_t* grad_output);
+BOAT_API void boat_flatten_layer_update(boat_flatten_layer_t* layer, float learning_rate);
 
 /* ---- include/boat/layers.h:95-107 (activation layers) ---- */
 typedef struct boat_relu_layer_t boat_relu_layer_t;
@@ -331,6 +363,10 @@ BOAT_API boat_layer_t* boat_hip_layer_relu(void);
 BOAT_API boat_layer_t* boat_hip_layer_gelu(void);
 /* register every trainable tensor of a layer with an optimizer */
 BOAT_API void boat_hip_optimizer_add_dense(boat_optimizer_t* opt, boat_dense_layer_t* layer);
+BOAT_API void boat_hip_optimizer_add_conv(boat_optimizer_t* opt, boat_conv_layer_t* layer);
+/* enable != 0: boat_conv_layer_backward returns the reference's input gradient (each tap paired with the mirrored
+ * weight, src/layers/conv.c:86-88) instead of the true one; process-wide, off by default */
+BOAT_API void boat_hip_conv_reference_input_grad(int enable);
 BOAT_API void boat_hip_optimizer_add_attention(boat_optimizer_t* opt, boat_attention_t* attention);
 BOAT_API void boat_hip_optimizer_add_layernorm(boat_optimizer_t* opt, boat_layernorm_t* norm);
 

@@ -138,6 +138,23 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
                      const float* d_out, float scale, int causal,
                      float* dq, float* dk, float* dv, int64_t bh, int64_t s, int64_t d);
 
+/* ---- 2-D convolution and max pooling, NCHW, square kernel/window (src/layers/conv.c:46-201,326-437; src/layers/pool.c:63-218) ----
+ * x [batch, in_channels, height, width]; w [out_channels, in_channels, kernel, kernel]; bias [out_channels] or NULL;
+ * y / dy [batch, out_channels, ho, wo] with ho = (height + 2*pad - kernel)/stride + 1.
+ * backward: dx (assigned; may be NULL), gw and gb (assigned unless accumulate; may be NULL).  flip_taps == 0 gives the
+ * true input gradient; flip_taps != 0 pairs each tap with the mirrored weight as conv.c:86-88 does. */
+int bh_conv2d_forward(const float* x, const float* w, const float* bias, float* y, int64_t batch, int64_t in_channels,
+                      int64_t height, int64_t width, int64_t out_channels, int64_t kernel, int64_t stride, int64_t pad);
+int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t batch,
+                       int64_t in_channels, int64_t height, int64_t width, int64_t out_channels, int64_t kernel,
+                       int64_t stride, int64_t pad, int accumulate, int flip_taps);
+/* planes = batch*channels images of [height, width]; argmax holds, per output, the offset of the window's first maximum
+ * inside its plane (-1 when the window holds no comparable value) */
+int bh_maxpool2d_forward(const float* x, float* y, int32_t* argmax, int64_t planes, int64_t height, int64_t width, int64_t pool,
+                         int64_t stride, int64_t pad);
+int bh_maxpool2d_backward(const float* dy, const int32_t* argmax, float* dx, int64_t planes, int64_t height, int64_t width,
+                          int64_t pool, int64_t stride, int64_t pad);
+
 /* ---- Adam (src/optimizers/adam.c:180-240) ----
  * timestep is the pre-increment value the reference passes to powf(beta, (float)(t+1)). */
 int bh_adam_update(float* p, const float* g, float* m, float* v, int64_t n,

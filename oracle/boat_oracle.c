@@ -433,6 +433,112 @@ void bo_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
     }
 }
 
+/* ------------------------------------------------------------- conv / pool */
+
+/* src/layers/conv.c:398-436: per (b, oc): for each input channel a running sum over the taps is added to the
+ * output element; the bias is added last. */
+void bo_conv2d_forward(const float* x, const float* w, const float* bias, float* y,
+                       int64_t batch, int64_t ic, int64_t h, int64_t wd, int64_t oc, int64_t k, int64_t stride, int64_t pad) {
+    const int64_t ho = (h + 2 * pad - k) / stride + 1, wo = (wd + 2 * pad - k) / stride + 1;
+    memset(y, 0, sizeof(float) * (size_t)(batch * oc * ho * wo));
+    for (int64_t b = 0; b < batch; b++)
+        for (int64_t o = 0; o < oc; o++) {
+            for (int64_t c = 0; c < ic; c++)
+                for (int64_t oh = 0; oh < ho; oh++)
+                    for (int64_t ow = 0; ow < wo; ow++) {
+                        float sum = 0.0f;
+                        for (int64_t kh = 0; kh < k; kh++) {
+                            int64_t ih = oh * stride - pad + kh;
+                            if (ih < 0 || ih >= h) continue;
+                            for (int64_t kw = 0; kw < k; kw++) {
+                                int64_t iw = ow * stride - pad + kw;
+                                if (iw < 0 || iw >= wd) continue;
+                                sum += x[((b * ic + c) * h + ih) * wd + iw] * w[((o * ic + c) * k + kh) * k + kw];
+                            }
+                        }
+                        y[((b * oc + o) * ho + oh) * wo + ow] += sum;
+                    }
+            if (bias)
+                for (int64_t i = 0; i < ho * wo; i++) y[(b * oc + o) * ho * wo + i] += bias[o];
+        }
+}
+
+/* src/layers/conv.c:46-201.  All three gradients are overwritten.  flip_taps != 0 is the reference as written:
+ * the input gradient pairs tap (kh, kw) with the weight of tap (k-1-kh, k-1-kw) (:86-88); flip_taps == 0 uses the
+ * weight of the same tap, which is the true gradient of bo_conv2d_forward. */
+void bo_conv2d_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb,
+                        int64_t batch, int64_t ic, int64_t h, int64_t wd, int64_t oc, int64_t k, int64_t stride, int64_t pad,
+                        int flip_taps) {
+    const int64_t ho = (h + 2 * pad - k) / stride + 1, wo = (wd + 2 * pad - k) / stride + 1;
+    if (dx) memset(dx, 0, sizeof(float) * (size_t)(batch * ic * h * wd));
+    if (gw) memset(gw, 0, sizeof(float) * (size_t)(oc * ic * k * k));
+    for (int64_t b = 0; b < batch; b++)
+        for (int64_t o = 0; o < oc; o++)
+            for (int64_t c = 0; c < ic; c++)
+                for (int64_t kh = 0; kh < k; kh++)
+                    for (int64_t kw = 0; kw < k; kw++)
+                        for (int64_t oh = 0; oh < ho; oh++) {
+                            int64_t ih = oh * stride - pad + kh;
+                            if (ih < 0 || ih >= h) continue;
+                            for (int64_t ow = 0; ow < wo; ow++) {
+                                int64_t iw = ow * stride - pad + kw;
+                                if (iw < 0 || iw >= wd) continue;
+                                const int64_t xi = ((b * ic + c) * h + ih) * wd + iw;
+                                const int64_t gi = ((b * oc + o) * ho + oh) * wo + ow;
+                                if (dx) {
+                                    const int64_t wi = flip_taps ? ((o * ic + c) * k + (k - 1 - kh)) * k + (k - 1 - kw)
+                                                                 : ((o * ic + c) * k + kh) * k + kw;
+                                    dx[xi] += w[wi] * dy[gi];
+                                }
+                                if (gw) gw[((o * ic + c) * k + kh) * k + kw] += x[xi] * dy[gi];
+                            }
+                        }
+    if (gb) {
+        memset(gb, 0, sizeof(float) * (size_t)oc);
+        for (int64_t b = 0; b < batch; b++)
+            for (int64_t o = 0; o < oc; o++) {
+                float sum = 0.0f;
+                for (int64_t i = 0; i < ho * wo; i++) sum += dy[(b * oc + o) * ho * wo + i];
+                gb[o] += sum;
+            }
+    }
+}
+
+/* src/layers/pool.c:100-133: window clamped to the image, first maximum wins (strict >); argmax is the flat input index or -1 */
+void bo_maxpool2d_forward(const float* x, float* y, int64_t* argmax, int64_t planes, int64_t h, int64_t wd,
+                          int64_t pool, int64_t stride, int64_t pad) {
+    const int64_t ho = (h + 2 * pad - pool) / stride + 1, wo = (wd + 2 * pad - pool) / stride + 1;
+    for (int64_t p = 0; p < planes; p++)
+        for (int64_t oh = 0; oh < ho; oh++)
+            for (int64_t ow = 0; ow < wo; ow++) {
+                int64_t h0 = oh * stride - pad, w0 = ow * stride - pad;
+                int64_t h1 = h0 + pool, w1 = w0 + pool;
+                h0 = h0 < 0 ? 0 : h0;
+                w0 = w0 < 0 ? 0 : w0;
+                h1 = h1 > h ? h : h1;
+                w1 = w1 > wd ? wd : w1;
+                float best = -INFINITY;
+                int64_t where = -1;
+                for (int64_t ph = h0; ph < h1; ph++)
+                    for (int64_t pw = w0; pw < w1; pw++) {
+                        const int64_t idx = (p * h + ph) * wd + pw;
+                        if (x[idx] > best) {
+                            best = x[idx];
+                            where = idx;
+                        }
+                    }
+                y[(p * ho + oh) * wo + ow] = best;
+                argmax[(p * ho + oh) * wo + ow] = where;
+            }
+}
+
+/* src/layers/pool.c:199-213 */
+void bo_maxpool2d_backward(const float* dy, const int64_t* argmax, float* dx, int64_t n_in, int64_t n_out) {
+    memset(dx, 0, sizeof(float) * (size_t)n_in);
+    for (int64_t i = 0; i < n_out; i++)
+        if (argmax[i] >= 0 && argmax[i] < n_in) dx[argmax[i]] += dy[i];
+}
+
 /* src/optimizers/rmsprop.c:197-210 */
 void bo_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps) {
     for (int64_t i = 0; i < n; i++) {

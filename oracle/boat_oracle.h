@@ -109,6 +109,19 @@ void bo_layernorm_forward(const float* x, const float* gamma, const float* beta,
 void bo_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
                     float lr, float beta1, float beta2, float eps, int64_t timestep);
 
+/* src/layers/conv.c:326-437 (NCHW, weight [oc, ic, k, k], bias may be NULL). */
+void bo_conv2d_forward(const float* x, const float* w, const float* bias, float* y,
+                       int64_t batch, int64_t ic, int64_t h, int64_t wd, int64_t oc, int64_t k, int64_t stride, int64_t pad);
+/* src/layers/conv.c:46-201; dx, gw, gb may be NULL.  flip_taps != 0 reproduces the reference's input gradient
+ * (mirrored taps, :86-88); flip_taps == 0 is the true gradient. */
+void bo_conv2d_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb,
+                        int64_t batch, int64_t ic, int64_t h, int64_t wd, int64_t oc, int64_t k, int64_t stride, int64_t pad,
+                        int flip_taps);
+/* src/layers/pool.c:63-218; planes = batch*channels; argmax = flat input index of each window's maximum. */
+void bo_maxpool2d_forward(const float* x, float* y, int64_t* argmax, int64_t planes, int64_t h, int64_t wd,
+                          int64_t pool, int64_t stride, int64_t pad);
+void bo_maxpool2d_backward(const float* dy, const int64_t* argmax, float* dx, int64_t n_in, int64_t n_out);
+
 /* src/optimizers/rmsprop.c:181-211 and src/optimizers/adagrad.c:167-197: one tensor, one step. */
 void bo_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps);
 void bo_adagrad_update(float* p, const float* g, float* sum, int64_t n, float lr, float eps);

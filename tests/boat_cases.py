@@ -395,3 +395,104 @@ def transformer_block_steps(api, x, target, params, heads, steps=1, lr=1e-3, bet
     for norm in ln:
         api.boat_layernorm_free(norm)
     return history
+
+
+def _make_conv(api, w, b, stride, pad):
+    oc, ic, k, _ = w.shape
+    layer = api.boat_conv_layer_create(ic, oc, k, stride, pad)
+    api.write(api.boat_conv_layer_get_weight(layer), w)        # in place (set_weight would swap tensors)
+    api.write(api.boat_conv_layer_get_bias(layer), b)
+    return layer
+
+
+def conv_layer(api, x, w, b, stride, pad, d_out_list):
+    """boat_conv_layer_forward once, then boat_conv_layer_backward per dY (parameter grads are overwritten per call).
+    Returns y and per call (dx, grad_weight, grad_bias)."""
+    layer = _make_conv(api, np.asarray(w, np.float32), np.asarray(b, np.float32), stride, pad)
+    tx = api.tensor(np.asarray(x, np.float32))
+    ty = api.boat_conv_layer_forward(layer, tx)
+    y = api.numpy(ty)
+    out = []
+    for dy in d_out_list:
+        tdy = api.tensor(np.asarray(dy, np.float32))
+        tdx = api.boat_conv_layer_backward(layer, tdy)
+        assert tdx, "boat_conv_layer_backward failed"
+        out.append((api.numpy(tdx), api.numpy(api.boat_conv_layer_get_grad_weight(layer)),
+                    api.numpy(api.boat_conv_layer_get_grad_bias(layer))))
+        api.boat_tensor_unref(tdx)
+        api.boat_tensor_unref(tdy)
+    api.boat_tensor_unref(ty)
+    api.boat_tensor_unref(tx)
+    api.boat_conv_layer_free(layer)
+    return y, out
+
+
+def pool_layer(api, x, pool, stride, pad, dy):
+    """boat_pool_layer_forward / backward.  Returns y, dx."""
+    layer = api.boat_pool_layer_create(pool, stride, pad)
+    tx = api.tensor(np.asarray(x, np.float32))
+    ty = api.boat_pool_layer_forward(layer, tx)
+    y = api.numpy(ty)
+    tdy = api.tensor(np.asarray(dy, np.float32))
+    tdx = api.boat_pool_layer_backward(layer, tdy)
+    assert tdx, "boat_pool_layer_backward failed"
+    dx = api.numpy(tdx)
+    for t in (tdx, tdy, ty, tx):
+        api.boat_tensor_unref(t)
+    api.boat_pool_layer_free(layer)
+    return y, dx
+
+
+def cnn_ce_grads(api, x, labels, p, pool=2):
+    """The MNIST network of examples/mnist/mnist_autodiff.c:536-557 on the tape, one forward + backward:
+    conv(3x3, pad 1) -> relu -> maxpool(2) -> conv -> relu -> maxpool -> flatten -> dense -> relu -> dense
+    -> log_softmax -> mul(onehot) -> sum -> mul(-1/B); boat_variable_backward_full.
+    p: dict cw1, cb1, cw2, cb2, w1, b1, w2, b2.  Returns dict(loss, logits, dx, g_<name>...)."""
+    x = np.asarray(x, np.float32)
+    B = x.shape[0]
+    classes = p["w2"].shape[1]
+    c1 = _make_conv(api, p["cw1"], p["cb1"], 1, 1)
+    c2 = _make_conv(api, p["cw2"], p["cb2"], 1, 1)
+    p1, p2 = api.boat_pool_layer_create(pool, pool, 0), api.boat_pool_layer_create(pool, pool, 0)
+    d1 = _make_dense(api, p["w1"], p["b1"])
+    d2 = _make_dense(api, p["w2"], p["b2"])
+    onehot = np.zeros((B, classes), np.float32)
+    onehot[np.arange(B), np.asarray(labels)] = 1.0
+    vx = _var(api, x, True)
+    a1 = api.boat_var_conv(vx, c1)
+    r1 = api.boat_var_relu(a1)
+    q1 = api.boat_var_pool(r1, p1)
+    a2 = api.boat_var_conv(q1, c2)
+    r2 = api.boat_var_relu(a2)
+    q2 = api.boat_var_pool(r2, p2)
+    fl = api.boat_var_flatten(q2)
+    h = api.boat_var_dense(fl, d1)
+    rh = api.boat_var_relu(h)
+    z = api.boat_var_dense(rh, d2)
+    ls = api.boat_var_log_softmax(z, 1)
+    voh = _var(api, onehot, False)
+    m = api.boat_var_mul(voh, ls)
+    s = api.boat_var_sum(m, None, 0, False)
+    vf = _var(api, np.array([-1.0 / B], np.float32), False)
+    loss = api.boat_var_mul(vf, s)
+    rec = {"loss": float(api.numpy(api.boat_variable_data(loss))[0]), "logits": api.numpy(api.boat_variable_data(z))}
+    with scratch_cwd():
+        api.boat_variable_backward_full(loss)
+    rec["dx"] = _grad(api, vx)
+    rec["g_cw1"] = api.numpy(api.boat_conv_layer_get_grad_weight(c1))
+    rec["g_cb1"] = api.numpy(api.boat_conv_layer_get_grad_bias(c1))
+    rec["g_cw2"] = api.numpy(api.boat_conv_layer_get_grad_weight(c2))
+    rec["g_cb2"] = api.numpy(api.boat_conv_layer_get_grad_bias(c2))
+    for name, layer in (("1", d1), ("2", d2)):
+        rec["g_w" + name] = api.numpy(api.boat_dense_layer_get_grad_weight(layer))
+        rec["g_b" + name] = api.numpy(api.boat_dense_layer_get_grad_bias(layer))
+    if api.is_amd:   # the reference cannot release a recorded tape
+        for v in (loss, vf, s, m, voh, ls, z, rh, h, fl, q2, r2, a2, q1, r1, a1, vx):
+            api.boat_variable_free(v)
+        api.boat_conv_layer_free(c1)
+        api.boat_conv_layer_free(c2)
+        api.boat_pool_layer_free(p1)
+        api.boat_pool_layer_free(p2)
+        api.boat_dense_layer_free(d1)
+        api.boat_dense_layer_free(d2)
+    return rec

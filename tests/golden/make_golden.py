@@ -23,7 +23,7 @@ sys.path.insert(0, str(ROOT / "tests"))
 
 import boat_cases as bc  # noqa: E402
 import oracle_lib  # noqa: E402
-from test_oracle_vs_reference import ATT_CASES, make_attention_inputs  # noqa: E402
+from test_oracle_vs_reference import ATT_CASES, CONV_CASES, POOL_CASES, cnn_params, conv_inputs, make_attention_inputs  # noqa: E402
 
 
 ONLY = set(sys.argv[1:])   # fixture names to (re)write; none given = all
@@ -184,6 +184,33 @@ def main():
     a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
     da, db = bc.fanout(ref, a, b)
     save("fanout_divergence", a=a, b=b, ref_da=da, ref_db=db)
+
+    # convolution (two backward calls: parameter gradients are overwritten), max pooling, the MNIST CNN chain
+    conv = {}
+    for i, case in enumerate(CONV_CASES[:3]):
+        d = conv_inputs(case, 500 + i)
+        y, calls = bc.conv_layer(ref, d["x"], d["w"], d["b"], case[6], case[7], [d["dy1"], d["dy2"]])
+        conv.update({f"c{i}_{k}": v for k, v in d.items()})
+        conv.update({f"c{i}_meta": np.array(case), f"c{i}_y": y})
+        for j, (dx, gw, gb) in enumerate(calls):
+            conv.update({f"c{i}_dx{j}": dx, f"c{i}_gw{j}": gw, f"c{i}_gb{j}": gb})
+    save("conv_layer", **conv)
+    r3 = np.random.default_rng(20250613)
+    pool = {}
+    for i, (B, ch, h, w, k, stride, pad) in enumerate(POOL_CASES):
+        x = r3.standard_normal((B, ch, h, w)).astype(np.float32)
+        x[0, 0, :2, :2] = 1.5
+        ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+        dy = r3.standard_normal((B, ch, ho, wo)).astype(np.float32)
+        y, dx = bc.pool_layer(ref, x, k, stride, pad, dy)
+        pool.update({f"p{i}_meta": np.array([k, stride, pad]), f"p{i}_x": x, f"p{i}_dy": dy, f"p{i}_y": y, f"p{i}_dx": dx})
+    save("pool_layer", **pool)
+    x = r3.random((3, 2, 8, 8), dtype=np.float32)
+    labels = r3.integers(0, 5, 3)
+    p = cnn_params(r3, 2, 4, 6, 8, 12, 5)
+    rec = bc.cnn_ce_grads(ref, x, labels, p)
+    save("cnn_chain", x=x, labels=labels, **{"p_" + k: v for k, v in p.items()},
+         **{k: (np.float32(v) if k == "loss" else v) for k, v in rec.items()})
 
     # ---- not the reference: float64 autograd of an independent library ----
     import torch

@@ -225,6 +225,43 @@ class Oracle:
                                 C.c_float(eps), L(t))
         return p, m, v
 
+    def conv2d_forward(self, x, w, bias, stride=1, pad=0):
+        x, w = f32(x), f32(w)
+        bias = None if bias is None else f32(bias)
+        B, ic, h, wd = x.shape
+        oc, _, k, _ = w.shape
+        ho, wo = (h + 2 * pad - k) // stride + 1, (wd + 2 * pad - k) // stride + 1
+        y = np.empty((B, oc, ho, wo), np.float32)
+        self.lib.bo_conv2d_forward(fp(x), fp(w), fp(bias), fp(y), L(B), L(ic), L(h), L(wd), L(oc), L(k), L(stride), L(pad))
+        return y
+
+    def conv2d_backward(self, x, w, dy, stride=1, pad=0, flip_taps=False):
+        """Returns dx, gw, gb (all overwritten).  flip_taps=True is the reference's input gradient."""
+        x, w, dy = f32(x), f32(w), f32(dy)
+        B, ic, h, wd = x.shape
+        oc, _, k, _ = w.shape
+        dx, gw, gb = np.empty_like(x), np.empty_like(w), np.empty(oc, np.float32)
+        self.lib.bo_conv2d_backward(fp(x), fp(w), fp(dy), fp(dx), fp(gw), fp(gb), L(B), L(ic), L(h), L(wd), L(oc), L(k),
+                                    L(stride), L(pad), C.c_int(int(flip_taps)))
+        return dx, gw, gb
+
+    def maxpool2d_forward(self, x, pool, stride, pad=0):
+        x = f32(x)
+        B, ch, h, wd = x.shape
+        ho, wo = (h + 2 * pad - pool) // stride + 1, (wd + 2 * pad - pool) // stride + 1
+        y = np.empty((B, ch, ho, wo), np.float32)
+        arg = np.empty((B, ch, ho, wo), np.int64)
+        self.lib.bo_maxpool2d_forward(fp(x), fp(y), arg.ctypes.data_as(C.POINTER(C.c_int64)), L(B * ch), L(h), L(wd), L(pool),
+                                      L(stride), L(pad))
+        return y, arg
+
+    def maxpool2d_backward(self, dy, argmax, in_shape):
+        dy = f32(dy)
+        argmax = np.ascontiguousarray(argmax, np.int64)
+        dx = np.empty(in_shape, np.float32)
+        self.lib.bo_maxpool2d_backward(fp(dy), argmax.ctypes.data_as(C.POINTER(C.c_int64)), fp(dx), L(dx.size), L(dy.size))
+        return dx
+
     def rmsprop_update(self, p, g, sq, lr, alpha, eps):
         """In place on copies; returns (p, sq)."""
         p, sq, g = f32(p).copy(), f32(sq).copy(), f32(g)

@@ -205,6 +205,34 @@ def test_oracle_f64_closed_forms_against_library_vectors(oracle):
     assert close_max(oracle.gelu_backward_f64(x32, dy32), g["dx"], 1e-6)
 
 
+def cnn_case(g):
+    p = {k[2:]: g[k] for k in g if k.startswith("p_")}
+    return g["x"], g["labels"], p
+
+
+def test_oracle_conv_pool_cnn_golden(oracle):
+    from test_oracle_vs_reference import CNN_KEYS, oracle_cnn_grads
+    g = load("conv_layer")
+    for i in range(3):
+        stride, pad = int(g[f"c{i}_meta"][6]), int(g[f"c{i}_meta"][7])
+        x, w, b = g[f"c{i}_x"], g[f"c{i}_w"], g[f"c{i}_b"]
+        assert same(oracle.conv2d_forward(x, w, b, stride, pad), g[f"c{i}_y"])
+        for j in range(2):
+            dx, gw, gb = oracle.conv2d_backward(x, w, g[f"c{i}_dy{j + 1}"], stride, pad, flip_taps=True)
+            assert same(dx, g[f"c{i}_dx{j}"]) and same(gw, g[f"c{i}_gw{j}"]) and same(gb, g[f"c{i}_gb{j}"]), (i, j)
+    g = load("pool_layer")
+    for i in range(4):
+        k, stride, pad = (int(v) for v in g[f"p{i}_meta"])
+        y, arg = oracle.maxpool2d_forward(g[f"p{i}_x"], k, stride, pad)
+        assert same(y, g[f"p{i}_y"]) and same(oracle.maxpool2d_backward(g[f"p{i}_dy"], arg, g[f"p{i}_x"].shape), g[f"p{i}_dx"]), i
+    g = load("cnn_chain")
+    x, labels, p = cnn_case(g)
+    want = oracle_cnn_grads(oracle, x, labels, p, flip_taps=True)
+    assert np.float32(want["loss"]) == g["loss"]
+    for key in CNN_KEYS:
+        assert same(want[key], g[key]), key
+
+
 def test_fanout_fixture_documents_the_reference_behaviour():
     g = load("fanout_divergence")
     assert same(g["ref_da"], 4 * g["b"]) and same(g["ref_db"], 4 * g["a"])
@@ -366,6 +394,48 @@ def test_gpu_ln_backward_and_gelu_against_library_vectors(hip):
     hip.check(hip.bh_activation_forward(hip.ACT_GELU, dxv.ptr, yv.ptr, x.size))
     hip.check(hip.bh_activation_backward(hip.ACT_GELU, dxv.ptr, ddy.ptr, gx.ptr, x.size, 0))
     assert close_max(yv.numpy(), g["y"], TOL_EW) and close_max(gx.numpy(), g["dx"], TOL_EW)
+
+
+@pytest.mark.gpu
+def test_gpu_conv_pool_cnn_golden(boat):
+    """Convolution, pooling and the CNN chain against the compiled reference's vectors.  The reference pairs each tap of
+    the input gradient with the mirrored weight (src/layers/conv.c:86-88); boat_hip_conv_reference_input_grad(1) selects
+    that pairing so every number can be compared; the default (true gradient) is checked against it through the turned
+    kernel: dx_true(w) == dx_reference(w turned by 180 degrees)."""
+    from test_oracle_vs_reference import CNN_KEYS
+    boat.boat_hip_conv_reference_input_grad(1)
+    try:
+        g = load("conv_layer")
+        for i in range(3):
+            stride, pad = int(g[f"c{i}_meta"][6]), int(g[f"c{i}_meta"][7])
+            x, w, b = g[f"c{i}_x"], g[f"c{i}_w"], g[f"c{i}_b"]
+            y, calls = bc.conv_layer(boat, x, w, b, stride, pad, [g[f"c{i}_dy1"], g[f"c{i}_dy2"]])
+            assert same(y, g[f"c{i}_y"]), i          # forward keeps the reference's operation order: bit exact
+            for j, (dx, gw, gb) in enumerate(calls):
+                assert close_max(dx, g[f"c{i}_dx{j}"], TOL_RED) and close_max(gw, g[f"c{i}_gw{j}"], TOL_RED), (i, j)
+                assert close_max(gb, g[f"c{i}_gb{j}"], TOL_RED), (i, j)
+        c = load("cnn_chain")
+        x, labels, p = cnn_case(c)
+        rec = bc.cnn_ce_grads(boat, x, labels, p)
+        assert abs(rec["loss"] - float(c["loss"])) <= TOL_RED * abs(float(c["loss"]))
+        for key in CNN_KEYS:
+            assert close_max(rec[key], c[key], TOL_GEMM if key.startswith("g_w") else TOL_RED), key
+    finally:
+        boat.boat_hip_conv_reference_input_grad(0)
+    # default mode = true gradient: equals the reference's operator applied to the turned kernel
+    i = 0
+    stride, pad = int(g[f"c{i}_meta"][6]), int(g[f"c{i}_meta"][7])
+    x, w, b, dy = g[f"c{i}_x"], g[f"c{i}_w"], g[f"c{i}_b"], g[f"c{i}_dy1"]
+    boat.boat_hip_conv_reference_input_grad(1)
+    dx_ref_turned = bc.conv_layer(boat, x, np.ascontiguousarray(w[:, :, ::-1, ::-1]), b, stride, pad, [dy])[1][0][0]
+    boat.boat_hip_conv_reference_input_grad(0)
+    dx_true = bc.conv_layer(boat, x, w, b, stride, pad, [dy])[1][0][0]
+    assert same(dx_true, dx_ref_turned)
+    pl = load("pool_layer")
+    for i in range(4):
+        k, stride, pad = (int(v) for v in pl[f"p{i}_meta"])
+        y, dx = bc.pool_layer(boat, pl[f"p{i}_x"], k, stride, pad, pl[f"p{i}_dy"])
+        assert same(y, pl[f"p{i}_y"]) and same(dx, pl[f"p{i}_dx"]), i      # no arithmetic reordering: bit exact
 
 
 @pytest.mark.gpu

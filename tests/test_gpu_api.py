@@ -341,3 +341,136 @@ def test_device_tensors_and_fused_losses(boat, oracle, rng):
     gm = C.c_void_p()
     tl = boat.boat_hip_mse_loss(boat.tensor(p), boat.tensor(t), C.byref(gm))
     assert abs(boat.numpy(tl)[0] - oracle.mse_loss(p, t)) <= TOL_RED and np.array_equal(boat.numpy(gm), oracle.mse_grad(p, t))
+
+
+# ---- convolution / pooling / flatten hooks and the MNIST CNN on the tape ----
+
+def test_conv_known_answer_and_hooks(boat):
+    # tests/test_conv_forward.c:20-165, weights injected with boat_conv_layer_set_weight as the reference's test does
+    x = np.arange(1, 10, dtype=np.float32).reshape(1, 1, 3, 3)
+    w = np.array([1, 0, 0, 1], np.float32).reshape(1, 1, 2, 2)
+    for stride, pad, want_shape in ((1, 0, (1, 1, 2, 2)), (1, 1, (1, 1, 4, 4)), (2, 0, (1, 1, 1, 1))):
+        layer = boat.boat_conv_layer_create(1, 1, 2, stride, pad)
+        tw = boat.tensor(w)
+        boat.boat_conv_layer_set_weight(layer, tw)
+        boat.boat_tensor_unref(tw)
+        tx = boat.tensor(x)
+        ty = boat.boat_conv_layer_forward(layer, tx)
+        y = boat.numpy(ty)
+        assert y.shape == want_shape
+        if pad == 0 and stride == 1:
+            assert y.reshape(-1).tolist() == [6, 8, 12, 14]
+        boat.boat_tensor_unref(ty)
+        boat.boat_tensor_unref(tx)
+        boat.boat_conv_layer_free(layer)
+    # error paths: backward before forward, wrong rank, wrong channel count (conv.c:326-360, 475-500)
+    layer = boat.boat_conv_layer_create(2, 3, 3, 1, 1)
+    g = boat.tensor(np.zeros((1, 3, 4, 4), np.float32))
+    with bc.scratch_cwd():
+        assert not boat.boat_conv_layer_backward(layer, g)
+        bad = boat.tensor(np.zeros((4, 4), np.float32))
+        assert not boat.boat_conv_layer_forward(layer, bad)
+        bad2 = boat.tensor(np.zeros((1, 5, 4, 4), np.float32))
+        assert not boat.boat_conv_layer_forward(layer, bad2)
+    for t in (g, bad, bad2):
+        boat.boat_tensor_unref(t)
+    assert not boat.boat_conv_layer_create(0, 3, 3, 1, 1)
+    # gradient tensors keep their identity across backward calls, so an optimizer may hold them
+    gw_before = boat.boat_conv_layer_get_grad_weight(layer)
+    tx = boat.tensor(np.ones((1, 2, 4, 4), np.float32))
+    ty = boat.boat_conv_layer_forward(layer, tx)
+    tdy = boat.tensor(np.ones((1, 3, 4, 4), np.float32))
+    for _ in range(2):
+        boat.boat_tensor_unref(boat.boat_conv_layer_backward(layer, tdy))
+    assert boat.boat_conv_layer_get_grad_weight(layer) == gw_before
+    assert boat.numpy(boat.boat_conv_layer_get_grad_bias(layer)).tolist() == [16, 16, 16]       # overwritten, not doubled
+    for t in (tdy, ty, tx):
+        boat.boat_tensor_unref(t)
+    boat.boat_conv_layer_free(layer)
+
+
+def test_flatten_layer_round_trip(boat, rng):
+    x = rng.standard_normal((3, 2, 4, 5)).astype(np.float32)
+    layer = boat.boat_flatten_layer_create()
+    tx = boat.tensor(x)
+    ty = boat.boat_flatten_layer_forward(layer, tx)
+    assert boat.shape(ty) == (3, 40) and np.array_equal(boat.numpy(ty), x.reshape(3, 40))
+    tb = boat.boat_flatten_layer_backward(layer, ty)
+    assert boat.shape(tb) == x.shape and np.array_equal(boat.numpy(tb), x)
+    for t in (tb, ty, tx):
+        boat.boat_tensor_unref(t)
+    boat.boat_flatten_layer_free(layer)
+
+
+@pytest.mark.parametrize("size", ["small", "mnist"])
+def test_cnn_chain_on_the_tape(boat, oracle, size):
+    """conv-relu-pool x2, flatten, dense-relu-dense, cross-entropy chain (examples/mnist/mnist_autodiff.c:536-557)
+    against the oracle: the reference's mirrored-tap input gradient with the switch on, the true gradient without."""
+    from test_oracle_vs_reference import CNN_KEYS, cnn_params, oracle_cnn_grads
+    rng = np.random.default_rng(2718)
+    if size == "small":
+        B, ic, c1, c2, side, hidden, classes = 3, 2, 4, 6, 8, 12, 5
+    else:
+        B, ic, c1, c2, side, hidden, classes = 8, 1, 32, 64, 28, 128, 10
+    x = rng.random((B, ic, side, side), dtype=np.float32)
+    labels = rng.integers(0, classes, B)
+    p = cnn_params(rng, ic, c1, c2, side, hidden, classes)
+    if size == "mnist":
+        for k in ("cw2", "w1", "w2"):
+            p[k] = (p[k] * 0.2).astype(np.float32)
+    for flip in (True, False):
+        boat.boat_hip_conv_reference_input_grad(int(flip))
+        try:
+            got = bc.cnn_ce_grads(boat, x, labels, p)
+        finally:
+            boat.boat_hip_conv_reference_input_grad(0)
+        want = oracle_cnn_grads(oracle, x, labels, p, flip_taps=flip)
+        assert abs(got["loss"] - want["loss"]) <= TOL_RED * abs(want["loss"])
+        for key in CNN_KEYS:
+            assert rel_fro(got[key], want[key]) <= TOL_GEMM, (key, flip)
+            assert np.max(np.abs(got[key] - want[key])) <= 10 * TOL_RED * np.abs(want[key]).max(), (key, flip)
+
+
+def test_cnn_training_with_registered_optimizer(boat):
+    """Adam registered once with the layers' gradient tensors; three steps reduce the loss (the reference replaces the
+    conv gradient tensors on every backward, conv.c:523-532, and would update from stale ones)."""
+    rng = np.random.default_rng(99)
+    B = 8
+    x = rng.random((B, 1, 12, 12), dtype=np.float32)
+    labels = rng.integers(0, 4, B)
+    onehot = np.zeros((B, 4), np.float32)
+    onehot[np.arange(B), labels] = 1
+    conv = boat.boat_conv_layer_create(1, 4, 3, 1, 1)
+    pool = boat.boat_pool_layer_create(2, 2, 0)
+    dense = boat.boat_dense_layer_create(4 * 6 * 6, 4, True)
+    opt = boat.boat_adam_optimizer_create(1e-2, 0.9, 0.999, 1e-8)
+    boat.boat_hip_optimizer_add_conv(opt, conv)
+    boat.boat_hip_optimizer_add_dense(opt, dense)
+    losses = []
+    for _ in range(4):
+        vx = boat.boat_variable_create(tx := boat.tensor(x), True)
+        a = boat.boat_var_conv(vx, conv)
+        r = boat.boat_var_relu(a)
+        q = boat.boat_var_pool(r, pool)
+        f = boat.boat_var_flatten(q)
+        z = boat.boat_var_dense(f, dense)
+        ls = boat.boat_var_log_softmax(z, 1)
+        voh = boat.boat_variable_create(toh := boat.tensor(onehot), False)
+        m = boat.boat_var_mul(voh, ls)
+        s = boat.boat_var_sum(m, None, 0, False)
+        vf = boat.boat_variable_create(tf := boat.tensor(np.array([-1.0 / B], np.float32)), False)
+        loss = boat.boat_var_mul(vf, s)
+        losses.append(float(boat.numpy(boat.boat_variable_data(loss))[0]))
+        boat.boat_optimizer_zero_grad(opt)
+        with bc.scratch_cwd():
+            boat.boat_variable_backward_full(loss)
+        boat.boat_optimizer_step(opt)
+        for v in (loss, vf, s, m, voh, ls, z, f, q, r, a, vx):
+            boat.boat_variable_free(v)
+        for t in (tx, toh, tf):
+            boat.boat_tensor_unref(t)
+    assert losses[-1] < losses[0], losses
+    boat.boat_optimizer_free(opt)
+    boat.boat_conv_layer_free(conv)
+    boat.boat_pool_layer_free(pool)
+    boat.boat_dense_layer_free(dense)

@@ -429,3 +429,67 @@ def test_sdpa_attention_matrix_output(hip, oracle, rng):
     _, _, wattn = oracle.sdpa_forward(q, k, v, 0.35)
     assert np.max(np.abs(attn.numpy() - wattn)) <= 1e-6
     assert np.allclose(attn.numpy().sum(-1), 1.0, atol=1e-5)
+
+
+# ------------------------------------------------------------------ convolution / max pooling
+
+CONV_SHAPES = [  # batch, ic, h, w, oc, k, stride, pad
+    (2, 3, 7, 6, 4, 3, 1, 1), (3, 1, 8, 8, 5, 3, 1, 0), (2, 2, 9, 7, 3, 2, 2, 1), (1, 4, 5, 5, 2, 5, 1, 2),
+    (2, 3, 10, 10, 2, 3, 3, 0), (1, 1, 1, 1, 1, 1, 1, 0),
+    (16, 1, 28, 28, 32, 3, 1, 1), (8, 32, 14, 14, 64, 3, 1, 1),      # the two layers of the MNIST network
+]
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_conv2d_forward_backward(hip, oracle, rng, shape):
+    B, ic, h, w, oc, k, stride, pad = shape
+    ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    x = rng.standard_normal((B, ic, h, w)).astype(np.float32)
+    wt = (0.3 * rng.standard_normal((oc, ic, k, k))).astype(np.float32)
+    b = rng.standard_normal(oc).astype(np.float32)
+    dy = rng.standard_normal((B, oc, ho, wo)).astype(np.float32)
+    dx_, dw_, db_, ddy = dev(hip, x), dev(hip, wt), dev(hip, b), dev(hip, dy)
+    y = hip.empty((B, oc, ho, wo))
+    hip.check(hip.bh_conv2d_forward(dx_.ptr, dw_.ptr, db_.ptr, y.ptr, B, ic, h, w, oc, k, stride, pad))
+    assert np.array_equal(y.numpy(), oracle.conv2d_forward(x, wt, b, stride, pad))       # same operation order: bit exact
+    hip.check(hip.bh_conv2d_forward(dx_.ptr, dw_.ptr, None, y.ptr, B, ic, h, w, oc, k, stride, pad))
+    assert np.array_equal(y.numpy(), oracle.conv2d_forward(x, wt, None, stride, pad))
+    for flip in (0, 1):
+        gx, gw, gb = hip.empty(x.shape), hip.empty(wt.shape), hip.empty(oc)
+        hip.check(hip.bh_conv2d_backward(dx_.ptr, dw_.ptr, ddy.ptr, gx.ptr, gw.ptr, gb.ptr, B, ic, h, w, oc, k, stride, pad, 0, flip))
+        o_dx, o_gw, o_gb = oracle.conv2d_backward(x, wt, dy, stride, pad, flip_taps=bool(flip))
+        for got, want in ((gx, o_dx), (gw, o_gw), (gb, o_gb)):
+            assert np.max(np.abs(got.numpy() - want)) <= TOL_RED * np.abs(want).max(), flip
+    # accumulate: a second call adds to the parameter gradients and leaves dx assigned
+    first_gw, first_gb = gw.numpy(), gb.numpy()
+    hip.check(hip.bh_conv2d_backward(dx_.ptr, dw_.ptr, ddy.ptr, None, gw.ptr, gb.ptr, B, ic, h, w, oc, k, stride, pad, 1, 0))
+    assert np.array_equal(gw.numpy(), 2 * first_gw) and np.array_equal(gb.numpy(), 2 * first_gb)     # g + g is exact
+
+
+def test_conv2d_refuses_bad_shapes(hip):
+    p = hip.empty(16)
+    assert hip.bh_conv2d_forward(p.ptr, p.ptr, None, p.ptr, 1, 1, 2, 2, 1, 3, 1, 0) == -1       # kernel larger than image
+    assert hip.bh_conv2d_forward(p.ptr, p.ptr, None, p.ptr, 1, 1, 2, 2, 1, 1, 0, 0) == -1       # stride 0
+    assert hip.bh_conv2d_forward(None, p.ptr, None, p.ptr, 1, 1, 2, 2, 1, 1, 1, 0) == -1
+    assert hip.bh_conv2d_forward(None, None, None, None, 0, 1, 2, 2, 1, 1, 1, 0) == 0           # empty batch: nothing to do
+    assert hip.bh_maxpool2d_forward(p.ptr, p.ptr, p.ptr, 1, 2, 2, 3, 1, 0) == -1
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 8, 8, 2, 2, 0), (1, 2, 7, 9, 3, 2, 1), (2, 1, 6, 6, 3, 1, 0), (1, 2, 5, 5, 2, 2, 1),
+                                   (16, 32, 28, 28, 2, 2, 0)], ids=lambda s: "x".join(map(str, s)))
+def test_maxpool2d_forward_backward(hip, oracle, rng, shape):
+    B, ch, h, w, pool, stride, pad = shape
+    ho, wo = (h + 2 * pad - pool) // stride + 1, (w + 2 * pad - pool) // stride + 1
+    x = rng.standard_normal((B, ch, h, w)).astype(np.float32)
+    x[0, 0, :2, :2] = 1.5                                    # ties: first maximum in scan order
+    x = np.maximum(x, 0) if B > 2 else x                     # post-ReLU input has many tied zeros
+    dy = rng.standard_normal((B, ch, ho, wo)).astype(np.float32)
+    dx_, ddy = dev(hip, x), dev(hip, dy)
+    y, arg, gx = hip.empty((B, ch, ho, wo)), hip.empty((B, ch, ho, wo), np.int32), hip.empty(x.shape)
+    hip.check(hip.bh_maxpool2d_forward(dx_.ptr, y.ptr, arg.ptr, B * ch, h, w, pool, stride, pad))
+    hip.check(hip.bh_maxpool2d_backward(ddy.ptr, arg.ptr, gx.ptr, B * ch, h, w, pool, stride, pad))
+    o_y, o_arg = oracle.maxpool2d_forward(x, pool, stride, pad)
+    assert np.array_equal(y.numpy(), o_y)
+    plane = (np.arange(B * ch) * h * w).reshape(B, ch, 1, 1)
+    assert np.array_equal(arg.numpy().astype(np.int64) + plane, o_arg)
+    assert np.array_equal(gx.numpy(), oracle.maxpool2d_backward(dy, o_arg, x.shape))

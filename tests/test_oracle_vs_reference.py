@@ -335,3 +335,177 @@ def test_fanout_divergence_is_documented(ref):
     a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
     da, db = bc.fanout(ref, a, b)
     assert np.array_equal(da, 4 * b) and np.array_equal(db, 4 * a)
+
+
+# ---- convolution / max pooling / the MNIST CNN chain (src/layers/conv.c, pool.c, flatten.c) ----
+
+def test_known_answer_conv_forward(ref, oracle):
+    # tests/test_conv_forward.c:20-91: 3x3 ramp image, 2x2 kernel [[1,0],[0,1]], zero bias -> [6, 8, 12, 14]
+    x = np.arange(1, 10, dtype=np.float32).reshape(1, 1, 3, 3)
+    w = np.array([1, 0, 0, 1], np.float32).reshape(1, 1, 2, 2)
+    b = np.zeros(1, np.float32)
+    y, _ = bc.conv_layer(ref, x, w, b, 1, 0, [])
+    assert y.reshape(-1).tolist() == [6, 8, 12, 14]
+    assert same(oracle.conv2d_forward(x, w, b, 1, 0), y)
+    # :93-165: padding 1 gives 4x4, stride 2 gives 1x1
+    assert bc.conv_layer(ref, x, w, b, 1, 1, [])[0].shape == (1, 1, 4, 4)
+    assert bc.conv_layer(ref, x, w, b, 2, 0, [])[0].shape == (1, 1, 1, 1)
+    assert oracle.conv2d_forward(x, w, b, 1, 1).shape == (1, 1, 4, 4)
+    assert oracle.conv2d_forward(x, w, b, 2, 0).shape == (1, 1, 1, 1)
+
+
+CONV_CASES = [  # B, ic, h, w, oc, k, stride, pad
+    (2, 3, 7, 6, 4, 3, 1, 1),
+    (3, 1, 8, 8, 5, 3, 1, 0),
+    (2, 2, 9, 7, 3, 2, 2, 1),
+    (1, 4, 5, 5, 2, 5, 1, 2),
+    (2, 3, 10, 10, 2, 3, 3, 0),
+]
+
+
+def conv_inputs(case, seed):
+    B, ic, h, w, oc, k, stride, pad = case
+    rng = np.random.default_rng(seed)
+    ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    return dict(x=rng.standard_normal((B, ic, h, w)).astype(np.float32),
+                w=(0.3 * rng.standard_normal((oc, ic, k, k))).astype(np.float32),
+                b=rng.standard_normal(oc).astype(np.float32),
+                dy1=rng.standard_normal((B, oc, ho, wo)).astype(np.float32),
+                dy2=rng.standard_normal((B, oc, ho, wo)).astype(np.float32))
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_conv_layer_bit_exact(ref, oracle, case):
+    stride, pad = case[6], case[7]
+    d = conv_inputs(case, 77)
+    y, calls = bc.conv_layer(ref, d["x"], d["w"], d["b"], stride, pad, [d["dy1"], d["dy2"]])
+    assert same(oracle.conv2d_forward(d["x"], d["w"], d["b"], stride, pad), y)
+    for dy, (dx, gw, gb) in zip((d["dy1"], d["dy2"]), calls):
+        o_dx, o_gw, o_gb = oracle.conv2d_backward(d["x"], d["w"], dy, stride, pad, flip_taps=True)
+        assert same(o_dx, dx) and same(o_gw, gw) and same(o_gb, gb)
+    # parameter gradients are overwritten, not accumulated, by the second call (conv.c:523-532)
+    assert not np.array_equal(calls[0][1], calls[1][1])
+
+
+def conv_f64(x, w, b, stride, pad):
+    """Textbook cross-correlation in float64 from numpy slices (independent of the oracle's loops)."""
+    x, w = x.astype(np.float64), w.astype(np.float64)
+    B, ic, h, wd = x.shape
+    oc, _, k, _ = w.shape
+    ho, wo = (h + 2 * pad - k) // stride + 1, (wd + 2 * pad - k) // stride + 1
+    xp = np.zeros((B, ic, h + 2 * pad, wd + 2 * pad))
+    xp[:, :, pad:pad + h, pad:pad + wd] = x
+    y = np.zeros((B, oc, ho, wo))
+    for kh in range(k):
+        for kw in range(k):
+            patch = xp[:, :, kh:kh + stride * ho:stride, kw:kw + stride * wo:stride]
+            y += np.einsum("bchw,oc->bohw", patch, w[:, :, kh, kw])
+    return y + (0 if b is None else b.astype(np.float64)[None, :, None, None])
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_conv_true_gradients_float64(oracle, case):
+    """flip_taps=False is the gradient of the forward: adjoint identities against an independent float64 forward.
+    <conv(u; w), dy> = <u, dx(dy)> for any u, and <conv(x; q), dy> = <q, gw(dy)> for any q (conv is bilinear)."""
+    stride, pad = case[6], case[7]
+    d = conv_inputs(case, 78)
+    dx, gw, gb = oracle.conv2d_backward(d["x"], d["w"], d["dy1"], stride, pad, flip_taps=False)
+    rng = np.random.default_rng(5)
+    dy = d["dy1"].astype(np.float64)
+    assert np.allclose(oracle.conv2d_forward(d["x"], d["w"], d["b"], stride, pad), conv_f64(d["x"], d["w"], d["b"], stride, pad),
+                       rtol=1e-5, atol=1e-5)
+    for _ in range(3):
+        u = rng.standard_normal(d["x"].shape)
+        q = rng.standard_normal(d["w"].shape)
+        lhs_x = np.sum(conv_f64(u, d["w"], None, stride, pad) * dy)
+        lhs_w = np.sum(conv_f64(d["x"], q, None, stride, pad) * dy)
+        assert abs(lhs_x - np.sum(u * dx)) <= 1e-4 * (abs(lhs_x) + 1)
+        assert abs(lhs_w - np.sum(q * gw)) <= 1e-4 * (abs(lhs_w) + 1)
+    assert np.allclose(gb, dy.sum((0, 2, 3)), rtol=1e-5, atol=1e-5)
+    # unit probes: dx at one input element equals the directional derivative along that element
+    u = np.zeros(d["x"].shape)
+    u[0, 0, 1, 2] = 1.0
+    assert abs(np.sum(conv_f64(u, d["w"], None, stride, pad) * dy) - dx[0, 0, 1, 2]) <= 1e-4 * (abs(dx[0, 0, 1, 2]) + 1)
+    # the reference's pairing is a different operator whenever the kernel is not symmetric under a 180 degree turn
+    dx_flip = oracle.conv2d_backward(d["x"], d["w"], d["dy1"], stride, pad, flip_taps=True)[0]
+    assert not np.allclose(dx_flip, dx, rtol=1e-3, atol=1e-3)
+    turned = np.ascontiguousarray(d["w"][:, :, ::-1, ::-1])
+    assert same(oracle.conv2d_backward(d["x"], turned, d["dy1"], stride, pad, flip_taps=False)[0], dx_flip)
+
+
+POOL_CASES = [  # B, ch, h, w, pool, stride, pad
+    (2, 3, 8, 8, 2, 2, 0),
+    (1, 2, 7, 9, 3, 2, 1),
+    (2, 1, 6, 6, 3, 1, 0),     # overlapping windows: several outputs route to one input
+    (1, 2, 5, 5, 2, 2, 1),
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_pool_layer_bit_exact(ref, oracle, case):
+    B, ch, h, w, pool, stride, pad = case
+    rng = np.random.default_rng(91)
+    x = rng.standard_normal((B, ch, h, w)).astype(np.float32)
+    x[0, 0, :2, :2] = 1.5                     # a tie: the first maximum in scan order wins
+    ho, wo = (h + 2 * pad - pool) // stride + 1, (w + 2 * pad - pool) // stride + 1
+    dy = rng.standard_normal((B, ch, ho, wo)).astype(np.float32)
+    y, dx = bc.pool_layer(ref, x, pool, stride, pad, dy)
+    o_y, arg = oracle.maxpool2d_forward(x, pool, stride, pad)
+    assert same(o_y, y)
+    assert same(oracle.maxpool2d_backward(dy, arg, x.shape), dx)
+    # invariants: outputs are maxima of their windows; the gradient is conserved
+    assert np.all(o_y.reshape(-1) == x.reshape(-1)[arg.reshape(-1)])
+    assert np.isclose(dx.sum(dtype=np.float64), dy.sum(dtype=np.float64), rtol=1e-5, atol=1e-5)
+
+
+def cnn_params(rng, ic, c1, c2, side, hidden, classes):
+    feat = c2 * (side // 4) ** 2
+    return dict(cw1=(0.3 * rng.standard_normal((c1, ic, 3, 3))).astype(np.float32), cb1=(0.1 * rng.standard_normal(c1)).astype(np.float32),
+                cw2=(0.2 * rng.standard_normal((c2, c1, 3, 3))).astype(np.float32), cb2=(0.1 * rng.standard_normal(c2)).astype(np.float32),
+                w1=(0.2 * rng.standard_normal((feat, hidden))).astype(np.float32), b1=(0.1 * rng.standard_normal(hidden)).astype(np.float32),
+                w2=(0.3 * rng.standard_normal((hidden, classes))).astype(np.float32), b2=np.zeros(classes, np.float32))
+
+
+def oracle_cnn_grads(oracle, x, labels, p, flip_taps):
+    """The chain of bc.cnn_ce_grads restated with oracle primitives."""
+    B, classes = x.shape[0], p["w2"].shape[1]
+    onehot = np.zeros((B, classes), np.float32)
+    onehot[np.arange(B), labels] = 1.0
+    a1 = oracle.conv2d_forward(x, p["cw1"], p["cb1"], 1, 1)
+    r1 = oracle.relu_forward(a1)
+    q1, i1 = oracle.maxpool2d_forward(r1, 2, 2, 0)
+    a2 = oracle.conv2d_forward(q1, p["cw2"], p["cb2"], 1, 1)
+    r2 = oracle.relu_forward(a2)
+    q2, i2 = oracle.maxpool2d_forward(r2, 2, 2, 0)
+    fl = q2.reshape(B, -1)
+    h = oracle.dense_forward(fl, p["w1"], p["b1"])
+    rh = oracle.relu_forward(h)
+    z = oracle.dense_forward(rh, p["w2"], p["b2"])
+    loss, dz = oracle.ce_chain(z, onehot)
+    drh, g_w2, g_b2 = oracle.dense_backward(rh, p["w2"], dz)
+    dh = oracle.relu_backward(h, drh)
+    dfl, g_w1, g_b1 = oracle.dense_backward(fl, p["w1"], dh)
+    dr2 = oracle.maxpool2d_backward(dfl.reshape(q2.shape), i2, r2.shape)
+    da2 = oracle.relu_backward(a2, dr2)
+    dq1, g_cw2, g_cb2 = oracle.conv2d_backward(q1, p["cw2"], da2, 1, 1, flip_taps)
+    dr1 = oracle.maxpool2d_backward(dq1, i1, r1.shape)
+    da1 = oracle.relu_backward(a1, dr1)
+    dx, g_cw1, g_cb1 = oracle.conv2d_backward(x, p["cw1"], da1, 1, 1, flip_taps)
+    return dict(loss=loss, logits=z, dx=dx, g_cw1=g_cw1, g_cb1=g_cb1, g_cw2=g_cw2, g_cb2=g_cb2,
+                g_w1=g_w1, g_b1=g_b1, g_w2=g_w2, g_b2=g_b2)
+
+
+CNN_KEYS = ("logits", "dx", "g_cw1", "g_cb1", "g_cw2", "g_cb2", "g_w1", "g_b1", "g_w2", "g_b2")
+
+
+def test_cnn_chain_bit_exact(ref, oracle):
+    """examples/mnist/mnist_autodiff.c:536-557 at a small size: conv-relu-pool x2, flatten, dense-relu-dense, CE chain."""
+    rng = np.random.default_rng(314)
+    x = rng.random((3, 2, 8, 8), dtype=np.float32)
+    labels = rng.integers(0, 5, 3)
+    p = cnn_params(rng, 2, 4, 6, 8, 12, 5)
+    got = bc.cnn_ce_grads(ref, x, labels, p)
+    want = oracle_cnn_grads(oracle, x, labels, p, flip_taps=True)
+    assert np.float32(got["loss"]) == np.float32(want["loss"])
+    for key in CNN_KEYS:
+        assert same(want[key], got[key]), key

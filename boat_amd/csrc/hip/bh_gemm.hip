@@ -29,6 +29,8 @@
 // folded by a second kernel (deterministic, no atomics).
 #include "bh_common.h"
 
+#include <stdint.h>
+
 namespace bh {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -136,10 +138,99 @@ struct Frags {
     }
 };
 
-template <typename Cfg, bool A_KC, bool B_KC>
+
+// ---- direct-to-LDS operand path (global_load_lds_dwordx4: no staging registers, no ds_write) ----
+// One instruction moves 1 KB: lane l supplies the address of its 16 bytes, and the 64 pieces land contiguously at the
+// LDS address in M0.  A k-tile (kBK = 16) of an R-row operand is R/16 such blocks:
+//   k-contiguous operand   block = 16 rows x 16 k.  Row stride is 16 floats with no room for padding, so the four
+//                          16-byte chunks of a row are swizzled instead: chunk q of row r sits in slot q ^ ((r >> 2) & 3),
+//                          which makes the fragment reads of 16 consecutive rows hit 16 different bank groups.
+//   row-contiguous operand block = 256 consecutive floats of k-rows (one k-row for R = 256, two for R = 128), blocks
+//                          padded by 4 floats so that the two half-wavefronts of a fragment read use different banks.
+// Rows or columns past the matrix edge are clamped to the last valid ones (their products are never stored); the
+// contraction range must be a multiple of kBK because nothing zero-fills a k tail.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <bool KC, int R> struct DirectTile {
+    static constexpr int blocks = R / 16;
+    static constexpr int block_stride = KC ? 256 : 260;   // floats
+    static constexpr int floats = blocks * block_stride;
+};
+
+__device__ __forceinline__ void load_block_to_lds(const float* src, unsigned lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_byte_addr) : "memory", "m0");
+}
+__device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+template <bool KC, int R, int NW>
+struct DirectLoader {
+    static constexpr int PER = DirectTile<KC, R>::blocks / NW;   // blocks per wavefront and k-tile
+    static_assert(DirectTile<KC, R>::blocks % NW == 0, "blocks must divide among the wavefronts");
+    const float* src[PER];
+    unsigned dst[PER];      // LDS byte address inside stage 0
+    int64_t step;           // floats from one k-tile to the next
+
+    __device__ __forceinline__ void init(const float* base, int64_t ld, int64_t row0, int64_t row_lim, int64_t k_begin,
+                                         const float* lds_tile, int wave, int lane) {
+        step = KC ? kBK : kBK * ld;
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int blk = wave + j * NW;
+            if (KC) {
+                int64_t row = row0 + 16 * blk + (lane >> 2);
+                if (row > row_lim - 1) row = row_lim - 1;
+                const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+                src[j] = base + row * ld + k_begin + 4 * chunk;
+            } else {
+                const int krow = R == 256 ? blk : 2 * blk + (lane >> 5);
+                int64_t col = row0 + 4 * (R == 256 ? lane : (lane & 31));
+                if (col > row_lim - 4) col = row_lim - 4;
+                src[j] = base + (k_begin + krow) * ld + col;
+            }
+            const unsigned addr = (unsigned)(uintptr_t)(lds_ptr_t)(lds_tile + blk * DirectTile<KC, R>::block_stride);
+            dst[j] = __builtin_amdgcn_readfirstlane(addr);
+        }
+    }
+    // issue this wavefront's blocks of the next k-tile into the stage at byte offset stage_bytes
+    __device__ __forceinline__ void issue(unsigned stage_bytes) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            load_block_to_lds(src[j], dst[j] + stage_bytes);
+            src[j] += step;
+        }
+    }
+};
+
+// Fragments from a direct-to-LDS tile: same register meaning as Frags.
+template <bool KC, int R, int T>
+struct DirectFrags {
+    float v[4][T];
+    __device__ __forceinline__ void load(const float* lds, int wave_off, int kb, int r, int half) {
+        if (KC) {
+            const int slot = ((kb >> 2) + half) ^ ((r >> 2) & 3);
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                float4 q = *reinterpret_cast<const float4*>(lds + (wave_off + t * 32 + r) * 16 + slot * 4);
+                v[0][t] = q.x; v[1][t] = q.y; v[2][t] = q.z; v[3][t] = q.w;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                const int kk = kb + 4 * half + s;
+                FragT<T> f;
+                f.load(lds + (R == 256 ? kk * 260 : (kk >> 1) * 260 + (kk & 1) * 128) + wave_off + T * r);
+#pragma unroll
+                for (int t = 0; t < T; t++) v[s][t] = f.v[t];
+            }
+        }
+    }
+};
+
+template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT>
 __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
-    constexpr int A_FLOATS = TileShape<A_KC, BM>::floats, B_FLOATS = TileShape<B_KC, BN>::floats;
+    constexpr int A_FLOATS = DIRECT ? DirectTile<A_KC, BM>::floats : TileShape<A_KC, BM>::floats;
+    constexpr int B_FLOATS = DIRECT ? DirectTile<B_KC, BN>::floats : TileShape<B_KC, BN>::floats;
     extern __shared__ __align__(16) float smem[];
     constexpr int STAGE = A_FLOATS + B_FLOATS;   // stage `cur` holds A at smem+cur*STAGE, B right after it
 
@@ -178,48 +269,93 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    TileLoader<A_KC, BM, NT> la;
-    TileLoader<B_KC, BN, NT> lb;
-
-    const int64_t kt_count = (k_end - k_begin + kBK - 1) / kBK;
-    if (kt_count > 0) {
-        la.load(A, g.lda, m0, g.m, k_begin, k_end, tid);
-        lb.load(B, g.ldb, n0, g.n, k_begin, k_end, tid);
-        la.store(smem, tid);
-        lb.store(smem + A_FLOATS, tid);
-    }
-    __syncthreads();
-
-    int cur = 0;
-    for (int64_t kt = 0; kt < kt_count; kt++) {
-        const bool more = kt + 1 < kt_count;
-        if (more) {
-            const int64_t k0 = k_begin + (kt + 1) * kBK;
-            la.load(A, g.lda, m0, g.m, k0, k_end, tid);
-            lb.load(B, g.ldb, n0, g.n, k0, k_end, tid);
+    if constexpr (DIRECT) {
+        // tile kt+1 streams straight into the other LDS stage while tile kt feeds the MFMAs; the wait for this
+        // wavefront's own loads and the barrier at the end of the k-tile publish it to the workgroup
+        constexpr int NW = NT / 64;
+        DirectLoader<A_KC, BM, NW> da;
+        DirectLoader<B_KC, BN, NW> db;
+        da.init(A, g.lda, m0, g.m, k_begin, smem, wave, lane);
+        db.init(B, g.ldb, n0, g.n, k_begin, smem + A_FLOATS, wave, lane);
+        const int64_t kt_count = (k_end - k_begin) / kBK;
+        if (kt_count > 0) {
+            da.issue(0);
+            db.issue(0);
         }
-        const float* sa = smem + cur * STAGE;
-        const float* sb = sa + A_FLOATS;
+        wait_direct_loads();
+        __syncthreads();
+        int cur = 0;
+        for (int64_t kt = 0; kt < kt_count; kt++) {
+            if (kt + 1 < kt_count) {
+                const unsigned stage_bytes = (unsigned)((cur ^ 1) * STAGE * sizeof(float));
+                da.issue(stage_bytes);
+                db.issue(stage_bytes);
+            }
+            const float* sa = smem + cur * STAGE;
+            const float* sb = sa + A_FLOATS;
 #pragma unroll
-        for (int kb = 0; kb < kBK; kb += 8) {
-            Frags<A_KC, BM, TM> fa;
-            Frags<B_KC, BN, TN> fb;
-            fa.load(sa, wm * Cfg::WM, kb, r, half);
-            fb.load(sb, wn * Cfg::WN, kb, r, half);
+            for (int kb = 0; kb < kBK; kb += 8) {
+                DirectFrags<A_KC, BM, TM> fa;
+                DirectFrags<B_KC, BN, TN> fb;
+                fa.load(sa, wm * Cfg::WM, kb, r, half);
+                fb.load(sb, wn * Cfg::WN, kb, r, half);
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+                for (int s = 0; s < 4; s++)
 #pragma unroll
-                for (int i = 0; i < TM; i++)
+                    for (int i = 0; i < TM; i++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < TN; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
+            }
+            wait_direct_loads();
+            __syncthreads();
+            cur ^= 1;
         }
-        if (more) {
-            la.store(smem + (cur ^ 1) * STAGE, tid);
-            lb.store(smem + (cur ^ 1) * STAGE + A_FLOATS, tid);
+    } else {
+        TileLoader<A_KC, BM, NT> la;
+        TileLoader<B_KC, BN, NT> lb;
+
+        const int64_t kt_count = (k_end - k_begin + kBK - 1) / kBK;
+        if (kt_count > 0) {
+            la.load(A, g.lda, m0, g.m, k_begin, k_end, tid);
+            lb.load(B, g.ldb, n0, g.n, k_begin, k_end, tid);
+            la.store(smem, tid);
+            lb.store(smem + A_FLOATS, tid);
         }
         __syncthreads();
-        cur ^= 1;
+
+        int cur = 0;
+        for (int64_t kt = 0; kt < kt_count; kt++) {
+            const bool more = kt + 1 < kt_count;
+            if (more) {
+                const int64_t k0 = k_begin + (kt + 1) * kBK;
+                la.load(A, g.lda, m0, g.m, k0, k_end, tid);
+                lb.load(B, g.ldb, n0, g.n, k0, k_end, tid);
+            }
+            const float* sa = smem + cur * STAGE;
+            const float* sb = sa + A_FLOATS;
+    #pragma unroll
+            for (int kb = 0; kb < kBK; kb += 8) {
+                Frags<A_KC, BM, TM> fa;
+                Frags<B_KC, BN, TN> fb;
+                fa.load(sa, wm * Cfg::WM, kb, r, half);
+                fb.load(sb, wn * Cfg::WN, kb, r, half);
+    #pragma unroll
+                for (int s = 0; s < 4; s++)
+    #pragma unroll
+                    for (int i = 0; i < TM; i++)
+    #pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
+            }
+            if (more) {
+                la.store(smem + (cur ^ 1) * STAGE, tid);
+                lb.store(smem + (cur ^ 1) * STAGE + A_FLOATS, tid);
+            }
+            __syncthreads();
+            cur ^= 1;
+        }
+
     }
 
     // ---- epilogue ----
@@ -277,6 +413,116 @@ __global__ __launch_bounds__(256) void splitk_fold_kernel(const float* __restric
         float* dst = c + bt * stride_c + row * ldc + col;
         if (bias) acc += bias[col];
         *dst = accumulate ? *dst + acc : acc;
+    }
+}
+
+// ---- small problems: one trip to memory per workgroup ----
+// A 64x64 output tile per workgroup (four wavefronts, one 32x32 accumulator each) and a k-chunk of at most kSmallK
+// that is loaded WHOLE into LDS before the first MFMA: a tiny GEMM is bound by the number of dependent round trips to
+// memory (about 2 us each), not by flops, so the chunk loop of the big kernels is replaced by one load phase, one
+// barrier and one MFMA chain; longer contractions are split over workgroups (blockIdx.z) and folded afterwards.
+// Loads are scalar and bounds-checked (any alignment, any leading dimension), walk the operand's contiguous
+// direction and are all issued before the first LDS store; both panels sit k-contiguous in LDS, rows padded by 4.
+constexpr int kSmallK = 112;   // two 64 x (112+4) panels = 58 KB of LDS
+constexpr int kSmallLd = kSmallK + 4;
+
+template <bool a_kfast, bool b_kfast>   // whether the operand's k index is the fast one in memory
+__global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
+    __shared__ __align__(16) float as[64 * kSmallLd];
+    __shared__ __align__(16) float bs[64 * kSmallLd];
+    const int tid = threadIdx.x;
+    const int tile_m = blockIdx.x % g.tiles_m, tile_n = blockIdx.x / g.tiles_m;
+    const int batch = blockIdx.y, split = blockIdx.z;
+    const int64_t k_begin = (int64_t)split * g.k_per_split;
+    int64_t k_end = k_begin + g.k_per_split;
+    if (k_end > g.k) k_end = g.k;
+    const int kc = (int)(k_end - k_begin);               // <= kSmallK
+    const int kc8 = (kc + 7) & ~7;                       // MFMA groups of 8; the tail is zero-filled
+    const float* A = g.a + (int64_t)batch * g.stride_a;
+    const float* B = g.b + (int64_t)batch * g.stride_b;
+    const int64_t m0 = (int64_t)tile_m * 64, n0 = (int64_t)tile_n * 64;
+
+    // Panel element (row, kk) of an operand whose k index is the fast one in memory sits at base[row*ld + kk], else at
+    // base[kk*ld + row].  All loads of a thread are issued before the first LDS store, so they are in flight together.
+    constexpr int PER = 64 * kSmallK / 256;
+    float va[PER], vb[PER];
+    // out-of-range elements read a clamped (valid) address and are zeroed afterwards: no divergent branches, so the
+    // loads really are issued back to back
+    const int64_t m_last = g.m - 1, n_last = g.n - 1;
+    const int k_last = kc > 0 ? kc - 1 : 0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) va[i] = vb[i] = 0.f;
+    if (kc > 0) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * 256;
+            const int row = a_kfast ? idx / kSmallK : idx & 63, kk = a_kfast ? idx % kSmallK : idx >> 6;
+            const int64_t gr = min(m0 + row, m_last), gk = k_begin + min(kk, k_last);
+            va[i] = a_kfast ? A[gr * g.lda + gk] : A[gk * g.lda + gr];
+            const int col = b_kfast ? idx / kSmallK : idx & 63, kk2 = b_kfast ? idx % kSmallK : idx >> 6;
+            const int64_t gc = min(n0 + col, n_last), gk2 = k_begin + min(kk2, k_last);
+            vb[i] = b_kfast ? B[gc * g.ldb + gk2] : B[gk2 * g.ldb + gc];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int idx = tid + i * 256;
+        const int row = a_kfast ? idx / kSmallK : idx & 63, kk = a_kfast ? idx % kSmallK : idx >> 6;
+        if (m0 + row > m_last || kk >= kc) va[i] = 0.f;
+        const int col = b_kfast ? idx / kSmallK : idx & 63, kk2 = b_kfast ? idx % kSmallK : idx >> 6;
+        if (n0 + col > n_last || kk2 >= kc) vb[i] = 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int idx = tid + i * 256;
+        const int row = a_kfast ? idx / kSmallK : idx & 63, kk = a_kfast ? idx % kSmallK : idx >> 6;
+        as[row * kSmallLd + kk] = va[i];
+        const int col = b_kfast ? idx / kSmallK : idx & 63, kk2 = b_kfast ? idx % kSmallK : idx >> 6;
+        bs[col * kSmallLd + kk2] = vb[i];
+    }
+    __syncthreads();
+
+    const int wave = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    floatx16 acc0, acc1;                                 // two chains, even and odd k-groups
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc0[e] = acc1[e] = 0.f;
+    const float* pa = as + (wm * 32 + r) * kSmallLd + 4 * half;
+    const float* pb = bs + (wn * 32 + r) * kSmallLd + 4 * half;
+    for (int kb = 0; kb < kc8; kb += 16) {
+        const float4 a0 = *reinterpret_cast<const float4*>(pa + kb);
+        const float4 b0 = *reinterpret_cast<const float4*>(pb + kb);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, b0.x, acc0, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, b0.y, acc0, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, b0.z, acc0, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, b0.w, acc0, 0, 0, 0);
+        if (kb + 8 < kc8) {
+            const float4 a1 = *reinterpret_cast<const float4*>(pa + kb + 8);
+            const float4 b1 = *reinterpret_cast<const float4*>(pb + kb + 8);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.x, b1.x, acc1, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.y, b1.y, acc1, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.z, b1.z, acc1, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.w, b1.w, acc1, 0, 0, 0);
+        }
+    }
+
+    float* C = g.c + (int64_t)batch * g.stride_c;
+    if (g.k_splits > 1) C += (int64_t)split * gridDim.y * g.stride_c;
+    const bool add_c = g.accumulate && g.k_splits <= 1;
+    const float* bias = g.k_splits <= 1 ? g.bias : nullptr;
+    const int64_t col = n0 + wn * 32 + r;
+    if (col < g.n) {
+        const float bv = bias ? bias[col] : 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int64_t row = m0 + wm * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+            if (row < g.m) {
+                float v = acc0[e] + acc1[e];
+                if (bias) v += bv;
+                float* dst = C + row * g.ldc + col;
+                *dst = add_c ? *dst + v : v;
+            }
+        }
     }
 }
 
@@ -343,31 +589,39 @@ using CfgMid = GemmCfg<128, 128, 2, 2>;   // 4 waves, 64x64 per wave
 using CfgTall = GemmCfg<256, 128, 4, 2>;  // 8 waves, 64x64 per wave
 using CfgWide = GemmCfg<128, 256, 2, 4>;  // 8 waves, 64x64 per wave
 
-template <typename Cfg, bool A_KC, bool B_KC>
+template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT>
 static int launch_mfma(const GemmArgs& g, int64_t batch) {
-    constexpr size_t lds = 2 * sizeof(float) * (TileShape<A_KC, Cfg::BM>::floats + TileShape<B_KC, Cfg::BN>::floats);
+    constexpr size_t lds = 2 * sizeof(float) *
+        (DIRECT ? DirectTile<A_KC, Cfg::BM>::floats + DirectTile<B_KC, Cfg::BN>::floats
+                : TileShape<A_KC, Cfg::BM>::floats + TileShape<B_KC, Cfg::BN>::floats);
     static bool attr_set = false;
     if (!attr_set) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC>),
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                            "hipFuncSetAttribute");
         if (rc) return rc;
         attr_set = true;
     }
     dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)(g.k_splits > 1 ? g.k_splits : 1));
-    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC>), grid, dim3(Cfg::NT), lds, stream(), g);
+    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT>), grid, dim3(Cfg::NT), lds, stream(), g);
     return BH_LAUNCH_CHECK("gemm_mfma_kernel");
 }
 
-template <typename Cfg>
-static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc) {
-    if (a_kc && b_kc) return launch_mfma<Cfg, true, true>(g, batch);
-    if (a_kc && !b_kc) return launch_mfma<Cfg, true, false>(g, batch);
-    if (!a_kc && b_kc) return launch_mfma<Cfg, false, true>(g, batch);
-    return launch_mfma<Cfg, false, false>(g, batch);
+template <typename Cfg, bool DIRECT>
+static int launch_mfma_layout2(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc) {
+    if (a_kc && b_kc) return launch_mfma<Cfg, true, true, DIRECT>(g, batch);
+    if (a_kc && !b_kc) return launch_mfma<Cfg, true, false, DIRECT>(g, batch);
+    if (!a_kc && b_kc) return launch_mfma<Cfg, false, true, DIRECT>(g, batch);
+    return launch_mfma<Cfg, false, false, DIRECT>(g, batch);
 }
 
-static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, -1 = heuristic
+template <typename Cfg>
+static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc, bool direct) {
+    return direct ? launch_mfma_layout2<Cfg, true>(g, batch, a_kc, b_kc) : launch_mfma_layout2<Cfg, false>(g, batch, a_kc, b_kc);
+}
+
+static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
+static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, -1 = heuristic
 
 }  // namespace bh
 
@@ -378,6 +632,12 @@ extern "C" {
 // test/benchmark hook: pin the kernel choice (-1 restores the heuristic)
 int bh_gemm_force_config(int cfg) {
     g_force_cfg = cfg;
+    return BH_OK;
+}
+
+// test/benchmark hook: 0 stages operand tiles through registers even where the direct-to-LDS loader applies
+int bh_gemm_force_direct(int mode) {
+    g_force_direct = mode;
     return BH_OK;
 }
 
@@ -410,16 +670,52 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
-        // measured on MI355X: the 256x256 tile wins once it fills the chip twice over with a long contraction;
-        // below that the 8-wavefront 128x256 / 256x128 tiles (same operand reuse per wavefront, twice the
-        // workgroups) beat both it and the 128x128 tile; narrow outputs keep the small tile
+        // measured on MI355X (forced-config sweep over the dense, block and attention-projection shapes, operands
+        // streamed straight to LDS): the 256x256 tile wins as soon as it fills the chip once; below that the
+        // eight-wavefront 128x256 / 256x128 tiles (same operand reuse per wavefront, twice the workgroups) beat both
+        // it and the 128x128 tile; narrow outputs keep the small tile
         const int64_t big_tiles = ceil_div(m, 256) * ceil_div(n, 256);
-        if (big_tiles >= 512 && k >= 2048) cfg = 2;
+        if (big_tiles >= 256) cfg = 2;
         else if (n >= 192 && m >= 96) cfg = 4;
         else if (m >= 192 && n >= 96) cfg = 3;
         else cfg = 1;
     }
-    if (g_force_cfg >= 0 && g_force_cfg <= 4 && (vec_ok || g_force_cfg == 0)) cfg = g_force_cfg;
+    // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
+    if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
+    if (g_force_cfg >= 0 && g_force_cfg <= 5 && (vec_ok || g_force_cfg == 0 || g_force_cfg == 5)) cfg = g_force_cfg;
+
+    if (cfg == 5) {
+        g.tiles_m = (int)ceil_div(m, 64);
+        g.tiles_n = (int)ceil_div(n, 64);
+        const int64_t splits = k > kSmallK ? ceil_div(k, kSmallK) : 1;
+        g.k_per_split = k > 0 ? ceil_div(ceil_div(k, splits), 8) * 8 : 8;
+        g.k_splits = (int)(k > 0 ? ceil_div(k, g.k_per_split) : 1);
+        BH_CHECK_ARG((int64_t)g.tiles_m * g.tiles_n <= 0x7fffffff && g.k_splits <= 65535, "problem too large for the small-GEMM kernel");
+        GemmArgs run = g;
+        float* ws = nullptr;
+        if (g.k_splits > 1) {
+            ws = (float*)bh_malloc(sizeof(float) * (size_t)(g.k_splits * batch * m * n));
+            if (!ws) return BH_ENOMEM;
+            run.c = ws;
+            run.ldc = n;
+            run.stride_c = m * n;
+        }
+        dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)g.k_splits);
+        if (a_kc && b_kc) hipLaunchKernelGGL((gemm_small_kernel<true, true>), grid, dim3(256), 0, stream(), run);
+        else if (a_kc) hipLaunchKernelGGL((gemm_small_kernel<true, false>), grid, dim3(256), 0, stream(), run);
+        else if (b_kc) hipLaunchKernelGGL((gemm_small_kernel<false, true>), grid, dim3(256), 0, stream(), run);
+        else hipLaunchKernelGGL((gemm_small_kernel<false, false>), grid, dim3(256), 0, stream(), run);
+        int rc = BH_LAUNCH_CHECK("gemm_small_kernel");
+        if (rc == BH_OK && g.k_splits > 1) {
+            int64_t blocks = ceil_div(m * n * batch, 256);
+            if (blocks > 4096) blocks = 4096;
+            hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), ws, c, bias, m, n, ldc,
+                               g.k_splits, batch, g.stride_c, accumulate);
+            rc = BH_LAUNCH_CHECK("splitk_fold_kernel");
+        }
+        if (ws) bh_free(ws);
+        return rc;
+    }
 
     if (cfg == 0) {
         if (k == 0 && !accumulate && !bias) {   // empty contraction: zeros (linear.c zero-fills its output)
@@ -459,12 +755,14 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         run.ldc = n;
         run.stride_c = m * n;
     }
+    // the direct-to-LDS loader cannot zero-fill a k tail, and its edge clamps need 4 valid floats in a row
+    const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4);
     int rc;
     switch (cfg) {
-        case 2: rc = launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc); break;
-        case 3: rc = launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc); break;
-        case 4: rc = launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc); break;
-        default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc); break;
+        case 2: rc = launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct); break;
+        case 3: rc = launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc, direct); break;
+        case 4: rc = launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc, direct); break;
+        default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc, direct); break;
     }
     if (rc == BH_OK && g.k_splits > 1) {
         int64_t blocks = ceil_div(m * n * batch, 256);

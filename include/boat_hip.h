@@ -175,8 +175,12 @@ int bh_adagrad_update_multi(float* const* p, const float* const* g, float* const
 
 /* ---- test hooks (no arithmetic of their own) ----
  * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256 MFMA tile,
- * -1 = heuristic (default).  bh_sdpa_force_general: 1 = always use the general attention kernels. */
+ * 5 = small-problem kernel (whole k-chunk in LDS, one trip to memory), -1 = heuristic (default).
+ * bh_gemm_force_direct: 0 = MFMA tiles stage their operands through registers; 1 or -1 (default) = operands go
+ * straight to LDS (global_load_lds) whenever the contraction length is a multiple of 16.
+ * bh_sdpa_force_general: 1 = always use the general attention kernels. */
 int bh_gemm_force_config(int cfg);
+int bh_gemm_force_direct(int mode);
 int bh_sdpa_force_general(int on);
 /* bh_layernorm_tune: cap on the workgroups of the LayerNorm backward (each writes one dgamma/dbeta partial);
  * 0 keeps the current value.  The second argument is reserved. */

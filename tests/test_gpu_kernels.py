@@ -310,7 +310,7 @@ def test_layernorm_backward(hip, oracle, rng, rows, hidden):
 
 # --------------------------------------------------------------------- gemm
 
-def gemm_case(hip, rng, ta, tb, m, n, k, accumulate=False, bias=False, batch=1, force=None):
+def gemm_case(hip, rng, ta, tb, m, n, k, accumulate=False, bias=False, batch=1, force=None, direct=None):
     a = rng.standard_normal((batch, k, m) if ta else (batch, m, k)).astype(np.float32)
     b = rng.standard_normal((batch, n, k) if tb else (batch, k, n)).astype(np.float32)
     c0 = rng.standard_normal((batch, m, n)).astype(np.float32)
@@ -325,11 +325,14 @@ def gemm_case(hip, rng, ta, tb, m, n, k, accumulate=False, bias=False, batch=1, 
     dc = dev(hip, c0)
     if force is not None:
         hip.bh_gemm_force_config(force)
+    if direct is not None:
+        hip.bh_gemm_force_direct(direct)
     try:
         hip.check(hip.bh_gemm(int(ta), int(tb), m, n, k, dev(hip, a).ptr, a.shape[2], dev(hip, b).ptr, b.shape[2], dc.ptr, n,
                               dev(hip, bv).ptr if bias else None, int(accumulate), batch))
     finally:
         hip.bh_gemm_force_config(-1)
+        hip.bh_gemm_force_direct(-1)
     got = dc.numpy()
     assert rel_fro(got, want) <= TOL_GEMM, (ta, tb, m, n, k, rel_fro(got, want))
     return got, want
@@ -347,7 +350,33 @@ def test_gemm_heuristic_path(hip, rng, ta, tb, m, n, k):
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 16), (256, 512, 64), (128, 128, 8), (260, 132, 36), (512, 768, 100), (1024, 1024, 256)])
 def test_gemm_mfma_tiles(hip, rng, force, ta, tb, m, n, k):
-    gemm_case(hip, rng, ta, tb, m, n, k, force=force)
+    # operands staged through registers (any contraction length) and, where k % 16 == 0, streamed straight to LDS
+    gemm_case(hip, rng, ta, tb, m, n, k, force=force, direct=0)
+    gemm_case(hip, rng, ta, tb, m, n, k, force=force, direct=1)
+
+
+@pytest.mark.parametrize("force", [1, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_direct_to_lds_edges_epilogues_and_split_k(hip, rng, force, ta, tb):
+    gemm_case(hip, rng, ta, tb, 260, 132, 48, force=force, direct=1, accumulate=True, bias=True)   # ragged edge tiles
+    gemm_case(hip, rng, ta, tb, 4, 2048, 32, force=force, direct=1)                                # a single row block
+    gemm_case(hip, rng, ta, tb, 1028, 8, 16, force=force, direct=1)                                # one k-tile
+    gemm_case(hip, rng, ta, tb, 256, 384, 2048, force=force, direct=1, accumulate=True)            # split-K
+    gemm_case(hip, rng, ta, tb, 128, 256, 64, force=force, direct=1, batch=3)
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (33, 17, 5), (64, 64, 112), (65, 63, 113), (37, 130, 225), (200, 70, 1000),
+                                   (256, 512, 64)])
+def test_gemm_small_problem_kernel(hip, rng, ta, tb, m, n, k):
+    gemm_case(hip, rng, ta, tb, m, n, k, force=5)
+    gemm_case(hip, rng, ta, tb, m, n, k, force=5, accumulate=True, bias=True)
+    gemm_case(hip, rng, ta, tb, m, n, k, force=0)                    # the bounds-checked fallback on the same shapes
+
+
+def test_gemm_small_problem_kernel_batched(hip, rng):
+    gemm_case(hip, rng, 0, 0, 5, 4, 6, batch=6, force=5)
+    gemm_case(hip, rng, 1, 1, 70, 40, 300, batch=3, force=5, accumulate=True)
 
 
 def test_gemm_epilogues_and_batch(hip, rng):

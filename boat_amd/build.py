@@ -31,7 +31,7 @@ HIP_FLAGS = [
     f"-I{ROOT / 'include'}", f"-I{CSRC / 'hip'}",
 ]
 C_FLAGS = [
-    "-O2", "-std=c11", "-fPIC", "-Wall", "-Wextra", "-fvisibility=hidden", "-D_GNU_SOURCE",
+    "-O2", "-std=c11", "-fPIC", "-ffp-contract=off", "-Wall", "-Wextra", "-fvisibility=hidden", "-D_GNU_SOURCE",
     f"-I{ROOT / 'include'}", f"-I{CSRC / 'host'}",
 ]
 

@@ -39,6 +39,8 @@ class LayerNormConfig(C.Structure):  # include/boat/layers/norm.h:21-26
                 ("elementwise_affine", C.c_bool), ("use_bias", C.c_bool)]
 
 
+LAMBDA_LR_FN = C.CFUNCTYPE(C.c_float, C.c_int, C.c_float)   # include/boat/schedulers.h:35-36
+
 _SIGS = {
     # tensor
     "boat_tensor_create": (P, [C.POINTER(C.c_int64), C.c_size_t, C.c_int, C.c_int]),
@@ -102,6 +104,13 @@ _SIGS = {
     "boat_flatten_layer_create": (P, []), "boat_flatten_layer_free": (None, [P]),
     "boat_flatten_layer_forward": (P, [P, P]), "boat_flatten_layer_backward": (P, [P, P]),
     "boat_var_conv": (P, [P, P]), "boat_var_pool": (P, [P, P]), "boat_var_flatten": (P, [P]),
+    # learning-rate schedulers
+    "boat_step_lr_scheduler_create": (P, [C.c_float, C.c_int, C.c_float]),
+    "boat_cosine_annealing_scheduler_create": (P, [C.c_float, C.c_int, C.c_float]),
+    "boat_lambda_lr_scheduler_create": (P, [C.c_float, LAMBDA_LR_FN]),
+    "boat_scheduler_step": (None, [P]), "boat_scheduler_reset": (None, [P]),
+    "boat_scheduler_get_last_lr": (C.c_float, [P]), "boat_scheduler_get_next_lr": (C.c_float, [P]),
+    "boat_scheduler_free": (None, [P]), "boat_scheduler_update_optimizer": (None, [P, P]),
     # relu / softmax hooks
     "boat_relu_layer_create": (P, []), "boat_relu_layer_free": (None, [P]),
     "boat_relu_layer_forward": (P, [P, P]), "boat_relu_layer_backward": (P, [P, P]),

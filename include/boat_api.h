@@ -308,6 +308,19 @@ BOAT_API void boat_optimizer_add_parameter(boat_optimizer_t* optimizer, boat_ten
 BOAT_API float boat_optimizer_get_learning_rate(const boat_optimizer_t* optimizer);
 BOAT_API void boat_optimizer_set_learning_rate(boat_optimizer_t* optimizer, float learning_rate);
 
+/* ---- include/boat/schedulers.h:15-52 (learning-rate schedulers; host arithmetic, one float per step) ---- */
+typedef enum { BOAT_SCHEDULER_STEP_LR, BOAT_SCHEDULER_COSINE_ANNEALING, BOAT_SCHEDULER_LAMBDA_LR } boat_scheduler_type_t;
+typedef struct boat_scheduler_t boat_scheduler_t;
+BOAT_API boat_scheduler_t* boat_step_lr_scheduler_create(float base_learning_rate, int step_size, float gamma);
+BOAT_API boat_scheduler_t* boat_cosine_annealing_scheduler_create(float base_learning_rate, int T_max, float eta_min);
+BOAT_API boat_scheduler_t* boat_lambda_lr_scheduler_create(float base_learning_rate, float (*lambda_fn)(int step, float base_lr));
+BOAT_API void boat_scheduler_step(boat_scheduler_t* scheduler);
+BOAT_API void boat_scheduler_reset(boat_scheduler_t* scheduler);
+BOAT_API float boat_scheduler_get_last_lr(const boat_scheduler_t* scheduler);
+BOAT_API float boat_scheduler_get_next_lr(const boat_scheduler_t* scheduler);
+BOAT_API void boat_scheduler_free(boat_scheduler_t* scheduler);
+BOAT_API void boat_scheduler_update_optimizer(const boat_scheduler_t* scheduler, boat_optimizer_t* optimizer);
+
 /* ---- include/boat/model.h:17-65 ---- */
 typedef struct boat_model_t boat_model_t;
 typedef struct boat_layer_ops_t boat_layer_ops_t;

@@ -496,3 +496,29 @@ def cnn_ce_grads(api, x, labels, p, pool=2):
         api.boat_dense_layer_free(d1)
         api.boat_dense_layer_free(d2)
     return rec
+
+
+def scheduler_trajectory(api, kind, base_lr, steps, **kw):
+    """Learning rates of a scheduler over `steps` calls of boat_scheduler_step: per step (next_lr before the call,
+    last_lr after it), then the pair after boat_scheduler_reset.  kind: "step" (step_size, gamma), "cosine" (T_max,
+    eta_min) or "lambda" (fn(step, base_lr) -> float)."""
+    from boat_amd.capi import LAMBDA_LR_FN
+    keep = None
+    if kind == "step":
+        s = api.boat_step_lr_scheduler_create(base_lr, kw["step_size"], kw["gamma"])
+    elif kind == "cosine":
+        s = api.boat_cosine_annealing_scheduler_create(base_lr, kw["T_max"], kw["eta_min"])
+    else:
+        keep = LAMBDA_LR_FN(kw["fn"])
+        s = api.boat_lambda_lr_scheduler_create(base_lr, keep)
+    if not s:
+        return None
+    out = [(np.float32(api.boat_scheduler_get_next_lr(s)), np.float32(api.boat_scheduler_get_last_lr(s)))]
+    for _ in range(steps):
+        nxt = api.boat_scheduler_get_next_lr(s)
+        api.boat_scheduler_step(s)
+        out.append((np.float32(nxt), np.float32(api.boat_scheduler_get_last_lr(s))))
+    api.boat_scheduler_reset(s)
+    out.append((np.float32(api.boat_scheduler_get_next_lr(s)), np.float32(api.boat_scheduler_get_last_lr(s))))
+    api.boat_scheduler_free(s)
+    return np.array(out, np.float32)

@@ -115,7 +115,7 @@ def bench_dense_backward(hip, steps, warmup):
         "ms_per_step": ms_per_step,
         "wall_ms_per_step": wall_ms,
         "roofline": {
-            "bound": "mfma", "kernel": "gemm_mfma_kernel (fp32 v_mfma_f32_32x32x2_f32, 256x256 tile)",
+            "bound": "mfma", "kernel": "gemm_mfma_kernel (fp32 v_mfma_f32_32x32x2_f32, 256x256 tile, operands direct to LDS)",
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(gemm_launch_ms, 4), "flops_per_launch": flops_per_launch,
@@ -207,52 +207,19 @@ def bench_sdpa(hip, steps, warmup):
 
 
 def bench_mlp_step(steps, warmup):
-    """Config 1 through Boat's C API: forward + boat_variable_backward_full + boat_optimizer_step, wall ms."""
-    from boat_amd.capi import default_api
-    api = default_api()
-    rng = np.random.default_rng(20250101)
-    B, d_in, d_h, d_out = 64, 784, 128, 10
-    x = rng.random((B, d_in), dtype=np.float32)
-    labels = rng.integers(0, d_out, B)
-    onehot = np.zeros((B, d_out), np.float32)
-    onehot[np.arange(B), labels] = 1
-    l1 = api.boat_dense_layer_create(d_in, d_h, True)
-    l2 = api.boat_dense_layer_create(d_h, d_out, True)
-    for layer, (fi, fo) in ((l1, (d_in, d_h)), (l2, (d_h, d_out))):
-        lim = np.sqrt(6.0 / (fi + fo))
-        api.write(api.boat_dense_layer_get_weight(layer), rng.uniform(-lim, lim, (fi, fo)).astype(np.float32))
-    opt = api.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
-    api.boat_hip_optimizer_add_dense(opt, l1)
-    api.boat_hip_optimizer_add_dense(opt, l2)
-    tx, toh = api.tensor(x), api.tensor(onehot)
-    tf = api.tensor(np.array([-1.0 / B], np.float32))
-
-    def step():
-        vx = api.boat_variable_create(tx, True)
-        voh = api.boat_variable_create(toh, False)
-        vf = api.boat_variable_create(tf, False)
-        h = api.boat_var_dense(vx, l1)
-        r = api.boat_var_relu(h)
-        z = api.boat_var_dense(r, l2)
-        ls = api.boat_var_log_softmax(z, 1)
-        mm = api.boat_var_mul(voh, ls)
-        s = api.boat_var_sum(mm, None, 0, False)
-        loss = api.boat_var_mul(vf, s)
-        api.boat_variable_backward_full(loss)
-        api.boat_optimizer_step(opt)
-        api.boat_optimizer_zero_grad(opt)
-        for var in (loss, s, mm, ls, z, r, h, vf, voh, vx):
-            api.boat_variable_free(var)
-
-    for _ in range(warmup):
-        step()
-    api.sync()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    api.sync()
-    return {"ms": round((time.perf_counter() - t0) * 1e3 / steps, 4), "bound": "launch latency",
-            "note": "MLP 784-128-10 B64 fwd+bwd+Adam through boat_var_* / boat_variable_backward_full / boat_optimizer_step, wall clock"}
+    """Config 1 through Boat's C API from a C program (boat_amd/examples/mlp_train_step.c, built beside the library):
+    forward + boat_variable_backward_full + boat_optimizer_step + zero_grad per step, wall ms measured inside it."""
+    import subprocess
+    exe = ROOT / "boat_amd" / "lib" / "mlp_train_step"
+    if not exe.exists():
+        raise FileNotFoundError(f"{exe} not found: build it first (python -m boat_amd.build)")
+    out = subprocess.run([str(exe), str(steps), str(warmup)], check=True, capture_output=True, text=True).stdout
+    rec = json.loads(out.strip().splitlines()[-1])
+    assert rec["loss_last"] < rec["loss_first"], f"MLP training does not reduce the loss: {rec}"
+    return {"ms": round(rec["ms_per_step"], 4), "bound": "launch latency", "steps": rec["steps"],
+            "loss_first_last": [rec["loss_first"], rec["loss_last"]],
+            "note": "MLP 784-128-10 B64 fwd+bwd+Adam+zero_grad through boat_var_* / boat_variable_backward_full / "
+                    "boat_optimizer_step, a C caller linked against libboat_amd.so, wall clock"}
 
 
 def bench_block_step(steps, warmup):
@@ -411,7 +378,7 @@ def main():
     if "sdpa" in legs:
         extra.update(bench_sdpa(hip, args.steps, args.warmup))
     if "mlp" in legs:
-        extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20), args.warmup)
+        extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20) * 25, max(args.warmup, 1) * 10)
     if "block" in legs:
         extra["transformer_block_step"] = bench_block_step(max(2, min(args.steps, 10)), min(args.warmup, 2))
     if extra:

@@ -21,6 +21,7 @@ HIPCC = str(ROCM / "bin" / "hipcc")
 
 HIP_SOURCES = sorted((CSRC / "hip").glob("*.hip"))
 C_SOURCES = sorted((CSRC / "host").glob("*.c"))
+EXAMPLES = sorted((ROOT / "boat_amd" / "examples").glob("*.c"))   # C programs against include/boat_api.h
 
 # -ffp-contract=off: a*b+c stays two roundings, like the reference's scalar C loops.
 # packed-fp32 ops are switched off for every device compile.
@@ -66,8 +67,12 @@ def build_all(jobs: int = 8, verbose: bool = True) -> Path:
         c_objs = list(pool.map(_compile_c, C_SOURCES))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB),
           *map(str, hip_objs), *map(str, c_objs), "-lm", f"-Wl,-rpath,{ROCM / 'lib'}"])
+    for src in EXAMPLES:   # linked against the library exactly as a Boat program would be re-linked
+        _run(["gcc", "-O2", "-std=c11", "-D_GNU_SOURCE", f"-I{ROOT / 'include'}", str(src), "-o", str(LIB.parent / src.stem),
+              f"-L{LIB.parent}", "-lboat_amd", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath-link,{ROCM / 'lib'}", "-lm"])
     if verbose:
-        print(f"built {LIB} ({LIB.stat().st_size // 1024} KiB) from {len(hip_objs)} HIP + {len(c_objs)} C sources")
+        print(f"built {LIB} ({LIB.stat().st_size // 1024} KiB) from {len(hip_objs)} HIP + {len(c_objs)} C sources, "
+              f"{len(EXAMPLES)} example program(s)")
     return LIB
 
 

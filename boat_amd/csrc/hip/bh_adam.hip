@@ -213,6 +213,33 @@ static AdamScalars make_scalars(float lr, float beta1, float beta2, float eps, i
     return s;
 }
 
+// zero up to kAdamMaxTensors tensors in one launch (gradient buffers before the next backward)
+struct ZeroTable {
+    float* p[kAdamMaxTensors];
+    int64_t n[kAdamMaxTensors];
+    int first_block[kAdamMaxTensors + 1];
+    int count;
+};
+
+__global__ __launch_bounds__(kAdamBlock) void zero_multi_kernel(ZeroTable t) {
+    int lo = 0, hi = t.count;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if ((int)blockIdx.x >= t.first_block[mid]) lo = mid; else hi = mid;
+    }
+    const int64_t idx = (int64_t)((int)blockIdx.x - t.first_block[lo]) * kAdamBlock + threadIdx.x;
+    float* p = t.p[lo];
+    const int64_t n = t.n[lo];
+    if ((reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+        const int64_t i = idx * 4;
+        if (i + 3 < n) *reinterpret_cast<float4*>(p + i) = make_float4(0.f, 0.f, 0.f, 0.f);
+        else for (int64_t j = i; j < n; j++) p[j] = 0.f;
+    } else {
+        const int64_t stride = (int64_t)(t.first_block[lo + 1] - t.first_block[lo]) * kAdamBlock;
+        for (int64_t i = idx; i < n; i += stride) p[i] = 0.f;
+    }
+}
+
 // workgroups that cover n elements with one float4 group per lane
 static int64_t blocks_for(int64_t n) {
     int64_t b = ceil_div(ceil_div(n, 4), kAdamBlock);
@@ -273,6 +300,35 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
         t.first_block[t.count] = (int)blocks;
         hipLaunchKernelGGL(adam_multi_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), t, s);
         int rc = BH_LAUNCH_CHECK("bh_adam_update_multi");
+        if (rc) return rc;
+    }
+    return BH_OK;
+}
+
+int bh_zero_multi(float* const* p, const int64_t* n, int count) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(count >= 0 && (count == 0 || (p && n)), "bad table");
+    int done = 0;
+    while (done < count) {
+        ZeroTable t;
+        t.count = 0;
+        int64_t blocks = 0;
+        while (done < count && t.count < kAdamMaxTensors) {
+            const int i = done++;
+            BH_CHECK_ARG(n[i] >= 0, "negative element count");
+            if (n[i] == 0) continue;
+            BH_CHECK_ARG(p[i], "null tensor pointer");
+            const int k = t.count++;
+            t.p[k] = p[i];
+            t.n[k] = n[i];
+            t.first_block[k] = (int)blocks;
+            blocks += blocks_for(n[i]);
+            BH_CHECK_ARG(blocks <= 0x7fffffff, "tensors too large for one launch");
+        }
+        if (t.count == 0) continue;
+        t.first_block[t.count] = (int)blocks;
+        hipLaunchKernelGGL(zero_multi_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), t);
+        int rc = BH_LAUNCH_CHECK("bh_zero_multi");
         if (rc) return rc;
     }
     return BH_OK;

@@ -88,6 +88,10 @@ static int launch_ew(const char* name, F f, float* out, const float* in0, const 
 
 // ---- functors (a, b, c = inputs; o = previous output) ----
 struct FFill { float v; __device__ float operator()(float, float, float, float) const { return v; } };
+// the scalar lives in device memory (a [1] gradient tensor): no readback to the host
+struct FFillAt { const float* s; __device__ float operator()(float, float, float, float) const { return s[0]; } };
+struct FMulAt { const float* s; __device__ float operator()(float a, float, float, float) const { return a * s[0]; } };
+struct FCopy { __device__ float operator()(float a, float, float, float) const { return a; } };
 struct FAddInto { __device__ float operator()(float a, float, float, float o) const { return o + a; } };
 struct FAdd { __device__ float operator()(float a, float b, float, float) const { return a + b; } };
 struct FSub { __device__ float operator()(float a, float b, float, float) const { return a - b; } };
@@ -267,6 +271,19 @@ int bh_binary_broadcast(int op, const float* a, const int64_t* a_shape, const fl
         default: return set_error(BH_EINVAL, "bh_binary_broadcast: unknown op %d", op);
     }
     return BH_LAUNCH_CHECK("bh_binary_broadcast");
+}
+
+int bh_scale_by_device_scalar(const float* in, const float* scalar, float* out, int64_t n) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(n >= 0 && ((scalar && out) || n == 0), "bad argument");
+    if (!in) return launch_ew<0, false>("bh_scale_by_device_scalar", FFillAt{scalar}, out, nullptr, nullptr, nullptr, n);
+    return launch_ew<1, false>("bh_scale_by_device_scalar", FMulAt{scalar}, out, in, nullptr, nullptr, n);
+}
+
+int bh_copy_f32(float* dst, const float* src, int64_t n) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(n >= 0 && ((dst && src) || n == 0), "bad argument");
+    return launch_ew<1, false>("bh_copy_f32", FCopy{}, dst, src, nullptr, nullptr, n);
 }
 
 int bh_scalar_op(int op, const float* a, float s, float* out, int64_t n) {

@@ -158,7 +158,9 @@ template <bool KC, int R> struct DirectTile {
 };
 
 __device__ __forceinline__ void load_block_to_lds(const float* src, unsigned lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_byte_addr) : "memory", "m0");
+    // M0 carries the LDS address of the block.  It is a reserved register that the compiler neither allocates nor keeps
+    // live in these kernels (no s_movrel / s_sendmsg / GWS), so nothing of its own is disturbed.
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_byte_addr) : "memory");
 }
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -423,13 +425,14 @@ __global__ __launch_bounds__(256) void splitk_fold_kernel(const float* __restric
 // barrier and one MFMA chain; longer contractions are split over workgroups (blockIdx.z) and folded afterwards.
 // Loads are scalar and bounds-checked (any alignment, any leading dimension), walk the operand's contiguous
 // direction and are all issued before the first LDS store; both panels sit k-contiguous in LDS, rows padded by 4.
-constexpr int kSmallK = 112;   // two 64 x (112+4) panels = 58 KB of LDS
+constexpr int kSmallK = 128;   // two 64 x (128+4) panels = 66 KB of dynamic LDS
 constexpr int kSmallLd = kSmallK + 4;
 
-template <bool a_kfast, bool b_kfast>   // whether the operand's k index is the fast one in memory
+template <bool a_kfast, bool b_kfast, int KCH>   // operand's k index is the fast one in memory; panel width (>= the k-chunk)
 __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
-    __shared__ __align__(16) float as[64 * kSmallLd];
-    __shared__ __align__(16) float bs[64 * kSmallLd];
+    extern __shared__ __align__(16) float smem[];
+    float* as = smem;
+    float* bs = smem + 64 * kSmallLd;
     const int tid = threadIdx.x;
     const int tile_m = blockIdx.x % g.tiles_m, tile_n = blockIdx.x / g.tiles_m;
     const int batch = blockIdx.y, split = blockIdx.z;
@@ -444,7 +447,7 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
 
     // Panel element (row, kk) of an operand whose k index is the fast one in memory sits at base[row*ld + kk], else at
     // base[kk*ld + row].  All loads of a thread are issued before the first LDS store, so they are in flight together.
-    constexpr int PER = 64 * kSmallK / 256;
+    constexpr int PER = 64 * KCH / 256;     // loads per lane and operand: a narrow chunk pays for a narrow panel only
     float va[PER], vb[PER];
     // out-of-range elements read a clamped (valid) address and are zeroed afterwards: no divergent branches, so the
     // loads really are issued back to back
@@ -456,10 +459,10 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int idx = tid + i * 256;
-            const int row = a_kfast ? idx / kSmallK : idx & 63, kk = a_kfast ? idx % kSmallK : idx >> 6;
+            const int row = a_kfast ? idx / KCH : idx & 63, kk = a_kfast ? idx % KCH : idx >> 6;
             const int64_t gr = min(m0 + row, m_last), gk = k_begin + min(kk, k_last);
             va[i] = a_kfast ? A[gr * g.lda + gk] : A[gk * g.lda + gr];
-            const int col = b_kfast ? idx / kSmallK : idx & 63, kk2 = b_kfast ? idx % kSmallK : idx >> 6;
+            const int col = b_kfast ? idx / KCH : idx & 63, kk2 = b_kfast ? idx % KCH : idx >> 6;
             const int64_t gc = min(n0 + col, n_last), gk2 = k_begin + min(kk2, k_last);
             vb[i] = b_kfast ? B[gc * g.ldb + gk2] : B[gk2 * g.ldb + gc];
         }
@@ -467,17 +470,17 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int idx = tid + i * 256;
-        const int row = a_kfast ? idx / kSmallK : idx & 63, kk = a_kfast ? idx % kSmallK : idx >> 6;
+        const int row = a_kfast ? idx / KCH : idx & 63, kk = a_kfast ? idx % KCH : idx >> 6;
         if (m0 + row > m_last || kk >= kc) va[i] = 0.f;
-        const int col = b_kfast ? idx / kSmallK : idx & 63, kk2 = b_kfast ? idx % kSmallK : idx >> 6;
+        const int col = b_kfast ? idx / KCH : idx & 63, kk2 = b_kfast ? idx % KCH : idx >> 6;
         if (n0 + col > n_last || kk2 >= kc) vb[i] = 0.f;
     }
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int idx = tid + i * 256;
-        const int row = a_kfast ? idx / kSmallK : idx & 63, kk = a_kfast ? idx % kSmallK : idx >> 6;
+        const int row = a_kfast ? idx / KCH : idx & 63, kk = a_kfast ? idx % KCH : idx >> 6;
         as[row * kSmallLd + kk] = va[i];
-        const int col = b_kfast ? idx / kSmallK : idx & 63, kk2 = b_kfast ? idx % kSmallK : idx >> 6;
+        const int col = b_kfast ? idx / KCH : idx & 63, kk2 = b_kfast ? idx % KCH : idx >> 6;
         bs[col * kSmallLd + kk2] = vb[i];
     }
     __syncthreads();
@@ -620,6 +623,25 @@ static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool 
     return direct ? launch_mfma_layout2<Cfg, true>(g, batch, a_kc, b_kc) : launch_mfma_layout2<Cfg, false>(g, batch, a_kc, b_kc);
 }
 
+template <bool A_KFAST, bool B_KFAST, int KCH>
+static int launch_small_one(const GemmArgs& g, dim3 grid, size_t lds) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_small_kernel<A_KFAST, B_KFAST, KCH>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_small_kernel<A_KFAST, B_KFAST, KCH>), grid, dim3(256), lds, stream(), g);
+    return BH_OK;
+}
+template <bool A_KFAST, bool B_KFAST>
+static int launch_small(int kch, const GemmArgs& g, dim3 grid, size_t lds) {
+    if (kch == 32) return launch_small_one<A_KFAST, B_KFAST, 32>(g, grid, lds);
+    if (kch == 64) return launch_small_one<A_KFAST, B_KFAST, 64>(g, grid, lds);
+    return launch_small_one<A_KFAST, B_KFAST, kSmallK>(g, grid, lds);
+}
+
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
 static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, -1 = heuristic
 
@@ -701,10 +723,17 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
             run.stride_c = m * n;
         }
         dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)g.k_splits);
-        if (a_kc && b_kc) hipLaunchKernelGGL((gemm_small_kernel<true, true>), grid, dim3(256), 0, stream(), run);
-        else if (a_kc) hipLaunchKernelGGL((gemm_small_kernel<true, false>), grid, dim3(256), 0, stream(), run);
-        else if (b_kc) hipLaunchKernelGGL((gemm_small_kernel<false, true>), grid, dim3(256), 0, stream(), run);
-        else hipLaunchKernelGGL((gemm_small_kernel<false, false>), grid, dim3(256), 0, stream(), run);
+        constexpr size_t lds = 2 * 64 * kSmallLd * sizeof(float);
+        const int kch = g.k_per_split <= 32 ? 32 : g.k_per_split <= 64 ? 64 : kSmallK;
+        int lrc;
+        if (a_kc && b_kc) lrc = launch_small<true, true>(kch, run, grid, lds);
+        else if (a_kc) lrc = launch_small<true, false>(kch, run, grid, lds);
+        else if (b_kc) lrc = launch_small<false, true>(kch, run, grid, lds);
+        else lrc = launch_small<false, false>(kch, run, grid, lds);
+        if (lrc) {
+            if (ws) bh_free(ws);
+            return lrc;
+        }
         int rc = BH_LAUNCH_CHECK("gemm_small_kernel");
         if (rc == BH_OK && g.k_splits > 1) {
             int64_t blocks = ceil_div(m * n * batch, 256);

@@ -26,6 +26,27 @@ __global__ __launch_bounds__(kRBlock) void sum_partial_kernel(const float* x, fl
     float t = block_sum<kRBlock / 64>(acc, red);
     if (threadIdx.x == 0) partial[blockIdx.x] = t;
 }
+// small inputs: one workgroup does both stages
+__global__ __launch_bounds__(kRBlock) void sum_small_kernel(const float* x, float* out, int64_t n) {
+    __shared__ double red[kRBlock / 64];
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int64_t i = threadIdx.x;
+    for (; i + 3 * kRBlock < n; i += 4 * kRBlock) {
+        a0 += x[i];
+        a1 += x[i + kRBlock];
+        a2 += x[i + 2 * kRBlock];
+        a3 += x[i + 3 * kRBlock];
+    }
+    for (; i < n; i += kRBlock) a0 += x[i];
+    double acc = wave_sum_f64((double)((a0 + a1) + (a2 + a3)));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int w = 0; w < kRBlock / 64; w++) t += red[w];
+        out[0] = (float)t;
+    }
+}
 __global__ __launch_bounds__(kRBlock) void sum_final_kernel(const float* partial, float* out, int n, float scale) {
     __shared__ double red[kRBlock / 64];
     double acc = 0.0;
@@ -137,6 +158,10 @@ extern "C" {
 int bh_sum_all(const float* x, float* out1, int64_t n) {
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(n >= 0 && out1 && (x || n == 0), "bad argument");
+    if (n <= 16 * kRBlock) {   // a few elements per lane: one launch
+        hipLaunchKernelGGL(sum_small_kernel, dim3(1), dim3(kRBlock), 0, stream(), x, out1, n);
+        return BH_LAUNCH_CHECK("bh_sum_all");
+    }
     int blocks = (int)ceil_div(n > 0 ? n : 1, (int64_t)kRBlock * 8);
     if (blocks > 1024) blocks = 1024;
     float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);
@@ -153,6 +178,11 @@ int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumu
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(rows >= 0 && cols >= 0 && (out || cols == 0) && (x || rows * cols == 0), "bad argument");
     if (cols == 0) return BH_OK;
+    if (rows <= 256) {   // few rows: the fold kernel (64 columns x 16 row lanes per workgroup) is the whole column sum
+        hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(cols, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0, stream(),
+                           x, rows, cols, out, (float*)nullptr, cols, accumulate);
+        return BH_LAUNCH_CHECK("bh_colsum");
+    }
     const int col_blocks = (int)ceil_div(cols, kRBlock);
     // enough row chunks to put ~2k blocks on the chip, at least 32 rows each
     int64_t chunks = ceil_div(2048, col_blocks);

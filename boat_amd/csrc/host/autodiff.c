@@ -401,12 +401,22 @@ static boat_tensor_t* row_softmax_grad(bool log_form, const boat_tensor_t* y, co
     return dx;
 }
 
-/* first element of a (scalar) gradient tensor, read back to the host: the reference reads
- * grad_output[0] as float for sum/dot (autodiff.c:1228, 1536) */
-static bool scalar_of(const boat_tensor_t* t, float* out) {
-    if (!t || t->nelements < 1) return false;
-    const float* p = bt_dev_read(t);
-    return p && boat_hip_ok(bh_memcpy_d2h(out, p, sizeof(float)), "scalar readback");
+/* like * dy[0] (like == NULL: a tensor of shape_of's shape filled with dy[0]).  The reference reads grad_output[0] on
+ * the host for sum and dot (autodiff.c:1228, 1536); here the scalar is read by the kernel, so backward never waits for
+ * the device. */
+static boat_tensor_t* scaled_by_first(const boat_tensor_t* shape_of, const boat_tensor_t* like, const boat_tensor_t* dy) {
+    if (!dy || dy->nelements < 1 || !bt_is_f32(dy) || !bt_is_f32(shape_of)) return NULL;
+    boat_tensor_t* g = bt_new_like_uninit(shape_of);
+    if (!g || g->nelements == 0) return g;
+    const float* pin = like ? bt_dev_read(like) : NULL;
+    const float* ps = bt_dev_read(dy);
+    float* pg = bt_dev_write(g);
+    if ((like && !pin) || !ps || !pg ||
+        !boat_hip_ok(bh_scale_by_device_scalar(pin, ps, pg, (int64_t)g->nelements), "scale by gradient scalar")) {
+        boat_tensor_free(g);
+        return NULL;
+    }
+    return g;
 }
 
 static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
@@ -446,13 +456,10 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
                 accumulate(b, g, true);
             }
             break;
-        case OP_DOT: {   /* :1205-1242 */
-            float s;
-            if (!scalar_of(dy, &s)) break;
-            if (a->requires_grad) accumulate(a, boat_mul_scalar(b->data, s), true);
-            if (b->requires_grad) accumulate(b, boat_mul_scalar(a->data, s), true);
+        case OP_DOT:     /* :1205-1242: da = b * dy[0], db = a * dy[0] */
+            if (a->requires_grad) accumulate(a, scaled_by_first(b->data, b->data, dy), true);
+            if (b->requires_grad) accumulate(b, scaled_by_first(a->data, a->data, dy), true);
             break;
-        }
         case OP_RELU:      /* :1244-1296, mask from the op input */
             if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_RELU, a->data, dy), true);
             break;
@@ -487,15 +494,9 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
             }
             break;
         }
-        case OP_SUM: {     /* :1498-1548: ones * (float)dy[0] */
-            float s;
-            if (!a->requires_grad || !scalar_of(dy, &s)) break;
-            boat_tensor_t* ones = ones_like(a->data);
-            boat_tensor_t* g = ones ? boat_mul_scalar(ones, s) : NULL;
-            boat_tensor_free(ones);
-            accumulate(a, g, true);
+        case OP_SUM:       /* :1498-1548: ones * (float)dy[0], i.e. dy[0] everywhere */
+            if (a->requires_grad) accumulate(a, scaled_by_first(a->data, NULL, dy), true);
             break;
-        }
         case OP_MEAN: {    /* :1550-1618: (ones * 1/n) * dy */
             if (!a->requires_grad) break;
             boat_tensor_t* ones = ones_like(a->data);

@@ -161,12 +161,18 @@ void boat_optimizer_zero_grad(boat_optimizer_t* optimizer) {
     if (!optimizer) return;
     adam_state_t* s = (adam_state_t*)optimizer;
     if (!known_type(s)) return;
+    /* one launch over all gradient tensors (the table arrays are sized for num_params) */
+    int count = 0;
     for (size_t i = 0; i < s->num_params; i++) {
         boat_tensor_t* g = s->grads[i];
-        if (!g || g->nelements == 0) continue;
+        if (!g || g->nelements == 0 || !bt_is_f32(g)) continue;
         float* p = bt_dev_write(g);
-        if (p) boat_hip_ok(bh_memset_zero(p, g->nbytes), "boat_optimizer_zero_grad");
+        if (!p) continue;
+        s->tp[count] = p;
+        s->tn[count] = (int64_t)g->nelements;
+        count++;
     }
+    if (count) boat_hip_ok(bh_zero_multi(s->tp, s->tn, count), "boat_optimizer_zero_grad");
 }
 
 void boat_optimizer_free(boat_optimizer_t* optimizer) {

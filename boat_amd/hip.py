@@ -37,7 +37,7 @@ _SIGS = {
     "bh_add_inplace": (I, [P, P, L]),
     "bh_binary": (I, [I, P, P, P, L]),
     "bh_binary_broadcast": (I, [I, P, C.POINTER(L), P, C.POINTER(L), P, C.POINTER(L), I]),
-    "bh_scalar_op": (I, [I, P, F, P, L]),
+    "bh_scalar_op": (I, [I, P, F, P, L]), "bh_copy_f32": (I, [P, P, L]), "bh_scale_by_device_scalar": (I, [P, P, P, L]),
     "bh_div_backward_b": (I, [P, P, P, P, L]),
     "bh_activation_forward": (I, [I, P, P, L]),
     "bh_activation_backward": (I, [I, P, P, P, L, I]),
@@ -63,6 +63,7 @@ _SIGS = {
     "bh_conv2d_backward": (I, [P, P, P, P, P, P] + [L] * 8 + [I, I]),
     "bh_maxpool2d_forward": (I, [P, P, P] + [L] * 6),
     "bh_maxpool2d_backward": (I, [P, P, P] + [L] * 6),
+    "bh_zero_multi": (I, [C.POINTER(P), C.POINTER(L), I]),
     "bh_rmsprop_update": (I, [P, P, P, L, F, F, F]),
     "bh_adagrad_update": (I, [P, P, P, L, F, F]),
     "bh_adam_update_multi": (I, [C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(L), I, F, F, F, F, L]),

@@ -71,6 +71,10 @@ int bh_binary(int op, const float* a, const float* b, float* out, int64_t n);   
 int bh_binary_broadcast(int op, const float* a, const int64_t* a_shape,
                         const float* b, const int64_t* b_shape,
                         float* out, const int64_t* out_shape, int ndim);
+/* out[i] = in[i] * scalar[0] (in == NULL: out[i] = scalar[0]) with the scalar read on the device: the gradient rules of
+ * sum and dot scale by grad_output[0] (src/autodiff.c:1228, 1536), which here never leaves HBM */
+int bh_scale_by_device_scalar(const float* in, const float* scalar, float* out, int64_t n);
+int bh_copy_f32(float* dst, const float* src, int64_t n);   /* dst = src on the stream (bh_memcpy_d2d uses it for whole floats) */
 int bh_scalar_op(int op, const float* a, float s, float* out, int64_t n);             /* boat_*_scalar */
 /* d(a/b)/db = (dy*-1) * (a/(b*b))  (src/autodiff.c:1172-1201) */
 int bh_div_backward_b(const float* a, const float* b, const float* dy, float* db, int64_t n);
@@ -172,6 +176,9 @@ int bh_rmsprop_update_multi(float* const* p, const float* const* g, float* const
                             float lr, float alpha, float eps);
 int bh_adagrad_update_multi(float* const* p, const float* const* g, float* const* sum, const int64_t* n, int count,
                             float lr, float eps);
+
+/* zero `count` tensors in one launch: adam_optimizer_zero_grad's per-tensor memset loop (src/optimizers/adam.c:243-263) */
+int bh_zero_multi(float* const* p, const int64_t* n, int count);
 
 /* ---- test hooks (no arithmetic of their own) ----
  * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256 MFMA tile,

@@ -213,7 +213,7 @@ def test_adam_zero_gradient_is_a_no_op(hip):
 
 # ------------------------------------------------------- reductions, softmax
 
-@pytest.mark.parametrize("n", [1, 63, 100000])
+@pytest.mark.parametrize("n", [1, 63, 4096, 4097, 100000])
 def test_sum_all(hip, oracle, rng, n):
     x = rng.standard_normal(n).astype(np.float32)
     out = hip.empty(1)
@@ -366,7 +366,7 @@ def test_gemm_direct_to_lds_edges_epilogues_and_split_k(hip, rng, force, ta, tb)
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
-@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (33, 17, 5), (64, 64, 112), (65, 63, 113), (37, 130, 225), (200, 70, 1000),
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (33, 17, 5), (64, 64, 128), (65, 63, 129), (37, 130, 225), (200, 70, 1000),
                                    (256, 512, 64)])
 def test_gemm_small_problem_kernel(hip, rng, ta, tb, m, n, k):
     gemm_case(hip, rng, ta, tb, m, n, k, force=5)
@@ -522,3 +522,40 @@ def test_maxpool2d_forward_backward(hip, oracle, rng, shape):
     plane = (np.arange(B * ch) * h * w).reshape(B, ch, 1, 1)
     assert np.array_equal(arg.numpy().astype(np.int64) + plane, o_arg)
     assert np.array_equal(gx.numpy(), oracle.maxpool2d_backward(dy, o_arg, x.shape))
+
+
+def test_zero_multi(hip, rng):
+    sizes = [1, 3, 4, 1000, 4097, 100352, 128, 1280, 10]
+    arrs = [dev(hip, rng.standard_normal(n).astype(np.float32)) for n in sizes]
+    guard = dev(hip, np.ones(8, np.float32))
+    ptrs = (C.c_void_p * len(sizes))(*[a.ptr for a in arrs])
+    ns = (C.c_int64 * len(sizes))(*sizes)
+    hip.check(hip.bh_zero_multi(ptrs, ns, len(sizes)))
+    for a in arrs:
+        assert not a.numpy().any()
+    assert guard.numpy().tolist() == [1.0] * 8
+    # an unaligned view (offset by one float) and a zero-length entry
+    base = dev(hip, np.ones(1001, np.float32))
+    ptrs2 = (C.c_void_p * 2)(base.ptr + 4, base.ptr)
+    ns2 = (C.c_int64 * 2)(999, 0)
+    hip.check(hip.bh_zero_multi(ptrs2, ns2, 2))
+    got = base.numpy()
+    assert got[0] == 1 and got[1000] == 1 and not got[1:1000].any()
+    assert hip.bh_zero_multi(None, None, 0) == 0
+
+
+@pytest.mark.parametrize("n,offset", [(1, 0), (1000, 0), (1003, 1), (1 << 20, 0), (4099, 3)])
+def test_device_to_device_copy(hip, rng, n, offset):
+    """bh_memcpy_d2d: bit-preserving (NaN payloads, -0.0), any float alignment, odd byte counts through the runtime."""
+    src = rng.standard_normal(n + 8).astype(np.float32)
+    src[:3] = [np.nan, -0.0, np.inf]
+    bits = src.view(np.uint32).copy()
+    bits[0] = 0x7FC12345                                     # a NaN with a payload
+    src = bits.view(np.float32)
+    d_src, d_dst = dev(hip, src), dev(hip, np.zeros(n + 8, np.float32))
+    hip.check(hip.bh_memcpy_d2d(d_dst.ptr + 4 * offset, d_src.ptr + 4 * offset, 4 * n))
+    got = d_dst.numpy().view(np.uint32)
+    assert np.array_equal(got[offset:offset + n], bits[offset:offset + n])
+    assert not got[:offset].any() and not got[offset + n:].any()
+    hip.check(hip.bh_memcpy_d2d(d_dst.ptr + 1, d_src.ptr + 1, 6))          # not whole floats: runtime copy
+    assert np.array_equal(d_dst.numpy().view(np.uint8)[1:7], src.view(np.uint8)[1:7])

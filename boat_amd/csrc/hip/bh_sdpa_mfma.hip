@@ -202,7 +202,8 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
 // whole kernel.
 // dQ = dS.K of a query tile contracts over all 128 keys of the workgroup, so the four wavefronts first
 // publish their dS blocks in LDS and then each computes a [32 queries][16 head-dim columns] slice with
-// v_mfma_f32_16x16x4_f32 and stores it straight to the key tile's partial dQ: no cross-wavefront sum.
+// v_mfma_f32_16x16x4_f32 (as the transposed product, so that a lane holds four consecutive head-dim columns of a query
+// row) and stores it straight to the key tile's partial dQ with 16-byte stores: no cross-wavefront sum.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
 
@@ -362,21 +363,22 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
             const float4 a1 = *reinterpret_cast<const float4*>(dsb + (16 + i16) * BwdSmem::kDsLd + 16 * g + 4 * kk);
             const float* kb = kall + (16 * g + 4 * kk) * kLd + 16 * w + i16;
             const float b0 = kb[0], b1 = kb[kLd], b2 = kb[2 * kLd], b3 = kb[3 * kLd];
-            acc_dq0 = MFMA16(a0.x, b0, acc_dq0);
-            acc_dq1 = MFMA16(a1.x, b0, acc_dq1);
-            acc_dq0 = MFMA16(a0.y, b1, acc_dq0);
-            acc_dq1 = MFMA16(a1.y, b1, acc_dq1);
-            acc_dq0 = MFMA16(a0.z, b2, acc_dq0);
-            acc_dq1 = MFMA16(a1.z, b2, acc_dq1);
-            acc_dq0 = MFMA16(a0.w, b3, acc_dq0);
-            acc_dq1 = MFMA16(a1.w, b3, acc_dq1);
+            // operands swapped: the product is the transpose dQ^T[d][query], so a lane ends up with four consecutive
+            // head-dim columns of one query row and stores them as one 16-byte piece
+            acc_dq0 = MFMA16(b0, a0.x, acc_dq0);
+            acc_dq1 = MFMA16(b0, a1.x, acc_dq1);
+            acc_dq0 = MFMA16(b1, a0.y, acc_dq0);
+            acc_dq1 = MFMA16(b1, a1.y, acc_dq1);
+            acc_dq0 = MFMA16(b2, a0.z, acc_dq0);
+            acc_dq1 = MFMA16(b2, a1.z, acc_dq1);
+            acc_dq0 = MFMA16(b3, a0.w, acc_dq0);
+            acc_dq1 = MFMA16(b3, a1.w, acc_dq1);
         }
-        // accumulator register e of lane (i16, kk) is query row 4*kk + e of the 16-row tile, column i16
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            dqh[(int64_t)(q0 + 4 * kk + e) * kD + 16 * w + i16] = acc_dq0[e];
-            dqh[(int64_t)(q0 + 16 + 4 * kk + e) * kD + 16 * w + i16] = acc_dq1[e];
-        }
+        // accumulator register e of lane (i16, kk) is head-dim column 16w + 4*kk + e of query row i16 of the 16-row tile
+        *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk) =
+            make_float4(acc_dq0[0], acc_dq0[1], acc_dq0[2], acc_dq0[3]);
+        *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + 16 + i16) * kD + 16 * w + 4 * kk) =
+            make_float4(acc_dq1[0], acc_dq1[1], acc_dq1[2], acc_dq1[3]);
         __syncthreads();   // dS tile free again; the next Q and dO tiles are in place
     }
 #undef BWD_LD

@@ -49,7 +49,7 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="all",
-                    help="comma list of dense,adam,ln_gelu,sdpa,mlp,block (default all); for profiling one workload at a time. "
+                    help="comma list of dense,adam,ln_gelu,sdpa,mlp,cnn,block (default all); for profiling one workload at a time. "
                          "Without the dense leg the line carries no value/roofline.")
     return ap.parse_args()
 
@@ -149,6 +149,13 @@ def bench_adam(hip, steps, warmup):
     gbs = 28.0 * n / (ms * 1e-3) / 1e9
     out["adam_flat_268M"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4),
                              "bytes": 28 * n}
+    # RMSprop and Adagrad over the same flat arrays (one state tensor: read p, g, state; write p, state = 20 B/param)
+    for name, fn in (("rmsprop_flat_268M", lambda: hip.bh_rmsprop_update(p.ptr, g.ptr, m.ptr, n, 1e-3, 0.99, 1e-8)),
+                     ("adagrad_flat_268M", lambda: hip.bh_adagrad_update(p.ptr, g.ptr, v.ptr, n, 1e-3, 1e-10))):
+        ms = time_steps(hip, lambda: hip.check(fn()), steps, warmup)
+        gbs = 20.0 * n / (ms * 1e-3) / 1e9
+        out[name] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4),
+                     "bytes": 20 * n}
     del p, g, m, v
     return out
 
@@ -220,6 +227,83 @@ def bench_mlp_step(steps, warmup):
             "loss_first_last": [rec["loss_first"], rec["loss_last"]],
             "note": "MLP 784-128-10 B64 fwd+bwd+Adam+zero_grad through boat_var_* / boat_variable_backward_full / "
                     "boat_optimizer_step, a C caller linked against libboat_amd.so, wall clock"}
+
+
+def bench_cnn_step(steps, warmup):
+    """The MNIST CNN of examples/mnist/mnist_autodiff.c:536-557 through Boat's C API, batch 64: conv(1->32, 3x3, pad 1),
+    relu, maxpool 2, conv(32->64), relu, maxpool 2, flatten, dense 3136->128, relu, dense 128->10, cross-entropy chain;
+    forward + boat_variable_backward_full + Adam + zero_grad, wall ms."""
+    from boat_amd.capi import default_api
+    api = default_api()
+    rng = np.random.default_rng(20250107)
+    B, classes = 64, 10
+    x = rng.random((B, 1, 28, 28), dtype=np.float32)
+    labels = rng.integers(0, classes, B)
+    onehot = np.zeros((B, classes), np.float32)
+    onehot[np.arange(B), labels] = 1
+    c1 = api.boat_conv_layer_create(1, 32, 3, 1, 1)
+    c2 = api.boat_conv_layer_create(32, 64, 3, 1, 1)
+    p1, p2 = api.boat_pool_layer_create(2, 2, 0), api.boat_pool_layer_create(2, 2, 0)
+    d1 = api.boat_dense_layer_create(64 * 7 * 7, 128, True)
+    d2 = api.boat_dense_layer_create(128, classes, True)
+    for layer, shape in ((c1, (32, 1, 3, 3)), (c2, (64, 32, 3, 3))):
+        s = np.sqrt(2.0 / (shape[1] * 9))
+        api.write(api.boat_conv_layer_get_weight(layer), rng.uniform(-s, s, shape).astype(np.float32))
+    for layer, (fi, fo) in ((d1, (3136, 128)), (d2, (128, classes))):
+        s = np.sqrt(2.0 / (fi + fo))
+        api.write(api.boat_dense_layer_get_weight(layer), rng.uniform(-s, s, (fi, fo)).astype(np.float32))
+    opt = api.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
+    api.boat_hip_optimizer_add_conv(opt, c1)
+    api.boat_hip_optimizer_add_conv(opt, c2)
+    api.boat_hip_optimizer_add_dense(opt, d1)
+    api.boat_hip_optimizer_add_dense(opt, d2)
+    tx, toh = api.tensor(x), api.tensor(onehot)
+    tf = api.tensor(np.array([-1.0 / B], np.float32))
+    losses = []
+
+    def step(keep_loss=False):
+        vx = api.boat_variable_create(tx, True)
+        voh = api.boat_variable_create(toh, False)
+        vf = api.boat_variable_create(tf, False)
+        a1 = api.boat_var_conv(vx, c1)
+        r1 = api.boat_var_relu(a1)
+        q1 = api.boat_var_pool(r1, p1)
+        a2 = api.boat_var_conv(q1, c2)
+        r2 = api.boat_var_relu(a2)
+        q2 = api.boat_var_pool(r2, p2)
+        fl = api.boat_var_flatten(q2)
+        h = api.boat_var_dense(fl, d1)
+        rh = api.boat_var_relu(h)
+        z = api.boat_var_dense(rh, d2)
+        ls = api.boat_var_log_softmax(z, 1)
+        mm = api.boat_var_mul(voh, ls)
+        sm = api.boat_var_sum(mm, None, 0, False)
+        loss = api.boat_var_mul(vf, sm)
+        assert loss, "CNN forward failed"
+        api.boat_variable_backward_full(loss)
+        api.boat_optimizer_step(opt)
+        api.boat_optimizer_zero_grad(opt)
+        if keep_loss:
+            losses.append(float(api.numpy(api.boat_variable_data(loss))[0]))
+        for var in (loss, sm, mm, ls, z, rh, h, fl, q2, r2, a2, q1, r1, a1, vf, voh, vx):
+            api.boat_variable_free(var)
+
+    step(keep_loss=True)
+    for _ in range(warmup):
+        step()
+    api.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.sync()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    step(keep_loss=True)
+    assert np.isfinite(losses).all() and losses[1] < losses[0], f"CNN training does not reduce the loss: {losses}"
+    conv_flops = 2.0 * B * (32 * 1 * 9 * 28 * 28 + 64 * 32 * 9 * 14 * 14) * 3       # forward + dX + dW of both conv layers
+    return {"ms": round(ms, 4), "bound": "launch latency / small kernels", "conv_flops": conv_flops,
+            "loss_first_last": [round(l, 6) for l in losses],
+            "note": "MNIST CNN B64 (conv 1->32, conv 32->64, dense 3136->128->10): fwd + bwd + Adam + zero_grad through the "
+                    "C API from Python, wall clock"}
 
 
 def bench_block_step(steps, warmup):
@@ -347,7 +431,7 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build (the path has no inter-GPU work)",
               file=sys.stderr)
         sys.exit(2)
-    all_legs = ["dense", "adam", "ln_gelu", "sdpa", "mlp", "block"]
+    all_legs = ["dense", "adam", "ln_gelu", "sdpa", "mlp", "cnn", "block"]
     legs = all_legs if args.legs == "all" else [l.strip() for l in args.legs.split(",") if l.strip()]
     unknown = [l for l in legs if l not in all_legs]
     if unknown:
@@ -379,6 +463,8 @@ def main():
         extra.update(bench_sdpa(hip, args.steps, args.warmup))
     if "mlp" in legs:
         extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20) * 25, max(args.warmup, 1) * 10)
+    if "cnn" in legs:
+        extra["mnist_cnn_step"] = bench_cnn_step(max(args.steps, 20), max(args.warmup, 3))
     if "block" in legs:
         extra["transformer_block_step"] = bench_block_step(max(2, min(args.steps, 10)), min(args.warmup, 2))
     if extra:

@@ -1,4 +1,4 @@
-// bh_conv.hip - direct 2-D convolution (NCHW, square kernel) and max pooling, forward and backward.
+// bh_conv.hip - 2-D convolution (NCHW, square kernel) and max pooling, forward and backward.
 //
 // Replaces the loops of the reference's convolution and pooling layers:
 //   boat_conv_layer_forward            src/layers/conv.c:326-437
@@ -6,20 +6,25 @@
 //   compute_bias_gradient              src/layers/conv.c:165-201
 //   compute_input_gradient             src/layers/conv.c:46-103
 //   boat_pool_layer_forward/backward   src/layers/pool.c:63-218
-// The shapes on this path are the small ones of the MNIST network (1->32 and 32->64 channels, 3x3, 28x28 and
-// 14x14 images, batches of tens), far too small to fill the matrix cores through an im2col GEMM, so every
-// kernel is a direct gather: one lane per output element, operands served by the caches, no atomics, and each
-// result is written exactly once (deterministic).
+//
+// Forward is a direct gather, one lane per output element, in the reference's fp32 operation order (per input
+// channel a running sum over the taps, added to the output, bias last): bit-identical, so the pooling layer behind it
+// picks the same maxima as the reference.
+//
+// Backward is three contractions on the matrix cores through bh_gemm, with K = in_channels*k*k and P = batch*ho*wo:
+//   dyp [oc][P]   = dy regrouped from [batch][oc][ho*wo]      (one permute kernel)
+//   col [P][K]    = patches of x (im2col, zero outside the image)
+//   gw  [oc][K]  (+)= dyp . col                                (the contraction runs over all P output positions)
+//   dcol[P][K]    = dyp^T . w                                  then dx gathers its <= k*k entries of dcol (col2im)
+//   gb  [oc]     (+)= row sums of dyp
+// No atomics; every result element is written once (deterministic).  The gradient sums run in MFMA and tree order,
+// so they agree with the reference to rounding, not bit for bit.
 //
 // Input gradient.  The reference pairs tap (kh, kw) of the scatter ih = oh*stride - pad + kh with the weight
 // of the mirrored tap (k-1-kh, k-1-kw) (conv.c:86-88); that is the gradient of a different layer, and its own
 // gradient check only looks at weight and bias gradients (tests/unit/test_conv_gradient_check.c:317-332).
 // flip_taps == 0 computes the true gradient dx[ih,iw] = sum w[oc,ic,kh,kw]*dy[oh,ow]; flip_taps != 0 reproduces
-// the reference's pairing, so that its numbers can be checked against.
-//
-// Forward keeps the reference's fp32 operation order (per input channel a running sum over the taps, added to
-// the output, bias last), so it is bit-identical; the gradient reductions add in wavefront trees and agree to
-// rounding.
+// the reference's pairing (the weights are mirrored into a scratch copy first), so that its numbers can be checked.
 #include "bh_common.h"
 
 #include <math.h>
@@ -32,9 +37,71 @@ struct ConvShape {
     int batch, ic, h, w, oc, k, stride, pad, ho, wo;
 };
 
+// One lane per output position, kOcTile output channels per lane: the k x k patch of an input channel is loaded once
+// and feeds kOcTile running sums; the weights of a workgroup's channel group are wave-uniform (the group comes from
+// blockIdx), so they arrive through the scalar path as whole k*k rows.  Per output element the operation order is the
+// reference's: for each input channel a sum over the taps in (kh, kw) order, taps outside the image skipped, added to
+// the output; bias last (conv.c:398-436).  "Skipped" is a select, not a branch: a tap outside the image reads a clamped
+// (valid) address and leaves the running sum untouched.
+constexpr int kOcTile = 8;
+
+template <int K>   // kernel size (compile time: the taps live in registers)
 __global__ __launch_bounds__(kCBlock) void conv2d_fwd_kernel(const float* __restrict__ x, const float* __restrict__ wt,
                                                              const float* __restrict__ bias, float* __restrict__ y,
-                                                             ConvShape c, int64_t total) {
+                                                             ConvShape c) {
+    const int per = c.ho * c.wo;
+    const int p = blockIdx.x * kCBlock + threadIdx.x;
+    const int oc0 = blockIdx.y * kOcTile;
+    const int b = blockIdx.z;
+    if (p >= per) return;
+    const int oh = p / c.wo, ow = p % c.wo;
+    const int ih0 = oh * c.stride - c.pad, iw0 = ow * c.stride - c.pad;
+    bool valid[K * K];
+    int off[K * K];
+#pragma unroll
+    for (int kh = 0; kh < K; kh++)
+#pragma unroll
+        for (int kw = 0; kw < K; kw++) {
+            const int ih = ih0 + kh, iw = iw0 + kw;
+            valid[kh * K + kw] = ih >= 0 && ih < c.h && iw >= 0 && iw < c.w;
+            off[kh * K + kw] = min(max(ih, 0), c.h - 1) * c.w + min(max(iw, 0), c.w - 1);
+        }
+    const float* wrow[kOcTile];      // channel group rows, clamped to the last real channel (extra lanes are not stored)
+#pragma unroll
+    for (int o = 0; o < kOcTile; o++) wrow[o] = wt + (int64_t)min(oc0 + o, c.oc - 1) * c.ic * K * K;
+    float out[kOcTile];
+#pragma unroll
+    for (int o = 0; o < kOcTile; o++) out[o] = 0.f;
+    const float* xp = x + (int64_t)b * c.ic * c.h * c.w;
+    for (int ci = 0; ci < c.ic; ci++, xp += c.h * c.w) {
+        float xv[K * K];
+#pragma unroll
+        for (int t = 0; t < K * K; t++) xv[t] = xp[off[t]];
+#pragma unroll
+        for (int o = 0; o < kOcTile; o++) {
+            const float* wp = wrow[o] + ci * K * K;
+            float sum = 0.f;
+#pragma unroll
+            for (int t = 0; t < K * K; t++) {
+                const float term = sum + xv[t] * wp[t];
+                sum = valid[t] ? term : sum;
+            }
+            out[o] += sum;
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < kOcTile; o++) {
+        if (oc0 + o >= c.oc) break;
+        float v = out[o];
+        if (bias) v += bias[oc0 + o];
+        y[((int64_t)b * c.oc + oc0 + o) * per + p] = v;
+    }
+}
+
+// any kernel size: one lane per output element, taps looped at run time, same operation order
+__global__ __launch_bounds__(kCBlock) void conv2d_fwd_generic_kernel(const float* __restrict__ x, const float* __restrict__ wt,
+                                                                     const float* __restrict__ bias, float* __restrict__ y,
+                                                                     ConvShape c, int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
     if (i >= total) return;
     const int ow = (int)(i % c.wo);
@@ -62,78 +129,87 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_kernel(const float* __rest
     y[i] = out;
 }
 
-// dx[b,ic,ih,iw] = sum_{oc,kh,kw} w[oc,ic,kh',kw'] * dy[b,oc,oh,ow] with oh*stride - pad + kh == ih
-__global__ __launch_bounds__(kCBlock) void conv2d_bwd_input_kernel(const float* __restrict__ wt, const float* __restrict__ dy,
-                                                                   float* __restrict__ dx, ConvShape c, int64_t total,
-                                                                   int flip_taps) {
+// dyp[oc][b][p] = dy[b][oc][p], p over the ho*wo output positions
+__global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __restrict__ dy, float* __restrict__ dyp, ConvShape c,
+                                                               int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
+    if (i >= total) return;
+    const int per = c.ho * c.wo;
+    const int p = (int)(i % per);
+    const int b = (int)((i / per) % c.batch);
+    const int oc = (int)(i / ((int64_t)per * c.batch));
+    dyp[i] = dy[((int64_t)b * c.oc + oc) * per + p];
+}
+
+// col[(b, oh, ow)][(ic, kh, kw)] = x[b, ic, oh*stride - pad + kh, ow*stride - pad + kw], zero outside the image
+__global__ __launch_bounds__(kCBlock) void im2col_kernel(const float* __restrict__ x, float* __restrict__ col, ConvShape c,
+                                                         int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
+    if (i >= total) return;
+    const int kk = c.ic * c.k * c.k;
+    const int t = (int)(i % kk);
+    const int64_t pos = i / kk;
+    const int kw = t % c.k, kh = (t / c.k) % c.k, ci = t / (c.k * c.k);
+    const int ow = (int)(pos % c.wo);
+    const int oh = (int)((pos / c.wo) % c.ho);
+    const int b = (int)(pos / ((int64_t)c.wo * c.ho));
+    const int ih = oh * c.stride - c.pad + kh, iw = ow * c.stride - c.pad + kw;
+    col[i] = (ih >= 0 && ih < c.h && iw >= 0 && iw < c.w) ? x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] : 0.f;
+}
+
+// dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(b, oh, ow)][(ic, kh, kw)]
+__global__ __launch_bounds__(kCBlock) void col2im_kernel(const float* __restrict__ dcol, float* __restrict__ dx, ConvShape c,
+                                                         int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
     if (i >= total) return;
     const int iw = (int)(i % c.w);
     const int ih = (int)((i / c.w) % c.h);
     const int ci = (int)((i / ((int64_t)c.w * c.h)) % c.ic);
     const int b = (int)(i / ((int64_t)c.w * c.h * c.ic));
+    const int kk = c.ic * c.k * c.k;
     float acc = 0.f;
-    for (int oc = 0; oc < c.oc; oc++) {
-        const float* wp = wt + ((int64_t)oc * c.ic + ci) * c.k * c.k;
-        const float* gp = dy + ((int64_t)b * c.oc + oc) * c.ho * c.wo;
-        for (int kh = 0; kh < c.k; kh++) {
-            const int t = ih + c.pad - kh;
-            if (t < 0 || t % c.stride) continue;
-            const int oh = t / c.stride;
-            if (oh >= c.ho) continue;
-            for (int kw = 0; kw < c.k; kw++) {
-                const int u = iw + c.pad - kw;
-                if (u < 0 || u % c.stride) continue;
-                const int ow = u / c.stride;
-                if (ow >= c.wo) continue;
-                const int wk = flip_taps ? (c.k - 1 - kh) * c.k + (c.k - 1 - kw) : kh * c.k + kw;
-                acc += wp[wk] * gp[oh * c.wo + ow];
-            }
+    for (int kh = 0; kh < c.k; kh++) {
+        const int t = ih + c.pad - kh;
+        if (t < 0 || t % c.stride) continue;
+        const int oh = t / c.stride;
+        if (oh >= c.ho) continue;
+        for (int kw = 0; kw < c.k; kw++) {
+            const int u = iw + c.pad - kw;
+            if (u < 0 || u % c.stride) continue;
+            const int ow = u / c.stride;
+            if (ow >= c.wo) continue;
+            acc += dcol[(((int64_t)b * c.ho + oh) * c.wo + ow) * kk + (ci * c.k + kh) * c.k + kw];
         }
     }
     dx[i] = acc;
 }
 
-// gw[oc,ic,kh,kw] (+)= sum_{b,oh,ow} x[b,ic,ih,iw] * dy[b,oc,oh,ow]: one wavefront per weight element
-__global__ __launch_bounds__(kCBlock) void conv2d_bwd_weight_kernel(const float* __restrict__ x, const float* __restrict__ dy,
-                                                                    float* __restrict__ gw, ConvShape c, int64_t n_weights,
-                                                                    int accumulate) {
-    const int lane = threadIdx.x & 63;
-    const int64_t wi = (int64_t)blockIdx.x * (kCBlock / 64) + (threadIdx.x >> 6);
-    if (wi >= n_weights) return;
-    const int kw = (int)(wi % c.k);
-    const int kh = (int)((wi / c.k) % c.k);
-    const int ci = (int)((wi / ((int64_t)c.k * c.k)) % c.ic);
-    const int oc = (int)(wi / ((int64_t)c.k * c.k * c.ic));
-    const int per_image = c.ho * c.wo;
-    const int64_t terms = (int64_t)c.batch * per_image;
-    float acc = 0.f;
-    for (int64_t t = lane; t < terms; t += 64) {
-        const int b = (int)(t / per_image);
-        const int rem = (int)(t % per_image);
-        const int oh = rem / c.wo, ow = rem % c.wo;
-        const int ih = oh * c.stride - c.pad + kh, iw = ow * c.stride - c.pad + kw;
-        if (ih < 0 || ih >= c.h || iw < 0 || iw >= c.w) continue;
-        acc += x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] * dy[((int64_t)b * c.oc + oc) * per_image + rem];
-    }
-    acc = wave_sum(acc);
-    if (lane == 0) gw[wi] = accumulate ? gw[wi] + acc : acc;
+// wf[oc, ic, kh, kw] = w[oc, ic, k-1-kh, k-1-kw]
+__global__ __launch_bounds__(kCBlock) void mirror_taps_kernel(const float* __restrict__ w, float* __restrict__ wf, int taps,
+                                                              int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
+    if (i >= total) return;
+    const int64_t plane = i / taps;
+    const int t = (int)(i % taps);
+    wf[i] = w[plane * taps + (taps - 1 - t)];
 }
 
-// gb[oc] (+)= sum_{b,oh,ow} dy[b,oc,oh,ow]: one workgroup per output channel
-__global__ __launch_bounds__(kCBlock) void conv2d_bwd_bias_kernel(const float* __restrict__ dy, float* __restrict__ gb,
-                                                                  ConvShape c, int accumulate) {
+// out[r] (+)= sum of row r of a [rows][n] matrix: one workgroup per row
+__global__ __launch_bounds__(kCBlock) void rowsum_kernel(const float* __restrict__ a, float* __restrict__ out, int64_t n,
+                                                         int accumulate) {
     __shared__ float red[kCBlock / 64];
-    const int oc = blockIdx.x;
-    const int per_image = c.ho * c.wo;
-    const int64_t terms = (int64_t)c.batch * per_image;
-    float acc = 0.f;
-    for (int64_t t = threadIdx.x; t < terms; t += kCBlock) {
-        const int64_t b = t / per_image, rem = t % per_image;
-        acc += dy[(b * c.oc + oc) * per_image + rem];
+    const float* row = a + (int64_t)blockIdx.x * n;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int64_t i = threadIdx.x;
+    for (; i + 3 * kCBlock < n; i += 4 * kCBlock) {
+        a0 += row[i];
+        a1 += row[i + kCBlock];
+        a2 += row[i + 2 * kCBlock];
+        a3 += row[i + 3 * kCBlock];
     }
-    const float total = block_sum<kCBlock / 64>(acc, red);
-    if (threadIdx.x == 0) gb[oc] = accumulate ? gb[oc] + total : total;
+    for (; i < n; i += kCBlock) a0 += row[i];
+    const float total = block_sum<kCBlock / 64>((a0 + a1) + (a2 + a3), red);
+    if (threadIdx.x == 0) out[blockIdx.x] = accumulate ? out[blockIdx.x] + total : total;
 }
 
 struct PoolShape {
@@ -226,8 +302,16 @@ int bh_conv2d_forward(const float* x, const float* w, const float* bias, float* 
     if (rc) return rc;
     if (batch == 0) return BH_OK;
     BH_CHECK_ARG(x && w && y, "null pointer");
-    const int64_t total = (int64_t)c.batch * c.oc * c.ho * c.wo;
-    hipLaunchKernelGGL(conv2d_fwd_kernel, dim3((unsigned)ceil_div(total, kCBlock)), dim3(kCBlock), 0, stream(), x, w, bias, y, c, total);
+    const dim3 grid((unsigned)ceil_div((int64_t)c.ho * c.wo, kCBlock), (unsigned)ceil_div(c.oc, kOcTile), (unsigned)c.batch);
+    if (c.k == 3 && grid.y <= 65535 && grid.z <= 65535) {
+        hipLaunchKernelGGL(conv2d_fwd_kernel<3>, grid, dim3(kCBlock), 0, stream(), x, w, bias, y, c);
+    } else if (c.k == 5 && grid.y <= 65535 && grid.z <= 65535) {
+        hipLaunchKernelGGL(conv2d_fwd_kernel<5>, grid, dim3(kCBlock), 0, stream(), x, w, bias, y, c);
+    } else {
+        const int64_t total = (int64_t)c.batch * c.oc * c.ho * c.wo;
+        hipLaunchKernelGGL(conv2d_fwd_generic_kernel, dim3((unsigned)ceil_div(total, kCBlock)), dim3(kCBlock), 0, stream(), x, w,
+                           bias, y, c, total);
+    }
     return BH_LAUNCH_CHECK("conv2d_fwd_kernel");
 }
 
@@ -238,27 +322,60 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
     ConvShape c;
     int rc = make_conv_shape(c, batch, in_channels, height, width, out_channels, kernel, stride, pad);
     if (rc) return rc;
-    BH_CHECK_ARG(dy || batch == 0, "null pointer");
-    if (dx && batch > 0) {
-        BH_CHECK_ARG(w, "null pointer");
-        const int64_t total = (int64_t)c.batch * c.ic * c.h * c.w;
-        hipLaunchKernelGGL(conv2d_bwd_input_kernel, dim3((unsigned)ceil_div(total, kCBlock)), dim3(kCBlock), 0, stream(), w, dy, dx,
-                           c, total, flip_taps);
-        rc = BH_LAUNCH_CHECK("conv2d_bwd_input_kernel");
-        if (rc) return rc;
+    const int64_t taps = (int64_t)c.k * c.k, kk = (int64_t)c.ic * taps;      // contraction length of the forward
+    const int64_t positions = (int64_t)c.batch * c.ho * c.wo;
+    if (batch == 0) {   // empty sums: the parameter gradients are zero (or left alone when accumulating)
+        if (gw && !accumulate) rc = bh_memset_zero(gw, sizeof(float) * (size_t)(c.oc * kk));
+        if (rc == BH_OK && gb && !accumulate) rc = bh_memset_zero(gb, sizeof(float) * (size_t)c.oc);
+        return rc;
     }
-    if (gw) {
-        BH_CHECK_ARG(x || batch == 0, "null pointer");
-        const int64_t n_weights = (int64_t)c.oc * c.ic * c.k * c.k;
-        hipLaunchKernelGGL(conv2d_bwd_weight_kernel, dim3((unsigned)ceil_div(n_weights, kCBlock / 64)), dim3(kCBlock), 0, stream(),
-                           x, dy, gw, c, n_weights, accumulate);
-        rc = BH_LAUNCH_CHECK("conv2d_bwd_weight_kernel");
-        if (rc) return rc;
+    BH_CHECK_ARG(dy, "null pointer");
+    BH_CHECK_ARG(!gw || x, "null pointer");
+    BH_CHECK_ARG(!dx || w, "null pointer");
+    BH_CHECK_ARG(positions * kk < ((int64_t)1 << 40), "conv2d: patch matrix too large");
+    if (!dx && !gw && !gb) return BH_OK;
+    auto blocks = [](int64_t n) { return dim3((unsigned)ceil_div(n, kCBlock)); };
+    float *dyp = nullptr, *col = nullptr, *wf = nullptr;
+    dyp = (float*)bh_malloc(sizeof(float) * (size_t)(c.oc * positions));
+    if (!dyp) return BH_ENOMEM;
+    hipLaunchKernelGGL(nchw_to_cnhw_kernel, blocks(c.oc * positions), dim3(kCBlock), 0, stream(), dy, dyp, c, c.oc * positions);
+    rc = BH_LAUNCH_CHECK("nchw_to_cnhw_kernel");
+    if (rc == BH_OK && gb) {
+        hipLaunchKernelGGL(rowsum_kernel, dim3((unsigned)c.oc), dim3(kCBlock), 0, stream(), dyp, gb, positions, accumulate);
+        rc = BH_LAUNCH_CHECK("rowsum_kernel");
     }
-    if (gb) {
-        hipLaunchKernelGGL(conv2d_bwd_bias_kernel, dim3((unsigned)c.oc), dim3(kCBlock), 0, stream(), dy, gb, c, accumulate);
-        rc = BH_LAUNCH_CHECK("conv2d_bwd_bias_kernel");
+    if (rc == BH_OK && (gw || dx)) {
+        col = (float*)bh_malloc(sizeof(float) * (size_t)(positions * kk));   // patches for gw, then reused as dcol
+        if (!col) rc = BH_ENOMEM;
     }
+    if (rc == BH_OK && gw) {
+        hipLaunchKernelGGL(im2col_kernel, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions * kk);
+        rc = BH_LAUNCH_CHECK("im2col_kernel");
+        // gw[oc][kk] (+)= dyp[oc][positions] . col[positions][kk]
+        if (rc == BH_OK) rc = bh_gemm(0, 0, c.oc, kk, positions, dyp, positions, col, kk, gw, kk, nullptr, accumulate, 1);
+    }
+    if (rc == BH_OK && dx) {
+        const float* wsrc = w;
+        if (flip_taps) {
+            wf = (float*)bh_malloc(sizeof(float) * (size_t)(c.oc * kk));
+            if (!wf) rc = BH_ENOMEM;
+            if (rc == BH_OK) {
+                hipLaunchKernelGGL(mirror_taps_kernel, blocks(c.oc * kk), dim3(kCBlock), 0, stream(), w, wf, (int)taps, c.oc * kk);
+                rc = BH_LAUNCH_CHECK("mirror_taps_kernel");
+                wsrc = wf;
+            }
+        }
+        // dcol[positions][kk] = dyp^T[positions][oc] . w[oc][kk]  (the stream orders it after the gw product that read col)
+        if (rc == BH_OK) rc = bh_gemm(1, 0, positions, kk, c.oc, dyp, positions, wsrc, kk, col, kk, nullptr, 0, 1);
+        if (rc == BH_OK) {
+            const int64_t total = (int64_t)c.batch * c.ic * c.h * c.w;
+            hipLaunchKernelGGL(col2im_kernel, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, total);
+            rc = BH_LAUNCH_CHECK("col2im_kernel");
+        }
+    }
+    if (wf) bh_free(wf);
+    if (col) bh_free(col);
+    bh_free(dyp);
     return rc;
 }
 

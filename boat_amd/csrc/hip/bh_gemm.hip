@@ -418,6 +418,26 @@ __global__ __launch_bounds__(256) void splitk_fold_kernel(const float* __restric
     }
 }
 
+// many partials of a small output (a long contraction cut into hundreds of chunks): one wavefront per output element,
+// the lanes striding over the partials
+__global__ __launch_bounds__(256) void splitk_fold_wide_kernel(const float* __restrict__ ws, float* __restrict__ c,
+                                                               const float* __restrict__ bias, int64_t m, int64_t n, int64_t ldc,
+                                                               int splits, int64_t batch_count, int64_t stride_c, int accumulate) {
+    const int lane = threadIdx.x & 63;
+    const int64_t per = m * n, total = per * batch_count;
+    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= total) return;
+    const int64_t bt = i / per, rem = i % per, row = rem / n, col = rem % n;
+    float acc = 0.f;
+    for (int s = lane; s < splits; s += 64) acc += ws[((int64_t)s * batch_count + bt) * per + rem];
+    acc = wave_sum(acc);
+    if (lane == 0) {
+        float* dst = c + bt * stride_c + row * ldc + col;
+        if (bias) acc += bias[col];
+        *dst = accumulate ? *dst + acc : acc;
+    }
+}
+
 // ---- small problems: one trip to memory per workgroup ----
 // A 64x64 output tile per workgroup (four wavefronts, one 32x32 accumulator each) and a k-chunk of at most kSmallK
 // that is loaded WHOLE into LDS before the first MFMA: a tiny GEMM is bound by the number of dependent round trips to
@@ -642,6 +662,22 @@ static int launch_small(int kch, const GemmArgs& g, dim3 grid, size_t lds) {
     return launch_small_one<A_KFAST, B_KFAST, kSmallK>(g, grid, lds);
 }
 
+// fold `splits` partial results in ws into c (one launch)
+static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, int64_t n, int64_t ldc, int splits, int64_t batch,
+                       int64_t stride_c, int accumulate) {
+    const int64_t total = m * n * batch;
+    if (splits >= 32 && total <= 16384) {
+        hipLaunchKernelGGL(splitk_fold_wide_kernel, dim3((unsigned)ceil_div(total, 4)), dim3(256), 0, stream(), ws, c, bias, m, n, ldc,
+                           splits, batch, stride_c, accumulate);
+    } else {
+        int64_t blocks = ceil_div(total, 256);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), ws, c, bias, m, n, ldc, splits, batch,
+                           stride_c, accumulate);
+    }
+    return BH_LAUNCH_CHECK("splitk_fold_kernel");
+}
+
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
 static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, -1 = heuristic
 
@@ -735,13 +771,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
             return lrc;
         }
         int rc = BH_LAUNCH_CHECK("gemm_small_kernel");
-        if (rc == BH_OK && g.k_splits > 1) {
-            int64_t blocks = ceil_div(m * n * batch, 256);
-            if (blocks > 4096) blocks = 4096;
-            hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), ws, c, bias, m, n, ldc,
-                               g.k_splits, batch, g.stride_c, accumulate);
-            rc = BH_LAUNCH_CHECK("splitk_fold_kernel");
-        }
+        if (rc == BH_OK && g.k_splits > 1) rc = launch_fold(ws, c, bias, m, n, ldc, g.k_splits, batch, g.stride_c, accumulate);
         if (ws) bh_free(ws);
         return rc;
     }
@@ -793,13 +823,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         case 4: rc = launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc, direct); break;
         default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc, direct); break;
     }
-    if (rc == BH_OK && g.k_splits > 1) {
-        int64_t blocks = ceil_div(m * n * batch, 256);
-        if (blocks > 4096) blocks = 4096;
-        hipLaunchKernelGGL(splitk_fold_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), ws, c, bias, m, n, ldc,
-                           g.k_splits, batch, g.stride_c, accumulate);
-        rc = BH_LAUNCH_CHECK("splitk_fold_kernel");
-    }
+    if (rc == BH_OK && g.k_splits > 1) rc = launch_fold(ws, c, bias, m, n, ldc, g.k_splits, batch, g.stride_c, accumulate);
     if (ws) bh_free(ws);
     return rc;
 }

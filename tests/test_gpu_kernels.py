@@ -559,3 +559,37 @@ def test_device_to_device_copy(hip, rng, n, offset):
     assert not got[:offset].any() and not got[offset + n:].any()
     hip.check(hip.bh_memcpy_d2d(d_dst.ptr + 1, d_src.ptr + 1, 6))          # not whole floats: runtime copy
     assert np.array_equal(d_dst.numpy().view(np.uint8)[1:7], src.view(np.uint8)[1:7])
+
+
+def test_gemm_random_sweep_with_padded_leading_dimensions(hip):
+    """Seeded sweep over shapes, layouts, epilogues and leading dimensions wider than the rows (every kernel behind
+    bh_gemm must honour lda / ldb / ldc), against float64."""
+    rng = np.random.default_rng(4242)
+    dims = [1, 3, 4, 16, 31, 64, 100, 128, 192, 256, 260, 384, 512, 700]
+    ks = [1, 5, 16, 32, 48, 100, 128, 256, 400, 1024]
+    for case in range(80):
+        m, n, k = (int(rng.choice(dims)), int(rng.choice(dims)), int(rng.choice(ks)))
+        ta, tb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        pad_a, pad_b, pad_c = (int(rng.choice([0, 0, 4, 8, 3])) for _ in range(3))
+        accumulate, bias = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        ra, ca = (k, m) if ta else (m, k)
+        rb, cb = (n, k) if tb else (k, n)
+        a = rng.standard_normal((ra, ca + pad_a)).astype(np.float32)
+        b = rng.standard_normal((rb, cb + pad_b)).astype(np.float32)
+        c0 = rng.standard_normal((m, n + pad_c)).astype(np.float32)
+        bv = rng.standard_normal(n).astype(np.float32)
+        A = a[:, :ca].T if ta else a[:, :ca]
+        B = b[:, :cb].T if tb else b[:, :cb]
+        want = A.astype(np.float64) @ B.astype(np.float64)
+        if bias:
+            want = want + bv
+        if accumulate:
+            want = want + c0[:, :n]
+        dc = dev(hip, c0)
+        hip.check(hip.bh_gemm(ta, tb, m, n, k, dev(hip, a).ptr, ca + pad_a, dev(hip, b).ptr, cb + pad_b, dc.ptr, n + pad_c,
+                              dev(hip, bv).ptr if bias else None, int(accumulate), 1))
+        got = dc.numpy()
+        tag = (case, ta, tb, m, n, k, pad_a, pad_b, pad_c, accumulate, bias)
+        assert rel_fro(got[:, :n], want) <= TOL_GEMM, tag
+        assert np.array_equal(got[:, n:], c0[:, n:]), tag            # the padding of C is never written
+        _KEEP.clear()

@@ -104,6 +104,9 @@ _SIGS = {
     "boat_flatten_layer_create": (P, []), "boat_flatten_layer_free": (None, [P]),
     "boat_flatten_layer_forward": (P, [P, P]), "boat_flatten_layer_backward": (P, [P, P]),
     "boat_var_conv": (P, [P, P]), "boat_var_pool": (P, [P, P]), "boat_var_flatten": (P, [P]),
+    # loss objects
+    "boat_mse_loss_create": (P, []), "boat_cross_entropy_loss_create": (P, []), "boat_huber_loss_create": (P, [C.c_float]),
+    "boat_loss_compute": (C.c_float, [P, P, P]), "boat_loss_free": (None, [P]),
     # learning-rate schedulers
     "boat_step_lr_scheduler_create": (P, [C.c_float, C.c_int, C.c_float]),
     "boat_cosine_annealing_scheduler_create": (P, [C.c_float, C.c_int, C.c_float]),

@@ -267,7 +267,45 @@ __global__ __launch_bounds__(kRBlock) void sse_partial_kernel(const float* p, co
     float s = block_sum<kRBlock / 64>(acc, red);
     if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
+// per-element loss terms of the reference's loss objects, summed: kind 0 (p-t)^2 (src/loss/mse.c:72-76),
+// 1 t*logf(clip(p, 1e-7, 1-1e-7)) (src/loss/cross_entropy.c:35-44, 91-95), 2 Huber with threshold delta (src/loss/huber.c)
+__global__ __launch_bounds__(kRBlock) void loss_terms_partial_kernel(int kind, const float* p, const float* t, float* partial,
+                                                                     int64_t n, float delta) {
+    __shared__ float red[kRBlock / 64];
+    float acc = 0.f;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const float pv = p[i], tv = t[i];
+        if (kind == 0) {
+            const float d = pv - tv;
+            acc += d * d;
+        } else if (kind == 1) {
+            const float eps = 1e-7f;
+            const float c = pv < eps ? eps : (pv > 1.0f - eps ? 1.0f - eps : pv);
+            acc += tv * logf(c);
+        } else {
+            const float d = fabsf(pv - tv);
+            acc += d <= delta ? 0.5f * d * d : delta * (d - 0.5f * delta);
+        }
+    }
+    float s = block_sum<kRBlock / 64>(acc, red);
+    if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
 }  // namespace bh
+
+extern "C" int bh_loss_terms_sum(int kind, const float* pred, const float* target, float* sum_out, int64_t n, float delta) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(kind >= 0 && kind <= 2 && n >= 0 && sum_out && ((pred && target) || n == 0), "bad argument");
+    int blocks = (int)bh::ceil_div(n > 0 ? n : 1, (int64_t)bh::kRBlock * 8);
+    if (blocks > 1024) blocks = 1024;
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);
+    if (!partial) return BH_ENOMEM;
+    hipLaunchKernelGGL(bh::loss_terms_partial_kernel, dim3(blocks), dim3(bh::kRBlock), 0, bh::stream(), kind, pred, target,
+                       partial, n, delta);
+    hipLaunchKernelGGL(bh::sum_final_kernel, dim3(1), dim3(bh::kRBlock), 0, bh::stream(), partial, sum_out, blocks, 1.0f);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK("bh_loss_terms_sum");
+}
 
 extern "C" int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n) {
     BH_REQUIRE_INIT();

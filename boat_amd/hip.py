@@ -64,6 +64,7 @@ _SIGS = {
     "bh_maxpool2d_forward": (I, [P, P, P] + [L] * 6),
     "bh_maxpool2d_backward": (I, [P, P, P] + [L] * 6),
     "bh_zero_multi": (I, [C.POINTER(P), C.POINTER(L), I]),
+    "bh_loss_terms_sum": (I, [I, P, P, P, L, F]),
     "bh_rmsprop_update": (I, [P, P, P, L, F, F, F]),
     "bh_adagrad_update": (I, [P, P, P, L, F, F]),
     "bh_adam_update_multi": (I, [C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(P), C.POINTER(L), I, F, F, F, F, L]),

@@ -308,6 +308,16 @@ BOAT_API void boat_optimizer_add_parameter(boat_optimizer_t* optimizer, boat_ten
 BOAT_API float boat_optimizer_get_learning_rate(const boat_optimizer_t* optimizer);
 BOAT_API void boat_optimizer_set_learning_rate(boat_optimizer_t* optimizer, float learning_rate);
 
+/* ---- include/boat/loss.h:12-27 (loss values; the reference has no loss-gradient function) ---- */
+typedef enum { BOAT_LOSS_MSE, BOAT_LOSS_CROSS_ENTROPY, BOAT_LOSS_HUBER } boat_loss_type_t;
+typedef struct boat_loss_t boat_loss_t;
+BOAT_API boat_loss_t* boat_mse_loss_create(void);
+BOAT_API boat_loss_t* boat_cross_entropy_loss_create(void);
+BOAT_API boat_loss_t* boat_huber_loss_create(float delta);
+/* predictions and targets are boat_tensor_t*; returns the mean loss on the host (waits for the device) */
+BOAT_API float boat_loss_compute(boat_loss_t* loss, const void* predictions, const void* targets);
+BOAT_API void boat_loss_free(boat_loss_t* loss);
+
 /* ---- include/boat/schedulers.h:15-52 (learning-rate schedulers; host arithmetic, one float per step) ---- */
 typedef enum { BOAT_SCHEDULER_STEP_LR, BOAT_SCHEDULER_COSINE_ANNEALING, BOAT_SCHEDULER_LAMBDA_LR } boat_scheduler_type_t;
 typedef struct boat_scheduler_t boat_scheduler_t;

@@ -90,6 +90,9 @@ int bh_activation_backward(int act, const float* saved, const float* dy, float* 
 
 int bh_bias_add_rows(float* y, const float* bias, int64_t rows, int64_t cols);        /* dense.c:180-184 */
 int bh_mse_grad(const float* pred, const float* target, float* grad, int64_t n);      /* tests/test_attention_training.c:28-41 */
+/* sum over the elements of the loss terms of the reference's loss objects (src/loss/mse.c, cross_entropy.c, huber.c):
+ * kind 0 (p-t)^2, 1 t*logf(clip(p, 1e-7, 1-1e-7)), 2 Huber(|p-t|, delta); sum_out is one float in device memory */
+int bh_loss_terms_sum(int kind, const float* pred, const float* target, float* sum_out, int64_t n, float delta);
 int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n);  /* src/loss/mse.c:70-78 */
 int bh_sgd_update(float* p, float* g, float lr, int64_t n, int zero_grad);            /* dense.c:297-329 */
 

@@ -539,6 +539,32 @@ void bo_maxpool2d_backward(const float* dy, const int64_t* argmax, float* dx, in
         if (argmax[i] >= 0 && argmax[i] < n_in) dx[argmax[i]] += dy[i];
 }
 
+/* ------------------------------------------------------------------ losses */
+
+/* mean loss of the reference's loss objects, fp32 left-to-right sums: kind 0 src/loss/mse.c:70-80, kind 1
+ * src/loss/cross_entropy.c:35-44,86-98 (returns the negated mean), kind 2 src/loss/huber.c (threshold delta) */
+float bo_loss_value(int kind, const float* p, const float* t, int64_t n, float delta) {
+    float sum = 0.0f;
+    for (int64_t i = 0; i < n; i++) {
+        if (kind == 0) {
+            float diff = p[i] - t[i];
+            sum += diff * diff;
+        } else if (kind == 1) {
+            const float eps = 1e-7f;
+            float c = p[i];
+            if (c < eps) c = eps;
+            else if (c > 1.0f - eps) c = 1.0f - eps;
+            sum += t[i] * logf(c);
+        } else {
+            float diff = fabsf(p[i] - t[i]);
+            if (diff <= delta) sum += 0.5f * diff * diff;
+            else sum += delta * (diff - 0.5f * delta);
+        }
+    }
+    const float mean = sum / (size_t)n;
+    return kind == 1 ? -mean : mean;
+}
+
 /* src/optimizers/rmsprop.c:197-210 */
 void bo_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps) {
     for (int64_t i = 0; i < n; i++) {

@@ -122,6 +122,9 @@ void bo_maxpool2d_forward(const float* x, float* y, int64_t* argmax, int64_t pla
                           int64_t pool, int64_t stride, int64_t pad);
 void bo_maxpool2d_backward(const float* dy, const int64_t* argmax, float* dx, int64_t n_in, int64_t n_out);
 
+/* src/loss/mse.c:37-88, cross_entropy.c:48-104, huber.c: kind 0 MSE, 1 cross entropy over probabilities, 2 Huber(delta). */
+float bo_loss_value(int kind, const float* p, const float* t, int64_t n, float delta);
+
 /* src/optimizers/rmsprop.c:181-211 and src/optimizers/adagrad.c:167-197: one tensor, one step. */
 void bo_rmsprop_update(float* p, const float* g, float* sq, int64_t n, float lr, float alpha, float eps);
 void bo_adagrad_update(float* p, const float* g, float* sum, int64_t n, float lr, float eps);

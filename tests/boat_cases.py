@@ -522,3 +522,22 @@ def scheduler_trajectory(api, kind, base_lr, steps, **kw):
     out.append((np.float32(api.boat_scheduler_get_next_lr(s)), np.float32(api.boat_scheduler_get_last_lr(s))))
     api.boat_scheduler_free(s)
     return np.array(out, np.float32)
+
+
+def loss_values(api, kind, pred, target, delta=1.0):
+    """boat_loss_compute of a fresh loss object, called twice (the object keeps running totals; the value must not
+    depend on them).  kind: "mse", "ce" or "huber".  Returns the two values, or None when creation is refused."""
+    if kind == "mse":
+        loss = api.boat_mse_loss_create()
+    elif kind == "ce":
+        loss = api.boat_cross_entropy_loss_create()
+    else:
+        loss = api.boat_huber_loss_create(delta)
+    if not loss:
+        return None
+    tp, tt = api.tensor(np.asarray(pred, np.float32)), api.tensor(np.asarray(target, np.float32))
+    vals = (api.boat_loss_compute(loss, tp, tt), api.boat_loss_compute(loss, tp, tt))
+    api.boat_tensor_unref(tp)
+    api.boat_tensor_unref(tt)
+    api.boat_loss_free(loss)
+    return vals

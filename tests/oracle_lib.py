@@ -262,6 +262,12 @@ class Oracle:
         self.lib.bo_maxpool2d_backward(fp(dy), argmax.ctypes.data_as(C.POINTER(C.c_int64)), fp(dx), L(dx.size), L(dy.size))
         return dx
 
+    def loss_value(self, kind, p, t, delta=1.0):
+        """kind: "mse", "ce" (p are probabilities) or "huber"."""
+        p, t = f32(p), f32(t)
+        self.lib.bo_loss_value.restype = C.c_float
+        return float(self.lib.bo_loss_value(C.c_int({"mse": 0, "ce": 1, "huber": 2}[kind]), fp(p), fp(t), L(p.size), C.c_float(delta)))
+
     def rmsprop_update(self, p, g, sq, lr, alpha, eps):
         """In place on copies; returns (p, sq)."""
         p, sq, g = f32(p).copy(), f32(sq).copy(), f32(g)

@@ -474,3 +474,26 @@ def test_cnn_training_with_registered_optimizer(boat):
     boat.boat_conv_layer_free(conv)
     boat.boat_pool_layer_free(pool)
     boat.boat_dense_layer_free(dense)
+
+
+@pytest.mark.parametrize("kind", ["mse", "ce", "huber"])
+@pytest.mark.parametrize("shape", [(7, 10), (64, 10), (3, 5, 1000), (1,)])
+def test_loss_objects(boat, oracle, rng, kind, shape):
+    if kind == "ce":
+        pred = rng.random(shape, dtype=np.float32)
+        pred.reshape(-1)[0] = 0.0
+        target = (rng.random(shape) < 0.2).astype(np.float32)
+    else:
+        pred = (2 * rng.standard_normal(shape)).astype(np.float32)
+        target = rng.standard_normal(shape).astype(np.float32)
+    v1, v2 = bc.loss_values(boat, kind, pred, target, 0.75)
+    want = oracle.loss_value(kind, pred, target, 0.75)
+    assert v1 == v2 and abs(v1 - want) <= TOL_RED * max(abs(want), 1e-6)
+    assert bc.loss_values(boat, "huber", pred, target, -1.0) is None
+    # shape or dtype mismatch: 0 without a message (mse.c:49-68)
+    loss = boat.boat_mse_loss_create()
+    a, b = boat.tensor(np.zeros((2, 3), np.float32)), boat.tensor(np.ones((3, 2), np.float32))
+    assert boat.boat_loss_compute(loss, a, b) == 0.0 and boat.boat_loss_compute(loss, a, None) == 0.0
+    boat.boat_tensor_unref(a)
+    boat.boat_tensor_unref(b)
+    boat.boat_loss_free(loss)

@@ -509,3 +509,31 @@ def test_cnn_chain_bit_exact(ref, oracle):
     assert np.float32(got["loss"]) == np.float32(want["loss"])
     for key in CNN_KEYS:
         assert same(want[key], got[key]), key
+
+
+# ---- loss objects (src/loss/*.c) ----
+
+@pytest.mark.parametrize("kind", ["mse", "ce", "huber"])
+def test_loss_values_bit_exact(ref, oracle, rng, kind):
+    shape = (7, 10)
+    if kind == "ce":
+        z = rng.standard_normal(shape)
+        pred = (np.exp(z) / np.exp(z).sum(1, keepdims=True)).astype(np.float32)
+        pred[0, 0], pred[0, 1] = 0.0, 1.0                      # both clip bounds
+        target = np.eye(10, dtype=np.float32)[rng.integers(0, 10, 7)]
+    else:
+        pred = (2 * rng.standard_normal(shape)).astype(np.float32)
+        target = rng.standard_normal(shape).astype(np.float32)
+    v1, v2 = bc.loss_values(ref, kind, pred, target, 0.75)
+    want = oracle.loss_value(kind, pred, target, 0.75)
+    assert np.float32(v1) == np.float32(want) and np.float32(v2) == np.float32(want)
+    # closed forms in float64
+    d = pred.astype(np.float64) - target
+    if kind == "mse":
+        assert abs(want - (d * d).mean()) <= 1e-5 * (d * d).mean()
+    elif kind == "huber":
+        a = np.abs(d)
+        assert abs(want - np.where(a <= 0.75, 0.5 * a * a, 0.75 * (a - 0.375)).mean()) <= 1e-5
+    else:
+        assert abs(want + (target * np.log(np.clip(pred.astype(np.float64), 1e-7, 1 - 1e-7))).mean()) <= 1e-5
+    assert bc.loss_values(ref, "huber", pred, target, 0.0) is None

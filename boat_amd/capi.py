@@ -104,6 +104,8 @@ _SIGS = {
     "boat_flatten_layer_create": (P, []), "boat_flatten_layer_free": (None, [P]),
     "boat_flatten_layer_forward": (P, [P, P]), "boat_flatten_layer_backward": (P, [P, P]),
     "boat_var_conv": (P, [P, P]), "boat_var_pool": (P, [P, P]), "boat_var_flatten": (P, [P]),
+    "boat_autodiff_set_grad_checkpointing": (None, [C.c_bool]), "boat_autodiff_print_graph": (None, [P]),
+    "boat_autodiff_graph_to_dot": (P, [P]), "boat_attention_set_dropout": (None, [P, C.c_float]),
     # loss objects
     "boat_mse_loss_create": (P, []), "boat_cross_entropy_loss_create": (P, []), "boat_huber_loss_create": (P, [C.c_float]),
     "boat_loss_compute": (C.c_float, [P, P, P]), "boat_loss_free": (None, [P]),

@@ -609,6 +609,96 @@ void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_outpu
     if (!grad_output) boat_tensor_unref(seed);
 }
 
+/* gradient checkpointing is a stub in the reference too (autodiff.c:652-655): every op keeps what its backward needs */
+void boat_autodiff_set_grad_checkpointing(bool enabled) { (void)enabled; }
+
+static const char* op_name(op_type_t t) {
+    static const char* names[] = {"add", "sub", "mul", "div", "relu", "sigmoid", "tanh", "matmul", "dot", "sum", "mean",
+                                  "softmax", "log_softmax", "flatten", "dense", "attention", "gelu", "layernorm", "conv", "pool"};
+    return (size_t)t < sizeof(names) / sizeof(names[0]) ? names[t] : "?";
+}
+
+/* the ops `variable` depends on, in recording order; caller frees.  (The reference declares graph printing and DOT
+ * export, autodiff.h:97-98, and leaves both empty, autodiff.c:727-736.) */
+static boat_op_t** tape_of(const boat_variable_t* variable, size_t* count) {
+    *count = 0;
+    if (!variable || !variable->producer) return NULL;
+    const uint64_t epoch = ++g_epoch;
+    size_t n = 0, cap = 64, head = 0;
+    boat_op_t** ops = (boat_op_t**)malloc(cap * sizeof(*ops));
+    if (!ops) return NULL;
+    variable->producer->mark = epoch;
+    ops[n++] = variable->producer;
+    while (head < n) {
+        boat_op_t* op = ops[head++];
+        for (size_t i = 0; i < op->num_inputs; i++) {
+            boat_variable_t* in = op->inputs[i];
+            if (!in || !in->producer || in->producer->mark == epoch) continue;
+            if (n == cap) {
+                boat_op_t** grown = (boat_op_t**)realloc(ops, 2 * cap * sizeof(*ops));
+                if (!grown) break;
+                ops = grown;
+                cap *= 2;
+            }
+            in->producer->mark = epoch;
+            ops[n++] = in->producer;
+        }
+    }
+    qsort(ops, n, sizeof(*ops), by_seq_desc);
+    for (size_t i = 0; i < n / 2; i++) {   /* ascending recording order */
+        boat_op_t* t = ops[i];
+        ops[i] = ops[n - 1 - i];
+        ops[n - 1 - i] = t;
+    }
+    *count = n;
+    return ops;
+}
+
+static int shape_text(char* buf, size_t cap, const boat_tensor_t* t) {
+    int off = snprintf(buf, cap, "[");
+    for (size_t i = 0; t && i < t->ndim && (size_t)off < cap; i++)
+        off += snprintf(buf + off, cap - (size_t)off, i ? ",%lld" : "%lld", (long long)t->shape[i]);
+    if ((size_t)off < cap) off += snprintf(buf + off, cap - (size_t)off, "]");
+    return off;
+}
+
+void boat_autodiff_print_graph(const boat_variable_t* variable) {
+    size_t n = 0;
+    boat_op_t** ops = tape_of(variable, &n);
+    if (!ops) return;
+    for (size_t i = 0; i < n; i++) {
+        char shape[128];
+        shape_text(shape, sizeof(shape), ops[i]->output ? ops[i]->output->data : NULL);
+        printf("%3zu: %-12s -> %s%s\n", i, op_name(ops[i]->type), shape,
+               ops[i]->output && ops[i]->output->requires_grad ? " (grad)" : "");
+    }
+    free(ops);
+}
+
+/* Graphviz text of the tape behind `variable` (malloc'ed; the caller frees it), NULL for a leaf */
+char* boat_autodiff_graph_to_dot(const boat_variable_t* variable) {
+    size_t n = 0;
+    boat_op_t** ops = tape_of(variable, &n);
+    if (!ops) return NULL;
+    size_t cap = 256 + n * 512, off = 0;
+    char* out = (char*)malloc(cap);
+    if (!out) {
+        free(ops);
+        return NULL;
+    }
+    off += (size_t)snprintf(out + off, cap - off, "digraph boat_tape {\n");
+    for (size_t i = 0; i < n && off + 400 < cap; i++) {
+        char shape[128];
+        shape_text(shape, sizeof(shape), ops[i]->output ? ops[i]->output->data : NULL);
+        off += (size_t)snprintf(out + off, cap - off, "  v%p [label=\"%s %s\"];\n", (void*)ops[i]->output, op_name(ops[i]->type), shape);
+        for (size_t j = 0; j < ops[i]->num_inputs; j++)
+            off += (size_t)snprintf(out + off, cap - off, "  v%p -> v%p;\n", (void*)ops[i]->inputs[j], (void*)ops[i]->output);
+    }
+    snprintf(out + off, cap - off, "}\n");
+    free(ops);
+    return out;
+}
+
 void boat_variable_backward_full(const boat_variable_t* variable) {
     if (!variable || !variable->requires_grad) return;
     boat_variable_backward((boat_variable_t*)variable, NULL);

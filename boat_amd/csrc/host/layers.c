@@ -562,6 +562,11 @@ void boat_attention_update(boat_attention_t* a, float lr) {
     sgd_step(a->bias_o, a->grad_bias_o, lr, false);
 }
 
+/* stored only: the reference's forward ignores dropout as well (attention.c:1061-1062) */
+void boat_attention_set_dropout(boat_attention_t* a, float dropout_prob) {
+    if (a) a->config.dropout_prob = dropout_prob;
+}
+
 void boat_attention_set_causal(boat_attention_t* a, bool causal) {
     if (a) a->config.causal_mask = causal;
 }

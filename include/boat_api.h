@@ -149,6 +149,9 @@ BOAT_API boat_variable_t* boat_var_div(const boat_variable_t* a, const boat_vari
 BOAT_API boat_variable_t* boat_var_matmul(const boat_variable_t* a, const boat_variable_t* b);
 BOAT_API boat_variable_t* boat_var_dot(const boat_variable_t* a, const boat_variable_t* b);
 BOAT_API boat_variable_t* boat_var_flatten(const boat_variable_t* input);
+BOAT_API void boat_autodiff_set_grad_checkpointing(bool enabled);               /* no effect, as in the reference (autodiff.c:652-655) */
+BOAT_API void boat_autodiff_print_graph(const boat_variable_t* variable);        /* lists the ops behind `variable` (empty in the reference, autodiff.c:727-730) */
+BOAT_API char* boat_autodiff_graph_to_dot(const boat_variable_t* variable);      /* malloc'ed Graphviz text, NULL for a leaf (returns NULL in the reference, :732-736) */
 BOAT_API boat_variable_t* boat_var_dense(const boat_variable_t* input, const struct boat_dense_layer_t* layer);
 BOAT_API boat_variable_t* boat_var_conv(const boat_variable_t* input, const struct boat_conv_layer_t* layer);
 BOAT_API boat_variable_t* boat_var_pool(const boat_variable_t* input, const struct boat_pool_layer_t* layer);
@@ -270,6 +273,7 @@ BOAT_API bool boat_attention_backward(boat_attention_t* attention, const boat_te
                                       boat_tensor_t** grad_query, boat_tensor_t** grad_key, boat_tensor_t** grad_value);
 BOAT_API void boat_attention_update(boat_attention_t* attention, float learning_rate);
 BOAT_API void boat_attention_set_causal(boat_attention_t* attention, bool causal);
+BOAT_API void boat_attention_set_dropout(boat_attention_t* attention, float dropout_prob);   /* stored, not applied (attention.c:1061-1062) */
 BOAT_API boat_tensor_t* boat_attention_get_weight_q(const boat_attention_t* attention);
 BOAT_API boat_tensor_t* boat_attention_get_weight_k(const boat_attention_t* attention);
 BOAT_API boat_tensor_t* boat_attention_get_weight_v(const boat_attention_t* attention);

@@ -497,3 +497,22 @@ def test_loss_objects(boat, oracle, rng, kind, shape):
     boat.boat_tensor_unref(a)
     boat.boat_tensor_unref(b)
     boat.boat_loss_free(loss)
+
+
+def test_tape_listing_and_dot_export(boat, rng):
+    a = bc._var(boat, rng.standard_normal((2, 3)).astype(np.float32), True)
+    b = bc._var(boat, rng.standard_normal((2, 3)).astype(np.float32), True)
+    c = boat.boat_var_mul(a, b)
+    d = boat.boat_var_relu(c)
+    e = boat.boat_var_sum(d, None, 0, False)
+    dot = boat.boat_autodiff_graph_to_dot(e)
+    text = C.string_at(dot).decode()
+    C.CDLL(None).free(C.c_void_p(dot))
+    assert text.startswith("digraph") and text.count("->") == 4 and "mul [2,3]" in text and "sum [1]" in text
+    assert text.index("mul") < text.index("relu") < text.index("sum")       # recording order
+    assert not boat.boat_autodiff_graph_to_dot(a) and not boat.boat_autodiff_graph_to_dot(None)
+    boat.boat_autodiff_print_graph(e)
+    boat.boat_autodiff_print_graph(None)
+    boat.boat_autodiff_set_grad_checkpointing(True)
+    for v in (e, d, c, b, a):
+        boat.boat_variable_free(v)

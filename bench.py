@@ -125,6 +125,21 @@ def bench_dense_backward(hip, steps, warmup):
     }
 
 
+def bench_dense_forward(hip, steps, warmup):
+    """Dense forward at the config-2 shape: Y = X.W + b, one GEMM with the bias in its epilogue."""
+    M, K, N = 8192, 4096, 4096
+    rng = np.random.default_rng(20250108)
+    X = hip.to_device(rng.standard_normal((M, K), dtype=np.float32))
+    W = hip.to_device((0.02 * rng.standard_normal((K, N), dtype=np.float32)).astype(np.float32))
+    b = hip.to_device(rng.standard_normal(N, dtype=np.float32))
+    Y = hip.empty((M, N))
+    ms = time_steps(hip, lambda: hip.check(hip.bh_gemm(0, 0, M, N, K, X.ptr, K, W.ptr, N, Y.ptr, N, b.ptr, 0, 1)), steps, warmup)
+    flops = 2.0 * M * K * N
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"dense_fwd_8192x4096x4096": {"ms": round(ms, 4), "bound": "mfma", "achieved_TFLOPs": round(tf, 2),
+                                         "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "flops": flops}}
+
+
 def bench_adam(hip, steps, warmup):
     """Config 5b: flat fused Adam over 268,435,456 parameters (28 B/param)."""
     out = {}
@@ -183,6 +198,18 @@ def bench_ln_gelu(hip, steps, warmup):
     gbs = nbytes / (ms * 1e-3) / 1e9
     out["gelu_bwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
                                   "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    # forward kernels of the same layers: LayerNorm forward emitting mean / rstd (read x, write y) and GELU forward
+    ms = time_steps(hip, lambda: hip.check(hip.bh_layernorm_forward(x.ptr, gamma.ptr, beta.ptr, y.ptr, mean.ptr, rstd.ptr, R, H, 1e-5)),
+                    steps, warmup)
+    nbytes = 2 * 4 * R * H + 4 * (2 * H + 2 * R)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out["layernorm_fwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
+                                       "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    ms = time_steps(hip, lambda: hip.check(hip.bh_activation_forward(hip.ACT_GELU, x.ptr, dx.ptr, R * H)), steps, warmup)
+    nbytes = 2 * 4 * R * H
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out["gelu_fwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
+                                  "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
     # streaming copy of known size (read 256 MiB, write 256 MiB): the practical HBM ceiling on this part and the
     # calibration kernel for the FETCH_SIZE / WRITE_SIZE counters
     ms = time_steps(hip, lambda: hip.check(hip.bh_scalar_op(2, x.ptr, 1.0, dx.ptr, R * H)), steps, warmup)
@@ -203,6 +230,12 @@ def bench_sdpa(hip, steps, warmup):
     o, lse = hip.empty((bh_, S, D)), hip.empty((bh_, S))
     scale = 1.0 / 8.0
     hip.check(hip.bh_sdpa_forward(q.ptr, k.ptr, vv.ptr, scale, 0, o.ptr, lse.ptr, None, bh_, S, D))
+    ms = time_steps(hip, lambda: hip.check(hip.bh_sdpa_forward(q.ptr, k.ptr, vv.ptr, scale, 0, o.ptr, lse.ptr, None, bh_, S, D)),
+                    steps, warmup)
+    flops = 2 * 2.0 * bh_ * S * S * D
+    tf = flops / (ms * 1e-3) / 1e12
+    out["sdpa_fwd_B8h16S1024D64"] = {"ms": round(ms, 4), "bound": "mfma", "achieved_TFLOPs": round(tf, 2),
+                                     "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "flops": flops}
     dq, dk, dv = hip.empty((bh_, S, D)), hip.empty((bh_, S, D)), hip.empty((bh_, S, D))
     ms = time_steps(hip, lambda: hip.check(hip.bh_sdpa_backward(q.ptr, k.ptr, vv.ptr, o.ptr, lse.ptr, go.ptr, scale, 0, dq.ptr, dk.ptr,
                                                                 dv.ptr, bh_, S, D)), steps, warmup)
@@ -455,6 +488,8 @@ def main():
                      "roofline": main_res["roofline"], "step_tflops": main_res["step_tflops"],
                      "wall_ms_per_step": round(main_res["wall_ms_per_step"], 4)})
     extra = {}
+    if "dense" in legs:
+        extra.update(bench_dense_forward(hip, args.steps, args.warmup))
     if "adam" in legs:
         extra.update(bench_adam(hip, args.steps, args.warmup))
     if "ln_gelu" in legs:

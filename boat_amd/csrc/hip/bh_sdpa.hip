@@ -11,7 +11,8 @@
 // Two implementations behind one entry point:
 //   * general kernels (any s, d): one workgroup per query row (forward, dQ) or per key row
 //     (dK, dV); scores of one row live in LDS.
-//   * MFMA kernels for d == 64 and s % 64 == 0 (the shapes of the attention benchmarks).
+//   * MFMA kernels for d == 64 and s >= 32 (the shapes of the attention benchmarks; a length that is not a
+//     multiple of 128 is handled by clamped loads, masked scores and guarded stores).
 #include "bh_common.h"
 
 #include <float.h>

@@ -1,4 +1,4 @@
-// bh_sdpa_mfma.hip - attention core on the fp32 matrix cores for head_dim 64 (seq % 128 == 0).
+// bh_sdpa_mfma.hip - attention core on the fp32 matrix cores for head_dim 64, any sequence length from 32 up.
 //
 // Same mathematics as the reference's scaled_dot_product_attention_impl / attention_backward
 // (src/layers/attention.c:997-1073, 1417-1520) on one [s, 64] block per (batch, head):
@@ -47,7 +47,7 @@ __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + 
 
 // ------------------------------------------------------------------ forward
 // grid (s/128, bh); 4 wavefronts, each owns 32 queries; key/value tiles of 64 rows double-buffered in LDS.
-template <bool CAUSAL>
+template <bool CAUSAL, bool RAGGED>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
 __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ out,
                                                             float* __restrict__ lse, int s, float scale_log2e) {
@@ -61,12 +61,13 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
     const float* vh = v + head * s * kD;
     const int q0 = blockIdx.x * 128 + w * 32;    // first query of this wavefront
     const int my_q = q0 + r;
+    const int ld_q = RAGGED ? min(my_q, s - 1) : my_q;
 
     // this lane's query row, pre-scaled so that scores come out in log2 units: step (g, e) <-> d = 8g + 4*half + e
     float qreg[32];
 #pragma unroll
     for (int g = 0; g < 8; g++) {
-        const float4 t = *reinterpret_cast<const float4*>(qh + (int64_t)my_q * kD + 8 * g + 4 * half);
+        const float4 t = *reinterpret_cast<const float4*>(qh + (int64_t)ld_q * kD + 8 * g + 4 * half);
         qreg[4 * g + 0] = t.x * scale_log2e;
         qreg[4 * g + 1] = t.y * scale_log2e;
         qreg[4 * g + 2] = t.z * scale_log2e;
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
     floatx16 acc_o[2] = {zero16(), zero16()};    // O^T: [d tile][...]; d = 2*row + tile, query = lane
     float m_run = -INFINITY, l_run = 0.f;
 
-    int n_tiles = s / KT;
+    int n_tiles = RAGGED ? (s + KT - 1) / KT : s / KT;
     if (CAUSAL) {
         const int last = (blockIdx.x * 128 + 127) / KT + 1;   // tiles that hold a key <= the last query of the workgroup
         if (last < n_tiles) n_tiles = last;
@@ -86,8 +87,9 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
 #define FWD_LD(i, K, V)                                                                                   \
     {                                                                                                     \
         const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
-        K = *reinterpret_cast<const float4*>(kh + (int64_t)(jt_ld * KT + row) * kD + c4 * 4);             \
-        V = *reinterpret_cast<const float4*>(vh + (int64_t)(jt_ld * KT + row) * kD + c4 * 4);             \
+        const int grow = RAGGED ? min(jt_ld * KT + row, s - 1) : jt_ld * KT + row;                        \
+        K = *reinterpret_cast<const float4*>(kh + (int64_t)grow * kD + c4 * 4);                           \
+        V = *reinterpret_cast<const float4*>(vh + (int64_t)grow * kD + c4 * 4);                           \
     }
 #define FWD_ST(i, K, V)                                                                                   \
     {                                                                                                     \
@@ -128,9 +130,9 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
-                    if (CAUSAL) {
+                    if (CAUSAL || RAGGED) {
                         const int key = jt * KT + t * 32 + acc_row(e, half);
-                        if (key > my_q) acc_s[t][e] = -INFINITY;
+                        if ((CAUSAL && key > my_q) || (RAGGED && key >= s)) acc_s[t][e] = -INFINITY;
                     }
                     mx = fmaxf(mx, acc_s[t][e]);
                 }
@@ -187,9 +189,9 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
     for (int it = 0; it < 8; it++) {
         const int row = it * 4 + (lane >> 4), c4 = lane & 15;
         const float4 val = *reinterpret_cast<const float4*>(os + row * kLd + c4 * 4);
-        *reinterpret_cast<float4*>(oh + (int64_t)(q0 + row) * kD + c4 * 4) = val;
+        if (!RAGGED || q0 + row < s) *reinterpret_cast<float4*>(oh + (int64_t)(q0 + row) * kD + c4 * 4) = val;
     }
-    if (half == 0) lse[head * s + my_q] = (m_run + log2f(l_run)) * kLn2;
+    if (half == 0 && (!RAGGED || my_q < s)) lse[head * s + my_q] = (m_run + log2f(l_run)) * kLn2;
 }
 
 // ----------------------------------------------------------------- backward
@@ -219,7 +221,7 @@ struct BwdSmem {
     static constexpr int TOTAL = OFF_STAT + 64;
 };
 
-template <bool CAUSAL>
+template <bool CAUSAL, bool RAGGED>
 __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                const float* __restrict__ v, const float* __restrict__ lse,
                                                                const float* __restrict__ delta, const float* __restrict__ d_out,
@@ -251,19 +253,19 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const int idx = lane + i * 64, row = idx >> 4, c4 = idx & 15;
-        *reinterpret_cast<float4*>(ks + row * kLd + c4 * 4) =
-            *reinterpret_cast<const float4*>(kh + (int64_t)(kv0 + row) * kD + c4 * 4);
+        const int grow = RAGGED ? min(kv0 + row, s - 1) : kv0 + row;
+        *reinterpret_cast<float4*>(ks + row * kLd + c4 * 4) = *reinterpret_cast<const float4*>(kh + (int64_t)grow * kD + c4 * 4);
     }
     // this lane's slice of V: key kv0 + r, head-dim 8g + 4*half .. +3 for g = 0..7
     float4 vreg[8];
 #pragma unroll
     for (int g = 0; g < 8; g++)
-        vreg[g] = *reinterpret_cast<const float4*>(vh + (int64_t)(kv0 + r) * kD + 8 * g + 4 * half);
+        vreg[g] = *reinterpret_cast<const float4*>(vh + (int64_t)(RAGGED ? min(kv0 + r, s - 1) : kv0 + r) * kD + 8 * g + 4 * half);
 
     floatx16 acc_dk[2] = {zero16(), zero16()};   // [d tile]: key = acc_row, d = 2*lane + tile
     floatx16 acc_dv[2] = {zero16(), zero16()};
 
-    const int n_qt = s / 32;
+    const int n_qt = RAGGED ? (s + 31) / 32 : s / 32;
     const int first_qt = CAUSAL ? kv_wg / 32 : 0;   // earlier query tiles see none of this workgroup's keys
     // their partial dQ rows are zero
     for (int i = tid; i < first_qt * 32 * (kD / 4); i += 256)
@@ -274,8 +276,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
 #define BWD_LD(i, Q, G)                                                                                   \
     {                                                                                                     \
         const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
-        Q = *reinterpret_cast<const float4*>(qh + (int64_t)(qt_ld * 32 + row) * kD + c4 * 4);             \
-        G = *reinterpret_cast<const float4*>(gh + (int64_t)(qt_ld * 32 + row) * kD + c4 * 4);             \
+        const int grow = RAGGED ? min(qt_ld * 32 + row, s - 1) : qt_ld * 32 + row;                        \
+        Q = *reinterpret_cast<const float4*>(qh + (int64_t)grow * kD + c4 * 4);                           \
+        G = *reinterpret_cast<const float4*>(gh + (int64_t)grow * kD + c4 * 4);                           \
     }
 #define BWD_ST(i, Q, G)                                                                                   \
     {                                                                                                     \
@@ -287,8 +290,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     {                                                                      \
         const int qt_ld = (QT);                                            \
         BWD_LD(0, qst0, gst0) BWD_LD(1, qst1, gst1)                        \
-        if (tid < 32) stat = lh[qt_ld * 32 + tid] * kLog2e;                \
-        else if (tid < 64) stat = dh[qt_ld * 32 + tid - 32];               \
+        if (tid < 32) stat = lh[RAGGED ? min(qt_ld * 32 + tid, s - 1) : qt_ld * 32 + tid] * kLog2e;                \
+        else if (tid < 64) stat = dh[RAGGED ? min(qt_ld * 32 + tid - 32, s - 1) : qt_ld * 32 + tid - 32];          \
     }
 #define BWD_STAGE_STORE()                                                  \
     {                                                                      \
@@ -330,6 +333,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                 const int row = acc_row(e, half);
                 float p = __builtin_amdgcn_exp2f(acc_s[e] * c1 - st[row]);
                 if (CAUSAL && kv0 + r > q0 + row) p = 0.f;
+                if (RAGGED && (kv0 + r >= s || q0 + row >= s)) p = 0.f;   // padding keys and queries carry no probability
                 acc_s[e] = p;
                 acc_dp[e] = p * (acc_dp[e] - st[32 + row]) * scale;
             }
@@ -375,10 +379,12 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
             acc_dq1 = MFMA16(b3, a1.w, acc_dq1);
         }
         // accumulator register e of lane (i16, kk) is head-dim column 16w + 4*kk + e of query row i16 of the 16-row tile
-        *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk) =
-            make_float4(acc_dq0[0], acc_dq0[1], acc_dq0[2], acc_dq0[3]);
-        *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + 16 + i16) * kD + 16 * w + 4 * kk) =
-            make_float4(acc_dq1[0], acc_dq1[1], acc_dq1[2], acc_dq1[3]);
+        if (!RAGGED || q0 + i16 < s)
+            *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk) =
+                make_float4(acc_dq0[0], acc_dq0[1], acc_dq0[2], acc_dq0[3]);
+        if (!RAGGED || q0 + 16 + i16 < s)
+            *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + 16 + i16) * kD + 16 * w + 4 * kk) =
+                make_float4(acc_dq1[0], acc_dq1[1], acc_dq1[2], acc_dq1[3]);
         __syncthreads();   // dS tile free again; the next Q and dO tiles are in place
     }
 #undef BWD_LD
@@ -391,6 +397,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
 #pragma unroll
     for (int e = 0; e < 16; e++) {
         const int64_t row = kv0 + acc_row(e, half);
+        if (RAGGED && row >= s) continue;
         *reinterpret_cast<float2*>(dkh + row * kD + 2 * r) = make_float2(acc_dk[0][e], acc_dk[1][e]);
         *reinterpret_cast<float2*>(dvh + row * kD + 2 * r) = make_float2(acc_dv[0][e], acc_dv[1][e]);
     }
@@ -407,7 +414,8 @@ __global__ __launch_bounds__(256) void dq_partial_sum_kernel(const float* __rest
     __builtin_nontemporal_store(acc, reinterpret_cast<f32x4*>(out) + i);
 }
 
-static bool mfma_shape(int64_t s, int64_t d) { return d == kD && s >= 128 && s % 128 == 0 && s <= (1 << 24); }
+// head_dim 64; any sequence length from 32 up (a length that is not a multiple of 128 takes the kernels' ragged form)
+static bool mfma_shape(int64_t s, int64_t d) { return d == kD && s >= 32 && s <= (1 << 24); }
 
 int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
                       int64_t bh_count, int64_t s, int64_t d) {
@@ -417,19 +425,25 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
     constexpr size_t lds = sizeof(float) * 2 * 2 * 64 * kLd;
     static bool attr = false;
     if (!attr) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
-        if (rc == BH_OK)
-            rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
-        if (rc) return rc;
+        const void* fns[4] = {reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, false>),
+                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, false>),
+                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, true>),
+                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, true>)};
+        for (const void* fn : fns) {
+            int rc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+            if (rc) return rc;
+        }
         attr = true;
     }
-    dim3 grid((unsigned)(s / 128), (unsigned)bh_count);
-    if (causal)
-        hipLaunchKernelGGL(sdpa_fwd_mfma_kernel<true>, grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, scale * kLog2e);
-    else
-        hipLaunchKernelGGL(sdpa_fwd_mfma_kernel<false>, grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, scale * kLog2e);
+    dim3 grid((unsigned)ceil_div(s, 128), (unsigned)bh_count);
+    const bool ragged = s % 128 != 0;
+    const float sl = scale * kLog2e;
+#define FWD_LAUNCH(C, R) hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, sl)
+    if (causal && ragged) FWD_LAUNCH(true, true);
+    else if (causal) FWD_LAUNCH(true, false);
+    else if (ragged) FWD_LAUNCH(false, true);
+    else FWD_LAUNCH(false, false);
+#undef FWD_LAUNCH
     return BH_LAUNCH_CHECK("sdpa_fwd_mfma_kernel");
 }
 
@@ -442,25 +456,30 @@ int sdpa_backward_mfma(const float* q, const float* k, const float* v, const flo
     constexpr size_t lds = sizeof(float) * BwdSmem::TOTAL;
     static bool attr = false;
     if (!attr) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
-        if (rc == BH_OK)
-            rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
-        if (rc) return rc;
+        const void* fns[4] = {reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, false>),
+                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, false>),
+                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, true>),
+                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, true>)};
+        for (const void* fn : fns) {
+            int arc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+            if (arc) return arc;
+        }
         attr = true;
     }
-    const int tiles = (int)(s / 128);
+    const int tiles = (int)ceil_div(s, 128);
+    const bool ragged = s % 128 != 0;
     const int64_t n = bh_count * s * d;
     float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one key tile: dq itself
     if (!partial) return BH_ENOMEM;
     dim3 grid((unsigned)tiles, (unsigned)bh_count);
-    if (causal)
-        hipLaunchKernelGGL(sdpa_bwd_mfma_kernel<true>, grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk,
-                           dv, (int)s, scale);
-    else
-        hipLaunchKernelGGL(sdpa_bwd_mfma_kernel<false>, grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk,
-                           dv, (int)s, scale);
+#define BWD_LAUNCH(C, R)                                                                                                   \
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk, dv, \
+                       (int)s, scale)
+    if (causal && ragged) BWD_LAUNCH(true, true);
+    else if (causal) BWD_LAUNCH(true, false);
+    else if (ragged) BWD_LAUNCH(false, true);
+    else BWD_LAUNCH(false, false);
+#undef BWD_LAUNCH
     int rc = BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
     if (tiles > 1) {
         if (rc == BH_OK) {

@@ -424,7 +424,7 @@ def test_transpose(hip, oracle, rng):
 # ---------------------------------------------------------------- attention
 
 SDPA_SHAPES = [(8, 4, 8), (4, 16, 16), (2, 8, 8), (3, 33, 20), (2, 64, 64), (4, 128, 64), (2, 256, 64), (3, 100, 64),
-               (2, 512, 64), (1, 1024, 64)]
+               (2, 512, 64), (1, 1024, 64), (2, 32, 64), (2, 77, 64), (1, 129, 64), (2, 191, 64), (1, 1000, 64)]
 
 
 @pytest.mark.parametrize("causal", [0, 1])

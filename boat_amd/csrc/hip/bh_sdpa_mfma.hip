@@ -55,11 +55,16 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
     constexpr int KT = 64;                       // keys per tile
     constexpr int TILE = KT * kLd;               // floats per K or V tile in LDS
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
-    const int64_t head = blockIdx.y;
+    // Workgroups are handed out in the order of their linear id.  Read it tile-major: all heads' workgroups of one query
+    // tile are neighbours, and with a causal mask the query tile with the most keys comes first, so that the short
+    // workgroups fill the end of the launch instead of the long ones stretching it.
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int64_t head = lin % (int)gridDim.y;
+    const int bx = CAUSAL ? (int)gridDim.x - 1 - lin / (int)gridDim.y : lin / (int)gridDim.y;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
     const float* vh = v + head * s * kD;
-    const int q0 = blockIdx.x * 128 + w * 32;    // first query of this wavefront
+    const int q0 = bx * 128 + w * 32;            // first query of this wavefront
     const int my_q = q0 + r;
     const int ld_q = RAGGED ? min(my_q, s - 1) : my_q;
 
@@ -78,7 +83,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
 
     int n_tiles = RAGGED ? (s + KT - 1) / KT : s / KT;
     if (CAUSAL) {
-        const int last = (blockIdx.x * 128 + 127) / KT + 1;   // tiles that hold a key <= the last query of the workgroup
+        const int last = (bx * 128 + 127) / KT + 1;   // tiles that hold a key <= the last query of the workgroup
         if (last < n_tiles) n_tiles = last;
     }
     // global -> register staging: 1024 float4 per tile and operand, 4 per lane (macros, not lambdas:
@@ -230,7 +235,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
-    const int64_t head = blockIdx.y;
+    // tile-major reading of the linear workgroup id, as in the forward kernel: key tile 0, which meets every query tile
+    // under a causal mask, is handed out first for all heads
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int64_t head = lin % (int)gridDim.y;
+    const int bx = lin / (int)gridDim.y;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
     const float* vh = v + head * s * kD;
@@ -238,8 +247,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     const float* lh = lse + head * s;
     const float* dh = delta + head * s;
     // partial dQ of this key tile: [key tile][bh][s][64]
-    float* dqh = dq_partial + ((int64_t)blockIdx.x * gridDim.y + head) * s * kD;
-    const int kv_wg = blockIdx.x * 128;          // first key of the workgroup
+    float* dqh = dq_partial + ((int64_t)bx * gridDim.y + head) * s * kD;
+    const int kv_wg = bx * 128;          // first key of the workgroup
     const int kv0 = kv_wg + w * 32;              // first key of this wavefront
     const float c1 = scale * kLog2e;
 

@@ -43,9 +43,7 @@ struct ConvShape {
 // reference's: for each input channel a sum over the taps in (kh, kw) order, taps outside the image skipped, added to
 // the output; bias last (conv.c:398-436).  "Skipped" is a select, not a branch: a tap outside the image reads a clamped
 // (valid) address and leaves the running sum untouched.
-constexpr int kOcTile = 8;
-
-template <int K>   // kernel size (compile time: the taps live in registers)
+template <int K, int kOcTile>   // kernel size (compile time: the taps live in registers) and output channels per lane
 __global__ __launch_bounds__(kCBlock) void conv2d_fwd_kernel(const float* __restrict__ x, const float* __restrict__ wt,
                                                              const float* __restrict__ bias, float* __restrict__ y,
                                                              ConvShape c) {
@@ -72,11 +70,14 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_kernel(const float* __rest
     float out[kOcTile];
 #pragma unroll
     for (int o = 0; o < kOcTile; o++) out[o] = 0.f;
+    // The loop on input channels is software pipelined: the taps of channel ci+1 are in flight while channel ci is summed
+    // (the weights are the same for the whole workgroup and come through the scalar cache).
     const float* xp = x + (int64_t)b * c.ic * c.h * c.w;
-    for (int ci = 0; ci < c.ic; ci++, xp += c.h * c.w) {
-        float xv[K * K];
+    const int plane = c.h * c.w;
+    float xv[K * K];
 #pragma unroll
-        for (int t = 0; t < K * K; t++) xv[t] = xp[off[t]];
+    for (int t = 0; t < K * K; t++) xv[t] = xp[off[t]];
+    const auto add_channel = [&](int ci) {
 #pragma unroll
         for (int o = 0; o < kOcTile; o++) {
             const float* wp = wrow[o] + ci * K * K;
@@ -88,7 +89,16 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_kernel(const float* __rest
             }
             out[o] += sum;
         }
+    };
+    for (int ci = 0; ci + 1 < c.ic; ci++) {
+        float xn[K * K];
+#pragma unroll
+        for (int t = 0; t < K * K; t++) xn[t] = xp[(int64_t)(ci + 1) * plane + off[t]];
+        add_channel(ci);
+#pragma unroll
+        for (int t = 0; t < K * K; t++) xv[t] = xn[t];
     }
+    add_channel(c.ic - 1);
 #pragma unroll
     for (int o = 0; o < kOcTile; o++) {
         if (oc0 + o >= c.oc) break;
@@ -302,11 +312,13 @@ int bh_conv2d_forward(const float* x, const float* w, const float* bias, float* 
     if (rc) return rc;
     if (batch == 0) return BH_OK;
     BH_CHECK_ARG(x && w && y, "null pointer");
-    const dim3 grid((unsigned)ceil_div((int64_t)c.ho * c.wo, kCBlock), (unsigned)ceil_div(c.oc, kOcTile), (unsigned)c.batch);
+    // 3x3: eight output channels per lane; 5x5: four (25 taps of two channels' worth of registers already fill the file)
+    const int oc_tile = c.k == 3 ? 8 : 4;
+    const dim3 grid((unsigned)ceil_div((int64_t)c.ho * c.wo, kCBlock), (unsigned)ceil_div(c.oc, oc_tile), (unsigned)c.batch);
     if (c.k == 3 && grid.y <= 65535 && grid.z <= 65535) {
-        hipLaunchKernelGGL(conv2d_fwd_kernel<3>, grid, dim3(kCBlock), 0, stream(), x, w, bias, y, c);
+        hipLaunchKernelGGL((conv2d_fwd_kernel<3, 8>), grid, dim3(kCBlock), 0, stream(), x, w, bias, y, c);
     } else if (c.k == 5 && grid.y <= 65535 && grid.z <= 65535) {
-        hipLaunchKernelGGL(conv2d_fwd_kernel<5>, grid, dim3(kCBlock), 0, stream(), x, w, bias, y, c);
+        hipLaunchKernelGGL((conv2d_fwd_kernel<5, 4>), grid, dim3(kCBlock), 0, stream(), x, w, bias, y, c);
     } else {
         const int64_t total = (int64_t)c.batch * c.oc * c.ho * c.wo;
         hipLaunchKernelGGL(conv2d_fwd_generic_kernel, dim3((unsigned)ceil_div(total, kCBlock)), dim3(kCBlock), 0, stream(), x, w,

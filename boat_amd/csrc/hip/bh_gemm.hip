@@ -549,6 +549,81 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
     }
 }
 
+// ---- tiny problems: latency, not throughput ----
+// A problem of a few million multiply-adds (the layers of a small MLP at batch 64) is over in the time one trip to memory
+// and one chain of products take, so this kernel makes both as short as they can be: a workgroup owns a 32x32 tile of
+// C and splits the contraction among its NW wavefronts in groups of 8 (a wavefront count and fetch depth that keep the kernel
+// free of register spills: one kernel that needs scratch memory slows every later launch of the process); every lane fetches its operand values straight
+// from global memory into the registers the products read (no staging, no barrier before the arithmetic), all of a
+// wavefront's fetches in flight together; the NW partial tiles are then summed through LDS in wavefront order (so the
+// result does not depend on timing) and stored with bias and accumulation applied.  No workspace, no second launch.
+template <bool a_kfast, bool b_kfast, int NW, int U>   // wavefronts per tile; groups of 8 k one wavefront fetches together
+__global__ __launch_bounds__(64 * NW) void gemm_tiny_kernel(GemmArgs g, int a_vec, int b_vec) {
+    __shared__ float red[NW * 1024];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int tile_m = blockIdx.x % g.tiles_m, tile_n = blockIdx.x / g.tiles_m;
+    const int64_t batch = blockIdx.y;
+    const int64_t m0 = (int64_t)tile_m * 32, n0 = (int64_t)tile_n * 32;
+    // rows and columns past the edge read the last valid one: they only feed outputs that are never stored
+    const int64_t row = min(m0 + r, g.m - 1), col = min(n0 + r, g.n - 1);
+    const float* pa = g.a + batch * g.stride_a + (a_kfast ? row * g.lda : row);
+    const float* pb = g.b + batch * g.stride_b + (b_kfast ? col * g.ldb : col);
+    const int64_t sa = a_kfast ? 1 : g.lda, sb = b_kfast ? 1 : g.ldb;   // distance between consecutive k
+    const int K = (int)g.k;
+    const int groups = (K + 7) >> 3;
+
+    floatx16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.f;
+    for (int g0 = wave; g0 < groups; g0 += NW * U) {
+        float av[U][4], bv[U][4];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int kk = (g0 + u * NW) * 8 + 4 * half;      // this lane's four k of the group; may lie past K
+            if (a_kfast && a_vec) {                          // K % 4 == 0 here: kk < K implies kk + 3 < K
+                const float4 t = *reinterpret_cast<const float4*>(pa + min(kk, K - 4));
+                av[u][0] = t.x; av[u][1] = t.y; av[u][2] = t.z; av[u][3] = t.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) av[u][j] = pa[(int64_t)min(kk + j, K - 1) * sa];
+            }
+            if (b_kfast && b_vec) {
+                const float4 t = *reinterpret_cast<const float4*>(pb + min(kk, K - 4));
+                bv[u][0] = t.x; bv[u][1] = t.y; bv[u][2] = t.z; bv[u][3] = t.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) bv[u][j] = pb[(int64_t)min(kk + j, K - 1) * sb];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int kk = (g0 + u * NW) * 8 + 4 * half;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float x = kk + j < K ? av[u][j] : 0.f;   // zero one operand past the end of the contraction
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, bv[u][j], acc, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; e++) red[wave * 1024 + e * 64 + lane] = acc[e];
+    __syncthreads();
+
+    float* C = g.c + batch * g.stride_c;
+    for (int o = tid; o < 1024; o += 64 * NW) {
+        float v = red[o];
+#pragma unroll
+        for (int w = 1; w < NW; w++) v += red[w * 1024 + o];
+        const int e = o >> 6, l = o & 63;
+        const int64_t orow = m0 + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3), ocol = n0 + (l & 31);
+        if (orow < g.m && ocol < g.n) {
+            if (g.bias) v += g.bias[ocol];
+            float* dst = C + orow * g.ldc + ocol;
+            *dst = g.accumulate ? *dst + v : v;
+        }
+    }
+}
+
 // ---- fallback: bounds-checked 32x32 LDS tiles, any shape / alignment ----
 __global__ __launch_bounds__(256) void gemm_fallback_kernel(GemmArgs g, int trans_a, int trans_b) {
     __shared__ float ta[32][33];
@@ -679,7 +754,7 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
 }
 
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
-static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, -1 = heuristic
+static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, 6 = tiny, -1 = heuristic
 
 }  // namespace bh
 
@@ -740,7 +815,34 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     }
     // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
     if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
-    if (g_force_cfg >= 0 && g_force_cfg <= 5 && (vec_ok || g_force_cfg == 0 || g_force_cfg == 5)) cfg = g_force_cfg;
+    // a few million multiply-adds in at most a few hundred 32x32 tiles: the single-trip kernel without staging.  An
+    // operand whose k index is the fast one in memory makes every lane fetch from a row of its own; measured, that is
+    // only worth it while the contraction is short (k <= 128: 4-7 us against 6.5-9 us; beyond, 10-30 us against 11-14)
+    if (k > 0 && m * n * k <= ((int64_t)1 << 24) && ceil_div(m, 32) * ceil_div(n, 32) * batch <= 512 &&
+        (k <= 128 || (!a_kc && !b_kc)))
+        cfg = 6;
+    if (g_force_cfg >= 0 && g_force_cfg <= 6 && (vec_ok || g_force_cfg == 0 || g_force_cfg >= 5)) cfg = g_force_cfg;
+    if (cfg == 6 && k == 0) cfg = 5;
+
+    if (cfg == 6) {
+        g.tiles_m = (int)ceil_div(m, 32);
+        g.tiles_n = (int)ceil_div(n, 32);
+        BH_CHECK_ARG((int64_t)g.tiles_m * g.tiles_n <= 0x7fffffff && k <= 0x7ffffff0, "problem too large for the tiny-GEMM kernel");
+        // 16-byte fetches along k need the operand's rows to start on 16 bytes and k % 4 == 0
+        const int a_vec = a_kc && al16(a) && lda % 4 == 0 && k % 4 == 0 && (g.stride_a % 4 == 0 || batch == 1);
+        const int b_vec = b_kc && al16(b) && ldb % 4 == 0 && k % 4 == 0 && (g.stride_b % 4 == 0 || batch == 1);
+        const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
+        const bool wide = k > 128;    // 8 wavefronts share a long contraction, 4 a short one    // 16 wavefronts share a long contraction (one trip to memory up to k = 1024), 4 a short one
+#define TINY_LAUNCH(AK, BK)                                                                                               \
+    if (wide) hipLaunchKernelGGL((gemm_tiny_kernel<AK, BK, 8, 8>), grid, dim3(512), 0, stream(), g, a_vec, b_vec);          \
+    else hipLaunchKernelGGL((gemm_tiny_kernel<AK, BK, 4, 4>), grid, dim3(256), 0, stream(), g, a_vec, b_vec)
+        if (a_kc && b_kc) { TINY_LAUNCH(true, true); }
+        else if (a_kc) { TINY_LAUNCH(true, false); }
+        else if (b_kc) { TINY_LAUNCH(false, true); }
+        else { TINY_LAUNCH(false, false); }
+#undef TINY_LAUNCH
+        return BH_LAUNCH_CHECK("gemm_tiny_kernel");
+    }
 
     if (cfg == 5) {
         g.tiles_m = (int)ceil_div(m, 64);

@@ -374,6 +374,24 @@ def test_gemm_small_problem_kernel(hip, rng, ta, tb, m, n, k):
     gemm_case(hip, rng, ta, tb, m, n, k, force=0)                    # the bounds-checked fallback on the same shapes
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (33, 17, 5), (64, 128, 784), (64, 784, 128), (784, 128, 64), (64, 10, 128),
+                                   (128, 10, 64), (64, 128, 10), (65, 63, 129), (37, 130, 225), (200, 70, 1000), (32, 32, 4096)])
+def test_gemm_tiny_problem_kernel(hip, rng, ta, tb, m, n, k):
+    """The staging-free single-trip kernel (forced: the heuristic only picks it for a few million multiply-adds): both
+    wavefront counts, 16-byte and 4-byte fetches (k % 4), ragged tiles, k tails, bias and accumulation."""
+    gemm_case(hip, rng, ta, tb, m, n, k, force=6)
+    gemm_case(hip, rng, ta, tb, m, n, k, force=6, accumulate=True, bias=True)
+
+
+def test_gemm_tiny_problem_kernel_batched_and_deterministic(hip, rng):
+    gemm_case(hip, rng, 0, 0, 5, 4, 6, batch=6, force=6)
+    gemm_case(hip, rng, 1, 1, 70, 40, 300, batch=3, force=6, accumulate=True)
+    got1, _ = gemm_case(hip, rng := np.random.default_rng(5), 0, 1, 64, 128, 784, force=6)
+    got2, _ = gemm_case(hip, np.random.default_rng(5), 0, 1, 64, 128, 784, force=6)
+    assert np.array_equal(got1, got2)          # partial tiles are summed in wavefront order, not arrival order
+
+
 def test_gemm_small_problem_kernel_batched(hip, rng):
     gemm_case(hip, rng, 0, 0, 5, 4, 6, batch=6, force=5)
     gemm_case(hip, rng, 1, 1, 70, 40, 300, batch=3, force=5, accumulate=True)

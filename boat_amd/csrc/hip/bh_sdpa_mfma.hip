@@ -226,6 +226,8 @@ struct BwdSmem {
     static constexpr int TOTAL = OFF_STAT + 64;
 };
 
+// RAGGED: rows past s are clamped on load; padding keys are masked, padding queries contribute nothing because their
+// dO rows and delta are staged as zeros; stores are guarded
 template <bool CAUSAL, bool RAGGED>
 __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                const float* __restrict__ v, const float* __restrict__ lse,
@@ -288,6 +290,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
         const int grow = RAGGED ? min(qt_ld * 32 + row, s - 1) : qt_ld * 32 + row;                        \
         Q = *reinterpret_cast<const float4*>(qh + (int64_t)grow * kD + c4 * 4);                           \
         G = *reinterpret_cast<const float4*>(gh + (int64_t)grow * kD + c4 * 4);                           \
+        if (RAGGED && qt_ld * 32 + row >= s) G = make_float4(0.f, 0.f, 0.f, 0.f);                         \
     }
 #define BWD_ST(i, Q, G)                                                                                   \
     {                                                                                                     \
@@ -300,7 +303,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
         const int qt_ld = (QT);                                            \
         BWD_LD(0, qst0, gst0) BWD_LD(1, qst1, gst1)                        \
         if (tid < 32) stat = lh[RAGGED ? min(qt_ld * 32 + tid, s - 1) : qt_ld * 32 + tid] * kLog2e;                \
-        else if (tid < 64) stat = dh[RAGGED ? min(qt_ld * 32 + tid - 32, s - 1) : qt_ld * 32 + tid - 32];          \
+        else if (tid < 64) {                                                                                       \
+            stat = dh[RAGGED ? min(qt_ld * 32 + tid - 32, s - 1) : qt_ld * 32 + tid - 32];                         \
+            if (RAGGED && qt_ld * 32 + tid - 32 >= s) stat = 0.f;                                                  \
+        }                                                                                                          \
     }
 #define BWD_STAGE_STORE()                                                  \
     {                                                                      \
@@ -313,6 +319,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     }
     __syncthreads();
 
+    const int my_key = kv0 + r;
+    const bool key_pad = RAGGED && my_key >= s;
     for (int qt = first_qt; qt < n_qt; qt++) {
         const bool more = qt + 1 < n_qt;
         if (more) BWD_STAGE_LOAD(qt + 1)
@@ -341,8 +349,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
             for (int e = 0; e < 16; e++) {
                 const int row = acc_row(e, half);
                 float p = __builtin_amdgcn_exp2f(acc_s[e] * c1 - st[row]);
-                if (CAUSAL && kv0 + r > q0 + row) p = 0.f;
-                if (RAGGED && (kv0 + r >= s || q0 + row >= s)) p = 0.f;   // padding keys and queries carry no probability
+                // masked pairs and padding keys carry no probability (padding queries need no mask: their dO rows
+                // and delta were staged as zeros, so everything they contribute below is zero)
+                if ((CAUSAL && my_key > q0 + row) || key_pad) p = 0.f;
                 acc_s[e] = p;
                 acc_dp[e] = p * (acc_dp[e] - st[32 + row]) * scale;
             }

@@ -513,6 +513,21 @@ def test_conv2d_forward_backward(hip, oracle, rng, shape):
     assert np.array_equal(gw.numpy(), 2 * first_gw) and np.array_equal(gb.numpy(), 2 * first_gb)     # g + g is exact
 
 
+@pytest.mark.parametrize("shape", [(64, 1, 28, 28, 32, 3, 1, 1), (64, 32, 14, 14, 64, 3, 1, 1), (64, 4, 28, 28, 16, 5, 1, 2),
+                                   (4, 8, 14, 14, 16, 5, 1, 2)], ids=lambda s: "x".join(map(str, s)))
+def test_conv2d_forward_output_channel_tiles(hip, oracle, rng, shape):
+    """Launches large enough for the forward kernel to keep eight or four output channels per lane (small ones fall
+    to two): whatever the tile, the sums run in the reference's order, so the result is bit exact."""
+    B, ic, h, w, oc, k, stride, pad = shape
+    ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    x = rng.standard_normal((B, ic, h, w)).astype(np.float32)
+    wt = (0.3 * rng.standard_normal((oc, ic, k, k))).astype(np.float32)
+    b = rng.standard_normal(oc).astype(np.float32)
+    y = hip.empty((B, oc, ho, wo))
+    hip.check(hip.bh_conv2d_forward(dev(hip, x).ptr, dev(hip, wt).ptr, dev(hip, b).ptr, y.ptr, B, ic, h, w, oc, k, stride, pad))
+    assert np.array_equal(y.numpy(), oracle.conv2d_forward(x, wt, b, stride, pad))
+
+
 def test_conv2d_refuses_bad_shapes(hip):
     p = hip.empty(16)
     assert hip.bh_conv2d_forward(p.ptr, p.ptr, None, p.ptr, 1, 1, 2, 2, 1, 3, 1, 0) == -1       # kernel larger than image

@@ -280,37 +280,62 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         da.init(A, g.lda, m0, g.m, k_begin, smem, wave, lane);
         db.init(B, g.ldb, n0, g.n, k_begin, smem + A_FLOATS, wave, lane);
         const int64_t kt_count = (k_end - k_begin) / kBK;
+        // Two tiles are in flight ahead of the arithmetic and the fragments are software pipelined across the one
+        // barrier of a k-tile, which sits between its two halves: the fragments of the second half are read while the
+        // first half's products run, those of the next tile's first half right after the barrier while the second
+        // half's products run, so no product ever waits for an LDS read it has just issued.
+        DirectFrags<A_KC, BM, TM> fa0, fa1;
+        DirectFrags<B_KC, BN, TN> fb0, fb1;
         if (kt_count > 0) {
             da.issue(0);
             db.issue(0);
         }
+        if (kt_count > 1) {
+            da.issue((unsigned)(STAGE * sizeof(float)));
+            db.issue((unsigned)(STAGE * sizeof(float)));
+        }
         wait_direct_loads();
         __syncthreads();
+        if (kt_count > 0) {
+            fa0.load(smem, wm * Cfg::WM, 0, r, half);
+            fb0.load(smem + A_FLOATS, wn * Cfg::WN, 0, r, half);
+        }
         int cur = 0;
         for (int64_t kt = 0; kt < kt_count; kt++) {
-            if (kt + 1 < kt_count) {
-                const unsigned stage_bytes = (unsigned)((cur ^ 1) * STAGE * sizeof(float));
+            const float* sa = smem + cur * STAGE;
+            const float* sb = sa + A_FLOATS;
+            fa1.load(sa, wm * Cfg::WM, 8, r, half);
+            fb1.load(sb, wn * Cfg::WN, 8, r, half);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0.v[s][i], fb0.v[s][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            wait_direct_loads();       // tile kt+1, issued a whole tile ago
+            __syncthreads();           // ... is visible to everyone, and everyone has its fragments of stage cur in registers
+            if (kt + 2 < kt_count) {
+                const unsigned stage_bytes = (unsigned)(cur * STAGE * sizeof(float));
                 da.issue(stage_bytes);
                 db.issue(stage_bytes);
             }
-            const float* sa = smem + cur * STAGE;
-            const float* sb = sa + A_FLOATS;
-#pragma unroll
-            for (int kb = 0; kb < kBK; kb += 8) {
-                DirectFrags<A_KC, BM, TM> fa;
-                DirectFrags<B_KC, BN, TN> fb;
-                fa.load(sa, wm * Cfg::WM, kb, r, half);
-                fb.load(sb, wn * Cfg::WN, kb, r, half);
-#pragma unroll
-                for (int s = 0; s < 4; s++)
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int j = 0; j < TN; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
+            if (kt + 1 < kt_count) {
+                const float* na = smem + (cur ^ 1) * STAGE;
+                fa0.load(na, wm * Cfg::WM, 0, r, half);
+                fb0.load(na + A_FLOATS, wn * Cfg::WN, 0, r, half);
             }
-            wait_direct_loads();
-            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1.v[s][i], fb1.v[s][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
             cur ^= 1;
         }
     } else {

@@ -1,0 +1,37 @@
+"""The C programs of boat_amd/examples, built beside the library, run as a user would run them: separate processes
+that link libboat_amd.so and speak only Boat's C API."""
+import json
+import subprocess
+from pathlib import Path
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+LIB_DIR = Path(__file__).resolve().parent.parent / "boat_amd" / "lib"
+
+
+def run_example(name, *args):
+    exe = LIB_DIR / name
+    if not exe.exists():
+        pytest.fail(f"{exe} is missing: build it first (python -m boat_amd.build)")
+    return subprocess.run([str(exe), *map(str, args)], capture_output=True, text=True, timeout=110)
+
+
+def test_api_tour_every_check_holds_and_nothing_stays_allocated():
+    """One pass over tensors, the tape, layer hooks, the model container, losses, optimizers, schedulers, attention and
+    convolution from plain C; the program checks its own invariants and frees everything it made."""
+    proc = run_example("api_tour")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().splitlines()
+    rec = json.loads(lines[0])
+    assert rec["failed_check_line"] == 0
+    assert rec["host_blocks_allocated"] == rec["host_blocks_freed"] > 0
+    assert "device in use 0 B" in lines[-1], lines[-1]
+
+
+def test_mlp_train_step_program_trains():
+    proc = run_example("mlp_train_step", 50, 5)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert rec["steps"] == 50 and rec["loss_last"] < rec["loss_first"]

@@ -185,7 +185,8 @@ int bh_zero_multi(float* const* p, const int64_t* n, int count);
 
 /* ---- test hooks (no arithmetic of their own) ----
  * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256 MFMA tile,
- * 5 = small-problem kernel (whole k-chunk in LDS, one trip to memory), -1 = heuristic (default).
+ * 5 = small-problem kernel (whole k-chunk in LDS, one trip to memory), 6 = tiny-problem kernel (operands straight
+ * into the MFMA registers, contraction split among a workgroup's wavefronts), -1 = heuristic (default).
  * bh_gemm_force_direct: 0 = MFMA tiles stage their operands through registers; 1 or -1 (default) = operands go
  * straight to LDS (global_load_lds) whenever the contraction length is a multiple of 16.
  * bh_sdpa_force_general: 1 = always use the general attention kernels. */

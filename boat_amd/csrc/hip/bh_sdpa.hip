@@ -199,11 +199,11 @@ int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale,
     BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
     if (bh_count == 0 || s == 0) return BH_OK;
     BH_CHECK_ARG(q && k && v && out, "null pointer");
-    BH_CHECK_ARG(bh_count <= 65535, "too many head blocks");
     if (!g_sdpa_force_general && !attn_out && lse) {
         int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, bh_count, s, d);
         if (rc <= 0) return rc;   // 0 done, <0 error, 1 shape not covered
     }
+    BH_CHECK_ARG(bh_count <= 65535, "too many head blocks for the general attention kernel");
     BH_CHECK_ARG(s + d <= kMaxRowFloats, "sequence too long for the general attention kernel");
     const size_t shmem = sizeof(float) * (size_t)(s + d);
     hipLaunchKernelGGL(sdpa_fwd_row_kernel, dim3((unsigned)s, (unsigned)bh_count), dim3(kSBlock), shmem, stream(), q, k, v,
@@ -217,7 +217,6 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
     BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
     if (bh_count == 0 || s == 0) return BH_OK;
     BH_CHECK_ARG(q && k && v && out && lse && d_out && dq && dk && dv, "null pointer");
-    BH_CHECK_ARG(bh_count <= 65535, "too many head blocks");
     const int64_t rows = bh_count * s;
     float* delta = (float*)bh_malloc(sizeof(float) * (size_t)rows);
     if (!delta) return BH_ENOMEM;
@@ -230,9 +229,9 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
             done = sdpa_backward_mfma(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);
         if (done < 0) rc = done;
         if (done == 1) {
-            if (2 * s + 2 * d > kMaxRowFloats) {
+            if (2 * s + 2 * d > kMaxRowFloats || bh_count > 65535) {
                 bh_free(delta);
-                return set_error(BH_EINVAL, "bh_sdpa_backward: sequence too long for the general attention kernel");
+                return set_error(BH_EINVAL, "bh_sdpa_backward: sequence too long or too many head blocks for the general attention kernel");
             }
             hipLaunchKernelGGL(sdpa_bwd_dq_row_kernel, dim3((unsigned)s, (unsigned)bh_count), dim3(kSBlock),
                                sizeof(float) * (size_t)(s + 2 * d), stream(), q, k, v, lse, delta, d_out, scale, causal, dq, s,

@@ -50,7 +50,7 @@ __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + 
 template <bool CAUSAL, bool RAGGED>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
 __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ out,
-                                                            float* __restrict__ lse, int s, float scale_log2e) {
+                                                            float* __restrict__ lse, int s, int n_heads, float scale_log2e) {
     extern __shared__ __align__(16) float smem[];
     constexpr int KT = 64;                       // keys per tile
     constexpr int TILE = KT * kLd;               // floats per K or V tile in LDS
@@ -58,9 +58,10 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
     // Workgroups are handed out in the order of their linear id.  Read it tile-major: all heads' workgroups of one query
     // tile are neighbours, and with a causal mask the query tile with the most keys comes first, so that the short
     // workgroups fill the end of the launch instead of the long ones stretching it.
-    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
-    const int64_t head = lin % (int)gridDim.y;
-    const int bx = CAUSAL ? (int)gridDim.x - 1 - lin / (int)gridDim.y : lin / (int)gridDim.y;
+    const int lin = blockIdx.x;                  // one-dimensional grid of tiles * n_heads workgroups
+    const int64_t head = lin % n_heads;
+    const int n_qtiles = gridDim.x / n_heads;
+    const int bx = CAUSAL ? n_qtiles - 1 - lin / n_heads : lin / n_heads;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
     const float* vh = v + head * s * kD;
@@ -233,15 +234,15 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                                                                const float* __restrict__ v, const float* __restrict__ lse,
                                                                const float* __restrict__ delta, const float* __restrict__ d_out,
                                                                float* __restrict__ dq_partial, float* __restrict__ dk,
-                                                               float* __restrict__ dv, int s, float scale) {
+                                                               float* __restrict__ dv, int s, int n_heads, float scale) {
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
     // tile-major reading of the linear workgroup id, as in the forward kernel: key tile 0, which meets every query tile
     // under a causal mask, is handed out first for all heads
-    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
-    const int64_t head = lin % (int)gridDim.y;
-    const int bx = lin / (int)gridDim.y;
+    const int lin = blockIdx.x;
+    const int64_t head = lin % n_heads;
+    const int bx = lin / n_heads;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
     const float* vh = v + head * s * kD;
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     const float* lh = lse + head * s;
     const float* dh = delta + head * s;
     // partial dQ of this key tile: [key tile][bh][s][64]
-    float* dqh = dq_partial + ((int64_t)bx * gridDim.y + head) * s * kD;
+    float* dqh = dq_partial + ((int64_t)bx * n_heads + head) * s * kD;
     const int kv_wg = bx * 128;          // first key of the workgroup
     const int kv0 = kv_wg + w * 32;              // first key of this wavefront
     const float c1 = scale * kLog2e;
@@ -434,10 +435,12 @@ __global__ __launch_bounds__(256) void dq_partial_sum_kernel(const float* __rest
 
 // head_dim 64; any sequence length from 32 up (a length that is not a multiple of 128 takes the kernels' ragged form)
 static bool mfma_shape(int64_t s, int64_t d) { return d == kD && s >= 32 && s <= (1 << 24); }
+// the grids are one-dimensional (tiles * heads workgroups): no 65535 limit on the number of heads
+static bool grid_fits(int64_t s, int64_t bh_count) { return ceil_div(s, 128) * bh_count <= 0x7fffffff && bh_count <= 0x7fffffff; }
 
 int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
                       int64_t bh_count, int64_t s, int64_t d) {
-    if (!mfma_shape(s, d)) return 1;
+    if (!mfma_shape(s, d) || !grid_fits(s, bh_count)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(out)) return 1;
     constexpr size_t lds = sizeof(float) * 2 * 2 * 64 * kLd;
@@ -453,10 +456,10 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
         }
         attr = true;
     }
-    dim3 grid((unsigned)ceil_div(s, 128), (unsigned)bh_count);
+    dim3 grid((unsigned)(ceil_div(s, 128) * bh_count));
     const bool ragged = s % 128 != 0;
     const float sl = scale * kLog2e;
-#define FWD_LAUNCH(C, R) hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, sl)
+#define FWD_LAUNCH(C, R) hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, (int)bh_count, sl)
     if (causal && ragged) FWD_LAUNCH(true, true);
     else if (causal) FWD_LAUNCH(true, false);
     else if (ragged) FWD_LAUNCH(false, true);
@@ -468,7 +471,7 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
 int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
                        const float* d_out, float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count,
                        int64_t s, int64_t d) {
-    if (!mfma_shape(s, d)) return 1;
+    if (!mfma_shape(s, d) || !grid_fits(s, bh_count)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(d_out) || !al(dq) || !al(dk) || !al(dv)) return 1;
     constexpr size_t lds = sizeof(float) * BwdSmem::TOTAL;
@@ -489,10 +492,10 @@ int sdpa_backward_mfma(const float* q, const float* k, const float* v, const flo
     const int64_t n = bh_count * s * d;
     float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one key tile: dq itself
     if (!partial) return BH_ENOMEM;
-    dim3 grid((unsigned)tiles, (unsigned)bh_count);
+    dim3 grid((unsigned)(tiles * bh_count));
 #define BWD_LAUNCH(C, R)                                                                                                   \
     hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk, dv, \
-                       (int)s, scale)
+                       (int)s, (int)bh_count, scale)
     if (causal && ragged) BWD_LAUNCH(true, true);
     else if (causal) BWD_LAUNCH(true, false);
     else if (ragged) BWD_LAUNCH(false, true);

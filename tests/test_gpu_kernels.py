@@ -478,6 +478,26 @@ def test_sdpa_attention_matrix_output(hip, oracle, rng):
     assert np.allclose(attn.numpy().sum(-1), 1.0, atol=1e-5)
 
 
+def test_sdpa_more_head_blocks_than_a_grid_dimension_holds(hip, oracle, rng):
+    """66000 [32, 64] blocks: the MFMA kernels number their workgroups along one grid dimension, so the 65535 limit of the
+    other two does not apply; first and last blocks against float64, forward and backward."""
+    bh, s, d = 66000, 32, 64
+    q, k, v, go = (rng.standard_normal((bh, s, d), dtype=np.float32) for _ in range(4))
+    dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)
+    o, lse = hip.empty((bh, s, d)), hip.empty((bh, s))
+    scale = 0.125
+    hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, 1, o.ptr, lse.ptr, None, bh, s, d))
+    gq, gk, gv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
+    hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, dgo.ptr, scale, 1, gq.ptr, gk.ptr, gv.ptr, bh, s, d))
+    got_o, got = o.numpy(), [x.numpy() for x in (gq, gk, gv)]
+    for sl in (slice(0, 3), slice(bh - 3, bh), slice(65534, 65537)):
+        want_o, _, wattn = oracle.sdpa_forward(q[sl], k[sl], v[sl], scale, 1)
+        wq, wk, wv = oracle.sdpa_backward(q[sl], k[sl], v[sl], wattn, go[sl], scale)
+        assert rel_fro(got_o[sl], want_o) <= TOL_GEMM
+        for g, w in zip(got, (wq, wk, wv)):
+            assert rel_fro(g[sl], w) <= TOL_GEMM
+
+
 # ------------------------------------------------------------------ convolution / max pooling
 
 CONV_SHAPES = [  # batch, ic, h, w, oc, k, stride, pad

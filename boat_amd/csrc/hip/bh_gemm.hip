@@ -625,8 +625,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_tiny_kernel(GemmArgs g, int a_ve
             const int kk = (g0 + u * NW) * 8 + 4 * half;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float x = kk + j < K ? av[u][j] : 0.f;   // zero one operand past the end of the contraction
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, bv[u][j], acc, 0, 0, 0);
+                const bool in = kk + j < K;                    // both operands are zero past the end of the contraction
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(in ? av[u][j] : 0.f, in ? bv[u][j] : 0.f, acc, 0, 0, 0);
             }
         }
     }
@@ -639,6 +639,142 @@ __global__ __launch_bounds__(64 * NW) void gemm_tiny_kernel(GemmArgs g, int a_ve
         float v = red[o];
 #pragma unroll
         for (int w = 1; w < NW; w++) v += red[w * 1024 + o];
+        const int e = o >> 6, l = o & 63;
+        const int64_t orow = m0 + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3), ocol = n0 + (l & 31);
+        if (orow < g.m && ocol < g.n) {
+            if (g.bias) v += g.bias[ocol];
+            float* dst = C + orow * g.ldc + ocol;
+            *dst = g.accumulate ? *dst + v : v;
+        }
+    }
+}
+
+// ---- tiny problems with a long contraction and an operand whose k index is the fast one in memory ----
+// Fetching such an operand straight into the MFMA layout makes every lane of a load touch a cache line of its own (one
+// row each), and the rate at which the vector cache looks lines up then bounds the kernel (measured: 7-16 us per trip).
+// Here a wavefront owns a contiguous range of k, fetches its 32 x 64 slice of a k-fast operand with whole lines
+// (16 lanes per row) and turns it into the MFMA layout through a slice of LDS that only this wavefront touches, so no
+// workgroup barrier stands before the arithmetic; a row-fast operand is fetched straight into registers as in
+// gemm_tiny_kernel.  The partial tiles meet in LDS at the end, summed in wavefront order.
+constexpr int kWidePanel = 32 * 68;   // floats of one staged 32 x 64 slice (rows padded by 4)
+
+template <bool a_kfast, bool b_kfast, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_tiny_wide_kernel(GemmArgs g, int a_vec, int b_vec) {
+    static_assert(a_kfast || b_kfast, "gemm_tiny_kernel covers two row-fast operands");
+    extern __shared__ __align__(16) float smem[];
+    constexpr int PER_WAVE = (a_kfast ? kWidePanel : 0) + (b_kfast ? kWidePanel : 0);   // >= 1024 floats: the partial tile fits
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int tile_m = blockIdx.x % g.tiles_m, tile_n = blockIdx.x / g.tiles_m;
+    const int64_t batch = blockIdx.y;
+    const int64_t m0 = (int64_t)tile_m * 32, n0 = (int64_t)tile_n * 32;
+    const float* A = g.a + batch * g.stride_a;
+    const float* B = g.b + batch * g.stride_b;
+    const int K = (int)g.k;
+    const int groups = (K + 7) >> 3;
+    const int gpw = (groups + NW - 1) / NW;                // groups of 8 k per wavefront
+    const int kw0 = wave * gpw * 8;
+    const int kw1 = min(K, kw0 + gpw * 8);                 // this wavefront contracts k in [kw0, kw1)
+    float* mine = smem + wave * PER_WAVE;
+    float* as = mine;
+    float* bs = mine + (a_kfast ? kWidePanel : 0);
+    // rows and columns past the edge read the last valid one: they only feed outputs that are never stored
+    const int64_t row = min(m0 + r, g.m - 1), col = min(n0 + r, g.n - 1);
+
+    floatx16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.f;
+    for (int kc = kw0; kc < kw1; kc += 64) {
+        // row-fast operands: this lane's values for the eight groups of the chunk, straight from memory
+        float av[8][4], bv[8][4];
+        if (!a_kfast) {
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) av[u][j] = A[(int64_t)min(kc + 8 * u + 4 * half + j, K - 1) * g.lda + row];
+        }
+        if (!b_kfast) {
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) bv[u][j] = B[(int64_t)min(kc + 8 * u + 4 * half + j, K - 1) * g.ldb + col];
+        }
+        // k-fast operands: 32 rows x 64 k as 512 16-byte pieces, 8 per lane, 16 lanes along a row
+        float4 sa[8], sb[8];
+        if (a_kfast) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int f = lane + 64 * i, rr = f >> 4, kk = kc + 4 * (f & 15);
+                const float* p = A + min(m0 + rr, g.m - 1) * g.lda;
+                if (a_vec) sa[i] = *reinterpret_cast<const float4*>(p + min(kk, K - 4));
+                else sa[i] = make_float4(p[min(kk, K - 1)], p[min(kk + 1, K - 1)], p[min(kk + 2, K - 1)], p[min(kk + 3, K - 1)]);
+            }
+        }
+        if (b_kfast) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int f = lane + 64 * i, rr = f >> 4, kk = kc + 4 * (f & 15);
+                const float* p = B + min(n0 + rr, g.n - 1) * g.ldb;
+                if (b_vec) sb[i] = *reinterpret_cast<const float4*>(p + min(kk, K - 4));
+                else sb[i] = make_float4(p[min(kk, K - 1)], p[min(kk + 1, K - 1)], p[min(kk + 2, K - 1)], p[min(kk + 3, K - 1)]);
+            }
+        }
+        if (a_kfast) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int f = lane + 64 * i;
+                *reinterpret_cast<float4*>(as + (f >> 4) * 68 + 4 * (f & 15)) = sa[i];
+            }
+        }
+        if (b_kfast) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int f = lane + 64 * i;
+                *reinterpret_cast<float4*>(bs + (f >> 4) * 68 + 4 * (f & 15)) = sb[i];
+            }
+        }
+        // the slice is private to this wavefront: its own LDS writes are ordered before its reads, the fences only keep
+        // the compiler from moving one across the other
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int kk = kc + 8 * u + 4 * half;
+            float a4[4], b4[4];
+            if (a_kfast) {
+                const float4 t = *reinterpret_cast<const float4*>(as + r * 68 + 8 * u + 4 * half);
+                a4[0] = t.x; a4[1] = t.y; a4[2] = t.z; a4[3] = t.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) a4[j] = av[u][j];
+            }
+            if (b_kfast) {
+                const float4 t = *reinterpret_cast<const float4*>(bs + r * 68 + 8 * u + 4 * half);
+                b4[0] = t.x; b4[1] = t.y; b4[2] = t.z; b4[3] = t.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) b4[j] = bv[u][j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const bool in = kk + j < kw1;                  // past this wavefront's range (or the contraction): no contribution
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(in ? a4[j] : 0.f, in ? b4[j] : 0.f, acc, 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    // the partial tile goes where the wavefront's slices were
+#pragma unroll
+    for (int e = 0; e < 16; e++) mine[e * 64 + lane] = acc[e];
+    __syncthreads();
+
+    float* C = g.c + batch * g.stride_c;
+    for (int o = tid; o < 1024; o += 64 * NW) {
+        float v = smem[o];
+#pragma unroll
+        for (int w = 1; w < NW; w++) v += smem[w * PER_WAVE + o];
         const int e = o >> 6, l = o & 63;
         const int64_t orow = m0 + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3), ocol = n0 + (l & 31);
         if (orow < g.m && ocol < g.n) {
@@ -840,11 +976,12 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     }
     // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
     if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
-    // a few million multiply-adds in at most a few hundred 32x32 tiles: the single-trip kernel without staging.  An
-    // operand whose k index is the fast one in memory makes every lane fetch from a row of its own; measured, that is
-    // only worth it while the contraction is short (k <= 128: 4-7 us against 6.5-9 us; beyond, 10-30 us against 11-14)
+    // A few million multiply-adds in at most a few hundred 32x32 tiles: the kernels without workgroup-wide staging.
+    // Measured against the staged small-problem kernel plus its fold (11-14 us beyond k = 128): two row-fast operands
+    // 6-10 us up to k = 1024; one k-fast operand 7.5-8 us up to k = 512 (one trip) and 12 us up to 1024 (two trips);
+    // two k-fast operands 9-11 us up to k = 512 and slower beyond.
     if (k > 0 && m * n * k <= ((int64_t)1 << 24) && ceil_div(m, 32) * ceil_div(n, 32) * batch <= 512 &&
-        (k <= 128 || (!a_kc && !b_kc)))
+        (k <= 512 || (k <= 1024 && !(a_kc && b_kc)) || (!a_kc && !b_kc)))
         cfg = 6;
     if (g_force_cfg >= 0 && g_force_cfg <= 6 && (vec_ok || g_force_cfg == 0 || g_force_cfg >= 5)) cfg = g_force_cfg;
     if (cfg == 6 && k == 0) cfg = 5;
@@ -857,7 +994,28 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         const int a_vec = a_kc && al16(a) && lda % 4 == 0 && k % 4 == 0 && (g.stride_a % 4 == 0 || batch == 1);
         const int b_vec = b_kc && al16(b) && ldb % 4 == 0 && k % 4 == 0 && (g.stride_b % 4 == 0 || batch == 1);
         const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
-        const bool wide = k > 128;    // 8 wavefronts share a long contraction, 4 a short one    // 16 wavefronts share a long contraction (one trip to memory up to k = 1024), 4 a short one
+        if (k > 128 && (a_kc || b_kc)) {
+            // long contraction with a k-fast operand: slices staged per wavefront (8 wavefronts, 64 k each per trip)
+            const size_t lds = sizeof(float) * 8 * (size_t)((a_kc ? kWidePanel : 0) + (b_kc ? kWidePanel : 0));
+#define WIDE_LAUNCH(AK, BK)                                                                                               \
+    {                                                                                                                     \
+        static bool attr = false;                                                                                         \
+        if (!attr) {                                                                                                      \
+            int arc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiny_wide_kernel<AK, BK, 8>),     \
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),                \
+                                "hipFuncSetAttribute");                                                                   \
+            if (arc) return arc;                                                                                          \
+            attr = true;                                                                                                  \
+        }                                                                                                                 \
+        hipLaunchKernelGGL((gemm_tiny_wide_kernel<AK, BK, 8>), grid, dim3(512), lds, stream(), g, a_vec, b_vec);          \
+    }
+            if (a_kc && b_kc) WIDE_LAUNCH(true, true)
+            else if (a_kc) WIDE_LAUNCH(true, false)
+            else WIDE_LAUNCH(false, true)
+#undef WIDE_LAUNCH
+            return BH_LAUNCH_CHECK("gemm_tiny_wide_kernel");
+        }
+        const bool wide = k > 128;    // two row-fast operands: 8 wavefronts share a long contraction, 4 a short one
 #define TINY_LAUNCH(AK, BK)                                                                                               \
     if (wide) hipLaunchKernelGGL((gemm_tiny_kernel<AK, BK, 8, 8>), grid, dim3(512), 0, stream(), g, a_vec, b_vec);          \
     else hipLaunchKernelGGL((gemm_tiny_kernel<AK, BK, 4, 4>), grid, dim3(256), 0, stream(), g, a_vec, b_vec)

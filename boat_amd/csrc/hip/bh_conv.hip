@@ -151,14 +151,16 @@ __global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __re
     dyp[i] = dy[((int64_t)b * c.oc + oc) * per + p];
 }
 
-// col[(b, oh, ow)][(ic, kh, kw)] = x[b, ic, oh*stride - pad + kh, ow*stride - pad + kw], zero outside the image
+// col[(ic, kh, kw)][(b, oh, ow)] = x[b, ic, oh*stride - pad + kh, ow*stride - pad + kw], zero outside the image.
+// The output position is the fast index of the patch matrix: neighbouring lanes read neighbouring pixels and write
+// neighbouring elements (with the tap as the fast index every lane of a load touched a line of its own and the kernel
+// ran at a seventh of the memory rate).
 __global__ __launch_bounds__(kCBlock) void im2col_kernel(const float* __restrict__ x, float* __restrict__ col, ConvShape c,
-                                                         int64_t total) {
+                                                         int64_t positions, int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
     if (i >= total) return;
-    const int kk = c.ic * c.k * c.k;
-    const int t = (int)(i % kk);
-    const int64_t pos = i / kk;
+    const int64_t pos = i % positions;
+    const int t = (int)(i / positions);
     const int kw = t % c.k, kh = (t / c.k) % c.k, ci = t / (c.k * c.k);
     const int ow = (int)(pos % c.wo);
     const int oh = (int)((pos / c.wo) % c.ho);
@@ -167,16 +169,15 @@ __global__ __launch_bounds__(kCBlock) void im2col_kernel(const float* __restrict
     col[i] = (ih >= 0 && ih < c.h && iw >= 0 && iw < c.w) ? x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] : 0.f;
 }
 
-// dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(b, oh, ow)][(ic, kh, kw)]
+// dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(ic, kh, kw)][(b, oh, ow)]
 __global__ __launch_bounds__(kCBlock) void col2im_kernel(const float* __restrict__ dcol, float* __restrict__ dx, ConvShape c,
-                                                         int64_t total) {
+                                                         int64_t positions, int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
     if (i >= total) return;
     const int iw = (int)(i % c.w);
     const int ih = (int)((i / c.w) % c.h);
     const int ci = (int)((i / ((int64_t)c.w * c.h)) % c.ic);
     const int b = (int)(i / ((int64_t)c.w * c.h * c.ic));
-    const int kk = c.ic * c.k * c.k;
     float acc = 0.f;
     for (int kh = 0; kh < c.k; kh++) {
         const int t = ih + c.pad - kh;
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(kCBlock) void col2im_kernel(const float* __restrict
             if (u < 0 || u % c.stride) continue;
             const int ow = u / c.stride;
             if (ow >= c.wo) continue;
-            acc += dcol[(((int64_t)b * c.ho + oh) * c.wo + ow) * kk + (ci * c.k + kh) * c.k + kw];
+            acc += dcol[(int64_t)((ci * c.k + kh) * c.k + kw) * positions + ((int64_t)b * c.ho + oh) * c.wo + ow];
         }
     }
     dx[i] = acc;
@@ -369,10 +370,10 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
         if (!col) rc = BH_ENOMEM;
     }
     if (rc == BH_OK && gw) {
-        hipLaunchKernelGGL(im2col_kernel, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions * kk);
+        hipLaunchKernelGGL(im2col_kernel, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions, positions * kk);
         rc = BH_LAUNCH_CHECK("im2col_kernel");
-        // gw[oc][kk] (+)= dyp[oc][positions] . col[positions][kk]
-        if (rc == BH_OK) rc = bh_gemm(0, 0, c.oc, kk, positions, dyp, positions, col, kk, gw, kk, nullptr, accumulate, 1);
+        // gw[oc][kk] (+)= dyp[oc][positions] . col[kk][positions]^T : both operands contiguous along the contraction
+        if (rc == BH_OK) rc = bh_gemm(0, 1, c.oc, kk, positions, dyp, positions, col, positions, gw, kk, nullptr, accumulate, 1);
     }
     if (rc == BH_OK && dx) {
         const float* wsrc = w;
@@ -385,11 +386,11 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
                 wsrc = wf;
             }
         }
-        // dcol[positions][kk] = dyp^T[positions][oc] . w[oc][kk]  (the stream orders it after the gw product that read col)
-        if (rc == BH_OK) rc = bh_gemm(1, 0, positions, kk, c.oc, dyp, positions, wsrc, kk, col, kk, nullptr, 0, 1);
+        // dcol[kk][positions] = w^T[kk][oc] . dyp[oc][positions]  (the stream orders it after the gw product that read col)
+        if (rc == BH_OK) rc = bh_gemm(1, 0, kk, positions, c.oc, wsrc, kk, dyp, positions, col, positions, nullptr, 0, 1);
         if (rc == BH_OK) {
             const int64_t total = (int64_t)c.batch * c.ic * c.h * c.w;
-            hipLaunchKernelGGL(col2im_kernel, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, total);
+            hipLaunchKernelGGL(col2im_kernel, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, positions, total);
             rc = BH_LAUNCH_CHECK("col2im_kernel");
         }
     }

@@ -670,10 +670,13 @@ __global__ __launch_bounds__(64 * NW) void gemm_tiny_wide_kernel(GemmArgs g, int
     const float* A = g.a + batch * g.stride_a;
     const float* B = g.b + batch * g.stride_b;
     const int K = (int)g.k;
-    const int groups = (K + 7) >> 3;
+    // a very long contraction is cut over blockIdx.z first (partial tiles go to the workspace and are folded afterwards)
+    const int ks0 = g.k_splits > 1 ? (int)(blockIdx.z * g.k_per_split) : 0;
+    const int ks1 = g.k_splits > 1 ? min(K, ks0 + (int)g.k_per_split) : K;
+    const int groups = (ks1 - ks0 + 7) >> 3;
     const int gpw = (groups + NW - 1) / NW;                // groups of 8 k per wavefront
-    const int kw0 = wave * gpw * 8;
-    const int kw1 = min(K, kw0 + gpw * 8);                 // this wavefront contracts k in [kw0, kw1)
+    const int kw0 = ks0 + wave * gpw * 8;
+    const int kw1 = min(ks1, kw0 + gpw * 8);               // this wavefront contracts k in [kw0, kw1)
     float* mine = smem + wave * PER_WAVE;
     float* as = mine;
     float* bs = mine + (a_kfast ? kWidePanel : 0);
@@ -771,6 +774,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_tiny_wide_kernel(GemmArgs g, int
     __syncthreads();
 
     float* C = g.c + batch * g.stride_c;
+    if (g.k_splits > 1) C += (int64_t)blockIdx.z * gridDim.y * g.stride_c;
+    const bool last_word = g.k_splits <= 1;                // bias and accumulation belong to the fold otherwise
     for (int o = tid; o < 1024; o += 64 * NW) {
         float v = smem[o];
 #pragma unroll
@@ -778,9 +783,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_tiny_wide_kernel(GemmArgs g, int
         const int e = o >> 6, l = o & 63;
         const int64_t orow = m0 + (e >> 2) * 8 + (l >> 5) * 4 + (e & 3), ocol = n0 + (l & 31);
         if (orow < g.m && ocol < g.n) {
-            if (g.bias) v += g.bias[ocol];
+            if (last_word && g.bias) v += g.bias[ocol];
             float* dst = C + orow * g.ldc + ocol;
-            *dst = g.accumulate ? *dst + v : v;
+            *dst = last_word && g.accumulate ? *dst + v : v;
         }
     }
 }
@@ -980,11 +985,20 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     // Measured against the staged small-problem kernel plus its fold (11-14 us beyond k = 128): two row-fast operands
     // 6-10 us up to k = 1024; one k-fast operand 7.5-8 us up to k = 512 (one trip) and 12 us up to 1024 (two trips);
     // two k-fast operands 9-11 us up to k = 512 and slower beyond.
-    if (k > 0 && m * n * k <= ((int64_t)1 << 24) && ceil_div(m, 32) * ceil_div(n, 32) * batch <= 512 &&
+    const int64_t tiles32 = ceil_div(m, 32) * ceil_div(n, 32) * batch;
+    if (k > 0 && m * n * k <= ((int64_t)1 << 24) && tiles32 <= 512 &&
         (k <= 512 || (k <= 1024 && !(a_kc && b_kc)) || (!a_kc && !b_kc)))
         cfg = 6;
+    // A small output with a very long contraction over k-fast operands (the weight gradient of a convolution: 64 x 288
+    // outputs, k = 12544): chunks of 512 k per workgroup of the same kernel, partials folded afterwards.
+    bool tiny_split = false;
+    if (k >= 2048 && tiles32 <= 64 && (a_kc || b_kc) && ceil_div(k, 512) <= 65535) {
+        cfg = 6;
+        tiny_split = true;
+    }
     if (g_force_cfg >= 0 && g_force_cfg <= 6 && (vec_ok || g_force_cfg == 0 || g_force_cfg >= 5)) cfg = g_force_cfg;
     if (cfg == 6 && k == 0) cfg = 5;
+    if (cfg != 6) tiny_split = false;
 
     if (cfg == 6) {
         g.tiles_m = (int)ceil_div(m, 32);
@@ -997,23 +1011,40 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         if (k > 128 && (a_kc || b_kc)) {
             // long contraction with a k-fast operand: slices staged per wavefront (8 wavefronts, 64 k each per trip)
             const size_t lds = sizeof(float) * 8 * (size_t)((a_kc ? kWidePanel : 0) + (b_kc ? kWidePanel : 0));
+            GemmArgs run = g;
+            float* ws = nullptr;
+            if (tiny_split) {
+                g.k_per_split = 512;
+                g.k_splits = (int)ceil_div(k, 512);
+                ws = (float*)bh_malloc(sizeof(float) * (size_t)(g.k_splits * batch * m * n));
+                if (!ws) return BH_ENOMEM;
+                run = g;
+                run.c = ws;
+                run.ldc = n;
+                run.stride_c = m * n;
+            }
+            const dim3 wgrid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)(g.k_splits > 1 ? g.k_splits : 1));
+            int lrc = BH_OK;
 #define WIDE_LAUNCH(AK, BK)                                                                                               \
     {                                                                                                                     \
         static bool attr = false;                                                                                         \
         if (!attr) {                                                                                                      \
-            int arc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiny_wide_kernel<AK, BK, 8>),     \
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),                \
-                                "hipFuncSetAttribute");                                                                   \
-            if (arc) return arc;                                                                                          \
-            attr = true;                                                                                                  \
+            lrc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiny_wide_kernel<AK, BK, 8>),         \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),                    \
+                            "hipFuncSetAttribute");                                                                       \
+            attr = lrc == BH_OK;                                                                                          \
         }                                                                                                                 \
-        hipLaunchKernelGGL((gemm_tiny_wide_kernel<AK, BK, 8>), grid, dim3(512), lds, stream(), g, a_vec, b_vec);          \
+        if (lrc == BH_OK)                                                                                                 \
+            hipLaunchKernelGGL((gemm_tiny_wide_kernel<AK, BK, 8>), wgrid, dim3(512), lds, stream(), run, a_vec, b_vec);   \
     }
             if (a_kc && b_kc) WIDE_LAUNCH(true, true)
             else if (a_kc) WIDE_LAUNCH(true, false)
             else WIDE_LAUNCH(false, true)
 #undef WIDE_LAUNCH
-            return BH_LAUNCH_CHECK("gemm_tiny_wide_kernel");
+            if (lrc == BH_OK) lrc = BH_LAUNCH_CHECK("gemm_tiny_wide_kernel");
+            if (lrc == BH_OK && g.k_splits > 1) lrc = launch_fold(ws, c, bias, m, n, ldc, g.k_splits, batch, g.stride_c, accumulate);
+            if (ws) bh_free(ws);
+            return lrc;
         }
         const bool wide = k > 128;    // two row-fast operands: 8 wavefronts share a long contraction, 4 a short one
 #define TINY_LAUNCH(AK, BK)                                                                                               \

@@ -140,14 +140,17 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_generic_kernel(const float
 }
 
 // dyp[oc][b][p] = dy[b][oc][p], p over the ho*wo output positions
+// (IDX: 32-bit index arithmetic whenever the element count allows it: 64-bit division costs tens of instructions and
+// these kernels do nothing else)
+template <typename IDX>
 __global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __restrict__ dy, float* __restrict__ dyp, ConvShape c,
                                                                int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= total) return;
-    const int per = c.ho * c.wo;
-    const int p = (int)(i % per);
-    const int b = (int)((i / per) % c.batch);
-    const int oc = (int)(i / ((int64_t)per * c.batch));
+    const IDX i = (IDX)blockIdx.x * kCBlock + threadIdx.x;
+    if (i >= (IDX)total) return;
+    const IDX per = c.ho * c.wo;
+    const IDX p = i % per;
+    const IDX q = i / per;
+    const IDX b = q % (IDX)c.batch, oc = q / (IDX)c.batch;
     dyp[i] = dy[((int64_t)b * c.oc + oc) * per + p];
 }
 
@@ -155,29 +158,34 @@ __global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __re
 // The output position is the fast index of the patch matrix: neighbouring lanes read neighbouring pixels and write
 // neighbouring elements (with the tap as the fast index every lane of a load touched a line of its own and the kernel
 // ran at a seventh of the memory rate).
+template <typename IDX>
 __global__ __launch_bounds__(kCBlock) void im2col_kernel(const float* __restrict__ x, float* __restrict__ col, ConvShape c,
                                                          int64_t positions, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= total) return;
-    const int64_t pos = i % positions;
-    const int t = (int)(i / positions);
+    const IDX i = (IDX)blockIdx.x * kCBlock + threadIdx.x;
+    if (i >= (IDX)total) return;
+    const IDX pos = i % (IDX)positions;
+    const int t = (int)(i / (IDX)positions);
     const int kw = t % c.k, kh = (t / c.k) % c.k, ci = t / (c.k * c.k);
-    const int ow = (int)(pos % c.wo);
-    const int oh = (int)((pos / c.wo) % c.ho);
-    const int b = (int)(pos / ((int64_t)c.wo * c.ho));
+    const int ow = (int)(pos % (IDX)c.wo);
+    const IDX rest = pos / (IDX)c.wo;
+    const int oh = (int)(rest % (IDX)c.ho);
+    const int b = (int)(rest / (IDX)c.ho);
     const int ih = oh * c.stride - c.pad + kh, iw = ow * c.stride - c.pad + kw;
     col[i] = (ih >= 0 && ih < c.h && iw >= 0 && iw < c.w) ? x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] : 0.f;
 }
 
 // dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(ic, kh, kw)][(b, oh, ow)]
+template <typename IDX>
 __global__ __launch_bounds__(kCBlock) void col2im_kernel(const float* __restrict__ dcol, float* __restrict__ dx, ConvShape c,
                                                          int64_t positions, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= total) return;
-    const int iw = (int)(i % c.w);
-    const int ih = (int)((i / c.w) % c.h);
-    const int ci = (int)((i / ((int64_t)c.w * c.h)) % c.ic);
-    const int b = (int)(i / ((int64_t)c.w * c.h * c.ic));
+    const IDX i = (IDX)blockIdx.x * kCBlock + threadIdx.x;
+    if (i >= (IDX)total) return;
+    const int iw = (int)(i % (IDX)c.w);
+    const IDX r1 = i / (IDX)c.w;
+    const int ih = (int)(r1 % (IDX)c.h);
+    const IDX r2 = r1 / (IDX)c.h;
+    const int ci = (int)(r2 % (IDX)c.ic);
+    const int b = (int)(r2 / (IDX)c.ic);
     float acc = 0.f;
     for (int kh = 0; kh < c.k; kh++) {
         const int t = ih + c.pad - kh;
@@ -205,22 +213,25 @@ __global__ __launch_bounds__(kCBlock) void mirror_taps_kernel(const float* __res
     wf[i] = w[plane * taps + (taps - 1 - t)];
 }
 
-// out[r] (+)= sum of row r of a [rows][n] matrix: one workgroup per row
-__global__ __launch_bounds__(kCBlock) void rowsum_kernel(const float* __restrict__ a, float* __restrict__ out, int64_t n,
-                                                         int accumulate) {
+// Row sums of a [rows][n] matrix in two stages: workgroup (r, ch) sums chunk ch of row r into partial[ch][r]; the
+// partials are then folded by fold_rows_kernel.  (One workgroup per row left 32-64 workgroups streaming 200 KB each.)
+__global__ __launch_bounds__(kCBlock) void rowsum_partial_kernel(const float* __restrict__ a, float* __restrict__ partial, int64_t n,
+                                                                 int64_t chunk) {
     __shared__ float red[kCBlock / 64];
+    const int64_t begin = (int64_t)blockIdx.y * chunk;
+    const int64_t end = begin + chunk < n ? begin + chunk : n;
     const float* row = a + (int64_t)blockIdx.x * n;
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int64_t i = threadIdx.x;
-    for (; i + 3 * kCBlock < n; i += 4 * kCBlock) {
+    int64_t i = begin + threadIdx.x;
+    for (; i + 3 * kCBlock < end; i += 4 * kCBlock) {
         a0 += row[i];
         a1 += row[i + kCBlock];
         a2 += row[i + 2 * kCBlock];
         a3 += row[i + 3 * kCBlock];
     }
-    for (; i < n; i += kCBlock) a0 += row[i];
+    for (; i < end; i += kCBlock) a0 += row[i];
     const float total = block_sum<kCBlock / 64>((a0 + a1) + (a2 + a3), red);
-    if (threadIdx.x == 0) out[blockIdx.x] = accumulate ? out[blockIdx.x] + total : total;
+    if (threadIdx.x == 0) partial[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = total;
 }
 
 struct PoolShape {
@@ -359,18 +370,37 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
     float *dyp = nullptr, *col = nullptr, *wf = nullptr;
     dyp = (float*)bh_malloc(sizeof(float) * (size_t)(c.oc * positions));
     if (!dyp) return BH_ENOMEM;
-    hipLaunchKernelGGL(nchw_to_cnhw_kernel, blocks(c.oc * positions), dim3(kCBlock), 0, stream(), dy, dyp, c, c.oc * positions);
+    const auto fits32 = [](int64_t n) { return n < ((int64_t)1 << 31) - kCBlock; };
+    if (fits32(c.oc * positions)) hipLaunchKernelGGL(nchw_to_cnhw_kernel<unsigned>, blocks(c.oc * positions), dim3(kCBlock), 0, stream(), dy, dyp, c, c.oc * positions);
+    else hipLaunchKernelGGL(nchw_to_cnhw_kernel<int64_t>, blocks(c.oc * positions), dim3(kCBlock), 0, stream(), dy, dyp, c, c.oc * positions);
     rc = BH_LAUNCH_CHECK("nchw_to_cnhw_kernel");
     if (rc == BH_OK && gb) {
-        hipLaunchKernelGGL(rowsum_kernel, dim3((unsigned)c.oc), dim3(kCBlock), 0, stream(), dyp, gb, positions, accumulate);
-        rc = BH_LAUNCH_CHECK("rowsum_kernel");
+        int64_t chunks = ceil_div(512, c.oc);                       // about two workgroups per compute unit ...
+        if (chunks > ceil_div(positions, 2048)) chunks = ceil_div(positions, 2048);   // ... of at least 2048 elements each
+        if (chunks > 65535) chunks = 65535;
+        const int64_t chunk = ceil_div(positions, chunks);
+        chunks = ceil_div(positions, chunk);
+        float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * c.oc));
+        if (!partial) rc = BH_ENOMEM;
+        if (rc == BH_OK) {
+            hipLaunchKernelGGL(rowsum_partial_kernel, dim3((unsigned)c.oc, (unsigned)chunks), dim3(kCBlock), 0, stream(), dyp, partial,
+                               positions, chunk);
+            rc = BH_LAUNCH_CHECK("rowsum_partial_kernel");
+        }
+        if (rc == BH_OK) {
+            hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(c.oc, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0, stream(),
+                               partial, chunks, (int64_t)c.oc, gb, (float*)nullptr, (int64_t)c.oc, accumulate);
+            rc = BH_LAUNCH_CHECK("fold_rows_kernel");
+        }
+        if (partial) bh_free(partial);
     }
     if (rc == BH_OK && (gw || dx)) {
         col = (float*)bh_malloc(sizeof(float) * (size_t)(positions * kk));   // patches for gw, then reused as dcol
         if (!col) rc = BH_ENOMEM;
     }
     if (rc == BH_OK && gw) {
-        hipLaunchKernelGGL(im2col_kernel, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions, positions * kk);
+        if (fits32(positions * kk)) hipLaunchKernelGGL(im2col_kernel<unsigned>, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions, positions * kk);
+        else hipLaunchKernelGGL(im2col_kernel<int64_t>, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions, positions * kk);
         rc = BH_LAUNCH_CHECK("im2col_kernel");
         // gw[oc][kk] (+)= dyp[oc][positions] . col[kk][positions]^T : both operands contiguous along the contraction
         if (rc == BH_OK) rc = bh_gemm(0, 1, c.oc, kk, positions, dyp, positions, col, positions, gw, kk, nullptr, accumulate, 1);
@@ -390,7 +420,8 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
         if (rc == BH_OK) rc = bh_gemm(1, 0, kk, positions, c.oc, wsrc, kk, dyp, positions, col, positions, nullptr, 0, 1);
         if (rc == BH_OK) {
             const int64_t total = (int64_t)c.batch * c.ic * c.h * c.w;
-            hipLaunchKernelGGL(col2im_kernel, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, positions, total);
+            if (fits32(total) && fits32(positions * kk)) hipLaunchKernelGGL(col2im_kernel<unsigned>, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, positions, total);
+            else hipLaunchKernelGGL(col2im_kernel<int64_t>, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, positions, total);
             rc = BH_LAUNCH_CHECK("col2im_kernel");
         }
     }

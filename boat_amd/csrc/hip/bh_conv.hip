@@ -140,67 +140,60 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_generic_kernel(const float
 }
 
 // dyp[oc][b][p] = dy[b][oc][p], p over the ho*wo output positions
-// (IDX: 32-bit index arithmetic whenever the element count allows it: 64-bit division costs tens of instructions and
-// these kernels do nothing else)
-template <typename IDX>
-__global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __restrict__ dy, float* __restrict__ dyp, ConvShape c,
-                                                               int64_t total) {
-    const IDX i = (IDX)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= (IDX)total) return;
-    const IDX per = c.ho * c.wo;
-    const IDX p = i % per;
-    const IDX q = i / per;
-    const IDX b = q % (IDX)c.batch, oc = q / (IDX)c.batch;
-    dyp[i] = dy[((int64_t)b * c.oc + oc) * per + p];
+// The three rearrangement kernels of the backward pass do no arithmetic, so their index computation is their cost:
+// the grid carries the outer indices (y, z) and a lane only splits its position inside one image plane (one 32-bit
+// division).  Written with a flat index and 64-bit div/mod they ran at a seventh of the memory rate.
+
+// dyp[oc][b][p] = dy[b][oc][p], p over the ho*wo output positions; grid (ceil(per/256), oc, batch)
+__global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __restrict__ dy, float* __restrict__ dyp, ConvShape c) {
+    const unsigned per = (unsigned)(c.ho * c.wo);
+    const unsigned p = blockIdx.x * kCBlock + threadIdx.x;
+    if (p >= per) return;
+    const unsigned oc = blockIdx.y, b = blockIdx.z;
+    dyp[((int64_t)oc * c.batch + b) * per + p] = dy[((int64_t)b * c.oc + oc) * per + p];
 }
 
 // col[(ic, kh, kw)][(b, oh, ow)] = x[b, ic, oh*stride - pad + kh, ow*stride - pad + kw], zero outside the image.
 // The output position is the fast index of the patch matrix: neighbouring lanes read neighbouring pixels and write
-// neighbouring elements (with the tap as the fast index every lane of a load touched a line of its own and the kernel
-// ran at a seventh of the memory rate).
-template <typename IDX>
+// neighbouring elements.  grid (ceil(per/256), ic*k*k, batch)
 __global__ __launch_bounds__(kCBlock) void im2col_kernel(const float* __restrict__ x, float* __restrict__ col, ConvShape c,
-                                                         int64_t positions, int64_t total) {
-    const IDX i = (IDX)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= (IDX)total) return;
-    const IDX pos = i % (IDX)positions;
-    const int t = (int)(i / (IDX)positions);
+                                                         int64_t positions) {
+    const unsigned per = (unsigned)(c.ho * c.wo);
+    const unsigned p = blockIdx.x * kCBlock + threadIdx.x;
+    if (p >= per) return;
+    const int t = blockIdx.y, b = blockIdx.z;                     // uniform over the workgroup
     const int kw = t % c.k, kh = (t / c.k) % c.k, ci = t / (c.k * c.k);
-    const int ow = (int)(pos % (IDX)c.wo);
-    const IDX rest = pos / (IDX)c.wo;
-    const int oh = (int)(rest % (IDX)c.ho);
-    const int b = (int)(rest / (IDX)c.ho);
+    const int oh = (int)(p / (unsigned)c.wo), ow = (int)(p - (unsigned)oh * (unsigned)c.wo);
     const int ih = oh * c.stride - c.pad + kh, iw = ow * c.stride - c.pad + kw;
-    col[i] = (ih >= 0 && ih < c.h && iw >= 0 && iw < c.w) ? x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] : 0.f;
+    const bool inside = ih >= 0 && ih < c.h && iw >= 0 && iw < c.w;
+    col[(int64_t)t * positions + (int64_t)b * per + p] = inside ? x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] : 0.f;
 }
 
-// dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(ic, kh, kw)][(b, oh, ow)]
-template <typename IDX>
+// dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(ic, kh, kw)][(b, oh, ow)];
+// grid (ceil(h*w/256), ic, batch)
 __global__ __launch_bounds__(kCBlock) void col2im_kernel(const float* __restrict__ dcol, float* __restrict__ dx, ConvShape c,
-                                                         int64_t positions, int64_t total) {
-    const IDX i = (IDX)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= (IDX)total) return;
-    const int iw = (int)(i % (IDX)c.w);
-    const IDX r1 = i / (IDX)c.w;
-    const int ih = (int)(r1 % (IDX)c.h);
-    const IDX r2 = r1 / (IDX)c.h;
-    const int ci = (int)(r2 % (IDX)c.ic);
-    const int b = (int)(r2 / (IDX)c.ic);
+                                                         int64_t positions) {
+    const unsigned plane = (unsigned)(c.h * c.w);
+    const unsigned q = blockIdx.x * kCBlock + threadIdx.x;
+    if (q >= plane) return;
+    const int ci = blockIdx.y, b = blockIdx.z;
+    const int ih = (int)(q / (unsigned)c.w), iw = (int)(q - (unsigned)ih * (unsigned)c.w);
+    const float* base = dcol + (int64_t)b * c.ho * c.wo;
     float acc = 0.f;
     for (int kh = 0; kh < c.k; kh++) {
         const int t = ih + c.pad - kh;
-        if (t < 0 || t % c.stride) continue;
-        const int oh = t / c.stride;
-        if (oh >= c.ho) continue;
+        if (t < 0) continue;
+        const int oh = c.stride == 1 ? t : t / c.stride;
+        if (oh * c.stride != t || oh >= c.ho) continue;
         for (int kw = 0; kw < c.k; kw++) {
             const int u = iw + c.pad - kw;
-            if (u < 0 || u % c.stride) continue;
-            const int ow = u / c.stride;
-            if (ow >= c.wo) continue;
-            acc += dcol[(int64_t)((ci * c.k + kh) * c.k + kw) * positions + ((int64_t)b * c.ho + oh) * c.wo + ow];
+            if (u < 0) continue;
+            const int ow = c.stride == 1 ? u : u / c.stride;
+            if (ow * c.stride != u || ow >= c.wo) continue;
+            acc += base[(int64_t)((ci * c.k + kh) * c.k + kw) * positions + oh * c.wo + ow];
         }
     }
-    dx[i] = acc;
+    dx[((int64_t)b * c.ic + ci) * plane + q] = acc;
 }
 
 // wf[oc, ic, kh, kw] = w[oc, ic, k-1-kh, k-1-kw]
@@ -367,12 +360,13 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
     BH_CHECK_ARG(positions * kk < ((int64_t)1 << 40), "conv2d: patch matrix too large");
     if (!dx && !gw && !gb) return BH_OK;
     auto blocks = [](int64_t n) { return dim3((unsigned)ceil_div(n, kCBlock)); };
+    // the rearrangement kernels carry channel and batch indices in grid.y / grid.z
+    BH_CHECK_ARG(c.oc <= 65535 && c.batch <= 65535 && kk <= 65535 && c.ic <= 65535, "conv2d backward: more than 65535 channels, taps or images");
     float *dyp = nullptr, *col = nullptr, *wf = nullptr;
     dyp = (float*)bh_malloc(sizeof(float) * (size_t)(c.oc * positions));
     if (!dyp) return BH_ENOMEM;
-    const auto fits32 = [](int64_t n) { return n < ((int64_t)1 << 31) - kCBlock; };
-    if (fits32(c.oc * positions)) hipLaunchKernelGGL(nchw_to_cnhw_kernel<unsigned>, blocks(c.oc * positions), dim3(kCBlock), 0, stream(), dy, dyp, c, c.oc * positions);
-    else hipLaunchKernelGGL(nchw_to_cnhw_kernel<int64_t>, blocks(c.oc * positions), dim3(kCBlock), 0, stream(), dy, dyp, c, c.oc * positions);
+    const unsigned per_blocks = (unsigned)ceil_div((int64_t)c.ho * c.wo, kCBlock);
+    hipLaunchKernelGGL(nchw_to_cnhw_kernel, dim3(per_blocks, (unsigned)c.oc, (unsigned)c.batch), dim3(kCBlock), 0, stream(), dy, dyp, c);
     rc = BH_LAUNCH_CHECK("nchw_to_cnhw_kernel");
     if (rc == BH_OK && gb) {
         int64_t chunks = ceil_div(512, c.oc);                       // about two workgroups per compute unit ...
@@ -399,8 +393,7 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
         if (!col) rc = BH_ENOMEM;
     }
     if (rc == BH_OK && gw) {
-        if (fits32(positions * kk)) hipLaunchKernelGGL(im2col_kernel<unsigned>, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions, positions * kk);
-        else hipLaunchKernelGGL(im2col_kernel<int64_t>, blocks(positions * kk), dim3(kCBlock), 0, stream(), x, col, c, positions, positions * kk);
+        hipLaunchKernelGGL(im2col_kernel, dim3(per_blocks, (unsigned)kk, (unsigned)c.batch), dim3(kCBlock), 0, stream(), x, col, c, positions);
         rc = BH_LAUNCH_CHECK("im2col_kernel");
         // gw[oc][kk] (+)= dyp[oc][positions] . col[kk][positions]^T : both operands contiguous along the contraction
         if (rc == BH_OK) rc = bh_gemm(0, 1, c.oc, kk, positions, dyp, positions, col, positions, gw, kk, nullptr, accumulate, 1);
@@ -419,9 +412,8 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
         // dcol[kk][positions] = w^T[kk][oc] . dyp[oc][positions]  (the stream orders it after the gw product that read col)
         if (rc == BH_OK) rc = bh_gemm(1, 0, kk, positions, c.oc, wsrc, kk, dyp, positions, col, positions, nullptr, 0, 1);
         if (rc == BH_OK) {
-            const int64_t total = (int64_t)c.batch * c.ic * c.h * c.w;
-            if (fits32(total) && fits32(positions * kk)) hipLaunchKernelGGL(col2im_kernel<unsigned>, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, positions, total);
-            else hipLaunchKernelGGL(col2im_kernel<int64_t>, blocks(total), dim3(kCBlock), 0, stream(), col, dx, c, positions, total);
+            hipLaunchKernelGGL(col2im_kernel, dim3((unsigned)ceil_div((int64_t)c.h * c.w, kCBlock), (unsigned)c.ic, (unsigned)c.batch),
+                               dim3(kCBlock), 0, stream(), col, dx, c, positions);
             rc = BH_LAUNCH_CHECK("col2im_kernel");
         }
     }

@@ -233,13 +233,14 @@ struct PoolShape {
 };
 
 // first maximum in row-major scan order wins (strict >, pool.c:118-123); index is the offset inside the plane, -1 if none
+// grid (planes, ceil(ho*wo/256)): the plane comes from the grid, a lane splits only its position inside the plane
 __global__ __launch_bounds__(kCBlock) void maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
-                                                              int32_t* __restrict__ idx, PoolShape p, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= total) return;
-    const int ow = (int)(i % p.wo);
-    const int oh = (int)((i / p.wo) % p.ho);
-    const int64_t plane = i / ((int64_t)p.wo * p.ho);
+                                                              int32_t* __restrict__ idx, PoolShape p) {
+    const unsigned q = blockIdx.y * kCBlock + threadIdx.x;
+    if (q >= (unsigned)(p.ho * p.wo)) return;
+    const int oh = (int)(q / (unsigned)p.wo), ow = (int)(q - (unsigned)oh * (unsigned)p.wo);
+    const int64_t plane = blockIdx.x;
+    const int64_t i = plane * p.ho * p.wo + q;
     const float* xp = x + plane * p.h * p.w;
     int h0 = oh * p.stride - p.pad, w0 = ow * p.stride - p.pad;
     int h1 = h0 + p.pool, w1 = w0 + p.pool;
@@ -264,12 +265,12 @@ __global__ __launch_bounds__(kCBlock) void maxpool_fwd_kernel(const float* __res
 // dx[plane, ih, iw] = sum of dy over the windows whose maximum sits at (ih, iw), visited in increasing output
 // index, which is the order in which the reference's scatter loop adds them (pool.c:207-212)
 __global__ __launch_bounds__(kCBlock) void maxpool_bwd_kernel(const float* __restrict__ dy, const int32_t* __restrict__ idx,
-                                                              float* __restrict__ dx, PoolShape p, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * kCBlock + threadIdx.x;
-    if (i >= total) return;
-    const int iw = (int)(i % p.w);
-    const int ih = (int)((i / p.w) % p.h);
-    const int64_t plane = i / ((int64_t)p.w * p.h);
+                                                              float* __restrict__ dx, PoolShape p) {
+    const unsigned q = blockIdx.y * kCBlock + threadIdx.x;     // grid (planes, ceil(h*w/256))
+    if (q >= (unsigned)(p.h * p.w)) return;
+    const int ih = (int)(q / (unsigned)p.w), iw = (int)(q - (unsigned)ih * (unsigned)p.w);
+    const int64_t plane = blockIdx.x;
+    const int64_t i = plane * p.h * p.w + q;
     const int me = ih * p.w + iw;
     // windows covering row ih: oh*stride - pad <= ih < oh*stride - pad + pool
     int oh_lo = ih + p.pad - p.pool + 1;
@@ -441,9 +442,9 @@ int bh_maxpool2d_forward(const float* x, float* y, int32_t* argmax, int64_t plan
     if (rc) return rc;
     if (planes == 0) return BH_OK;
     BH_CHECK_ARG(x && y && argmax, "null pointer");
-    const int64_t total = planes * p.ho * p.wo;
-    BH_CHECK_ARG(ceil_div(total, kCBlock) <= 0x7fffffff, "tensor too large");
-    hipLaunchKernelGGL(maxpool_fwd_kernel, dim3((unsigned)ceil_div(total, kCBlock)), dim3(kCBlock), 0, stream(), x, y, argmax, p, total);
+    const int64_t per_blocks = ceil_div((int64_t)p.ho * p.wo, kCBlock);
+    BH_CHECK_ARG(planes <= 0x7fffffff && per_blocks <= 65535, "tensor too large");
+    hipLaunchKernelGGL(maxpool_fwd_kernel, dim3((unsigned)planes, (unsigned)per_blocks), dim3(kCBlock), 0, stream(), x, y, argmax, p);
     return BH_LAUNCH_CHECK("maxpool_fwd_kernel");
 }
 
@@ -455,9 +456,9 @@ int bh_maxpool2d_backward(const float* dy, const int32_t* argmax, float* dx, int
     if (rc) return rc;
     if (planes == 0) return BH_OK;
     BH_CHECK_ARG(dy && argmax && dx, "null pointer");
-    const int64_t total = planes * p.h * p.w;
-    BH_CHECK_ARG(ceil_div(total, kCBlock) <= 0x7fffffff, "tensor too large");
-    hipLaunchKernelGGL(maxpool_bwd_kernel, dim3((unsigned)ceil_div(total, kCBlock)), dim3(kCBlock), 0, stream(), dy, argmax, dx, p, total);
+    const int64_t per_blocks = ceil_div((int64_t)p.h * p.w, kCBlock);
+    BH_CHECK_ARG(planes <= 0x7fffffff && per_blocks <= 65535, "tensor too large");
+    hipLaunchKernelGGL(maxpool_bwd_kernel, dim3((unsigned)planes, (unsigned)per_blocks), dim3(kCBlock), 0, stream(), dy, argmax, dx, p);
     return BH_LAUNCH_CHECK("maxpool_bwd_kernel");
 }
 

@@ -155,18 +155,26 @@ __global__ __launch_bounds__(kCBlock) void nchw_to_cnhw_kernel(const float* __re
 
 // col[(ic, kh, kw)][(b, oh, ow)] = x[b, ic, oh*stride - pad + kh, ow*stride - pad + kw], zero outside the image.
 // The output position is the fast index of the patch matrix: neighbouring lanes read neighbouring pixels and write
-// neighbouring elements.  grid (ceil(per/256), ic*k*k, batch)
+// neighbouring elements.  grid (ceil(per/256), ic, batch); a lane writes all k*k taps of its position and channel
+// (one workgroup per tap made the launch itself the cost: 18432 workgroups of one element per lane).
 __global__ __launch_bounds__(kCBlock) void im2col_kernel(const float* __restrict__ x, float* __restrict__ col, ConvShape c,
                                                          int64_t positions) {
     const unsigned per = (unsigned)(c.ho * c.wo);
     const unsigned p = blockIdx.x * kCBlock + threadIdx.x;
     if (p >= per) return;
-    const int t = blockIdx.y, b = blockIdx.z;                     // uniform over the workgroup
-    const int kw = t % c.k, kh = (t / c.k) % c.k, ci = t / (c.k * c.k);
+    const int ci = blockIdx.y, b = blockIdx.z;                    // uniform over the workgroup
     const int oh = (int)(p / (unsigned)c.wo), ow = (int)(p - (unsigned)oh * (unsigned)c.wo);
-    const int ih = oh * c.stride - c.pad + kh, iw = ow * c.stride - c.pad + kw;
-    const bool inside = ih >= 0 && ih < c.h && iw >= 0 && iw < c.w;
-    col[(int64_t)t * positions + (int64_t)b * per + p] = inside ? x[(((int64_t)b * c.ic + ci) * c.h + ih) * c.w + iw] : 0.f;
+    const int ih0 = oh * c.stride - c.pad, iw0 = ow * c.stride - c.pad;
+    const float* xp = x + ((int64_t)b * c.ic + ci) * c.h * c.w;
+    float* out = col + (int64_t)ci * c.k * c.k * positions + (int64_t)b * per + p;
+    for (int kh = 0; kh < c.k; kh++) {
+        const int ih = ih0 + kh;
+        for (int kw = 0; kw < c.k; kw++) {
+            const int iw = iw0 + kw;
+            const bool inside = ih >= 0 && ih < c.h && iw >= 0 && iw < c.w;
+            out[(int64_t)(kh * c.k + kw) * positions] = inside ? xp[ih * c.w + iw] : 0.f;
+        }
+    }
 }
 
 // dx[b, ic, ih, iw] = sum over the taps (kh, kw) whose output position (oh, ow) exists of dcol[(ic, kh, kw)][(b, oh, ow)];
@@ -362,7 +370,7 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
     if (!dx && !gw && !gb) return BH_OK;
     auto blocks = [](int64_t n) { return dim3((unsigned)ceil_div(n, kCBlock)); };
     // the rearrangement kernels carry channel and batch indices in grid.y / grid.z
-    BH_CHECK_ARG(c.oc <= 65535 && c.batch <= 65535 && kk <= 65535 && c.ic <= 65535, "conv2d backward: more than 65535 channels, taps or images");
+    BH_CHECK_ARG(c.oc <= 65535 && c.batch <= 65535 && c.ic <= 65535, "conv2d backward: more than 65535 channels or images");
     float *dyp = nullptr, *col = nullptr, *wf = nullptr;
     dyp = (float*)bh_malloc(sizeof(float) * (size_t)(c.oc * positions));
     if (!dyp) return BH_ENOMEM;
@@ -394,7 +402,7 @@ int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* d
         if (!col) rc = BH_ENOMEM;
     }
     if (rc == BH_OK && gw) {
-        hipLaunchKernelGGL(im2col_kernel, dim3(per_blocks, (unsigned)kk, (unsigned)c.batch), dim3(kCBlock), 0, stream(), x, col, c, positions);
+        hipLaunchKernelGGL(im2col_kernel, dim3(per_blocks, (unsigned)c.ic, (unsigned)c.batch), dim3(kCBlock), 0, stream(), x, col, c, positions);
         rc = BH_LAUNCH_CHECK("im2col_kernel");
         // gw[oc][kk] (+)= dyp[oc][positions] . col[kk][positions]^T : both operands contiguous along the contraction
         if (rc == BH_OK) rc = bh_gemm(0, 1, c.oc, kk, positions, dyp, positions, col, positions, gw, kk, nullptr, accumulate, 1);

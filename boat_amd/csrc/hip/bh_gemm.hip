@@ -1014,8 +1014,9 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
             GemmArgs run = g;
             float* ws = nullptr;
             if (tiny_split) {
-                g.k_per_split = 512;
-                g.k_splits = (int)ceil_div(k, 512);
+                // one trip (512 k) per workgroup unless that makes more workgroups than the chip holds at once
+                g.k_per_split = tiles32 * ceil_div(k, 512) > 384 ? 1024 : 512;
+                g.k_splits = (int)ceil_div(k, g.k_per_split);
                 ws = (float*)bh_malloc(sizeof(float) * (size_t)(g.k_splits * batch * m * n));
                 if (!ws) return BH_ENOMEM;
                 run = g;

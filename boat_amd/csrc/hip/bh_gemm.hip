@@ -986,7 +986,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     // 6-10 us up to k = 1024; one k-fast operand 7.5-8 us up to k = 512 (one trip) and 12 us up to 1024 (two trips);
     // two k-fast operands 9-11 us up to k = 512 and slower beyond.
     const int64_t tiles32 = ceil_div(m, 32) * ceil_div(n, 32) * batch;
-    if (k > 0 && m * n * k <= ((int64_t)1 << 24) && tiles32 <= 512 &&
+    if (k > 0 && m * n * k <= ((int64_t)1 << (k <= 128 ? 25 : 24)) && tiles32 <= 512 &&
         (k <= 512 || (k <= 1024 && !(a_kc && b_kc)) || (!a_kc && !b_kc)))
         cfg = 6;
     // A small output with a very long contraction over k-fast operands (the weight gradient of a convolution: 64 x 288

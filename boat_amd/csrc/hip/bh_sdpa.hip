@@ -8,9 +8,12 @@
 // with A recomputed as exp(score - lse).  The row term rowsum(dA*A) is evaluated as
 // rowsum(dO*O), which is the same number (A.V = O) without needing A.
 //
-// Two implementations behind one entry point:
+// Three implementations behind one entry point:
 //   * general kernels (any s, d): one workgroup per query row (forward, dQ) or per key row
 //     (dK, dV); scores of one row live in LDS.
+//   * the reference's own decomposition on the matrix cores for any other shape with s >= 64: batched GEMMs through
+//     bh_gemm for Q.K^T, P.V, P^T.dO, dO.V^T, dS.K, dS^T.Q with row kernels for softmax and dS in between; the [s, s]
+//     matrices exist for a bounded chunk of heads at a time.
 //   * MFMA kernels for d == 64 and s >= 32 (the shapes of the attention benchmarks; a length that is not a
 //     multiple of 128 is handled by clamped loads, masked scores and guarded stores).
 #include "bh_common.h"
@@ -171,6 +174,107 @@ __global__ __launch_bounds__(kSBlock) void sdpa_bwd_dkv_row_kernel(const float* 
     }
 }
 
+// ---- row kernels of the GEMM-based path: one workgroup per row of a [rows][s] score matrix (row = head*s + query) ----
+
+// in place: P = softmax(scale * S) with keys after the query masked; lse = max + log(sum)
+__global__ __launch_bounds__(kSBlock) void sdpa_softmax_rows_kernel(float* __restrict__ sc, float* __restrict__ lse, int64_t s,
+                                                                    float scale, int causal) {
+    __shared__ float red[kSBlock / 64];
+    const int64_t row = blockIdx.x, i = row % s;
+    float* p = sc + row * s;
+    const int64_t lim = causal ? i + 1 : s;            // keys j < lim are visible
+    float mx = -FLT_MAX;
+    for (int64_t j = threadIdx.x; j < lim; j += kSBlock) mx = fmaxf(mx, p[j] * scale);
+    mx = block_max<kSBlock / 64>(mx, red);
+    float sum = 0.f;
+    for (int64_t j = threadIdx.x; j < lim; j += kSBlock) sum += expf(p[j] * scale - mx);
+    sum = block_sum<kSBlock / 64>(sum, red);
+    const float inv = 1.0f / sum;
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) p[j] = j < lim ? expf(p[j] * scale - mx) * inv : 0.f;
+    if (threadIdx.x == 0 && lse) lse[row] = mx + logf(sum);
+}
+
+// in place: P = exp(scale * S - lse), masked keys 0
+__global__ __launch_bounds__(kSBlock) void sdpa_probs_rows_kernel(float* __restrict__ sc, const float* __restrict__ lse, int64_t s,
+                                                                  float scale, int causal) {
+    const int64_t row = blockIdx.x, i = row % s;
+    float* p = sc + row * s;
+    const float l = lse[row];
+    const int64_t lim = causal ? i + 1 : s;
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) p[j] = j < lim ? expf(p[j] * scale - l) : 0.f;
+}
+
+// in place on dP: dS = P * (dP - delta) * scale
+__global__ __launch_bounds__(kSBlock) void sdpa_ds_rows_kernel(const float* __restrict__ prob, float* __restrict__ dp,
+                                                               const float* __restrict__ delta, int64_t s, float scale) {
+    const int64_t row = blockIdx.x;
+    const float dl = delta[row];
+    const float* p = prob + row * s;
+    float* g = dp + row * s;
+    for (int64_t j = threadIdx.x; j < s; j += kSBlock) g[j] = p[j] * (g[j] - dl) * scale;
+}
+
+// heads per pass of the GEMM-based path: the [heads, s, s] matrices of one pass stay under 1 GiB each
+static int64_t heads_per_pass(int64_t bh_count, int64_t s) {
+    int64_t h = ((int64_t)1 << 28) / (s * s);
+    if (h < 1) h = 1;
+    if (h > 32768) h = 32768;                          // bh_gemm's batch limit with room to spare
+    return h < bh_count ? h : bh_count;
+}
+
+static int sdpa_forward_gemm(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
+                             float* attn_out, int64_t bh_count, int64_t s, int64_t d) {
+    const int64_t hp = heads_per_pass(bh_count, s);
+    float* scratch = attn_out ? nullptr : (float*)bh_malloc(sizeof(float) * (size_t)(hp * s * s));
+    if (!attn_out && !scratch) return BH_ENOMEM;
+    int rc = BH_OK;
+    for (int64_t h0 = 0; h0 < bh_count && rc == BH_OK; h0 += hp) {
+        const int64_t nh = bh_count - h0 < hp ? bh_count - h0 : hp;
+        float* sc = attn_out ? attn_out + h0 * s * s : scratch;
+        const int64_t off = h0 * s * d;
+        rc = bh_gemm(0, 1, s, s, d, q + off, d, k + off, d, sc, s, nullptr, 0, nh);              // S = Q.K^T
+        if (rc != BH_OK) break;
+        hipLaunchKernelGGL(sdpa_softmax_rows_kernel, dim3((unsigned)(nh * s)), dim3(kSBlock), 0, stream(), sc,
+                           lse ? lse + h0 * s : nullptr, s, scale, causal);
+        rc = BH_LAUNCH_CHECK("sdpa_softmax_rows_kernel");
+        if (rc == BH_OK) rc = bh_gemm(0, 0, s, d, s, sc, s, v + off, d, out + off, d, nullptr, 0, nh);   // O = P.V
+    }
+    if (scratch) bh_free(scratch);
+    return rc;
+}
+
+static int sdpa_backward_gemm(const float* q, const float* k, const float* v, const float* lse, const float* delta,
+                              const float* d_out, float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count,
+                              int64_t s, int64_t d) {
+    const int64_t hp = heads_per_pass(bh_count, s);
+    float* prob = (float*)bh_malloc(sizeof(float) * (size_t)(hp * s * s));
+    float* ds = prob ? (float*)bh_malloc(sizeof(float) * (size_t)(hp * s * s)) : nullptr;
+    if (!prob || !ds) {
+        if (prob) bh_free(prob);
+        return BH_ENOMEM;
+    }
+    int rc = BH_OK;
+    for (int64_t h0 = 0; h0 < bh_count && rc == BH_OK; h0 += hp) {
+        const int64_t nh = bh_count - h0 < hp ? bh_count - h0 : hp;
+        const int64_t off = h0 * s * d;
+        const dim3 rows((unsigned)(nh * s));
+        rc = bh_gemm(0, 1, s, s, d, q + off, d, k + off, d, prob, s, nullptr, 0, nh);            // S = Q.K^T
+        if (rc != BH_OK) break;
+        hipLaunchKernelGGL(sdpa_probs_rows_kernel, rows, dim3(kSBlock), 0, stream(), prob, lse + h0 * s, s, scale, causal);
+        rc = BH_LAUNCH_CHECK("sdpa_probs_rows_kernel");
+        if (rc == BH_OK) rc = bh_gemm(1, 0, s, d, s, prob, s, d_out + off, d, dv + off, d, nullptr, 0, nh);     // dV = P^T.dO
+        if (rc == BH_OK) rc = bh_gemm(0, 1, s, s, d, d_out + off, d, v + off, d, ds, s, nullptr, 0, nh);        // dP = dO.V^T
+        if (rc != BH_OK) break;
+        hipLaunchKernelGGL(sdpa_ds_rows_kernel, rows, dim3(kSBlock), 0, stream(), prob, ds, delta + h0 * s, s, scale);
+        rc = BH_LAUNCH_CHECK("sdpa_ds_rows_kernel");
+        if (rc == BH_OK) rc = bh_gemm(0, 0, s, d, s, ds, s, k + off, d, dq + off, d, nullptr, 0, nh);           // dQ = dS.K
+        if (rc == BH_OK) rc = bh_gemm(1, 0, s, d, s, ds, s, q + off, d, dk + off, d, nullptr, 0, nh);           // dK = dS^T.Q
+    }
+    bh_free(ds);
+    bh_free(prob);
+    return rc;
+}
+
 }  // namespace bh
 
 using namespace bh;
@@ -187,7 +291,7 @@ static int g_sdpa_force_general = 0;
 
 extern "C" {
 
-// test hook: 1 forces the general kernels even where the MFMA path applies
+// test hook: 1 forces the row kernels, 2 the GEMM-based path, even where the fused MFMA kernels apply; 0 = heuristic
 int bh_sdpa_force_general(int on) {
     g_sdpa_force_general = on;
     return BH_OK;
@@ -203,6 +307,9 @@ int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale,
         int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, bh_count, s, d);
         if (rc <= 0) return rc;   // 0 done, <0 error, 1 shape not covered
     }
+    // from 64 keys on the six products are worth a trip through the matrix cores
+    if (g_sdpa_force_general == 2 || (g_sdpa_force_general == 0 && s >= 64 && s <= 16384))
+        return sdpa_forward_gemm(q, k, v, scale, causal, out, lse, attn_out, bh_count, s, d);
     BH_CHECK_ARG(bh_count <= 65535, "too many head blocks for the general attention kernel");
     BH_CHECK_ARG(s + d <= kMaxRowFloats, "sequence too long for the general attention kernel");
     const size_t shmem = sizeof(float) * (size_t)(s + d);
@@ -228,6 +335,10 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
         if (!g_sdpa_force_general)
             done = sdpa_backward_mfma(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);
         if (done < 0) rc = done;
+        if (done == 1 && (g_sdpa_force_general == 2 || (g_sdpa_force_general == 0 && s >= 64 && s <= 16384))) {
+            rc = sdpa_backward_gemm(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);
+            done = 0;
+        }
         if (done == 1) {
             if (2 * s + 2 * d > kMaxRowFloats || bh_count > 65535) {
                 bh_free(delta);

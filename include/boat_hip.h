@@ -189,7 +189,8 @@ int bh_zero_multi(float* const* p, const int64_t* n, int count);
  * into the MFMA registers, contraction split among a workgroup's wavefronts), -1 = heuristic (default).
  * bh_gemm_force_direct: 0 = MFMA tiles stage their operands through registers; 1 or -1 (default) = operands go
  * straight to LDS (global_load_lds) whenever the contraction length is a multiple of 16.
- * bh_sdpa_force_general: 1 = always use the general attention kernels. */
+ * bh_sdpa_force_general: 0 = heuristic (default); 1 = always the row kernels; 2 = always the GEMM-based path (batched
+ * bh_gemm products with row kernels for softmax and dS in between, what shapes other than head_dim 64 use from 64 keys on). */
 int bh_gemm_force_config(int cfg);
 int bh_gemm_force_direct(int mode);
 int bh_sdpa_force_general(int on);

@@ -441,13 +441,13 @@ def test_transpose(hip, oracle, rng):
 
 # ---------------------------------------------------------------- attention
 
-SDPA_SHAPES = [(8, 4, 8), (4, 16, 16), (2, 8, 8), (3, 33, 20), (2, 64, 64), (4, 128, 64), (2, 256, 64), (3, 100, 64),
+SDPA_SHAPES = [(8, 4, 8), (4, 16, 16), (2, 8, 8), (3, 33, 20), (2, 64, 64), (3, 130, 32), (2, 200, 128), (2, 96, 20), (4, 128, 64), (2, 256, 64), (3, 100, 64),
                (2, 512, 64), (1, 1024, 64), (2, 32, 64), (2, 77, 64), (1, 129, 64), (2, 191, 64), (1, 1000, 64)]
 
 
 @pytest.mark.parametrize("causal", [0, 1])
 @pytest.mark.parametrize("bh,s,d", SDPA_SHAPES)
-@pytest.mark.parametrize("general", [0, 1])
+@pytest.mark.parametrize("general", [0, 1, 2])      # heuristic; row kernels; GEMM-based path
 def test_sdpa_forward_backward(hip, oracle, rng, bh, s, d, causal, general):
     q, k, v, go = (rng.standard_normal((bh, s, d)).astype(np.float32) for _ in range(4))
     scale = float(np.float32(1.0) / np.sqrt(np.float32(d)))
@@ -468,14 +468,15 @@ def test_sdpa_forward_backward(hip, oracle, rng, bh, s, d, causal, general):
     assert rel_fro(gq.numpy(), wdq) <= TOL_GEMM and rel_fro(gk.numpy(), wdk) <= TOL_GEMM and rel_fro(gv.numpy(), wdv) <= TOL_GEMM
 
 
-def test_sdpa_attention_matrix_output(hip, oracle, rng):
-    bh, s, d = 3, 12, 8
+@pytest.mark.parametrize("bh,s,d", [(3, 12, 8), (2, 80, 24)])      # row kernels; GEMM-based path (s >= 64)
+def test_sdpa_attention_matrix_output(hip, oracle, rng, bh, s, d):
     q, k, v = (rng.standard_normal((bh, s, d)).astype(np.float32) for _ in range(3))
     out, lse, attn = hip.empty((bh, s, d)), hip.empty((bh, s)), hip.empty((bh, s, s))
-    hip.check(hip.bh_sdpa_forward(dev(hip, q).ptr, dev(hip, k).ptr, dev(hip, v).ptr, 0.35, 0, out.ptr, lse.ptr, attn.ptr, bh, s, d))
-    _, _, wattn = oracle.sdpa_forward(q, k, v, 0.35)
+    hip.check(hip.bh_sdpa_forward(dev(hip, q).ptr, dev(hip, k).ptr, dev(hip, v).ptr, 0.35, 1, out.ptr, lse.ptr, attn.ptr, bh, s, d))
+    wo, _, wattn = oracle.sdpa_forward(q, k, v, 0.35, 1)
     assert np.max(np.abs(attn.numpy() - wattn)) <= 1e-6
     assert np.allclose(attn.numpy().sum(-1), 1.0, atol=1e-5)
+    assert rel_fro(out.numpy(), wo) <= TOL_GEMM
 
 
 def test_sdpa_more_head_blocks_than_a_grid_dimension_holds(hip, oracle, rng):

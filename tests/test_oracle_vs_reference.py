@@ -272,6 +272,8 @@ ATT_CASES = [
     dict(B=2, S=4, H=32, heads=4, causal=True, bias=True),
     dict(B=1, S=16, H=64, heads=4, causal=False, bias=False),
     dict(B=1, S=16, H=64, heads=4, causal=True, bias=True),
+    dict(B=2, S=70, H=96, heads=3, causal=True, bias=True),     # head size 32 from 64 keys on: the GEMM-based device path
+    dict(B=1, S=40, H=128, heads=2, causal=False, bias=True),   # head size 64, 40 keys: the fused device kernels, ragged length
 ]
 
 

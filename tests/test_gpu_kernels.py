@@ -479,6 +479,36 @@ def test_sdpa_attention_matrix_output(hip, oracle, rng, bh, s, d):
     assert rel_fro(out.numpy(), wo) <= TOL_GEMM
 
 
+@pytest.mark.parametrize("general", [0, 1, 2])
+@pytest.mark.parametrize("causal", [0, 1])
+def test_sdpa_large_scores_stay_finite(hip, oracle, rng, causal, general):
+    """Scores of several hundred (one key dominates each row, most exponentials underflow): max-subtracted softmax in
+    every path, so outputs, log-sum-exp and gradients stay finite and match the float64-accurate oracle."""
+    bh, s, d = 2, 160, 64
+    q, k, v, go = (rng.standard_normal((bh, s, d)).astype(np.float32) for _ in range(4))
+    q *= 9.0
+    k *= 9.0
+    scale = 1.0
+    wo, wlse, wattn = oracle.sdpa_forward(q, k, v, scale, causal)
+    wdq, wdk, wdv = oracle.sdpa_backward(q, k, v, wattn, go, scale)
+    assert np.abs(wlse).max() > 300
+    dq_, dk_, dv_ = dev(hip, q), dev(hip, k), dev(hip, v)
+    out, lse = hip.empty((bh, s, d)), hip.empty((bh, s))
+    gq, gk, gv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
+    hip.bh_sdpa_force_general(general)
+    try:
+        hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, causal, out.ptr, lse.ptr, None, bh, s, d))
+        hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, out.ptr, lse.ptr, dev(hip, go).ptr, scale, causal,
+                                       gq.ptr, gk.ptr, gv.ptr, bh, s, d))
+    finally:
+        hip.bh_sdpa_force_general(0)
+    for got, want in ((out, wo), (gq, wdq), (gk, wdk), (gv, wdv)):
+        g = got.numpy()
+        assert np.isfinite(g).all()
+        assert rel_fro(g, want) <= TOL_GEMM
+    assert np.max(np.abs(lse.numpy() - wlse)) <= 1e-4 * np.abs(wlse).max()
+
+
 def test_sdpa_more_head_blocks_than_a_grid_dimension_holds(hip, oracle, rng):
     """66000 [32, 64] blocks: the MFMA kernels number their workgroups along one grid dimension, so the 65535 limit of the
     other two does not apply; first and last blocks against float64, forward and backward."""

@@ -469,6 +469,71 @@ def cpu_baseline():
     }
 
 
+def cpu_beside_other_configs():
+    """The CPU path timed beside the other configurations, each on a bounded sample on ONE host core (a few seconds in
+    total): the compiled reference where it has the routine, the oracle's restatement where the reference has a stub."""
+    sys.path.insert(0, str(ROOT / "tests"))
+    import oracle_lib
+    import boat_cases as bc
+    out = {}
+    rng = np.random.default_rng(5)
+    oracle = oracle_lib.load()
+    ref = oracle_lib.load_reference()
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    # config 5b, flat Adam: 2^24 parameters, scaled by element count
+    n = 1 << 24
+    p, g = (rng.standard_normal(n, dtype=np.float32) for _ in range(2))
+    if ref is not None:
+        tp, tg = ref.tensor(p), ref.tensor(g)
+        opt = ref.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
+        ref.boat_optimizer_add_parameter(opt, tp, tg)
+        sec = timed(lambda: ref.boat_optimizer_step(opt))
+        ref.boat_optimizer_free(opt)
+        ref.boat_tensor_unref(tp)
+        ref.boat_tensor_unref(tg)
+        what = "boat_optimizer_step (Adam) of the compiled reference"
+    else:
+        m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        sec = timed(lambda: oracle.adam_update(p.copy(), g, m, v, 1e-3, 0.9, 0.999, 1e-8, 0))
+        what = "oracle adam_update"
+    out["adam_flat_268M"] = {"ms_extrapolated": round(sec * 1e3 * 268435456 / n, 1), "sample": f"{what} on {n} parameters: {sec * 1e3:.1f} ms"}
+    # config 3: the reference has stubs for both kernels; float64 restatements of the oracle on 512 x 4096
+    rows, hidden = 512, 4096
+    x, dy = (rng.standard_normal((rows, hidden), dtype=np.float32) for _ in range(2))
+    gamma = rng.standard_normal(hidden, dtype=np.float32)
+    mean = x.mean(1).astype(np.float32)
+    rstd = (1.0 / np.sqrt(x.var(1) + 1e-5)).astype(np.float32)
+    sec = timed(lambda: oracle.layernorm_backward_f64(x, gamma, dy, mean, rstd))
+    out["layernorm_bwd_16384x4096"] = {"ms_extrapolated": round(sec * 1e3 * 16384 / rows, 1),
+                                       "sample": f"oracle layernorm_backward_f64 on {rows} x {hidden}: {sec * 1e3:.1f} ms (the reference's routine is a stub)"}
+    sec = timed(lambda: oracle.gelu_backward_f64(x, dy))
+    out["gelu_bwd_16384x4096"] = {"ms_extrapolated": round(sec * 1e3 * 16384 / rows, 1),
+                                  "sample": f"oracle gelu_backward_f64 on {rows} x {hidden}: {sec * 1e3:.1f} ms (the reference's routine is a stub)"}
+    # config 4: attention core backward, 4 blocks of S=256, D=64, scaled by flops (bh * S^2)
+    bh_, S, D = 4, 256, 64
+    q, k, v, go = (rng.standard_normal((bh_, S, D), dtype=np.float32) for _ in range(4))
+    _, _, attn = oracle.sdpa_forward(q, k, v, 0.125)
+    sec = timed(lambda: oracle.sdpa_backward(q, k, v, attn, go, 0.125))
+    out["sdpa_bwd_B8h16S1024D64"] = {"ms_extrapolated": round(sec * 1e3 * (128 * 1024 * 1024) / (bh_ * S * S), 1),
+                                     "sample": f"oracle sdpa_backward (loop-order restatement of src/layers/attention.c:1417-1520) on {bh_} blocks of S={S}: {sec * 1e3:.1f} ms"}
+    # config 1: the MLP step at full size
+    xb = rng.random((64, 784), dtype=np.float32)
+    labels = rng.integers(0, 10, 64)
+    w1 = (0.05 * rng.standard_normal((784, 128), dtype=np.float32)).astype(np.float32)
+    w2 = (0.05 * rng.standard_normal((128, 10), dtype=np.float32)).astype(np.float32)
+    b1, b2 = np.zeros(128, np.float32), np.zeros(10, np.float32)
+    if ref is not None:
+        steps = 5
+        sec = timed(lambda: bc.mlp_ce_adam(ref, xb, labels, w1, b1, w2, b2, steps=steps)) / steps
+        out["mlp_784_128_10_step"] = {"ms": round(sec * 1e3, 3), "sample": f"compiled reference, {steps} steps of the same tape chain through its C API (full size)"}
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -517,6 +582,8 @@ def main():
         line["extra"] = extra
     if not args.no_cpu and "dense" in legs:
         line["cpu_baseline"] = cpu_baseline()
+        if not args.no_extra:
+            line["cpu_beside_other_configs"] = cpu_beside_other_configs()
     print(json.dumps(line))
 
 

@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
 
-A step is one dense-layer backward at BASELINE config 2 (the GEMM-bound configuration the
+A step is one dense-layer backward at benchmark configuration 2 (the GEMM-bound configuration the
 metric is quoted on): X[8192x4096] ~N(0,1), W[4096x4096] ~N(0,0.02), dY[8192x4096] ~N(0,1);
 dX = dY.W^T, dW += X^T.dY, db += colsum(dY) -- the three launches bh_dense_backward makes,
 issued here one by one so that HIP events on the library stream can time the GEMM launches
@@ -554,7 +554,7 @@ def main():
         "metric": METRIC, "value": None, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "dense layer backward (BASELINE config 2): X[8192x4096], W[4096x4096], dY[8192x4096] -> dX, dW, db; "
+        "config": {"workload": "dense layer backward (benchmark configuration 2): X[8192x4096], W[4096x4096], dY[8192x4096] -> dX, dW, db; "
                                "549.76 GFLOP per step", "M": 8192, "K": 4096, "N": 4096,
                    "device": hip.bh_device_name().decode().strip(), "compute_units": hip.bh_device_cu_count()},
     }

@@ -1,4 +1,4 @@
-"""Pre-LN transformer encoder block training step (BASELINE config 5, scaled down): forward,
+"""Pre-LN transformer encoder block training step (benchmark configuration 5, scaled down): forward,
 boat_variable_backward and fused Adam over the block's 16 parameter tensors.
 
 The expected values are composed from oracle primitives that are each pinned to the compiled

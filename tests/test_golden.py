@@ -297,7 +297,7 @@ def test_gpu_mlp_golden(boat):
 
 @pytest.mark.gpu
 def test_gpu_mlp_config1_golden(boat):
-    """BASELINE config 1 at its real size: MLP 784-128-10, batch 64, forward + backward + one Adam step."""
+    """Benchmark configuration 1 at its real size: MLP 784-128-10, batch 64, forward + backward + one Adam step."""
     g = load("mlp_config1_step")
     x, labels, w1, b1, w2, b2, chk = config1_inputs(g)
     rec = bc.mlp_ce_adam(boat, x, labels, w1, b1, w2, b2, steps=1)[0]

@@ -199,3 +199,35 @@ def test_config5a_block_step_full_size_batch_independence(boat):
         acc_w2 += one["g_w2"]
         acc_bq += one["g_bq"]
     assert rel_fro(full["g_w2"] * B, acc_w2) <= TOL_GEMM and rel_fro(full["g_bq"] * B, acc_bq) <= TOL_GEMM
+
+
+def test_more_than_two_to_the_31_elements(hip):
+    """Flat kernels past the 32-bit element count (2^31 + 4099 floats, 8.6 GB per array): fill, scale, Adam and the
+    sum reduction index with 64 bits.  Checked through the tail of the arrays and through sums with known values."""
+    n = (1 << 31) + 4099
+    tail = 4099 + 1024
+
+    def tail_of(arr):
+        out = np.empty(tail, np.float32)
+        hip.check(hip.lib.bh_memcpy_d2h(out.ctypes.data, arr.ptr + 4 * (n - tail), 4 * tail), "d2h tail")
+        return out
+
+    p, g, m, v = (hip.empty((n,)) for _ in range(4))
+    hip.check(hip.bh_fill(p.ptr, 0.5, n))
+    hip.check(hip.bh_fill(g.ptr, 0.25, n))
+    hip.check(hip.lib.bh_memset_zero(m.ptr, 4 * n))
+    hip.check(hip.lib.bh_memset_zero(v.ptr, 4 * n))
+    assert np.all(tail_of(p) == 0.5) and np.all(tail_of(v) == 0.0)
+    total = hip.empty((1,))
+    hip.check(hip.bh_sum_all(g.ptr, total.ptr, n))
+    assert abs(float(total.numpy()[0]) - 0.25 * n) <= 1e-6 * 0.25 * n          # partial sums of 0.25 are exact until the final adds
+    hip.check(hip.bh_scalar_op(2, g.ptr, 2.0, g.ptr, n))                       # g *= 2, in place
+    assert np.all(tail_of(g) == 0.5)
+    # first Adam step from zero moments: p -= lr * g / (|g| + eps) up to rounding, the same number everywhere
+    hip.check(hip.bh_adam_update(p.ptr, g.ptr, m.ptr, v.ptr, n, 0.01, 0.9, 0.999, 1e-8, 0))
+    pt, mt, vt = tail_of(p), tail_of(m), tail_of(v)
+    assert np.all(pt == pt[0]) and abs(float(pt[0]) - 0.49) < 1e-6
+    assert np.all(mt == mt[0]) and abs(float(mt[0]) - 0.05) < 1e-7 and np.all(vt == vt[0]) and abs(float(vt[0]) - 0.00025) < 1e-8
+    first = np.empty(8, np.float32)
+    hip.check(hip.lib.bh_memcpy_d2h(first.ctypes.data, p.ptr, 32), "d2h head")
+    assert np.all(first == pt[0])

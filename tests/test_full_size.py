@@ -231,3 +231,37 @@ def test_more_than_two_to_the_31_elements(hip):
     first = np.empty(8, np.float32)
     hip.check(hip.lib.bh_memcpy_d2h(first.ctypes.data, p.ptr, 32), "d2h head")
     assert np.all(first == pt[0])
+
+
+def test_gemm_operand_and_result_past_two_to_the_31_elements(hip):
+    """GEMM addressing with 64-bit offsets: an A operand and a C result of 2.29e9 elements each.  Rows of A below and
+    above the 2^31-element mark hold different constants, so an offset that wrapped would show as the wrong multiple
+    of the column sums of B."""
+    rng = np.random.default_rng(11)
+    m, k, n = 70000, 32768, 64
+    split = 66000                                         # row 65536 starts at element 2^31
+    a = hip.empty((m, k))
+    hip.check(hip.bh_fill(a.ptr, 1.0, split * k))
+    hip.check(hip.bh_fill(a.ptr + 4 * split * k, 2.0, (m - split) * k))
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    db = hip.to_device(b)
+    c = hip.empty((m, n))
+    hip.check(hip.bh_gemm(0, 0, m, n, k, a.ptr, k, db.ptr, n, c.ptr, n, None, 0, 1))
+    got = c.numpy()
+    colsum = b.astype(np.float64).sum(0)
+    scale = np.abs(b).astype(np.float64).sum(0).max()
+    assert np.abs(got[:split] - colsum).max() <= 1e-5 * scale
+    assert np.abs(got[split:] - 2 * colsum).max() <= 2e-5 * scale
+    del a, c
+    # a result of m x k2 elements past 2^31: C = A2 . B2 with a short contraction; check the first and the last rows
+    k2, n2 = 16, 32768
+    a2 = rng.standard_normal((m, k2)).astype(np.float32)
+    b2 = rng.standard_normal((k2, n2)).astype(np.float32)
+    c2 = hip.empty((m, n2))
+    da2, db2 = hip.to_device(a2), hip.to_device(b2)
+    hip.check(hip.bh_gemm(0, 0, m, n2, k2, da2.ptr, k2, db2.ptr, n2, c2.ptr, n2, None, 0, 1))
+    for r0 in (0, 65530, m - 8):
+        rows = np.empty((8, n2), np.float32)
+        hip.check(hip.lib.bh_memcpy_d2h(rows.ctypes.data, c2.ptr + 4 * r0 * n2, rows.nbytes), "d2h rows")
+        want = a2[r0:r0 + 8].astype(np.float64) @ b2.astype(np.float64)
+        assert np.abs(rows - want).max() <= 1e-5 * np.abs(want).max()

@@ -28,6 +28,12 @@ _DT = {np.dtype(v): k for k, v in _NP.items()}
 P = C.c_void_p
 
 
+class MemoryStats(C.Structure):
+    """boat_memory_stats_t (returned by value)."""
+    _fields_ = [("allocated_bytes", C.c_size_t), ("allocated_blocks", C.c_size_t), ("peak_allocated_bytes", C.c_size_t),
+                ("freed_bytes", C.c_size_t), ("freed_blocks", C.c_size_t)]
+
+
 class AttentionConfig(C.Structure):  # include/boat/layers/attention.h:21-30
     _fields_ = [("hidden_size", C.c_size_t), ("num_heads", C.c_size_t), ("head_size", C.c_size_t),
                 ("dropout_prob", C.c_float), ("causal_mask", C.c_bool), ("use_bias", C.c_bool),
@@ -179,7 +185,7 @@ _EXT_SIGS = {
     "boat_hip_optimizer_add_layernorm": (None, [P, P]),
     "boat_layernorm_update": (None, [P, C.c_float]),
     "boat_get_last_error_message": (C.c_char_p, []),
-    "boat_memory_get_stats": (None, []),
+    "boat_memory_get_stats": (MemoryStats, []),
 }
 
 

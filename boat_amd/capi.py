@@ -51,6 +51,8 @@ _SIGS = {
     # tensor
     "boat_tensor_create": (P, [C.POINTER(C.c_int64), C.c_size_t, C.c_int, C.c_int]),
     "boat_tensor_create_like": (P, [P]),
+    "boat_tensor_from_data": (P, [C.POINTER(C.c_int64), C.c_size_t, C.c_int, P]),
+    "boat_dtype_size": (C.c_size_t, [C.c_int]),
     "boat_tensor_free": (None, [P]),
     "boat_tensor_ref": (None, [P]),
     "boat_tensor_unref": (None, [P]),
@@ -96,6 +98,7 @@ _SIGS = {
     "boat_dense_layer_backward": (P, [P, P]),
     "boat_dense_layer_update": (None, [P, C.c_float]),
     "boat_dense_layer_get_weight": (P, [P]), "boat_dense_layer_get_bias": (P, [P]),
+    "boat_dense_layer_set_weight": (None, [P, P]), "boat_dense_layer_set_bias": (None, [P, P]),
     "boat_dense_layer_get_grad_weight": (P, [P]), "boat_dense_layer_get_grad_bias": (P, [P]),
     # conv / pool / flatten
     "boat_conv_layer_create": (P, [C.c_size_t] * 5), "boat_conv_layer_free": (None, [P]),

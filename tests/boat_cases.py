@@ -541,3 +541,127 @@ def loss_values(api, kind, pred, target, delta=1.0):
     api.boat_tensor_unref(tt)
     api.boat_loss_free(loss)
     return vals
+
+
+# ---- the example's weight checkpoint (examples/mnist/mnist_autodiff.c:775-995) over the C API ----
+CKPT_MAGIC, CKPT_VERSION = 0x4D4E4953, 1
+
+
+def _ckpt_write_tensor(api, f, t):
+    """save_tensor_to_file, mnist_autodiff.c:775-811: u32 null marker, u32 ndim, u32 dims, u32 dtype, raw payload."""
+    import struct
+    if not t:
+        f.write(struct.pack("<I", 1))
+        return
+    ndim = api.boat_tensor_ndim(t)
+    shape = api.boat_tensor_shape(t)
+    f.write(struct.pack("<II", 0, ndim))
+    f.write(struct.pack("<%dI" % ndim, *[shape[i] for i in range(ndim)]))
+    f.write(struct.pack("<I", api.boat_tensor_dtype(t)))
+    f.write(C.string_at(api.boat_tensor_const_data(t), api.boat_tensor_nbytes(t)))
+
+
+def _ckpt_read_tensor(api, f):
+    """load_tensor_from_file, mnist_autodiff.c:814-882: the payload goes through boat_tensor_from_data."""
+    import struct
+    (is_null,) = struct.unpack("<I", f.read(4))
+    if is_null:
+        return None
+    (ndim,) = struct.unpack("<I", f.read(4))
+    dims = struct.unpack("<%dI" % ndim, f.read(4 * ndim))
+    (dtype,) = struct.unpack("<I", f.read(4))
+    nbytes = int(np.prod(dims, dtype=np.int64)) * api.boat_dtype_size(dtype)
+    payload = f.read(nbytes)
+    assert len(payload) == nbytes
+    shape = (C.c_int64 * ndim)(*dims)
+    buf = C.create_string_buffer(payload, nbytes)
+    return api.boat_tensor_from_data(shape, ndim, dtype, C.cast(buf, C.c_void_p))
+
+
+class CnnLayers:
+    """conv1, pool, conv2, pool, flatten, fc1, fc2 of the MNIST example (mnist_autodiff.c:536-557), as layer objects."""
+
+    def __init__(self, api, p, pool=2):
+        self.api = api
+        self.c1 = _make_conv(api, p["cw1"], p["cb1"], 1, 1)
+        self.c2 = _make_conv(api, p["cw2"], p["cb2"], 1, 1)
+        self.p1, self.p2 = api.boat_pool_layer_create(pool, pool, 0), api.boat_pool_layer_create(pool, pool, 0)
+        self.fl = api.boat_flatten_layer_create()
+        self.d1 = _make_dense(api, p["w1"], p["b1"])
+        self.d2 = _make_dense(api, p["w2"], p["b2"])
+
+    def parameters(self):
+        a = self.api
+        return [(self.c1, "conv", a.boat_conv_layer_get_weight(self.c1), a.boat_conv_layer_get_bias(self.c1)),
+                (self.c2, "conv", a.boat_conv_layer_get_weight(self.c2), a.boat_conv_layer_get_bias(self.c2)),
+                (self.d1, "dense", a.boat_dense_layer_get_weight(self.d1), a.boat_dense_layer_get_bias(self.d1)),
+                (self.d2, "dense", a.boat_dense_layer_get_weight(self.d2), a.boat_dense_layer_get_bias(self.d2))]
+
+    def logits(self, x):
+        """Forward through the layer hooks (the chain of mnist_autodiff.c:2345-2412 without the tape)."""
+        a = self.api
+        t = [a.tensor(np.asarray(x, np.float32))]
+        for step in (lambda v: a.boat_conv_layer_forward(self.c1, v), a.boat_relu,
+                     lambda v: a.boat_pool_layer_forward(self.p1, v),
+                     lambda v: a.boat_conv_layer_forward(self.c2, v), a.boat_relu,
+                     lambda v: a.boat_pool_layer_forward(self.p2, v),
+                     lambda v: a.boat_flatten_layer_forward(self.fl, v),
+                     lambda v: a.boat_dense_layer_forward(self.d1, v), a.boat_relu,
+                     lambda v: a.boat_dense_layer_forward(self.d2, v)):
+            nxt = step(t[-1])
+            assert nxt, "a layer's forward failed"
+            t.append(nxt)
+        out = a.numpy(t[-1])
+        for h in t:
+            a.boat_tensor_unref(h)
+        return out
+
+    def save(self, path):
+        """save_mnist_model, mnist_autodiff.c:885-927."""
+        import struct
+        with open(path, "wb") as f:
+            f.write(struct.pack("<II", CKPT_MAGIC, CKPT_VERSION))
+            for _layer, _kind, w, b in self.parameters():
+                _ckpt_write_tensor(self.api, f, w)
+                _ckpt_write_tensor(self.api, f, b)
+
+    def load(self, path):
+        """load_mnist_model, mnist_autodiff.c:930-995: set_weight / set_bias swap the layer's tensors for the loaded ones."""
+        import struct
+        a = self.api
+        with open(path, "rb") as f:
+            magic, version = struct.unpack("<II", f.read(8))
+            if magic != CKPT_MAGIC or version != CKPT_VERSION:
+                return False
+            for layer, kind, _w, _b in self.parameters():
+                set_w = a.boat_conv_layer_set_weight if kind == "conv" else a.boat_dense_layer_set_weight
+                set_b = a.boat_conv_layer_set_bias if kind == "conv" else a.boat_dense_layer_set_bias
+                w, b = _ckpt_read_tensor(a, f), _ckpt_read_tensor(a, f)
+                if w:
+                    set_w(layer, w)
+                    a.boat_tensor_unref(w)
+                if b:
+                    set_b(layer, b)
+                    a.boat_tensor_unref(b)
+        return True
+
+    def free(self):
+        a = self.api
+        a.boat_conv_layer_free(self.c1)
+        a.boat_conv_layer_free(self.c2)
+        a.boat_pool_layer_free(self.p1)
+        a.boat_pool_layer_free(self.p2)
+        a.boat_flatten_layer_free(self.fl)
+        a.boat_dense_layer_free(self.d1)
+        a.boat_dense_layer_free(self.d2)
+
+
+def checkpoint_bytes(p):
+    """The checkpoint file of parameters p built without any library: what save_mnist_model must write."""
+    import struct
+    out = [struct.pack("<II", CKPT_MAGIC, CKPT_VERSION)]
+    for name in ("cw1", "cb1", "cw2", "cb2", "w1", "b1", "w2", "b2"):
+        arr = np.ascontiguousarray(p[name], np.float32)
+        out.append(struct.pack("<II", 0, arr.ndim) + struct.pack("<%dI" % arr.ndim, *arr.shape) + struct.pack("<I", 1))
+        out.append(arr.tobytes())
+    return b"".join(out)

@@ -211,6 +211,16 @@ def main():
     rec = bc.cnn_ce_grads(ref, x, labels, p)
     save("cnn_chain", x=x, labels=labels, **{"p_" + k: v for k, v in p.items()},
          **{k: (np.float32(v) if k == "loss" else v) for k, v in rec.items()})
+    # the example's weight checkpoint: written by the reference from a model holding p, read back into a model
+    # created with other weights; logits of the loaded model (layer hooks, no tape)
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        path = str(Path(tmp) / "model.bin")
+        holder = bc.CnnLayers(ref, p)
+        holder.save(path)
+        other = bc.CnnLayers(ref, {k: np.full_like(v, 0.01) for k, v in p.items()})
+        assert other.load(path)
+        save("cnn_checkpoint", content=np.frombuffer(Path(path).read_bytes(), np.uint8), x=x, logits=other.logits(x))
 
     # ---- not the reference: float64 autograd of an independent library ----
     import torch

@@ -233,6 +233,16 @@ def test_oracle_conv_pool_cnn_golden(oracle):
         assert same(want[key], g[key]), key
 
 
+def test_checkpoint_fixture_is_the_documented_layout():
+    """The file the reference wrote (examples/mnist/mnist_autodiff.c:775-927 over its API) is magic, version and eight
+    (null marker, ndim, dims, dtype, payload) records of the parameters; reading it back gave the same logits as the
+    model the parameters were set into directly."""
+    g, c = load("cnn_checkpoint"), load("cnn_chain")
+    _x, _labels, p = cnn_case(c)
+    assert g["content"].tobytes() == bc.checkpoint_bytes(p)
+    assert same(g["x"], c["x"]) and same(g["logits"], c["logits"])
+
+
 def test_fanout_fixture_documents_the_reference_behaviour():
     g = load("fanout_divergence")
     assert same(g["ref_da"], 4 * g["b"]) and same(g["ref_db"], 4 * g["a"])
@@ -443,3 +453,32 @@ def test_gpu_fanout_is_the_true_gradient_not_the_reference_value(boat):
     g = load("fanout_divergence")
     da, db = bc.fanout(boat, g["a"], g["b"])
     assert same(da, 2 * g["b"]) and same(db, 2 * g["a"])      # the reference reports 4b, 4a (see the fixture)
+
+
+@pytest.mark.gpu
+def test_gpu_checkpoint_roundtrip_golden(boat, tmp_path):
+    """The example's checkpoint routines over this library: a model holding the fixture's parameters writes the very
+    bytes the reference wrote; the reference's file read into a model created with other weights gives the logits
+    of the model built from the parameters directly (bit for bit) and the reference's logits (to tolerance); a file
+    with another magic number is refused."""
+    g, c = load("cnn_checkpoint"), load("cnn_chain")
+    x, labels, p = cnn_case(c)
+    holder = bc.CnnLayers(boat, p)
+    path = tmp_path / "model.bin"
+    holder.save(str(path))
+    assert path.read_bytes() == g["content"].tobytes()
+    direct = holder.logits(x)
+    ref_file = tmp_path / "reference.bin"
+    ref_file.write_bytes(g["content"].tobytes())
+    other = bc.CnnLayers(boat, {k: np.full_like(v, 0.01) for k, v in p.items()})
+    assert not same(other.logits(x), direct)
+    assert other.load(str(ref_file))
+    loaded = other.logits(x)
+    assert same(loaded, direct)
+    assert close_max(loaded, g["logits"], TOL_RED)
+    bad = tmp_path / "bad.bin"
+    bad.write_bytes(b"\0" * 8 + g["content"].tobytes()[8:])
+    assert not other.load(str(bad))                            # wrong magic: refused, nothing changed
+    assert same(other.logits(x), direct)
+    holder.free()
+    other.free()

@@ -513,6 +513,25 @@ def test_cnn_chain_bit_exact(ref, oracle):
         assert same(want[key], got[key]), key
 
 
+def test_checkpoint_written_through_the_reference_api(ref, tmp_path):
+    """The example's checkpoint routines (examples/mnist/mnist_autodiff.c:775-995) restated over the C API in
+    boat_cases.CnnLayers: the reference writes exactly the documented records, and a model created with other weights
+    that reads the file computes the logits of the model that wrote it."""
+    rng = np.random.default_rng(271)
+    x = rng.random((2, 2, 8, 8), dtype=np.float32)
+    p = cnn_params(rng, 2, 3, 5, 8, 7, 4)
+    holder = bc.CnnLayers(ref, p)
+    path = str(tmp_path / "model.bin")
+    holder.save(path)
+    with open(path, "rb") as f:
+        assert f.read() == bc.checkpoint_bytes(p)
+    other = bc.CnnLayers(ref, {k: np.full_like(v, 0.01) for k, v in p.items()})
+    want = holder.logits(x)
+    assert not same(other.logits(x), want)
+    assert other.load(path)
+    assert same(other.logits(x), want)
+
+
 # ---- loss objects (src/loss/*.c) ----
 
 @pytest.mark.parametrize("kind", ["mse", "ce", "huber"])

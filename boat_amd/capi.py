@@ -65,7 +65,20 @@ _SIGS = {
     "boat_tensor_data": (P, [P]),
     "boat_tensor_const_data": (P, [P]),
     "boat_tensor_reshape": (P, [P, C.POINTER(C.c_int64), C.c_size_t]),
+    "boat_tensor_is_contiguous": (C.c_bool, [P]),
+    "boat_dtype_name": (C.c_char_p, [C.c_int]),
+    # memory and error reporting
+    "boat_memory_allocate": (P, [C.c_size_t, C.c_int, C.c_char_p, C.c_int]), "boat_memory_free": (None, [P]),
+    "boat_memory_allocate_device": (P, [C.c_size_t, C.c_int, C.c_char_p, C.c_int]), "boat_memory_free_device": (None, [P, C.c_int]),
+    "boat_memory_copy": (None, [P, P, C.c_size_t, C.c_int, C.c_int]),
+    "boat_memory_set": (None, [P, C.c_int, C.c_size_t, C.c_int]), "boat_memory_reset_stats": (None, []),
+    "boat_error_string": (C.c_char_p, [C.c_int]), "boat_get_last_error": (C.c_int, []),
+    "boat_get_last_error_message": (C.c_char_p, []),
+    "boat_set_error": (None, [C.c_int, C.c_char_p]), "boat_clear_error": (None, []), "boat_has_error": (C.c_bool, []),
     # ops
+    "boat_add_scalar": (P, [P, C.c_double]), "boat_sub_scalar": (P, [P, C.c_double]), "boat_div_scalar": (P, [P, C.c_double]),
+    "boat_sub_": (None, [P, P]), "boat_mul_": (None, [P, P]), "boat_div_": (None, [P, P]),
+    "boat_dot": (P, [P, P]), "boat_sigmoid": (P, [P]), "boat_tanh": (P, [P]),
     "boat_add": (P, [P, P]), "boat_sub": (P, [P, P]), "boat_mul": (P, [P, P]), "boat_div": (P, [P, P]),
     "boat_add_": (None, [P, P]),
     "boat_mul_scalar": (P, [P, C.c_double]),
@@ -81,6 +94,13 @@ _SIGS = {
     "boat_variable_grad": (P, [P]),
     "boat_variable_requires_grad": (C.c_bool, [P]),
     "boat_variable_zero_grad": (None, [P]),
+    "boat_variable_create_with_shape": (P, [C.POINTER(C.c_int64), C.c_size_t, C.c_int, C.c_bool]),
+    "boat_variable_set_requires_grad": (None, [P, C.c_bool]), "boat_variable_retain_grad": (None, [P, C.c_bool]),
+    "boat_variable_reset_data": (C.c_bool, [P, P]),
+    "boat_autodiff_context_create": (P, []), "boat_autodiff_context_free": (None, [P]),
+    "boat_autodiff_context_enable_grad": (None, [P]), "boat_autodiff_context_disable_grad": (None, [P]),
+    "boat_autodiff_context_grad_enabled": (C.c_bool, [P]),
+    "boat_autodiff_set_current_context": (None, [P]), "boat_autodiff_get_current_context": (P, []),
     "boat_variable_backward": (None, [P, P]),
     "boat_variable_backward_full": (None, [P]),
     "boat_var_add": (P, [P, P]), "boat_var_sub": (P, [P, P]), "boat_var_mul": (P, [P, P]), "boat_var_div": (P, [P, P]),
@@ -128,6 +148,7 @@ _SIGS = {
     # relu / softmax hooks
     "boat_relu_layer_create": (P, []), "boat_relu_layer_free": (None, [P]),
     "boat_relu_layer_forward": (P, [P, P]), "boat_relu_layer_backward": (P, [P, P]),
+    "boat_relu_layer_update": (None, [P, C.c_float]), "boat_softmax_layer_update": (None, [P, C.c_float]),
     "boat_softmax_layer_create": (P, [C.c_int]), "boat_softmax_layer_free": (None, [P]),
     "boat_softmax_layer_forward": (P, [P, P]), "boat_softmax_layer_backward": (P, [P, P]),
     # layernorm
@@ -136,6 +157,8 @@ _SIGS = {
     "boat_layernorm_forward": (P, [P, P]),
     "boat_layernorm_backward": (P, [P, P]),
     "boat_layernorm_set_weight": (None, [P, P]), "boat_layernorm_set_bias": (None, [P, P]),
+    "boat_layer_norm_grad": (P, [P, P, P, C.POINTER(C.c_int64), C.c_size_t, C.c_float]),
+    "boat_norm_layer_update": (None, [P, C.c_float]),
     "boat_norm_layer_create": (P, [C.c_size_t, C.c_float, C.c_bool]),
     "boat_norm_layer_free": (None, [P]),
     "boat_norm_layer_forward": (P, [P, P]), "boat_norm_layer_backward": (P, [P, P]),
@@ -187,7 +210,6 @@ _EXT_SIGS = {
     "boat_hip_optimizer_add_attention": (None, [P, P]),
     "boat_hip_optimizer_add_layernorm": (None, [P, P]),
     "boat_layernorm_update": (None, [P, C.c_float]),
-    "boat_get_last_error_message": (C.c_char_p, []),
     "boat_memory_get_stats": (MemoryStats, []),
 }
 

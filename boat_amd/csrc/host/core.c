@@ -13,7 +13,7 @@
 /* ------------------------------------------------------------------ errors */
 
 static _Thread_local boat_error_t g_last_error = BOAT_SUCCESS;
-static _Thread_local char g_last_message[512] = "";
+static _Thread_local char g_last_message[256] = "";   /* the size of the reference's buffer (error.c:18): longer messages are cut at 255 bytes */
 
 void boat_fail(boat_error_t code, const char* fmt, ...) {
     va_list ap;
@@ -47,7 +47,8 @@ const char* boat_error_string(boat_error_t error) {
         case BOAT_ERROR_FILE_IO: return "File I/O error";
         case BOAT_ERROR_FORMAT: return "Format error";
         case BOAT_ERROR_NOT_IMPLEMENTED: return "Not implemented";
-        default: return "Unknown error";
+        case BOAT_ERROR_UNKNOWN: return "Unknown error";
+        default: return "Invalid error code";
     }
 }
 boat_error_t boat_get_last_error(void) { return g_last_error; }

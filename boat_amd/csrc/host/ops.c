@@ -206,9 +206,9 @@ boat_tensor_t* boat_mean(const boat_tensor_t* a, const int64_t* dims, size_t n_d
 }
 
 boat_tensor_t* boat_dot(const boat_tensor_t* a, const boat_tensor_t* b) {
-    if (!a || !b || a->nelements != b->nelements) return NULL;
-    boat_tensor_t* prod = NULL;
-    if (bt_same_shape(a, b)) prod = boat_mul(a, b);
+    /* vectors of one length only, as linear.c:176-189 */
+    if (!a || !b || a->ndim != 1 || b->ndim != 1 || a->shape[0] != b->shape[0] || a->dtype != b->dtype) return NULL;
+    boat_tensor_t* prod = boat_mul(a, b);
     if (!prod) return NULL;
     boat_tensor_t* out = boat_sum(prod, NULL, 0, false);
     boat_tensor_free(prod);

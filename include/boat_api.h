@@ -114,8 +114,8 @@ BOAT_API boat_tensor_t* boat_matmul(const boat_tensor_t* a, const boat_tensor_t*
 BOAT_API boat_tensor_t* boat_dot(const boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1);
 BOAT_API boat_tensor_t* boat_relu(const boat_tensor_t* a);
-BOAT_API boat_tensor_t* boat_sigmoid(const boat_tensor_t* a);
-BOAT_API boat_tensor_t* boat_tanh(const boat_tensor_t* a);
+BOAT_API boat_tensor_t* boat_sigmoid(const boat_tensor_t* a);   /* stub in the reference (activation.c:286-290); here the forward of boat_var_sigmoid */
+BOAT_API boat_tensor_t* boat_tanh(const boat_tensor_t* a);      /* stub in the reference (activation.c:292-296); here the forward of boat_var_tanh */
 BOAT_API boat_tensor_t* boat_softmax(const boat_tensor_t* a, int axis);
 BOAT_API boat_tensor_t* boat_log_softmax(const boat_tensor_t* a, int axis);
 BOAT_API boat_tensor_t* boat_gelu(const boat_tensor_t* a);                          /* stub in the reference (src/ops/activation.c:298-302) */
@@ -167,7 +167,7 @@ BOAT_API boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims,
 BOAT_API boat_autodiff_context_t* boat_autodiff_context_create(void);
 BOAT_API void boat_autodiff_context_free(const boat_autodiff_context_t* context);
 BOAT_API void boat_autodiff_context_enable_grad(boat_autodiff_context_t* context);
-BOAT_API void boat_autodiff_context_disable_grad(boat_autodiff_context_t* context);
+BOAT_API void boat_autodiff_context_disable_grad(boat_autodiff_context_t* context);   /* the reference stores the flag and never reads it (autodiff.c:625-632); here ops recorded while the current context has it off get no tape entry */
 BOAT_API bool boat_autodiff_context_grad_enabled(const boat_autodiff_context_t* context);
 BOAT_API void boat_autodiff_set_current_context(const boat_autodiff_context_t* context);
 BOAT_API boat_autodiff_context_t* boat_autodiff_get_current_context(void);

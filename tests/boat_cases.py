@@ -665,3 +665,140 @@ def checkpoint_bytes(p):
         out.append(struct.pack("<II", 0, arr.ndim) + struct.pack("<%dI" % arr.ndim, *arr.shape) + struct.pack("<I", 1))
         out.append(arr.tobytes())
     return b"".join(out)
+
+
+# ---- the rest of the API on the path: tensor-level ops, variable helpers, contexts, error reporting ----
+def tensor_ops(api, a, b, row, col, v1, v2):
+    """Tensor-level arithmetic and activations (src/ops/arithmetic.c:157-484, src/ops/linear.c:173-236,
+    src/ops/activation.c): a, b same shape [m, n]; row [n], col [m, 1] broadcast against a; v1, v2 vectors."""
+    out = {}
+    ta, tb, trow, tcol = (api.tensor(np.asarray(t, np.float32)) for t in (a, b, row, col))
+    t1, t2 = api.tensor(np.asarray(v1, np.float32)), api.tensor(np.asarray(v2, np.float32))
+
+    def take(name, t):
+        out[name] = None if not t else api.numpy(t)
+        if t:
+            api.boat_tensor_unref(t)
+
+    for name in ("add", "sub", "mul", "div"):
+        fn = getattr(api, "boat_" + name)
+        take(name, fn(ta, tb))
+        take(name + "_row", fn(ta, trow))
+        take(name + "_col", fn(tcol, ta))
+        take(name + "_scalar", getattr(api, f"boat_{name}_scalar")(ta, 1.75))
+    for name in ("add_", "sub_", "mul_", "div_"):
+        work = api.tensor(np.asarray(a, np.float32))
+        getattr(api, "boat_" + name)(work, tb)
+        out[name] = api.numpy(work)
+        getattr(api, "boat_" + name)(work, t1)                 # element counts differ: left as it is
+        out[name + "_mismatch_unchanged"] = bool(np.array_equal(api.numpy(work), out[name]))
+        api.boat_tensor_unref(work)
+    take("dot", api.boat_dot(t1, t2))
+    out["dot_of_matrices_is_null"] = not api.boat_dot(ta, tb)
+    for name in ("relu", "sigmoid", "tanh"):
+        take(name, getattr(api, "boat_" + name)(ta))
+    take("softmax", api.boat_softmax(ta, -1))
+    take("log_softmax", api.boat_log_softmax(ta, -1))
+    out["is_contiguous"] = bool(api.boat_tensor_is_contiguous(ta))
+    out["dtype_names"] = [api.boat_dtype_name(d).decode() for d in (0, 1, 5, 6, 10, 77)]
+    out["dtype_sizes"] = [int(api.boat_dtype_size(d)) for d in (0, 1, 5, 6)]
+    for t in (ta, tb, trow, tcol, t1, t2):
+        api.boat_tensor_unref(t)
+    return out
+
+
+def variable_helpers(api):
+    """boat_variable_create_with_shape / set_requires_grad / reset_data / retain_grad (src/autodiff.c:208-298)."""
+    out = {}
+    shape = (C.c_int64 * 2)(2, 3)
+    v = api.boat_variable_create_with_shape(shape, 2, 1, False)
+    out["with_shape_data"] = api.numpy(api.boat_variable_data(v))
+    out["requires_grad_before"] = bool(api.boat_variable_requires_grad(v))
+    api.boat_variable_set_requires_grad(v, True)
+    out["requires_grad_after"] = bool(api.boat_variable_requires_grad(v))
+    api.boat_variable_retain_grad(v, True)                                    # accepted, no observable effect
+    api.boat_variable_backward_full(v)
+    out["grad_after_backward"] = api.numpy(api.boat_variable_grad(v))
+    fresh = api.tensor(np.arange(6, dtype=np.float32).reshape(2, 3))
+    out["reset_leaf"] = bool(api.boat_variable_reset_data(v, fresh))
+    out["data_after_reset"] = api.numpy(api.boat_variable_data(v))
+    out["grad_dropped_by_reset"] = not api.boat_variable_grad(v)
+    out["reset_null"] = bool(api.boat_variable_reset_data(v, None))
+    api.boat_tensor_unref(fresh)
+    out["data_survives_callers_unref"] = api.numpy(api.boat_variable_data(v))  # the variable holds its own reference
+    if api.is_amd:
+        api.boat_variable_free(v)
+    return out
+
+
+def context_and_errors(api):
+    """Context objects (src/autodiff.c:606-649) and the error state (src/core/error.c:21-62)."""
+    out = {}
+    ctx = api.boat_autodiff_context_create()
+    out["enabled_at_creation"] = bool(api.boat_autodiff_context_grad_enabled(ctx))
+    api.boat_autodiff_context_disable_grad(ctx)
+    out["enabled_after_disable"] = bool(api.boat_autodiff_context_grad_enabled(ctx))
+    api.boat_autodiff_context_enable_grad(ctx)
+    out["enabled_after_enable"] = bool(api.boat_autodiff_context_grad_enabled(ctx))
+    out["enabled_of_null"] = bool(api.boat_autodiff_context_grad_enabled(None))
+    before = api.boat_autodiff_get_current_context()
+    api.boat_autodiff_set_current_context(ctx)
+    out["current_is_the_one_set"] = api.boat_autodiff_get_current_context() == ctx
+    api.boat_autodiff_set_current_context(before)
+    api.boat_autodiff_context_free(ctx)
+    api.boat_clear_error()
+    out["error_after_clear"] = (int(api.boat_get_last_error()), api.boat_get_last_error_message().decode(), bool(api.boat_has_error()))
+    api.boat_set_error(3, b"the operation is not valid here")
+    out["error_after_set"] = (int(api.boat_get_last_error()), api.boat_get_last_error_message().decode(), bool(api.boat_has_error()))
+    api.boat_set_error(5, b"x" * 400)                                          # longer than the 256-byte message buffer
+    out["long_message_length"] = len(api.boat_get_last_error_message())
+    api.boat_set_error(2, None)
+    out["error_with_null_message"] = (int(api.boat_get_last_error()), api.boat_get_last_error_message().decode())
+    api.boat_clear_error()
+    out["error_strings"] = [api.boat_error_string(e).decode() for e in range(0, 10)] + [api.boat_error_string(-1).decode()]
+    # host memory helpers
+    p = api.boat_memory_allocate(64, 0, b"boat_cases.py", 1)
+    api.boat_memory_set(p, 0x5A, 64, 0)
+    q = api.boat_memory_allocate(64, 0, b"boat_cases.py", 2)
+    api.boat_memory_copy(q, p, 64, 0, 0)
+    out["memory_set_then_copy"] = C.string_at(q, 64) == b"\x5a" * 64
+    api.boat_memory_free(p)
+    api.boat_memory_free(q)
+    return out
+
+
+def sgd_hooks(api, x, w, b, dy, lr):
+    """boat_dense_layer_update (src/layers/dense.c:297-329): p -= lr * g, gradients cleared; then a second backward
+    accumulates from zero.  Returns ((gw, gb) of the first backward, w1, b1, gw_after_update, w2)."""
+    layer = _make_dense(api, w, b)
+    tx, tdy = api.tensor(np.asarray(x, np.float32)), api.tensor(np.asarray(dy, np.float32))
+    ty = api.boat_dense_layer_forward(layer, tx)
+    tdx = api.boat_dense_layer_backward(layer, tdy)
+    g0 = api.numpy(api.boat_dense_layer_get_grad_weight(layer)), api.numpy(api.boat_dense_layer_get_grad_bias(layer))
+    api.boat_dense_layer_update(layer, lr)
+    w1, b1 = api.numpy(api.boat_dense_layer_get_weight(layer)), api.numpy(api.boat_dense_layer_get_bias(layer))
+    gw = api.numpy(api.boat_dense_layer_get_grad_weight(layer))
+    api.boat_tensor_unref(tdx)
+    tdx = api.boat_dense_layer_backward(layer, tdy)
+    api.boat_dense_layer_update(layer, lr)
+    w2 = api.numpy(api.boat_dense_layer_get_weight(layer))
+    for t in (tdx, ty, tdy, tx):
+        api.boat_tensor_unref(t)
+    api.boat_dense_layer_free(layer)
+    return g0, w1, b1, gw, w2
+
+
+def conv_sgd_hook(api, x, w, b, dy, lr):
+    """boat_conv_layer_update (src/layers/conv.c:539-562): p -= lr * g through boat_mul_scalar + boat_sub_, gradients kept."""
+    layer = _make_conv(api, np.asarray(w, np.float32), np.asarray(b, np.float32), 1, 1)
+    tx, tdy = api.tensor(np.asarray(x, np.float32)), api.tensor(np.asarray(dy, np.float32))
+    ty = api.boat_conv_layer_forward(layer, tx)
+    tdx = api.boat_conv_layer_backward(layer, tdy)
+    gw, gb = api.numpy(api.boat_conv_layer_get_grad_weight(layer)), api.numpy(api.boat_conv_layer_get_grad_bias(layer))
+    api.boat_conv_layer_update(layer, lr)
+    w1, b1 = api.numpy(api.boat_conv_layer_get_weight(layer)), api.numpy(api.boat_conv_layer_get_bias(layer))
+    gw_after = api.numpy(api.boat_conv_layer_get_grad_weight(layer))
+    for t in (tdx, ty, tdy, tx):
+        api.boat_tensor_unref(t)
+    api.boat_conv_layer_free(layer)
+    return w1, b1, gw, gb, gw_after

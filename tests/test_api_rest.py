@@ -1,0 +1,226 @@
+"""Entry points of Boat's API that the training scenarios do not reach: tensor-level arithmetic, variable helpers,
+context objects, the error state, host memory helpers and the layers' own SGD hooks.  Each scenario of
+boat_cases.py runs against the compiled reference (CPU) and against libboat_amd.so (GPU) and is held to the same
+expectations, which are closed forms: one IEEE operation per element, or literal values read off the reference's
+sources (src/core/error.c:21-62, src/autodiff.c:208-298,606-649, src/layers/dense.c:297-329, conv.c:539-562).
+"""
+import numpy as np
+import pytest
+
+import boat_cases as bc
+
+F = np.float32
+
+
+def inputs():
+    rng = np.random.default_rng(77)
+    a = rng.standard_normal((5, 8)).astype(F)
+    b = (rng.standard_normal((5, 8)) + 3).astype(F)
+    a[0, :3] = [0.0, -0.0, 1e-30]
+    return a, b, b[1].copy(), b[:, 2:3].copy(), a[2].copy(), b[3].copy()
+
+
+def check_tensor_ops(out, stubs_return_null):
+    a, b, row, col, v1, v2 = inputs()
+    np_op = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}
+    np.seterr(divide="ignore")                                                # a holds zeros on purpose
+    for name, fn in np_op.items():
+        assert np.array_equal(out[name], fn(a, b)), name
+        assert np.array_equal(out[name + "_row"], fn(a, row)), name           # [5,8] op [8]
+        assert np.array_equal(out[name + "_col"], fn(col, a)), name           # [5,1] op [5,8]
+        assert np.array_equal(out[name + "_scalar"], fn(a, F(1.75))), name
+        assert np.array_equal(out[name + "_"], fn(a, b)), name                # in place
+        assert out[name + "__mismatch_unchanged"], name
+    acc = F(0)
+    for x, y in zip(v1, v2):                                                  # linear.c:206-213: sequential fp32
+        acc = F(acc + F(x * y))
+    assert out["dot"].shape == (1,) and abs(out["dot"][0] - acc) <= 1e-5 * abs(acc)
+    assert out["dot_of_matrices_is_null"]
+    assert np.array_equal(out["relu"], np.maximum(a, 0) * (a > 0))
+    a64 = a.astype(np.float64)
+    if stubs_return_null:                                                     # activation.c:286-296
+        assert out["sigmoid"] is None and out["tanh"] is None
+    else:
+        assert np.max(np.abs(out["sigmoid"] - 1 / (1 + np.exp(-a64)))) <= 1e-6
+        assert np.max(np.abs(out["tanh"] - np.tanh(a64))) <= 1e-6
+    e = np.exp(a64 - a64.max(1, keepdims=True))
+    assert np.max(np.abs(out["softmax"] - e / e.sum(1, keepdims=True))) <= 1e-6
+    assert np.max(np.abs(out["log_softmax"] - np.log(e / e.sum(1, keepdims=True)))) <= 1e-5
+    assert out["is_contiguous"] is True
+    assert out["dtype_names"] == ["float64", "float32", "int64", "int32", "bool", "unknown"]
+    assert out["dtype_sizes"] == [8, 4, 8, 4]
+
+
+def check_variable_helpers(out):
+    assert np.array_equal(out["with_shape_data"], np.zeros((2, 3), F))
+    assert (out["requires_grad_before"], out["requires_grad_after"]) == (False, True)
+    assert np.array_equal(out["grad_after_backward"], np.ones((2, 3), F))
+    assert out["reset_leaf"] is True and out["grad_dropped_by_reset"] is True and out["reset_null"] is False
+    want = np.arange(6, dtype=F).reshape(2, 3)
+    assert np.array_equal(out["data_after_reset"], want) and np.array_equal(out["data_survives_callers_unref"], want)
+
+
+CONTEXT_AND_ERRORS = {
+    "enabled_at_creation": True, "enabled_after_disable": False, "enabled_after_enable": True, "enabled_of_null": False,
+    "current_is_the_one_set": True,
+    "error_after_clear": (0, "", False), "error_after_set": (3, "the operation is not valid here", True),
+    "long_message_length": 255, "error_with_null_message": (2, ""),
+    "error_strings": ["Success", "Invalid argument", "Out of memory", "Invalid operation", "Device error", "File I/O error",
+                      "Format error", "Not implemented", "Unknown error", "Invalid error code", "Invalid error code"],
+    "memory_set_then_copy": True,
+}
+
+
+def sgd_inputs():
+    rng = np.random.default_rng(78)
+    return (rng.standard_normal((6, 5)).astype(F), rng.standard_normal((5, 3)).astype(F), rng.standard_normal(3).astype(F),
+            rng.standard_normal((6, 3)).astype(F), 0.05)
+
+
+def check_sgd(api):
+    x, w, b, dy, lr = sgd_inputs()
+    (gw, gb), w1, b1, gw_after, w2 = bc.sgd_hooks(api, x, w, b, dy, lr)
+    assert np.max(np.abs(gw - x.T.astype(np.float64) @ dy)) <= 1e-5 and np.max(np.abs(gb - dy.sum(0, dtype=np.float64))) <= 1e-5
+    assert np.array_equal(w1, w - F(lr) * gw) and np.array_equal(b1, b - F(lr) * gb)     # one multiply, one subtract
+    assert not gw_after.any()                                                             # cleared by the update
+    assert np.array_equal(w2, w1 - F(lr) * gw)                                            # so the second step is the same size
+    rng = np.random.default_rng(79)
+    xc, wc = rng.standard_normal((2, 2, 6, 6)).astype(F), rng.standard_normal((3, 2, 3, 3)).astype(F)
+    bcv, dyc = rng.standard_normal(3).astype(F), rng.standard_normal((2, 3, 6, 6)).astype(F)
+    w1, b1, gw, gb, gw_after = bc.conv_sgd_hook(api, xc, wc, bcv, dyc, lr)
+    assert np.array_equal(w1, wc - F(lr) * gw) and np.array_equal(b1, bcv - F(lr) * gb)
+    assert np.array_equal(gw_after, gw) and gw.any()                                      # conv.c:561: gradients are kept
+
+
+def test_reference_tensor_ops(ref):
+    check_tensor_ops(bc.tensor_ops(ref, *inputs()), stubs_return_null=True)
+
+
+def test_reference_variable_helpers_contexts_errors(ref):
+    check_variable_helpers(bc.variable_helpers(ref))
+    assert bc.context_and_errors(ref) == CONTEXT_AND_ERRORS
+
+
+def test_reference_sgd_hooks(ref):
+    check_sgd(ref)
+
+
+@pytest.mark.gpu
+def test_gpu_tensor_ops(boat):
+    check_tensor_ops(bc.tensor_ops(boat, *inputs()), stubs_return_null=False)
+
+
+@pytest.mark.gpu
+def test_gpu_variable_helpers_contexts_errors(boat):
+    check_variable_helpers(bc.variable_helpers(boat))
+    assert bc.context_and_errors(boat) == CONTEXT_AND_ERRORS
+
+
+@pytest.mark.gpu
+def test_gpu_sgd_hooks(boat):
+    check_sgd(boat)
+
+
+@pytest.mark.gpu
+def test_gpu_disabled_context_records_nothing(boat):
+    """The reference keeps the flag without reading it; here an operation recorded while the current context has
+    gradients off leaves no tape entry, so its result is a leaf."""
+    ctx = boat.boat_autodiff_context_create()
+    before = boat.boat_autodiff_get_current_context()
+    boat.boat_autodiff_set_current_context(ctx)
+    a, b = bc._var(boat, [1, 2, 3], True), bc._var(boat, [4, 5, 6], True)
+    boat.boat_autodiff_context_disable_grad(ctx)
+    off = boat.boat_var_mul(a, b)
+    boat.boat_variable_backward_full(off)
+    assert not boat.boat_variable_grad(a) and not boat.boat_variable_grad(b)
+    assert boat.numpy(boat.boat_variable_data(off)).tolist() == [4, 10, 18]
+    boat.boat_autodiff_context_enable_grad(ctx)
+    on = boat.boat_var_mul(a, b)
+    boat.boat_variable_backward_full(on)
+    assert boat.numpy(boat.boat_variable_grad(a)).tolist() == [4, 5, 6]
+    boat.boat_autodiff_set_current_context(before)
+    for v in (on, off, a, b):
+        boat.boat_variable_free(v)
+    boat.boat_autodiff_context_free(ctx)
+
+
+@pytest.mark.gpu
+def test_gpu_layer_norm_grad_and_norm_layer_adapters(boat, oracle):
+    """boat_layer_norm_grad (a stub in the reference, src/layers/norm.c:450-463) and the boat_norm_layer_* adapters
+    (:523-550) against the float64 closed form of the oracle."""
+    import ctypes as C
+    rng = np.random.default_rng(80)
+    x, dy = rng.standard_normal((7, 48)).astype(F), rng.standard_normal((7, 48)).astype(F)
+    tx, tdy = boat.tensor(x), boat.tensor(dy)
+    shape = (C.c_int64 * 1)(48)
+    tdx = boat.boat_layer_norm_grad(tdy, tx, None, shape, 1, 1e-5)
+    assert tdx
+    _y, mean, rstd = oracle.layernorm_forward(x, None, None, 1e-5)
+    want_dx, _, _ = oracle.layernorm_backward_f64(x, None, dy, mean, rstd)
+    assert np.max(np.abs(boat.numpy(tdx) - want_dx)) <= 1e-4 * np.abs(want_dx).max()
+    assert not boat.boat_layer_norm_grad(tdy, tx, None, shape, 2, 1e-5)       # only the last axis is supported
+    layer = boat.boat_norm_layer_create(48, 1e-5, True)
+    ty = boat.boat_norm_layer_forward(layer, tx)
+    y = boat.numpy(ty)
+    assert np.max(np.abs(y.mean(1))) <= 1e-6 and np.max(np.abs(y.var(1) - 1)) <= 1e-3
+    tdx2 = boat.boat_norm_layer_backward(layer, tdy)
+    assert np.array_equal(boat.numpy(tdx2), boat.numpy(tdx))                  # gamma = 1, beta = 0 at creation
+    boat.boat_norm_layer_update(layer, 0.1)
+    for t in (tdx2, ty, tdx, tdy, tx):
+        boat.boat_tensor_unref(t)
+    boat.boat_norm_layer_free(layer)
+
+
+@pytest.mark.gpu
+def test_gpu_small_hooks(boat):
+    """What is left: hooks that do nothing in the reference either (relu.c:74-78, softmax.c:60-64, pool.c:220-224,
+    flatten.c:91-95), boat_softmax_layer_forward (softmax.c:34-41), the reference count of a tensor
+    (tensor.c:164-191), memory statistics, and boat_layernorm_update (a stub in the reference, norm.c:411-415; here
+    the same SGD step as the dense layer's)."""
+    rng = np.random.default_rng(81)
+    x = rng.standard_normal((4, 6)).astype(F)
+    tx = boat.tensor(x)
+    sm = boat.boat_softmax_layer_create(-1)
+    ty = boat.boat_softmax_layer_forward(sm, tx)
+    tz = boat.boat_softmax(tx, -1)
+    assert np.array_equal(boat.numpy(ty), boat.numpy(tz))
+    boat.boat_softmax_layer_update(sm, 0.1)
+    relu, pool, flat = boat.boat_relu_layer_create(), boat.boat_pool_layer_create(2, 2, 0), boat.boat_flatten_layer_create()
+    boat.boat_relu_layer_update(relu, 0.1)
+    boat.boat_pool_layer_update(pool, 0.1)
+    boat.boat_flatten_layer_update(flat, 0.1)
+    assert np.array_equal(boat.numpy(tx), x)
+    boat.boat_tensor_ref(tx)                      # two owners
+    boat.boat_tensor_free(tx)                     # free is unref: one owner left, contents intact
+    assert np.array_equal(boat.numpy(tx), x)
+    for t in (tz, ty, tx):
+        boat.boat_tensor_unref(t)
+    boat.boat_softmax_layer_free(sm)
+    boat.boat_relu_layer_free(relu)
+    boat.boat_pool_layer_free(pool)
+    boat.boat_flatten_layer_free(flat)
+
+    boat.boat_memory_reset_stats()
+    s0 = boat.boat_memory_get_stats()
+    assert (s0.allocated_bytes, s0.allocated_blocks, s0.freed_bytes, s0.freed_blocks, s0.peak_allocated_bytes) == (0, 0, 0, 0, 0)
+    p = boat.boat_memory_allocate_device(4096, 0, b"test", 1)
+    assert p and boat.boat_memory_get_stats().allocated_blocks == 1
+    boat.boat_memory_free_device(p, 0)
+    s1 = boat.boat_memory_get_stats()
+    assert s1.freed_blocks == 1 and s1.freed_bytes == s1.allocated_bytes >= 4096
+
+    from boat_amd.capi import LayerNormConfig
+    import ctypes as C
+    cfg = LayerNormConfig(6, 1e-5, True, True)
+    norm = boat.boat_layernorm_create(C.byref(cfg))
+    tx, tdy = boat.tensor(x), boat.tensor(rng.standard_normal((4, 6)).astype(F))
+    ty = boat.boat_layernorm_forward(norm, tx)
+    tdx = boat.boat_layernorm_backward(norm, tdy)
+    gw = boat.numpy(boat.boat_hip_layernorm_get_grad_weight(norm))
+    assert gw.any()
+    boat.boat_layernorm_update(norm, 0.5)
+    assert np.array_equal(boat.numpy(boat.boat_hip_layernorm_get_weight(norm)), np.ones(6, F) - F(0.5) * gw)
+    assert not boat.numpy(boat.boat_hip_layernorm_get_grad_weight(norm)).any()
+    for t in (tdx, ty, tdy, tx):
+        boat.boat_tensor_unref(t)
+    boat.boat_layernorm_free(norm)

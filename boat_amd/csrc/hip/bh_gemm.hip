@@ -853,6 +853,22 @@ using CfgMid = GemmCfg<128, 128, 2, 2>;   // 4 waves, 64x64 per wave
 using CfgTall = GemmCfg<256, 128, 4, 2>;  // 8 waves, 64x64 per wave
 using CfgWide = GemmCfg<128, 256, 2, 4>;  // 8 waves, 64x64 per wave
 
+// out[a][d1][b][d0][c] = in[a][d0][b][d1][c]: two dimensions of a dense tensor swapped, anything between and after
+// them carried along (the general case of boat_transpose, linear.c:238-406).  One output element per lane and trip;
+// consecutive lanes write consecutive addresses, and read consecutive ones whenever c has an extent.
+__global__ __launch_bounds__(256) void swap_dims_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t d0,
+                                                        int64_t b, int64_t d1, int64_t c, int64_t total) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        int64_t t = i;
+        const int64_t ic = t % c; t /= c;
+        const int64_t i0 = t % d0; t /= d0;
+        const int64_t ib = t % b; t /= b;
+        const int64_t i1 = t % d1;
+        const int64_t ia = t / d1;
+        out[i] = in[(((ia * d0 + i0) * b + ib) * d1 + i1) * c + ic];
+    }
+}
+
 template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT>
 static int launch_mfma(const GemmArgs& g, int64_t batch) {
     constexpr size_t lds = 2 * sizeof(float) *
@@ -1154,6 +1170,21 @@ int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, 
     BH_CHECK_ARG(grid.y <= 65535, "too many rows");
     hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, stream(), a, out, rows, cols);
     return BH_LAUNCH_CHECK("transpose_kernel");
+}
+
+int bh_swap_dims(const float* in, float* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(a >= 0 && d0 >= 0 && b >= 0 && d1 >= 0 && c >= 0, "negative dimension");
+    const double elems = (double)a * (double)d0 * (double)b * (double)d1 * (double)c;
+    BH_CHECK_ARG(elems < 9.0e18, "tensor too large");
+    const int64_t total = a * d0 * b * d1 * c;
+    if (total == 0) return BH_OK;
+    BH_CHECK_ARG(in && out, "null pointer");
+    if (b == 1 && c == 1 && a <= 65535 && ceil_div(d0, 32) <= 65535) return bh_transpose_last2(in, out, a, d0, d1);
+    int64_t blocks = ceil_div(total, 256);
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(swap_dims_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), in, out, d0, b, d1, c, total);
+    return BH_LAUNCH_CHECK("swap_dims_kernel");
 }
 
 int bh_dense_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t m,

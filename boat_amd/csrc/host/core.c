@@ -239,6 +239,10 @@ static boat_tensor_t* tensor_alloc(const int64_t* shape, size_t ndim, boat_dtype
     t->device = device;
     t->nelements = n;
     t->nbytes = n * boat_dtype_size(dtype);
+    /* packed types, tensor.c:105-115 */
+    if (dtype == BOAT_DTYPE_FLOAT4) t->nbytes = (n + 1) / 2;
+    else if (dtype == BOAT_DTYPE_BITS2) t->nbytes = (n + 3) / 4;
+    else if (dtype == BOAT_DTYPE_BITS1) t->nbytes = (n + 7) / 8;
     t->is_contiguous = true;
     t->ref_count = 1;
     if (share) {

@@ -143,24 +143,21 @@ boat_tensor_t* boat_matmul(const boat_tensor_t* a, const boat_tensor_t* b) {
 boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1) {
     if (!a || !bt_is_f32(a)) return NULL;
     const int nd = (int)a->ndim;
-    if (dim0 < 0) dim0 += nd;
-    if (dim1 < 0) dim1 += nd;
-    if (dim0 < 0 || dim1 < 0 || dim0 >= nd || dim1 >= nd) return NULL;
+    if (dim0 < 0 || dim1 < 0 || dim0 >= nd || dim1 >= nd) return NULL;   /* linear.c:241-244 (negative ints compare as huge) */
     if (dim0 == dim1) return boat_tensor_clone(a);
     if (dim0 > dim1) {
         int t = dim0;
         dim0 = dim1;
         dim1 = t;
     }
-    /* the hot path only swaps the last two dims ((0,1) on 2-D, (2,3) on 4-D) */
-    if (dim0 != nd - 2 || dim1 != nd - 1) {
-        boat_fail(BOAT_ERROR_NOT_IMPLEMENTED, "boat_transpose: only the last two dimensions can be swapped");
-        return NULL;
-    }
     int64_t shape[BOAT_MAX_DIMS];
-    int64_t batch = 1;
-    for (int i = 0; i < nd; i++) shape[i] = a->shape[i];
-    for (int i = 0; i < nd - 2; i++) batch *= a->shape[i];
+    int64_t before = 1, between = 1, after = 1;
+    for (int i = 0; i < nd; i++) {
+        shape[i] = a->shape[i];
+        if (i < dim0) before *= a->shape[i];
+        else if (i > dim0 && i < dim1) between *= a->shape[i];
+        else if (i > dim1) after *= a->shape[i];
+    }
     shape[dim0] = a->shape[dim1];
     shape[dim1] = a->shape[dim0];
     boat_tensor_t* out = bt_new_uninit(shape, a->ndim, a->device);
@@ -169,9 +166,14 @@ boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1) {
     float* po = bt_dev_write(out);
     bool ok = pa && po;
     const int64_t rows = a->shape[dim0], cols = a->shape[dim1];
-    for (int64_t b0 = 0; ok && b0 < batch; b0 += 32768) {
-        const int64_t nb = batch - b0 < 32768 ? batch - b0 : 32768;
-        ok = boat_hip_ok(bh_transpose_last2(pa + b0 * rows * cols, po + b0 * rows * cols, nb, rows, cols), "boat_transpose");
+    if (ok && between == 1 && after == 1) {
+        /* the hot path's case, the last two dimensions: the tiled kernel, in slabs its grid can index */
+        for (int64_t b0 = 0; ok && b0 < before; b0 += 32768) {
+            const int64_t nb = before - b0 < 32768 ? before - b0 : 32768;
+            ok = boat_hip_ok(bh_transpose_last2(pa + b0 * rows * cols, po + b0 * rows * cols, nb, rows, cols), "boat_transpose");
+        }
+    } else if (ok) {
+        ok = boat_hip_ok(bh_swap_dims(pa, po, before, rows, between, cols, after), "boat_transpose");
     }
     if (!ok) {
         boat_tensor_free(out);

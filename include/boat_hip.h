@@ -130,6 +130,9 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
             const float* a, int64_t lda, const float* b, int64_t ldb,
             float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch);
 int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, int64_t cols); /* linear.c:238-406 */
+/* out[a][d1][b][d0][c] = in[a][d0][b][d1][c]: boat_transpose of any two dimensions of a dense tensor (linear.c:238-406;
+ * a, b, c are the products of the extents before, between and after the two) */
+int bh_swap_dims(const float* in, float* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c);
 /* dense layer backward in one call: dx = dy.W^T, gw += x^T.dy, gb += colsum(dy)  (dense.c:190-295) */
 int bh_dense_backward(const float* x, const float* w, const float* dy,
                       float* dx, float* gw, float* gb, int64_t m, int64_t k, int64_t n,

@@ -802,3 +802,67 @@ def conv_sgd_hook(api, x, w, b, dy, lr):
         api.boat_tensor_unref(t)
     api.boat_conv_layer_free(layer)
     return w1, b1, gw, gb, gw_after
+
+
+def tensor_facts(api):
+    """Observable facts of tensor creation, views and argument checks (src/core/tensor.c:65-300,
+    src/ops/arithmetic.c:136-156, src/ops/linear.c:12-60,238-262)."""
+    out = {}
+
+    def shp(*dims):
+        return (C.c_int64 * max(len(dims), 1))(*dims)
+
+    def facts(t):
+        if not t:
+            return None
+        f = (int(api.boat_tensor_ndim(t)), int(api.boat_tensor_nelements(t)), int(api.boat_tensor_nbytes(t)),
+             int(api.boat_tensor_dtype(t)), int(api.boat_tensor_device(t)), bool(api.boat_tensor_is_contiguous(t)))
+        return f
+
+    def take(name, t):
+        out[name] = facts(t)
+        if t:
+            api.boat_tensor_unref(t)
+
+    if api.is_amd:   # the reference aborts here: zero bytes fail to allocate and the clean-up frees the wrong pointers (tensor.c:118-124)
+        take("scalar_null_shape", api.boat_tensor_create(None, 0, 1, 0))
+    take("null_shape_with_dims", api.boat_tensor_create(None, 2, 1, 0))
+    take("f32_2x3", api.boat_tensor_create(shp(2, 3), 2, 1, 0))
+    take("f64_2x3", api.boat_tensor_create(shp(2, 3), 2, 0, 0))
+    take("i32_5", api.boat_tensor_create(shp(5), 1, 6, 0))
+    take("i64_5", api.boat_tensor_create(shp(5), 1, 5, 0))
+    take("f4_5", api.boat_tensor_create(shp(5), 1, 4, 0))
+    take("bits1_9", api.boat_tensor_create(shp(9), 1, 9, 0))
+    take("eight_dims", api.boat_tensor_create(shp(1, 2, 1, 2, 1, 2, 1, 2), 8, 1, 0))
+    base = api.tensor(np.arange(12, dtype=np.float32).reshape(3, 4))
+    view = api.boat_tensor_reshape(base, shp(2, 6), 2)
+    out["view"] = facts(view)
+    out["view_shape"] = api.shape(view)
+    out["view_shares_data"] = api.boat_tensor_data(view) == api.boat_tensor_data(base)
+    api.boat_tensor_unref(base)                                  # the view keeps its parent alive
+    out["view_after_parent_unref"] = api.numpy(view).tolist()
+    api.boat_tensor_unref(view)
+    base = api.tensor(np.arange(12, dtype=np.float32).reshape(3, 4))
+    out["reshape_wrong_count"] = facts(api.boat_tensor_reshape(base, shp(5, 2), 2))
+    out["reshape_null_shape"] = facts(api.boat_tensor_reshape(base, None, 2))
+    like = api.boat_tensor_create_like(base)
+    out["like"] = facts(like)
+    out["like_is_zero"] = not api.numpy(like).any()
+    api.boat_tensor_unref(like)
+    f64 = api.tensor(np.ones((3, 4), np.float64))
+    vec3, vec4 = api.tensor(np.ones(3, np.float32)), api.tensor(np.ones(4, np.float32))
+    take("add_mixed_dtypes", api.boat_add(base, f64))
+    take("add_3x4_and_3", api.boat_add(base, vec3))
+    take("add_3x4_and_4", api.boat_add(base, vec4))
+    take("matmul_inner_mismatch", api.boat_matmul(base, base))
+    take("matmul_3x4_4", api.boat_matmul(base, vec4))
+    take("transpose_bad_dim", api.boat_transpose(base, 0, 2))
+    take("transpose_same_dim", api.boat_transpose(base, 1, 1))
+    take("transpose_negative", api.boat_transpose(base, -1, -2))
+    take("sum_all", api.boat_sum(base, None, 0, False))
+    take("softmax_vector", api.boat_softmax(vec4, -1))
+    take("relu_f64", api.boat_relu(f64))
+    take("mul_scalar_f64", api.boat_mul_scalar(f64, 2.0))
+    for t in (base, f64, vec3, vec4):
+        api.boat_tensor_unref(t)
+    return out

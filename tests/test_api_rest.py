@@ -224,3 +224,57 @@ def test_gpu_small_hooks(boat):
     for t in (tdx, ty, tdy, tx):
         boat.boat_tensor_unref(t)
     boat.boat_layernorm_free(norm)
+
+
+TENSOR_FACTS = {   # (ndim, nelements, nbytes, dtype, device, is_contiguous) or None for a refused call
+    "null_shape_with_dims": None,
+    "f32_2x3": (2, 6, 24, 1, 0, True), "f64_2x3": (2, 6, 48, 0, 0, True), "i32_5": (1, 5, 20, 6, 0, True),
+    "i64_5": (1, 5, 40, 5, 0, True), "f4_5": (1, 5, 3, 4, 0, True), "bits1_9": (1, 9, 2, 9, 0, True),
+    "eight_dims": (8, 16, 64, 1, 0, True),
+    "view": (2, 12, 48, 1, 0, False),                           # tensor.c:288: a reshaped view reports non-contiguous
+    "view_shape": (2, 6), "view_shares_data": True,
+    "view_after_parent_unref": [[0.0, 1.0, 2.0, 3.0, 4.0, 5.0], [6.0, 7.0, 8.0, 9.0, 10.0, 11.0]],
+    "reshape_wrong_count": None, "reshape_null_shape": None,
+    "like": (2, 12, 48, 1, 0, True), "like_is_zero": True,
+    "add_mixed_dtypes": None, "add_3x4_and_3": None, "add_3x4_and_4": (2, 12, 48, 1, 0, True),
+    "matmul_inner_mismatch": None, "matmul_3x4_4": None,
+    "transpose_bad_dim": None, "transpose_same_dim": (2, 12, 48, 1, 0, True), "transpose_negative": None,
+    "sum_all": (1, 1, 4, 1, 0, True), "softmax_vector": (1, 4, 16, 1, 0, True),
+    "relu_f64": (2, 12, 96, 0, 0, True), "mul_scalar_f64": (2, 12, 96, 0, 0, True),
+}
+
+
+def test_reference_tensor_facts(ref):
+    assert bc.tensor_facts(ref) == TENSOR_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_tensor_facts(boat):
+    got = bc.tensor_facts(boat)
+    scalar = got.pop("scalar_null_shape")          # the reference aborts on this call; here a one-element tensor or a refusal
+    assert scalar is None or scalar[:2] == (0, 1)
+    # the path is float32: arithmetic on other element types is refused here (no host fall-back), not computed
+    assert got.pop("relu_f64") is None and got.pop("mul_scalar_f64") is None
+    diff = {k: (got.get(k), v) for k, v in TENSOR_FACTS.items() if k in got and got[k] != v}
+    assert not diff and set(got) == set(TENSOR_FACTS) - {"relu_f64", "mul_scalar_f64"}, diff
+
+
+TRANSPOSE_CASES = [((3, 4), 0, 1), ((3, 4), 1, 0), ((2, 3, 4), 0, 1), ((2, 3, 4), 0, 2), ((2, 3, 4), 1, 2),
+                   ((2, 3, 4, 5), 1, 2), ((2, 3, 4, 5), 0, 3), ((2, 3, 4, 5), 2, 3), ((2, 1, 4, 3, 2), 1, 4)]
+
+
+def check_transposes(api, cases):
+    rng = np.random.default_rng(82)
+    for shape, d0, d1 in cases:
+        x = rng.standard_normal(shape).astype(F)
+        got = bc.transpose(api, x, d0, d1)
+        assert got.shape == np.swapaxes(x, d0, d1).shape and np.array_equal(got, np.swapaxes(x, d0, d1)), (shape, d0, d1)
+
+
+def test_reference_transposes_any_two_dimensions(ref):
+    check_transposes(ref, TRANSPOSE_CASES)
+
+
+@pytest.mark.gpu
+def test_gpu_transposes_any_two_dimensions(boat):
+    check_transposes(boat, TRANSPOSE_CASES + [((70, 33, 65), 0, 2), ((5, 130, 3, 70), 1, 3), ((4, 300, 260), 1, 2)])

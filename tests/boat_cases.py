@@ -866,3 +866,137 @@ def tensor_facts(api):
     for t in (base, f64, vec3, vec4):
         api.boat_tensor_unref(t)
     return out
+
+
+def layer_facts(api, only=None):
+    """Argument checks and object life cycle of layers, optimizers and the model container: a dict of small facts
+    (shapes, NULL or not, scalars).  `only` limits the probes to the named groups."""
+    from boat_amd.capi import AttentionConfig, LayerNormConfig
+    out = {}
+    rng = np.random.default_rng(9)
+
+    def T(*shape):
+        return api.tensor(rng.standard_normal(shape).astype(np.float32))
+
+    def shape_of(t, free=True):
+        if not t:
+            return None
+        s = api.shape(t)
+        if free:
+            api.boat_tensor_unref(t)
+        return s
+
+    def group(name):
+        return only is None or name in only
+
+    if group("matmul"):
+        a2, b2, a3, b3, a4, b4, b3x, v = T(3, 4), T(4, 5), T(2, 3, 4), T(2, 4, 5), T(2, 2, 3, 4), T(2, 2, 4, 5), T(3, 4, 5), T(4)
+        out["matmul_2d"] = shape_of(api.boat_matmul(a2, b2))
+        out["matmul_3d"] = shape_of(api.boat_matmul(a3, b3))
+        out["matmul_4d"] = shape_of(api.boat_matmul(a4, b4))
+        out["matmul_batch_mismatch"] = shape_of(api.boat_matmul(a3, b3x))
+        out["matmul_3d_with_2d"] = shape_of(api.boat_matmul(a3, b2))
+        out["matmul_with_vector"] = shape_of(api.boat_matmul(a2, v))
+        t3 = api.boat_matmul(a3, b3)
+        out["matmul_3d_value_ok"] = bool(np.allclose(api.numpy(t3), api.numpy(a3) @ api.numpy(b3), rtol=1e-5, atol=1e-5))
+        api.boat_tensor_unref(t3)
+        for t in (a2, b2, a3, b3, a4, b4, b3x, v):
+            api.boat_tensor_unref(t)
+
+    if group("dense"):
+        nb = api.boat_dense_layer_create(4, 3, False)
+        out["dense_no_bias_has_bias"] = bool(api.boat_dense_layer_get_bias(nb))
+        out["dense_no_bias_has_grad_bias"] = bool(api.boat_dense_layer_get_grad_bias(nb))
+        out["dense_weight_shape"] = shape_of(api.boat_dense_layer_get_weight(nb), free=False)
+        out["dense_grad_weight_zero_at_creation"] = not api.numpy(api.boat_dense_layer_get_grad_weight(nb)).any()
+        x2, x3, xbad, dy = T(2, 4), T(2, 5, 4), T(2, 3), T(2, 3)
+        out["dense_forward_2d"] = shape_of(api.boat_dense_layer_forward(nb, x2))
+        tdx = api.boat_dense_layer_backward(nb, dy)
+        out["dense_backward_no_bias"] = shape_of(tdx)
+        out["dense_forward_3d"] = shape_of(api.boat_dense_layer_forward(nb, x3))
+        out["dense_forward_wrong_features"] = shape_of(api.boat_dense_layer_forward(nb, xbad))
+        api.boat_dense_layer_set_bias(nb, dy)                      # refused: the layer has no bias
+        out["dense_set_bias_on_no_bias_layer"] = bool(api.boat_dense_layer_get_bias(nb))
+        wbad = T(3, 4)
+        api.boat_dense_layer_set_weight(nb, wbad)                  # refused: wrong shape
+        out["dense_set_weight_wrong_shape_kept"] = shape_of(api.boat_dense_layer_get_weight(nb), free=False)
+        for t in (x2, x3, xbad, dy, wbad):
+            api.boat_tensor_unref(t)
+        api.boat_dense_layer_free(nb)
+
+    if group("optimizer"):
+        p, g = T(3, 2), T(3, 2)
+        before = api.numpy(p)
+        for kind, make, bad in (
+                ("adam", lambda: api.boat_adam_optimizer_create(0.1, 0.9, 0.999, 1e-8),
+                 [lambda: api.boat_adam_optimizer_create(-1.0, 0.9, 0.999, 1e-8), lambda: api.boat_adam_optimizer_create(0.1, 0.9, 1.5, 1e-8),
+                  lambda: api.boat_adam_optimizer_create(0.1, 0.9, 0.999, 0.0), lambda: api.boat_adam_optimizer_create(0.1, 0.9, 0.999, -1.0)]),
+                ("rmsprop", lambda: api.boat_rmsprop_optimizer_create(0.1, 0.99, 1e-8),
+                 [lambda: api.boat_rmsprop_optimizer_create(0.0, 0.99, 1e-8), lambda: api.boat_rmsprop_optimizer_create(0.1, 1.0, 1e-8),
+                  lambda: api.boat_rmsprop_optimizer_create(0.1, 0.99, 0.0)]),
+                ("adagrad", lambda: api.boat_adagrad_optimizer_create(0.1, 1e-8),
+                 [lambda: api.boat_adagrad_optimizer_create(0.0, 1e-8), lambda: api.boat_adagrad_optimizer_create(0.1, 0.0)])):
+            out[kind + "_bad_arguments_refused"] = [not f() for f in bad]
+            opt = make()
+            out[kind + "_lr"] = round(float(api.boat_optimizer_get_learning_rate(opt)), 6)
+            api.boat_optimizer_set_learning_rate(opt, 0.25)
+            out[kind + "_lr_after_set"] = round(float(api.boat_optimizer_get_learning_rate(opt)), 6)
+            api.boat_optimizer_step(opt)                            # no parameters: nothing to do
+            api.boat_optimizer_add_parameter(opt, p, None)          # refused without a gradient tensor
+            api.boat_optimizer_step(opt)
+            out[kind + "_null_grad_ignored"] = bool(np.array_equal(api.numpy(p), before))
+            api.boat_optimizer_add_parameter(opt, p, g)
+            api.boat_optimizer_zero_grad(opt)
+            out[kind + "_zero_grad_clears"] = not api.numpy(g).any()
+            api.boat_optimizer_step(opt)                            # zero gradient: parameters stay
+            out[kind + "_zero_grad_step_keeps_params"] = bool(np.array_equal(api.numpy(p), before))
+            api.boat_optimizer_free(opt)
+            api.write(g, rng.standard_normal((3, 2)).astype(np.float32))
+        api.boat_tensor_unref(p)
+        api.boat_tensor_unref(g)
+
+    if group("attention"):
+        def cfg(hidden, heads, bias=True):
+            return AttentionConfig(hidden, heads, 0, 0.0, False, bias, False, 10000.0)
+        out["attention_heads_do_not_divide"] = not api.boat_attention_create(C.byref(cfg(10, 3)))
+        out["attention_zero_heads"] = not api.boat_attention_create(C.byref(cfg(8, 0)))
+        out["attention_null_config"] = not api.boat_attention_create(None)
+        att = api.boat_attention_create(C.byref(cfg(8, 2, bias=False)))
+        out["attention_no_bias_has_bias_q"] = bool(api.boat_attention_get_bias_q(att))
+        out["attention_weight_shape"] = shape_of(api.boat_attention_get_weight_q(att), free=False)
+        out["attention_grad_before_backward"] = bool(api.boat_attention_get_grad_weight_q(att))
+        x = T(2, 3, 8)
+        ty = api.boat_attention_forward(att, x, x, x, None)
+        out["attention_forward"] = shape_of(ty)
+        api.boat_tensor_unref(x)
+        api.boat_attention_free(att)
+
+    if group("layernorm"):
+        plain = api.boat_layernorm_create(C.byref(LayerNormConfig(6, 1e-5, False, False)))
+        x, xbad = T(4, 6), T(4, 5)
+        out["layernorm_plain_forward"] = shape_of(api.boat_layernorm_forward(plain, x))
+        out["layernorm_wrong_width"] = shape_of(api.boat_layernorm_forward(plain, xbad))
+        out["layernorm_zero_width"] = not api.boat_layernorm_create(C.byref(LayerNormConfig(0, 1e-5, True, True)))
+        api.boat_tensor_unref(x)
+        api.boat_tensor_unref(xbad)
+        api.boat_layernorm_free(plain)
+
+    if group("conv"):
+        conv = api.boat_conv_layer_create(2, 3, 3, 1, 1)
+        x, xbad, x3 = T(2, 2, 5, 5), T(2, 4, 5, 5), T(2, 5, 5)
+        out["conv_forward"] = shape_of(api.boat_conv_layer_forward(conv, x))
+        out["conv_wrong_channels"] = shape_of(api.boat_conv_layer_forward(conv, xbad))
+        out["conv_3d_input"] = shape_of(api.boat_conv_layer_forward(conv, x3))
+        out["conv_weight_shape"] = shape_of(api.boat_conv_layer_get_weight(conv), free=False)
+        out["conv_bias_shape"] = shape_of(api.boat_conv_layer_get_bias(conv), free=False)
+        pool = api.boat_pool_layer_create(2, 2, 0)
+        out["pool_forward"] = shape_of(api.boat_pool_layer_forward(pool, x))
+        out["pool_3d_input"] = shape_of(api.boat_pool_layer_forward(pool, x3))
+        flat = api.boat_flatten_layer_create()
+        out["flatten_forward"] = shape_of(api.boat_flatten_layer_forward(flat, x))
+        for t in (x, xbad, x3):
+            api.boat_tensor_unref(t)
+        api.boat_conv_layer_free(conv)
+        api.boat_pool_layer_free(pool)
+        api.boat_flatten_layer_free(flat)
+    return out

@@ -278,3 +278,39 @@ def test_reference_transposes_any_two_dimensions(ref):
 @pytest.mark.gpu
 def test_gpu_transposes_any_two_dimensions(boat):
     check_transposes(boat, TRANSPOSE_CASES + [((70, 33, 65), 0, 2), ((5, 130, 3, 70), 1, 3), ((4, 300, 260), 1, 2)])
+
+
+LAYER_FACTS = {
+    "matmul_2d": (3, 5), "matmul_3d": (2, 3, 5), "matmul_4d": (2, 2, 3, 5), "matmul_batch_mismatch": None,
+    "matmul_3d_with_2d": None, "matmul_with_vector": None, "matmul_3d_value_ok": True,
+    "dense_no_bias_has_bias": False, "dense_no_bias_has_grad_bias": False, "dense_weight_shape": (4, 3),
+    "dense_grad_weight_zero_at_creation": True, "dense_forward_2d": (2, 3), "dense_backward_no_bias": (2, 4),
+    "dense_forward_3d": None, "dense_forward_wrong_features": None, "dense_set_bias_on_no_bias_layer": False,
+    "dense_set_weight_wrong_shape_kept": (4, 3),
+    "adam_bad_arguments_refused": [True, True, False, False],           # adam.c:45-53 checks lr and the betas, not epsilon
+    "adam_lr": 0.1, "adam_lr_after_set": 0.25, "adam_null_grad_ignored": True, "adam_zero_grad_clears": True,
+    "adam_zero_grad_step_keeps_params": True,
+    "rmsprop_bad_arguments_refused": [True, True, True], "rmsprop_lr": 0.1, "rmsprop_lr_after_set": 0.25,
+    "rmsprop_null_grad_ignored": True, "rmsprop_zero_grad_clears": True, "rmsprop_zero_grad_step_keeps_params": True,
+    "adagrad_bad_arguments_refused": [True, True], "adagrad_lr": 0.1, "adagrad_lr_after_set": 0.25,
+    "adagrad_null_grad_ignored": True, "adagrad_zero_grad_clears": True, "adagrad_zero_grad_step_keeps_params": True,
+    "attention_heads_do_not_divide": True, "attention_zero_heads": True, "attention_null_config": True,
+    "attention_no_bias_has_bias_q": False, "attention_weight_shape": (8, 8), "attention_grad_before_backward": False,
+    "attention_forward": (2, 3, 8),
+    "layernorm_plain_forward": (4, 6), "layernorm_wrong_width": None, "layernorm_zero_width": True,
+    "conv_forward": (2, 3, 5, 5), "conv_wrong_channels": None, "conv_3d_input": None, "conv_weight_shape": (3, 2, 3, 3),
+    "conv_bias_shape": (3,), "pool_forward": (2, 2, 2, 2), "pool_3d_input": None, "flatten_forward": (2, 50),
+}
+
+
+def test_reference_layer_facts(ref):
+    with bc.scratch_cwd():
+        assert bc.layer_facts(ref) == LAYER_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_layer_facts(boat):
+    got = bc.layer_facts(boat)
+    want = LAYER_FACTS
+    diff = {k: (got.get(k), v) for k, v in want.items() if got.get(k) != v}
+    assert not diff and set(got) == set(want), diff

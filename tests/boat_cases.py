@@ -1000,3 +1000,111 @@ def layer_facts(api, only=None):
         api.boat_pool_layer_free(pool)
         api.boat_flatten_layer_free(flat)
     return out
+
+
+def autodiff_facts(api):
+    """How the tape propagates requires_grad and shapes (src/autodiff.c:138-206,2070-2347,2155,2221,2287,530-548)."""
+    out = {}
+    rng = np.random.default_rng(10)
+
+    def V(shape, rg):
+        return _var(api, rng.standard_normal(shape).astype(np.float32), rg)
+
+    def rg(v):
+        return None if not v else bool(api.boat_variable_requires_grad(v))
+
+    def shape_of(v):
+        return None if not v else api.shape(api.boat_variable_data(v))
+
+    a, b, c, d = V((3, 4), False), V((3, 4), True), V((3, 4), False), V((4, 2), True)
+    out["add_false_true"] = rg(api.boat_var_add(a, b))
+    out["add_false_false"] = rg(api.boat_var_add(a, c))
+    out["mul_true_false"] = rg(api.boat_var_mul(b, a))
+    out["matmul_false_true"] = rg(api.boat_var_matmul(a, d))
+    out["relu_false"] = rg(api.boat_var_relu(a))
+    out["relu_true"] = rg(api.boat_var_relu(b))
+    out["add_shape_mismatch"] = shape_of(api.boat_var_add(a, d))
+    out["matmul_shape"] = shape_of(api.boat_var_matmul(a, d))
+    out["matmul_inner_mismatch"] = shape_of(api.boat_var_matmul(a, b))
+    out["sum_all_shape"] = shape_of(api.boat_var_sum(b, None, 0, False))
+    x = rng.standard_normal((3, 4)).astype(np.float32)
+    vx = _var(api, x, True)
+    s_last, s_axis0 = api.boat_var_softmax(vx, -1), api.boat_var_softmax(vx, 0)
+    out["softmax_axis_is_ignored"] = bool(np.array_equal(api.numpy(api.boat_variable_data(s_last)), api.numpy(api.boat_variable_data(s_axis0))))
+    out["softmax_rows_sum_to_one"] = bool(np.allclose(api.numpy(api.boat_variable_data(s_axis0)).sum(1), 1, atol=1e-6))
+    out["flatten_shape"] = shape_of(api.boat_var_flatten(_var(api, rng.standard_normal((2, 3, 4, 5)).astype(np.float32), True)))
+    # a dense layer on the tape: the output needs a gradient only if the INPUT does, whatever the layer's parameters
+    layer = _make_dense(api, rng.standard_normal((4, 2)).astype(np.float32), np.zeros(2, np.float32))
+    y_off = api.boat_var_dense(a, layer)
+    out["dense_of_input_without_grad"] = rg(y_off)
+    with scratch_cwd():
+        api.boat_variable_backward_full(y_off)                        # silently nothing
+    out["dense_grads_untouched_without_input_grad"] = not api.numpy(api.boat_dense_layer_get_grad_weight(layer)).any()
+    y_on = api.boat_var_dense(b, layer)
+    out["dense_of_input_with_grad"] = rg(y_on)
+    with scratch_cwd():
+        api.boat_variable_backward_full(y_on)
+    out["dense_grads_filled_with_input_grad"] = bool(api.numpy(api.boat_dense_layer_get_grad_weight(layer)).any())
+    out["input_grad_shape"] = None if not api.boat_variable_grad(b) else api.shape(api.boat_variable_grad(b))
+    return out
+
+
+# ---- the model container with vtables written by the caller (tests/test_model_graph_integration.c:8-77) ----
+_FWD = C.CFUNCTYPE(C.c_void_p, C.c_void_p, C.c_void_p)
+_UPD = C.CFUNCTYPE(None, C.c_void_p, C.c_float)
+_FREE = C.CFUNCTYPE(None, C.c_void_p)
+
+
+class _LayerOps(C.Structure):      # include/boat/model.h:29-34
+    _fields_ = [("forward", _FWD), ("backward", _FWD), ("update", _UPD), ("free", _FREE)]
+
+
+class _Layer(C.Structure):         # include/boat/model.h:23-27
+    _fields_ = [("data", C.c_void_p), ("ops", C.POINTER(_LayerOps))]
+
+
+def model_over_callers_vtables(api, x, weights, biases, dy=None, lr=None):
+    """A boat_model_t of dense layers, each behind a boat_layer_ops_t table the CALLER wrote (here: Python callbacks
+    that forward to boat_dense_layer_*), as tests/test_model_graph_integration.c:8-41 does in C.  Returns
+    dict(count, y, dx or None when boat_model_backward returns NULL, freed = how many free hooks ran, weights after
+    boat_model_update when lr is given)."""
+    dense = [_make_dense(api, w, b) for w, b in zip(weights, biases)]
+    freed = []
+    keep = []
+
+    def data_of(layer_ptr):
+        return C.cast(layer_ptr, C.POINTER(_Layer)).contents.data
+
+    ops = _LayerOps(_FWD(lambda l, t: api.boat_dense_layer_forward(data_of(l), t)),
+                    _FWD(lambda l, g: api.boat_dense_layer_backward(data_of(l), g)),
+                    _UPD(lambda l, r: api.boat_dense_layer_update(data_of(l), r)),
+                    _FREE(lambda l: freed.append(data_of(l))))
+    model = api.boat_model_create()
+    for d in dense:
+        wrapper = _Layer(d, C.pointer(ops))
+        keep.append(wrapper)
+        api.boat_model_add_layer(model, C.addressof(wrapper))
+    rec = {"count": int(api.boat_model_layer_count(model))}
+    tx = api.tensor(np.asarray(x, np.float32))
+    ty = api.boat_model_forward(model, tx)
+    rec["y"] = None if not ty else api.numpy(ty)
+    rec["dx"] = None
+    if dy is not None:
+        tdy = api.tensor(np.asarray(dy, np.float32))
+        tdx = api.boat_model_backward(model, tdy)
+        if tdx:
+            rec["dx"] = api.numpy(tdx)
+            api.boat_tensor_unref(tdx)
+        rec["gw"] = [api.numpy(api.boat_dense_layer_get_grad_weight(d)) for d in dense]
+        api.boat_tensor_unref(tdy)
+    if lr is not None:
+        api.boat_model_update(model, lr)
+        rec["w_after"] = [api.numpy(api.boat_dense_layer_get_weight(d)) for d in dense]
+    if ty:
+        api.boat_tensor_unref(ty)
+    api.boat_tensor_unref(tx)
+    api.boat_model_free(model)
+    rec["freed"] = len(freed)
+    for d in dense:
+        api.boat_dense_layer_free(d)
+    return rec

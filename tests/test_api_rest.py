@@ -314,3 +314,59 @@ def test_gpu_layer_facts(boat):
     want = LAYER_FACTS
     diff = {k: (got.get(k), v) for k, v in want.items() if got.get(k) != v}
     assert not diff and set(got) == set(want), diff
+
+
+AUTODIFF_FACTS = {
+    "add_false_true": True, "add_false_false": False, "mul_true_false": True, "matmul_false_true": True,
+    "relu_false": False, "relu_true": True, "add_shape_mismatch": None, "matmul_shape": (3, 2),
+    "matmul_inner_mismatch": None, "sum_all_shape": (1,),
+    "softmax_axis_is_ignored": True, "softmax_rows_sum_to_one": True,        # autodiff.c:530-535: always the last axis
+    "flatten_shape": (2, 60),
+    "dense_of_input_without_grad": False, "dense_grads_untouched_without_input_grad": True,   # autodiff.c:2287
+    "dense_of_input_with_grad": True, "dense_grads_filled_with_input_grad": True, "input_grad_shape": (3, 4),
+}
+
+
+def test_reference_autodiff_facts(ref):
+    assert bc.autodiff_facts(ref) == AUTODIFF_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_autodiff_facts(boat):
+    got = bc.autodiff_facts(boat)
+    boat.boat_autodiff_clear_computation_graph()
+    diff = {k: (got.get(k), v) for k, v in AUTODIFF_FACTS.items() if got.get(k) != v}
+    assert not diff and set(got) == set(AUTODIFF_FACTS), diff
+
+
+def model_case():
+    rng = np.random.default_rng(83)
+    x = rng.standard_normal((5, 6)).astype(F)
+    ws = [rng.standard_normal((6, 4)).astype(F), rng.standard_normal((4, 3)).astype(F)]
+    bs = [rng.standard_normal(4).astype(F), rng.standard_normal(3).astype(F)]
+    return x, ws, bs, rng.standard_normal((5, 3)).astype(F)
+
+
+def test_reference_model_over_callers_vtables(ref, oracle):
+    x, ws, bs, dy = model_case()
+    rec = bc.model_over_callers_vtables(ref, x, ws, bs, dy=dy, lr=0.1)
+    assert rec["count"] == 2 and rec["freed"] == 2
+    assert np.array_equal(rec["y"], oracle.dense_forward(oracle.dense_forward(x, ws[0], bs[0]), ws[1], bs[1]))
+    assert rec["dx"] is None and not any(g.any() for g in rec["gw"])          # model.c:354-359: backward is a stub
+    assert all(np.array_equal(a, b) for a, b in zip(rec["w_after"], ws))       # model.c:361-365: so is update
+
+
+@pytest.mark.gpu
+def test_gpu_model_over_callers_vtables(boat, oracle):
+    """The same caller-written tables on this library: forward as the reference, and the two stubs do their work
+    (layers[n-1..0] through ops->backward, then ops->update)."""
+    x, ws, bs, dy = model_case()
+    rec = bc.model_over_callers_vtables(boat, x, ws, bs, dy=dy, lr=0.1)
+    assert rec["count"] == 2 and rec["freed"] == 2
+    h = oracle.dense_forward(x, ws[0], bs[0])
+    assert np.max(np.abs(rec["y"] - oracle.dense_forward(h, ws[1], bs[1]))) <= 1e-5
+    dh, gw2, _ = oracle.dense_backward(h, ws[1], dy)
+    dx, gw1, _ = oracle.dense_backward(x, ws[0], dh)
+    assert np.max(np.abs(rec["dx"] - dx)) <= 1e-5 and np.max(np.abs(rec["gw"][0] - gw1)) <= 1e-5
+    assert np.max(np.abs(rec["gw"][1] - gw2)) <= 1e-5
+    assert all(np.array_equal(a, w - F(0.1) * g) for a, w, g in zip(rec["w_after"], ws, rec["gw"]))

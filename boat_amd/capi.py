@@ -193,7 +193,7 @@ _EXT_SIGS = {
     "boat_gelu": (P, [P]),
     "boat_tensor_to_device": (P, [P, C.c_int]),
     "boat_tensor_clone": (P, [P]),
-    "boat_hip_synchronize": (None, []),
+    "boat_hip_synchronize": (None, []), "boat_hip_set_coherent_pointers": (None, [C.c_int]),
     "boat_hip_variable_ensure_grad": (P, [P]),
     "boat_hip_var_gelu": (P, [P]),
     "boat_hip_var_layernorm": (P, [P, P]),

@@ -856,7 +856,8 @@ using CfgWide = GemmCfg<128, 256, 2, 4>;  // 8 waves, 64x64 per wave
 // out[a][d1][b][d0][c] = in[a][d0][b][d1][c]: two dimensions of a dense tensor swapped, anything between and after
 // them carried along (the general case of boat_transpose, linear.c:238-406).  One output element per lane and trip;
 // consecutive lanes write consecutive addresses, and read consecutive ones whenever c has an extent.
-__global__ __launch_bounds__(256) void swap_dims_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t d0,
+template <typename T>
+__global__ __launch_bounds__(256) void swap_dims_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t d0,
                                                         int64_t b, int64_t d1, int64_t c, int64_t total) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         int64_t t = i;
@@ -1172,19 +1173,33 @@ int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, 
     return BH_LAUNCH_CHECK("transpose_kernel");
 }
 
-int bh_swap_dims(const float* in, float* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c) {
+}  // extern "C"
+
+template <typename T>
+static int swap_dims(const T* in, T* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c) {
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(a >= 0 && d0 >= 0 && b >= 0 && d1 >= 0 && c >= 0, "negative dimension");
     const double elems = (double)a * (double)d0 * (double)b * (double)d1 * (double)c;
-    BH_CHECK_ARG(elems < 9.0e18, "tensor too large");
+    BH_CHECK_ARG(elems < 9.0e18 / sizeof(T), "tensor too large");
     const int64_t total = a * d0 * b * d1 * c;
     if (total == 0) return BH_OK;
     BH_CHECK_ARG(in && out, "null pointer");
-    if (b == 1 && c == 1 && a <= 65535 && ceil_div(d0, 32) <= 65535) return bh_transpose_last2(in, out, a, d0, d1);
     int64_t blocks = ceil_div(total, 256);
     if (blocks > 16384) blocks = 16384;
-    hipLaunchKernelGGL(swap_dims_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), in, out, d0, b, d1, c, total);
+    hipLaunchKernelGGL((swap_dims_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), in, out, d0, b, d1, c, total);
     return BH_LAUNCH_CHECK("swap_dims_kernel");
+}
+
+extern "C" {
+
+int bh_swap_dims(const float* in, float* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c) {
+    if (in && out && a > 0 && d0 > 0 && d1 > 0 && b == 1 && c == 1 && a <= 65535 && ceil_div(d0, 32) <= 65535)
+        return bh_transpose_last2(in, out, a, d0, d1);
+    return swap_dims<float>(in, out, a, d0, b, d1, c);
+}
+
+int bh_swap_dims_f64(const double* in, double* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c) {
+    return swap_dims<double>(in, out, a, d0, b, d1, c);
 }
 
 int bh_dense_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t m,

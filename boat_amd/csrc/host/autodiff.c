@@ -129,6 +129,7 @@ void boat_variable_zero_grad(boat_variable_t* v) {
     if (v->persistent_grad) {
         float* g = bt_dev_write(v->grad);
         if (g) boat_hip_ok(bh_memset_zero(g, v->grad->nbytes), "boat_variable_zero_grad");
+        bt_flush_exposed();
     } else {
         boat_tensor_unref(v->grad);   /* the reference drops the tensor (autodiff.c:285-292) */
         v->grad = NULL;
@@ -560,7 +561,7 @@ static int by_seq_desc(const void* x, const void* y) {
     return a->seq < b->seq ? 1 : a->seq > b->seq ? -1 : 0;
 }
 
-void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_output) {
+static void boat_variable_backward_unflushed(boat_variable_t* variable, boat_tensor_t* grad_output) {
     if (!variable || !variable->requires_grad) return;
     boat_tensor_t* seed = grad_output;
     if (!seed) {
@@ -607,6 +608,10 @@ void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_outpu
     }
     free(ops);
     if (!grad_output) boat_tensor_unref(seed);
+}
+void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_output) {
+    boat_variable_backward_unflushed(variable, grad_output);
+    bt_flush_exposed();
 }
 
 /* gradient checkpointing is a stub in the reference too (autodiff.c:652-655): every op keeps what its backward needs */

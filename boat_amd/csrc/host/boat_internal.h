@@ -14,6 +14,8 @@ typedef struct boat_storage {
     bool host_valid;       /* host mirror holds the current values */
     bool dev_valid;        /* device buffer holds the current values */
     size_t refs;
+    bool exposed;          /* coherent-pointer mode: the caller holds the host pointer and may use it at any time */
+    bool pending;          /* coherent-pointer mode: written on the device since the last write-back to the host */
 } boat_storage_t;
 
 struct boat_tensor_t {
@@ -29,12 +31,19 @@ struct boat_tensor_t {
     bool is_view;
 };
 
+/* Coherent-pointer mode (boat_hip_set_coherent_pointers): copies every tensor whose host pointer the caller holds and
+ * that this call wrote on the device back to the host.  Public functions that write tensors which existed before
+ * the call end with it; a no-op in the default mode. */
+void bt_flush_exposed(void);
 /* device pointer for reading: uploads the host mirror first if it is the newer copy */
 const float* bt_dev_read(const boat_tensor_t* t);
 /* device pointer for a full overwrite: nothing is uploaded, the device copy becomes the current one */
 float* bt_dev_write(boat_tensor_t* t);
 /* device pointer for read-modify-write */
 float* bt_dev_rw(boat_tensor_t* t);
+/* what boat_tensor_data() returns, for the library's own host-side writes (initial weights): the pointer does not
+ * leave the library, so the tensor does not become "exposed" in coherent-pointer mode */
+void* bt_host_rw(boat_tensor_t* t);
 /* new fp32 tensor with the shape/device of `like`, contents unspecified (to be fully written by a kernel) */
 boat_tensor_t* bt_new_like_uninit(const boat_tensor_t* like);
 boat_tensor_t* bt_new_uninit(const int64_t* shape, size_t ndim, boat_device_t device);

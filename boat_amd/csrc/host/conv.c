@@ -47,7 +47,7 @@ boat_conv_layer_t* boat_conv_layer_create(size_t in_channels, size_t out_channel
     l->bias = boat_tensor_create(bshape, 1, BOAT_DTYPE_FLOAT32, BOAT_DEVICE_CPU);
     l->grad_weight = boat_tensor_create(wshape, 4, BOAT_DTYPE_FLOAT32, BOAT_DEVICE_CPU);
     l->grad_bias = boat_tensor_create(bshape, 1, BOAT_DTYPE_FLOAT32, BOAT_DEVICE_CPU);
-    float* w = l->weight ? (float*)boat_tensor_data(l->weight) : NULL;
+    float* w = l->weight ? (float*)bt_host_rw(l->weight) : NULL;
     if (!w || !l->bias || !l->grad_weight || !l->grad_bias) {
         boat_conv_layer_free(l);
         return NULL;
@@ -108,7 +108,7 @@ boat_tensor_t* boat_conv_layer_forward(boat_conv_layer_t* l, const boat_tensor_t
     return out;
 }
 
-boat_tensor_t* boat_conv_layer_backward(boat_conv_layer_t* l, const boat_tensor_t* grad_output) {
+static boat_tensor_t* boat_conv_layer_backward_unflushed(boat_conv_layer_t* l, const boat_tensor_t* grad_output) {
     if (!l || !grad_output) {
         fprintf(stderr, "Error: conv backward: NULL input\n");
         return NULL;
@@ -142,6 +142,11 @@ boat_tensor_t* boat_conv_layer_backward(boat_conv_layer_t* l, const boat_tensor_
     }
     return dx;
 }
+boat_tensor_t* boat_conv_layer_backward(boat_conv_layer_t* l, const boat_tensor_t* grad_output) {
+    boat_tensor_t* result = boat_conv_layer_backward_unflushed(l, grad_output);
+    bt_flush_exposed();
+    return result;
+}
 
 /* weight -= lr * grad (conv.c:537-560); the gradients are left in place, the next backward overwrites them */
 void boat_conv_layer_update(boat_conv_layer_t* l, float learning_rate) {
@@ -154,6 +159,7 @@ void boat_conv_layer_update(boat_conv_layer_t* l, float learning_rate) {
         float* pg = bt_dev_rw(g);
         if (pp && pg) boat_hip_ok(bh_sgd_update(pp, pg, learning_rate, (int64_t)p->nelements, 0), "conv update");
     }
+    bt_flush_exposed();
 }
 
 void boat_conv_layer_set_weight(boat_conv_layer_t* l, boat_tensor_t* weight) {

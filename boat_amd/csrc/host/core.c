@@ -287,6 +287,56 @@ boat_tensor_t* bt_new_like_uninit(const boat_tensor_t* like) {
     return like ? boat_tensor_create(like->shape, like->ndim, BOAT_DTYPE_FLOAT32, like->device) : NULL;
 }
 
+/* ---- coherent-pointer mode ----
+ * Boat's callers keep the float* that boat_tensor_data() gave them: they write through it before a later call
+ * (tests/unit/test_attention_gradient_check.c:22-41) and read results through it after one
+ * (tests/unit/test_optimizer_adam.c:96-108).  The default protocol only promises the pointer until the next call
+ * that takes the tensor, which keeps parameters resident on the device.  In this mode a tensor whose pointer was
+ * handed out is "exposed": its host mirror is uploaded before every device read (the caller may have written), and
+ * device writes to it are copied back before the public call returns (the caller may read).  Correct for any caller,
+ * at the price of PCIe transfers for exposed tensors. */
+static int g_coherent = -1;
+static boat_storage_t** g_pending = NULL;
+static size_t g_pending_n = 0, g_pending_cap = 0;
+
+static bool coherent_mode(void) {
+    if (g_coherent < 0) {
+        const char* e = getenv("BOAT_HIP_COHERENT_POINTERS");
+        g_coherent = e && *e && *e != '0';
+    }
+    return g_coherent != 0;
+}
+void boat_hip_set_coherent_pointers(int enable) {
+    bt_flush_exposed();
+    g_coherent = enable != 0;
+}
+
+static void mark_device_write(boat_storage_t* st) {
+    if (!st->exposed || st->pending) return;
+    if (g_pending_n == g_pending_cap) {
+        const size_t cap = g_pending_cap ? 2 * g_pending_cap : 64;
+        boat_storage_t** grown = (boat_storage_t**)realloc(g_pending, cap * sizeof(*grown));
+        if (!grown) return;   /* the tensor stays readable through boat_tensor_data(), which downloads */
+        g_pending = grown;
+        g_pending_cap = cap;
+    }
+    st->pending = true;
+    st->refs++;               /* alive until written back */
+    g_pending[g_pending_n++] = st;
+}
+
+void bt_flush_exposed(void) {
+    while (g_pending_n > 0) {
+        boat_storage_t* st = g_pending[--g_pending_n];
+        st->pending = false;
+        if (st->refs > 1 && st->host && st->dev && st->dev_valid && !st->host_valid) {
+            if (boat_hip_ok(bh_memcpy_d2h(st->host, bh_buffer_ptr(st->dev), st->nbytes), "write-back of an exposed tensor"))
+                st->host_valid = true;
+        }
+        storage_unref(st);
+    }
+}
+
 static bool storage_host_ready(boat_storage_t* st) {
     if (!st->host) {
         st->host = calloc(1, st->nbytes ? st->nbytes : 1);
@@ -314,6 +364,8 @@ static bool storage_dev_ready(boat_storage_t* st, bool need_contents) {
         }
         if (zero) st->dev_valid = true;
     }
+    /* an exposed tensor may have been written through the caller's pointer since the last upload */
+    if (need_contents && st->exposed && !st->pending && st->host_valid) st->dev_valid = false;
     if (need_contents && !st->dev_valid) {
         if (st->host_valid) {
             if (!boat_hip_ok(bh_memcpy_h2d(bh_buffer_ptr(st->dev), st->host, st->nbytes), "tensor upload")) return false;
@@ -335,11 +387,13 @@ float* bt_dev_write(boat_tensor_t* t) {
     if (!storage_dev_ready(t->st, false)) return NULL;
     t->st->dev_valid = true;
     t->st->host_valid = false;
+    mark_device_write(t->st);
     return (float*)bh_buffer_ptr(t->st->dev);
 }
 float* bt_dev_rw(boat_tensor_t* t) {
     if (!t || !storage_dev_ready(t->st, true)) return NULL;
     t->st->host_valid = false;
+    mark_device_write(t->st);
     return (float*)bh_buffer_ptr(t->st->dev);
 }
 
@@ -347,7 +401,7 @@ boat_tensor_t* boat_tensor_from_data(const int64_t* shape, size_t ndim, boat_dty
     boat_tensor_t* t = boat_tensor_create(shape, ndim, dtype, BOAT_DEVICE_CPU);
     if (!t) return NULL;
     if (data) {
-        void* dst = boat_tensor_data(t);
+        void* dst = bt_host_rw(t);
         if (!dst) {
             boat_tensor_free(t);
             return NULL;
@@ -378,18 +432,24 @@ size_t boat_tensor_nbytes(const boat_tensor_t* t) { return t ? t->nbytes : 0; }
 size_t boat_tensor_nelements(const boat_tensor_t* t) { return t ? t->nelements : 0; }
 bool boat_tensor_is_contiguous(const boat_tensor_t* t) { return t ? t->is_contiguous : false; }
 
-void* boat_tensor_data(const boat_tensor_t* tensor) {
+void* bt_host_rw(boat_tensor_t* tensor) {
     if (!tensor) return NULL;
     boat_storage_t* st = tensor->st;
-    if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_rw((boat_tensor_t*)tensor);
+    if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_rw(tensor);
     if (!storage_host_ready(st)) return NULL;
-    st->dev_valid = false;   /* the caller may write through the pointer */
+    st->dev_valid = false;   /* written through the pointer */
     return st->host;
+}
+void* boat_tensor_data(const boat_tensor_t* tensor) {
+    void* p = bt_host_rw((boat_tensor_t*)tensor);
+    if (p && tensor->device != BOAT_DEVICE_HIP && coherent_mode()) tensor->st->exposed = true;   /* the caller keeps it */
+    return p;
 }
 const void* boat_tensor_const_data(const boat_tensor_t* tensor) {
     if (!tensor) return NULL;
     if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_read(tensor);
     if (!storage_host_ready(tensor->st)) return NULL;
+    if (coherent_mode()) tensor->st->exposed = true;
     return tensor->st->host;
 }
 
@@ -418,7 +478,7 @@ boat_tensor_t* boat_tensor_clone(const boat_tensor_t* tensor) {
             return NULL;
         }
     } else if (st->host_valid) {
-        void* dst = boat_tensor_data(c);
+        void* dst = bt_host_rw(c);
         if (!dst) {
             boat_tensor_free(c);
             return NULL;
@@ -444,7 +504,7 @@ boat_tensor_t* boat_tensor_to_device(const boat_tensor_t* tensor, boat_device_t 
             return NULL;
         }
     } else {
-        void* dst = boat_tensor_data(out);
+        void* dst = bt_host_rw(out);
         bool ok = dst != NULL;
         if (ok && src->host_valid) memcpy(dst, src->host, tensor->nbytes);
         else if (ok) ok = boat_hip_ok(bh_memcpy_d2h(dst, bh_buffer_ptr(src->dev), tensor->nbytes), "boat_tensor_to_device");

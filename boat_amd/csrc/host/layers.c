@@ -23,7 +23,7 @@ static boat_tensor_t* create_linear_weights(size_t in_features, size_t out_featu
     const int64_t shape[] = {(int64_t)in_features, (int64_t)out_features};
     boat_tensor_t* w = boat_tensor_create(shape, 2, BOAT_DTYPE_FLOAT32, BOAT_DEVICE_CPU);
     if (!w) return NULL;
-    float* data = (float*)boat_tensor_data(w);
+    float* data = (float*)bt_host_rw(w);
     if (!data) {
         boat_tensor_free(w);
         return NULL;
@@ -96,7 +96,7 @@ boat_tensor_t* boat_dense_layer_forward(boat_dense_layer_t* layer, const boat_te
     return out;
 }
 
-boat_tensor_t* boat_dense_layer_backward(boat_dense_layer_t* layer, const boat_tensor_t* grad_output) {
+static boat_tensor_t* boat_dense_layer_backward_unflushed(boat_dense_layer_t* layer, const boat_tensor_t* grad_output) {
     if (!layer || !grad_output || !layer->cache_input) return NULL;
     const boat_tensor_t* input = layer->cache_input;
     if (input->ndim != 2 || grad_output->ndim != 2) {
@@ -128,6 +128,11 @@ boat_tensor_t* boat_dense_layer_backward(boat_dense_layer_t* layer, const boat_t
     }
     return dx;
 }
+boat_tensor_t* boat_dense_layer_backward(boat_dense_layer_t* layer, const boat_tensor_t* grad_output) {
+    boat_tensor_t* result = boat_dense_layer_backward_unflushed(layer, grad_output);
+    bt_flush_exposed();
+    return result;
+}
 
 static void sgd_step(boat_tensor_t* p, boat_tensor_t* g, float lr, bool clear) {
     if (!p || !g || p->nelements != g->nelements || p->nelements == 0) return;
@@ -140,6 +145,7 @@ void boat_dense_layer_update(boat_dense_layer_t* layer, float learning_rate) {
     if (!layer) return;
     sgd_step(layer->weight, layer->grad_weight, learning_rate, true);
     if (layer->use_bias) sgd_step(layer->bias, layer->grad_bias, learning_rate, true);
+    bt_flush_exposed();
 }
 
 void boat_dense_layer_set_weight(boat_dense_layer_t* layer, boat_tensor_t* weight) {
@@ -219,7 +225,7 @@ boat_layernorm_t* boat_layernorm_create(const boat_layernorm_config_t* config) {
     if (config->elementwise_affine) {
         norm->weight = create_vector(config->normalized_shape);
         norm->grad_weight = create_vector(config->normalized_shape);
-        float* g = norm->weight ? (float*)boat_tensor_data(norm->weight) : NULL;
+        float* g = norm->weight ? (float*)bt_host_rw(norm->weight) : NULL;
         if (!g || !norm->grad_weight) {
             boat_layernorm_free(norm);
             return NULL;
@@ -320,7 +326,7 @@ boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_t
     return dx;
 }
 
-boat_tensor_t* boat_layernorm_backward(boat_layernorm_t* norm, const boat_tensor_t* grad_output) {
+static boat_tensor_t* boat_layernorm_backward_unflushed(boat_layernorm_t* norm, const boat_tensor_t* grad_output) {
     if (!norm || !grad_output) return NULL;
     if (!norm->cache_input || !norm->cache_mean || !norm->cache_rstd) {
         fprintf(stderr, "Error: LayerNorm backward called before forward\n");
@@ -328,11 +334,17 @@ boat_tensor_t* boat_layernorm_backward(boat_layernorm_t* norm, const boat_tensor
     }
     return boat_layernorm_backward_impl(norm, norm->cache_input, norm->cache_mean, norm->cache_rstd, grad_output);
 }
+boat_tensor_t* boat_layernorm_backward(boat_layernorm_t* norm, const boat_tensor_t* grad_output) {
+    boat_tensor_t* result = boat_layernorm_backward_unflushed(norm, grad_output);
+    bt_flush_exposed();
+    return result;
+}
 
 void boat_layernorm_update(boat_layernorm_t* norm, float learning_rate) {
     if (!norm) return;
     sgd_step(norm->weight, norm->grad_weight, learning_rate, true);
     sgd_step(norm->bias, norm->grad_bias, learning_rate, true);
+    bt_flush_exposed();
 }
 
 void boat_layernorm_set_weight(boat_layernorm_t* norm, boat_tensor_t* weight) {
@@ -495,8 +507,16 @@ static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor
     return dx;
 }
 
+static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_query,
+                                         boat_tensor_t** grad_key, boat_tensor_t** grad_value);
 bool boat_attention_backward(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_query,
                              boat_tensor_t** grad_key, boat_tensor_t** grad_value) {
+    const bool ok = attention_backward_unflushed(a, grad_output, grad_query, grad_key, grad_value);
+    bt_flush_exposed();
+    return ok;
+}
+static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_query,
+                                         boat_tensor_t** grad_key, boat_tensor_t** grad_value) {
     if (!a || !grad_output) {
         fprintf(stderr, "[ERROR] boat_attention_backward: invalid arguments\n");
         return false;
@@ -560,6 +580,7 @@ void boat_attention_update(boat_attention_t* a, float lr) {
     sgd_step(a->bias_k, a->grad_bias_k, lr, false);
     sgd_step(a->bias_v, a->grad_bias_v, lr, false);
     sgd_step(a->bias_o, a->grad_bias_o, lr, false);
+    bt_flush_exposed();
 }
 
 /* stored only: the reference's forward ignores dropout as well (attention.c:1061-1062) */

@@ -80,6 +80,7 @@ static void inplace_op(int op, boat_tensor_t* a, const boat_tensor_t* b) {
     if (!pa || !pb) return;
     if (op == 0) boat_hip_ok(bh_add_inplace(pa, pb, (int64_t)a->nelements), "boat_add_");
     else boat_hip_ok(bh_binary(op, pa, pb, pa, (int64_t)a->nelements), "in-place op");
+    bt_flush_exposed();
 }
 void boat_add_(boat_tensor_t* a, const boat_tensor_t* b) { inplace_op(0, a, b); }
 void boat_sub_(boat_tensor_t* a, const boat_tensor_t* b) { inplace_op(1, a, b); }
@@ -141,9 +142,19 @@ boat_tensor_t* boat_matmul(const boat_tensor_t* a, const boat_tensor_t* b) {
 }
 
 boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1) {
-    if (!a || !bt_is_f32(a)) return NULL;
+    if (!a) return NULL;
     const int nd = (int)a->ndim;
     if (dim0 < 0 || dim1 < 0 || dim0 >= nd || dim1 >= nd) return NULL;   /* linear.c:241-244 (negative ints compare as huge) */
+    if (a->dtype != BOAT_DTYPE_FLOAT32 && a->dtype != BOAT_DTYPE_FLOAT64) {
+        /* linear.c:399-402: other element types get the swapped shape over an untransposed copy of the payload */
+        boat_tensor_t* copy = boat_tensor_clone(a);
+        if (copy) {
+            const int64_t t = copy->shape[dim0];
+            copy->shape[dim0] = copy->shape[dim1];
+            copy->shape[dim1] = t;
+        }
+        return copy;
+    }
     if (dim0 == dim1) return boat_tensor_clone(a);
     if (dim0 > dim1) {
         int t = dim0;
@@ -160,13 +171,15 @@ boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1) {
     }
     shape[dim0] = a->shape[dim1];
     shape[dim1] = a->shape[dim0];
-    boat_tensor_t* out = bt_new_uninit(shape, a->ndim, a->device);
+    boat_tensor_t* out = boat_tensor_create(shape, a->ndim, a->dtype, a->device);
     if (!out || out->nelements == 0) return out;
     const float* pa = bt_dev_read(a);
     float* po = bt_dev_write(out);
     bool ok = pa && po;
     const int64_t rows = a->shape[dim0], cols = a->shape[dim1];
-    if (ok && between == 1 && after == 1) {
+    if (ok && a->dtype == BOAT_DTYPE_FLOAT64) {
+        ok = boat_hip_ok(bh_swap_dims_f64((const double*)pa, (double*)po, before, rows, between, cols, after), "boat_transpose");
+    } else if (ok && between == 1 && after == 1) {
         /* the hot path's case, the last two dimensions: the tiled kernel, in slabs its grid can index */
         for (int64_t b0 = 0; ok && b0 < before; b0 += 32768) {
             const int64_t nb = before - b0 < 32768 ? before - b0 : 32768;

@@ -155,6 +155,7 @@ void boat_optimizer_step(boat_optimizer_t* optimizer) {
     if (!optimizer) return;
     adam_state_t* s = (adam_state_t*)optimizer;
     if (known_type(s)) adam_step(s);
+    bt_flush_exposed();
 }
 
 void boat_optimizer_zero_grad(boat_optimizer_t* optimizer) {
@@ -173,6 +174,7 @@ void boat_optimizer_zero_grad(boat_optimizer_t* optimizer) {
         count++;
     }
     if (count) boat_hip_ok(bh_zero_multi(s->tp, s->tn, count), "boat_optimizer_zero_grad");
+    bt_flush_exposed();
 }
 
 void boat_optimizer_free(boat_optimizer_t* optimizer) {

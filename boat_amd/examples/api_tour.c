@@ -139,11 +139,21 @@ static void tour_tape(void) {
     const boat_tensor_t* ga = boat_variable_grad(a);
     const boat_tensor_t* gb = boat_variable_grad(b);
     CHECK(ga && gb && boat_tensor_nelements(ga) == 20 && isfinite(sum_abs(ga)) && sum_abs(ga) > 0.0f && isfinite(sum_abs(gb)));
-    boat_variable_zero_grad(a);
-    boat_variable_t* dotp = boat_var_dot(a, b);
+    CHECK(boat_var_dot(a, b) == NULL);                               /* vectors only (src/ops/linear.c:176-183) */
+    const int64_t len[1] = {3};
+    boat_variable_t* u = boat_variable_create_with_shape(len, 1, BOAT_DTYPE_FLOAT32, true);
+    boat_variable_t* w = boat_variable_create_with_shape(len, 1, BOAT_DTYPE_FLOAT32, true);
+    float* pu = (float*)boat_tensor_data(boat_variable_data(u));
+    float* pw = (float*)boat_tensor_data(boat_variable_data(w));
+    for (int i = 0; i < 3; i++) {
+        pu[i] = (float)(i + 1);
+        pw[i] = (float)(i + 4);
+    }
+    boat_variable_t* dotp = boat_var_dot(u, w);
+    CHECK(dotp && first_value(boat_variable_data(dotp)) == 32.0f);
     boat_variable_backward(dotp, NULL);
-    CHECK(boat_variable_grad(a) && fabsf(first_value(boat_variable_grad(a)) - pb[0]) < 1e-6f);   /* d(a.b)/da = b */
-    boat_variable_t* owned[] = {dotp, mean, mm, rs, fl, ge, lsm, sm, act, sg, re, div, mul, sub, add, b, a};
+    CHECK(boat_variable_grad(u) && first_value(boat_variable_grad(u)) == 4.0f);   /* d(u.w)/du = w */
+    boat_variable_t* owned[] = {dotp, w, u, mean, mm, rs, fl, ge, lsm, sm, act, sg, re, div, mul, sub, add, b, a};
     for (size_t i = 0; i < sizeof(owned) / sizeof(owned[0]); i++) boat_variable_free(owned[i]);
     boat_autodiff_clear_computation_graph();
     boat_tensor_unref(ta);

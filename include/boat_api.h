@@ -362,6 +362,13 @@ BOAT_API void boat_sequential_add(boat_sequential_model_t* model, boat_layer_t* 
 /* ---- additions with no counterpart in the reference (named boat_hip_*) ---- */
 /* wait for all queued GPU work */
 BOAT_API void boat_hip_synchronize(void);
+/* Coherent-pointer mode, for callers that keep the float* of boat_tensor_data() across calls, write through it before
+ * a later call and read results through it afterwards (the reference's own tests do: test_attention_gradient_check.c:22-41,
+ * test_optimizer_adam.c:96-108).  Off by default: a data pointer is then good until the next call that takes the
+ * tensor, and parameters stay on the device.  On (this call, or BOAT_HIP_COHERENT_POINTERS=1 in the environment): a
+ * tensor whose pointer was handed out is uploaded before every use and copied back after every call that writes it,
+ * so such callers run unchanged, paying PCIe transfers for those tensors. */
+BOAT_API void boat_hip_set_coherent_pointers(int enable);
 /* gradient tensor of a variable, created zero-filled if absent and kept across boat_variable_zero_grad
  * (which then zero-fills in place), so it can be registered with an optimizer before the first backward */
 BOAT_API boat_tensor_t* boat_hip_variable_ensure_grad(boat_variable_t* variable);

@@ -133,6 +133,8 @@ int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, 
 /* out[a][d1][b][d0][c] = in[a][d0][b][d1][c]: boat_transpose of any two dimensions of a dense tensor (linear.c:238-406;
  * a, b, c are the products of the extents before, between and after the two) */
 int bh_swap_dims(const float* in, float* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c);
+/* the same for 8-byte elements (the float64 case of boat_transpose, linear.c:339-398): data movement only */
+int bh_swap_dims_f64(const double* in, double* out, int64_t a, int64_t d0, int64_t b, int64_t d1, int64_t c);
 /* dense layer backward in one call: dx = dy.W^T, gw += x^T.dy, gb += colsum(dy)  (dense.c:190-295) */
 int bh_dense_backward(const float* x, const float* w, const float* dy,
                       float* dx, float* gw, float* gb, int64_t m, int64_t k, int64_t n,

@@ -370,3 +370,46 @@ def test_gpu_model_over_callers_vtables(boat, oracle):
     assert np.max(np.abs(rec["dx"] - dx)) <= 1e-5 and np.max(np.abs(rec["gw"][0] - gw1)) <= 1e-5
     assert np.max(np.abs(rec["gw"][1] - gw2)) <= 1e-5
     assert all(np.array_equal(a, w - F(0.1) * g) for a, w, g in zip(rec["w_after"], ws, rec["gw"]))
+
+
+@pytest.mark.gpu
+def test_gpu_coherent_pointer_mode(boat):
+    """A caller that keeps the float* of boat_tensor_data() across calls: in the default mode the pointer is only good
+    until the next call that takes the tensor; in coherent-pointer mode writes through it reach the next call and the
+    results of a call are visible through it."""
+    import ctypes as C
+    boat.boat_hip_set_coherent_pointers(1)
+    try:
+        p, g = boat.tensor(np.array([5.0], F)), boat.tensor(np.array([2.0], F))
+        pp = C.cast(boat.boat_tensor_data(p), C.POINTER(C.c_float))
+        gp = C.cast(boat.boat_tensor_data(g), C.POINTER(C.c_float))
+        opt = boat.boat_adam_optimizer_create(0.01, 0.9, 0.999, 1e-8)
+        boat.boat_optimizer_add_parameter(opt, p, g)
+        boat.boat_optimizer_step(opt)
+        assert abs(pp[0] - 4.99) < 1e-6                         # read through the pointer taken before the step
+        gp[0] = -2.0                                            # written through the pointer taken before the step
+        boat.boat_optimizer_step(opt)
+        assert pp[0] > 4.99                                     # the step saw the new gradient
+        boat.boat_optimizer_zero_grad(opt)
+        assert gp[0] == 0.0
+        w = boat.tensor(np.ones((3, 2), F))
+        x = boat.tensor(np.ones((1, 3), F))
+        wp = C.cast(boat.boat_tensor_data(w), C.POINTER(C.c_float))
+        y1 = boat.boat_matmul(x, w)
+        wp[0] = 11.0
+        y2 = boat.boat_matmul(x, w)
+        assert boat.numpy(y1).tolist() == [[3.0, 3.0]] and boat.numpy(y2).tolist() == [[13.0, 3.0]]
+        for t in (y1, y2, x, w, p, g):
+            boat.boat_tensor_unref(t)
+        boat.boat_optimizer_free(opt)
+    finally:
+        boat.boat_hip_set_coherent_pointers(0)
+    # default mode: a tensor created now is not tracked, results stay on the device until asked for
+    p, g = boat.tensor(np.array([5.0], F)), boat.tensor(np.array([2.0], F))
+    opt = boat.boat_adam_optimizer_create(0.01, 0.9, 0.999, 1e-8)
+    boat.boat_optimizer_add_parameter(opt, p, g)
+    boat.boat_optimizer_step(opt)
+    assert abs(boat.numpy(p)[0] - 4.99) < 1e-6
+    boat.boat_optimizer_free(opt)
+    boat.boat_tensor_unref(p)
+    boat.boat_tensor_unref(g)

@@ -1,0 +1,62 @@
+"""The reference's OWN test programs, linked against libboat_amd.so instead of libboat.
+
+`make -C oracle reftests` compiles tests/unit/*.c and tests/*.c of the reference from where they lie, with the
+reference's headers, and links them with this repository's library (outputs in oracle/_ref/reftests, built where the
+reference tree exists).  They run here unchanged, in coherent-pointer mode: these programs keep the float* of
+boat_tensor_data() across calls (finite differences write weights through it, the optimizer tests read the updated
+parameter through it).  Programs that need the graph IR, the arena allocator or model loaders are outside the
+training path and are not built.
+
+test_schedulers aborts at its line 56 on the compiled reference too (a Release build of the reference compiles its
+asserts out): the scheduler here reproduces the reference's learning rates bit for bit (tests/test_schedulers.py), so
+it has to stop at the same assertion.
+"""
+import os
+import subprocess
+from pathlib import Path
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+BIN = Path(__file__).resolve().parent.parent / "oracle" / "_ref" / "reftests"
+
+PASSING = {   # program -> a line of its own success report
+    "test_autodiff": "Autodiff tests passed!",
+    "test_optimizer_adam": "All Adam optimizer tests passed!",
+    "test_optimizer_rmsprop": "All RMSprop optimizer tests passed!",
+    "test_optimizer_adagrad": "All Adagrad optimizer tests passed!",
+    "test_attention_gradient_check": "All gradient checks PASSED",
+    "test_conv_gradient_check": "All convolution gradient checks PASSED",
+    "test_attention_training": "Training test completed successfully",
+    "test_dense_forward": "Test PASSED",
+    "test_conv_forward": "Test PASSED",
+    "test_layernorm_simple": "Test completed",
+    "test_transpose": "All transpose tests PASSED",
+    "test_tensor": "Tensor tests passed!",
+    "test_basic": "All tests passed!",
+    "test_simple": None,
+    "test_layer_link": None,
+}
+
+
+def run(name, tmp_path):
+    exe = BIN / name
+    if not exe.exists():
+        pytest.skip(f"{exe} not built (make -C oracle reftests needs the reference tree)")
+    env = dict(os.environ, BOAT_HIP_COHERENT_POINTERS="1")
+    return subprocess.run([str(exe)], cwd=tmp_path, env=env, capture_output=True, text=True, errors="replace", timeout=100)
+
+
+@pytest.mark.parametrize("name", sorted(PASSING))
+def test_reference_program_passes_on_this_library(name, tmp_path):
+    proc = run(name, tmp_path)
+    assert proc.returncode == 0, (proc.stdout[-1500:], proc.stderr[-1500:])
+    if PASSING[name]:
+        assert PASSING[name] in proc.stdout, proc.stdout[-1500:]
+    assert "FAILED" not in proc.stdout
+
+
+def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):
+    proc = run("test_schedulers", tmp_path)
+    assert proc.returncode == -6 and "test_schedulers.c:56" in proc.stderr, (proc.returncode, proc.stderr[-500:])

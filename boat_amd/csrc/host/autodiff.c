@@ -48,7 +48,28 @@ struct boat_variable_t {
 
 struct boat_autodiff_context_t {
     bool grad_enabled;
+    const boat_graph_t* graph;   /* carried for the caller, never read here */
 };
+
+/* The reference hangs its tape on a graph object (the sources under src/graph) and lets callers hand one to a context
+ * (tests/unit/test_gradient_check.c:341-348).  The tape here needs none; the handle exists so that such callers link
+ * and run: it can be created, attached, fetched back and freed, nothing more. */
+struct boat_graph_t {
+    boat_device_t device;
+};
+boat_graph_t* boat_graph_create_with_device(boat_device_t device) {
+    boat_graph_t* g = (boat_graph_t*)calloc(1, sizeof(*g));
+    if (g) g->device = device;
+    return g;
+}
+boat_graph_t* boat_graph_create(void) { return boat_graph_create_with_device(BOAT_DEVICE_CPU); }
+void boat_graph_free(boat_graph_t* graph) { free(graph); }
+void boat_autodiff_context_set_graph(boat_autodiff_context_t* context, const boat_graph_t* graph) {
+    if (context) context->graph = graph;
+}
+boat_graph_t* boat_autodiff_context_get_graph(const boat_autodiff_context_t* context) {
+    return context ? (boat_graph_t*)context->graph : NULL;
+}
 
 static _Thread_local boat_autodiff_context_t* g_current = NULL;
 static boat_variable_t* g_live = NULL;

@@ -75,13 +75,14 @@ typedef struct {
 
 static boat_memory_stats_t g_stats;
 
+/* memory.c:28-43: allocated_bytes is what is live now, the block counts only grow */
 static void stats_alloc(size_t size) {
     g_stats.allocated_bytes += size;
     g_stats.allocated_blocks++;
-    size_t live = g_stats.allocated_bytes - g_stats.freed_bytes;
-    if (live > g_stats.peak_allocated_bytes) g_stats.peak_allocated_bytes = live;
+    if (g_stats.allocated_bytes > g_stats.peak_allocated_bytes) g_stats.peak_allocated_bytes = g_stats.allocated_bytes;
 }
 static void stats_free(size_t size) {
+    g_stats.allocated_bytes -= size < g_stats.allocated_bytes ? size : g_stats.allocated_bytes;   /* a reset may lie between */
     g_stats.freed_bytes += size;
     g_stats.freed_blocks++;
 }
@@ -127,6 +128,7 @@ static bool device_block_free(void* ptr) {
 void* boat_memory_allocate(size_t size, boat_device_t device, const char* file, int line) {
     (void)file;
     (void)line;
+    if (size == 0) return NULL;   /* memory.c:48-50 */
     if (device == BOAT_DEVICE_HIP) return device_block_alloc(size);
     mem_header_t* h = (mem_header_t*)malloc(sizeof(mem_header_t) + size);
     if (!h) return NULL;
@@ -152,6 +154,29 @@ void boat_memory_free(void* ptr) {
     h->magic = 0;
     stats_free(h->size);
     free(h);
+}
+void* boat_memory_reallocate(void* ptr, size_t new_size, boat_device_t device, const char* file, int line) {
+    /* memory.c:85-120: NULL allocates, size 0 frees, otherwise the block keeps its contents up to the smaller size */
+    if (!ptr) return boat_memory_allocate(new_size, device, file, line);
+    if (new_size == 0) {
+        boat_memory_free(ptr);
+        return NULL;
+    }
+    mem_header_t* h = (mem_header_t*)ptr - 1;
+    if (device == BOAT_DEVICE_HIP || h->magic != BOAT_MEM_MAGIC) {
+        boat_fail(BOAT_ERROR_INVALID_ARGUMENT, "boat_memory_reallocate: only host blocks of boat_memory_allocate can be resized");
+        return NULL;
+    }
+    const size_t old_size = h->size;
+    mem_header_t* grown = (mem_header_t*)realloc(h, sizeof(mem_header_t) + new_size);
+    if (!grown) {
+        fprintf(stderr, "Memory reallocation failed: %zu bytes at %s:%d\n", new_size, file ? file : "?", line);
+        return NULL;
+    }
+    grown->size = new_size;
+    stats_free(old_size);
+    stats_alloc(new_size);
+    return grown + 1;
 }
 void* boat_memory_allocate_device(size_t size, boat_device_t device, const char* file, int line) {
     return boat_memory_allocate(size, device, file, line);
@@ -188,7 +213,7 @@ boat_memory_stats_t boat_memory_get_stats(void) { return g_stats; }
 void boat_memory_reset_stats(void) { memset(&g_stats, 0, sizeof(g_stats)); }
 void boat_memory_print_stats(FILE* stream) {
     if (!stream) stream = stdout;
-    fprintf(stream, "Memory: allocated %zu B in %zu blocks, freed %zu B in %zu blocks, peak %zu B; device in use %zu B, cached %zu B\n",
+    fprintf(stream, "Memory: live %zu B, %zu blocks allocated so far, freed %zu B in %zu blocks, peak %zu B; device in use %zu B, cached %zu B\n",
             g_stats.allocated_bytes, g_stats.allocated_blocks, g_stats.freed_bytes, g_stats.freed_blocks,
             g_stats.peak_allocated_bytes, bh_bytes_in_use(), bh_bytes_cached());
 }

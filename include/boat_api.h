@@ -75,6 +75,7 @@ typedef struct {
 BOAT_API void* boat_memory_allocate(size_t size, boat_device_t device, const char* file, int line);
 BOAT_API void* boat_memory_allocate_zero(size_t size, boat_device_t device, const char* file, int line);
 BOAT_API void boat_memory_free(void* ptr);
+BOAT_API void* boat_memory_reallocate(void* ptr, size_t new_size, boat_device_t device, const char* file, int line);
 BOAT_API void* boat_memory_allocate_device(size_t size, boat_device_t device, const char* file, int line);
 BOAT_API void boat_memory_free_device(void* ptr, boat_device_t device);
 BOAT_API void boat_memory_copy(void* dest, const void* src, size_t size, boat_device_t dest_device, boat_device_t src_device);
@@ -164,6 +165,14 @@ BOAT_API boat_variable_t* boat_var_softmax(const boat_variable_t* a, int axis);
 BOAT_API boat_variable_t* boat_var_log_softmax(const boat_variable_t* a, int axis);
 BOAT_API boat_variable_t* boat_var_sum(const boat_variable_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
 BOAT_API boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim);
+/* include/boat/graph.h:18,41-43 and autodiff.h:87-88: an opaque handle that a context can carry for its caller.  The
+ * graph IR itself (nodes, edges, traversal) is outside the training path and is not provided. */
+typedef struct boat_graph_t boat_graph_t;
+BOAT_API boat_graph_t* boat_graph_create(void);
+BOAT_API boat_graph_t* boat_graph_create_with_device(boat_device_t device);
+BOAT_API void boat_graph_free(boat_graph_t* graph);
+BOAT_API void boat_autodiff_context_set_graph(boat_autodiff_context_t* context, const boat_graph_t* graph);
+BOAT_API boat_graph_t* boat_autodiff_context_get_graph(const boat_autodiff_context_t* context);
 BOAT_API boat_autodiff_context_t* boat_autodiff_context_create(void);
 BOAT_API void boat_autodiff_context_free(const boat_autodiff_context_t* context);
 BOAT_API void boat_autodiff_context_enable_grad(boat_autodiff_context_t* context);

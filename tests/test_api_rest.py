@@ -206,8 +206,9 @@ def test_gpu_small_hooks(boat):
     p = boat.boat_memory_allocate_device(4096, 0, b"test", 1)
     assert p and boat.boat_memory_get_stats().allocated_blocks == 1
     boat.boat_memory_free_device(p, 0)
-    s1 = boat.boat_memory_get_stats()
-    assert s1.freed_blocks == 1 and s1.freed_bytes == s1.allocated_bytes >= 4096
+    s1 = boat.boat_memory_get_stats()               # memory.c:28-43: allocated_bytes counts what is live
+    assert (s1.allocated_bytes, s1.allocated_blocks, s1.freed_blocks) == (0, 1, 1) and s1.freed_bytes == s1.peak_allocated_bytes >= 4096
+    assert not boat.boat_memory_allocate(0, 0, b"test", 2)         # memory.c:48-50
 
     from boat_amd.capi import LayerNormConfig
     import ctypes as C

@@ -4,8 +4,8 @@
 reference's headers, and links them with this repository's library (outputs in oracle/_ref/reftests, built where the
 reference tree exists).  They run here unchanged, in coherent-pointer mode: these programs keep the float* of
 boat_tensor_data() across calls (finite differences write weights through it, the optimizer tests read the updated
-parameter through it).  Programs that need the graph IR, the arena allocator or model loaders are outside the
-training path and are not built.
+parameter through it).  Programs that need the graph IR's nodes and edges, the arena allocator or model loaders are
+outside the training path and are not built.
 
 test_schedulers aborts at its line 56 on the compiled reference too (a Release build of the reference compiles its
 asserts out): the scheduler here reproduces the reference's learning rates bit for bit (tests/test_schedulers.py), so
@@ -35,6 +35,7 @@ PASSING = {   # program -> a line of its own success report
     "test_transpose": "All transpose tests PASSED",
     "test_tensor": "Tensor tests passed!",
     "test_basic": "All tests passed!",
+    "test_memory": "Memory tests passed!",
     "test_simple": None,
     "test_layer_link": None,
 }
@@ -55,6 +56,22 @@ def test_reference_program_passes_on_this_library(name, tmp_path):
     if PASSING[name]:
         assert PASSING[name] in proc.stdout, proc.stdout[-1500:]
     assert "FAILED" not in proc.stdout
+
+
+def test_gradient_check_program_reports_what_it_reports_on_the_reference(tmp_path):
+    """tests/unit/test_gradient_check.c compares analytical gradients with float32 central differences at a tolerance
+    the differences do not meet: on the compiled reference it passes addition and reports two mismatches for
+    multiplication (numerical -0.0160933 / -0.00417233 against analytical -0.0163637 / -0.00411147) and exits 1.  The
+    same binary on this library prints the same lines: the analytical values agree to every printed digit."""
+    proc = run("test_gradient_check", tmp_path)
+    assert proc.returncode == 1
+    out = proc.stdout
+    addition, multiplication = out.split("Testing multiplication operation gradient...")
+    assert "Testing addition operation gradient..." in addition and "  PASSED" in addition and "Mismatch" not in addition
+    out = multiplication
+    assert "Mismatch for b[1]: analytical=-0.0163637, numerical=-0.0160933" in out
+    assert "Mismatch for b[3]: analytical=-0.00411147, numerical=-0.00417233" in out
+    assert "FAILED: 2 mismatches" in out
 
 
 def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):

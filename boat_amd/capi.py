@@ -65,6 +65,7 @@ _SIGS = {
     "boat_tensor_data": (P, [P]),
     "boat_tensor_const_data": (P, [P]),
     "boat_tensor_reshape": (P, [P, C.POINTER(C.c_int64), C.c_size_t]),
+    "boat_tensor_slice": (P, [P, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "boat_tensor_is_contiguous": (C.c_bool, [P]),
     "boat_dtype_name": (C.c_char_p, [C.c_int]),
     # memory and error reporting

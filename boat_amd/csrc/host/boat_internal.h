@@ -24,6 +24,7 @@ struct boat_tensor_t {
     boat_dtype_t dtype;
     boat_device_t device;
     boat_storage_t* st;
+    size_t offset;         /* bytes into the storage; non-zero only for a slice (tensor.c:368-431) */
     size_t nbytes;
     size_t nelements;
     bool is_contiguous;

@@ -404,11 +404,13 @@ static bool storage_dev_ready(boat_storage_t* st, bool need_contents) {
 
 const float* bt_dev_read(const boat_tensor_t* t) {
     if (!t || !storage_dev_ready(t->st, true)) return NULL;
-    return (const float*)bh_buffer_ptr(t->st->dev);
+    return (const float*)((const char*)bh_buffer_ptr(t->st->dev) + t->offset);
 }
 float* bt_dev_write(boat_tensor_t* t) {
     if (!t) return NULL;
-    /* a view covers its whole parent payload (reshape only), so a full overwrite is still full */
+    /* a reshaped view covers its whole parent payload, so a full overwrite is still full; a slice covers a part of
+     * it and the rest has to stay what it is */
+    if (t->nbytes != t->st->nbytes) return bt_dev_rw(t);
     if (!storage_dev_ready(t->st, false)) return NULL;
     t->st->dev_valid = true;
     t->st->host_valid = false;
@@ -419,7 +421,7 @@ float* bt_dev_rw(boat_tensor_t* t) {
     if (!t || !storage_dev_ready(t->st, true)) return NULL;
     t->st->host_valid = false;
     mark_device_write(t->st);
-    return (float*)bh_buffer_ptr(t->st->dev);
+    return (float*)((char*)bh_buffer_ptr(t->st->dev) + t->offset);
 }
 
 boat_tensor_t* boat_tensor_from_data(const int64_t* shape, size_t ndim, boat_dtype_t dtype, const void* data) {
@@ -463,7 +465,7 @@ void* bt_host_rw(boat_tensor_t* tensor) {
     if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_rw(tensor);
     if (!storage_host_ready(st)) return NULL;
     st->dev_valid = false;   /* written through the pointer */
-    return st->host;
+    return (char*)st->host + tensor->offset;
 }
 void* boat_tensor_data(const boat_tensor_t* tensor) {
     void* p = bt_host_rw((boat_tensor_t*)tensor);
@@ -475,7 +477,7 @@ const void* boat_tensor_const_data(const boat_tensor_t* tensor) {
     if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_read(tensor);
     if (!storage_host_ready(tensor->st)) return NULL;
     if (coherent_mode()) tensor->st->exposed = true;
-    return tensor->st->host;
+    return (const char*)tensor->st->host + tensor->offset;
 }
 
 boat_tensor_t* boat_tensor_reshape(const boat_tensor_t* tensor, const int64_t* new_shape, size_t new_ndim) {
@@ -487,7 +489,66 @@ boat_tensor_t* boat_tensor_reshape(const boat_tensor_t* tensor, const int64_t* n
         return NULL;
     }
     boat_tensor_t* v = tensor_alloc(new_shape, new_ndim, tensor->dtype, tensor->device, tensor->st);
-    if (v) v->is_contiguous = false;   /* the reference marks reshaped views so (tensor.c:289) */
+    if (v) {
+        v->is_contiguous = false;   /* the reference marks reshaped views so (tensor.c:289) */
+        v->offset = tensor->offset;
+    }
+    return v;
+}
+
+/* tensor.c:302-456: a view that starts at element `start` (row-major) of a contiguous tensor and is read as a dense
+ * tensor of the new extents, i.e. exact for ranges of the leading dimension (a batch of samples), which is how the
+ * callers use it (examples/mnist/mnist_autodiff.c:2387-2392).  Steps other than 1 are refused, as there. */
+boat_tensor_t* boat_tensor_slice(const boat_tensor_t* tensor, const size_t* start, const size_t* end, const size_t* step) {
+    if (!tensor || !start || !end) return NULL;
+    const size_t ndim = tensor->ndim;
+    if (ndim == 0) {
+        fprintf(stderr, "Error: Cannot slice scalar tensor\n");
+        return NULL;
+    }
+    int64_t shape[BOAT_MAX_DIMS];
+    for (size_t i = 0; i < ndim; i++) {
+        if (step && step[i] == 0) {
+            fprintf(stderr, "Error: Step cannot be zero\n");
+            return NULL;
+        }
+    }
+    for (size_t i = 0; i < ndim; i++) {
+        const size_t dim = (size_t)tensor->shape[i], st = step ? step[i] : 1;
+        if (start[i] >= dim || end[i] > dim || start[i] > end[i]) {
+            fprintf(stderr, "Error: Invalid slice range for dimension %zu: [%zu, %zu) (dim size: %zu)\n", i, start[i], end[i], dim);
+            return NULL;
+        }
+        shape[i] = (int64_t)((end[i] - start[i] + st - 1) / st);
+        if (shape[i] == 0) {
+            fprintf(stderr, "Error: Slice results in zero-size dimension %zu\n", i);
+            return NULL;
+        }
+    }
+    if (!tensor->is_contiguous) {
+        fprintf(stderr, "Error: Slicing non-contiguous tensors not supported\n");
+        return NULL;
+    }
+    size_t first = 0, stride = 1;
+    for (size_t i = ndim; i-- > 0;) {
+        first += start[i] * stride;
+        stride *= (size_t)tensor->shape[i];
+    }
+    for (size_t i = 0; i < ndim; i++) {
+        if (step && step[i] != 1) {
+            fprintf(stderr, "Error: Non-unit step slicing not yet implemented\n");
+            return NULL;
+        }
+    }
+    boat_tensor_t* v = tensor_alloc(shape, ndim, tensor->dtype, tensor->device, tensor->st);
+    if (!v) return NULL;
+    v->offset = tensor->offset + first * boat_dtype_size(tensor->dtype);
+    v->is_contiguous = false;   /* tensor.c:436 */
+    if (v->offset + v->nbytes > tensor->st->nbytes) {   /* a range that is not made of whole leading rows can run past the payload */
+        fprintf(stderr, "Error: slice does not fit the tensor's payload\n");
+        boat_tensor_free(v);
+        return NULL;
+    }
     return v;
 }
 
@@ -498,7 +559,7 @@ boat_tensor_t* boat_tensor_clone(const boat_tensor_t* tensor) {
     boat_storage_t* st = tensor->st;
     if (st->dev_valid) {
         float* dst = bt_dev_write(c);
-        if (!dst || !boat_hip_ok(bh_memcpy_d2d(dst, bh_buffer_ptr(st->dev), tensor->nbytes), "boat_tensor_clone")) {
+        if (!dst || !boat_hip_ok(bh_memcpy_d2d(dst, (const char*)bh_buffer_ptr(st->dev) + tensor->offset, tensor->nbytes), "boat_tensor_clone")) {
             boat_tensor_free(c);
             return NULL;
         }
@@ -508,7 +569,7 @@ boat_tensor_t* boat_tensor_clone(const boat_tensor_t* tensor) {
             boat_tensor_free(c);
             return NULL;
         }
-        memcpy(dst, st->host, tensor->nbytes);
+        memcpy(dst, (const char*)st->host + tensor->offset, tensor->nbytes);
     }
     return c;
 }
@@ -522,8 +583,8 @@ boat_tensor_t* boat_tensor_to_device(const boat_tensor_t* tensor, boat_device_t 
     if (dev == BOAT_DEVICE_HIP) {
         float* dst = bt_dev_write(out);
         bool ok = dst != NULL;
-        if (ok && src->dev_valid) ok = boat_hip_ok(bh_memcpy_d2d(dst, bh_buffer_ptr(src->dev), tensor->nbytes), "boat_tensor_to_device");
-        else if (ok) ok = boat_hip_ok(bh_memcpy_h2d(dst, src->host, tensor->nbytes), "boat_tensor_to_device");
+        if (ok && src->dev_valid) ok = boat_hip_ok(bh_memcpy_d2d(dst, (const char*)bh_buffer_ptr(src->dev) + tensor->offset, tensor->nbytes), "boat_tensor_to_device");
+        else if (ok) ok = boat_hip_ok(bh_memcpy_h2d(dst, (const char*)src->host + tensor->offset, tensor->nbytes), "boat_tensor_to_device");
         if (!ok) {
             boat_tensor_free(out);
             return NULL;
@@ -531,8 +592,8 @@ boat_tensor_t* boat_tensor_to_device(const boat_tensor_t* tensor, boat_device_t 
     } else {
         void* dst = bt_host_rw(out);
         bool ok = dst != NULL;
-        if (ok && src->host_valid) memcpy(dst, src->host, tensor->nbytes);
-        else if (ok) ok = boat_hip_ok(bh_memcpy_d2h(dst, bh_buffer_ptr(src->dev), tensor->nbytes), "boat_tensor_to_device");
+        if (ok && src->host_valid) memcpy(dst, (const char*)src->host + tensor->offset, tensor->nbytes);
+        else if (ok) ok = boat_hip_ok(bh_memcpy_d2h(dst, (const char*)bh_buffer_ptr(src->dev) + tensor->offset, tensor->nbytes), "boat_tensor_to_device");
         if (!ok) {
             boat_tensor_free(out);
             return NULL;

@@ -57,6 +57,7 @@ BOAT_API size_t boat_tensor_nelements(const boat_tensor_t* tensor);
 BOAT_API bool boat_tensor_is_contiguous(const boat_tensor_t* tensor);
 BOAT_API void* boat_tensor_data(const boat_tensor_t* tensor);
 BOAT_API const void* boat_tensor_const_data(const boat_tensor_t* tensor);
+BOAT_API boat_tensor_t* boat_tensor_slice(const boat_tensor_t* tensor, const size_t* start, const size_t* end, const size_t* step);   /* tensor.h:87; a view */
 BOAT_API boat_tensor_t* boat_tensor_reshape(const boat_tensor_t* tensor, const int64_t* new_shape, size_t new_ndim);
 BOAT_API boat_tensor_t* boat_tensor_to_device(const boat_tensor_t* tensor, boat_device_t dev);   /* declared only in the reference (tensor.h:92) */
 BOAT_API boat_tensor_t* boat_tensor_clone(const boat_tensor_t* tensor);

@@ -1108,3 +1108,44 @@ def model_over_callers_vtables(api, x, weights, biases, dy=None, lr=None):
     for d in dense:
         api.boat_dense_layer_free(d)
     return rec
+
+
+def slice_facts(api):
+    """boat_tensor_slice (src/core/tensor.c:302-456): views on ranges of the leading dimension, as the MNIST example
+    batches its samples (examples/mnist/mnist_autodiff.c:2387-2392)."""
+    out = {}
+
+    def idx(*v):
+        return (C.c_size_t * len(v))(*v)
+
+    base_np = np.arange(24, dtype=np.float32).reshape(6, 4)
+    base = api.tensor(base_np)
+    rows = api.boat_tensor_slice(base, idx(2, 0), idx(5, 4), None)
+    out["shape"] = api.shape(rows)
+    out["values"] = api.numpy(rows).tolist()
+    out["is_contiguous"] = bool(api.boat_tensor_is_contiguous(rows))
+    out["pointer_offset"] = api.boat_tensor_data(rows) - api.boat_tensor_data(base)
+    out["nbytes"] = int(api.boat_tensor_nbytes(rows))
+    out["step_two_refused"] = not api.boat_tensor_slice(base, idx(0, 0), idx(6, 4), idx(2, 1))
+    out["step_zero_refused"] = not api.boat_tensor_slice(base, idx(0, 0), idx(6, 4), idx(0, 1))
+    out["start_past_end_refused"] = not api.boat_tensor_slice(base, idx(6, 0), idx(6, 4), None)
+    out["reversed_range_refused"] = not api.boat_tensor_slice(base, idx(3, 0), idx(2, 4), None)
+    out["empty_range_refused"] = not api.boat_tensor_slice(base, idx(3, 0), idx(3, 4), None)
+    view = api.boat_tensor_reshape(base, (C.c_int64 * 2)(4, 6), 2)
+    out["slice_of_a_view_refused"] = not api.boat_tensor_slice(view, idx(0, 0), idx(2, 6), None)
+    api.boat_tensor_unref(view)
+    # the slice is a window on its parent: an in-place operation on it changes those rows of the parent and no others
+    ones = api.tensor(np.ones((3, 4), np.float32))
+    api.boat_add_(rows, ones)
+    out["parent_after_add_on_slice"] = api.numpy(base).tolist()
+    # arithmetic on a slice that does not start on 16 bytes
+    odd = api.tensor(np.arange(18, dtype=np.float32).reshape(6, 3))
+    win = api.boat_tensor_slice(odd, idx(1, 0), idx(4, 3), None)
+    w = api.tensor(np.array([[1, 0], [0, 1], [1, 1]], np.float32))
+    prod = api.boat_matmul(win, w)
+    out["matmul_on_slice"] = api.numpy(prod).tolist()
+    api.boat_tensor_unref(base)                                    # the slice keeps its parent's payload alive
+    out["values_after_parent_unref"] = api.numpy(rows).tolist()
+    for t in (prod, w, win, odd, ones, rows):
+        api.boat_tensor_unref(t)
+    return out

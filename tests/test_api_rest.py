@@ -414,3 +414,51 @@ def test_gpu_coherent_pointer_mode(boat):
     boat.boat_optimizer_free(opt)
     boat.boat_tensor_unref(p)
     boat.boat_tensor_unref(g)
+
+
+SLICE_FACTS = {
+    "shape": (3, 4), "values": [[8.0, 9.0, 10.0, 11.0], [12.0, 13.0, 14.0, 15.0], [16.0, 17.0, 18.0, 19.0]],
+    "is_contiguous": False, "pointer_offset": 32, "nbytes": 48,
+    "step_two_refused": True, "step_zero_refused": True, "start_past_end_refused": True, "reversed_range_refused": True,
+    "empty_range_refused": True, "slice_of_a_view_refused": True,
+    "parent_after_add_on_slice": [[0.0, 1.0, 2.0, 3.0], [4.0, 5.0, 6.0, 7.0], [9.0, 10.0, 11.0, 12.0], [13.0, 14.0, 15.0, 16.0],
+                                  [17.0, 18.0, 19.0, 20.0], [20.0, 21.0, 22.0, 23.0]],
+    "matmul_on_slice": [[8.0, 9.0], [14.0, 15.0], [20.0, 21.0]],
+    "values_after_parent_unref": [[9.0, 10.0, 11.0, 12.0], [13.0, 14.0, 15.0, 16.0], [17.0, 18.0, 19.0, 20.0]],
+}
+
+
+def test_reference_slice_facts(ref):
+    assert bc.slice_facts(ref) == SLICE_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_slice_facts(boat):
+    got = bc.slice_facts(boat)
+    diff = {k: (got.get(k), v) for k, v in SLICE_FACTS.items() if got.get(k) != v}
+    assert not diff and set(got) == set(SLICE_FACTS), diff
+
+
+@pytest.mark.gpu
+def test_gpu_slices_feed_the_layers(boat, oracle):
+    """Batches cut from one sample tensor with boat_tensor_slice go through a dense layer forward and backward
+    (the loop of examples/mnist/mnist_autodiff.c:2380-2440), including a batch that starts off a 16-byte boundary."""
+    import ctypes as C
+    rng = np.random.default_rng(84)
+    data = rng.standard_normal((10, 7)).astype(F)
+    w, b = rng.standard_normal((7, 5)).astype(F), rng.standard_normal(5).astype(F)
+    samples = boat.tensor(data)
+    layer = bc._make_dense(boat, w, b)
+    for lo, hi in ((0, 4), (3, 8), (9, 10)):
+        batch = boat.boat_tensor_slice(samples, (C.c_size_t * 2)(lo, 0), (C.c_size_t * 2)(hi, 7), None)
+        ty = boat.boat_dense_layer_forward(layer, batch)
+        assert np.max(np.abs(boat.numpy(ty) - oracle.dense_forward(data[lo:hi], w, b))) <= 1e-5
+        tdy = boat.tensor(np.ones((hi - lo, 5), F))
+        tdx = boat.boat_dense_layer_backward(layer, tdy)
+        want_dx, _, _ = oracle.dense_backward(data[lo:hi], w, np.ones((hi - lo, 5), F))
+        assert np.max(np.abs(boat.numpy(tdx) - want_dx)) <= 1e-5
+        for t in (tdx, tdy, ty, batch):
+            boat.boat_tensor_unref(t)
+    assert np.array_equal(boat.numpy(samples), data)
+    boat.boat_tensor_unref(samples)
+    boat.boat_dense_layer_free(layer)

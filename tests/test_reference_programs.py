@@ -1,6 +1,6 @@
-"""The reference's OWN test programs, linked against libboat_amd.so instead of libboat.
+"""The reference's OWN test programs (and its optimizer benchmark), linked against libboat_amd.so instead of libboat.
 
-`make -C oracle reftests` compiles tests/unit/*.c and tests/*.c of the reference from where they lie, with the
+`make -C oracle reftests` compiles tests/unit/*.c, tests/*.c and benchmarks/linear_regression.c of the reference from where they lie, with the
 reference's headers, and links them with this repository's library (outputs in oracle/_ref/reftests, built where the
 reference tree exists).  They run here unchanged, in coherent-pointer mode: these programs keep the float* of
 boat_tensor_data() across calls (finite differences write weights through it, the optimizer tests read the updated
@@ -72,6 +72,18 @@ def test_gradient_check_program_reports_what_it_reports_on_the_reference(tmp_pat
     assert "Mismatch for b[1]: analytical=-0.0163637, numerical=-0.0160933" in out
     assert "Mismatch for b[3]: analytical=-0.00411147, numerical=-0.00417233" in out
     assert "FAILED: 2 mismatches" in out
+
+
+def test_optimizer_benchmark_of_the_reference_reports_the_same_losses(tmp_path):
+    """benchmarks/linear_regression.c: 1000 steps each with Adam, Adam + StepLR, RMSprop and Adagrad on synthetic data
+    from rand().  It registers boat_variable_grad() before the first backward, when that is still NULL
+    (benchmarks/linear_regression.c:304-305), so on the reference every optimizer leaves the loss where it starts,
+    1.273380; linked against this library the program reports the same final loss four times."""
+    proc = run("linear_regression", tmp_path)
+    assert proc.returncode == 0, proc.stderr[-1000:]
+    summary = proc.stdout.split("Benchmark Results Summary")[1]
+    rows = [line.split() for line in summary.splitlines() if line.startswith(("Adam", "RMSprop", "Adagrad"))]
+    assert len(rows) == 4 and all("1.273380" in r for r in rows), summary
 
 
 def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):

@@ -10,6 +10,12 @@ come from an independent library, torch autograd in float64 on the CPU.
 Run from the repository root in a container that has the reference tree:
     make -C oracle ref && python tests/golden/make_golden.py
 Fixtures are plain numpy archives (np.load with allow_pickle=False reads them).
+
+One fixture is text: scheduler_usage_lines.txt holds the learning-rate lines that examples/scheduler_usage.c of the
+reference printed when built against the compiled reference:
+    gcc -O2 -std=c11 -Dthread_local=_Thread_local -I$REF/include $REF/examples/scheduler_usage.c \
+        -Loracle/_ref -lboat_ref -Wl,-rpath,$PWD/oracle/_ref -lm -o /tmp/scheduler_usage && /tmp/scheduler_usage \
+        | grep -i "learning rate\|LR" | grep -v "create called\|create:" > tests/golden/scheduler_usage_lines.txt
 """
 import sys
 from pathlib import Path

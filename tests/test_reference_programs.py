@@ -86,6 +86,23 @@ def test_optimizer_benchmark_of_the_reference_reports_the_same_losses(tmp_path):
     assert len(rows) == 4 and all("1.273380" in r for r in rows), summary
 
 
+def test_scheduler_example_prints_the_learning_rates_it_prints_on_the_reference(tmp_path):
+    """examples/scheduler_usage.c (step, cosine and caller-function schedules driving Adam and RMSprop): its
+    learning-rate lines on this library are, character for character, the lines it printed on the compiled reference
+    (tests/golden/scheduler_usage_lines.txt, written from that run)."""
+    proc = run("scheduler_usage", tmp_path)
+    assert proc.returncode == 0, proc.stderr[-1000:]
+    want = (Path(__file__).resolve().parent / "golden" / "scheduler_usage_lines.txt").read_text().splitlines()
+    got = [line for line in proc.stdout.splitlines() if ("learning rate" in line.lower() or "LR" in line)
+           and "create called" not in line and "create:" not in line]
+    assert got == want and len(want) > 40
+
+
+def test_relu_example_of_the_reference(tmp_path):
+    proc = run("test_relu", tmp_path)
+    assert proc.returncode == 0 and "Result data: 0.0 0.0 0.0 0.0 1.0 2.0" in proc.stdout, proc.stdout[-500:]
+
+
 def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):
     proc = run("test_schedulers", tmp_path)
     assert proc.returncode == -6 and "test_schedulers.c:56" in proc.stderr, (proc.returncode, proc.stderr[-500:])

@@ -1149,3 +1149,15 @@ def slice_facts(api):
     for t in (prod, w, win, odd, ones, rows):
         api.boat_tensor_unref(t)
     return out
+
+
+def write_mnist_example_files(folder, train_images, train_labels, test_images, test_labels):
+    """The four files examples/mnist/mnist.c reads from ./data (its loader, mnist.c:29-95: u32 ndim, u32 extents, raw
+    payload; images as float32 [n, 28, 28], labels as bytes [n])."""
+    import struct
+    data = folder / "data"
+    data.mkdir(parents=True, exist_ok=True)
+    for name, arr in (("train_images_small.bin", np.asarray(train_images, np.float32)), ("train_labels_small.bin", np.asarray(train_labels, np.uint8)),
+                      ("test_images_small.bin", np.asarray(test_images, np.float32)), ("test_labels_small.bin", np.asarray(test_labels, np.uint8))):
+        with open(data / name, "wb") as f:
+            f.write(struct.pack("<I", arr.ndim) + struct.pack("<%dI" % arr.ndim, *arr.shape) + arr.tobytes())

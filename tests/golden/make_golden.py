@@ -228,6 +228,34 @@ def main():
         assert other.load(path)
         save("cnn_checkpoint", content=np.frombuffer(Path(path).read_bytes(), np.uint8), x=x, logits=other.logits(x))
 
+    # ---- the reference's layer-based MNIST example on a small synthetic set: what it prints on the reference ----
+    if not ONLY or "mnist_synthetic" in ONLY:
+        import re
+        import subprocess
+        import tempfile
+        r4 = np.random.default_rng(4)
+        sets = {}
+        for name, count in (("train", 80), ("test", 16)):
+            labels = r4.integers(0, 10, count).astype(np.uint8)
+            images = r4.integers(0, 40, (count, 28, 28)).astype(np.uint8)
+            for i, c in enumerate(labels):                      # a bright patch whose place tells the class
+                row, col = divmod(int(c), 4)
+                images[i, 4 + 7 * row: 11 + 7 * row, 2 + 6 * col: 8 + 6 * col] += 200
+            sets[name] = (images, labels)
+        with tempfile.TemporaryDirectory() as tmp:
+            bc.write_mnist_example_files(Path(tmp), *sets["train"], *sets["test"])
+            exe = Path(tmp) / "mnist"
+            ref_root = Path("/root/reference")
+            subprocess.run(["gcc", "-O2", "-std=c11", "-w", "-Dthread_local=_Thread_local", "-D_POSIX_C_SOURCE=200809L",
+                            f"-I{ref_root / 'include'}", f"-I{ref_root / 'src'}", str(ref_root / "examples/mnist/mnist.c"),
+                            "-o", str(exe), f"-L{ROOT / 'oracle/_ref'}", "-lboat_ref", f"-Wl,-rpath,{ROOT / 'oracle/_ref'}", "-lm"],
+                           check=True)
+            out = subprocess.run([str(exe)], cwd=tmp, capture_output=True, text=True, errors="replace", check=True).stdout
+        lines = [re.sub(r"time=[0-9.]+s, ", "", line) for line in out.splitlines() if re.match(r"Epoch \d|Test accuracy", line)]
+        print("\n".join(lines))
+        save("mnist_synthetic", train_images=sets["train"][0], train_labels=sets["train"][1], test_images=sets["test"][0],
+             test_labels=sets["test"][1], reference_lines=np.array(lines))
+
     # ---- not the reference: float64 autograd of an independent library ----
     import torch
     torch.manual_seed(0)

@@ -103,6 +103,31 @@ def test_relu_example_of_the_reference(tmp_path):
     assert proc.returncode == 0 and "Result data: 0.0 0.0 0.0 0.0 1.0 2.0" in proc.stdout, proc.stdout[-500:]
 
 
+@pytest.mark.parametrize("coherent", ["1", "0"])
+def test_mnist_example_of_the_reference_trains_as_on_the_reference(tmp_path, coherent):
+    """examples/mnist/mnist.c, the layer-hook training loop (conv, pool, dense, softmax; forward, backward and update
+    per batch, mnist.c:197-246) on a small synthetic set: 80 training and 16 test images whose bright patch tells the
+    class (tests/golden/mnist_synthetic.npz, which also holds the lines the program printed on the compiled reference).
+    Linked against this library it prints the same accuracy after every epoch and on the test set, in coherent-pointer
+    mode and in the default mode alike (the program fetches data pointers anew whenever it needs them)."""
+    import re
+
+    import numpy as np
+
+    import boat_cases as bc
+    with np.load(Path(__file__).resolve().parent / "golden" / "mnist_synthetic.npz", allow_pickle=False) as z:
+        g = {k: z[k] for k in z.files}
+    bc.write_mnist_example_files(tmp_path, g["train_images"], g["train_labels"], g["test_images"], g["test_labels"])
+    exe = BIN / "mnist"
+    if not exe.exists():
+        pytest.skip(f"{exe} not built (make -C oracle reftests needs the reference tree)")
+    env = dict(os.environ, BOAT_HIP_COHERENT_POINTERS=coherent)
+    proc = subprocess.run([str(exe)], cwd=tmp_path, env=env, capture_output=True, text=True, errors="replace", timeout=100)
+    assert proc.returncode == 0, proc.stderr[-1000:]
+    lines = [re.sub(r"time=[0-9.]+s, ", "", line) for line in proc.stdout.splitlines() if re.match(r"Epoch \d|Test accuracy", line)]
+    assert lines == [str(line) for line in g["reference_lines"]] and len(lines) == 6
+
+
 def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):
     proc = run("test_schedulers", tmp_path)
     assert proc.returncode == -6 and "test_schedulers.c:56" in proc.stderr, (proc.returncode, proc.stderr[-500:])

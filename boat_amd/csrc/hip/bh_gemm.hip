@@ -228,7 +228,7 @@ struct DirectFrags {
     }
 };
 
-template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT>
+template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1>   // KT: k-tiles per LDS stage (and per barrier)
 __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int A_FLOATS = DIRECT ? DirectTile<A_KC, BM>::floats : TileShape<A_KC, BM>::floats;
@@ -271,7 +271,69 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    if constexpr (DIRECT) {
+    if constexpr (DIRECT && KT == 2) {
+        // Two k-tiles per stage and one barrier per pair: the same pipeline as below with the barrier (where every
+        // matrix core of the workgroup drains) paid once per 32 k instead of once per 16.  The contraction range is a
+        // multiple of 32 here (the host checks), so every stage is whole.
+        constexpr int NW = NT / 64;
+        constexpr unsigned TILE_BYTES = (unsigned)(STAGE * sizeof(float));
+        DirectLoader<A_KC, BM, NW> da;
+        DirectLoader<B_KC, BN, NW> db;
+        da.init(A, g.lda, m0, g.m, k_begin, smem, wave, lane);
+        db.init(B, g.ldb, n0, g.n, k_begin, smem + A_FLOATS, wave, lane);
+        const int64_t pairs = (k_end - k_begin) / (2 * kBK);
+        DirectFrags<A_KC, BM, TM> fa0, fa1;
+        DirectFrags<B_KC, BN, TN> fb0, fb1;
+        auto products = [&](const DirectFrags<A_KC, BM, TM>& fa, const DirectFrags<B_KC, BN, TN>& fb) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto issue_pair = [&](unsigned stage) {     // the next two k-tiles of this wavefront's blocks into stage `stage`
+            da.issue(stage * 2 * TILE_BYTES);
+            db.issue(stage * 2 * TILE_BYTES);
+            da.issue(stage * 2 * TILE_BYTES + TILE_BYTES);
+            db.issue(stage * 2 * TILE_BYTES + TILE_BYTES);
+        };
+        if (pairs > 0) issue_pair(0);
+        if (pairs > 1) issue_pair(1);
+        wait_direct_loads();
+        __syncthreads();
+        if (pairs > 0) {
+            fa0.load(smem, wm * Cfg::WM, 0, r, half);
+            fb0.load(smem + A_FLOATS, wn * Cfg::WN, 0, r, half);
+        }
+        int cur = 0;
+        for (int64_t p = 0; p < pairs; p++) {
+            const float* sa0 = smem + cur * 2 * STAGE;     // first k-tile of the pair: A, then B
+            const float* sa1 = sa0 + STAGE;                // second k-tile
+            fa1.load(sa0, wm * Cfg::WM, 8, r, half);
+            fb1.load(sa0 + A_FLOATS, wn * Cfg::WN, 8, r, half);
+            products(fa0, fb0);
+            fa0.load(sa1, wm * Cfg::WM, 0, r, half);
+            fb0.load(sa1 + A_FLOATS, wn * Cfg::WN, 0, r, half);
+            products(fa1, fb1);
+            fa1.load(sa1, wm * Cfg::WM, 8, r, half);
+            fb1.load(sa1 + A_FLOATS, wn * Cfg::WN, 8, r, half);
+            products(fa0, fb0);
+            wait_direct_loads();       // pair p+1, issued a whole pair ago
+            __syncthreads();           // ... is visible to everyone, and everyone has the last fragments of stage cur in registers
+            if (p + 2 < pairs) issue_pair((unsigned)cur);
+            if (p + 1 < pairs) {
+                const float* na = smem + (cur ^ 1) * 2 * STAGE;
+                fa0.load(na, wm * Cfg::WM, 0, r, half);
+                fb0.load(na + A_FLOATS, wn * Cfg::WN, 0, r, half);
+            }
+            products(fa1, fb1);
+            cur ^= 1;
+        }
+    } else if constexpr (DIRECT) {
         // tile kt+1 streams straight into the other LDS stage while tile kt feeds the MFMAs; the wait for this
         // wavefront's own loads and the barrier at the end of the k-tile publish it to the workgroup
         constexpr int NW = NT / 64;
@@ -870,21 +932,21 @@ __global__ __launch_bounds__(256) void swap_dims_kernel(const T* __restrict__ in
     }
 }
 
-template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT>
+template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1>
 static int launch_mfma(const GemmArgs& g, int64_t batch) {
-    constexpr size_t lds = 2 * sizeof(float) *
+    constexpr size_t lds = KT * 2 * sizeof(float) *
         (DIRECT ? DirectTile<A_KC, Cfg::BM>::floats + DirectTile<B_KC, Cfg::BN>::floats
                 : TileShape<A_KC, Cfg::BM>::floats + TileShape<B_KC, Cfg::BN>::floats);
     static bool attr_set = false;
     if (!attr_set) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT>),
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT, KT>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                            "hipFuncSetAttribute");
         if (rc) return rc;
         attr_set = true;
     }
     dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)(g.k_splits > 1 ? g.k_splits : 1));
-    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT>), grid, dim3(Cfg::NT), lds, stream(), g);
+    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT, KT>), grid, dim3(Cfg::NT), lds, stream(), g);
     return BH_LAUNCH_CHECK("gemm_mfma_kernel");
 }
 
@@ -896,9 +958,19 @@ static int launch_mfma_layout2(const GemmArgs& g, int64_t batch, bool a_kc, bool
     return launch_mfma<Cfg, false, false, DIRECT>(g, batch);
 }
 
+// the big tile with two k-tiles per barrier (direct loads, contraction a multiple of 32, no split)
+static int launch_mfma_big_pairs(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc);
+
 template <typename Cfg>
 static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc, bool direct) {
     return direct ? launch_mfma_layout2<Cfg, true>(g, batch, a_kc, b_kc) : launch_mfma_layout2<Cfg, false>(g, batch, a_kc, b_kc);
+}
+
+static int launch_mfma_big_pairs(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc) {
+    if (a_kc && b_kc) return launch_mfma<CfgBig, true, true, true, 2>(g, batch);
+    if (a_kc && !b_kc) return launch_mfma<CfgBig, true, false, true, 2>(g, batch);
+    if (!a_kc && b_kc) return launch_mfma<CfgBig, false, true, true, 2>(g, batch);
+    return launch_mfma<CfgBig, false, false, true, 2>(g, batch);
 }
 
 template <bool A_KFAST, bool B_KFAST, int KCH>
@@ -936,6 +1008,7 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
     return BH_LAUNCH_CHECK("splitk_fold_kernel");
 }
 
+static int g_pairs = 1;           // test hook: 0 = the big tile keeps one k-tile per barrier
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
 static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, 6 = tiny, -1 = heuristic
 
@@ -953,7 +1026,8 @@ int bh_gemm_force_config(int cfg) {
 
 // test/benchmark hook: 0 stages operand tiles through registers even where the direct-to-LDS loader applies
 int bh_gemm_force_direct(int mode) {
-    g_force_direct = mode;
+    g_pairs = !(mode & 2);       // bit 1 set: one k-tile per barrier also for the big tile
+    g_force_direct = mode < 0 ? -1 : (mode & 1);
     return BH_OK;
 }
 
@@ -1152,7 +1226,10 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4);
     int rc;
     switch (cfg) {
-        case 2: rc = launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct); break;
+        case 2:
+            if (direct && g_pairs && g.k_splits == 1 && k % (2 * kBK) == 0) rc = launch_mfma_big_pairs(run, batch, a_kc, b_kc);
+            else rc = launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct);
+            break;
         case 3: rc = launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc, direct); break;
         case 4: rc = launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc, direct); break;
         default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc, direct); break;

@@ -366,6 +366,18 @@ def test_gemm_direct_to_lds_edges_epilogues_and_split_k(hip, rng, force, ta, tb)
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("k", [32, 64, 96, 160, 1024])
+def test_gemm_big_tile_with_one_or_two_k_tiles_per_barrier(hip, rng, ta, tb, k):
+    """The 256x256 tile keeps two k-tiles per LDS stage when the contraction is a multiple of 32 (mode 1) and one
+    otherwise or on request (mode 3).  Both walk k in the same order, so the results are the same bits."""
+    state = rng.bit_generator.state
+    one, _ = gemm_case(hip, rng, ta, tb, 520, 300, k, force=2, direct=3, accumulate=True, bias=True)
+    rng.bit_generator.state = state
+    two, _ = gemm_case(hip, rng, ta, tb, 520, 300, k, force=2, direct=1, accumulate=True, bias=True)
+    assert np.array_equal(one, two)
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (33, 17, 5), (64, 64, 128), (65, 63, 129), (37, 130, 225), (200, 70, 1000),
                                    (256, 512, 64)])
 def test_gemm_small_problem_kernel(hip, rng, ta, tb, m, n, k):

@@ -54,16 +54,17 @@ struct boat_autodiff_context_t {
 /* The reference hangs its tape on a graph object (the sources under src/graph) and lets callers hand one to a context
  * (tests/unit/test_gradient_check.c:341-348).  The tape here needs none; the handle exists so that such callers link
  * and run: it can be created, attached, fetched back and freed, nothing more. */
-struct boat_graph_t {
-    boat_device_t device;
-};
 boat_graph_t* boat_graph_create_with_device(boat_device_t device) {
     boat_graph_t* g = (boat_graph_t*)calloc(1, sizeof(*g));
     if (g) g->device = device;
     return g;
 }
 boat_graph_t* boat_graph_create(void) { return boat_graph_create_with_device(BOAT_DEVICE_CPU); }
-void boat_graph_free(boat_graph_t* graph) { free(graph); }
+void boat_graph_free(boat_graph_t* graph) {
+    if (!graph) return;
+    free(graph->nodes);
+    free(graph);
+}
 void boat_autodiff_context_set_graph(boat_autodiff_context_t* context, const boat_graph_t* graph) {
     if (context) context->graph = graph;
 }

@@ -32,6 +32,19 @@ struct boat_tensor_t {
     bool is_view;
 };
 
+/* What exists of the reference's graph objects (include/boat/graph.h): a handle a context can carry, and the chain of
+ * a model's layers seen as nodes (one per layer, in order, joined by count - 1 edges), which is all the model container
+ * ever puts into its graph (src/model/model.c:434-455). */
+struct boat_node_t {
+    void* data;
+    boat_node_type_t type;
+};
+struct boat_graph_t {
+    boat_device_t device;
+    struct boat_node_t* nodes;
+    size_t node_count, node_capacity;
+};
+
 /* Coherent-pointer mode (boat_hip_set_coherent_pointers): copies every tensor whose host pointer the caller holds and
  * that this call wrote on the device back to the host.  Public functions that write tensors which existed before
  * the call end with it; a no-op in the default mode. */

@@ -14,9 +14,32 @@
 struct boat_model_t {
     boat_layer_t** layers;
     size_t layer_count, layer_capacity;
+    boat_graph_t* graph;   /* the layers as a chain of nodes, for callers that look at boat_model_graph() */
 };
 
-boat_model_t* boat_model_create(void) { return (boat_model_t*)calloc(1, sizeof(boat_model_t)); }
+boat_model_t* boat_model_create(void) {
+    boat_model_t* model = (boat_model_t*)calloc(1, sizeof(boat_model_t));
+    if (model) model->graph = boat_graph_create();
+    return model;
+}
+boat_graph_t* boat_model_graph(const boat_model_t* model) { return model ? model->graph : NULL; }
+size_t boat_graph_node_count(const boat_graph_t* graph) { return graph ? graph->node_count : 0; }
+size_t boat_graph_edge_count(const boat_graph_t* graph) { return graph && graph->node_count > 1 ? graph->node_count - 1 : 0; }
+boat_node_t* boat_graph_get_node_at_index(const boat_graph_t* graph, size_t index) {
+    return graph && index < graph->node_count ? &graph->nodes[index] : NULL;
+}
+void* boat_node_data(const boat_node_t* node) { return node ? node->data : NULL; }
+boat_node_type_t boat_node_type(const boat_node_t* node) { return node ? node->type : BOAT_NODE_TYPE_VARIABLE; }
+const char* boat_node_type_name(boat_node_type_t type) {   /* src/graph/node.c:289-298 */
+    switch (type) {
+        case BOAT_NODE_TYPE_VARIABLE: return "VARIABLE";
+        case BOAT_NODE_TYPE_OPERATION: return "OPERATION";
+        case BOAT_NODE_TYPE_CONSTANT: return "CONSTANT";
+        case BOAT_NODE_TYPE_PLACEHOLDER: return "PLACEHOLDER";
+        case BOAT_NODE_TYPE_OUTPUT: return "OUTPUT";
+        default: return "UNKNOWN";
+    }
+}
 boat_sequential_model_t* boat_sequential_create(void) { return boat_model_create(); }
 
 void boat_model_free(boat_model_t* model) {
@@ -26,6 +49,7 @@ void boat_model_free(boat_model_t* model) {
         if (l && l->ops && l->ops->free) l->ops->free(l);
     }
     free(model->layers);
+    boat_graph_free(model->graph);
     free(model);
 }
 
@@ -42,6 +66,19 @@ void boat_model_add_layer(boat_model_t* model, boat_layer_t* layer) {
         model->layer_capacity = cap;
     }
     model->layers[model->layer_count++] = layer;
+    boat_graph_t* g = model->graph;
+    if (g) {   /* model.c:434-455: one operation node per layer, linked to the one before */
+        if (g->node_count == g->node_capacity) {
+            const size_t cap = g->node_capacity ? 2 * g->node_capacity : 8;
+            struct boat_node_t* grown = (struct boat_node_t*)realloc(g->nodes, cap * sizeof(*grown));
+            if (!grown) return;
+            g->nodes = grown;
+            g->node_capacity = cap;
+        }
+        g->nodes[g->node_count].data = layer;
+        g->nodes[g->node_count].type = BOAT_NODE_TYPE_OPERATION;
+        g->node_count++;
+    }
 }
 void boat_sequential_add(boat_sequential_model_t* model, boat_layer_t* layer) { boat_model_add_layer(model, layer); }
 size_t boat_model_layer_count(const boat_model_t* model) { return model ? model->layer_count : 0; }

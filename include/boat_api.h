@@ -169,6 +169,18 @@ BOAT_API boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims,
 /* include/boat/graph.h:18,41-43 and autodiff.h:87-88: an opaque handle that a context can carry for its caller.  The
  * graph IR itself (nodes, edges, traversal) is outside the training path and is not provided. */
 typedef struct boat_graph_t boat_graph_t;
+typedef struct boat_node_t boat_node_t;
+typedef enum {   /* graph.h:23-29 */
+    BOAT_NODE_TYPE_VARIABLE, BOAT_NODE_TYPE_OPERATION, BOAT_NODE_TYPE_CONSTANT, BOAT_NODE_TYPE_PLACEHOLDER, BOAT_NODE_TYPE_OUTPUT
+} boat_node_type_t;
+BOAT_API const char* boat_node_type_name(boat_node_type_t type);
+/* read-only view of a model's layers as the chain the reference's model container records (graph.h:52-53,72-75,
+ * model.h:42; src/model/model.c:434-455): node i carries layer i, consecutive nodes are joined by an edge */
+BOAT_API size_t boat_graph_node_count(const boat_graph_t* graph);
+BOAT_API size_t boat_graph_edge_count(const boat_graph_t* graph);
+BOAT_API boat_node_t* boat_graph_get_node_at_index(const boat_graph_t* graph, size_t index);
+BOAT_API void* boat_node_data(const boat_node_t* node);
+BOAT_API boat_node_type_t boat_node_type(const boat_node_t* node);
 BOAT_API boat_graph_t* boat_graph_create(void);
 BOAT_API boat_graph_t* boat_graph_create_with_device(boat_device_t device);
 BOAT_API void boat_graph_free(boat_graph_t* graph);
@@ -362,6 +374,7 @@ BOAT_API boat_model_t* boat_model_create(void);
 BOAT_API void boat_model_free(boat_model_t* model);
 BOAT_API void boat_model_add_layer(boat_model_t* model, boat_layer_t* layer);
 BOAT_API size_t boat_model_layer_count(const boat_model_t* model);
+BOAT_API boat_graph_t* boat_model_graph(const boat_model_t* model);   /* model.h:42; the chain view declared with the tape's contexts above */
 BOAT_API boat_tensor_t* boat_model_forward(const boat_model_t* model, const boat_tensor_t* input);
 BOAT_API boat_tensor_t* boat_model_backward(const boat_model_t* model, const boat_tensor_t* grad_output);  /* stub in the reference (model.c:354-359) */
 BOAT_API void boat_model_update(const boat_model_t* model, float learning_rate);                          /* stub in the reference (model.c:361-365) */

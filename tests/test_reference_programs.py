@@ -36,6 +36,7 @@ PASSING = {   # program -> a line of its own success report
     "test_tensor": "Tensor tests passed!",
     "test_basic": "All tests passed!",
     "test_memory": "Memory tests passed!",
+    "test_model_graph_integration": "All tests passed!",
     "test_simple": None,
     "test_layer_link": None,
 }

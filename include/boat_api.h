@@ -84,6 +84,23 @@ BOAT_API void boat_memory_set(void* dest, int value, size_t size, boat_device_t 
 BOAT_API boat_memory_stats_t boat_memory_get_stats(void);
 BOAT_API void boat_memory_reset_stats(void);
 BOAT_API void boat_memory_print_stats(FILE* stream);
+/* include/boat/memory.h:58-77: host-side pool of equal blocks and bump arena (no GPU involvement) */
+typedef struct boat_memory_pool_t boat_memory_pool_t;
+BOAT_API boat_memory_pool_t* boat_memory_pool_create(size_t block_size, size_t initial_blocks);
+BOAT_API void boat_memory_pool_free(boat_memory_pool_t* pool);
+BOAT_API void* boat_memory_pool_alloc(boat_memory_pool_t* pool, size_t size);
+BOAT_API void boat_memory_pool_free_block(boat_memory_pool_t* pool, void* block);
+BOAT_API void boat_memory_pool_clear(boat_memory_pool_t* pool);
+BOAT_API size_t boat_memory_pool_allocated_blocks(const boat_memory_pool_t* pool);
+BOAT_API size_t boat_memory_pool_free_blocks(const boat_memory_pool_t* pool);
+BOAT_API size_t boat_memory_pool_total_memory(const boat_memory_pool_t* pool);
+typedef struct boat_memory_arena_t boat_memory_arena_t;
+BOAT_API boat_memory_arena_t* boat_memory_arena_create(size_t initial_size);
+BOAT_API void boat_memory_arena_free(boat_memory_arena_t* arena);
+BOAT_API void* boat_memory_arena_alloc(boat_memory_arena_t* arena, size_t size);
+BOAT_API void boat_memory_arena_reset(boat_memory_arena_t* arena);
+BOAT_API size_t boat_memory_arena_used(const boat_memory_arena_t* arena);
+BOAT_API size_t boat_memory_arena_capacity(const boat_memory_arena_t* arena);
 
 /* ---- include/boat.h:64-94 (error reporting; declared there, mostly undefined in the reference) ---- */
 typedef enum {

@@ -72,6 +72,20 @@ _SIGS = {
     "boat_memory_allocate": (P, [C.c_size_t, C.c_int, C.c_char_p, C.c_int]), "boat_memory_free": (None, [P]),
     "boat_memory_allocate_device": (P, [C.c_size_t, C.c_int, C.c_char_p, C.c_int]), "boat_memory_free_device": (None, [P, C.c_int]),
     "boat_memory_copy": (None, [P, P, C.c_size_t, C.c_int, C.c_int]),
+    "boat_memory_reallocate": (P, [P, C.c_size_t, C.c_int, C.c_char_p, C.c_int]),
+    "boat_memory_pool_create": (P, [C.c_size_t, C.c_size_t]), "boat_memory_pool_free": (None, [P]),
+    "boat_memory_pool_alloc": (P, [P, C.c_size_t]), "boat_memory_pool_free_block": (None, [P, P]),
+    "boat_memory_pool_clear": (None, [P]), "boat_memory_pool_allocated_blocks": (C.c_size_t, [P]),
+    "boat_memory_pool_free_blocks": (C.c_size_t, [P]), "boat_memory_pool_total_memory": (C.c_size_t, [P]),
+    "boat_memory_arena_create": (P, [C.c_size_t]), "boat_memory_arena_free": (None, [P]),
+    "boat_memory_arena_alloc": (P, [P, C.c_size_t]), "boat_memory_arena_reset": (None, [P]),
+    "boat_memory_arena_used": (C.c_size_t, [P]), "boat_memory_arena_capacity": (C.c_size_t, [P]),
+    # graph handle and the model's chain view
+    "boat_graph_create": (P, []), "boat_graph_create_with_device": (P, [C.c_int]), "boat_graph_free": (None, [P]),
+    "boat_autodiff_context_set_graph": (None, [P, P]), "boat_autodiff_context_get_graph": (P, [P]),
+    "boat_model_graph": (P, [P]), "boat_graph_node_count": (C.c_size_t, [P]), "boat_graph_edge_count": (C.c_size_t, [P]),
+    "boat_graph_get_node_at_index": (P, [P, C.c_size_t]), "boat_node_data": (P, [P]), "boat_node_type": (C.c_int, [P]),
+    "boat_node_type_name": (C.c_char_p, [C.c_int]),
     "boat_memory_set": (None, [P, C.c_int, C.c_size_t, C.c_int]), "boat_memory_reset_stats": (None, []),
     "boat_error_string": (C.c_char_p, [C.c_int]), "boat_get_last_error": (C.c_int, []),
     "boat_get_last_error_message": (C.c_char_p, []),

@@ -1161,3 +1161,49 @@ def write_mnist_example_files(folder, train_images, train_labels, test_images, t
                       ("test_images_small.bin", np.asarray(test_images, np.float32)), ("test_labels_small.bin", np.asarray(test_labels, np.uint8))):
         with open(data / name, "wb") as f:
             f.write(struct.pack("<I", arr.ndim) + struct.pack("<%dI" % arr.ndim, *arr.shape) + arr.tobytes())
+
+
+def host_allocator_facts(api):
+    """Pool, arena and reallocate of the memory header (src/core/memory.c:85-120,283-520) and the model's chain view."""
+    out = {}
+    pool = api.boat_memory_pool_create(1024, 4)
+    blocks = [api.boat_memory_pool_alloc(pool, n) for n in (512, 768, 1024)]
+    out["pool_three_taken"] = (int(api.boat_memory_pool_allocated_blocks(pool)), int(api.boat_memory_pool_free_blocks(pool)))
+    out["pool_total_memory"] = int(api.boat_memory_pool_total_memory(pool))
+    out["pool_refuses_larger_than_a_block"] = not api.boat_memory_pool_alloc(pool, 1025)
+    last = api.boat_memory_pool_alloc(pool, 1)
+    out["pool_refuses_when_empty"] = bool(last) and not api.boat_memory_pool_alloc(pool, 1)
+    api.boat_memory_pool_free_block(pool, blocks[1])
+    api.boat_memory_pool_free_block(pool, blocks[1])            # a second time: ignored
+    out["pool_after_one_back"] = (int(api.boat_memory_pool_allocated_blocks(pool)), int(api.boat_memory_pool_free_blocks(pool)))
+    api.boat_memory_pool_clear(pool)
+    out["pool_after_clear"] = (int(api.boat_memory_pool_allocated_blocks(pool)), int(api.boat_memory_pool_free_blocks(pool)))
+    api.boat_memory_pool_free(pool)
+    out["pool_of_nothing_refused"] = not api.boat_memory_pool_create(0, 4) and not api.boat_memory_pool_create(16, 0)
+    arena = api.boat_memory_arena_create(4096)
+    a = api.boat_memory_arena_alloc(arena, 10)
+    b = api.boat_memory_arena_alloc(arena, 1)
+    out["arena_rounds_to_eight"] = (b - a, int(api.boat_memory_arena_used(arena)))
+    out["arena_refuses_zero"] = not api.boat_memory_arena_alloc(arena, 0)
+    api.boat_memory_arena_alloc(arena, 9000)                    # does not fit: the capacity doubles until it does
+    out["arena_grows"] = (int(api.boat_memory_arena_used(arena)), int(api.boat_memory_arena_capacity(arena)))
+    api.boat_memory_arena_reset(arena)
+    out["arena_after_reset"] = (int(api.boat_memory_arena_used(arena)), int(api.boat_memory_arena_capacity(arena)))
+    api.boat_memory_arena_free(arena)
+    p = api.boat_memory_allocate(16, 0, b"boat_cases.py", 1)
+    C.memmove(p, b"0123456789abcdef", 16)
+    q = api.boat_memory_reallocate(p, 64, 0, b"boat_cases.py", 2)
+    out["reallocate_keeps_contents"] = C.string_at(q, 16)
+    out["reallocate_to_zero_frees"] = not api.boat_memory_reallocate(q, 0, 0, b"boat_cases.py", 3)
+    r = api.boat_memory_reallocate(None, 8, 0, b"boat_cases.py", 4)
+    out["reallocate_of_null_allocates"] = bool(r)
+    api.boat_memory_free(r)
+    graph = api.boat_graph_create_with_device(0)
+    ctx = api.boat_autodiff_context_create()
+    api.boat_autodiff_context_set_graph(ctx, graph)
+    out["context_carries_the_graph"] = api.boat_autodiff_context_get_graph(ctx) == graph
+    out["fresh_graph_is_empty"] = (int(api.boat_graph_node_count(graph)), int(api.boat_graph_edge_count(graph)))
+    api.boat_autodiff_context_free(ctx)
+    api.boat_graph_free(graph)
+    out["node_type_names"] = [api.boat_node_type_name(t).decode() for t in range(6)]
+    return out

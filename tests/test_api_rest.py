@@ -462,3 +462,22 @@ def test_gpu_slices_feed_the_layers(boat, oracle):
     assert np.array_equal(boat.numpy(samples), data)
     boat.boat_tensor_unref(samples)
     boat.boat_dense_layer_free(layer)
+
+
+HOST_ALLOCATOR_FACTS = {
+    "pool_three_taken": (3, 1), "pool_total_memory": 4192, "pool_refuses_larger_than_a_block": True,
+    "pool_refuses_when_empty": True, "pool_after_one_back": (3, 1), "pool_after_clear": (0, 4), "pool_of_nothing_refused": True,
+    "arena_rounds_to_eight": (16, 24), "arena_refuses_zero": True, "arena_grows": (9024, 16384), "arena_after_reset": (0, 16384),
+    "reallocate_keeps_contents": b"0123456789abcdef", "reallocate_to_zero_frees": True, "reallocate_of_null_allocates": True,
+    "context_carries_the_graph": True, "fresh_graph_is_empty": (0, 0),
+    "node_type_names": ["VARIABLE", "OPERATION", "CONSTANT", "PLACEHOLDER", "OUTPUT", "UNKNOWN"],
+}
+
+
+def test_reference_host_allocator_facts(ref):
+    assert bc.host_allocator_facts(ref) == HOST_ALLOCATOR_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_host_allocator_facts(boat):
+    assert bc.host_allocator_facts(boat) == HOST_ALLOCATOR_FACTS

@@ -1,11 +1,11 @@
 """The reference's OWN test programs (and its optimizer benchmark), linked against libboat_amd.so instead of libboat.
 
-`make -C oracle reftests` compiles tests/unit/*.c, tests/*.c and benchmarks/linear_regression.c of the reference from where they lie, with the
+`make -C oracle reftests` compiles tests/unit/*.c, tests/*.c, benchmarks/*.c and three examples of the reference from where they lie, with the
 reference's headers, and links them with this repository's library (outputs in oracle/_ref/reftests, built where the
 reference tree exists).  They run here unchanged, in coherent-pointer mode: these programs keep the float* of
 boat_tensor_data() across calls (finite differences write weights through it, the optimizer tests read the updated
 parameter through it).  Programs that build graphs of their own (test_graph_phase2/3) or need a Windows header
-(test_export, benchmarks/attention_performance) are not built.
+(test_export) are not built.
 
 test_schedulers aborts at its line 56 on the compiled reference too (a Release build of the reference compiles its
 asserts out): the scheduler here reproduces the reference's learning rates bit for bit (tests/test_schedulers.py), so
@@ -128,6 +128,14 @@ def test_mnist_example_of_the_reference_trains_as_on_the_reference(tmp_path, coh
     assert proc.returncode == 0, proc.stderr[-1000:]
     lines = [re.sub(r"time=[0-9.]+s, ", "", line) for line in proc.stdout.splitlines() if re.match(r"Epoch \d|Test accuracy", line)]
     assert lines == [str(line) for line in g["reference_lines"]] and len(lines) == 6
+
+
+def test_attention_benchmark_of_the_reference_runs(tmp_path):
+    """benchmarks/attention_performance.c (B4 S16 H64, 8 heads, causal; 50 forward and backward passes through
+    boat_attention_forward / boat_attention_backward): runs to its report on this library."""
+    proc = run("attention_performance", tmp_path)
+    assert proc.returncode == 0, proc.stderr[-1000:]
+    assert "Forward pass:" in proc.stdout and "Backward pass:" in proc.stdout and "Benchmark completed." in proc.stdout
 
 
 def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):

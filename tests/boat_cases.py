@@ -1207,3 +1207,36 @@ def host_allocator_facts(api):
     api.boat_graph_free(graph)
     out["node_type_names"] = [api.boat_node_type_name(t).decode() for t in range(6)]
     return out
+
+
+def loss_and_scheduler_facts(api):
+    """Argument checks of the loss objects (src/loss/*.c) and the schedulers (src/schedulers/*.c)."""
+    out = {}
+    rng = np.random.default_rng(11)
+    pred, target = api.tensor(rng.random((4, 5)).astype(np.float32)), api.tensor(rng.random((4, 5)).astype(np.float32))
+    other = api.tensor(rng.random((4, 6)).astype(np.float32))
+    for kind, make in (("mse", api.boat_mse_loss_create), ("ce", api.boat_cross_entropy_loss_create), ("huber", lambda: api.boat_huber_loss_create(1.0))):
+        loss = make()
+        out[kind + "_created"] = bool(loss)
+        v = float(api.boat_loss_compute(loss, pred, target))
+        out[kind + "_finite_and_positive"] = bool(np.isfinite(v) and v > 0)
+        out[kind + "_shape_mismatch"] = round(float(api.boat_loss_compute(loss, pred, other)), 6)
+        out[kind + "_null_prediction"] = round(float(api.boat_loss_compute(loss, None, target)), 6)
+        api.boat_loss_free(loss)
+    out["loss_compute_on_null_loss"] = round(float(api.boat_loss_compute(None, pred, target)), 6)
+    out["step_bad"] = [not api.boat_step_lr_scheduler_create(0.0, 10, 0.5), not api.boat_step_lr_scheduler_create(0.1, 0, 0.5),
+                       not api.boat_step_lr_scheduler_create(0.1, 10, 0.0), not api.boat_step_lr_scheduler_create(0.1, 10, 1.5)]
+    out["cosine_bad"] = [not api.boat_cosine_annealing_scheduler_create(0.0, 10, 0.0), not api.boat_cosine_annealing_scheduler_create(0.1, 0, 0.0),
+                         not api.boat_cosine_annealing_scheduler_create(0.1, 10, -1.0), not api.boat_cosine_annealing_scheduler_create(0.1, 10, 0.2)]
+    out["null_scheduler_lr"] = (round(float(api.boat_scheduler_get_last_lr(None)), 6), round(float(api.boat_scheduler_get_next_lr(None)), 6))
+    sch = api.boat_step_lr_scheduler_create(0.1, 2, 0.5)
+    opt = api.boat_adam_optimizer_create(0.3, 0.9, 0.999, 1e-8)
+    api.boat_scheduler_update_optimizer(sch, opt)
+    out["update_optimizer_sets_last_lr"] = round(float(api.boat_optimizer_get_learning_rate(opt)), 6)
+    api.boat_scheduler_update_optimizer(None, opt)
+    api.boat_scheduler_update_optimizer(sch, None)
+    api.boat_scheduler_free(sch)
+    api.boat_optimizer_free(opt)
+    for t in (pred, target, other):
+        api.boat_tensor_unref(t)
+    return out

@@ -481,3 +481,24 @@ def test_reference_host_allocator_facts(ref):
 @pytest.mark.gpu
 def test_gpu_host_allocator_facts(boat):
     assert bc.host_allocator_facts(boat) == HOST_ALLOCATOR_FACTS
+
+
+LOSS_AND_SCHEDULER_FACTS = {
+    "mse_created": True, "mse_finite_and_positive": True, "mse_shape_mismatch": 0.0, "mse_null_prediction": 0.0,
+    "ce_created": True, "ce_finite_and_positive": True, "ce_shape_mismatch": 0.0, "ce_null_prediction": 0.0,
+    "huber_created": True, "huber_finite_and_positive": True, "huber_shape_mismatch": 0.0, "huber_null_prediction": 0.0,
+    "loss_compute_on_null_loss": 0.0,
+    "step_bad": [True, True, True, False],          # a decay factor above 1 is accepted (step_lr.c checks gamma <= 0 only)
+    "cosine_bad": [True, True, True, True], "null_scheduler_lr": (0.0, 0.0), "update_optimizer_sets_last_lr": 0.1,
+}
+
+
+def test_reference_loss_and_scheduler_facts(ref):
+    assert bc.loss_and_scheduler_facts(ref) == LOSS_AND_SCHEDULER_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_loss_and_scheduler_facts(boat):
+    got = bc.loss_and_scheduler_facts(boat)
+    diff = {k: (got.get(k), v) for k, v in LOSS_AND_SCHEDULER_FACTS.items() if got.get(k) != v}
+    assert not diff and set(got) == set(LOSS_AND_SCHEDULER_FACTS), diff

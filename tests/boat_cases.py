@@ -1240,3 +1240,37 @@ def loss_and_scheduler_facts(api):
     for t in (pred, target, other):
         api.boat_tensor_unref(t)
     return out
+
+
+def attention_facts(api):
+    """What boat_attention_forward / backward accept and ignore (src/layers/attention.c:247-466,468-560,1012-1025,1061-1062)."""
+    from boat_amd.capi import AttentionConfig
+    out = {}
+    rng = np.random.default_rng(12)
+
+    def T(*shape):
+        return api.tensor(rng.standard_normal(shape).astype(np.float32))
+
+    att = api.boat_attention_create(C.byref(AttentionConfig(8, 2, 0, 0.5, True, True, False, 10000.0)))   # dropout 0.5, causal
+    x, mask = T(2, 3, 8), api.tensor(np.zeros((2, 3, 3), np.float32))
+    with scratch_cwd():
+        out["backward_before_forward"] = bool(api.boat_attention_backward(att, x, None, None, None))
+        y1 = api.boat_attention_forward(att, x, x, x, None)
+        y2 = api.boat_attention_forward(att, x, x, x, mask)
+        y3 = api.boat_attention_forward(att, x, x, x, None)
+        out["mask_is_ignored"] = bool(np.array_equal(api.numpy(y1), api.numpy(y2)))
+        out["dropout_is_ignored"] = bool(np.array_equal(api.numpy(y1), api.numpy(y3)))
+        out["forward_null_query"] = not api.boat_attention_forward(att, None, x, x, None)
+        wrong = T(2, 3, 6)
+        out["forward_wrong_hidden"] = not api.boat_attention_forward(att, wrong, wrong, wrong, None)
+        flat = T(6, 8)
+        y2d = api.boat_attention_forward(att, flat, flat, flat, None)
+        out["forward_2d_input"] = None if not y2d else api.shape(y2d)
+        api.boat_attention_forward(att, x, x, x, None)
+        dq, dk, dv = C.c_void_p(), C.c_void_p(), C.c_void_p()
+        ok = api.boat_attention_backward(att, x, C.byref(dq), C.byref(dk), C.byref(dv))
+        out["backward_ok"] = bool(ok)
+        out["backward_grad_shapes"] = tuple(api.shape(g.value) for g in (dq, dk, dv))
+        out["grads_exist_after_backward"] = bool(api.boat_attention_get_grad_weight_q(att)) and bool(api.boat_attention_get_grad_bias_o(att))
+        out["backward_wrong_shape"] = bool(api.boat_attention_backward(att, wrong, None, None, None))
+    return out

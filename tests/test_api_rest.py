@@ -502,3 +502,22 @@ def test_gpu_loss_and_scheduler_facts(boat):
     got = bc.loss_and_scheduler_facts(boat)
     diff = {k: (got.get(k), v) for k, v in LOSS_AND_SCHEDULER_FACTS.items() if got.get(k) != v}
     assert not diff and set(got) == set(LOSS_AND_SCHEDULER_FACTS), diff
+
+
+ATTENTION_FACTS = {
+    "backward_before_forward": False, "mask_is_ignored": True, "dropout_is_ignored": True,       # attention.c:1022-1025,1061-1062
+    "forward_null_query": True, "forward_wrong_hidden": True, "forward_2d_input": None,
+    "backward_ok": True, "backward_grad_shapes": ((2, 3, 8), (2, 3, 8), (2, 3, 8)), "grads_exist_after_backward": True,
+    "backward_wrong_shape": False,
+}
+
+
+def test_reference_attention_facts(ref):
+    assert bc.attention_facts(ref) == ATTENTION_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_attention_facts(boat):
+    got = bc.attention_facts(boat)
+    diff = {k: (got.get(k), v) for k, v in ATTENTION_FACTS.items() if got.get(k) != v}
+    assert not diff and set(got) == set(ATTENTION_FACTS), diff

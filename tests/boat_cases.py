@@ -1274,3 +1274,41 @@ def attention_facts(api):
         out["grads_exist_after_backward"] = bool(api.boat_attention_get_grad_weight_q(att)) and bool(api.boat_attention_get_grad_bias_o(att))
         out["backward_wrong_shape"] = bool(api.boat_attention_backward(att, wrong, None, None, None))
     return out
+
+
+def conv_pool_facts(api):
+    """Argument checks of the convolution, pooling and flatten hooks (src/layers/conv.c:240-330,475-537,
+    src/layers/pool.c:30-62,173-218, src/layers/flatten.c)."""
+    out = {}
+    rng = np.random.default_rng(13)
+
+    def T(*shape):
+        return api.tensor(rng.standard_normal(shape).astype(np.float32))
+
+    def shape_of(t):
+        if not t:
+            return None
+        s = api.shape(t)
+        api.boat_tensor_unref(t)
+        return s
+
+    conv = api.boat_conv_layer_create(2, 3, 3, 1, 0)
+    x, small, dy_bad = T(2, 2, 6, 6), T(2, 2, 2, 2), T(2, 3, 5, 5)
+    out["conv_backward_before_forward"] = shape_of(api.boat_conv_layer_backward(conv, dy_bad))
+    out["conv_forward_no_padding"] = shape_of(api.boat_conv_layer_forward(conv, x))
+    out["conv_backward_wrong_shape"] = shape_of(api.boat_conv_layer_backward(conv, dy_bad))
+    out["conv_input_smaller_than_kernel"] = shape_of(api.boat_conv_layer_forward(conv, small))
+    out["conv_null_input"] = shape_of(api.boat_conv_layer_forward(conv, None))
+    strided = api.boat_conv_layer_create(2, 3, 3, 2, 1)
+    out["conv_stride_two_pad_one"] = shape_of(api.boat_conv_layer_forward(strided, x))
+    pool = api.boat_pool_layer_create(2, 2, 0)
+    out["pool_backward_before_forward"] = shape_of(api.boat_pool_layer_backward(pool, x))
+    out["pool_forward_odd_side"] = shape_of(api.boat_pool_layer_forward(pool, T(1, 1, 5, 5)))
+    out["pool_backward_wrong_shape"] = shape_of(api.boat_pool_layer_backward(pool, T(1, 1, 3, 3)))
+    out["pool_backward"] = shape_of(api.boat_pool_layer_backward(pool, T(1, 1, 2, 2)))
+    flat = api.boat_flatten_layer_create()
+    out["flatten_backward_before_forward"] = shape_of(api.boat_flatten_layer_backward(flat, x))
+    out["flatten_2d_input"] = shape_of(api.boat_flatten_layer_forward(flat, T(3, 4)))
+    out["flatten_4d_input"] = shape_of(api.boat_flatten_layer_forward(flat, x))
+    out["flatten_backward"] = shape_of(api.boat_flatten_layer_backward(flat, T(2, 72)))
+    return out

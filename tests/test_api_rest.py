@@ -521,3 +521,23 @@ def test_gpu_attention_facts(boat):
     got = bc.attention_facts(boat)
     diff = {k: (got.get(k), v) for k, v in ATTENTION_FACTS.items() if got.get(k) != v}
     assert not diff and set(got) == set(ATTENTION_FACTS), diff
+
+
+CONV_POOL_FACTS = {
+    "conv_backward_before_forward": None, "conv_forward_no_padding": (2, 3, 4, 4), "conv_backward_wrong_shape": None,
+    "conv_input_smaller_than_kernel": None, "conv_null_input": None, "conv_stride_two_pad_one": (2, 3, 3, 3),
+    "pool_backward_before_forward": None, "pool_forward_odd_side": (1, 1, 2, 2), "pool_backward_wrong_shape": None,
+    "pool_backward": (1, 1, 5, 5), "flatten_backward_before_forward": None, "flatten_2d_input": (3, 4),
+    "flatten_4d_input": (2, 72), "flatten_backward": (2, 2, 6, 6),
+}
+
+
+def test_reference_conv_pool_facts(ref):
+    assert bc.conv_pool_facts(ref) == CONV_POOL_FACTS
+
+
+@pytest.mark.gpu
+def test_gpu_conv_pool_facts(boat):
+    got = bc.conv_pool_facts(boat)
+    diff = {k: (got.get(k), v) for k, v in CONV_POOL_FACTS.items() if got.get(k) != v}
+    assert not diff and set(got) == set(CONV_POOL_FACTS), diff

@@ -102,13 +102,13 @@ BOAT_API void boat_memory_arena_reset(boat_memory_arena_t* arena);
 BOAT_API size_t boat_memory_arena_used(const boat_memory_arena_t* arena);
 BOAT_API size_t boat_memory_arena_capacity(const boat_memory_arena_t* arena);
 
-/* ---- include/boat.h:64-94 (error reporting; declared there, mostly undefined in the reference) ---- */
+/* ---- include/boat.h:64-94 (error reporting; src/core/error.c:21-62: a thread-local code and a 256-byte message) ---- */
 typedef enum {
     BOAT_SUCCESS = 0, BOAT_ERROR_INVALID_ARGUMENT, BOAT_ERROR_OUT_OF_MEMORY, BOAT_ERROR_INVALID_OPERATION,
     BOAT_ERROR_DEVICE, BOAT_ERROR_FILE_IO, BOAT_ERROR_FORMAT, BOAT_ERROR_NOT_IMPLEMENTED, BOAT_ERROR_UNKNOWN
 } boat_error_t;
-BOAT_API void boat_init(void);
-BOAT_API void boat_cleanup(void);
+BOAT_API void boat_init(void);      /* declared in include/boat.h, defined nowhere in the reference; here it brings the device up */
+BOAT_API void boat_cleanup(void);   /* likewise; releases the stream and the cached device blocks */
 BOAT_API const char* boat_error_string(boat_error_t error);
 BOAT_API boat_error_t boat_get_last_error(void);
 BOAT_API const char* boat_get_last_error_message(void);

@@ -16,6 +16,7 @@ hipStream_t stream();
 int set_error(int code, const char* fmt, ...);
 int check_hip(hipError_t e, const char* what);
 bool ready();
+int ln_scratch_setup();   // bh_layernorm.hip: resolves the current device's copy of the no-alloc scratch array
 
 #define BH_REQUIRE_INIT()                                   \
     do {                                                    \

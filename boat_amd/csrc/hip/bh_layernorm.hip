@@ -19,6 +19,14 @@ namespace bh {
 
 constexpr int kLnBlock = 256;
 
+// Scratch of bh_layernorm_backward_noalloc: the per-workgroup dgamma/dbeta partials that bh_layernorm_backward
+// takes from bh_malloc.  One copy per GPU, held until the process ends.  Host code never uses the array's name
+// as an address: ln_scratch_setup() asks the runtime for the device address once per device and keeps it.
+constexpr size_t kLnScratchFloats = size_t(4) << 20;   // 16 MiB
+static __device__ __align__(256) float ln_scratch[kLnScratchFloats];
+constexpr int kMaxDevices = 16;
+static float* g_ln_scratch_ptr[kMaxDevices] = {};
+
 __device__ __forceinline__ float4 ld4(const float* p, int64_t i4) { return reinterpret_cast<const float4*>(p)[i4]; }
 __device__ __forceinline__ void st4(float* p, int64_t i4, float4 v) { reinterpret_cast<float4*>(p)[i4] = v; }
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -347,6 +355,21 @@ static LnPlan plan_for(int64_t hidden, const void* p0, const void* p1, const voi
     return p;
 }
 
+// Called by bh_init with the library's device current: resolves that device's copy of ln_scratch.
+int ln_scratch_setup() {
+    int dev = -1;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    if (dev < 0 || dev >= kMaxDevices) return set_error(BH_EDEVICE, "ln_scratch_setup: device index %d out of range", dev);
+    if (g_ln_scratch_ptr[dev]) return BH_OK;
+    float* p = nullptr;
+    rc = check_hip(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(ln_scratch)), "hipGetSymbolAddress(ln_scratch)");
+    if (rc) return rc;
+    if (!p) return set_error(BH_EDEVICE, "ln_scratch_setup: the runtime returned no address for ln_scratch");
+    g_ln_scratch_ptr[dev] = p;
+    return BH_OK;
+}
+
 }  // namespace bh
 
 using namespace bh;
@@ -400,6 +423,43 @@ int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, 
     return BH_LAUNCH_CHECK("bh_layernorm_forward");
 }
 
+// The register-resident path: ln_bwd_kernel writes one dgamma/dbeta partial per workgroup into `partial`
+// (blocks x 2 x hidden floats), fold_rows_kernel sums them.
+static int ln_backward_vector(const LnPlan& plan, size_t shmem, int64_t blocks, float* partial, const float* x,
+                              const float* gamma, const float* dy, const float* mean, const float* rstd, float* dx,
+                              float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
+    const int groups = kLnBlock / plan.tpr;
+    const int64_t iters = ceil_div(rows, blocks * groups);
+    BH_LN_DISPATCH(ln_bwd_kernel, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
+                   (int)hidden, iters);
+    if (dgamma || dbeta)
+        hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
+                           stream(), partial, blocks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
+    return BH_LAUNCH_CHECK("bh_layernorm_backward");
+}
+
+// Dynamic LDS of the vector path (the cross-group fold when a workgroup holds several row groups); the path is
+// not taken when this plus the kernel's static LDS would pass the 64 KiB a launch gets without an opt-in.
+static bool ln_backward_plan(LnPlan& plan, size_t& shmem, const float* x, const float* gamma, const float* dy, float* dx,
+                             int64_t hidden) {
+    plan = plan_for(hidden, x, dy, dx);
+    if (plan.vector && gamma && (reinterpret_cast<uintptr_t>(gamma) & 15)) plan.vector = false;
+    const int groups = plan.vector ? kLnBlock / plan.tpr : 1;
+    shmem = (plan.vector && groups > 1) ? sizeof(float) * (size_t)groups * 2 * (size_t)hidden : 0;
+    if (shmem + 256 > 64 * 1024) {
+        // one row group per workgroup needs no fold through LDS
+        if (plan.vector && (hidden >> 2) >= 256) {
+            plan.tpr = 256;
+            const int64_t need = ceil_div(hidden >> 2, 256);
+            plan.vpt = need <= 4 ? 4 : 8;
+            shmem = 0;
+        } else {
+            plan.vector = false;
+        }
+    }
+    return plan.vector;
+}
+
 int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
                           float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
     BH_REQUIRE_INIT();
@@ -413,27 +473,21 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, c
         return BH_OK;
     }
     BH_CHECK_ARG(x && dy && mean && rstd && dx, "null pointer");
-    LnPlan plan = plan_for(hidden, x, dy, dx);
-    if (plan.vector && gamma && (reinterpret_cast<uintptr_t>(gamma) & 15)) plan.vector = false;
-    const int groups = plan.vector ? kLnBlock / plan.tpr : 1;
-    const size_t shmem = (plan.vector && groups > 1) ? sizeof(float) * (size_t)groups * 2 * (size_t)hidden : 0;
-    if (shmem > 64 * 1024) plan.vector = false;
+    LnPlan plan;
+    size_t shmem;
+    ln_backward_plan(plan, shmem, x, gamma, dy, dx, hidden);
 
     int rc;
     if (plan.vector) {
+        const int groups = kLnBlock / plan.tpr;
         int64_t blocks = ceil_div(rows, groups);
         const int64_t cap = g_ln_bwd_blocks;   // per-block dgamma/dbeta partials cost 2*hidden floats each way
         if (blocks > cap) blocks = cap;
-        const int64_t iters = ceil_div(rows, blocks * groups);
         float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(blocks * 2 * hidden));
         if (!partial) return BH_ENOMEM;
-        BH_LN_DISPATCH(ln_bwd_kernel, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
-                       (int)hidden, iters);
-        if (dgamma || dbeta)
-            hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
-                               stream(), partial, blocks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
+        rc = ln_backward_vector(plan, shmem, blocks, partial, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden,
+                                accumulate);
         bh_free(partial);
-        rc = BH_LAUNCH_CHECK("bh_layernorm_backward");
     } else {
         hipLaunchKernelGGL(ln_bwd_dx_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, dy, mean,
                            rstd, dx, rows, hidden);
@@ -454,6 +508,44 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, c
         }
     }
     return rc;
+}
+
+// bh_layernorm_backward for callers that may not allocate: same kernels, the partials live in ln_scratch.
+// No hipMalloc/hipFree, no bh_malloc; the library must already be initialised (bh_init creates the stream and
+// resolves the scratch address).  Calls on one GPU share the array: they must not overlap.
+int bh_layernorm_backward_noalloc(const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
+                                  float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
+    if (!ready()) return set_error(BH_EINVAL, "bh_layernorm_backward_noalloc: call bh_init() first (this entry point sets nothing up)");
+    int dev = -1;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    float* scratch = (dev >= 0 && dev < kMaxDevices) ? g_ln_scratch_ptr[dev] : nullptr;
+    if (!scratch) return set_error(BH_EDEVICE, "bh_layernorm_backward_noalloc: no scratch address for device %d", dev);
+    BH_CHECK_ARG(rows >= 0 && hidden > 0, "bad shape");
+    if (rows == 0) {
+        if (!accumulate) {
+            if (dgamma) bh_memset_zero(dgamma, sizeof(float) * (size_t)hidden);
+            if (dbeta) bh_memset_zero(dbeta, sizeof(float) * (size_t)hidden);
+        }
+        return BH_OK;
+    }
+    BH_CHECK_ARG(x && dy && mean && rstd && dx, "null pointer");
+    LnPlan plan;
+    size_t shmem;
+    if (hidden > BH_LN_NOALLOC_MAX_HIDDEN || !ln_backward_plan(plan, shmem, x, gamma, dy, dx, hidden))
+        return set_error(BH_EINVAL,
+                         "bh_layernorm_backward_noalloc: hidden=%lld is not supported: it must be a multiple of 4, at most %d, "
+                         "with 16-byte aligned x, dy, dx and gamma (use bh_layernorm_backward)",
+                         (long long)hidden, BH_LN_NOALLOC_MAX_HIDDEN);
+    const int groups = kLnBlock / plan.tpr;
+    int64_t blocks = ceil_div(rows, groups);
+    int64_t cap = g_ln_bwd_blocks;
+    const int64_t fit = (int64_t)(kLnScratchFloats / (size_t)(2 * hidden));   // >= 256 for every supported hidden
+    if (cap > fit) cap = fit;
+    if (blocks > cap) blocks = cap;
+    // every partial the fold reads is written by this call's ln_bwd_kernel first: nothing to clear
+    return ln_backward_vector(plan, shmem, blocks, scratch, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden,
+                              accumulate);
 }
 
 }  // extern "C"

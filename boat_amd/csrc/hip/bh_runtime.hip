@@ -74,6 +74,8 @@ int bh_init(void) {
     g_cus = prop.multiProcessorCount;
     rc = check_hip(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking), "hipStreamCreate");
     if (rc) return rc;
+    rc = ln_scratch_setup();
+    if (rc) return rc;
     g_ready = true;
     return BH_OK;
 }

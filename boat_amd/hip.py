@@ -51,6 +51,7 @@ _SIGS = {
     "bh_softmax_ce_grad": (I, [P, P, P, P, L, L]),
     "bh_layernorm_forward": (I, [P, P, P, P, P, P, L, L, F]),
     "bh_layernorm_backward": (I, [P, P, P, P, P, P, P, P, L, L, I]),
+    "bh_layernorm_backward_noalloc": (I, [P, P, P, P, P, P, P, P, L, L, I]),
     "bh_gemm": (I, [I, I, L, L, L, P, L, P, L, P, L, P, I, L]),
     "bh_gemm_force_config": (I, [I]), "bh_gemm_force_direct": (I, [I]),
     "bh_transpose_last2": (I, [P, P, L, L, L]),

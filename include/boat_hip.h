@@ -118,6 +118,19 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy,
                           float* dx, float* dgamma, float* dbeta,
                           int64_t rows, int64_t hidden, int accumulate);
 
+/* bh_layernorm_backward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels and
+ * the same results as bh_layernorm_backward; the per-workgroup dgamma/dbeta partials live in a 16 MiB device array
+ * that is part of the library image (one copy per GPU, held until the process ends) instead of coming from bh_malloc.
+ * It calls no hipMalloc/hipFree and sets nothing up: bh_init() must have returned BH_OK before.  hidden must be a
+ * multiple of 4 and at most BH_LN_NOALLOC_MAX_HIDDEN, and x, dy, dx, gamma 16-byte aligned; anything else returns
+ * BH_EINVAL with a message.  Every call on a GPU uses that GPU's one array: calls that overlap in time race. */
+#define BH_LN_NOALLOC_MAX_HIDDEN 8192
+int bh_layernorm_backward_noalloc(const float* x, const float* gamma, const float* dy,
+                                  const float* mean, const float* rstd,
+                                  float* dx, float* dgamma, float* dbeta,
+                                  int64_t rows, int64_t hidden, int accumulate);
+
 /* ---- GEMM on fp32 MFMA (src/ops/linear.c:12-170 with the transposes of :238-406 folded in) ----
  * C[M,N] (+)= op(A) . op(B) (+ bias[N]), row-major.
  *   trans_a == 0: A is [M,K] with leading dimension lda;  trans_a != 0: A is stored [K,M]

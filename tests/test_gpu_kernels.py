@@ -269,7 +269,8 @@ def test_fused_softmax_ce_matches_tape_chain(hip, oracle, rng, rows, cols):
 
 # ---------------------------------------------------------------- layernorm
 
-LN_SHAPES = [(1, 4), (7, 64), (10, 48), (33, 768), (64, 1024), (17, 4096), (5, 8192), (6, 50), (3, 9000)]
+LN_SHAPES = [(1, 4), (7, 64), (10, 48), (33, 768), (64, 1024), (17, 4096), (5, 8192), (6, 50), (3, 9000),
+             (40, 2048), (21, 2044), (9, 2040)]
 
 
 @pytest.mark.parametrize("rows,hidden", LN_SHAPES)

@@ -45,6 +45,11 @@ class LayerNormConfig(C.Structure):  # include/boat/layers/norm.h:21-26
                 ("elementwise_affine", C.c_bool), ("use_bias", C.c_bool)]
 
 
+class RmsNormConfig(C.Structure):  # include/boat/layers/norm.h:28-32
+    _fields_ = [("normalized_shape", C.c_size_t), ("eps", C.c_float), ("elementwise_affine", C.c_bool)]
+
+
+FREE_FN = C.CFUNCTYPE(None, C.c_void_p)                     # include/boat/model.h: user-data destructor
 LAMBDA_LR_FN = C.CFUNCTYPE(C.c_float, C.c_int, C.c_float)   # include/boat/schedulers.h:35-36
 
 _SIGS = {
@@ -102,7 +107,16 @@ _SIGS = {
     "boat_relu": (P, [P]),
     "boat_softmax": (P, [P, C.c_int]), "boat_log_softmax": (P, [P, C.c_int]),
     "boat_sum": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_bool]),
+    "boat_mod": (P, [P, P]), "boat_pow_scalar": (P, [P, C.c_double]),
+    "boat_add_scalar_": (None, [P, C.c_double]), "boat_sub_scalar_": (None, [P, C.c_double]),
+    "boat_mul_scalar_": (None, [P, C.c_double]), "boat_div_scalar_": (None, [P, C.c_double]),
+    "boat_inverse": (P, [P]), "boat_selu": (P, [P]),
+    "boat_reset_error": (None, []), "boat_memory_free_safe": (None, [C.POINTER(P)]),
+    "boat_memory_allocate_aligned": (P, [C.c_size_t, C.c_size_t, C.c_int, C.c_char_p, C.c_int]),
+    "boat_memory_free_aligned": (None, [P]),
     # autodiff
+    "boat_var_max": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_bool]),
+    "boat_var_min": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_bool]),
     "boat_variable_create": (P, [P, C.c_bool]),
     "boat_variable_free": (None, [P]),
     "boat_variable_data": (P, [P]),
@@ -177,7 +191,17 @@ _SIGS = {
     "boat_norm_layer_create": (P, [C.c_size_t, C.c_float, C.c_bool]),
     "boat_norm_layer_free": (None, [P]),
     "boat_norm_layer_forward": (P, [P, P]), "boat_norm_layer_backward": (P, [P, P]),
+    # rmsnorm and the stateless forms
+    "boat_rmsnorm_create": (P, [C.POINTER(RmsNormConfig)]), "boat_rmsnorm_free": (None, [P]),
+    "boat_rmsnorm_forward": (P, [P, P]), "boat_rmsnorm_backward": (P, [P, P]), "boat_rmsnorm_update": (None, [P, C.c_float]),
+    "boat_layer_norm": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_float]),
+    "boat_rms_norm": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_float]),
+    "boat_rms_norm_grad": (P, [P, P, P, C.POINTER(C.c_int64), C.c_size_t, C.c_float]),
     # attention
+    "boat_scaled_dot_product_attention": (P, [P, P, P, C.c_float, P, C.c_bool, C.c_float]),
+    "boat_multihead_attention": (P, [P, C.c_size_t, C.c_float, C.c_bool, P]),
+    "boat_rotary_position_encoding": (P, [P, C.c_size_t, C.c_size_t, C.c_float]),
+    "boat_apply_rotary_embedding": (None, [P, P, C.c_size_t, C.c_size_t, C.c_float]),
     "boat_attention_create": (P, [C.POINTER(AttentionConfig)]),
     "boat_attention_free": (None, [P]),
     "boat_attention_forward": (P, [P, P, P, P, P]),
@@ -198,6 +222,9 @@ _SIGS = {
     "boat_model_add_layer": (None, [P, P]), "boat_model_layer_count": (C.c_size_t, [P]),
     "boat_model_forward": (P, [P, P]), "boat_model_backward": (P, [P, P]),
     "boat_model_update": (None, [P, C.c_float]),
+    "boat_model_create_with_graph": (P, [P]), "boat_model_set_graph": (None, [P, P]),
+    "boat_model_get_user_data": (P, [P]), "boat_model_set_user_data": (None, [P, P, FREE_FN]),
+    "boat_model_load": (P, [C.c_char_p]), "boat_model_save": (C.c_bool, [P, C.c_char_p]),
 }
 for _n in "qkvo":
     for _k in ("weight", "bias", "grad_weight", "grad_bias"):
@@ -209,12 +236,14 @@ _EXT_SIGS = {
     "boat_tensor_to_device": (P, [P, C.c_int]),
     "boat_tensor_clone": (P, [P]),
     "boat_hip_synchronize": (None, []), "boat_hip_set_coherent_pointers": (None, [C.c_int]),
+    "boat_hip_set_reference_exact": (None, [C.c_int]),
     "boat_hip_variable_ensure_grad": (P, [P]),
     "boat_hip_var_gelu": (P, [P]),
     "boat_hip_var_layernorm": (P, [P, P]),
     "boat_hip_var_reshape": (P, [P, C.POINTER(C.c_int64), C.c_size_t]),
     "boat_hip_layernorm_get_weight": (P, [P]), "boat_hip_layernorm_get_bias": (P, [P]),
     "boat_hip_layernorm_get_grad_weight": (P, [P]), "boat_hip_layernorm_get_grad_bias": (P, [P]),
+    "boat_hip_rmsnorm_get_weight": (P, [P]), "boat_hip_rmsnorm_get_grad_weight": (P, [P]),
     "boat_hip_softmax_cross_entropy": (P, [P, P, C.POINTER(P)]),
     "boat_hip_mse_loss": (P, [P, P, C.POINTER(P)]),
     "boat_hip_layer_from_dense": (P, [P]), "boat_hip_layer_from_norm": (P, [P]),

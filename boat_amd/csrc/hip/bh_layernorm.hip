@@ -67,7 +67,9 @@ __device__ __forceinline__ void row_sum2(float& a, float& b, float* lds, int gro
 }
 
 // ---------------------------------------------------------------- forward
-template <int TPR, int VPT>
+// RMS: the RMSNorm of src/layers/norm.c:212-229,366-389 instead: r = sqrtf(mean(x^2)), y = x * (1/(r+eps)) * weight,
+// no mean, no bias; `rstd` then receives 1/(r+eps).
+template <int TPR, int VPT, bool RMS>
 __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                           const float* __restrict__ beta, float* __restrict__ y,
                                                           float* __restrict__ mean, float* __restrict__ rstd,
@@ -100,8 +102,11 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
             xv[i] = (live && c4 < h4) ? ld4_stream(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
             s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
         }
-        row_sum2<TPR>(s, dummy, lds, group);
-        const float mu = s / (float)hidden;
+        float mu = 0.f;
+        if (!RMS) {
+            row_sum2<TPR>(s, dummy, lds, group);
+            mu = s / (float)hidden;
+        }
         float q = 0.f;
         dummy = 0.f;
 #pragma unroll
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
         }
         row_sum2<TPR>(q, dummy, lds, group);
         const float var = q / (float)hidden;
-        const float rs = 1.0f / sqrtf(var + eps);
+        const float rs = RMS ? 1.0f / (sqrtf(var) + eps) : 1.0f / sqrtf(var + eps);
         if (live) {
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
@@ -142,20 +147,21 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
 __global__ __launch_bounds__(kLnBlock) void ln_fwd_generic_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                                   const float* __restrict__ beta, float* __restrict__ y,
                                                                   float* __restrict__ mean, float* __restrict__ rstd,
-                                                                  int64_t rows, int64_t hidden, float eps) {
+                                                                  int64_t rows, int64_t hidden, float eps, int rms) {
     __shared__ float red[kLnBlock / 64];
     const int64_t r = blockIdx.x;
     const float* xr = x + r * hidden;
     float s = 0.f;
-    for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) s += xr[c];
-    const float mu = block_sum<kLnBlock / 64>(s, red) / (float)hidden;
+    if (!rms)
+        for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) s += xr[c];
+    const float mu = rms ? 0.f : block_sum<kLnBlock / 64>(s, red) / (float)hidden;
     float q = 0.f;
     for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
         float d = xr[c] - mu;
         q += d * d;
     }
     const float var = block_sum<kLnBlock / 64>(q, red) / (float)hidden;
-    const float rs = 1.0f / sqrtf(var + eps);
+    const float rs = rms ? 1.0f / (sqrtf(var) + eps) : 1.0f / sqrtf(var + eps);
     for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
         float o = (xr[c] - mu) * rs;
         if (gamma) o *= gamma[c];
@@ -176,12 +182,16 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_generic_kernel(const float* _
 // chunks.  The loop is software-pipelined: the loads of the next row are issued before the current
 // row's reduction barrier and dx stores, so memory requests stay in flight across the barrier.
 // x, dy and dx are streamed once each and marked non-temporal.
-template <int TPR, int VPT>
+//
+// RMS: backward of y = x*s*w with s = 1/(r+eps), r = sqrtf(mean(x^2)) (`rstd` holds s, `mean` is not read).  With
+// xhat = x*s and g = dy*w:  dx = s*(g - xhat*mean_h(g*xhat)/c), c = r*s = 1 - eps*s (a row of zeros has c = 0 and
+// xhat = 0: the second term is dropped); dweight = sum_rows dy*xhat.  The dbeta half of a partial is then unused.
+template <int TPR, int VPT, bool RMS>
 __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                           const float* __restrict__ dy, const float* __restrict__ mean,
                                                           const float* __restrict__ rstd, float* __restrict__ dx,
                                                           float* __restrict__ partial, int64_t rows, int hidden,
-                                                          int64_t iters) {
+                                                          int64_t iters, float eps) {
     constexpr int GROUPS = kLnBlock / TPR;
     extern __shared__ float dyn_lds[];           // GROUPS>1: [GROUPS][2][hidden] for the cross-group fold
     __shared__ float lds[GROUPS * (TPR / 64) * 2 + 2];
@@ -202,7 +212,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
     // prologue: first row of this group
     int64_t row = g_id;
     bool live = row < rows;
-    float mu = live ? mean[row] : 0.f, rs = live ? rstd[row] : 0.f;
+    float mu = (live && !RMS) ? mean[row] : 0.f, rs = live ? rstd[row] : 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int c4 = t + i * TPR;
@@ -230,7 +240,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
         // issue the next row's loads before the barrier
         row = (it + 1) * total_groups + g_id;
         live = (it + 1 < iters) && row < rows;
-        mu = live ? mean[row] : 0.f;
+        mu = (live && !RMS) ? mean[row] : 0.f;
         rs = live ? rstd[row] : 0.f;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
@@ -242,6 +252,11 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
         row_sum2<TPR>(s1, s2, lds, group);
         s1 *= inv_h;
         s2 *= inv_h;
+        if (RMS) {
+            const float c = 1.0f - eps * cur_rs;
+            s1 = 0.f;
+            s2 = c > 0.f ? s2 / c : 0.f;
+        }
         if (cur_live) {
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
@@ -292,10 +307,10 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
 __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_generic_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                                      const float* __restrict__ dy, const float* __restrict__ mean,
                                                                      const float* __restrict__ rstd, float* __restrict__ dx,
-                                                                     int64_t rows, int64_t hidden) {
+                                                                     int64_t rows, int64_t hidden, int rms, float eps) {
     __shared__ float red[kLnBlock / 64];
     const int64_t r = blockIdx.x;
-    const float mu = mean[r], rs = rstd[r];
+    const float mu = rms ? 0.f : mean[r], rs = rstd[r];
     float s1 = 0.f, s2 = 0.f;
     for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
         float xh = (x[r * hidden + c] - mu) * rs;
@@ -305,6 +320,11 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_generic_kernel(const float
     }
     s1 = block_sum<kLnBlock / 64>(s1, red) / (float)hidden;
     s2 = block_sum<kLnBlock / 64>(s2, red) / (float)hidden;
+    if (rms) {
+        const float cc = 1.0f - eps * rs;
+        s1 = 0.f;
+        s2 = cc > 0.f ? s2 / cc : 0.f;
+    }
     for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
         float xh = (x[r * hidden + c] - mu) * rs;
         float g = dy[r * hidden + c] * (gamma ? gamma[c] : 1.0f);
@@ -314,7 +334,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_generic_kernel(const float
 __global__ __launch_bounds__(kLnBlock) void ln_bwd_param_generic_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                                         const float* __restrict__ mean, const float* __restrict__ rstd,
                                                                         float* __restrict__ partial, int64_t rows, int64_t hidden,
-                                                                        int64_t rows_per_block) {
+                                                                        int64_t rows_per_block, int rms) {
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= hidden) return;
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
@@ -323,7 +343,7 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_param_generic_kernel(const fl
     float dg = 0.f, db = 0.f;
     for (int64_t r = r0; r < r1; r++) {
         float gy = dy[r * hidden + c];
-        dg += gy * ((x[r * hidden + c] - mean[r]) * rstd[r]);
+        dg += gy * ((x[r * hidden + c] - (rms ? 0.f : mean[r])) * rstd[r]);
         db += gy;
     }
     partial[((int64_t)blockIdx.y * 2) * hidden + c] = dg;
@@ -374,21 +394,26 @@ int ln_scratch_setup() {
 
 using namespace bh;
 
-#define BH_LN_DISPATCH(KERNEL, plan, grid, shmem, ...)                                                         \
+#define BH_LN_DISPATCH_1(KERNEL, RMS, plan, grid, shmem, ...)                                                   \
     do {                                                                                                       \
         if ((plan).tpr == 64) {                                                                                \
             switch ((plan).vpt) {                                                                              \
-                case 1: hipLaunchKernelGGL((KERNEL<64, 1>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
-                case 2: hipLaunchKernelGGL((KERNEL<64, 2>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
-                case 4: hipLaunchKernelGGL((KERNEL<64, 4>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
-                default: hipLaunchKernelGGL((KERNEL<64, 8>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                case 1: hipLaunchKernelGGL((KERNEL<64, 1, RMS>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                case 2: hipLaunchKernelGGL((KERNEL<64, 2, RMS>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                case 4: hipLaunchKernelGGL((KERNEL<64, 4, RMS>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                default: hipLaunchKernelGGL((KERNEL<64, 8, RMS>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
             }                                                                                                  \
         } else {                                                                                               \
             switch ((plan).vpt) {                                                                              \
-                case 4: hipLaunchKernelGGL((KERNEL<256, 4>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
-                default: hipLaunchKernelGGL((KERNEL<256, 8>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                case 4: hipLaunchKernelGGL((KERNEL<256, 4, RMS>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
+                default: hipLaunchKernelGGL((KERNEL<256, 8, RMS>), grid, dim3(kLnBlock), shmem, stream(), __VA_ARGS__); break; \
             }                                                                                                  \
         }                                                                                                      \
+    } while (0)
+#define BH_LN_DISPATCH(KERNEL, rms, plan, grid, shmem, ...)                         \
+    do {                                                                            \
+        if (rms) BH_LN_DISPATCH_1(KERNEL, true, plan, grid, shmem, __VA_ARGS__);    \
+        else BH_LN_DISPATCH_1(KERNEL, false, plan, grid, shmem, __VA_ARGS__);       \
     } while (0)
 
 extern "C" {
@@ -400,6 +425,24 @@ int bh_layernorm_tune(int bwd_blocks, int reserved) {
     return BH_OK;
 }
 
+static int norm_forward(bool rms, const char* name, const float* x, const float* gamma, const float* beta, float* y,
+                        float* mean, float* rstd, int64_t rows, int64_t hidden, float eps) {
+    LnPlan plan = plan_for(hidden, x, y, gamma ? (const void*)gamma : (const void*)x);
+    if (plan.vector && beta && (reinterpret_cast<uintptr_t>(beta) & 15)) plan.vector = false;
+    if (!plan.vector) {
+        hipLaunchKernelGGL(ln_fwd_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, beta, y,
+                           mean, rstd, rows, hidden, eps, rms ? 1 : 0);
+        return BH_LAUNCH_CHECK(name);
+    }
+    const int groups = kLnBlock / plan.tpr;
+    int64_t blocks = ceil_div(rows, groups);
+    const int64_t cap = 256 * 8;
+    if (blocks > cap) blocks = cap;
+    const int64_t rpg = ceil_div(rows, blocks * groups);
+    BH_LN_DISPATCH(ln_fwd_kernel, rms, plan, dim3((unsigned)blocks), 0, x, gamma, beta, y, mean, rstd, rows, (int)hidden, eps, rpg);
+    return BH_LAUNCH_CHECK(name);
+}
+
 int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, float* y, float* mean, float* rstd,
                          int64_t rows, int64_t hidden, float eps) {
     BH_REQUIRE_INIT();
@@ -407,35 +450,31 @@ int bh_layernorm_forward(const float* x, const float* gamma, const float* beta, 
     if (rows == 0) return BH_OK;
     BH_CHECK_ARG(x && y, "null pointer");
     BH_CHECK_ARG(hidden < (int64_t(1) << 30), "hidden too large");
-    LnPlan plan = plan_for(hidden, x, y, gamma ? (const void*)gamma : (const void*)x);
-    if (plan.vector && beta && (reinterpret_cast<uintptr_t>(beta) & 15)) plan.vector = false;
-    if (!plan.vector) {
-        hipLaunchKernelGGL(ln_fwd_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, beta, y,
-                           mean, rstd, rows, hidden, eps);
-        return BH_LAUNCH_CHECK("bh_layernorm_forward");
-    }
-    const int groups = kLnBlock / plan.tpr;
-    int64_t blocks = ceil_div(rows, groups);
-    const int64_t cap = 256 * 8;
-    if (blocks > cap) blocks = cap;
-    const int64_t rpg = ceil_div(rows, blocks * groups);
-    BH_LN_DISPATCH(ln_fwd_kernel, plan, dim3((unsigned)blocks), 0, x, gamma, beta, y, mean, rstd, rows, (int)hidden, eps, rpg);
-    return BH_LAUNCH_CHECK("bh_layernorm_forward");
+    return norm_forward(false, "bh_layernorm_forward", x, gamma, beta, y, mean, rstd, rows, hidden, eps);
+}
+
+int bh_rmsnorm_forward(const float* x, const float* weight, float* y, float* inv_rms, int64_t rows, int64_t hidden, float eps) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && hidden > 0, "bad shape");
+    if (rows == 0) return BH_OK;
+    BH_CHECK_ARG(x && y, "null pointer");
+    BH_CHECK_ARG(hidden < (int64_t(1) << 30), "hidden too large");
+    return norm_forward(true, "bh_rmsnorm_forward", x, weight, nullptr, y, nullptr, inv_rms, rows, hidden, eps);
 }
 
 // The register-resident path: ln_bwd_kernel writes one dgamma/dbeta partial per workgroup into `partial`
 // (blocks x 2 x hidden floats), fold_rows_kernel sums them.
-static int ln_backward_vector(const LnPlan& plan, size_t shmem, int64_t blocks, float* partial, const float* x,
-                              const float* gamma, const float* dy, const float* mean, const float* rstd, float* dx,
-                              float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
+static int ln_backward_vector(bool rms, float eps, const LnPlan& plan, size_t shmem, int64_t blocks, float* partial,
+                              const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
+                              float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
     const int groups = kLnBlock / plan.tpr;
     const int64_t iters = ceil_div(rows, blocks * groups);
-    BH_LN_DISPATCH(ln_bwd_kernel, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
-                   (int)hidden, iters);
+    BH_LN_DISPATCH(ln_bwd_kernel, rms, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
+                   (int)hidden, iters, eps);
     if (dgamma || dbeta)
         hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
                            stream(), partial, blocks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
-    return BH_LAUNCH_CHECK("bh_layernorm_backward");
+    return BH_LAUNCH_CHECK("norm backward");
 }
 
 // Dynamic LDS of the vector path (the cross-group fold when a workgroup holds several row groups); the path is
@@ -460,6 +499,46 @@ static bool ln_backward_plan(LnPlan& plan, size_t& shmem, const float* x, const 
     return plan.vector;
 }
 
+static int norm_backward(bool rms, float eps, const float* x, const float* gamma, const float* dy, const float* mean,
+                         const float* rstd, float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden,
+                         int accumulate) {
+    LnPlan plan;
+    size_t shmem;
+    ln_backward_plan(plan, shmem, x, gamma, dy, dx, hidden);
+
+    int rc;
+    if (plan.vector) {
+        const int groups = kLnBlock / plan.tpr;
+        int64_t blocks = ceil_div(rows, groups);
+        const int64_t cap = g_ln_bwd_blocks;   // per-block dgamma/dbeta partials cost 2*hidden floats each way
+        if (blocks > cap) blocks = cap;
+        float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(blocks * 2 * hidden));
+        if (!partial) return BH_ENOMEM;
+        rc = ln_backward_vector(rms, eps, plan, shmem, blocks, partial, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows,
+                                hidden, accumulate);
+        bh_free(partial);
+    } else {
+        hipLaunchKernelGGL(ln_bwd_dx_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, dy, mean,
+                           rstd, dx, rows, hidden, rms ? 1 : 0, eps);
+        rc = BH_LAUNCH_CHECK("norm backward dx");
+        if (rc == BH_OK && (dgamma || dbeta)) {
+            int64_t chunks = ceil_div(rows, 64);
+            if (chunks > 256) chunks = 256;
+            const int64_t rpb = ceil_div(rows, chunks);
+            chunks = ceil_div(rows, rpb);
+            float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * 2 * hidden));
+            if (!partial) return BH_ENOMEM;
+            hipLaunchKernelGGL(ln_bwd_param_generic_kernel, dim3((unsigned)ceil_div(hidden, kLnBlock), (unsigned)chunks),
+                               dim3(kLnBlock), 0, stream(), x, dy, mean, rstd, partial, rows, hidden, rpb, rms ? 1 : 0);
+            hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
+                               stream(), partial, chunks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
+            bh_free(partial);
+            rc = BH_LAUNCH_CHECK("norm backward params");
+        }
+    }
+    return rc;
+}
+
 int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
                           float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
     BH_REQUIRE_INIT();
@@ -473,41 +552,20 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, c
         return BH_OK;
     }
     BH_CHECK_ARG(x && dy && mean && rstd && dx, "null pointer");
-    LnPlan plan;
-    size_t shmem;
-    ln_backward_plan(plan, shmem, x, gamma, dy, dx, hidden);
+    return norm_backward(false, 0.f, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden, accumulate);
+}
 
-    int rc;
-    if (plan.vector) {
-        const int groups = kLnBlock / plan.tpr;
-        int64_t blocks = ceil_div(rows, groups);
-        const int64_t cap = g_ln_bwd_blocks;   // per-block dgamma/dbeta partials cost 2*hidden floats each way
-        if (blocks > cap) blocks = cap;
-        float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(blocks * 2 * hidden));
-        if (!partial) return BH_ENOMEM;
-        rc = ln_backward_vector(plan, shmem, blocks, partial, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden,
-                                accumulate);
-        bh_free(partial);
-    } else {
-        hipLaunchKernelGGL(ln_bwd_dx_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, dy, mean,
-                           rstd, dx, rows, hidden);
-        rc = BH_LAUNCH_CHECK("bh_layernorm_backward dx");
-        if (rc == BH_OK && (dgamma || dbeta)) {
-            int64_t chunks = ceil_div(rows, 64);
-            if (chunks > 256) chunks = 256;
-            const int64_t rpb = ceil_div(rows, chunks);
-            chunks = ceil_div(rows, rpb);
-            float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * 2 * hidden));
-            if (!partial) return BH_ENOMEM;
-            hipLaunchKernelGGL(ln_bwd_param_generic_kernel, dim3((unsigned)ceil_div(hidden, kLnBlock), (unsigned)chunks),
-                               dim3(kLnBlock), 0, stream(), x, dy, mean, rstd, partial, rows, hidden, rpb);
-            hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
-                               stream(), partial, chunks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
-            bh_free(partial);
-            rc = BH_LAUNCH_CHECK("bh_layernorm_backward params");
-        }
+int bh_rmsnorm_backward(const float* x, const float* weight, const float* dy, const float* inv_rms, float* dx, float* dweight,
+                        int64_t rows, int64_t hidden, float eps, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && hidden > 0, "bad shape");
+    BH_CHECK_ARG(hidden < (int64_t(1) << 30), "hidden too large");
+    if (rows == 0) {
+        if (!accumulate && dweight) bh_memset_zero(dweight, sizeof(float) * (size_t)hidden);
+        return BH_OK;
     }
-    return rc;
+    BH_CHECK_ARG(x && dy && inv_rms && dx, "null pointer");
+    return norm_backward(true, eps, x, weight, dy, nullptr, inv_rms, dx, dweight, nullptr, rows, hidden, accumulate);
 }
 
 // bh_layernorm_backward for callers that may not allocate: same kernels, the partials live in ln_scratch.
@@ -544,8 +602,8 @@ int bh_layernorm_backward_noalloc(const float* x, const float* gamma, const floa
     if (cap > fit) cap = fit;
     if (blocks > cap) blocks = cap;
     // every partial the fold reads is written by this call's ln_bwd_kernel first: nothing to clear
-    return ln_backward_vector(plan, shmem, blocks, scratch, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden,
-                              accumulate);
+    return ln_backward_vector(false, 0.f, plan, shmem, blocks, scratch, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows,
+                              hidden, accumulate);
 }
 
 }  // extern "C"

@@ -211,7 +211,8 @@ void boat_autodiff_clear_computation_graph(void) {
 
 /* ------------------------------------------------------------- recording */
 
-static bool recording(void) { return !g_current || g_current->grad_enabled; }
+/* the reference stores a context's grad flag and never reads it (autodiff.c:625-632): in reference-exact mode every op is recorded */
+static bool recording(void) { return !g_current || g_current->grad_enabled || bt_reference_exact(); }
 
 static boat_variable_t* record(op_type_t type, boat_variable_t* const* inputs, size_t n, boat_tensor_t* out_tensor,
                                bool requires_grad, void* layer) {
@@ -291,6 +292,15 @@ boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims, size_t n
     }
     boat_tensor_free(m);
     return unary(OP_MEAN, a, out);
+}
+/* no reduction along chosen dimensions exists in the reference either: both return NULL (autodiff.c:595-603) */
+boat_variable_t* boat_var_max(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim) {
+    (void)a; (void)dims; (void)n_dims; (void)keepdim;
+    return NULL;
+}
+boat_variable_t* boat_var_min(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim) {
+    (void)a; (void)dims; (void)n_dims; (void)keepdim;
+    return NULL;
 }
 boat_variable_t* boat_var_flatten(const boat_variable_t* a) {
     if (!a) return NULL;
@@ -583,6 +593,23 @@ static int by_seq_desc(const void* x, const void* y) {
     return a->seq < b->seq ? 1 : a->seq > b->seq ? -1 : 0;
 }
 
+/* Reference-exact mode: the reference's own walk (autodiff.c:373-450), depth first from the root: run the op's gradient
+ * rule, then descend into every non-leaf input with that input's gradient AS ACCUMULATED SO FAR.  A non-leaf variable
+ * with several consumers is therefore descended into once per consumer, each time with a larger gradient: z = y + y,
+ * y = a*b gives da = 4b where the true gradient is 2b. */
+static void backward_depth_first(boat_variable_t* v, const boat_tensor_t* dy) {
+    boat_op_t* op = v->producer;
+    backward_op(op, dy);
+    for (size_t i = 0; i < op->num_inputs; i++) {
+        boat_variable_t* in = op->inputs[i];
+        if (!in || !in->requires_grad || !in->grad || !in->producer) continue;
+        boat_tensor_t* g = in->grad;
+        boat_tensor_ref(g);
+        backward_depth_first(in, g);
+        boat_tensor_unref(g);
+    }
+}
+
 static void boat_variable_backward_unflushed(boat_variable_t* variable, boat_tensor_t* grad_output) {
     if (!variable || !variable->requires_grad) return;
     boat_tensor_t* seed = grad_output;
@@ -593,6 +620,11 @@ static void boat_variable_backward_unflushed(boat_variable_t* variable, boat_ten
     }
     if (!variable->producer) {
         accumulate(variable, seed, false);  /* leaf: grad += dY (autodiff.c:346-361) */
+        if (!grad_output) boat_tensor_unref(seed);
+        return;
+    }
+    if (bt_reference_exact()) {
+        backward_depth_first(variable, seed);
         if (!grad_output) boat_tensor_unref(seed);
         return;
     }

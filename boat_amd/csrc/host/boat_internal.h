@@ -64,6 +64,9 @@ boat_tensor_t* bt_new_uninit(const int64_t* shape, size_t ndim, boat_device_t de
 bool bt_same_shape(const boat_tensor_t* a, const boat_tensor_t* b);
 bool bt_is_f32(const boat_tensor_t* t);
 
+/* true in reference-exact mode (boat_hip_set_reference_exact / BOAT_HIP_REFERENCE_EXACT=1) */
+bool bt_reference_exact(void);
+
 void boat_fail(boat_error_t code, const char* fmt, ...);
 /* turns a bh_* return code into a Boat error; returns true when rc == 0 */
 bool boat_hip_ok(int rc, const char* what);
@@ -88,6 +91,14 @@ struct boat_layernorm_t {
     boat_tensor_t* cache_input;
     boat_tensor_t* cache_mean;   /* [rows] */
     boat_tensor_t* cache_rstd;   /* [rows]; the reference's field is named cache_variance and never written */
+};
+
+struct boat_rmsnorm_t {
+    boat_rmsnorm_config_t config;
+    boat_tensor_t* weight;       /* ones at creation when elementwise_affine (norm.c:149-158) */
+    boat_tensor_t* grad_weight;
+    boat_tensor_t* cache_input;
+    boat_tensor_t* cache_inv_rms;   /* [rows]: 1/(rms + eps); the reference's cache_rms is never written */
 };
 
 struct boat_attention_t {

@@ -10,8 +10,8 @@
  *   - the gradient tensors keep their identity across backward calls (the reference frees and replaces
  *     them, conv.c:523-532, which leaves a registered optimizer holding dangling pointers);
  *   - the input gradient is the true one by default; the reference pairs each tap with the mirrored weight
- *     (conv.c:86-88).  boat_hip_conv_reference_input_grad(1) switches to the reference's pairing for callers
- *     that need its numbers.
+ *     (conv.c:86-88).  boat_hip_conv_reference_input_grad(1), or reference-exact mode, switches to the reference's
+ *     pairing for callers that need its numbers.
  */
 #include "boat_internal.h"
 
@@ -19,9 +19,10 @@
 #include <stdlib.h>
 #include <string.h>
 
-static int g_reference_input_grad = 0;
+static int g_reference_input_grad = -1;   /* -1: not set by a call, follow reference-exact mode */
 
-void boat_hip_conv_reference_input_grad(int enable) { g_reference_input_grad = enable != 0; }
+void boat_hip_conv_reference_input_grad(int enable) { g_reference_input_grad = enable < 0 ? -1 : enable != 0; }
+static int reference_input_grad(void) { return g_reference_input_grad >= 0 ? g_reference_input_grad : (bt_reference_exact() ? 1 : 0); }
 
 struct boat_conv_layer_t {
     size_t in_channels, out_channels, kernel_size, stride, padding;
@@ -135,7 +136,7 @@ static boat_tensor_t* boat_conv_layer_backward_unflushed(boat_conv_layer_t* l, c
     if (!px || !pw || !pg || !pdx || !pgw ||
         !boat_hip_ok(bh_conv2d_backward(px, pw, pg, pdx, pgw, pgb, x->shape[0], (int64_t)l->in_channels, x->shape[2], x->shape[3],
                                         (int64_t)l->out_channels, (int64_t)l->kernel_size, (int64_t)l->stride, (int64_t)l->padding,
-                                        0, g_reference_input_grad),
+                                        0, reference_input_grad()),
                      "conv backward")) {
         boat_tensor_free(dx);
         return NULL;

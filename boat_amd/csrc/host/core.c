@@ -57,6 +57,15 @@ void boat_set_error(boat_error_t error, const char* message) {
     g_last_error = error;
     snprintf(g_last_message, sizeof(g_last_message), "%s", message ? message : "");
 }
+/* src/core/error.c:64-80 */
+void boat_set_errorf(boat_error_t error, const char* format, ...) {
+    va_list ap;
+    va_start(ap, format);
+    g_last_error = error;
+    vsnprintf(g_last_message, sizeof(g_last_message), format ? format : "", ap);
+    va_end(ap);
+}
+void boat_reset_error(void) { boat_clear_error(); }
 void boat_clear_error(void) {
     g_last_error = BOAT_SUCCESS;
     g_last_message[0] = 0;
@@ -154,6 +163,42 @@ void boat_memory_free(void* ptr) {
     h->magic = 0;
     stats_free(h->size);
     free(h);
+}
+void boat_memory_free_safe(void** ptr_ptr) {   /* memory.c:137-142 */
+    if (ptr_ptr && *ptr_ptr) {
+        boat_memory_free(*ptr_ptr);
+        *ptr_ptr = NULL;
+    }
+}
+/* memory.c:189-227: a host block over-allocated by alignment + one word, the original pointer kept in the word before the
+ * aligned address.  Device blocks come from hipMalloc, which aligns to 256 bytes and more: they are handed out as they are
+ * when that satisfies the request (a header cannot be written into device memory from here). */
+void* boat_memory_allocate_aligned(size_t size, size_t alignment, boat_device_t device, const char* file, int line) {
+    if (alignment < sizeof(void*)) alignment = sizeof(void*);
+    if (alignment & (alignment - 1)) {
+        boat_fail(BOAT_ERROR_INVALID_ARGUMENT, "boat_memory_allocate_aligned: alignment %zu is not a power of two", alignment);
+        return NULL;
+    }
+    if (device == BOAT_DEVICE_HIP) {
+        void* p = boat_memory_allocate(size, device, file, line);
+        if (p && ((uintptr_t)p & (alignment - 1))) {
+            boat_memory_free(p);
+            boat_fail(BOAT_ERROR_INVALID_ARGUMENT, "boat_memory_allocate_aligned: device blocks are aligned to 256 bytes, %zu was asked", alignment);
+            return NULL;
+        }
+        return p;
+    }
+    const size_t total = size + alignment + sizeof(size_t);
+    void* ptr = boat_memory_allocate(total, device, file, line);
+    if (!ptr) return NULL;
+    const uintptr_t aligned = ((uintptr_t)ptr + alignment + sizeof(size_t)) & ~(uintptr_t)(alignment - 1);
+    *(void**)(aligned - sizeof(size_t)) = ptr;
+    return (void*)aligned;
+}
+void boat_memory_free_aligned(const void* aligned_ptr) {
+    if (!aligned_ptr) return;
+    if (device_block_free((void*)aligned_ptr)) return;
+    boat_memory_free(*(void**)((uintptr_t)aligned_ptr - sizeof(size_t)));
 }
 void* boat_memory_reallocate(void* ptr, size_t new_size, boat_device_t device, const char* file, int line) {
     /* memory.c:85-120: NULL allocates, size 0 frees, otherwise the block keeps its contents up to the smaller size */
@@ -315,19 +360,32 @@ boat_tensor_t* bt_new_like_uninit(const boat_tensor_t* like) {
 /* ---- coherent-pointer mode ----
  * Boat's callers keep the float* that boat_tensor_data() gave them: they write through it before a later call
  * (tests/unit/test_attention_gradient_check.c:22-41) and read results through it after one
- * (tests/unit/test_optimizer_adam.c:96-108).  The default protocol only promises the pointer until the next call
- * that takes the tensor, which keeps parameters resident on the device.  In this mode a tensor whose pointer was
- * handed out is "exposed": its host mirror is uploaded before every device read (the caller may have written), and
- * device writes to it are copied back before the public call returns (the caller may read).  Correct for any caller,
- * at the price of PCIe transfers for exposed tensors. */
+ * (tests/unit/test_optimizer_adam.c:96-108).  The reference's pointer IS the tensor's storage, so this mode is the
+ * default: a tensor whose pointer was handed out is "exposed": its host mirror is uploaded before every device read
+ * (the caller may have written), and device writes to it are copied back before the public call returns (the caller
+ * may read).  Correct for any caller, at the price of PCIe transfers for exposed tensors.  Switched off
+ * (boat_hip_set_coherent_pointers(0) or BOAT_HIP_COHERENT_POINTERS=0), a pointer is only promised until the next call
+ * that takes the tensor, and parameters stay resident on the device whatever the caller looked at. */
 static int g_coherent = -1;
+static int g_reference_exact = -1;
+
+/* Reference-exact mode: every place where this library deliberately computes something else than the reference does
+ * follows the reference instead (see boat_hip_set_reference_exact in boat_api.h). */
+bool bt_reference_exact(void) {
+    if (g_reference_exact < 0) {
+        const char* e = getenv("BOAT_HIP_REFERENCE_EXACT");
+        g_reference_exact = e && *e && *e != '0';
+    }
+    return g_reference_exact != 0;
+}
+void boat_hip_set_reference_exact(int enable) { g_reference_exact = enable != 0; }
 static boat_storage_t** g_pending = NULL;
 static size_t g_pending_n = 0, g_pending_cap = 0;
 
 static bool coherent_mode(void) {
     if (g_coherent < 0) {
-        const char* e = getenv("BOAT_HIP_COHERENT_POINTERS");
-        g_coherent = e && *e && *e != '0';
+        const char* e = getenv("BOAT_HIP_COHERENT_POINTERS");   /* on unless the environment says 0 */
+        g_coherent = !(e && *e == '0');
     }
     return g_coherent != 0;
 }

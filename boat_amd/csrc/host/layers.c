@@ -377,6 +377,137 @@ boat_tensor_t* boat_layer_norm_grad(const boat_tensor_t* grad_output, const boat
     return dx;
 }
 
+/* stateless forms (stubs in the reference, norm.c:424-448): normalisation over the last dimension, no affine */
+boat_tensor_t* boat_layer_norm(const boat_tensor_t* input, const int64_t* normalized_shape, size_t normalized_shape_len, float eps) {
+    if (!input || !normalized_shape || normalized_shape_len != 1) return NULL;
+    boat_layernorm_config_t cfg = {(size_t)normalized_shape[0], eps, false, false};
+    boat_layernorm_t* tmp = boat_layernorm_create(&cfg);
+    if (!tmp) return NULL;
+    boat_tensor_t* y = boat_layernorm_forward(tmp, input);
+    boat_layernorm_free(tmp);
+    return y;
+}
+
+/* ----------------------------------------------------------------- rmsnorm
+ * src/layers/norm.c:136-181 (create/free), :319-395 (forward: rms = sqrtf(mean(x^2)), y = x/(rms+eps)*weight, eps OUTSIDE
+ * the root); backward and update are stubs in the reference (:404-421) and are implemented here like LayerNorm's. */
+boat_rmsnorm_t* boat_rmsnorm_create(const boat_rmsnorm_config_t* config) {
+    if (!config || config->normalized_shape == 0) return NULL;
+    boat_rmsnorm_t* norm = (boat_rmsnorm_t*)calloc(1, sizeof(*norm));
+    if (!norm) return NULL;
+    norm->config = *config;
+    if (config->elementwise_affine) {
+        norm->weight = create_vector(config->normalized_shape);
+        norm->grad_weight = create_vector(config->normalized_shape);
+        float* g = norm->weight ? (float*)bt_host_rw(norm->weight) : NULL;
+        if (!g || !norm->grad_weight) {
+            boat_rmsnorm_free(norm);
+            return NULL;
+        }
+        for (size_t i = 0; i < config->normalized_shape; i++) g[i] = 1.0f;
+    }
+    return norm;
+}
+
+void boat_rmsnorm_free(boat_rmsnorm_t* norm) {
+    if (!norm) return;
+    boat_tensor_free(norm->weight);
+    boat_tensor_free(norm->grad_weight);
+    boat_tensor_free(norm->cache_input);
+    boat_tensor_free(norm->cache_inv_rms);
+    free(norm);
+}
+
+boat_tensor_t* boat_rmsnorm_forward(boat_rmsnorm_t* norm, const boat_tensor_t* input) {
+    if (!norm || !input || input->ndim < 1 || !bt_is_f32(input)) return NULL;
+    const int64_t hidden = (int64_t)norm->config.normalized_shape;
+    if (input->shape[input->ndim - 1] != hidden) return NULL;
+    const int64_t rows = layernorm_rows(input);   /* the same loop nest as LayerNorm's (norm.c:360-362) */
+    const bool covers_all = rows * hidden == (int64_t)input->nelements;
+    boat_tensor_t* out = covers_all ? bt_new_like_uninit(input) : boat_tensor_create_like(input);
+    const int64_t rshape[] = {rows};
+    boat_tensor_t* inv = bt_new_uninit(rshape, 1, input->device);
+    bool ok = out && inv;
+    if (ok && rows > 0) {
+        const float* px = bt_dev_read(input);
+        const float* pw = norm->weight ? bt_dev_read(norm->weight) : NULL;
+        float* py = covers_all ? bt_dev_write(out) : bt_dev_rw(out);
+        ok = px && py && boat_hip_ok(bh_rmsnorm_forward(px, pw, py, bt_dev_write(inv), rows, hidden, norm->config.eps), "rmsnorm forward");
+    }
+    if (!ok) {
+        boat_tensor_free(out);
+        boat_tensor_free(inv);
+        return NULL;
+    }
+    swap_tensor(&norm->cache_input, (boat_tensor_t*)input);
+    boat_tensor_free(norm->cache_inv_rms);
+    norm->cache_inv_rms = inv;
+    return out;
+}
+
+boat_tensor_t* boat_rmsnorm_backward(boat_rmsnorm_t* norm, const boat_tensor_t* grad_output) {
+    if (!norm || !grad_output) return NULL;
+    if (!norm->cache_input || !norm->cache_inv_rms) {
+        fprintf(stderr, "Error: RMSNorm backward called before forward\n");
+        return NULL;
+    }
+    const boat_tensor_t* x = norm->cache_input;
+    if (!bt_is_f32(grad_output) || grad_output->nelements != x->nelements) {
+        fprintf(stderr, "Error: RMSNorm backward shape mismatch\n");
+        return NULL;
+    }
+    const int64_t hidden = (int64_t)norm->config.normalized_shape;
+    const int64_t rows = (int64_t)norm->cache_inv_rms->nelements;
+    const bool covers_all = rows * hidden == (int64_t)x->nelements;
+    boat_tensor_t* dx = covers_all ? bt_new_like_uninit(x) : boat_tensor_create_like(x);
+    if (!dx || rows == 0) return dx;
+    const float* px = bt_dev_read(x);
+    const float* pdy = bt_dev_read(grad_output);
+    const float* pw = norm->weight ? bt_dev_read(norm->weight) : NULL;
+    float* pdx = covers_all ? bt_dev_write(dx) : bt_dev_rw(dx);
+    float* pgw = norm->grad_weight ? bt_dev_rw(norm->grad_weight) : NULL;
+    /* the parameter gradient accumulates across calls like the dense layer's (dense.c:255-291) */
+    if (!px || !pdy || !pdx ||
+        !boat_hip_ok(bh_rmsnorm_backward(px, pw, pdy, bt_dev_read(norm->cache_inv_rms), pdx, pgw, rows, hidden, norm->config.eps, 1),
+                     "rmsnorm backward")) {
+        boat_tensor_free(dx);
+        dx = NULL;
+    }
+    bt_flush_exposed();
+    return dx;
+}
+
+void boat_rmsnorm_update(boat_rmsnorm_t* norm, float learning_rate) {
+    if (!norm) return;
+    sgd_step(norm->weight, norm->grad_weight, learning_rate, true);
+    bt_flush_exposed();
+}
+boat_tensor_t* boat_hip_rmsnorm_get_weight(const boat_rmsnorm_t* n) { return n ? n->weight : NULL; }
+boat_tensor_t* boat_hip_rmsnorm_get_grad_weight(const boat_rmsnorm_t* n) { return n ? n->grad_weight : NULL; }
+
+boat_tensor_t* boat_rms_norm(const boat_tensor_t* input, const int64_t* normalized_shape, size_t normalized_shape_len, float eps) {
+    if (!input || !normalized_shape || normalized_shape_len != 1) return NULL;
+    boat_rmsnorm_config_t cfg = {(size_t)normalized_shape[0], eps, false};
+    boat_rmsnorm_t* tmp = boat_rmsnorm_create(&cfg);
+    if (!tmp) return NULL;
+    boat_tensor_t* y = boat_rmsnorm_forward(tmp, input);
+    boat_rmsnorm_free(tmp);
+    return y;
+}
+boat_tensor_t* boat_rms_norm_grad(const boat_tensor_t* grad_output, const boat_tensor_t* input, const boat_tensor_t* output,
+                                  const int64_t* normalized_shape, size_t normalized_shape_len, float eps) {
+    (void)output;
+    if (!grad_output || !input || !normalized_shape || normalized_shape_len != 1) return NULL;
+    boat_rmsnorm_config_t cfg = {(size_t)normalized_shape[0], eps, false};
+    boat_rmsnorm_t* tmp = boat_rmsnorm_create(&cfg);
+    if (!tmp) return NULL;
+    boat_tensor_t* y = boat_rmsnorm_forward(tmp, input);
+    boat_tensor_t* dx = y ? boat_rmsnorm_backward(tmp, grad_output) : NULL;
+    boat_tensor_free(y);
+    boat_rmsnorm_free(tmp);
+    return dx;
+}
+
 boat_norm_layer_t* boat_norm_layer_create(size_t normalized_shape, float eps, bool elementwise_affine) {
     boat_layernorm_config_t config = {normalized_shape, eps, elementwise_affine, elementwise_affine};
     return boat_layernorm_create(&config);
@@ -481,6 +612,62 @@ boat_tensor_t* boat_attention_forward(boat_attention_t* a, const boat_tensor_t* 
                      "attention core forward"))
         return NULL;
     return project(a->cache_attention_output, a->weight_o, a->bias_o, rows, h);
+}
+
+/* attention.c:1082-1092 over :882-1079: softmax(scale * Q.K^T) . V on [batch, heads, seq, head_size] tensors of one shape;
+ * the mask argument and dropout are ignored there (:1022-1025, 1061-1062) and here.  Operands that are not 4-D get a copy
+ * of `value` back, as the reference's compatibility branch does (:905-917). */
+boat_tensor_t* boat_scaled_dot_product_attention(const boat_tensor_t* query, const boat_tensor_t* key, const boat_tensor_t* value,
+                                                 float scale_factor, const boat_tensor_t* attention_mask, bool causal_mask,
+                                                 float dropout_prob) {
+    (void)attention_mask;
+    (void)dropout_prob;
+    if (!query || !key || !value) return NULL;
+    if (query->ndim < 3 || key->ndim < 3 || value->ndim < 3) return NULL;
+    if (query->ndim != 4 || key->ndim != 4 || value->ndim != 4) return boat_tensor_clone(value);
+    if (!bt_same_shape(query, key) || !bt_same_shape(query, value)) return NULL;
+    if (!bt_is_f32(query) || !bt_is_f32(key) || !bt_is_f32(value)) return NULL;
+    boat_tensor_t* out = bt_new_like_uninit(value);
+    if (!out || out->nelements == 0) return out;
+    const int64_t heads = query->shape[0] * query->shape[1], seq = query->shape[2], hd = query->shape[3];
+    const int64_t lshape[] = {heads, seq};
+    boat_tensor_t* lse = bt_new_uninit(lshape, 2, value->device);
+    const float* pq = bt_dev_read(query);
+    const float* pk = bt_dev_read(key);
+    const float* pv = bt_dev_read(value);
+    float* po = bt_dev_write(out);
+    float* pl = lse ? bt_dev_write(lse) : NULL;
+    if (!pq || !pk || !pv || !po || !pl ||
+        !boat_hip_ok(bh_sdpa_forward(pq, pk, pv, scale_factor, causal_mask ? 1 : 0, po, pl, NULL, heads, seq, hd),
+                     "scaled dot-product attention")) {
+        boat_tensor_free(out);
+        out = NULL;
+    }
+    boat_tensor_free(lse);
+    return out;
+}
+
+/* attention.c:830-880: self-attention through a throw-away layer with fresh random projections (bias on) */
+boat_tensor_t* boat_multihead_attention(const boat_tensor_t* input, size_t num_heads, float dropout_prob, bool causal_mask,
+                                        const boat_tensor_t* attention_mask) {
+    if (!input || input->ndim != 3 || num_heads == 0) return NULL;
+    const size_t hidden = (size_t)input->shape[2];
+    if (hidden % num_heads != 0) return NULL;
+    boat_attention_config_t config = {hidden, num_heads, hidden / num_heads, dropout_prob, causal_mask, true, false, 10000.0f};
+    boat_attention_t* attention = boat_attention_create(&config);
+    if (!attention) return NULL;
+    boat_tensor_t* output = boat_attention_forward(attention, input, input, input, attention_mask);
+    boat_attention_free(attention);
+    return output;
+}
+
+/* not implemented in the reference either (attention.c:1094-1120): NULL and no effect */
+boat_tensor_t* boat_rotary_position_encoding(const boat_tensor_t* tensor, size_t seq_len, size_t head_size, float theta) {
+    (void)tensor; (void)seq_len; (void)head_size; (void)theta;
+    return NULL;
+}
+void boat_apply_rotary_embedding(boat_tensor_t* query, boat_tensor_t* key, size_t seq_len, size_t head_size, float theta) {
+    (void)query; (void)key; (void)seq_len; (void)head_size; (void)theta;
 }
 
 /* linear_projection_backward, attention.c:1186-1285: dx = dy.w^T ; *gw = x^T.dy ; *gb = colsum(dy), all overwritten */

@@ -15,12 +15,43 @@ struct boat_model_t {
     boat_layer_t** layers;
     size_t layer_count, layer_capacity;
     boat_graph_t* graph;   /* the layers as a chain of nodes, for callers that look at boat_model_graph() */
+    void* user_data;                  /* model.c:382-397: carried for the caller, released with the model */
+    void (*free_user_data)(void*);
 };
 
 boat_model_t* boat_model_create(void) {
     boat_model_t* model = (boat_model_t*)calloc(1, sizeof(boat_model_t));
     if (model) model->graph = boat_graph_create();
     return model;
+}
+/* model.c:59-83: the model takes the graph over (it is freed with the model) */
+boat_model_t* boat_model_create_with_graph(const boat_graph_t* graph) {
+    if (!graph) return NULL;
+    boat_model_t* model = (boat_model_t*)calloc(1, sizeof(boat_model_t));
+    if (model) model->graph = (boat_graph_t*)graph;
+    return model;
+}
+void boat_model_set_graph(boat_model_t* model, boat_graph_t* graph) {   /* model.c:133-145 */
+    if (!model || !graph) return;
+    if (model->graph && model->graph != graph) boat_graph_free(model->graph);
+    model->graph = graph;
+}
+void* boat_model_get_user_data(const boat_model_t* model) { return model ? model->user_data : NULL; }
+void boat_model_set_user_data(boat_model_t* model, void* user_data, void (*free_fn)(void*)) {
+    if (!model) return;
+    if (model->user_data && model->free_user_data) model->free_user_data(model->user_data);
+    model->user_data = user_data;
+    model->free_user_data = free_fn;
+}
+/* no file format exists for a model in the reference: both are stubs there too (model.c:368-379) */
+boat_model_t* boat_model_load(const char* filename) {
+    (void)filename;
+    return NULL;
+}
+bool boat_model_save(const boat_model_t* model, const char* filename) {
+    (void)model;
+    (void)filename;
+    return false;
 }
 boat_graph_t* boat_model_graph(const boat_model_t* model) { return model ? model->graph : NULL; }
 size_t boat_graph_node_count(const boat_graph_t* graph) { return graph ? graph->node_count : 0; }
@@ -50,6 +81,7 @@ void boat_model_free(boat_model_t* model) {
     }
     free(model->layers);
     boat_graph_free(model->graph);
+    if (model->user_data && model->free_user_data) model->free_user_data(model->user_data);
     free(model);
 }
 

@@ -27,12 +27,47 @@ static bool broadcast_shape(const boat_tensor_t* a, const boat_tensor_t* b, int6
     return true;
 }
 
-static boat_tensor_t* binary_op(int op, const boat_tensor_t* a, const boat_tensor_t* b) {
-    if (!a || !b) return NULL;
-    if (!bt_is_f32(a) || !bt_is_f32(b)) {
-        boat_fail(BOAT_ERROR_NOT_IMPLEMENTED, "elementwise ops take float32 tensors only");
+/* element types the reference's arithmetic switches on (arithmetic.c:197-282): float32, float64, int32, int64 */
+static int typed_code(boat_dtype_t dtype) {
+    switch (dtype) {
+        case BOAT_DTYPE_FLOAT32: return BH_DT_F32;
+        case BOAT_DTYPE_FLOAT64: return BH_DT_F64;
+        case BOAT_DTYPE_INT32: return BH_DT_I32;
+        case BOAT_DTYPE_INT64: return BH_DT_I64;
+        default: return -1;
+    }
+}
+
+/* the same operators on float64 / int32 / int64 tensors, and boat_mod on all four types (arithmetic.c:157-360) */
+static boat_tensor_t* binary_op_typed(int op, const boat_tensor_t* a, const boat_tensor_t* b) {
+    const int code = typed_code(a->dtype);
+    if (a->dtype != b->dtype || code < 0) return NULL;   /* arithmetic.c:166-170, 278-281 */
+    if (!same_device(a, b)) {
+        boat_fail(BOAT_ERROR_DEVICE, "elementwise op on tensors of different devices");
         return NULL;
     }
+    int64_t shape[BOAT_MAX_DIMS], sa[BOAT_MAX_DIMS], sb[BOAT_MAX_DIMS];
+    size_t nd = 0;
+    if (!broadcast_shape(a, b, shape, &nd)) return NULL;
+    boat_tensor_t* out = boat_tensor_create(shape, nd, a->dtype, a->device);
+    if (!out || out->nelements == 0) return out;
+    for (size_t i = 0; i < nd; i++) {
+        sa[i] = i < nd - a->ndim ? 1 : a->shape[i - (nd - a->ndim)];
+        sb[i] = i < nd - b->ndim ? 1 : b->shape[i - (nd - b->ndim)];
+    }
+    const void* pa = bt_dev_read(a);
+    const void* pb = bt_dev_read(b);
+    void* po = bt_dev_write(out);
+    if (!pa || !pb || !po || !boat_hip_ok(bh_binary_typed(code, op, pa, sa, pb, sb, po, shape, (int)nd), "elementwise op")) {
+        boat_tensor_free(out);
+        return NULL;
+    }
+    return out;
+}
+
+static boat_tensor_t* binary_op(int op, const boat_tensor_t* a, const boat_tensor_t* b) {
+    if (!a || !b) return NULL;
+    if (!bt_is_f32(a) || !bt_is_f32(b)) return binary_op_typed(op, a, b);
     if (!same_device(a, b)) {
         boat_fail(BOAT_ERROR_DEVICE, "elementwise op on tensors of different devices");
         return NULL;
@@ -70,11 +105,22 @@ boat_tensor_t* boat_add(const boat_tensor_t* a, const boat_tensor_t* b) { return
 boat_tensor_t* boat_sub(const boat_tensor_t* a, const boat_tensor_t* b) { return binary_op(1, a, b); }
 boat_tensor_t* boat_mul(const boat_tensor_t* a, const boat_tensor_t* b) { return binary_op(2, a, b); }
 boat_tensor_t* boat_div(const boat_tensor_t* a, const boat_tensor_t* b) { return binary_op(3, a, b); }
+boat_tensor_t* boat_mod(const boat_tensor_t* a, const boat_tensor_t* b) { return (a && b) ? binary_op_typed(4, a, b) : NULL; }   /* arithmetic.c:288-360 */
 
 static void inplace_op(int op, boat_tensor_t* a, const boat_tensor_t* b) {
     if (!a || !b) return;
     if (a->nelements != b->nelements || a->dtype != b->dtype) return;   /* arithmetic.c:372-376: silent */
-    if (!bt_is_f32(a) || !same_device(a, b) || a->nelements == 0) return;
+    if (!same_device(a, b) || a->nelements == 0) return;
+    if (!bt_is_f32(a)) {   /* float64 / int32 / int64 (arithmetic.c:388-412): flat, no broadcasting */
+        const int code = typed_code(a->dtype);
+        const int64_t n = (int64_t)a->nelements;
+        if (code < 0) return;
+        const void* pb = bt_dev_read(b);
+        void* pa = bt_dev_rw(a);
+        if (pa && pb) boat_hip_ok(bh_binary_typed(code, op, pa, &n, pb, &n, pa, &n, 1), "in-place op");
+        bt_flush_exposed();
+        return;
+    }
     const float* pb = bt_dev_read(b);
     float* pa = bt_dev_rw(a);
     if (!pa || !pb) return;
@@ -87,8 +133,24 @@ void boat_sub_(boat_tensor_t* a, const boat_tensor_t* b) { inplace_op(1, a, b); 
 void boat_mul_(boat_tensor_t* a, const boat_tensor_t* b) { inplace_op(2, a, b); }
 void boat_div_(boat_tensor_t* a, const boat_tensor_t* b) { inplace_op(3, a, b); }
 
+/* out = a op scalar on float64 / int32 / int64 tensors, and powf/pow (arithmetic.c:425-518); in_place writes into a */
+static boat_tensor_t* scalar_op_typed(int op, const boat_tensor_t* a, double scalar, bool in_place) {
+    const int code = typed_code(a->dtype);
+    if (code < 0 || (op == 5 && code > BH_DT_F64)) return NULL;
+    boat_tensor_t* out = in_place ? (boat_tensor_t*)a : boat_tensor_create(a->shape, a->ndim, a->dtype, a->device);
+    if (!out || out->nelements == 0) return out;
+    const void* pa = in_place ? bt_dev_rw(out) : bt_dev_read(a);
+    void* po = in_place ? (void*)pa : bt_dev_write(out);
+    if (!pa || !po || !boat_hip_ok(bh_scalar_op_typed(code, op, pa, scalar, po, (int64_t)a->nelements), "scalar op")) {
+        if (!in_place) boat_tensor_free(out);
+        return NULL;
+    }
+    return out;
+}
+
 static boat_tensor_t* scalar_op(int op, const boat_tensor_t* a, double scalar) {
-    if (!a || !bt_is_f32(a)) return NULL;
+    if (!a) return NULL;
+    if (!bt_is_f32(a)) return scalar_op_typed(op, a, scalar, false);
     boat_tensor_t* out = bt_new_like_uninit(a);
     if (!out || out->nelements == 0) return out;
     const float* pa = bt_dev_read(a);
@@ -103,6 +165,26 @@ boat_tensor_t* boat_add_scalar(const boat_tensor_t* a, double s) { return scalar
 boat_tensor_t* boat_sub_scalar(const boat_tensor_t* a, double s) { return scalar_op(1, a, s); }
 boat_tensor_t* boat_mul_scalar(const boat_tensor_t* a, double s) { return scalar_op(2, a, s); }
 boat_tensor_t* boat_div_scalar(const boat_tensor_t* a, double s) { return scalar_op(3, a, s); }
+boat_tensor_t* boat_pow_scalar(const boat_tensor_t* a, double s) { return a ? scalar_op_typed(5, a, s, false) : NULL; }   /* arithmetic.c:486-518 */
+/* in-place forms (arithmetic.c:521-570) */
+static void scalar_op_inplace(int op, boat_tensor_t* a, double scalar) {
+    if (!a) return;
+    scalar_op_typed(op, a, scalar, true);
+    bt_flush_exposed();
+}
+void boat_add_scalar_(boat_tensor_t* a, double s) { scalar_op_inplace(0, a, s); }
+void boat_sub_scalar_(boat_tensor_t* a, double s) { scalar_op_inplace(1, a, s); }
+void boat_mul_scalar_(boat_tensor_t* a, double s) { scalar_op_inplace(2, a, s); }
+void boat_div_scalar_(boat_tensor_t* a, double s) { scalar_op_inplace(3, a, s); }
+/* stubs in the reference as well (src/ops/linear.c:409-413, src/ops/activation.c:304-308) */
+boat_tensor_t* boat_inverse(const boat_tensor_t* a) {
+    (void)a;
+    return NULL;
+}
+boat_tensor_t* boat_selu(const boat_tensor_t* a) {
+    (void)a;
+    return NULL;
+}
 
 boat_tensor_t* boat_matmul(const boat_tensor_t* a, const boat_tensor_t* b) {
     if (!a || !b) return NULL;
@@ -242,7 +324,11 @@ static boat_tensor_t* activation(int act, const boat_tensor_t* a) {
     }
     return out;
 }
-boat_tensor_t* boat_relu(const boat_tensor_t* a) { return activation(BH_ACT_RELU, a); }
+boat_tensor_t* boat_relu(const boat_tensor_t* a) {
+    /* activation.c:266-282: float32 is rectified, any other element type comes back as a copy */
+    if (a && !bt_is_f32(a)) return boat_tensor_clone(a);
+    return activation(BH_ACT_RELU, a);
+}
 boat_tensor_t* boat_sigmoid(const boat_tensor_t* a) { return activation(BH_ACT_SIGMOID, a); }
 boat_tensor_t* boat_tanh(const boat_tensor_t* a) { return activation(BH_ACT_TANH, a); }
 boat_tensor_t* boat_gelu(const boat_tensor_t* a) { return activation(BH_ACT_GELU, a); }

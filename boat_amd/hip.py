@@ -51,6 +51,10 @@ _SIGS = {
     "bh_softmax_ce_grad": (I, [P, P, P, P, L, L]),
     "bh_layernorm_forward": (I, [P, P, P, P, P, P, L, L, F]),
     "bh_layernorm_backward": (I, [P, P, P, P, P, P, P, P, L, L, I]),
+    "bh_rmsnorm_forward": (I, [P, P, P, P, L, L, F]),
+    "bh_rmsnorm_backward": (I, [P, P, P, P, P, P, L, L, F, I]),
+    "bh_binary_typed": (I, [I, I, P, C.POINTER(L), P, C.POINTER(L), P, C.POINTER(L), I]),
+    "bh_scalar_op_typed": (I, [I, I, P, C.c_double, P, L]),
     "bh_layernorm_backward_noalloc": (I, [P, P, P, P, P, P, P, P, L, L, I]),
     "bh_gemm": (I, [I, I, L, L, L, P, L, P, L, P, L, P, I, L]),
     "bh_gemm_force_config": (I, [I]), "bh_gemm_force_direct": (I, [I]),

@@ -12,7 +12,8 @@
  * GPU slot, value 1; alias BOAT_DEVICE_HIP) lives in HBM only and boat_tensor_data() returns the
  * device pointer.
  *
- * Only fp32 tensors take part in arithmetic, as on the reference's hot path.
+ * Layers, the tape and the optimizers take fp32 tensors, as on the reference's hot path; the eager elementwise
+ * ops also take float64, int32 and int64 tensors, like the reference's (src/ops/arithmetic.c:197-282).
  */
 #ifndef BOAT_API_H
 #define BOAT_API_H
@@ -76,6 +77,9 @@ typedef struct {
 BOAT_API void* boat_memory_allocate(size_t size, boat_device_t device, const char* file, int line);
 BOAT_API void* boat_memory_allocate_zero(size_t size, boat_device_t device, const char* file, int line);
 BOAT_API void boat_memory_free(void* ptr);
+BOAT_API void boat_memory_free_safe(void** ptr_ptr);
+BOAT_API void* boat_memory_allocate_aligned(size_t size, size_t alignment, boat_device_t device, const char* file, int line);
+BOAT_API void boat_memory_free_aligned(const void* aligned_ptr);
 BOAT_API void* boat_memory_reallocate(void* ptr, size_t new_size, boat_device_t device, const char* file, int line);
 BOAT_API void* boat_memory_allocate_device(size_t size, boat_device_t device, const char* file, int line);
 BOAT_API void boat_memory_free_device(void* ptr, boat_device_t device);
@@ -114,6 +118,8 @@ BOAT_API boat_error_t boat_get_last_error(void);
 BOAT_API const char* boat_get_last_error_message(void);
 BOAT_API void boat_set_error(boat_error_t error, const char* message);
 BOAT_API void boat_clear_error(void);
+BOAT_API void boat_set_errorf(boat_error_t error, const char* format, ...);
+BOAT_API void boat_reset_error(void);
 BOAT_API bool boat_has_error(void);
 
 /* ---- include/boat/ops.h:15-60 (the ops the backward pass is built from) ---- */
@@ -121,6 +127,7 @@ BOAT_API boat_tensor_t* boat_add(const boat_tensor_t* a, const boat_tensor_t* b)
 BOAT_API boat_tensor_t* boat_sub(const boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API boat_tensor_t* boat_mul(const boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API boat_tensor_t* boat_div(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_mod(const boat_tensor_t* a, const boat_tensor_t* b);   /* fmodf / fmod / % by element type (arithmetic.c:288-360) */
 BOAT_API void boat_add_(boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API void boat_sub_(boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API void boat_mul_(boat_tensor_t* a, const boat_tensor_t* b);
@@ -129,6 +136,12 @@ BOAT_API boat_tensor_t* boat_add_scalar(const boat_tensor_t* a, double scalar);
 BOAT_API boat_tensor_t* boat_sub_scalar(const boat_tensor_t* a, double scalar);
 BOAT_API boat_tensor_t* boat_mul_scalar(const boat_tensor_t* a, double scalar);
 BOAT_API boat_tensor_t* boat_div_scalar(const boat_tensor_t* a, double scalar);
+BOAT_API boat_tensor_t* boat_pow_scalar(const boat_tensor_t* a, double scalar);     /* float32 / float64 (arithmetic.c:486-518) */
+BOAT_API void boat_add_scalar_(boat_tensor_t* a, double scalar);
+BOAT_API void boat_sub_scalar_(boat_tensor_t* a, double scalar);
+BOAT_API void boat_mul_scalar_(boat_tensor_t* a, double scalar);
+BOAT_API void boat_div_scalar_(boat_tensor_t* a, double scalar);
+BOAT_API boat_tensor_t* boat_inverse(const boat_tensor_t* a);                       /* returns NULL, as the reference's stub (linear.c:409-413) */
 BOAT_API boat_tensor_t* boat_matmul(const boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API boat_tensor_t* boat_dot(const boat_tensor_t* a, const boat_tensor_t* b);
 BOAT_API boat_tensor_t* boat_transpose(const boat_tensor_t* a, int dim0, int dim1);
@@ -138,6 +151,7 @@ BOAT_API boat_tensor_t* boat_tanh(const boat_tensor_t* a);      /* stub in the r
 BOAT_API boat_tensor_t* boat_softmax(const boat_tensor_t* a, int axis);
 BOAT_API boat_tensor_t* boat_log_softmax(const boat_tensor_t* a, int axis);
 BOAT_API boat_tensor_t* boat_gelu(const boat_tensor_t* a);                          /* stub in the reference (src/ops/activation.c:298-302) */
+BOAT_API boat_tensor_t* boat_selu(const boat_tensor_t* a);                          /* returns NULL, as the reference's stub (activation.c:304-308) */
 BOAT_API boat_tensor_t* boat_sum(const boat_tensor_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
 BOAT_API boat_tensor_t* boat_mean(const boat_tensor_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
 
@@ -183,6 +197,8 @@ BOAT_API boat_variable_t* boat_var_softmax(const boat_variable_t* a, int axis);
 BOAT_API boat_variable_t* boat_var_log_softmax(const boat_variable_t* a, int axis);
 BOAT_API boat_variable_t* boat_var_sum(const boat_variable_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
 BOAT_API boat_variable_t* boat_var_mean(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim);
+BOAT_API boat_variable_t* boat_var_max(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim);   /* NULL, as in the reference (autodiff.c:595-603) */
+BOAT_API boat_variable_t* boat_var_min(const boat_variable_t* a, int64_t* dims, size_t n_dims, bool keepdim);
 /* include/boat/graph.h:18,41-43 and autodiff.h:87-88: an opaque handle that a context can carry for its caller.  The
  * graph IR itself (nodes, edges, traversal) is outside the training path and is not provided. */
 typedef struct boat_graph_t boat_graph_t;
@@ -284,6 +300,24 @@ BOAT_API boat_tensor_t* boat_layernorm_backward(boat_layernorm_t* norm, const bo
 BOAT_API void boat_layernorm_update(boat_layernorm_t* norm, float learning_rate);                          /* stub in the reference (norm.c:411-415) */
 BOAT_API void boat_layernorm_set_weight(boat_layernorm_t* norm, boat_tensor_t* weight);
 BOAT_API void boat_layernorm_set_bias(boat_layernorm_t* norm, boat_tensor_t* bias);
+/* RMSNorm (norm.h:28-32,42-46): y = x / (sqrtf(mean(x^2)) + eps) * weight, eps outside the root (norm.c:226,376);
+ * backward and update are stubs in the reference (norm.c:404-421) and work here like LayerNorm's */
+typedef struct boat_rmsnorm_t boat_rmsnorm_t;
+typedef struct {
+    size_t normalized_shape;
+    float eps;
+    bool elementwise_affine;
+} boat_rmsnorm_config_t;
+BOAT_API boat_rmsnorm_t* boat_rmsnorm_create(const boat_rmsnorm_config_t* config);
+BOAT_API void boat_rmsnorm_free(boat_rmsnorm_t* norm);
+BOAT_API boat_tensor_t* boat_rmsnorm_forward(boat_rmsnorm_t* norm, const boat_tensor_t* input);
+BOAT_API boat_tensor_t* boat_rmsnorm_backward(boat_rmsnorm_t* norm, const boat_tensor_t* grad_output);
+BOAT_API void boat_rmsnorm_update(boat_rmsnorm_t* norm, float learning_rate);
+/* stateless forms over the last dimension, no affine (NULL stubs in the reference, norm.c:424-463) */
+BOAT_API boat_tensor_t* boat_layer_norm(const boat_tensor_t* input, const int64_t* normalized_shape, size_t normalized_shape_len, float eps);
+BOAT_API boat_tensor_t* boat_rms_norm(const boat_tensor_t* input, const int64_t* normalized_shape, size_t normalized_shape_len, float eps);
+BOAT_API boat_tensor_t* boat_rms_norm_grad(const boat_tensor_t* grad_output, const boat_tensor_t* input, const boat_tensor_t* output,
+                                           const int64_t* normalized_shape, size_t normalized_shape_len, float eps);
 BOAT_API boat_tensor_t* boat_layer_norm_grad(const boat_tensor_t* grad_output, const boat_tensor_t* input, const boat_tensor_t* output,
                                              const int64_t* normalized_shape, size_t normalized_shape_len, float eps);  /* stub in the reference (norm.c:450-463) */
 BOAT_API boat_norm_layer_t* boat_norm_layer_create(size_t normalized_shape, float eps, bool elementwise_affine);
@@ -312,6 +346,16 @@ BOAT_API bool boat_attention_backward(boat_attention_t* attention, const boat_te
                                       boat_tensor_t** grad_query, boat_tensor_t** grad_key, boat_tensor_t** grad_value);
 BOAT_API void boat_attention_update(boat_attention_t* attention, float learning_rate);
 BOAT_API void boat_attention_set_causal(boat_attention_t* attention, bool causal);
+/* attention.h:63-76: the attention core on [batch, heads, seq, head_size] operands (attention.c:1082-1092), and
+ * self-attention through a throw-away layer (attention.c:830-880) */
+BOAT_API boat_tensor_t* boat_multihead_attention(const boat_tensor_t* input, size_t num_heads, float dropout_prob, bool causal_mask,
+                                                 const boat_tensor_t* attention_mask);
+BOAT_API boat_tensor_t* boat_scaled_dot_product_attention(const boat_tensor_t* query, const boat_tensor_t* key, const boat_tensor_t* value,
+                                                          float scale_factor, const boat_tensor_t* attention_mask, bool causal_mask,
+                                                          float dropout_prob);
+/* attention.h:79-90: not implemented in the reference (attention.c:1094-1120): NULL / no effect here too */
+BOAT_API boat_tensor_t* boat_rotary_position_encoding(const boat_tensor_t* tensor, size_t seq_len, size_t head_size, float theta);
+BOAT_API void boat_apply_rotary_embedding(boat_tensor_t* query, boat_tensor_t* key, size_t seq_len, size_t head_size, float theta);
 BOAT_API void boat_attention_set_dropout(boat_attention_t* attention, float dropout_prob);   /* stored, not applied (attention.c:1061-1062) */
 BOAT_API boat_tensor_t* boat_attention_get_weight_q(const boat_attention_t* attention);
 BOAT_API boat_tensor_t* boat_attention_get_weight_k(const boat_attention_t* attention);
@@ -391,6 +435,12 @@ BOAT_API boat_model_t* boat_model_create(void);
 BOAT_API void boat_model_free(boat_model_t* model);
 BOAT_API void boat_model_add_layer(boat_model_t* model, boat_layer_t* layer);
 BOAT_API size_t boat_model_layer_count(const boat_model_t* model);
+BOAT_API boat_model_t* boat_model_create_with_graph(const boat_graph_t* graph);   /* the model takes the graph over (model.c:59-83) */
+BOAT_API void boat_model_set_graph(boat_model_t* model, boat_graph_t* graph);
+BOAT_API void* boat_model_get_user_data(const boat_model_t* model);
+BOAT_API void boat_model_set_user_data(boat_model_t* model, void* user_data, void (*free_fn)(void*));
+BOAT_API boat_model_t* boat_model_load(const char* filename);                       /* NULL / false, as the reference's stubs (model.c:368-379) */
+BOAT_API bool boat_model_save(const boat_model_t* model, const char* filename);
 BOAT_API boat_graph_t* boat_model_graph(const boat_model_t* model);   /* model.h:42; the chain view declared with the tape's contexts above */
 BOAT_API boat_tensor_t* boat_model_forward(const boat_model_t* model, const boat_tensor_t* input);
 BOAT_API boat_tensor_t* boat_model_backward(const boat_model_t* model, const boat_tensor_t* grad_output);  /* stub in the reference (model.c:354-359) */
@@ -404,11 +454,24 @@ BOAT_API void boat_sequential_add(boat_sequential_model_t* model, boat_layer_t* 
 BOAT_API void boat_hip_synchronize(void);
 /* Coherent-pointer mode, for callers that keep the float* of boat_tensor_data() across calls, write through it before
  * a later call and read results through it afterwards (the reference's own tests do: test_attention_gradient_check.c:22-41,
- * test_optimizer_adam.c:96-108).  Off by default: a data pointer is then good until the next call that takes the
- * tensor, and parameters stay on the device.  On (this call, or BOAT_HIP_COHERENT_POINTERS=1 in the environment): a
- * tensor whose pointer was handed out is uploaded before every use and copied back after every call that writes it,
- * so such callers run unchanged, paying PCIe transfers for those tensors. */
+ * test_optimizer_adam.c:96-108; there the pointer is the tensor's storage).  ON by default: a tensor whose pointer was
+ * handed out is uploaded before every use and copied back after every call that writes it, so such callers run
+ * unchanged, paying PCIe transfers for those tensors.  Off (this call with 0, or BOAT_HIP_COHERENT_POINTERS=0 in the
+ * environment), for callers that fetch the pointer again after each call (as examples/mnist/mnist_autodiff.c does per
+ * batch): a data pointer is then good until the next call that takes the tensor, and parameters stay on the device. */
 BOAT_API void boat_hip_set_coherent_pointers(int enable);
+/* Reference-exact mode (this call, or BOAT_HIP_REFERENCE_EXACT=1 in the environment; off by default).  In three places
+ * this library computes something else than the reference on purpose; the mode switches all three to the reference's
+ * behaviour at once, for callers that need its numbers:
+ *   - boat_variable_backward walks the tape as the reference does (depth first, descending into a non-leaf variable once
+ *     per consumer with the gradient accumulated so far, src/autodiff.c:431-450): a non-leaf used twice propagates
+ *     twice (z = y + y, y = a*b gives da = 4b).  Default: every op once, the true gradient (2b).
+ *   - boat_conv_layer_backward returns the reference's input gradient, which pairs each kernel tap with the mirrored
+ *     weight (src/layers/conv.c:86-88).  Default: the gradient of the layer's own forward.
+ *     (boat_hip_conv_reference_input_grad, when called, overrides the mode for this one.)
+ *   - boat_autodiff_context_disable_grad is stored and ignored, as in the reference (src/autodiff.c:625-632).  Default:
+ *     ops run while the current context has gradients off are not recorded. */
+BOAT_API void boat_hip_set_reference_exact(int enable);
 /* gradient tensor of a variable, created zero-filled if absent and kept across boat_variable_zero_grad
  * (which then zero-fills in place), so it can be registered with an optimizer before the first backward */
 BOAT_API boat_tensor_t* boat_hip_variable_ensure_grad(boat_variable_t* variable);
@@ -423,6 +486,8 @@ BOAT_API boat_tensor_t* boat_hip_layernorm_get_weight(const boat_layernorm_t* no
 BOAT_API boat_tensor_t* boat_hip_layernorm_get_bias(const boat_layernorm_t* norm);
 BOAT_API boat_tensor_t* boat_hip_layernorm_get_grad_weight(const boat_layernorm_t* norm);
 BOAT_API boat_tensor_t* boat_hip_layernorm_get_grad_bias(const boat_layernorm_t* norm);
+BOAT_API boat_tensor_t* boat_hip_rmsnorm_get_weight(const boat_rmsnorm_t* norm);        /* the reference has no accessor or setter for it */
+BOAT_API boat_tensor_t* boat_hip_rmsnorm_get_grad_weight(const boat_rmsnorm_t* norm);
 /* fused loss + gradient of the tape chain log_softmax -> mul(onehot) -> sum -> mul(-1/B)
  * (examples/mnist/mnist_autodiff.c:397-522): labels is an INT32 or UINT8 tensor of class indices;
  * returns the [1] loss tensor and, through *dlogits, (softmax(z)-onehot)/B */
@@ -438,8 +503,9 @@ BOAT_API boat_layer_t* boat_hip_layer_gelu(void);
 /* register every trainable tensor of a layer with an optimizer */
 BOAT_API void boat_hip_optimizer_add_dense(boat_optimizer_t* opt, boat_dense_layer_t* layer);
 BOAT_API void boat_hip_optimizer_add_conv(boat_optimizer_t* opt, boat_conv_layer_t* layer);
-/* enable != 0: boat_conv_layer_backward returns the reference's input gradient (each tap paired with the mirrored
- * weight, src/layers/conv.c:86-88) instead of the true one; process-wide, off by default */
+/* enable > 0: boat_conv_layer_backward returns the reference's input gradient (each tap paired with the mirrored
+ * weight, src/layers/conv.c:86-88) instead of the true one; 0: the true one; < 0 (the initial state): whatever
+ * reference-exact mode says.  Process-wide. */
 BOAT_API void boat_hip_conv_reference_input_grad(int enable);
 BOAT_API void boat_hip_optimizer_add_attention(boat_optimizer_t* opt, boat_attention_t* attention);
 BOAT_API void boat_hip_optimizer_add_layernorm(boat_optimizer_t* opt, boat_layernorm_t* norm);

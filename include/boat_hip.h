@@ -88,6 +88,17 @@ int bh_activation_forward(int act, const float* x, float* y, int64_t n);        
  * accumulate!=0 adds into dx instead of assigning. */
 int bh_activation_backward(int act, const float* saved, const float* dy, float* dx, int64_t n, int accumulate);
 
+/* the reference's elementwise arithmetic on its other element types (src/ops/arithmetic.c:157-360 with boat_mod,
+ * :425-560 scalar ops and boat_pow_scalar): op 0 add, 1 sub, 2 mul, 3 div, 4 mod (fmodf / fmod / %), 5 pow (scalar form,
+ * float types only).  Shapes are right-aligned to ndim <= 8, numpy broadcasting.  An integer division by zero yields 0. */
+#define BH_DT_F32 0
+#define BH_DT_F64 1
+#define BH_DT_I32 2
+#define BH_DT_I64 3
+int bh_binary_typed(int dtype, int op, const void* a, const int64_t* a_shape, const void* b, const int64_t* b_shape,
+                    void* out, const int64_t* out_shape, int ndim);
+int bh_scalar_op_typed(int dtype, int op, const void* a, double scalar, void* out, int64_t n);
+
 int bh_bias_add_rows(float* y, const float* bias, int64_t rows, int64_t cols);        /* dense.c:180-184 */
 int bh_mse_grad(const float* pred, const float* target, float* grad, int64_t n);      /* tests/test_attention_training.c:28-41 */
 /* sum over the elements of the loss terms of the reference's loss objects (src/loss/mse.c, cross_entropy.c, huber.c):
@@ -117,6 +128,14 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy,
                           const float* mean, const float* rstd,
                           float* dx, float* dgamma, float* dbeta,
                           int64_t rows, int64_t hidden, int accumulate);
+
+/* ---- RMSNorm (forward: src/layers/norm.c:212-229,319-395; backward: stub there, :404-409) ----
+ * r = sqrtf(mean_h(x^2)), s = 1/(r + eps) (eps outside the root, as the reference), y = x*s*weight.  inv_rms (may be
+ * NULL) receives s per row.  backward: dx (assigned) and dweight (assigned unless accumulate) from the saved s;
+ * weight may be NULL (no scale). */
+int bh_rmsnorm_forward(const float* x, const float* weight, float* y, float* inv_rms, int64_t rows, int64_t hidden, float eps);
+int bh_rmsnorm_backward(const float* x, const float* weight, const float* dy, const float* inv_rms,
+                        float* dx, float* dweight, int64_t rows, int64_t hidden, float eps, int accumulate);
 
 /* bh_layernorm_backward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels and

@@ -416,6 +416,28 @@ void bo_layernorm_forward(const float* x, const float* gamma, const float* beta,
     }
 }
 
+/* src/layers/norm.c:212-229 (compute_rms) and :366-389 (apply) */
+void bo_rmsnorm_forward(const float* x, const float* weight, float* y, float* inv_rms,
+                        int64_t rows, int64_t hidden, float eps) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float* xr = x + r * hidden;
+        float* yr = y + r * hidden;
+        float sum_sq = 0.0f;
+        for (int64_t h = 0; h < hidden; h++) {
+            float val = xr[h];
+            sum_sq += val * val;
+        }
+        float rms = sqrtf(sum_sq / (float)(size_t)hidden);
+        float scale = 1.0f / (rms + eps);
+        for (int64_t h = 0; h < hidden; h++) {
+            float nrm = xr[h] * scale;
+            if (weight) nrm = nrm * weight[h];
+            yr[h] = nrm;
+        }
+        if (inv_rms) inv_rms[r] = scale;
+    }
+}
+
 /* -------------------------------------------------------------------- adam */
 
 /* src/optimizers/adam.c:203-222 */
@@ -631,6 +653,30 @@ void bo_layernorm_backward_f64(const float* x, const float* gamma, const float* 
                 double g = (double)gr[h] * (gamma ? (double)gamma[h] : 1.0);
                 dx[r * hidden + h] = rs * (g - s1 - xh * s2);
             }
+        }
+    }
+}
+
+/* y_j = x_j*w_j*s with s = 1/(r+eps), r = sqrt(mean_h x^2):
+ * dx_j = s*g_j - s^2 * (sum_i g_i x_i) * x_j/(H r)   (g = dy*w; the second term is absent for a row of zeros);
+ * dw_j = sum_rows dy_j x_j s */
+void bo_rmsnorm_backward_f64(const float* x, const float* weight, const float* dy, double* dx, double* dweight,
+                             int64_t rows, int64_t hidden, double eps) {
+    if (dweight) memset(dweight, 0, sizeof(double) * (size_t)hidden);
+    for (int64_t r = 0; r < rows; r++) {
+        const float* xr = x + r * hidden;
+        const float* gr = dy + r * hidden;
+        double sq = 0.0, gx = 0.0;
+        for (int64_t h = 0; h < hidden; h++) {
+            sq += (double)xr[h] * (double)xr[h];
+            gx += (double)gr[h] * (weight ? (double)weight[h] : 1.0) * (double)xr[h];
+        }
+        const double rms = sqrt(sq / (double)hidden);
+        const double s = 1.0 / (rms + eps);
+        for (int64_t h = 0; h < hidden; h++) {
+            const double g = (double)gr[h] * (weight ? (double)weight[h] : 1.0);
+            if (dx) dx[r * hidden + h] = s * g - (rms > 0.0 ? s * s * gx * (double)xr[h] / ((double)hidden * rms) : 0.0);
+            if (dweight) dweight[h] += (double)gr[h] * (double)xr[h] * s;
         }
     }
 }

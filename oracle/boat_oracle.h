@@ -10,8 +10,8 @@
  * vectors).
  *
  * Routines whose names end in _f64 have NO counterpart in the reference (the
- * reference ships stubs for them): LayerNorm backward, GELU forward/backward
- * and the MSE gradient.  They are double-precision closed forms, pinned by
+ * reference ships stubs for them): LayerNorm and RMSNorm backward, GELU
+ * forward/backward and the MSE gradient.  They are double-precision closed forms, pinned by
  * finite differences and by an independent autograd library's vectors, and
  * their parity with the reference is by construction "unpinned".
  *
@@ -104,6 +104,11 @@ void bo_attention_backward(const float* query, const float* key, const float* va
 void bo_layernorm_forward(const float* x, const float* gamma, const float* beta, float* y,
                           float* mean, float* rstd, int64_t rows, int64_t hidden, float eps);
 
+/* src/layers/norm.c:212-229 (rms = sqrtf(sum_sq / hidden)) and :366-389 (scale = 1/(rms + eps), then * weight).
+ * weight and inv_rms may be NULL; inv_rms receives the per-row scale. */
+void bo_rmsnorm_forward(const float* x, const float* weight, float* y, float* inv_rms,
+                        int64_t rows, int64_t hidden, float eps);
+
 /* src/optimizers/adam.c:180-223 for one tensor at the given (pre-increment)
  * timestep; the caller increments the timestep after all tensors (:226-240). */
 void bo_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
@@ -137,6 +142,10 @@ void bo_layernorm_backward_f64(const float* x, const float* gamma, const float* 
                                const float* mean, const float* rstd,
                                double* dx, double* dgamma, double* dbeta,
                                int64_t rows, int64_t hidden);
+/* RMSNorm backward (stub in the reference, src/layers/norm.c:404-409): derivative of y = x*w/(sqrt(mean(x^2)) + eps)
+ * in double precision, straight from x (no saved statistics) */
+void bo_rmsnorm_backward_f64(const float* x, const float* weight, const float* dy, double* dx, double* dweight,
+                             int64_t rows, int64_t hidden, double eps);
 void bo_gelu_forward_f64(const float* x, double* y, int64_t n);
 void bo_gelu_backward_f64(const float* x, const float* dy, double* dx, int64_t n);
 /* gradient of the mean-squared error, 2(o-t)/n, as tests/test_attention_training.c:28-41 writes it */

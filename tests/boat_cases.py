@@ -130,6 +130,23 @@ def fanout(api, a, b):
     return _grad(api, va), _grad(api, vb)
 
 
+def grad_under_disabled_context(api, a, b):
+    """y = a*b recorded while the current context has gradients switched off, then backward: the gradient of a, or None
+    when the op left no tape entry."""
+    ctx = api.boat_autodiff_context_create()
+    before = api.boat_autodiff_get_current_context()
+    api.boat_autodiff_set_current_context(ctx)
+    api.boat_autodiff_context_disable_grad(ctx)
+    va, vb = _var(api, a, True), _var(api, b, True)
+    vy = api.boat_var_mul(va, vb)
+    api.boat_variable_backward_full(vy)
+    g = api.boat_variable_grad(va)
+    out = api.numpy(g) if g else None
+    api.boat_autodiff_set_current_context(before)
+    api.boat_autodiff_context_free(ctx)
+    return out
+
+
 def _make_dense(api, w, b):
     layer = api.boat_dense_layer_create(w.shape[0], w.shape[1], b is not None)
     api.write(api.boat_dense_layer_get_weight(layer), w)      # in place, never set_weight (dangling optimizer pointers)
@@ -267,6 +284,67 @@ def layernorm_forward(api, x, gamma, beta, eps):
     api.boat_tensor_unref(tx)
     api.boat_layernorm_free(norm)
     return y
+
+
+def rmsnorm_forward(api, x, eps, affine=True):
+    """boat_rmsnorm_forward through the layer object (the reference offers no way to set the weight: it stays ones)."""
+    from boat_amd.capi import RmsNormConfig
+    x = np.asarray(x, np.float32)
+    cfg = RmsNormConfig(x.shape[-1], eps, affine)
+    norm = api.boat_rmsnorm_create(C.byref(cfg))
+    tx = api.tensor(x)
+    ty = api.boat_rmsnorm_forward(norm, tx)
+    y = api.numpy(ty)
+    api.boat_tensor_unref(ty)
+    api.boat_tensor_unref(tx)
+    api.boat_rmsnorm_free(norm)
+    return y
+
+
+def sdpa_public(api, q, k, v, scale, causal):
+    """boat_scaled_dot_product_attention on [batch, heads, seq, head_size] operands."""
+    ts = [api.tensor(np.asarray(a, np.float32)) for a in (q, k, v)]
+    to = api.boat_scaled_dot_product_attention(ts[0], ts[1], ts[2], scale, None, causal, 0.0)
+    out = api.numpy(to) if to else None
+    if to:
+        api.boat_tensor_unref(to)
+    for t in ts:
+        api.boat_tensor_unref(t)
+    return out
+
+
+def typed_arithmetic(api, a, b, scalar):
+    """The eager elementwise ops on tensors of a's dtype (float64 / int32 / int64 / float32): a dict of results.
+    b broadcasts against a; scalar is a Python float."""
+    out = {}
+    ta, tb = api.tensor(a), api.tensor(b)
+    for name in ("add", "sub", "mul", "div", "mod"):
+        t = getattr(api, f"boat_{name}")(ta, tb)
+        out[name] = api.numpy(t)
+        api.boat_tensor_unref(t)
+    for name in ("add", "sub", "mul", "div"):
+        t = getattr(api, f"boat_{name}_scalar")(ta, scalar)
+        out[f"{name}_scalar"] = api.numpy(t)
+        api.boat_tensor_unref(t)
+        tc = api.tensor(a)
+        getattr(api, f"boat_{name}_scalar_")(tc, scalar)
+        out[f"{name}_scalar_inplace"] = api.numpy(tc)
+        api.boat_tensor_unref(tc)
+    if a.shape == b.shape:
+        for name in ("add", "sub", "mul", "div"):
+            tc = api.tensor(a)
+            getattr(api, f"boat_{name}_")(tc, tb)
+            out[f"{name}_inplace"] = api.numpy(tc)
+            api.boat_tensor_unref(tc)
+    if a.dtype.kind == "f":
+        t = api.boat_pow_scalar(ta, scalar)
+        out["pow_scalar"] = api.numpy(t)
+        api.boat_tensor_unref(t)
+    else:
+        out["pow_scalar_is_null"] = np.array(not api.boat_pow_scalar(ta, scalar))
+    api.boat_tensor_unref(ta)
+    api.boat_tensor_unref(tb)
+    return out
 
 
 def attention(api, xq, xk, xv, weights, biases, heads, causal, d_out_list):

@@ -256,6 +256,46 @@ def main():
         save("mnist_synthetic", train_images=sets["train"][0], train_labels=sets["train"][1], test_images=sets["test"][0],
              test_labels=sets["test"][1], reference_lines=np.array(lines))
 
+    # ---- RMSNorm forward, the public attention core and the non-float32 elementwise ops (own generator: fixtures
+    # above keep their values when this block changes) ----
+    r5 = np.random.default_rng(20251125)
+    rn = {}
+    for tag, shape in (("a", (2, 5, 48)), ("b", (7, 64)), ("c", (32,)), ("d", (2, 3, 2, 8))):   # d: only 2*3 rows are visited
+        x = (r5.standard_normal(shape) * 10 ** r5.uniform(-2, 1)).astype(np.float32)
+        rn.update({f"{tag}_x": x, f"{tag}_y": bc.rmsnorm_forward(ref, x, 1e-6), f"{tag}_y_plain": bc.rmsnorm_forward(ref, x, 1e-3, affine=False)})
+    rn["zero_x"] = np.zeros((3, 8), np.float32)
+    rn["zero_y"] = bc.rmsnorm_forward(ref, rn["zero_x"], 1e-6)
+    save("rmsnorm_fwd", **rn)
+
+    sd = {}
+    for tag, (shape, causal) in (("a", ((2, 3, 16, 8), False)), ("b", ((1, 2, 40, 16), True)), ("c", ((2, 2, 64, 64), False))):
+        q, k, v = (r5.standard_normal(shape).astype(np.float32) for _ in range(3))
+        scale = float(1.0 / np.sqrt(np.float32(shape[-1])))
+        sd.update({f"{tag}_q": q, f"{tag}_k": k, f"{tag}_v": v, f"{tag}_scale": np.float32(scale), f"{tag}_causal": np.array(causal),
+                   f"{tag}_out": bc.sdpa_public(ref, q, k, v, scale, causal)})
+    sd["three_d_q"] = r5.standard_normal((2, 5, 8)).astype(np.float32)          # not 4-D: the reference hands back a copy of value
+    sd["three_d_v"] = r5.standard_normal((2, 5, 8)).astype(np.float32)
+    sd["three_d_out"] = bc.sdpa_public(ref, sd["three_d_q"], sd["three_d_q"], sd["three_d_v"], 0.5, False)
+    save("sdpa_public", **sd)
+
+    ty = {}
+    for tag, dt in (("f64", np.float64), ("i32", np.int32), ("i64", np.int64), ("f32", np.float32)):
+        if dt in (np.float64, np.float32):
+            a = (r5.standard_normal((4, 3, 5)) * 3).astype(dt)
+            b = (r5.standard_normal((3, 1)) + 2.5).astype(dt)
+            a2 = np.abs(a) + dt(0.25)
+        else:
+            a = r5.integers(-1000, 1000, (4, 3, 5)).astype(dt)
+            b = r5.integers(1, 37, (3, 1)).astype(dt) * np.where(r5.random((3, 1)) < 0.5, -1, 1).astype(dt)
+            a2 = a
+        same_shape_b = np.broadcast_to(b, a.shape).copy()
+        ty.update({f"{tag}_a": a, f"{tag}_b": b})
+        for key, val in bc.typed_arithmetic(ref, a, b, 2.75).items():
+            ty[f"{tag}_bc_{key}"] = val
+        for key, val in bc.typed_arithmetic(ref, a2, same_shape_b, -1.5 if dt in (np.float64, np.float32) else 3.0).items():
+            ty[f"{tag}_eq_{key}"] = val
+    save("typed_ops", **ty)
+
     # ---- not the reference: float64 autograd of an independent library ----
     import torch
     torch.manual_seed(0)
@@ -271,6 +311,17 @@ def main():
     y = torch.nn.functional.gelu(x, approximate="none")
     y.backward(dy)
     save("gelu_ref64", x=x.detach().numpy(), dy=dy.numpy(), y=y.detach().numpy(), dx=x.grad.numpy())
+    # RMSNorm as the reference defines it (eps outside the root), backward is a stub there
+    torch.manual_seed(1)
+    for tag, eps in (("a", 1e-6), ("b", 1e-2)):
+        x = (torch.randn(11, 96, dtype=torch.float64) * (0.05 if tag == "b" else 1.0)).requires_grad_()
+        w = (1 + 0.2 * torch.randn(96, dtype=torch.float64)).requires_grad_()
+        dy = torch.randn(11, 96, dtype=torch.float64)
+        y = x / (torch.sqrt((x * x).mean(-1, keepdim=True)) + eps) * w
+        y.backward(dy)
+        rm = {"x": x.detach().numpy(), "w": w.detach().numpy(), "dy": dy.numpy(), "y": y.detach().numpy(), "dx": x.grad.numpy(),
+              "dw": w.grad.numpy(), "eps": np.float64(eps)}
+        save(f"rmsnorm_bwd_ref64_{tag}", **rm)
 
 
 if __name__ == "__main__":

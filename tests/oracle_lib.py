@@ -205,6 +205,26 @@ class Oracle:
         self.lib.bo_layernorm_backward_f64(fp(x), fp(gamma), fp(dy), fp(mean), fp(rstd), dp(dx), dp(dg), dp(db), L(rows), L(h))
         return dx, dg, db
 
+    def rmsnorm_forward(self, x, weight, eps):
+        x = f32(x)
+        h = x.shape[-1]
+        rows = x.size // h
+        weight = None if weight is None else f32(weight)
+        y = np.empty_like(x)
+        inv = np.empty(rows, np.float32)
+        self.lib.bo_rmsnorm_forward(fp(x), fp(weight), fp(y), fp(inv), L(rows), L(h), C.c_float(eps))
+        return y, inv
+
+    def rmsnorm_backward_f64(self, x, weight, dy, eps):
+        x, dy = f32(x), f32(dy)
+        h = x.shape[-1]
+        rows = x.size // h
+        weight = None if weight is None else f32(weight)
+        dx = np.empty(x.shape, np.float64)
+        dw = np.empty(h, np.float64)
+        self.lib.bo_rmsnorm_backward_f64(fp(x), fp(weight), fp(dy), dp(dx), dp(dw), L(rows), L(h), C.c_double(eps))
+        return dx, dw
+
     def gelu_forward_f64(self, x):
         x = f32(x)
         y = np.empty(x.shape, np.float64)

@@ -33,6 +33,39 @@ def test_every_declared_symbol_is_exported(lib, header):
     assert not missing, f"declared in include/{header} but not exported: {missing}"
 
 
+def _reference_abi():
+    import json
+    return json.loads((ROOT / "tests" / "golden" / "reference_abi.json").read_text())
+
+
+def test_library_exports_what_the_reference_headers_declare(lib):
+    """tests/golden/reference_abi.json lists every function the REFERENCE's headers declare inside the line ranges that
+    include/boat_api.h cites (written by tests/golden/make_abi_list.py from the reference tree).  Whatever the reference
+    also defines must be exported here: a program that links against the reference must link against this library."""
+    abi = _reference_abi()
+    assert len(abi["functions"]) > 250
+    missing = [f"{f['name']} ({f['header']}:{f['line']})" for f in abi["functions"] if f["defined"] and not hasattr(lib, f["name"])]
+    assert not missing, f"declared and defined by the reference, not exported by libboat_amd.so: {missing}"
+
+
+def test_prototypes_match_the_reference_headers():
+    """Same list: every function of it that include/boat_api.h declares is declared with the reference's prototype
+    (return type and parameter types after removing export macros, parameter names and spacing), and every function
+    the reference defines is declared."""
+    import sys
+    sys.path.insert(0, str(ROOT / "tests" / "golden"))
+    import make_abi_list as m
+
+    ours = {name: proto for _, name, proto in m.declarations((ROOT / "include" / "boat_api.h").read_text())}
+    abi = _reference_abi()
+    # the ranges recorded in the list are the ones the header cites today
+    assert {h: [list(x) for x in s] for h, s in m.cited_ranges((ROOT / "include" / "boat_api.h").read_text()).items()} == abi["cited_ranges"]
+    undeclared = [f["name"] for f in abi["functions"] if f["defined"] and f["name"] not in ours]
+    assert not undeclared, f"defined by the reference inside the cited ranges, not declared in include/boat_api.h: {undeclared}"
+    different = [(f["prototype"], ours[f["name"]]) for f in abi["functions"] if f["name"] in ours and ours[f["name"]] != f["prototype"]]
+    assert not different, different
+
+
 def test_no_oracle_or_reference_symbols_in_the_product(lib):
     # the CPU checker must never be linked into the library under test
     for name in ("bo_matmul", "bo_adam_update", "bo_dense_backward"):

@@ -168,6 +168,92 @@ def test_oracle_layernorm_golden(oracle):
         assert same(y, g[f"{tag}_y"])
 
 
+def test_oracle_rmsnorm_golden(oracle):
+    g = load("rmsnorm_fwd")
+    for tag in "abc":
+        x = g[f"{tag}_x"]
+        assert same(oracle.rmsnorm_forward(x, np.ones(x.shape[-1], np.float32), 1e-6)[0], g[f"{tag}_y"]), tag
+        assert same(oracle.rmsnorm_forward(x, None, 1e-3)[0], g[f"{tag}_y_plain"]), tag
+    x = g["d_x"].reshape(-1, 8)                      # 4-D input: the reference visits shape0*shape1 = 6 rows only
+    y = g["d_y"].reshape(-1, 8)
+    assert same(oracle.rmsnorm_forward(x[:6], np.ones(8, np.float32), 1e-6)[0], y[:6]) and not y[6:].any()
+    assert not g["zero_y"].any() and not oracle.rmsnorm_forward(g["zero_x"], None, 1e-6)[0].any()
+
+
+def test_oracle_rmsnorm_backward_against_independent_library(oracle):
+    """The reference has no RMSNorm backward (stub, norm.c:404-409): the oracle's float64 closed form is pinned by float64
+    autograd vectors of an independent library for y = x/(sqrt(mean(x^2)) + eps)*w, at a small and at a large eps."""
+    for tag in "ab":
+        g = load(f"rmsnorm_bwd_ref64_{tag}")
+        x32, w32, dy32 = (g[k].astype(np.float32) for k in ("x", "w", "dy"))
+        dx, dw = oracle.rmsnorm_backward_f64(x32, w32, dy32, float(g["eps"]))
+        # inputs are rounded to float32 for the oracle: compare with that rounding's effect allowed for
+        assert close_max(dx, g["dx"], 1e-5) and close_max(dw, g["dw"], 1e-5), tag
+        y, _ = oracle.rmsnorm_forward(x32, w32, float(g["eps"]))
+        assert close_max(y, g["y"], 1e-5)
+    # dropping the second term of dx (the derivative of the scale) must fail the same check
+    g = load("rmsnorm_bwd_ref64_a")
+    s = 1 / (np.sqrt((g["x"] ** 2).mean(-1, keepdims=True)) + float(g["eps"]))
+    assert not close_max(s * g["dy"] * g["w"], g["dx"], 1e-3)
+
+
+def test_oracle_public_sdpa_golden(oracle):
+    g = load("sdpa_public")
+    for tag in "abc":
+        out, _, _ = oracle.sdpa_forward(g[f"{tag}_q"], g[f"{tag}_k"], g[f"{tag}_v"], float(g[f"{tag}_scale"]), bool(g[f"{tag}_causal"]))
+        assert same(out, g[f"{tag}_out"]), tag
+    assert same(g["three_d_out"], g["three_d_v"])
+
+
+def c_div(a, b):
+    """C's integer division truncates toward zero; numpy's // floors."""
+    q = np.abs(a) // np.abs(b)
+    return (q * np.sign(a) * np.sign(b)).astype(a.dtype)
+
+
+def typed_expectations(a, b, scalar):
+    """What one C operator per element gives (src/ops/arithmetic.c:197-282, 425-570), written with numpy."""
+    dt = a.dtype
+    s = dt.type(scalar)                                   # the scalar is narrowed to the element type first
+    is_f = dt.kind == "f"
+    want = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b if is_f else c_div(a, np.broadcast_to(b, a.shape)),
+            "mod": np.fmod(a, b),
+            "add_scalar": a + s, "sub_scalar": a - s, "mul_scalar": a * s, "div_scalar": a / s if is_f else c_div(a, np.full_like(a, s))}
+    for k in ("add", "sub", "mul", "div"):
+        want[f"{k}_scalar_inplace"] = want[f"{k}_scalar"]
+        if a.shape == b.shape:
+            want[f"{k}_inplace"] = want[k]
+    return {k: np.asarray(v, dt) for k, v in want.items()}
+
+
+def check_typed(get, tol_pow):
+    g = load("typed_ops")
+    for tag, dt in (("f64", np.float64), ("i32", np.int32), ("i64", np.int64), ("f32", np.float32)):
+        a, b = g[f"{tag}_a"], g[f"{tag}_b"]
+        assert a.dtype == dt
+        a2 = np.abs(a) + dt(0.25) if dt in (np.float64, np.float32) else a
+        for prefix, aa, bb, sc in (("bc", a, b, 2.75), ("eq", a2, np.broadcast_to(b, a.shape).copy(), -1.5 if a.dtype.kind == "f" else 3.0)):
+            got = get(tag, prefix, aa, bb, sc)
+            for key, want in typed_expectations(aa, bb, sc).items():
+                assert got[key].dtype == dt and np.array_equal(got[key], want), (tag, prefix, key)
+            if a.dtype.kind == "f":
+                with np.errstate(invalid="ignore"):
+                    pw = np.power(aa.astype(np.float64), dt(sc))
+                assert max_rel(got["pow_scalar"][np.isfinite(got["pow_scalar"])],
+                               pw[np.isfinite(got["pow_scalar"])]) <= tol_pow[tag], (tag, prefix)
+                assert np.array_equal(np.isnan(got["pow_scalar"]), np.isnan(pw))
+            else:
+                assert bool(got["pow_scalar_is_null"])
+
+
+def test_typed_arithmetic_fixture_is_one_c_operator_per_element():
+    """The non-float32 elementwise ops have no oracle routine: the expectation is numpy's IEEE / two's-complement operator
+    per element, and this test pins that expectation on what the compiled reference produced (tests/golden/typed_ops.npz)."""
+    g = load("typed_ops")
+    check_typed(lambda tag, prefix, a, b, s: {k[len(tag) + len(prefix) + 2:]: g[k] for k in g if k.startswith(f"{tag}_{prefix}_")},
+                {"f64": 1e-14, "f32": 1e-6})
+
+
 def test_oracle_adam_golden(oracle):
     g = load("adam_traj")
     for i in range(3):
@@ -358,6 +444,42 @@ def test_gpu_layernorm_golden(boat):
 
 
 @pytest.mark.gpu
+def test_gpu_rmsnorm_golden(boat):
+    g = load("rmsnorm_fwd")
+    for tag in "abcd":
+        assert close_max(bc.rmsnorm_forward(boat, g[f"{tag}_x"], 1e-6), g[f"{tag}_y"], TOL_RED), tag
+        assert close_max(bc.rmsnorm_forward(boat, g[f"{tag}_x"], 1e-3, affine=False), g[f"{tag}_y_plain"], TOL_RED), tag
+    assert not bc.rmsnorm_forward(boat, g["d_x"], 1e-6).reshape(-1, 8)[6:].any()     # rows the reference does not visit stay zero
+    assert not bc.rmsnorm_forward(boat, g["zero_x"], 1e-6).any()
+
+
+@pytest.mark.gpu
+def test_gpu_public_sdpa_golden(boat):
+    g = load("sdpa_public")
+    for tag in "abc":                                 # c has head size 64: the matrix-core kernel
+        out = bc.sdpa_public(boat, g[f"{tag}_q"], g[f"{tag}_k"], g[f"{tag}_v"], float(g[f"{tag}_scale"]), bool(g[f"{tag}_causal"]))
+        assert rel_fro(out, g[f"{tag}_out"]) <= TOL_GEMM and close_max(out, g[f"{tag}_out"], 1e-5), tag
+    assert same(bc.sdpa_public(boat, g["three_d_q"], g["three_d_q"], g["three_d_v"], 0.5, False), g["three_d_v"])
+
+
+@pytest.mark.gpu
+def test_gpu_typed_arithmetic_golden(boat):
+    """float64 / int32 / int64 (and float32 through the same entry points) elementwise ops, bit for bit against the
+    reference's results; pow within the tolerance of the device's pow routine."""
+    g = load("typed_ops")
+
+    def run(tag, prefix, a, b, s):
+        got = bc.typed_arithmetic(boat, a, b, s)
+        for key, val in got.items():
+            ref_val = g[f"{tag}_{prefix}_{key}"]
+            if key == "pow_scalar":
+                continue
+            assert np.array_equal(val, ref_val), (tag, prefix, key)
+        return got
+    check_typed(run, {"f64": 1e-13, "f32": 2e-6})
+
+
+@pytest.mark.gpu
 def test_gpu_adam_golden_bit_exact(boat):
     g = load("adam_traj")
     params = [g[f"p{i}"] for i in range(3)]
@@ -431,14 +553,14 @@ def test_gpu_conv_pool_cnn_golden(boat):
         for key in CNN_KEYS:
             assert close_max(rec[key], c[key], TOL_GEMM if key.startswith("g_w") else TOL_RED), key
     finally:
-        boat.boat_hip_conv_reference_input_grad(0)
+        boat.boat_hip_conv_reference_input_grad(-1)      # back to following reference-exact mode (off: the true gradient)
     # default mode = true gradient: equals the reference's operator applied to the turned kernel
     i = 0
     stride, pad = int(g[f"c{i}_meta"][6]), int(g[f"c{i}_meta"][7])
     x, w, b, dy = g[f"c{i}_x"], g[f"c{i}_w"], g[f"c{i}_b"], g[f"c{i}_dy1"]
     boat.boat_hip_conv_reference_input_grad(1)
     dx_ref_turned = bc.conv_layer(boat, x, np.ascontiguousarray(w[:, :, ::-1, ::-1]), b, stride, pad, [dy])[1][0][0]
-    boat.boat_hip_conv_reference_input_grad(0)
+    boat.boat_hip_conv_reference_input_grad(-1)
     dx_true = bc.conv_layer(boat, x, w, b, stride, pad, [dy])[1][0][0]
     assert same(dx_true, dx_ref_turned)
     pl = load("pool_layer")
@@ -453,6 +575,36 @@ def test_gpu_fanout_is_the_true_gradient_not_the_reference_value(boat):
     g = load("fanout_divergence")
     da, db = bc.fanout(boat, g["a"], g["b"])
     assert same(da, 2 * g["b"]) and same(db, 2 * g["a"])      # the reference reports 4b, 4a (see the fixture)
+
+
+@pytest.mark.gpu
+def test_gpu_reference_exact_mode(boat):
+    """boat_hip_set_reference_exact(1): the three deliberate divergences follow the reference at once -- the depth-first
+    walk that counts a non-leaf's fan-out once per consumer (fixture fanout_divergence), the mirrored-tap convolution
+    input gradient (fixtures conv_layer, cnn_chain) and the ignored disable_grad flag."""
+    from test_oracle_vs_reference import CNN_KEYS
+    f = load("fanout_divergence")
+    a, b = f["a"], f["b"]
+    assert bc.grad_under_disabled_context(boat, a, b) is None                 # default: not recorded, no gradient
+    boat.boat_hip_set_reference_exact(1)
+    try:
+        da, db = bc.fanout(boat, a, b)
+        assert same(da, f["ref_da"]) and same(db, f["ref_db"])                # 4b, 4a
+        assert same(bc.grad_under_disabled_context(boat, a, b), b)            # the flag is ignored: da = b
+        g = load("conv_layer")
+        for i in range(3):
+            stride, pad = int(g[f"c{i}_meta"][6]), int(g[f"c{i}_meta"][7])
+            y, calls = bc.conv_layer(boat, g[f"c{i}_x"], g[f"c{i}_w"], g[f"c{i}_b"], stride, pad, [g[f"c{i}_dy1"]])
+            assert same(y, g[f"c{i}_y"]) and close_max(calls[0][0], g[f"c{i}_dx0"], TOL_RED), i
+        c = load("cnn_chain")
+        x, labels, p = cnn_case(c)
+        rec = bc.cnn_ce_grads(boat, x, labels, p)                             # a chain: the depth-first walk visits each op once
+        for key in CNN_KEYS:
+            assert close_max(rec[key], c[key], TOL_GEMM if key.startswith("g_w") else TOL_RED), key
+    finally:
+        boat.boat_hip_set_reference_exact(0)
+    da, db = bc.fanout(boat, a, b)
+    assert same(da, 2 * b) and same(db, 2 * a)
 
 
 @pytest.mark.gpu

@@ -229,6 +229,132 @@ def test_layernorm_backward_hook(boat, oracle, rng):
     boat.boat_layernorm_free(norm)
 
 
+def test_rmsnorm_layer_hooks(boat, oracle, rng):
+    """boat_rmsnorm_*: forward as the reference (the oracle is bit-exact to it), backward and update implemented here
+    (stubs there, norm.c:404-421) and checked against the float64 closed form; the stateless forms agree with the layer."""
+    from boat_amd.capi import RmsNormConfig
+    x = rng.standard_normal((3, 5, 64)).astype(np.float32)
+    dy = rng.standard_normal((3, 5, 64)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    assert not boat.boat_rmsnorm_create(C.byref(RmsNormConfig(0, 1e-6, True)))          # norm.c:137-139
+    norm = boat.boat_rmsnorm_create(C.byref(RmsNormConfig(64, 1e-6, True)))
+    tx, tdy = boat.tensor(x), boat.tensor(dy)
+    assert not boat.boat_rmsnorm_backward(norm, tdy)                                      # before forward: NULL
+    assert not boat.boat_rmsnorm_forward(norm, boat.tensor(np.zeros((2, 63), np.float32)))   # wrong width: NULL (norm.c:333-335)
+    assert np.array_equal(boat.numpy(boat.boat_hip_rmsnorm_get_weight(norm)), np.ones(64, np.float32))
+    boat.write(boat.boat_hip_rmsnorm_get_weight(norm), w)
+    ty = boat.boat_rmsnorm_forward(norm, tx)
+    wy, _ = oracle.rmsnorm_forward(x, w, 1e-6)
+    assert np.max(np.abs(boat.numpy(ty) - wy)) <= TOL_RED * np.abs(wy).max()
+    wdx, wdw = oracle.rmsnorm_backward_f64(x, w, dy, 1e-6)
+    for call in (1, 2):                                                                   # the parameter gradient accumulates
+        tdx = boat.boat_rmsnorm_backward(norm, tdy)
+        assert np.max(np.abs(boat.numpy(tdx) - wdx)) <= TOL_RED * np.abs(wdx).max()
+        got = boat.numpy(boat.boat_hip_rmsnorm_get_grad_weight(norm))
+        assert np.max(np.abs(got - call * wdw)) <= call * TOL_RED * np.abs(wdw).max()
+        boat.boat_tensor_unref(tdx)
+    boat.boat_rmsnorm_update(norm, 0.5)                                                   # SGD step, then the gradient is cleared
+    assert np.max(np.abs(boat.numpy(boat.boat_hip_rmsnorm_get_weight(norm)) - (w - 0.5 * 2 * wdw))) <= 1e-3
+    assert not boat.numpy(boat.boat_hip_rmsnorm_get_grad_weight(norm)).any()
+    boat.boat_rmsnorm_free(norm)
+    # stateless forms: last dimension, no affine
+    shape = (C.c_int64 * 1)(64)
+    plain_y, _ = oracle.rmsnorm_forward(x, None, 1e-6)
+    t = boat.boat_rms_norm(tx, shape, 1, 1e-6)
+    assert np.max(np.abs(boat.numpy(t) - plain_y)) <= TOL_RED * np.abs(plain_y).max()
+    tg = boat.boat_rms_norm_grad(tdy, tx, t, shape, 1, 1e-6)
+    pdx, _ = oracle.rmsnorm_backward_f64(x, None, dy, 1e-6)
+    assert np.max(np.abs(boat.numpy(tg) - pdx)) <= TOL_RED * np.abs(pdx).max()
+    tl = boat.boat_layer_norm(tx, shape, 1, 1e-5)
+    ly, _, _ = oracle.layernorm_forward(x, None, None, 1e-5)
+    assert np.max(np.abs(boat.numpy(tl) - ly)) <= TOL_RED * np.abs(ly).max()
+    assert not boat.boat_rms_norm(tx, shape, 2, 1e-6) and not boat.boat_layer_norm(None, shape, 1, 1e-5)
+    for t_ in (t, tg, tl, ty, tx, tdy):
+        boat.boat_tensor_unref(t_)
+
+
+@pytest.mark.parametrize("shape,causal", [((2, 3, 16, 8), False), ((2, 2, 40, 16), True), ((2, 4, 128, 64), False), ((1, 2, 200, 64), True)])
+def test_public_attention_core(boat, oracle, rng, shape, causal):
+    """boat_scaled_dot_product_attention (attention.c:1082-1092) against the oracle's restatement of the same routine."""
+    q, k, v = (rng.standard_normal(shape).astype(np.float32) for _ in range(3))
+    scale = float(1.0 / np.sqrt(np.float32(shape[-1])))
+    out = bc.sdpa_public(boat, q, k, v, scale, causal)
+    want, _, _ = oracle.sdpa_forward(q, k, v, scale, causal)
+    assert out.shape == shape and rel_fro(out, want) <= TOL_GEMM and np.max(np.abs(out - want)) <= 1e-5
+    assert bc.sdpa_public(boat, q, k[:, :1], v, scale, causal) is None                    # shapes must agree (attention.c:929-933)
+
+
+def test_multihead_attention_is_a_throwaway_layer(boat, rng):
+    """boat_multihead_attention (attention.c:830-880) = create a layer with fresh rand() weights and bias, run self-attention,
+    free it: with the generator seeded the same way it must equal that sequence done by hand."""
+    import ctypes.util
+    from boat_amd.capi import AttentionConfig
+    libc = C.CDLL(ctypes.util.find_library("c"))
+    x = rng.standard_normal((2, 12, 32)).astype(np.float32)
+    tx = boat.tensor(x)
+    libc.srand(1234)
+    t = boat.boat_multihead_attention(tx, 4, 0.0, True, None)
+    got = boat.numpy(t)
+    libc.srand(1234)
+    att = boat.boat_attention_create(C.byref(AttentionConfig(32, 4, 8, 0.0, True, True, False, 10000.0)))
+    t2 = boat.boat_attention_forward(att, tx, tx, tx, None)
+    assert got.shape == x.shape and np.array_equal(got, boat.numpy(t2))
+    assert not boat.boat_multihead_attention(tx, 5, 0.0, False, None)                     # 32 % 5 != 0
+    assert not boat.boat_multihead_attention(boat.tensor(x[0]), 4, 0.0, False, None)      # not 3-D
+    boat.boat_attention_free(att)
+    for t_ in (t, t2, tx):
+        boat.boat_tensor_unref(t_)
+
+
+def test_symbols_that_are_stubs_in_the_reference_too(boat, rng):
+    """NULL / no effect in the reference (autodiff.c:595-603, attention.c:1094-1120, linear.c:409-413, activation.c:304-308,
+    model.c:368-379), the same here; plus the small host-side helpers of the cited header ranges."""
+    x = rng.standard_normal((2, 4, 8)).astype(np.float32)
+    tx = boat.tensor(x)
+    v = boat.boat_variable_create(tx, True)
+    dims = (C.c_int64 * 1)(0)
+    assert not boat.boat_var_max(v, dims, 1, False) and not boat.boat_var_min(v, dims, 1, False)
+    assert not boat.boat_rotary_position_encoding(tx, 4, 8, 10000.0)
+    boat.boat_apply_rotary_embedding(tx, tx, 4, 8, 10000.0)
+    assert np.array_equal(boat.numpy(tx), x)
+    assert not boat.boat_inverse(tx) and not boat.boat_selu(tx)
+    assert not boat.boat_model_load(b"/nonexistent") 
+    model = boat.boat_model_create()
+    assert boat.boat_model_save(model, b"/tmp/never_written.boat") is False
+    # user data travels with the model and its destructor runs once, at replacement or when the model is freed (model.c:382-397, 119-121)
+    from boat_amd.capi import FREE_FN
+    freed = []
+    cb = FREE_FN(lambda p: freed.append(p))
+    assert not boat.boat_model_get_user_data(model)
+    boat.boat_model_set_user_data(model, 0x1000, cb)
+    assert boat.boat_model_get_user_data(model) == 0x1000 and freed == []
+    boat.boat_model_set_user_data(model, 0x2000, cb)
+    assert freed == [0x1000]
+    boat.boat_model_free(model)
+    assert freed == [0x1000, 0x2000]
+    g = boat.boat_graph_create()
+    m2 = boat.boat_model_create_with_graph(g)
+    assert boat.boat_model_graph(m2) == g and not boat.boat_model_create_with_graph(None)
+    g2 = boat.boat_graph_create()
+    boat.boat_model_set_graph(m2, g2)                                                     # frees g, owns g2
+    assert boat.boat_model_graph(m2) == g2
+    boat.boat_model_free(m2)
+    # error state and aligned host blocks
+    boat.boat_set_error(3, b"x")
+    boat.boat_reset_error()
+    assert boat.boat_get_last_error() == 0
+    p = boat.boat_memory_allocate_aligned(100, 256, 0, b"t", 1)
+    assert p and p % 256 == 0
+    C.memset(p, 7, 100)
+    boat.boat_memory_free_aligned(p)
+    block = C.c_void_p(boat.boat_memory_allocate(64, 0, b"t", 2))
+    boat.boat_memory_free_safe(C.byref(block))
+    assert block.value is None
+    boat.boat_memory_free_safe(C.byref(block))                                            # NULL inside: nothing happens
+    boat.boat_variable_free(v)
+    boat.boat_tensor_unref(tx)
+
+
 @pytest.mark.parametrize("case", ATT_CASES, ids=lambda c: f"B{c['B']}S{c['S']}H{c['H']}{'c' if c['causal'] else ''}{'b' if c['bias'] else ''}")
 def test_attention_layer(boat, oracle, case):
     xs, w, b, dys = make_attention_inputs(case, 99)

@@ -309,6 +309,31 @@ def test_layernorm_backward(hip, oracle, rng, rows, hidden):
     assert np.max(np.abs(db.numpy() - 2 * wdb)) <= 2 * TOL_RED * max(1.0, np.abs(wdb).max())
 
 
+@pytest.mark.parametrize("rows,hidden", LN_SHAPES + [(1000, 1024), (300, 4096)])
+def test_rmsnorm_forward_backward(hip, oracle, rng, rows, hidden):
+    """RMSNorm (eps outside the root, src/layers/norm.c:212-229,366-389): forward against the oracle's fp32 restatement,
+    backward (a stub in the reference) against the float64 closed form; the LayerNorm tolerance applies."""
+    x = (rng.standard_normal((rows, hidden)) * 10 ** rng.uniform(-1, 1)).astype(np.float32)
+    x[0] = 0.0                                       # a row of zeros: scale 1/eps, output and gradient term stay finite
+    w = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    dy = rng.standard_normal((rows, hidden)).astype(np.float32)
+    for eps, weight in ((1e-6, w), (1e-2, None)):
+        dw_ = None if weight is None else dev(hip, weight).ptr
+        y, inv = hip.empty((rows, hidden)), hip.empty(rows)
+        hip.check(hip.bh_rmsnorm_forward(dev(hip, x).ptr, dw_, y.ptr, inv.ptr, rows, hidden, eps))
+        wy, winv = oracle.rmsnorm_forward(x, weight, eps)
+        assert np.max(np.abs(y.numpy() - wy)) <= TOL_RED * max(np.abs(wy).max(), 1e-30)
+        assert max_rel(inv.numpy(), winv) <= TOL_RED
+        dx, dg = hip.empty((rows, hidden)), hip.zeros(hidden)
+        args = (dev(hip, x).ptr, dw_, dev(hip, dy).ptr, dev(hip, winv).ptr)
+        hip.check(hip.bh_rmsnorm_backward(*args, dx.ptr, dg.ptr, rows, hidden, eps, 0))
+        wdx, wdw = oracle.rmsnorm_backward_f64(x, weight, dy, eps)
+        assert np.max(np.abs(dx.numpy() - wdx)) <= TOL_RED * np.abs(wdx).max()
+        assert np.max(np.abs(dg.numpy() - wdw)) <= TOL_RED * max(1.0, np.abs(wdw).max())
+        hip.check(hip.bh_rmsnorm_backward(*args, dx.ptr, dg.ptr, rows, hidden, eps, 1))
+        assert np.max(np.abs(dg.numpy() - 2 * wdw)) <= 2 * TOL_RED * max(1.0, np.abs(wdw).max())
+
+
 # --------------------------------------------------------------------- gemm
 
 def gemm_case(hip, rng, ta, tb, m, n, k, accumulate=False, bias=False, batch=1, force=None, direct=None):

@@ -258,6 +258,57 @@ def test_layernorm_forward_bit_exact(ref, oracle, rng, shape):
     assert np.allclose(mean, mu.ravel(), atol=1e-6) and np.allclose(rstd, 1 / np.sqrt(var.ravel() + 1e-5), rtol=1e-5)
 
 
+def test_reference_ignores_a_contexts_disabled_grad_flag(ref):
+    # src/autodiff.c:625-632 stores the flag; nothing reads it: the op is recorded and backward reaches the leaf
+    a, b = np.array([1.5, -2.0], np.float32), np.array([3.0, 0.5], np.float32)
+    assert same(bc.grad_under_disabled_context(ref, a, b), b)
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 48), (7, 64), (4, 768), (33,)])
+def test_rmsnorm_forward_bit_exact(ref, oracle, rng, shape):
+    # src/layers/norm.c:212-229,319-395: eps is added to the root, not under it
+    x = (rng.standard_normal(shape) * 10 ** rng.uniform(-2, 1)).astype(np.float32)
+    for eps, affine in ((1e-6, True), (1e-2, False)):
+        y = bc.rmsnorm_forward(ref, x, eps, affine)
+        o_y, inv = oracle.rmsnorm_forward(x, np.ones(shape[-1], np.float32) if affine else None, eps)
+        assert same(o_y, y)
+        xd = x.astype(np.float64).reshape(-1, shape[-1])
+        want = xd / (np.sqrt((xd * xd).mean(-1, keepdims=True)) + eps)
+        assert np.allclose(y.reshape(want.shape), want, rtol=2e-6, atol=1e-7)
+        assert np.allclose(inv, 1 / (np.sqrt((xd * xd).mean(-1)) + eps), rtol=2e-6)
+        # had eps been under the root the rows would differ by far more than rounding at eps = 1e-2
+        wrong = xd / np.sqrt((xd * xd).mean(-1, keepdims=True) + eps)
+        if eps == 1e-2:
+            assert np.max(np.abs(wrong - want)) > 1e-4
+
+
+def test_rmsnorm_rows_the_reference_visits(ref, oracle, rng):
+    # norm.c:360-362: a 4-D input is treated as [shape0, shape1, hidden]: only the first shape0*shape1 rows are written
+    x = rng.standard_normal((2, 3, 2, 8)).astype(np.float32)
+    y = bc.rmsnorm_forward(ref, x, 1e-6)
+    o_y, _ = oracle.rmsnorm_forward(x.reshape(-1, 8)[:6], np.ones(8, np.float32), 1e-6)
+    assert same(y.reshape(-1, 8)[:6], o_y) and not y.reshape(-1, 8)[6:].any()
+
+
+@pytest.mark.parametrize("shape,causal", [((2, 3, 16, 8), False), ((1, 2, 40, 16), True), ((1, 1, 5, 4), True)])
+def test_public_sdpa_bit_exact(ref, oracle, rng, shape, causal):
+    # boat_scaled_dot_product_attention (attention.c:1082-1092) is the routine the layer's forward runs per head
+    q, k, v = (rng.standard_normal(shape).astype(np.float32) for _ in range(3))
+    scale = float(1.0 / np.sqrt(np.float32(shape[-1])))
+    out = bc.sdpa_public(ref, q, k, v, scale, causal)
+    o_out, _, attn = oracle.sdpa_forward(q, k, v, scale, causal)
+    assert same(o_out, out)
+    # textbook softmax(scale*QK^T)V in float64
+    sc = np.einsum("bhid,bhjd->bhij", q.astype(np.float64), k.astype(np.float64)) * scale
+    if causal:
+        sc = np.where(np.triu(np.ones(sc.shape[-2:], bool), 1), -np.inf, sc)
+    pr = np.exp(sc - sc.max(-1, keepdims=True))
+    pr /= pr.sum(-1, keepdims=True)
+    assert np.allclose(out, pr @ v.astype(np.float64), atol=2e-6)
+    # operands that are not 4-D come back as a copy of value (attention.c:905-917)
+    assert same(bc.sdpa_public(ref, q[0], k[0], v[0], scale, causal), v[0])
+
+
 def test_layernorm_pattern_input(ref, oracle):
     # tests/test_layernorm_simple.c: pattern (i % 10) * 0.1, H = 768, eps 1e-5
     x = ((np.arange(2 * 3 * 768) % 10) * 0.1).astype(np.float32).reshape(2, 3, 768)

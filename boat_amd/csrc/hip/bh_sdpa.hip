@@ -334,6 +334,9 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
         int done = 1;
         if (!g_sdpa_force_general)
             done = sdpa_backward_mfma(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);
+        // the matrix-core kernel's dQ workspace grows with s^2: when it cannot be had, the GEMM-based path, whose
+        // [s, s] matrices are held for a bounded chunk of heads at a time, takes the shape
+        if (done == BH_ENOMEM && s >= 64 && s <= 16384) done = 1;
         if (done < 0) rc = done;
         if (done == 1 && (g_sdpa_force_general == 2 || (g_sdpa_force_general == 0 && s >= 64 && s <= 16384))) {
             rc = sdpa_backward_gemm(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);

@@ -51,5 +51,6 @@ def boat(hip):
 
 @pytest.fixture
 def rng(request):
-    seed = abs(hash(request.node.name)) % (2**31)
+    import zlib
+    seed = zlib.crc32(request.node.nodeid.encode()) % (2**31)     # the same data in every run (str hashes change per process)
     return np.random.default_rng(seed)

@@ -337,3 +337,19 @@ def max_rel(a, b, floor=1e-30):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor))) if a.size else 0.0
+
+
+def fp32_gemm_bound(k):
+    """Relative Frobenius error that a contraction of length k keeps when products and sums are carried in full fp32
+    (about 6e-8 * sqrt(k) / 3 for a sequential sum, less for blocked ones); an operand or accumulator narrowed to 10 or 7
+    mantissa bits (tf32, bf16) lands near 3e-4 and 2e-3 and fails it."""
+    return max(2e-6, 1.5e-7 * float(np.sqrt(k)))
+
+
+FP32_ATTENTION_BOUND = 2e-5    # attention outputs and gradients against the fp32 oracle: two rounding paths of about 1e-6 each
+
+
+def narrow_mantissa(a, bits):
+    """float32 values truncated to `bits` explicit mantissa bits (7 = bf16, 10 = tf32 / fp16)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    return (u & np.uint32(0xFFFFFFFF << (23 - bits) & 0xFFFFFFFF)).view(np.float32)

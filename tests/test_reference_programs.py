@@ -17,7 +17,6 @@ from pathlib import Path
 
 import pytest
 
-pytestmark = pytest.mark.gpu
 
 BIN = Path(__file__).resolve().parent.parent / "oracle" / "_ref" / "reftests"
 
@@ -51,6 +50,7 @@ def run(name, tmp_path):
     return subprocess.run([str(exe)], cwd=tmp_path, env=env, capture_output=True, text=True, errors="replace", timeout=100)
 
 
+@pytest.mark.gpu
 @pytest.mark.parametrize("name", sorted(PASSING))
 def test_reference_program_passes_on_this_library(name, tmp_path):
     proc = run(name, tmp_path)
@@ -60,6 +60,7 @@ def test_reference_program_passes_on_this_library(name, tmp_path):
     assert "FAILED" not in proc.stdout
 
 
+@pytest.mark.gpu
 def test_gradient_check_program_reports_what_it_reports_on_the_reference(tmp_path):
     """tests/unit/test_gradient_check.c compares analytical gradients with float32 central differences at a tolerance
     the differences do not meet: on the compiled reference it passes addition and reports two mismatches for
@@ -76,6 +77,7 @@ def test_gradient_check_program_reports_what_it_reports_on_the_reference(tmp_pat
     assert "FAILED: 2 mismatches" in out
 
 
+@pytest.mark.gpu
 def test_optimizer_benchmark_of_the_reference_reports_the_same_losses(tmp_path):
     """benchmarks/linear_regression.c: 1000 steps each with Adam, Adam + StepLR, RMSprop and Adagrad on synthetic data
     from rand().  It registers boat_variable_grad() before the first backward, when that is still NULL
@@ -88,6 +90,7 @@ def test_optimizer_benchmark_of_the_reference_reports_the_same_losses(tmp_path):
     assert len(rows) == 4 and all("1.273380" in r for r in rows), summary
 
 
+@pytest.mark.gpu
 def test_scheduler_example_prints_the_learning_rates_it_prints_on_the_reference(tmp_path):
     """examples/scheduler_usage.c (step, cosine and caller-function schedules driving Adam and RMSprop): its
     learning-rate lines on this library are, character for character, the lines it printed on the compiled reference
@@ -100,11 +103,13 @@ def test_scheduler_example_prints_the_learning_rates_it_prints_on_the_reference(
     assert got == want and len(want) > 40
 
 
+@pytest.mark.gpu
 def test_relu_example_of_the_reference(tmp_path):
     proc = run("test_relu", tmp_path)
     assert proc.returncode == 0 and "Result data: 0.0 0.0 0.0 0.0 1.0 2.0" in proc.stdout, proc.stdout[-500:]
 
 
+@pytest.mark.gpu
 @pytest.mark.parametrize("coherent", ["1", "0"])
 def test_mnist_example_of_the_reference_trains_as_on_the_reference(tmp_path, coherent):
     """examples/mnist/mnist.c, the layer-hook training loop (conv, pool, dense, softmax; forward, backward and update
@@ -130,6 +135,7 @@ def test_mnist_example_of_the_reference_trains_as_on_the_reference(tmp_path, coh
     assert lines == [str(line) for line in g["reference_lines"]] and len(lines) == 6
 
 
+@pytest.mark.gpu
 def test_attention_benchmark_of_the_reference_runs(tmp_path):
     """benchmarks/attention_performance.c (B4 S16 H64, 8 heads, causal; 50 forward and backward passes through
     boat_attention_forward / boat_attention_backward): runs to its report on this library."""
@@ -139,5 +145,7 @@ def test_attention_benchmark_of_the_reference_runs(tmp_path):
 
 
 def test_zz_scheduler_program_stops_where_it_stops_on_the_reference(tmp_path):
+    """tests/unit/test_schedulers.c fails a host assert of its own (:56) on the reference as well, before it creates a
+    tensor: no GPU is involved, so this test carries no gpu mark."""
     proc = run("test_schedulers", tmp_path)
     assert proc.returncode == -6 and "test_schedulers.c:56" in proc.stderr, (proc.returncode, proc.stderr[-500:])

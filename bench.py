@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the training hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--legs ...]
 
-A step is one dense-layer backward at benchmark configuration 2 (the GEMM-bound configuration the
-metric is quoted on): X[8192x4096] ~N(0,1), W[4096x4096] ~N(0,0.02), dY[8192x4096] ~N(0,1);
-dX = dY.W^T, dW += X^T.dY, db += colsum(dY) -- the three launches bh_dense_backward makes,
-issued here one by one so that HIP events on the library stream can time the GEMM launches
-inside the timed region.  Inputs are resident in HBM before timing starts.
+A step is benchmark configuration 5, the one configuration that is literally "backward + Adam step": one training
+step of a pre-LN transformer encoder block (d_model 1024, 16 heads, FFN 4096 with GELU, seq 512, batch 16: forward,
+boat_variable_backward, fused Adam over the block's 12,596,224 parameters, zero_grad) driven through Boat's C API,
+followed by the standalone fused Adam over 268,435,456 flat fp32 parameters.  Inputs, weights, gradients and moments
+are resident in HBM before timing starts; the K timed steps are bracketed by HIP events on the library stream.
 
-Prints ONE JSON line: the step time in ms (value), the roofline of the dominant kernel
-(fp32 MFMA GEMM: algorithmic 2*M*K*N flops per launch / measured average launch duration,
-against the 157.3 TFLOP/s fp32-MFMA peak), the CPU baseline (the compiled reference's
-boat_dense_layer_backward, or the oracle port when the reference library is absent, timed on
-one host core on a bounded sample and scaled by flops), and -- under "extra" -- the other
-configurations of the path with their own roofline fractions.
+Prints ONE JSON line: the step time in ms (value); the roofline of the dominant kernel family (the fp32-MFMA GEMM
+launches of the step: their algorithmic 2*m*n*k flops / their durations, both summed over the timed region, each launch
+bracketed by HIP events through bh_profile_enable, against the 157.3 TFLOP/s fp32-MFMA peak); the CPU baseline (the
+compiled reference's routines timed on one host core on a bounded sample and scaled by flops and by element count);
+and -- under "extra" -- the step's breakdown and the other configurations of the path with their own roofline fractions.
+
+The library keeps host pointers coherent by default (what an unchanged Boat caller needs); the legs that run through
+Boat's API switch that off (boat_hip_set_coherent_pointers(0)), as a training loop that fetches pointers per batch
+would, so that parameters stay resident in HBM.
 """
 from __future__ import annotations
 
@@ -35,10 +38,11 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 PEAK_FP32_MFMA_TFLOPS = 157.3
 METRIC = "backward+Adam step ms; GB/s & TFLOP/s as % of MI355X roofline (1 GPU)"
 
-# HBM bytes per GEMM launch (average of the dX and dW launches of a step) measured with rocprofv3 --pmc:
+# HBM bytes per GEMM launch of configuration 2 (average of its dX and dW launches) measured with rocprofv3 --pmc:
 # FETCH_SIZE 409,880 KiB x 2.000 + WRITE_SIZE 98,304 KiB x 1.000, the factors being what the same counters read for
-# a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).
-GEMM_TRAFFIC_BYTES = int((2.0 * 409880.2 + 98304.0) * 1024)
+# a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).  A constant taken from that profile, not a
+# measurement of this run.
+GEMM_TRAFFIC_BYTES_CONFIG2 = int((2.0 * 409880.2 + 98304.0) * 1024)
 
 
 def parse_args():
@@ -49,8 +53,8 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="all",
-                    help="comma list of dense,adam,ln_gelu,sdpa,mlp,cnn,block (default all); for profiling one workload at a time. "
-                         "Without the dense leg the line carries no value/roofline.")
+                    help="comma list of step,dense,adam,ln_gelu,sdpa,mlp,cnn (default all); for profiling one workload at a time. "
+                         "Without the step leg the line carries no value/roofline.")
     return ap.parse_args()
 
 
@@ -134,7 +138,7 @@ def bench_dense_backward(hip, steps, warmup):
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(gemm_launch_ms, 4), "flops_per_launch": flops_per_launch,
-            "traffic": GEMM_TRAFFIC_BYTES,
+            "traffic": GEMM_TRAFFIC_BYTES_CONFIG2, "traffic_source": "profile constant (profiles/pmc_hbm_traffic_and_mfma.md), not measured in this run",
         },
         "step_tflops": round(2 * flops_per_launch / (ms_per_step * 1e-3) / 1e12, 2),
     }
@@ -263,18 +267,31 @@ def bench_sdpa(hip, steps, warmup):
 
 def bench_mlp_step(steps, warmup):
     """Config 1 through Boat's C API from a C program (boat_amd/examples/mlp_train_step.c, built beside the library):
-    forward + boat_variable_backward_full + boat_optimizer_step + zero_grad per step, wall ms measured inside it."""
+    forward + boat_variable_backward_full + boat_optimizer_step + zero_grad per step, wall ms measured inside it.
+    Three runs: the op-by-op loss chain with parameters resident (BOAT_HIP_COHERENT_POINTERS=0), the same with the
+    four-op loss chain replaced by the fused softmax + cross-entropy kernel, and the chain in the library's default
+    configuration (every tensor whose pointer the program once held is kept coherent with the host on every call)."""
     import subprocess
     exe = ROOT / "boat_amd" / "lib" / "mlp_train_step"
     if not exe.exists():
         raise FileNotFoundError(f"{exe} not found: build it first (python -m boat_amd.build)")
-    out = subprocess.run([str(exe), str(steps), str(warmup)], check=True, capture_output=True, text=True).stdout
-    rec = json.loads(out.strip().splitlines()[-1])
-    assert rec["loss_last"] < rec["loss_first"], f"MLP training does not reduce the loss: {rec}"
-    return {"ms": round(rec["ms_per_step"], 4), "bound": "launch latency", "steps": rec["steps"],
-            "loss_first_last": [rec["loss_first"], rec["loss_last"]],
+
+    def run(coherent, *extra):
+        env = dict(os.environ, BOAT_HIP_COHERENT_POINTERS=coherent)
+        out = subprocess.run([str(exe), str(steps), str(warmup), *extra], check=True, capture_output=True, text=True, env=env).stdout
+        rec = json.loads(out.strip().splitlines()[-1])
+        assert rec["loss_last"] < rec["loss_first"], f"MLP training does not reduce the loss: {rec}"
+        return rec
+
+    chain, fused, default = run("0"), run("0", "fused"), run("1")
+    return {"ms": round(chain["ms_per_step"], 4), "bound": "launch latency", "steps": chain["steps"],
+            "ms_fused_softmax_cross_entropy": round(fused["ms_per_step"], 4),
+            "ms_default_coherent_pointers": round(default["ms_per_step"], 4),
+            "loss_first_last": [chain["loss_first"], chain["loss_last"]],
+            "loss_first_last_fused": [fused["loss_first"], fused["loss_last"]],
             "note": "MLP 784-128-10 B64 fwd+bwd+Adam+zero_grad through boat_var_* / boat_variable_backward_full / "
-                    "boat_optimizer_step, a C caller linked against libboat_amd.so, wall clock"}
+                    "boat_optimizer_step, a C caller linked against libboat_amd.so, wall clock; 'fused' replaces log_softmax, "
+                    "mul(onehot), sum, mul(-1/B) and their backward by boat_hip_softmax_cross_entropy"}
 
 
 def bench_cnn_step(steps, warmup):
@@ -283,6 +300,7 @@ def bench_cnn_step(steps, warmup):
     forward + boat_variable_backward_full + Adam + zero_grad, wall ms."""
     from boat_amd.capi import default_api
     api = default_api()
+    api.boat_hip_set_coherent_pointers(0)       # weights written below stay resident in HBM afterwards
     rng = np.random.default_rng(20250107)
     B, classes = 64, 10
     x = rng.random((B, 1, 28, 28), dtype=np.float32)
@@ -352,87 +370,176 @@ def bench_cnn_step(steps, warmup):
                     "C API from Python, wall clock"}
 
 
-def bench_block_step(steps, warmup):
+class Block:
     """Config 5a through Boat's C API: pre-LN encoder block d_model 1024, 16 heads, FFN 4096 (GELU), seq 512, batch 16;
-    forward + boat_variable_backward + fused Adam over the block's 12,596,224 parameters (16 tensors), wall ms."""
-    from boat_amd.capi import AttentionConfig, LayerNormConfig, default_api
-    api = default_api()
-    rng = np.random.default_rng(20250105)
+    step() = forward + boat_variable_backward + fused Adam over the block's 12,596,224 parameters (16 tensors) + zero_grad."""
     B, S, H, heads, ffn = 16, 512, 1024, 16, 4096
-    T = B * S
 
-    def normal(shape, std):
-        return (std * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
+    def __init__(self):
+        from boat_amd.capi import AttentionConfig, LayerNormConfig, default_api
+        self.api = api = default_api()
+        api.boat_hip_set_coherent_pointers(0)       # parameters written below stay resident in HBM afterwards
+        rng = np.random.default_rng(20250105)
+        B, S, H, heads, ffn = self.B, self.S, self.H, self.heads, self.ffn
 
-    ln = []
-    for _ in range(2):
-        cfg = LayerNormConfig(H, 1e-5, True, True)
-        ln.append(api.boat_layernorm_create(C.byref(cfg)))          # gamma = 1, beta = 0
-    cfg = AttentionConfig(H, heads, H // heads, 0.0, False, True, False, 10000.0)
-    att = api.boat_attention_create(C.byref(cfg))
-    for n in "qkvo":
-        api.write(getattr(api, f"boat_attention_get_weight_{n}")(att), normal((H, H), 0.02))
-    d1 = api.boat_dense_layer_create(H, ffn, True)
-    d2 = api.boat_dense_layer_create(ffn, H, True)
-    api.write(api.boat_dense_layer_get_weight(d1), normal((H, ffn), 0.02))
-    api.write(api.boat_dense_layer_get_weight(d2), normal((ffn, H), 0.02))
-    opt = api.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
-    api.boat_hip_optimizer_add_layernorm(opt, ln[0])
-    api.boat_hip_optimizer_add_attention(opt, att)
-    api.boat_hip_optimizer_add_layernorm(opt, ln[1])
-    api.boat_hip_optimizer_add_dense(opt, d1)
-    api.boat_hip_optimizer_add_dense(opt, d2)
-    tx = api.tensor(normal((B, S, H), 1.0))
-    tt = api.tensor(normal((B, S, H), 1.0))
-    shape2 = (C.c_int64 * 2)(T, H)
-    shape3 = (C.c_int64 * 3)(B, S, H)
-    losses = []
+        def normal(shape, std):
+            return (std * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
 
-    def step(keep_loss=False):
-        vx = api.boat_variable_create(tx, True)
+        self.ln = []
+        for _ in range(2):
+            cfg = LayerNormConfig(H, 1e-5, True, True)
+            self.ln.append(api.boat_layernorm_create(C.byref(cfg)))          # gamma = 1, beta = 0
+        cfg = AttentionConfig(H, heads, H // heads, 0.0, False, True, False, 10000.0)
+        self.att = api.boat_attention_create(C.byref(cfg))
+        for n in "qkvo":
+            api.write(getattr(api, f"boat_attention_get_weight_{n}")(self.att), normal((H, H), 0.02))
+        self.d1 = api.boat_dense_layer_create(H, ffn, True)
+        self.d2 = api.boat_dense_layer_create(ffn, H, True)
+        api.write(api.boat_dense_layer_get_weight(self.d1), normal((H, ffn), 0.02))
+        api.write(api.boat_dense_layer_get_weight(self.d2), normal((ffn, H), 0.02))
+        self.opt = api.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
+        api.boat_hip_optimizer_add_layernorm(self.opt, self.ln[0])
+        api.boat_hip_optimizer_add_attention(self.opt, self.att)
+        api.boat_hip_optimizer_add_layernorm(self.opt, self.ln[1])
+        api.boat_hip_optimizer_add_dense(self.opt, self.d1)
+        api.boat_hip_optimizer_add_dense(self.opt, self.d2)
+        self.tx = api.tensor(normal((B, S, H), 1.0))
+        self.tt = api.tensor(normal((B, S, H), 1.0))
+        self.shape2 = (C.c_int64 * 2)(B * S, H)
+        self.shape3 = (C.c_int64 * 3)(B, S, H)
+        self.losses = []
+        T = B * S
+        # linear layers forward + dX + dW, attention core forward (2 contractions) + backward (4 credited)
+        self.flops = 2.0 * T * (4 * H * H + 2 * H * ffn) * 3 + 3 * 2 * 2.0 * (B * heads) * S * S * (H // heads)
+        self.n_params = 4 * (H * H + H) + 4 * H + 2 * H * ffn + ffn + H
+
+    def step(self, keep_loss=False):
+        api, ln = self.api, self.ln
+        vx = api.boat_variable_create(self.tx, True)
         h1 = api.boat_hip_var_layernorm(vx, ln[0])
-        a = api.boat_var_attention(h1, h1, h1, att, None)
+        a = api.boat_var_attention(h1, h1, h1, self.att, None)
         x1 = api.boat_var_add(vx, a)
         h2 = api.boat_hip_var_layernorm(x1, ln[1])
-        h2f = api.boat_hip_var_reshape(h2, shape2, 2)
-        f1 = api.boat_var_dense(h2f, d1)
+        h2f = api.boat_hip_var_reshape(h2, self.shape2, 2)
+        f1 = api.boat_var_dense(h2f, self.d1)
         g1 = api.boat_hip_var_gelu(f1)
-        f2 = api.boat_var_dense(g1, d2)
-        f2r = api.boat_hip_var_reshape(f2, shape3, 3)
+        f2 = api.boat_var_dense(g1, self.d2)
+        f2r = api.boat_hip_var_reshape(f2, self.shape3, 3)
         y = api.boat_var_add(x1, f2r)
         grad = C.c_void_p()
-        tloss = api.boat_hip_mse_loss(api.boat_variable_data(y), tt, C.byref(grad))
+        tloss = api.boat_hip_mse_loss(api.boat_variable_data(y), self.tt, C.byref(grad))
         assert tloss and grad, "block forward failed"
         api.boat_variable_backward(y, grad)
-        api.boat_optimizer_step(opt)
-        api.boat_optimizer_zero_grad(opt)
+        api.boat_optimizer_step(self.opt)
+        api.boat_optimizer_zero_grad(self.opt)
         if keep_loss:
-            losses.append(float(api.numpy(tloss)[0]))
+            self.losses.append(float(api.numpy(tloss)[0]))
         api.boat_tensor_unref(tloss)
         api.boat_tensor_unref(grad)
         for v in (y, f2r, f2, g1, f1, h2f, h2, x1, a, h1, vx):
             api.boat_variable_free(v)
 
-    step(keep_loss=True)
-    warm_clocks(api.sync, step, max(warmup - 1, 1))
+
+class FlatAdam:
+    """Config 5b: fused Adam over 268,435,456 flat fp32 parameters (p ~N(0,0.02), g ~N(0,1e-3), m = v = 0): 28 B/param."""
+    n = 268435456
+
+    def __init__(self, hip):
+        self.hip = hip
+        rng = np.random.default_rng(20250103)
+        n = self.n
+        self.p, self.g, self.m, self.v = (hip.empty(n) for _ in range(4))
+        chunk = 1 << 24
+        noise_p = (0.02 * rng.standard_normal(chunk, dtype=np.float32)).astype(np.float32)
+        noise_g = (1e-3 * rng.standard_normal(chunk, dtype=np.float32)).astype(np.float32)
+        for off in range(0, n, chunk):   # tiled from one 16M-element draw
+            hip.check(hip.bh_memcpy_h2d(self.p.ptr + 4 * off, noise_p.ctypes.data, 4 * chunk))
+            hip.check(hip.bh_memcpy_h2d(self.g.ptr + 4 * off, noise_g.ctypes.data, 4 * chunk))
+        hip.check(hip.bh_memset_zero(self.m.ptr, 4 * n))
+        hip.check(hip.bh_memset_zero(self.v.ptr, 4 * n))
+        self.t = 0
+
+    def step(self):
+        hip = self.hip
+        hip.check(hip.bh_adam_update(self.p.ptr, self.g.ptr, self.m.ptr, self.v.ptr, self.n, 1e-3, 0.9, 0.999, 1e-8, self.t))
+        self.t += 1
+
+
+def bench_training_step(hip, steps, warmup):
+    """The headline: config 5 = block step + flat Adam, K steps between two HIP events on the library stream.  Every
+    GEMM, attention, LayerNorm, column-sum and optimizer launch inside the timed region is bracketed by its own event
+    pair (bh_profile_enable), which gives the dominant kernel family's duration live."""
+    block, flat = Block(), FlatAdam(hip)
+    block.step(keep_loss=True)
+    for _ in range(warmup):
+        block.step()
+        flat.step()
+    hip.synchronize()
+    mid = [hip.bh_event_create() for _ in range(2 * steps)]
+    hip.check(hip.bh_profile_enable(128 * steps), "bh_profile_enable")
     t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    api.sync()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
-    step(keep_loss=True)
+    timer = hip.Timer()
+    with timer:
+        for i in range(steps):
+            block.step()
+            hip.check(hip.bh_event_record(mid[2 * i]))
+            flat.step()
+            hip.check(hip.bh_event_record(mid[2 * i + 1]))
+    hip.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms_per_step = timer.ms / steps
+    flat_ms = sum(hip.bh_event_elapsed_ms(mid[2 * i], mid[2 * i + 1]) for i in range(steps)) / steps
+    for e in mid:
+        hip.bh_event_destroy(e)
+    classes = {}
+    for name, cls in (("gemm", hip.PROF_GEMM), ("attention_core_fwd", hip.PROF_SDPA_FWD), ("attention_core_bwd", hip.PROF_SDPA_BWD),
+                      ("layernorm", hip.PROF_NORM), ("adam", hip.PROF_OPTIMIZER), ("colsum", hip.PROF_COLSUM)):
+        ms, work, calls = hip.profile_read(cls)
+        classes[name] = (ms / steps, work / steps, calls // steps)
+    hip.check(hip.bh_profile_enable(0))
+    block.step(keep_loss=True)
+    losses = block.losses
     assert np.isfinite(losses).all() and losses[1] < losses[0], f"block training does not reduce the loss: {losses}"
-    flops = 2.0 * T * (4 * H * H + 2 * H * ffn) * 3 + 3 * 2 * 2.0 * (B * heads) * S * S * (H // heads)   # linear fwd+bwd, attention core fwd+bwd
-    n_params = 4 * (H * H + H) + 4 * H + 2 * H * ffn + ffn + H
-    return {"ms": round(ms, 4), "bound": "mixed", "achieved_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 2),
-            "frac_of_fp32_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4), "flops": flops,
-            "adam_params": n_params, "loss_first_last": [round(l, 6) for l in losses],
-            "note": "pre-LN block d1024 h16 ffn4096 S512 B16: forward + boat_variable_backward + boat_optimizer_step + zero_grad "
-                    "through the C API, wall clock"}
+    block_ms = ms_per_step - flat_ms
+    g_ms, g_flops, g_calls = classes["gemm"]
+    achieved = g_flops / (g_ms * 1e-3) / 1e12
+    breakdown = {"block_step_ms": round(block_ms, 4), "flat_adam_268M_ms": round(flat_ms, 4)}
+    for name, (ms, work, calls) in classes.items():
+        entry = {"ms_per_step": round(ms, 4), "launches_per_step": calls}
+        if name in ("gemm", "attention_core_fwd", "attention_core_bwd"):
+            entry.update(TFLOPs=round(work / (ms * 1e-3) / 1e12, 2), frac=round(work / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                         flops_per_step=work)
+        else:
+            entry.update(GBps=round(work / (ms * 1e-3) / 1e9, 1), frac=round(work / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), bytes_per_step=work)
+        breakdown[name] = entry
+    accounted = sum(ms for ms, _, _ in classes.values())
+    breakdown["other_kernels_and_gaps_ms"] = round(ms_per_step - accounted, 4)
+    flat_gbs = 28.0 * flat.n / (flat_ms * 1e-3) / 1e9
+    return {
+        "ms_per_step": ms_per_step, "wall_ms_per_step": wall_ms,
+        "roofline": {
+            "bound": "mfma", "kernel": "gemm_mfma_kernel family (fp32 v_mfma_f32_32x32x2_f32 tiles, operands direct to LDS): the "
+                                       f"{g_calls} bh_gemm launches of one step (projections, FFN, their dX and dW)",
+            "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+            "avg_launch_ms": round(g_ms / max(g_calls, 1), 4), "flops_per_launch": g_flops / max(g_calls, 1),
+            "launches_per_step": g_calls, "traffic": None,
+        },
+        "breakdown": breakdown,
+        "block": {"ms": round(block_ms, 4), "flops": block.flops, "achieved_TFLOPs": round(block.flops / (block_ms * 1e-3) / 1e12, 2),
+                  "frac_of_fp32_mfma_peak": round(block.flops / (block_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                  "adam_params": block.n_params, "loss_first_last": [round(l, 6) for l in losses]},
+        "flat_adam": {"ms": round(flat_ms, 4), "bound": "hbm", "achieved_GBps": round(flat_gbs, 1), "frac": round(flat_gbs / PEAK_HBM_GBS, 4),
+                      "bytes": 28 * flat.n},
+    }
 
 
 def cpu_baseline():
-    """Dense-layer backward of the reference on ONE host core, bounded sample, scaled by flops to config 2."""
+    """Configuration 5 on ONE host core of this box, on a bounded sample: the reference's routines for the two things
+    that make up the step's time -- dense-layer backward (its matmul, where 92 % of the block's flops go) at
+    M=K=N=1024, scaled by flops to the block's 670 GFLOP, and boat_optimizer_step (Adam) on 2^24 parameters, scaled by
+    element count to the 268,435,456 + 12,596,224 parameters of the step.  (The block itself cannot run on the
+    reference: its LayerNorm backward and GELU are stubs.)"""
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_lib
     m = k = n = 1024
@@ -440,11 +547,14 @@ def cpu_baseline():
     x = rng.standard_normal((m, k), dtype=np.float32)
     w = (0.02 * rng.standard_normal((k, n), dtype=np.float32)).astype(np.float32)
     dy = rng.standard_normal((m, n), dtype=np.float32)
-    full_flops = 2 * 2.0 * 8192 * 4096 * 4096
+    B, S, H, heads, ffn = Block.B, Block.S, Block.H, Block.heads, Block.ffn
+    block_flops = 2.0 * B * S * (4 * H * H + 2 * H * ffn) * 3 + 3 * 2 * 2.0 * (B * heads) * S * S * (H // heads)
+    adam_params = FlatAdam.n + 4 * (H * H + H) + 4 * H + 2 * H * ffn + ffn + H
     sample_flops = 2 * 2.0 * m * k * n
+    n_adam = 1 << 24
+    p, g = (rng.standard_normal(n_adam, dtype=np.float32) for _ in range(2))
     ref = oracle_lib.load_reference()
     if ref is not None:
-        import boat_cases as bc
         layer = ref.boat_dense_layer_create(k, n, True)
         ref.write(ref.boat_dense_layer_get_weight(layer), w)
         tx, tdy = ref.tensor(x), ref.tensor(dy)
@@ -452,20 +562,33 @@ def cpu_baseline():
         t0 = time.perf_counter()
         tdx = ref.boat_dense_layer_backward(layer, tdy)
         sec = time.perf_counter() - t0
-        assert tdx, "reference backward failed"
-        kind, what = "reference", "boat_dense_layer_backward of the compiled reference (oracle/_ref)"
+        assert ty and tdx, "reference backward failed"
+        tp, tg = ref.tensor(p), ref.tensor(g)
+        opt = ref.boat_adam_optimizer_create(1e-3, 0.9, 0.999, 1e-8)
+        ref.boat_optimizer_add_parameter(opt, tp, tg)
+        t0 = time.perf_counter()
+        ref.boat_optimizer_step(opt)
+        sec_adam = time.perf_counter() - t0
+        kind, what = "reference", "boat_dense_layer_backward and boat_optimizer_step (Adam) of the compiled reference (oracle/_ref)"
     else:
         oracle = oracle_lib.load()
         t0 = time.perf_counter()
         oracle.dense_backward(x, w, dy)
         sec = time.perf_counter() - t0
-        kind, what = "port", "oracle dense_backward (loop-order restatement of src/layers/dense.c:190-295)"
+        mm, vv = np.zeros(n_adam, np.float32), np.zeros(n_adam, np.float32)
+        t0 = time.perf_counter()
+        oracle.adam_update(p, g, mm, vv, 1e-3, 0.9, 0.999, 1e-8, 0)
+        sec_adam = time.perf_counter() - t0
+        kind, what = "port", "oracle dense_backward and adam_update (loop-order restatements of src/layers/dense.c:190-295, src/optimizers/adam.c:203-222)"
+    block_ms = sec * 1e3 * block_flops / sample_flops
+    adam_ms = sec_adam * 1e3 * adam_params / n_adam
     return {
-        "value": round(sec * 1e3 * full_flops / sample_flops, 1), "unit": "ms", "cores": 1, "kind": kind,
+        "value": round(block_ms + adam_ms, 1), "unit": "ms", "cores": 1, "kind": kind,
         "host_cores_total": os.cpu_count(),
-        "sample": f"{what} at M=K=N={m} ({sample_flops / 1e9:.2f} GFLOP) took {sec:.2f} s = "
-                  f"{sample_flops / sec / 1e9:.2f} GFLOP/s; value is that time scaled by flops to the "
-                  f"{full_flops / 1e9:.2f} GFLOP workload (extrapolated)",
+        "sample": f"{what}: dense backward at M=K=N={m} ({sample_flops / 1e9:.2f} GFLOP) took {sec:.2f} s = "
+                  f"{sample_flops / sec / 1e9:.2f} GFLOP/s, Adam on {n_adam} parameters took {sec_adam * 1e3:.1f} ms; value = the "
+                  f"block's {block_flops / 1e9:.1f} GFLOP at that rate ({block_ms / 1e3:.0f} s) + Adam over {adam_params} parameters "
+                  f"({adam_ms:.0f} ms), both extrapolated",
     }
 
 
@@ -540,13 +663,13 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build (the path has no inter-GPU work)",
               file=sys.stderr)
         sys.exit(2)
-    all_legs = ["dense", "adam", "ln_gelu", "sdpa", "mlp", "cnn", "block"]
+    all_legs = ["step", "dense", "adam", "ln_gelu", "sdpa", "mlp", "cnn"]
     legs = all_legs if args.legs == "all" else [l.strip() for l in args.legs.split(",") if l.strip()]
     unknown = [l for l in legs if l not in all_legs]
     if unknown:
         sys.exit(f"unknown leg(s) {unknown}; choose from {all_legs}")
     if args.no_extra:
-        legs = [l for l in legs if l == "dense"]
+        legs = [l for l in legs if l == "step"]
     from boat_amd import hip
     hip.check(hip.bh_init(), "bh_init")
 
@@ -554,17 +677,25 @@ def main():
         "metric": METRIC, "value": None, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "dense layer backward (benchmark configuration 2): X[8192x4096], W[4096x4096], dY[8192x4096] -> dX, dW, db; "
-                               "549.76 GFLOP per step", "M": 8192, "K": 4096, "N": 4096,
+        "config": {"workload": "benchmark configuration 5: pre-LN transformer encoder block training step (d_model 1024, 16 heads, FFN 4096 "
+                               "GELU, seq 512, batch 16; forward + boat_variable_backward + fused Adam over 12,596,224 parameters + zero_grad, "
+                               "about 670 GFLOP) followed by fused Adam over 268,435,456 flat fp32 parameters (7.516 GB)",
+                   "d_model": 1024, "heads": 16, "ffn": 4096, "seq": 512, "batch": 16, "flat_adam_params": 268435456,
                    "device": hip.bh_device_name().decode().strip(), "compute_units": hip.bh_device_cu_count()},
     }
-    if "dense" in legs:
-        main_res = bench_dense_backward(hip, args.steps, args.warmup)
-        line.update({"value": round(main_res["ms_per_step"], 4), "ms_per_step": round(main_res["ms_per_step"], 4),
-                     "roofline": main_res["roofline"], "step_tflops": main_res["step_tflops"],
-                     "wall_ms_per_step": round(main_res["wall_ms_per_step"], 4)})
     extra = {}
+    if "step" in legs:
+        res = bench_training_step(hip, args.steps, args.warmup)
+        line.update({"value": round(res["ms_per_step"], 4), "ms_per_step": round(res["ms_per_step"], 4), "roofline": res["roofline"],
+                     "wall_ms_per_step": round(res["wall_ms_per_step"], 4)})
+        extra["step_breakdown"] = res["breakdown"]
+        extra["transformer_block_step"] = res["block"]
+        extra["adam_flat_268M_in_step"] = res["flat_adam"]
     if "dense" in legs:
+        d = bench_dense_backward(hip, args.steps, args.warmup)
+        extra["dense_backward_config2"] = {"ms": round(d["ms_per_step"], 4), "bound": "mfma", "step_TFLOPs": d["step_tflops"],
+                                           "frac": round(d["step_tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "flops": 2 * d["roofline"]["flops_per_launch"],
+                                           "gemm_launch": d["roofline"]}
         extra.update(bench_dense_forward(hip, args.steps, args.warmup))
     if "adam" in legs:
         extra.update(bench_adam(hip, args.steps, args.warmup))
@@ -576,11 +707,9 @@ def main():
         extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20) * 25, max(args.warmup, 1) * 100)
     if "cnn" in legs:
         extra["mnist_cnn_step"] = bench_cnn_step(max(args.steps, 20), max(args.warmup, 3))
-    if "block" in legs:
-        extra["transformer_block_step"] = bench_block_step(max(2, min(args.steps, 10)), min(args.warmup, 2))
     if extra:
         line["extra"] = extra
-    if not args.no_cpu and "dense" in legs:
+    if not args.no_cpu and "step" in legs:
         line["cpu_baseline"] = cpu_baseline()
         if not args.no_extra:
             line["cpu_beside_other_configs"] = cpu_beside_other_configs()

@@ -258,6 +258,7 @@ int bh_adam_update(float* p, const float* g, float* m, float* v, int64_t n, floa
     BH_CHECK_ARG(n >= 0 && timestep >= 0, "negative size or timestep");
     if (n == 0) return BH_OK;
     BH_CHECK_ARG(p && g && m && v, "null pointer");
+    ProfScope prof(BH_PROF_OPTIMIZER, 28.0 * (double)n);
     AdamScalars s = make_scalars(lr, beta1, beta2, eps, timestep);
     const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
                        reinterpret_cast<uintptr_t>(v)) & 15) == 0;
@@ -275,6 +276,9 @@ int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(count >= 0 && timestep >= 0, "negative count or timestep");
     BH_CHECK_ARG(count == 0 || (p && g && m && v && n), "null table");
+    double total = 0.0;
+    for (int i = 0; i < count; i++) total += n[i] > 0 ? (double)n[i] : 0.0;
+    ProfScope prof(BH_PROF_OPTIMIZER, 28.0 * total);
     AdamScalars s = make_scalars(lr, beta1, beta2, eps, timestep);
     int done = 0;
     while (done < count) {

@@ -18,6 +18,16 @@ int check_hip(hipError_t e, const char* what);
 bool ready();
 int ln_scratch_setup();   // bh_layernorm.hip: resolves the current device's copy of the no-alloc scratch array
 
+// Per-class timing of the library's launches with HIP events on the library stream (bh_profile_* in boat_hip.h).
+// An entry point opens a scope after its argument checks; when profiling is off this is one branch.
+void prof_open(int cls, double work, int* slot);
+void prof_close(int slot);
+struct ProfScope {
+    int slot = -1;   // -1: profiling off; -2: open but not recorded (nested, or no events left); >= 0: record index
+    ProfScope(int cls, double work) { prof_open(cls, work, &slot); }
+    ~ProfScope() { if (slot != -1) prof_close(slot); }
+};
+
 #define BH_REQUIRE_INIT()                                   \
     do {                                                    \
         if (!::bh::ready()) {                               \

@@ -1039,6 +1039,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     BH_CHECK_ARG(a && b && c, "null pointer");
     BH_CHECK_ARG(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "leading dimension too small");
     BH_CHECK_ARG(batch <= 65535, "batch too large");
+    ProfScope prof(BH_PROF_GEMM, 2.0 * (double)m * (double)n * (double)k * (double)batch);
 
     GemmArgs g;
     g.a = a; g.b = b; g.c = c; g.bias = bias;

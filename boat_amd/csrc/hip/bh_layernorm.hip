@@ -427,6 +427,7 @@ int bh_layernorm_tune(int bwd_blocks, int reserved) {
 
 static int norm_forward(bool rms, const char* name, const float* x, const float* gamma, const float* beta, float* y,
                         float* mean, float* rstd, int64_t rows, int64_t hidden, float eps) {
+    ProfScope prof(BH_PROF_NORM, 8.0 * (double)rows * (double)hidden);
     LnPlan plan = plan_for(hidden, x, y, gamma ? (const void*)gamma : (const void*)x);
     if (plan.vector && beta && (reinterpret_cast<uintptr_t>(beta) & 15)) plan.vector = false;
     if (!plan.vector) {
@@ -502,6 +503,7 @@ static bool ln_backward_plan(LnPlan& plan, size_t& shmem, const float* x, const 
 static int norm_backward(bool rms, float eps, const float* x, const float* gamma, const float* dy, const float* mean,
                          const float* rstd, float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden,
                          int accumulate) {
+    ProfScope prof(BH_PROF_NORM, 12.0 * (double)rows * (double)hidden);
     LnPlan plan;
     size_t shmem;
     ln_backward_plan(plan, shmem, x, gamma, dy, dx, hidden);

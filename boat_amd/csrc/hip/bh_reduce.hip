@@ -178,6 +178,7 @@ int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumu
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(rows >= 0 && cols >= 0 && (out || cols == 0) && (x || rows * cols == 0), "bad argument");
     if (cols == 0) return BH_OK;
+    ProfScope prof(BH_PROF_COLSUM, 4.0 * (double)rows * (double)cols);
     if (rows <= 256) {   // few rows: the fold kernel (64 columns x 16 row lanes per workgroup) is the whole column sum
         hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(cols, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0, stream(),
                            x, rows, cols, out, (float*)nullptr, cols, accumulate);

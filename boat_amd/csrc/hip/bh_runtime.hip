@@ -13,6 +13,7 @@
 #include <string.h>
 
 #include <map>
+#include <vector>
 #include <mutex>
 #include <unordered_map>
 
@@ -44,6 +45,38 @@ int set_error(int code, const char* fmt, ...) {
 int check_hip(hipError_t e, const char* what) {
     if (e == hipSuccess) return BH_OK;
     return set_error(BH_EDEVICE, "%s: %s", what, hipGetErrorString(e));
+}
+
+// ---- profiling: one start/stop event pair per instrumented call, taken from a pool created when profiling is
+// switched on (nothing is created inside a timed region); a nested scope (bh_dense_backward calling bh_gemm) is
+// recorded for the innermost call only
+struct ProfRec {
+    int cls;
+    double work;
+    hipEvent_t a, b;
+};
+static bool g_prof_on = false;
+static std::vector<ProfRec> g_prof;
+static std::vector<hipEvent_t> g_prof_pool;
+static int g_prof_depth = 0;
+
+void prof_open(int cls, double work, int* slot) {
+    *slot = -1;
+    if (!g_prof_on) return;
+    *slot = -2;
+    if (g_prof_depth++ > 0) return;          // called from an instrumented entry point: the outer call is the record
+    if (g_prof_pool.size() < 2) return;
+    ProfRec r{cls, work, g_prof_pool.back(), nullptr};
+    g_prof_pool.pop_back();
+    r.b = g_prof_pool.back();
+    g_prof_pool.pop_back();
+    if (hipEventRecord(r.a, g_stream) != hipSuccess) return;
+    g_prof.push_back(r);
+    *slot = (int)g_prof.size() - 1;
+}
+void prof_close(int slot) {
+    if (g_prof_depth > 0) g_prof_depth--;
+    if (slot >= 0 && slot < (int)g_prof.size()) (void)hipEventRecord(g_prof[slot].b, g_stream);
 }
 
 static size_t round_capacity(size_t n) {
@@ -221,6 +254,53 @@ int bh_memcpy_d2d(void* dst, const void* src, size_t nbytes) {
     if (((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | nbytes) & 3) == 0)
         return bh_copy_f32(static_cast<float*>(dst), static_cast<const float*>(src), (int64_t)(nbytes / 4));
     return check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, g_stream), "memcpy d2d");
+}
+
+int bh_profile_enable(int max_calls) {
+    BH_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lk(g_mu);
+    (void)hipStreamSynchronize(g_stream);
+    for (auto& r : g_prof) {
+        g_prof_pool.push_back(r.a);
+        if (r.b) g_prof_pool.push_back(r.b);
+    }
+    g_prof.clear();
+    g_prof_depth = 0;
+    if (max_calls <= 0) {
+        g_prof_on = false;
+        for (hipEvent_t e : g_prof_pool) (void)hipEventDestroy(e);
+        g_prof_pool.clear();
+        return BH_OK;
+    }
+    while (g_prof_pool.size() < 2 * (size_t)max_calls) {
+        hipEvent_t e;
+        int rc = check_hip(hipEventCreate(&e), "hipEventCreate");
+        if (rc) return rc;
+        g_prof_pool.push_back(e);
+    }
+    g_prof.reserve((size_t)max_calls);
+    g_prof_on = true;
+    return BH_OK;
+}
+
+int bh_profile_read(int cls, double* total_ms, double* total_work, int64_t* calls) {
+    BH_REQUIRE_INIT();
+    int rc = check_hip(hipStreamSynchronize(g_stream), "hipStreamSynchronize");
+    if (rc) return rc;
+    double ms = 0.0, work = 0.0;
+    int64_t n = 0;
+    for (const ProfRec& r : g_prof) {
+        if (r.cls != cls || !r.b) continue;
+        float t = 0.f;
+        if (hipEventElapsedTime(&t, r.a, r.b) != hipSuccess) continue;
+        ms += t;
+        work += r.work;
+        n++;
+    }
+    if (total_ms) *total_ms = ms;
+    if (total_work) *total_work = work;
+    if (calls) *calls = n;
+    return BH_OK;
 }
 
 struct bh_event {

@@ -303,6 +303,7 @@ int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale,
     BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
     if (bh_count == 0 || s == 0) return BH_OK;
     BH_CHECK_ARG(q && k && v && out, "null pointer");
+    ProfScope prof(BH_PROF_SDPA_FWD, 4.0 * (double)bh_count * (double)s * (double)s * (double)d);
     if (!g_sdpa_force_general && !attn_out && lse) {
         int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, bh_count, s, d);
         if (rc <= 0) return rc;   // 0 done, <0 error, 1 shape not covered
@@ -324,6 +325,7 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
     BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
     if (bh_count == 0 || s == 0) return BH_OK;
     BH_CHECK_ARG(q && k && v && out && lse && d_out && dq && dk && dv, "null pointer");
+    ProfScope prof(BH_PROF_SDPA_BWD, 8.0 * (double)bh_count * (double)s * (double)s * (double)d);
     const int64_t rows = bh_count * s;
     float* delta = (float*)bh_malloc(sizeof(float) * (size_t)rows);
     if (!delta) return BH_ENOMEM;

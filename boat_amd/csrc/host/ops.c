@@ -367,29 +367,35 @@ boat_tensor_t* boat_hip_softmax_cross_entropy(const boat_tensor_t* logits, const
     const int64_t rows = logits->shape[0], cols = logits->shape[1];
     if ((int64_t)labels->nelements != rows || rows == 0 || cols == 0) return NULL;
     if (labels->dtype != BOAT_DTYPE_INT32 && labels->dtype != BOAT_DTYPE_UINT8) return NULL;
-    int32_t* host_labels = (int32_t*)malloc(sizeof(int32_t) * (size_t)rows);
-    if (!host_labels) return NULL;
-    const void* src = boat_tensor_const_data(labels);
-    if (labels->device == BOAT_DEVICE_HIP || !src) {   /* class indices are host data */
-        free(host_labels);
-        return NULL;
-    }
-    for (int64_t i = 0; i < rows; i++)
-        host_labels[i] = labels->dtype == BOAT_DTYPE_INT32 ? ((const int32_t*)src)[i] : (int32_t)((const uint8_t*)src)[i];
-    int32_t* dev_labels = (int32_t*)bh_malloc(sizeof(int32_t) * (size_t)rows);
     const int64_t one = 1;
     boat_tensor_t* loss = bt_new_uninit(&one, 1, logits->device);
     boat_tensor_t* grad = dlogits ? bt_new_like_uninit(logits) : NULL;
-    bool ok = dev_labels && loss && (!dlogits || grad);
-    if (ok) ok = boat_hip_ok(bh_memcpy_h2d(dev_labels, host_labels, sizeof(int32_t) * (size_t)rows), "labels upload");
+    bool ok = loss && (!dlogits || grad);
+    int32_t* staged = NULL;   /* device copy of widened UINT8 labels */
+    const int32_t* dev_labels = NULL;
+    if (ok && labels->dtype == BOAT_DTYPE_INT32) {
+        /* INT32 indices are used where they are: the tensor's device copy (uploaded once, like any tensor) */
+        dev_labels = (const int32_t*)bt_dev_read(labels);
+        ok = dev_labels != NULL;
+    } else if (ok) {
+        const void* src = labels->device == BOAT_DEVICE_HIP ? NULL : boat_tensor_const_data(labels);
+        int32_t* host_labels = src ? (int32_t*)malloc(sizeof(int32_t) * (size_t)rows) : NULL;
+        staged = host_labels ? (int32_t*)bh_malloc(sizeof(int32_t) * (size_t)rows) : NULL;
+        ok = staged != NULL;
+        if (ok) {
+            for (int64_t i = 0; i < rows; i++) host_labels[i] = (int32_t)((const uint8_t*)src)[i];
+            ok = boat_hip_ok(bh_memcpy_h2d(staged, host_labels, sizeof(int32_t) * (size_t)rows), "labels upload");
+        }
+        free(host_labels);
+        dev_labels = staged;
+    }
     if (ok) {
         const float* pz = bt_dev_read(logits);
         float* pl = bt_dev_write(loss);
         float* pg = grad ? bt_dev_write(grad) : NULL;
         ok = pz && pl && boat_hip_ok(bh_softmax_ce_grad(pz, dev_labels, pg, pl, rows, cols), "softmax cross-entropy");
     }
-    free(host_labels);
-    if (dev_labels) bh_free(dev_labels);
+    if (staged) bh_free(staged);
     if (!ok) {
         boat_tensor_free(loss);
         boat_tensor_free(grad);

@@ -10,7 +10,13 @@
  *
  *   gcc mlp_train_step.c -I<repo>/include -L<repo>/boat_amd/lib -lboat_amd -Wl,-rpath,<repo>/boat_amd/lib -lm
  *
- * usage: mlp_train_step [steps] [warmup]   -> one JSON line: wall ms per step, first and last loss
+ * usage: mlp_train_step [steps] [warmup] [fused]   -> one JSON line: wall ms per step, first and last loss
+ *
+ * With a third argument "fused" the four-op loss chain and its backward are replaced by one call of
+ * boat_hip_softmax_cross_entropy (loss and d(loss)/d(logits) from one kernel), and backward starts at the logits.
+ *
+ * The program writes through boat_tensor_data() pointers during set-up only and never keeps one across a call; run it
+ * with BOAT_HIP_COHERENT_POINTERS=0 to let the tensors it touched stay resident on the device.
  */
 #include <stdio.h>
 #include <stdlib.h>
@@ -38,6 +44,7 @@ static double now_ms(void) {
 int main(int argc, char** argv) {
     const int steps = argc > 1 ? atoi(argv[1]) : 200;
     const int warmup = argc > 2 ? atoi(argv[2]) : 20;
+    const int fused = argc > 3 && argv[3][0] == 'f';
 
     boat_dense_layer_t* l1 = boat_dense_layer_create(D_IN, D_H, true);
     boat_dense_layer_t* l2 = boat_dense_layer_create(D_H, D_OUT, true);
@@ -57,8 +64,14 @@ int main(int argc, char** argv) {
     boat_tensor_t* factor = boat_tensor_create(one, 1, BOAT_DTYPE_FLOAT32, BOAT_DEVICE_CPU);
     float* px = (float*)boat_tensor_data(x);
     for (int i = 0; i < B * D_IN; i++) px[i] = uniform01();
+    const int64_t ls_shape[1] = {B};
+    boat_tensor_t* labels = boat_tensor_create(ls_shape, 1, BOAT_DTYPE_INT32, BOAT_DEVICE_CPU);
     float* poh = (float*)boat_tensor_data(onehot);
-    for (int b = 0; b < B; b++) poh[b * D_OUT + (int)(uniform01() * D_OUT) % D_OUT] = 1.0f;
+    int32_t* plab = (int32_t*)boat_tensor_data(labels);
+    for (int b = 0; b < B; b++) {
+        plab[b] = (int)(uniform01() * D_OUT) % D_OUT;
+        poh[b * D_OUT + plab[b]] = 1.0f;
+    }
     ((float*)boat_tensor_data(factor))[0] = -1.0f / B;
 
     boat_optimizer_t* opt = boat_adam_optimizer_create(1e-3f, 0.9f, 0.999f, 1e-8f);
@@ -71,6 +84,28 @@ int main(int argc, char** argv) {
         if (it == warmup) {
             boat_hip_synchronize();
             t0 = now_ms();
+        }
+        if (fused) {
+            boat_variable_t* vx = boat_variable_create(x, true);
+            boat_variable_t* h = boat_var_dense(vx, l1);
+            boat_variable_t* r = boat_var_relu(h);
+            boat_variable_t* z = boat_var_dense(r, l2);
+            boat_tensor_t* dz = NULL;
+            boat_tensor_t* tl = z ? boat_hip_softmax_cross_entropy(boat_variable_data(z), labels, &dz) : NULL;
+            if (!tl || !dz) return 2;
+            boat_variable_backward(z, dz);
+            boat_optimizer_step(opt);
+            boat_optimizer_zero_grad(opt);
+            if (it == 0 || it == warmup + steps - 1) {
+                const float v = ((const float*)boat_tensor_const_data(tl))[0];
+                if (it == 0) first = v;
+                else last = v;
+            }
+            boat_tensor_unref(tl);
+            boat_tensor_unref(dz);
+            boat_variable_t* vars[] = {z, r, h, vx};
+            for (size_t i = 0; i < sizeof(vars) / sizeof(vars[0]); i++) boat_variable_free(vars[i]);
+            continue;
         }
         boat_variable_t* vx = boat_variable_create(x, true);
         boat_variable_t* voh = boat_variable_create(onehot, false);
@@ -96,11 +131,12 @@ int main(int argc, char** argv) {
     }
     boat_hip_synchronize();
     const double ms = (now_ms() - t0) / steps;
-    printf("{\"ms_per_step\": %.5f, \"steps\": %d, \"warmup\": %d, \"loss_first\": %.6f, \"loss_last\": %.6f}\n", ms, steps,
-           warmup, first, last);
+    printf("{\"ms_per_step\": %.5f, \"steps\": %d, \"warmup\": %d, \"fused_loss\": %d, \"loss_first\": %.6f, \"loss_last\": %.6f}\n",
+           ms, steps, warmup, fused, first, last);
     boat_optimizer_free(opt);
     boat_tensor_unref(x);
     boat_tensor_unref(onehot);
+    boat_tensor_unref(labels);
     boat_tensor_unref(factor);
     boat_dense_layer_free(l1);
     boat_dense_layer_free(l2);

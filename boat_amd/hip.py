@@ -33,6 +33,8 @@ _SIGS = {
     "bh_memset_zero": (I, [P, Z]),
     "bh_event_create": (P, []), "bh_event_destroy": (None, [P]), "bh_event_record": (I, [P]),
     "bh_event_elapsed_ms": (F, [P, P]),
+    "bh_profile_enable": (I, [I]),
+    "bh_profile_read": (I, [I, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(L)]),
     "bh_fill": (I, [P, F, L]),
     "bh_add_inplace": (I, [P, P, L]),
     "bh_binary": (I, [I, P, P, P, L]),
@@ -81,6 +83,14 @@ for _name, (_res, _args) in _SIGS.items():
     globals()[_name] = _fn
 
 ACT_RELU, ACT_SIGMOID, ACT_TANH, ACT_GELU = 0, 1, 2, 3
+PROF_GEMM, PROF_SDPA_FWD, PROF_SDPA_BWD, PROF_NORM, PROF_OPTIMIZER, PROF_COLSUM = range(6)
+
+
+def profile_read(cls):
+    """(total ms, total declared work, calls) of one class of launches since bh_profile_enable."""
+    ms, work, calls = C.c_double(), C.c_double(), L()
+    check(lib.bh_profile_read(cls, C.byref(ms), C.byref(work), C.byref(calls)), "bh_profile_read")
+    return ms.value, work.value, calls.value
 
 
 class HipError(RuntimeError):

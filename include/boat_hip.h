@@ -63,6 +63,22 @@ void        bh_event_destroy(bh_event_t* e);
 int         bh_event_record(bh_event_t* e);
 float       bh_event_elapsed_ms(bh_event_t* start, bh_event_t* stop);    /* synchronises on stop */
 
+/* ---- per-class timing of the library's own launches, for benchmarks that drive whole training steps through Boat's API
+ * and still need the duration of one kernel family inside the step.  bh_profile_enable(max_calls > 0) creates
+ * 2*max_calls events and starts recording one start/stop pair on the library stream around each instrumented entry point
+ * (an entry point called from another instrumented one is not recorded twice); bh_profile_enable(0) stops and frees.
+ * Each call to enable starts a fresh recording.  bh_profile_read waits for the stream and sums, for one class, the
+ * event-to-event time in ms, the algorithmic work the calls declared (flops for the matrix classes, bytes for the
+ * memory-bound ones) and the number of calls.  Calls beyond max_calls are not recorded. */
+#define BH_PROF_GEMM       0   /* bh_gemm: 2*m*n*k*batch flops */
+#define BH_PROF_SDPA_FWD   1   /* bh_sdpa_forward: 2 * 2*bh*s*s*d flops */
+#define BH_PROF_SDPA_BWD   2   /* bh_sdpa_backward: 4 * 2*bh*s*s*d flops (the reference's four contractions) */
+#define BH_PROF_NORM       3   /* LayerNorm / RMSNorm forward (2 passes) and backward (3 passes): bytes of x, y or x, dy, dx */
+#define BH_PROF_OPTIMIZER  4   /* Adam (28 B/param), RMSprop / Adagrad (20 B/param) */
+#define BH_PROF_COLSUM     5   /* bh_colsum: bytes read */
+int bh_profile_enable(int max_calls);
+int bh_profile_read(int cls, double* total_ms, double* total_work, int64_t* calls);
+
 /* ---- elementwise (src/ops/arithmetic.c:157-285,362-484; src/autodiff.c:1002-1452) ---- */
 int bh_fill(float* x, float value, int64_t n);
 int bh_add_inplace(float* a, const float* b, int64_t n);                              /* boat_add_ */

@@ -476,7 +476,6 @@ def bench_training_step(hip, steps, warmup):
         flat.step()
     hip.synchronize()
     mid = [hip.bh_event_create() for _ in range(2 * steps)]
-    hip.check(hip.bh_profile_enable(128 * steps), "bh_profile_enable")
     t0 = time.perf_counter()
     timer = hip.Timer()
     with timer:
@@ -491,6 +490,17 @@ def bench_training_step(hip, steps, warmup):
     flat_ms = sum(hip.bh_event_elapsed_ms(mid[2 * i], mid[2 * i + 1]) for i in range(steps)) / steps
     for e in mid:
         hip.bh_event_destroy(e)
+    # The same K steps once more, now with an event pair around every instrumented launch.  An event costs the stream
+    # about 5 us (the kernel after it waits for the marker), some 0.25 ms per step with 35 instrumented calls, so this
+    # pass is kept out of the timed region above; the durations it yields are those of the same kernels on the same data.
+    hip.check(hip.bh_profile_enable(128 * steps), "bh_profile_enable")
+    profiled = hip.Timer()
+    with profiled:
+        for i in range(steps):
+            block.step()
+            flat.step()
+    hip.synchronize()
+    profiled_ms = profiled.ms / steps
     classes = {}
     for name, cls in (("gemm", hip.PROF_GEMM), ("attention_core_fwd", hip.PROF_SDPA_FWD), ("attention_core_bwd", hip.PROF_SDPA_BWD),
                       ("layernorm", hip.PROF_NORM), ("adam", hip.PROF_OPTIMIZER), ("colsum", hip.PROF_COLSUM)):
@@ -514,6 +524,7 @@ def bench_training_step(hip, steps, warmup):
         breakdown[name] = entry
     accounted = sum(ms for ms, _, _ in classes.values())
     breakdown["other_kernels_and_gaps_ms"] = round(ms_per_step - accounted, 4)
+    breakdown["ms_per_step_with_launch_events"] = round(profiled_ms, 4)
     flat_gbs = 28.0 * flat.n / (flat_ms * 1e-3) / 1e9
     return {
         "ms_per_step": ms_per_step, "wall_ms_per_step": wall_ms,
@@ -524,6 +535,8 @@ def bench_training_step(hip, steps, warmup):
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(g_ms / max(g_calls, 1), 4), "flops_per_launch": g_flops / max(g_calls, 1),
             "launches_per_step": g_calls, "traffic": None,
+            "measured": "HIP event pairs around each bh_gemm launch of K further steps run right after the timed K (the events "
+                        "themselves cost about 5 us each on the stream, so they stay out of the timed region)",
         },
         "breakdown": breakdown,
         "block": {"ms": round(block_ms, 4), "flops": block.flops, "achieved_TFLOPs": round(block.flops / (block_ms * 1e-3) / 1e12, 2),

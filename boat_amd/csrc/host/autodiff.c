@@ -41,6 +41,7 @@ struct boat_variable_t {
     boat_tensor_t* grad;
     bool requires_grad;
     bool persistent_grad;        /* grad buffer survives zero_grad (boat_hip_variable_ensure_grad) */
+    bool grad_shared;            /* grad is a tensor other holders read too: replace it, never add into it */
     boat_op_t* producer;
     size_t refs;
     struct boat_variable_t *prev, *next;   /* live-variable list of the library */
@@ -372,8 +373,20 @@ boat_variable_t* boat_hip_var_layernorm(const boat_variable_t* a, boat_layernorm
 static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
     if (!g) return;
     if (!v->grad) {
+        v->grad_shared = false;
         if (own && g->ref_count == 1 && !g->is_view && g->nelements == v->data->nelements) {
             v->grad = g;
+            return;
+        }
+        /* The first contribution to a NON-LEAF variable that cannot be taken over (the consumer's own gradient handed
+         * on by an add or a reshape) is shared, not copied: in the reverse walk a gradient is complete before it is
+         * handed on, so nobody adds into it afterwards, and this variable replaces it (below) instead of adding into it
+         * if a second contribution comes.  Leaves keep a buffer of their own, which outlives the walk.  The
+         * reference-exact walk hands on gradients that are still growing, so it copies. */
+        if (v->producer && !bt_reference_exact() && bt_is_f32(g) && bt_same_shape(g, v->data)) {
+            if (!own) boat_tensor_ref(g);
+            v->grad = g;
+            v->grad_shared = true;
             return;
         }
         if (bt_is_f32(g) && bt_is_f32(v->data) && g->nelements == v->data->nelements && g->nelements > 0) {
@@ -390,7 +403,22 @@ static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
         }
         v->grad = boat_tensor_create_like(v->data);
     }
-    if (v->grad) boat_add_(v->grad, g);
+    if (v->grad && v->grad_shared) {
+        /* out of place: the shared tensor stays what it is for its other holders (same cost as adding in place) */
+        boat_tensor_t* sum = g->nelements == v->grad->nelements && bt_is_f32(g) ? bt_new_like_uninit(v->grad) : NULL;
+        const float* pa = sum ? bt_dev_read(v->grad) : NULL;
+        const float* pb = pa ? bt_dev_read(g) : NULL;
+        float* ps = pb ? bt_dev_write(sum) : NULL;
+        if (ps && boat_hip_ok(bh_binary(0, pa, pb, ps, (int64_t)sum->nelements), "gradient sum")) {
+            boat_tensor_unref(v->grad);
+            v->grad = sum;
+            v->grad_shared = false;
+        } else {
+            boat_tensor_free(sum);
+        }
+    } else if (v->grad) {
+        boat_add_(v->grad, g);
+    }
     if (own) boat_tensor_unref(g);
 }
 
@@ -574,6 +602,16 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
             break;
         }
         case OP_ATTENTION: {   /* :2458-2532 */
+            if (op->inputs[0] == op->inputs[1] && op->inputs[0] == op->inputs[2] && !bt_reference_exact()) {
+                /* self-attention: the three input gradients go to one variable; the key and value projections' input
+                 * gradients are added into the query projection's by their GEMM epilogues */
+                boat_tensor_t* g_in = NULL;
+                if (boat_attention_backward_self((boat_attention_t*)op->layer, dy, &g_in) && op->inputs[0]->requires_grad)
+                    accumulate(op->inputs[0], g_in, true);
+                else
+                    boat_tensor_free(g_in);
+                break;
+            }
             boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
             if (!boat_attention_backward((boat_attention_t*)op->layer, dy, &gq, &gk, &gv)) break;
             boat_variable_t* in[3] = {op->inputs[0], op->inputs[1], op->inputs[2]};

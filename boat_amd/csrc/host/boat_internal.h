@@ -113,6 +113,10 @@ struct boat_attention_t {
     boat_tensor_t* cache_attention_output;   /* [B,S,H] before the output projection */
 };
 
+/* boat_attention_backward for a layer whose query, key and value were one tensor: *grad_input = dq + dk + dv, the sums
+ * made by the input projections' GEMM epilogues (used by the tape) */
+bool boat_attention_backward_self(boat_attention_t* attention, const boat_tensor_t* grad_output, boat_tensor_t** grad_input);
+
 /* layernorm backward used by both the layer hook and the tape */
 boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
                                             const boat_tensor_t* rstd, const boat_tensor_t* grad_output);

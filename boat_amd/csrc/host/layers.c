@@ -671,9 +671,13 @@ void boat_apply_rotary_embedding(boat_tensor_t* query, boat_tensor_t* key, size_
 }
 
 /* linear_projection_backward, attention.c:1186-1285: dx = dy.w^T ; *gw = x^T.dy ; *gb = colsum(dy), all overwritten */
+/* `into` non-NULL: dx is added into that tensor by the GEMM's epilogue (and a new reference to it is returned) instead of
+ * being written to a new one */
 static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor_t* w, const boat_tensor_t* bias,
-                                       const boat_tensor_t* dy, boat_tensor_t** gw, boat_tensor_t** gb, int64_t rows, int64_t h) {
-    boat_tensor_t* dx = bt_new_like_uninit(x);
+                                       const boat_tensor_t* dy, boat_tensor_t** gw, boat_tensor_t** gb, int64_t rows, int64_t h,
+                                       boat_tensor_t* into) {
+    boat_tensor_t* dx = into ? into : bt_new_like_uninit(x);
+    if (into) boat_tensor_ref(into);
     if (!*gw) *gw = boat_tensor_create_like(w);
     if (bias && !*gb) *gb = boat_tensor_create_like(bias);
     if (!dx || !*gw || (bias && !*gb)) {
@@ -683,11 +687,14 @@ static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor
     const float* px = bt_dev_read(x);
     const float* pw = bt_dev_read(w);
     const float* pdy = bt_dev_read(dy);
-    float* pdx = bt_dev_write(dx);
+    float* pdx = into ? bt_dev_rw(dx) : bt_dev_write(dx);
     float* pgw = bt_dev_write(*gw);
     float* pgb = bias ? bt_dev_write(*gb) : NULL;
-    if (!px || !pw || !pdy || !pdx || !pgw ||
-        !boat_hip_ok(bh_dense_backward(px, pw, pdy, pdx, pgw, pgb, rows, h, h, 0), "attention projection backward")) {
+    bool ok = px && pw && pdy && pdx && pgw;
+    /* dx (+)= dy.w^T ; gw = x^T.dy ; gb = colsum(dy) */
+    if (ok) ok = boat_hip_ok(bh_gemm(0, 1, rows, h, h, pdy, h, pw, h, pdx, h, NULL, into ? 1 : 0, 1), "attention projection backward");
+    if (ok) ok = boat_hip_ok(bh_dense_backward(px, pw, pdy, NULL, pgw, pgb, rows, h, h, 0), "attention projection backward");
+    if (!ok) {
         boat_tensor_free(dx);
         return NULL;
     }
@@ -696,6 +703,30 @@ static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor
 
 static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_query,
                                          boat_tensor_t** grad_key, boat_tensor_t** grad_value);
+static boat_tensor_t* g_sum_into = NULL;   /* set by boat_attention_backward_self for the duration of one call */
+bool boat_attention_backward_self(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_input) {
+    *grad_input = NULL;
+    boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
+    const bool same = a && a->cache_query && a->cache_query == a->cache_key && a->cache_query == a->cache_value;
+    g_sum_into = same ? (boat_tensor_t*)a->cache_query : NULL;   /* non-NULL: sum the three input gradients into the first */
+    const bool ok = attention_backward_unflushed(a, grad_output, &gq, &gk, &gv);
+    g_sum_into = NULL;
+    bt_flush_exposed();
+    if (!ok) return false;
+    if (same) {          /* gk and gv are further references to gq */
+        boat_tensor_unref(gk);
+        boat_tensor_unref(gv);
+        *grad_input = gq;
+        return true;
+    }
+    /* the inputs were different tensors after all: add on the device */
+    boat_add_(gq, gk);
+    boat_add_(gq, gv);
+    boat_tensor_unref(gk);
+    boat_tensor_unref(gv);
+    *grad_input = gq;
+    return true;
+}
 bool boat_attention_backward(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_query,
                              boat_tensor_t** grad_key, boat_tensor_t** grad_value) {
     const bool ok = attention_backward_unflushed(a, grad_output, grad_query, grad_key, grad_value);
@@ -722,7 +753,7 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
     }
     /* 1. output projection */
     boat_tensor_t* d_ao = project_backward(a->cache_attention_output, a->weight_o, a->bias_o, grad_output, &a->grad_weight_o,
-                                           &a->grad_bias_o, rows, h);
+                                           &a->grad_bias_o, rows, h, NULL);
     if (!d_ao) return false;
     /* 2. attention core on [B*nh, S, hd] blocks */
     boat_tensor_t* dqp = bt_new_like_uninit(q);
@@ -738,9 +769,11 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
     boat_tensor_free(d_ao);
     /* 3. input projections */
     boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
-    if (ok) gq = project_backward(a->cache_query, a->weight_q, a->bias_q, dqp, &a->grad_weight_q, &a->grad_bias_q, rows, h);
-    if (ok && gq) gk = project_backward(a->cache_key, a->weight_k, a->bias_k, dkp, &a->grad_weight_k, &a->grad_bias_k, rows, h);
-    if (ok && gk) gv = project_backward(a->cache_value, a->weight_v, a->bias_v, dvp, &a->grad_weight_v, &a->grad_bias_v, rows, h);
+    /* self-attention through the tape: the key and value projections add their input gradients into the query's */
+    const bool sum = g_sum_into != NULL;
+    if (ok) gq = project_backward(a->cache_query, a->weight_q, a->bias_q, dqp, &a->grad_weight_q, &a->grad_bias_q, rows, h, NULL);
+    if (ok && gq) gk = project_backward(a->cache_key, a->weight_k, a->bias_k, dkp, &a->grad_weight_k, &a->grad_bias_k, rows, h, sum ? gq : NULL);
+    if (ok && gk) gv = project_backward(a->cache_value, a->weight_v, a->bias_v, dvp, &a->grad_weight_v, &a->grad_bias_v, rows, h, sum ? gq : NULL);
     boat_tensor_free(dqp);
     boat_tensor_free(dkp);
     boat_tensor_free(dvp);

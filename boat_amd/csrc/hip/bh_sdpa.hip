@@ -83,6 +83,27 @@ __global__ __launch_bounds__(kSBlock) void sdpa_fwd_row_kernel(const float* __re
     }
 }
 
+// delta for head sizes that are a multiple of 4 and at most 256: d/4 lanes per row (a power of two), each one 16-byte
+// piece of O and dO, rows packed into the wavefront; the lanes of a row fold through the wavefront
+template <int LANES>
+__global__ __launch_bounds__(kSBlock) void sdpa_delta_vec_kernel(const float* __restrict__ o, const float* __restrict__ d_out,
+                                                                 float* __restrict__ delta, int64_t rows) {
+    constexpr int ROWS_PER_BLOCK = kSBlock / LANES;
+    const int sub = threadIdx.x % LANES;
+    const int64_t r = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LANES;
+    float acc = 0.f;
+    if (r < rows) {
+        const float4 a = reinterpret_cast<const float4*>(o)[r * LANES + sub];
+        const float4 b = reinterpret_cast<const float4*>(d_out)[r * LANES + sub];
+        acc = (a.x * b.x + a.y * b.y) + (a.z * b.z + a.w * b.w);
+    }
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (sub == 0 && r < rows) delta[r] = acc;
+}
+
+static void launch_delta(const float* o, const float* d_out, float* delta, int64_t rows, int64_t d);
+
 // delta[i] = sum_d dO[i,d] * O[i,d], one wavefront per row
 __global__ __launch_bounds__(kSBlock) void sdpa_delta_kernel(const float* __restrict__ o, const float* __restrict__ d_out,
                                                              float* __restrict__ delta, int64_t rows, int64_t d) {
@@ -93,6 +114,20 @@ __global__ __launch_bounds__(kSBlock) void sdpa_delta_kernel(const float* __rest
     for (int64_t t = lane; t < d; t += 64) acc += o[r * d + t] * d_out[r * d + t];
     acc = wave_sum(acc);
     if (lane == 0) delta[r] = acc;
+}
+
+static void launch_delta(const float* o, const float* d_out, float* delta, int64_t rows, int64_t d) {
+    const bool al = ((reinterpret_cast<uintptr_t>(o) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0;
+#define DELTA_VEC(L)                                                                                                      \
+    hipLaunchKernelGGL((sdpa_delta_vec_kernel<L>), dim3((unsigned)ceil_div(rows, kSBlock / L)), dim3(kSBlock), 0, stream(), o, \
+                       d_out, delta, rows)
+    if (al && d == 64 && ceil_div(rows, kSBlock / 16) <= 0x7fffffff) DELTA_VEC(16);
+    else if (al && d == 128 && ceil_div(rows, kSBlock / 32) <= 0x7fffffff) DELTA_VEC(32);
+    else if (al && d == 32 && ceil_div(rows, kSBlock / 8) <= 0x7fffffff) DELTA_VEC(8);
+    else
+        hipLaunchKernelGGL(sdpa_delta_kernel, dim3((unsigned)ceil_div(rows, kSBlock / 64)), dim3(kSBlock), 0, stream(), o, d_out,
+                           delta, rows, d);
+#undef DELTA_VEC
 }
 
 // ---- general backward, dQ: block per (head-block, query row) ----
@@ -329,8 +364,7 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
     const int64_t rows = bh_count * s;
     float* delta = (float*)bh_malloc(sizeof(float) * (size_t)rows);
     if (!delta) return BH_ENOMEM;
-    hipLaunchKernelGGL(sdpa_delta_kernel, dim3((unsigned)ceil_div(rows, kSBlock / 64)), dim3(kSBlock), 0, stream(), out,
-                       d_out, delta, rows, d);
+    launch_delta(out, d_out, delta, rows, d);
     int rc = BH_LAUNCH_CHECK("sdpa_delta_kernel");
     if (rc == BH_OK) {
         int done = 1;

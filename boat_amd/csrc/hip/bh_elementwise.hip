@@ -28,17 +28,20 @@ static inline int grid_for(int64_t work_items) {
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // out[i] = f(in0[i], in1[i], in2[i], out[i]); NIN inputs are read, out is read when RO.
-// One float4 per lane per input, one workgroup per 256 float4: the grid is as large as the data, so
+// One float4 per lane per input, one single-wavefront workgroup per 64 float4: the grid is as large as the data, so
 // the resident workgroups sweep memory as one contiguous moving window (measured faster on MI355X
 // than a persistent grid-stride loop), and the accesses are marked non-temporal (streamed once).
+// Workgroups of one wavefront: a compute unit takes a new one whenever any wavefront slot frees (measured on the
+// seven-stream Adam step: 6.44 TB/s with 64 lanes per workgroup, 6.06 with 256, 5.85 with 1024).
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kVecBlock = 64;
 
 template <int NIN, bool RO, typename F>
-__global__ __launch_bounds__(kBlock) void ew_vec4(F f, float* __restrict__ out, const float* __restrict__ in0,
+__global__ __launch_bounds__(kVecBlock) void ew_vec4(F f, float* __restrict__ out, const float* __restrict__ in0,
                                                   const float* __restrict__ in1, const float* __restrict__ in2,
                                                   int64_t n) {
     const int64_t n4 = n >> 2;
-    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t i = (int64_t)blockIdx.x * kVecBlock + threadIdx.x;
     if (i < n4) {
         const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
         f32x4 a = NIN > 0 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(in0) + i) : zero;
@@ -75,9 +78,9 @@ static int launch_ew(const char* name, F f, float* out, const float* in0, const 
     const bool vec = aligned16(out) && (NIN < 1 || aligned16(in0)) && (NIN < 2 || aligned16(in1)) &&
                      (NIN < 3 || aligned16(in2));
     if (vec) {
-        const int64_t blocks = ceil_div((n >> 2) > 0 ? (n >> 2) : 1, kBlock);
+        const int64_t blocks = ceil_div((n >> 2) > 0 ? (n >> 2) : 1, kVecBlock);
         if (blocks > 0x7fffffff) return set_error(BH_EINVAL, "%s: tensor too large", name);
-        hipLaunchKernelGGL((ew_vec4<NIN, RO, F>), dim3((unsigned)blocks), dim3(kBlock), 0, stream(), f, out, in0, in1,
+        hipLaunchKernelGGL((ew_vec4<NIN, RO, F>), dim3((unsigned)blocks), dim3(kVecBlock), 0, stream(), f, out, in0, in1,
                            in2, n);
     } else {
         hipLaunchKernelGGL((ew_scalar<NIN, RO, F>), dim3(grid_for(n)), dim3(kBlock), 0, stream(), f, out, in0, in1,

@@ -505,6 +505,39 @@ __global__ __launch_bounds__(256) void splitk_fold_kernel(const float* __restric
     }
 }
 
+// the same for a dense output (ldc == n, batches back to back) whose size is a multiple of 4: one 16-byte piece per
+// lane, single-wavefront workgroups, the grid as large as the output, everything streamed once.  The partials are
+// summed in the order of the splits, as in the scalar kernel.
+typedef float fold_f32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(64) void splitk_fold_vec_kernel(const float* __restrict__ ws, float* __restrict__ c,
+                                                             const float* __restrict__ bias, int64_t total4, int64_t n,
+                                                             int splits, int accumulate) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= total4) return;
+    const fold_f32x4* w4 = reinterpret_cast<const fold_f32x4*>(ws);
+    fold_f32x4 acc = __builtin_nontemporal_load(w4 + i);
+    // four partials in flight at a time
+    int sp = 1;
+    for (; sp + 3 < splits; sp += 4) {
+        const fold_f32x4 a = __builtin_nontemporal_load(w4 + (int64_t)sp * total4 + i);
+        const fold_f32x4 b = __builtin_nontemporal_load(w4 + (int64_t)(sp + 1) * total4 + i);
+        const fold_f32x4 d = __builtin_nontemporal_load(w4 + (int64_t)(sp + 2) * total4 + i);
+        const fold_f32x4 e = __builtin_nontemporal_load(w4 + (int64_t)(sp + 3) * total4 + i);
+        acc += a;
+        acc += b;
+        acc += d;
+        acc += e;
+    }
+    for (; sp < splits; sp++) acc += __builtin_nontemporal_load(w4 + (int64_t)sp * total4 + i);
+    if (bias) {
+        const int64_t col = (i * 4) % n;    // n % 4 == 0: the four elements share a row
+        acc += *reinterpret_cast<const fold_f32x4*>(bias + col);
+    }
+    fold_f32x4* dst = reinterpret_cast<fold_f32x4*>(c) + i;
+    if (accumulate) acc = __builtin_nontemporal_load(dst) + acc;
+    __builtin_nontemporal_store(acc, dst);
+}
+
 // many partials of a small output (a long contraction cut into hundreds of chunks): one wavefront per output element,
 // the lanes striding over the partials
 __global__ __launch_bounds__(256) void splitk_fold_wide_kernel(const float* __restrict__ ws, float* __restrict__ c,
@@ -999,6 +1032,11 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
     if (splits >= 32 && total <= 16384) {
         hipLaunchKernelGGL(splitk_fold_wide_kernel, dim3((unsigned)ceil_div(total, 4)), dim3(256), 0, stream(), ws, c, bias, m, n, ldc,
                            splits, batch, stride_c, accumulate);
+    } else if (ldc == n && (batch == 1 || stride_c == m * n) && n % 4 == 0 &&
+               ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(bias)) & 15) == 0 &&
+               ceil_div(total / 4, 64) <= 0x7fffffff) {
+        hipLaunchKernelGGL(splitk_fold_vec_kernel, dim3((unsigned)ceil_div(total / 4, 64)), dim3(64), 0, stream(), ws, c, bias,
+                           total / 4, n, splits, accumulate);
     } else {
         int64_t blocks = ceil_div(total, 256);
         if (blocks > 4096) blocks = 4096;
@@ -1008,6 +1046,7 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
     return BH_LAUNCH_CHECK("splitk_fold_kernel");
 }
 
+static int g_force_splits = 0;    // test hook: > 0 = this many k-splits for the MFMA tiles
 static int g_pairs = 1;           // test hook: 0 = the big tile keeps one k-tile per barrier
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
 static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, 6 = tiny, -1 = heuristic
@@ -1021,6 +1060,12 @@ extern "C" {
 // test/benchmark hook: pin the kernel choice (-1 restores the heuristic)
 int bh_gemm_force_config(int cfg) {
     g_force_cfg = cfg;
+    return BH_OK;
+}
+
+// test/benchmark hook: number of k-splits where the heuristic would split (0 restores the heuristic)
+int bh_gemm_force_splits(int splits) {
+    g_force_splits = splits;
     return BH_OK;
 }
 
@@ -1058,6 +1103,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     bool vec_ok = al16(a) && al16(b) && (lda % 4 == 0) && (ldb % 4 == 0) && k > 0;
     vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
     int cfg;   // 0 fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256
+    int plan_splits = 0;   // > 0: the tile choice below came with its own number of k-splits
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
@@ -1067,6 +1113,20 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         // it and the 128x128 tile; narrow outputs keep the small tile
         const int64_t big_tiles = ceil_div(m, 256) * ceil_div(n, 256);
         if (big_tiles >= 256) cfg = 2;
+        else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096 && (256 / big_tiles) * 2048 <= k) {
+            // a mid-sized output under a long contraction (the weight gradient of a wide layer): 256x256 tiles with the
+            // contraction cut so that the tiles fill the chip once, at least 2048 k each (4096x1024x8192: 512 us with
+            // the fold against 530 for two-way split 128x256 tiles)
+            cfg = 2;
+            plan_splits = (int)(256 / big_tiles);
+        } else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096) {
+            // smaller still (1024x1024x8192): 128x128 tiles, two workgroups per compute unit, 1024 k each where that
+            // fills the chip (145 us with the fold against 155 for sixteen-way split 128x256 tiles)
+            cfg = 1;
+            const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128);
+            plan_splits = (int)ceil_div(512, t128);
+            while (plan_splits > 1 && k / plan_splits < 1024) plan_splits--;
+        }
         else if (n >= 192 && m >= 96) cfg = 4;
         else if (m >= 192 && n >= 96) cfg = 3;
         else cfg = 1;
@@ -1210,6 +1270,8 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         int64_t splits = ceil_div(512, tiles);
         if (splits > k / min_k) splits = k / min_k;
         if (splits > 32) splits = 32;
+        if (plan_splits > 0 && g_force_cfg < 0) splits = plan_splits;
+        if (g_force_splits > 0 && g_force_splits <= k / kBK) splits = g_force_splits;
         if (splits > 1) {
             g.k_per_split = ceil_div(ceil_div(k, splits), kBK) * kBK;
             g.k_splits = (int)ceil_div(k, g.k_per_split);

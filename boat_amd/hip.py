@@ -59,7 +59,7 @@ _SIGS = {
     "bh_scalar_op_typed": (I, [I, I, P, C.c_double, P, L]),
     "bh_layernorm_backward_noalloc": (I, [P, P, P, P, P, P, P, P, L, L, I]),
     "bh_gemm": (I, [I, I, L, L, L, P, L, P, L, P, L, P, I, L]),
-    "bh_gemm_force_config": (I, [I]), "bh_gemm_force_direct": (I, [I]),
+    "bh_gemm_force_config": (I, [I]), "bh_gemm_force_direct": (I, [I]), "bh_gemm_force_splits": (I, [I]),
     "bh_transpose_last2": (I, [P, P, L, L, L]),
     "bh_dense_backward": (I, [P, P, P, P, P, P, L, L, L, I]),
     "bh_sdpa_forward": (I, [P, P, P, F, I, P, P, P, L, L, L]),

@@ -248,10 +248,12 @@ int bh_zero_multi(float* const* p, const int64_t* n, int count);
  * bh_gemm products with row kernels for softmax and dS in between, what shapes other than head_dim 64 use from 64 keys on). */
 int bh_gemm_force_config(int cfg);
 int bh_gemm_force_direct(int mode);
+/* bh_gemm_force_splits: where the MFMA tiles would split the contraction, split it this many ways (0 = heuristic) */
+int bh_gemm_force_splits(int splits);
 int bh_sdpa_force_general(int on);
-/* bh_layernorm_tune: cap on the workgroups of the LayerNorm backward (each writes one dgamma/dbeta partial);
- * 0 keeps the current value.  The second argument is reserved. */
-int bh_layernorm_tune(int bwd_blocks, int reserved);
+/* bh_layernorm_tune: cap on the workgroups of the LayerNorm backward (each writes one dgamma/dbeta partial) and of
+ * the forward; 0 keeps the current value. */
+int bh_layernorm_tune(int bwd_blocks, int fwd_blocks);
 
 #ifdef __cplusplus
 }

@@ -452,6 +452,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     if (g.k_splits > 1) C += (int64_t)split * gridDim.y * g.stride_c;
     const bool add_c = g.accumulate && g.k_splits <= 1;
     const float* bias = g.k_splits <= 1 ? g.bias : nullptr;
+    // a lane's TN columns are the same for every row it stores: their bias values are fetched once, not once per element
+    float bias_v[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
+        bias_v[j] = (bias && col < g.n) ? bias[col] : 0.f;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -465,8 +472,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                 for (int j = 0; j < TN; j++) {
                     const int64_t col = n0 + wn * Cfg::WN + j * 32 + r;
                     if (col < g.n) {
-                        float v = acc[i][j][e];
-                        if (bias) v += bias[col];
+                        float v = acc[i][j][e] + bias_v[j];
                         if (add_c) v += crow[col];
                         crow[col] = v;
                     }
@@ -477,8 +483,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                 for (int j = 0; j < TN; j++) {
                     const int64_t col = col0 + j;
                     if (col < g.n) {
-                        float v = acc[i][j][e];
-                        if (bias) v += bias[col];
+                        float v = acc[i][j][e] + bias_v[j];
                         if (add_c) v += crow[col];
                         crow[col] = v;
                     }
@@ -1344,13 +1349,19 @@ int bh_swap_dims_f64(const double* in, double* out, int64_t a, int64_t d0, int64
 
 int bh_dense_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t m,
                       int64_t k, int64_t n, int accumulate) {
+    return bh_dense_backward_into(x, w, dy, dx, gw, gb, m, k, n, accumulate, 0);
+}
+
+int bh_dense_backward_into(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t m,
+                           int64_t k, int64_t n, int accumulate, int accumulate_dx) {
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(m >= 0 && k >= 0 && n >= 0, "negative dimension");
     BH_CHECK_ARG(x && w && dy, "null pointer");
     int rc = BH_OK;
-    // dX[m,k] = dY[m,n] . W[k,n]^T
-    if (dx) rc = bh_gemm(0, 1, m, k, n, dy, n, w, n, dx, k, nullptr, 0, 1);
+    // dX[m,k] (+)= dY[m,n] . W[k,n]^T
+    if (dx) rc = bh_gemm(0, 1, m, k, n, dy, n, w, n, dx, k, nullptr, accumulate_dx, 1);
     // dW[k,n] (+)= X[m,k]^T . dY[m,n]
+    // (running the two products side by side on two streams was measured: 6.30 ms per block step against 5.88)
     if (rc == BH_OK && gw) rc = bh_gemm(1, 0, k, n, m, x, k, dy, n, gw, n, nullptr, accumulate, 1);
     if (rc == BH_OK && gb) rc = bh_colsum(dy, gb, m, n, accumulate);
     return rc;

@@ -692,8 +692,7 @@ static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor
     float* pgb = bias ? bt_dev_write(*gb) : NULL;
     bool ok = px && pw && pdy && pdx && pgw;
     /* dx (+)= dy.w^T ; gw = x^T.dy ; gb = colsum(dy) */
-    if (ok) ok = boat_hip_ok(bh_gemm(0, 1, rows, h, h, pdy, h, pw, h, pdx, h, NULL, into ? 1 : 0, 1), "attention projection backward");
-    if (ok) ok = boat_hip_ok(bh_dense_backward(px, pw, pdy, NULL, pgw, pgb, rows, h, h, 0), "attention projection backward");
+    if (ok) ok = boat_hip_ok(bh_dense_backward_into(px, pw, pdy, pdx, pgw, pgb, rows, h, h, 0, into ? 1 : 0), "attention projection backward");
     if (!ok) {
         boat_tensor_free(dx);
         return NULL;

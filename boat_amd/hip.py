@@ -62,6 +62,7 @@ _SIGS = {
     "bh_gemm_force_config": (I, [I]), "bh_gemm_force_direct": (I, [I]), "bh_gemm_force_splits": (I, [I]),
     "bh_transpose_last2": (I, [P, P, L, L, L]),
     "bh_dense_backward": (I, [P, P, P, P, P, P, L, L, L, I]),
+    "bh_dense_backward_into": (I, [P, P, P, P, P, P, L, L, L, I, I]),
     "bh_sdpa_forward": (I, [P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_backward": (I, [P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_force_general": (I, [I]),

@@ -187,6 +187,12 @@ int bh_swap_dims_f64(const double* in, double* out, int64_t a, int64_t d0, int64
 int bh_dense_backward(const float* x, const float* w, const float* dy,
                       float* dx, float* gw, float* gb, int64_t m, int64_t k, int64_t n,
                       int accumulate);
+/* the same with the input gradient added into dx when accumulate_dx != 0 (the key and value projections of a
+ * self-attention layer add into the query projection's input gradient, src/layers/attention.c:1186-1285 run three times
+ * on one input) */
+int bh_dense_backward_into(const float* x, const float* w, const float* dy,
+                           float* dx, float* gw, float* gb, int64_t m, int64_t k, int64_t n,
+                           int accumulate, int accumulate_dx);
 
 /* ---- scaled dot-product attention on [bh, s, d] blocks (src/layers/attention.c:882-1079,1388-1534) ----
  * forward keeps O and the row log-sum-exp instead of the reference's [bh,s,s] softmax matrix;

@@ -459,6 +459,34 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
         bias_v[j] = (bias && col < g.n) ? bias[col] : 0.f;
     }
+    // accumulate: the old values of one 32-row slab are fetched by loads that depend on nothing, then added; a load
+    // placed between the stores below would have to wait for them (the compiler cannot tell the rows apart)
+    // (wavefront tiles of 128x64 have no registers to spare for this and keep the load next to its store)
+    constexpr bool kPrefetchC = TM * TN <= 4;
+    if (kPrefetchC && add_c) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int eg = 0; eg < 16; eg += 8) {
+                float prev[8][TN];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int ri = ((eg + e) >> 2) * 8 + half * 4 + (e & 3);
+                    const int64_t row = m0 + wm * Cfg::WM + (A_KC ? i * 32 + ri : TM * ri + i);
+                    const float* crow = C + row * g.ldc;
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
+                        prev[e][j] = (row < g.m && col < g.n) ? __builtin_nontemporal_load(crow + col) : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j][eg + e] += prev[e][j];
+            }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -467,26 +495,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             const int64_t row = m0 + wm * Cfg::WM + (A_KC ? i * 32 + ri : TM * ri + i);
             if (row >= g.m) continue;
             float* crow = C + row * g.ldc;
-            if (B_KC) {
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int64_t col = n0 + wn * Cfg::WN + j * 32 + r;
-                    if (col < g.n) {
-                        float v = acc[i][j][e] + bias_v[j];
-                        if (add_c) v += crow[col];
-                        crow[col] = v;
-                    }
-                }
-            } else {
-                const int64_t col0 = n0 + wn * Cfg::WN + TN * r;
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int64_t col = col0 + j;
-                    if (col < g.n) {
-                        float v = acc[i][j][e] + bias_v[j];
-                        if (add_c) v += crow[col];
-                        crow[col] = v;
-                    }
+            for (int j = 0; j < TN; j++) {
+                const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
+                if (col < g.n) {
+                    float v = acc[i][j][e] + bias_v[j];
+                    if (!kPrefetchC && add_c) v += crow[col];
+                    crow[col] = v;
                 }
             }
         }

@@ -43,6 +43,8 @@ METRIC = "backward+Adam step ms; GB/s & TFLOP/s as % of MI355X roofline (1 GPU)"
 # a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).  A constant taken from that profile, not a
 # measurement of this run.
 GEMM_TRAFFIC_BYTES_CONFIG2 = int((2.0 * 409880.2 + 98304.0) * 1024)
+# HBM bytes per GEMM launch of the block training step, averaged over the step's 18 launches (same file, same counters)
+GEMM_TRAFFIC_BYTES_STEP = 268_700_000
 
 
 def parse_args():
@@ -534,7 +536,9 @@ def bench_training_step(hip, steps, warmup):
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(g_ms / max(g_calls, 1), 4), "flops_per_launch": g_flops / max(g_calls, 1),
-            "launches_per_step": g_calls, "traffic": None,
+            "launches_per_step": g_calls, "traffic": GEMM_TRAFFIC_BYTES_STEP,
+            "traffic_source": "profile constant (profiles/pmc_hbm_traffic_and_mfma.md: 2.0 x FETCH_SIZE + WRITE_SIZE per launch, averaged "
+                              "over the step's launches), not measured in this run",
             "measured": "HIP event pairs around each bh_gemm launch of K further steps run right after the timed K (the events "
                         "themselves cost about 5 us each on the stream, so they stay out of the timed region)",
         },

@@ -365,11 +365,48 @@ def bench_cnn_step(steps, warmup):
     ms = (time.perf_counter() - t0) * 1e3 / steps
     step(keep_loss=True)
     assert np.isfinite(losses).all() and losses[1] < losses[0], f"CNN training does not reduce the loss: {losses}"
+    # the same loop with the 32->64 layer's forward on the matrix cores (opt-in: not bit-identical to the reference)
+    api.boat_hip_conv_forward_matrix_cores(1)
+    warm_clocks(api.sync, step, warmup)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.sync()
+    ms_mfma = (time.perf_counter() - t0) * 1e3 / steps
+    api.boat_hip_conv_forward_matrix_cores(0)
     conv_flops = 2.0 * B * (32 * 1 * 9 * 28 * 28 + 64 * 32 * 9 * 14 * 14) * 3       # forward + dX + dW of both conv layers
     return {"ms": round(ms, 4), "bound": "launch latency / small kernels", "conv_flops": conv_flops,
+            "ms_conv_forward_on_matrix_cores": round(ms_mfma, 4), "conv_forward_kernels": bench_conv_forward_kernels(),
             "loss_first_last": [round(l, 6) for l in losses],
             "note": "MNIST CNN B64 (conv 1->32, conv 32->64, dense 3136->128->10): fwd + bwd + Adam + zero_grad through the "
                     "C API from Python, wall clock"}
+
+
+def bench_conv_forward_kernels():
+    """bh_conv2d_forward (direct, the reference's operation order) against bh_conv2d_forward_mfma (one contraction on the
+    fp32 matrix cores) on the MNIST network's 32->64 layer at batch 64 and on a layer with many channels; HIP events."""
+    from boat_amd import hip
+    rng = np.random.default_rng(20250108)
+    out = {}
+    for name, (B, ic, h, w, oc) in (("64x32x14x14_to_64", (64, 32, 14, 14, 64)), ("32x128x28x28_to_256", (32, 128, 28, 28, 256))):
+        x = hip.to_device(rng.standard_normal((B, ic, h, w), dtype=np.float32))
+        wt = hip.to_device((0.1 * rng.standard_normal((oc, ic, 3, 3), dtype=np.float32)).astype(np.float32))
+        b = hip.to_device(rng.standard_normal(oc, dtype=np.float32))
+        y = hip.empty((B, oc, h, w))
+        flops = 2.0 * B * oc * h * w * ic * 9
+        res = {}
+        for label, fn in (("direct", hip.bh_conv2d_forward), ("matrix_cores", hip.bh_conv2d_forward_mfma)):
+            call = lambda: hip.check(fn(x.ptr, wt.ptr, b.ptr, y.ptr, B, ic, h, w, oc, 3, 1, 1))
+            warm_clocks(hip.synchronize, call, 10)
+            timer = hip.Timer()
+            with timer:
+                for _ in range(50):
+                    call()
+            ms = timer.ms / 50
+            res[label] = {"us": round(ms * 1e3, 1), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1)}
+        res["speedup"] = round(res["direct"]["us"] / res["matrix_cores"]["us"], 2)
+        out[name] = res
+    return out
 
 
 class Block:

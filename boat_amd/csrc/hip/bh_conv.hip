@@ -32,6 +32,7 @@
 namespace bh {
 
 constexpr int kCBlock = 256;
+typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 struct ConvShape {
     int batch, ic, h, w, oc, k, stride, pad, ho, wo;
@@ -137,6 +138,156 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_generic_kernel(const float
     }
     if (bias) out += bias[oc];
     y[i] = out;
+}
+
+// ---- forward on the matrix cores, 3x3 kernels (opt-in: the sums run in MFMA order, so the result agrees with the
+// reference to rounding, not bit for bit, and a pooling layer behind it may pick another of two near-equal maxima) ----
+// The convolution as one contraction y[oc][n] = sum_kk w[oc][kk] * patch[kk][n], kk = (ci, kh, kw), n = (b, oh, ow),
+// on v_mfma_f32_32x32x2_f32 without a patch matrix in memory: output channel = accumulator row, output position =
+// lane, so a lane fetches the patch values of its own position straight from x (neighbouring lanes read neighbouring
+// pixels; taps outside the image and channels past the last read a clamped address and count as zero) and the stores
+// of one accumulator register are 32 consecutive positions of one channel plane.  One matrix instruction contracts two
+// consecutive kk; the lane half decides which of the two a lane supplies, so per pair of input channels (18 kk) a lane
+// needs nine patch values and, per 32 output channels, nine weights.  The weights of the workgroup's 64 output channels
+// and of up to 32 input channels sit in LDS, split by kk parity ([oc][kk & 1][kk >> 1], row stride odd: conflict free
+// 4-byte reads).
+// Workgroup: 8 wavefronts = 64 channels x 64 positions; a wavefront owns 32 positions, both 32-channel halves (a patch
+// value feeds two products) and every fourth pair of input channels: small layers are bound by the latency of the
+// patch loads, and four wavefronts per position tile have four times the loads in flight.  The four partial sums are
+// added in a fixed order through LDS.  grid (ceil(P/64), ceil(oc/64)).
+constexpr int kFmCi = 32;                       // input channels per LDS stage
+constexpr int kFmKk = kFmCi * 9;                // 288 contraction indices per stage
+constexpr int kFmRow = kFmKk + 1;               // LDS row stride in floats
+constexpr int kFmSplit = 4;                     // wavefronts that share a position tile
+
+__global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wt,
+                                                                 const float* __restrict__ bias, float* __restrict__ y,
+                                                                 ConvShape c, int positions) {
+    extern __shared__ __align__(16) float wl[];          // [64][kFmRow] + bias[64]; the weights' part holds the partial sums afterwards
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int wn = wv & 1, kg = wv >> 1;
+    const int oc0 = blockIdx.y * 64;
+    const int per = c.ho * c.wo, plane = c.h * c.w;
+    const int n_raw = blockIdx.x * 64 + wn * 32 + r;
+    const int n = min(n_raw, positions - 1);
+    const int b = n / per, p = n - b * per;
+    const int oh = p / c.wo, ow = p - oh * c.wo;
+    const int ih0 = oh * c.stride - c.pad, iw0 = ow * c.stride - c.pad;
+    // the nine contraction indices 2j + half of a channel pair: which of the two channels, pixel offset, inside the image?
+    int off[9];
+    unsigned inside = 0, second_bits = 0;
+#pragma unroll
+    for (int j = 0; j < 9; j++) {
+        const int kk = 2 * j + half, cp = kk >= 9 ? 1 : 0, tap = kk - 9 * cp;
+        const int kh = tap / 3, kw = tap - 3 * kh;
+        const int ih = ih0 + kh, iw = iw0 + kw;
+        if (ih >= 0 && ih < c.h && iw >= 0 && iw < c.w) inside |= 1u << j;
+        second_bits |= (unsigned)cp << j;
+        off[j] = min(max(ih, 0), c.h - 1) * c.w + min(max(iw, 0), c.w - 1);
+    }
+    const float* xp = x + (int64_t)b * c.ic * plane;      // 32-bit offsets from here on: a tensor has fewer than 2^30 elements
+    const float* wrow = wl + r * kFmRow + half * (kFmKk / 2);
+    floatx16 acc[2];
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[0][e] = acc[1][e] = 0.f;
+
+    // patch values of channels ci, ci + 1: the loads go to clamped (valid) addresses and nothing looks at their results
+    // until mask() runs three turns later -- a select right behind a load would make the wavefront wait for it there
+    const auto fetch = [&](int ci, float (&v)[9]) {
+#pragma unroll
+        for (int j = 0; j < 9; j++) v[j] = xp[min(ci + (int)((second_bits >> j) & 1u), c.ic - 1) * plane + off[j]];
+    };
+    const auto mask = [&](int ci, float (&v)[9]) {         // taps outside the image and channels past the last count as zero
+#pragma unroll
+        for (int j = 0; j < 9; j++) v[j] = (((inside >> j) & 1u) && ci + (int)((second_bits >> j) & 1u) < c.ic) ? v[j] : 0.f;
+    };
+    const int l16 = tid & 15, rg = tid >> 4;               // weight staging: 16 lanes per row, 32 rows per pass
+    // the bias of the 64 channels travels with the first stage's weights and waits in LDS behind them: fetched at the end
+    // it would cost a trip to memory of its own
+    float* bl = wl + 64 * kFmRow;
+    float bias_in = 0.f;
+    if (tid < 64 && bias && oc0 + tid < c.oc) bias_in = bias[oc0 + tid];
+    for (int ci0 = 0; ci0 < c.ic; ci0 += kFmCi) {
+        if (ci0) __syncthreads();                          // every wavefront is done with the previous stage's weights
+        const int chunk = min(kFmCi, c.ic - ci0);
+        const int pairs = (chunk + 1) / 2, real = chunk * 9;
+        // this wavefront's pairs are kg, kg + 4, ...; their patch values run three turns ahead (a turn's 18 products take
+        // a quarter of a trip to memory), the first three fetches of a stage are in flight while its weights are staged
+        float x0[9], x1[9], x2[9], x3[9];
+        fetch(ci0 + 2 * kg, x0);
+        fetch(ci0 + 2 * (kg + kFmSplit), x1);
+        fetch(ci0 + 2 * (kg + 2 * kFmSplit), x2);
+        // weights of the stage: row oc of w holds its ic*9 values contiguously, so a stage's run of chunk*9 is contiguous;
+        // what lies past it (an odd channel count's partner, a short last stage) is zero.  A lane's 36 loads are in flight
+        // together before their LDS stores.
+        {
+            float v[2][18];
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const int o = rg + 32 * q;
+                const float* src = wt + ((int64_t)min(oc0 + o, c.oc - 1) * c.ic + ci0) * 9;
+#pragma unroll
+                for (int i = 0; i < 18; i++) {
+                    const int kk = l16 + 16 * i;
+                    v[q][i] = (oc0 + o < c.oc && kk < real) ? src[kk] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                float* dst = wl + (rg + 32 * q) * kFmRow;
+#pragma unroll
+                for (int i = 0; i < 18; i++) {
+                    const int kk = l16 + 16 * i;
+                    dst[(kk & 1) * (kFmKk / 2) + (kk >> 1)] = v[q][i];
+                }
+            }
+        }
+        if (ci0 == 0 && tid < 64) bl[tid] = bias_in;
+        __syncthreads();
+        // the four buffers take turns (a register copy would have to wait for the loads it copies)
+        const auto products = [&](int cp, float (&cur)[9], float (&ahead)[9]) {
+            if (cp + 3 * kFmSplit < pairs) fetch(ci0 + 2 * (cp + 3 * kFmSplit), ahead);
+            mask(ci0 + 2 * cp, cur);
+            const float* wp = wrow + cp * 9;
+#pragma unroll
+            for (int j = 0; j < 9; j++) {
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], cur[j], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * kFmRow + j], cur[j], acc[1], 0, 0, 0);
+            }
+        };
+        for (int cp = kg; cp < pairs; cp += 4 * kFmSplit) {
+            products(cp, x0, x3);
+            if (cp + kFmSplit < pairs) products(cp + kFmSplit, x1, x0);
+            if (cp + 2 * kFmSplit < pairs) products(cp + 2 * kFmSplit, x2, x1);
+            if (cp + 3 * kFmSplit < pairs) products(cp + 3 * kFmSplit, x3, x2);
+        }
+    }
+    __syncthreads();                                       // the weights are no longer needed: their LDS holds the partial sums
+    if (kg > 0) {
+        float* red = wl + (((kg - 1) * 2 + wn) * 32) * 64 + lane;  // [kg - 1][wn][t * 16 + e][lane]
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) red[(t * 16 + e) * 64] = acc[t][e];
+    }
+    __syncthreads();
+    if (kg > 0 || n_raw >= positions) return;
+#pragma unroll
+    for (int g = 0; g < kFmSplit - 1; g++) {
+        const float* src = wl + ((g * 2 + wn) * 32) * 64 + lane;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[t][e] += src[(t * 16 + e) * 64];
+    }
+    float* yp = y + (int64_t)b * c.oc * per + p;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int oc = oc0 + t * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+            if (oc < c.oc) yp[(int64_t)oc * per] = acc[t][e] + bl[oc - oc0];
+        }
 }
 
 // dyp[oc][b][p] = dy[b][oc][p], p over the ho*wo output positions
@@ -347,6 +498,30 @@ int bh_conv2d_forward(const float* x, const float* w, const float* bias, float* 
                            bias, y, c, total);
     }
     return BH_LAUNCH_CHECK("conv2d_fwd_kernel");
+}
+
+int bh_conv2d_forward_mfma(const float* x, const float* w, const float* bias, float* y, int64_t batch, int64_t in_channels,
+                           int64_t height, int64_t width, int64_t out_channels, int64_t kernel, int64_t stride, int64_t pad) {
+    BH_REQUIRE_INIT();
+    ConvShape c;
+    int rc = make_conv_shape(c, batch, in_channels, height, width, out_channels, kernel, stride, pad);
+    if (rc) return rc;
+    BH_CHECK_ARG(kernel == 3, "conv2d on the matrix cores: 3x3 kernels only");
+    if (batch == 0) return BH_OK;
+    BH_CHECK_ARG(x && w && y, "null pointer");
+    const int64_t positions = (int64_t)c.batch * c.ho * c.wo;
+    BH_CHECK_ARG(ceil_div(c.oc, 64) <= 65535, "conv2d on the matrix cores: too many output channels");
+    constexpr size_t lds = sizeof(float) * (64 * kFmRow + 64);      // weights + bias
+    static bool attr = false;
+    if (!attr) {
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr = true;
+    }
+    const dim3 grid((unsigned)ceil_div(positions, 64), (unsigned)ceil_div(c.oc, 64));
+    hipLaunchKernelGGL(conv2d_fwd_mfma_kernel, grid, dim3(512), lds, stream(), x, w, bias, y, c, (int)positions);
+    return BH_LAUNCH_CHECK("conv2d_fwd_mfma_kernel");
 }
 
 int bh_conv2d_backward(const float* x, const float* w, const float* dy, float* dx, float* gw, float* gb, int64_t batch,

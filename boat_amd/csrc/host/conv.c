@@ -22,6 +22,18 @@
 static int g_reference_input_grad = -1;   /* -1: not set by a call, follow reference-exact mode */
 
 void boat_hip_conv_reference_input_grad(int enable) { g_reference_input_grad = enable < 0 ? -1 : enable != 0; }
+/* forward on the matrix cores (3x3 kernels with at least 8 input channels); off by default because the direct kernel's
+ * output is bit-identical to the reference's and the MFMA order is not.  BOAT_HIP_CONV_FORWARD_MFMA=1 in the
+ * environment sets the initial value. */
+static int g_forward_mfma = -1;
+void boat_hip_conv_forward_matrix_cores(int enable) { g_forward_mfma = enable != 0; }
+static int forward_mfma(void) {
+    if (g_forward_mfma < 0) {
+        const char* e = getenv("BOAT_HIP_CONV_FORWARD_MFMA");
+        g_forward_mfma = e && *e && *e != '0';
+    }
+    return g_forward_mfma;
+}
 static int reference_input_grad(void) { return g_reference_input_grad >= 0 ? g_reference_input_grad : (bt_reference_exact() ? 1 : 0); }
 
 struct boat_conv_layer_t {
@@ -100,8 +112,10 @@ boat_tensor_t* boat_conv_layer_forward(boat_conv_layer_t* l, const boat_tensor_t
     const float* pw = bt_dev_read(l->weight);
     const float* pb = (l->use_bias && l->bias) ? bt_dev_read(l->bias) : NULL;
     float* py = bt_dev_write(out);
+    const int mfma = forward_mfma() && k == 3 && l->in_channels >= 8;
     if (!px || !pw || !py ||
-        !boat_hip_ok(bh_conv2d_forward(px, pw, pb, py, batch, (int64_t)l->in_channels, h, w, (int64_t)l->out_channels, k, s, p),
+        !boat_hip_ok((mfma ? bh_conv2d_forward_mfma : bh_conv2d_forward)(px, pw, pb, py, batch, (int64_t)l->in_channels, h, w,
+                                                                         (int64_t)l->out_channels, k, s, p),
                      "conv forward")) {
         boat_tensor_free(out);
         return NULL;

@@ -68,6 +68,7 @@ _SIGS = {
     "bh_sdpa_force_general": (I, [I]),
     "bh_adam_update": (I, [P, P, P, P, L, F, F, F, F, L]),
     "bh_conv2d_forward": (I, [P, P, P, P] + [L] * 8),
+    "bh_conv2d_forward_mfma": (I, [P, P, P, P] + [L] * 8),
     "bh_conv2d_backward": (I, [P, P, P, P, P, P] + [L] * 8 + [I, I]),
     "bh_maxpool2d_forward": (I, [P, P, P] + [L] * 6),
     "bh_maxpool2d_backward": (I, [P, P, P] + [L] * 6),

@@ -515,6 +515,32 @@ def test_conv_known_answer_and_hooks(boat):
     boat.boat_conv_layer_free(layer)
 
 
+def test_conv_forward_on_the_matrix_cores_is_opt_in(boat, oracle, rng):
+    """boat_conv_layer_forward is bit-identical to the reference's loop order by default (src/layers/conv.c:326-437); after
+    boat_hip_conv_forward_matrix_cores(1) a 3x3 layer with at least 8 input channels runs as one MFMA contraction and
+    agrees to fp32 rounding; layers the switch does not cover (few channels, other kernel sizes) stay bit-identical."""
+    x = rng.standard_normal((4, 16, 10, 9)).astype(np.float32)
+    w = (0.2 * rng.standard_normal((24, 16, 3, 3))).astype(np.float32)
+    b = rng.standard_normal(24).astype(np.float32)
+    want = oracle.conv2d_forward(x, w, b, 1, 1)
+    y_default, _ = bc.conv_layer(boat, x, w, b, 1, 1, [])
+    assert np.array_equal(y_default, want)
+    x_small = rng.standard_normal((2, 3, 8, 8)).astype(np.float32)
+    w_small = (0.2 * rng.standard_normal((5, 3, 3, 3))).astype(np.float32)
+    b_small = rng.standard_normal(5).astype(np.float32)
+    boat.boat_hip_conv_forward_matrix_cores(1)
+    try:
+        y_mfma, grads = bc.conv_layer(boat, x, w, b, 1, 1, [np.ones_like(want)])
+        y_small, _ = bc.conv_layer(boat, x_small, w_small, b_small, 1, 1, [])
+    finally:
+        boat.boat_hip_conv_forward_matrix_cores(0)
+    assert np.max(np.abs(y_mfma - want)) <= 1e-5 * np.abs(want).max()
+    assert grads[0][2].tolist() == [4.0 * 10 * 9] * 24                      # the backward hooks are untouched
+    assert np.array_equal(y_small, oracle.conv2d_forward(x_small, w_small, b_small, 1, 1))
+    y_again, _ = bc.conv_layer(boat, x, w, b, 1, 1, [])
+    assert np.array_equal(y_again, want)
+
+
 def test_flatten_layer_round_trip(boat, rng):
     x = rng.standard_normal((3, 2, 4, 5)).astype(np.float32)
     layer = boat.boat_flatten_layer_create()

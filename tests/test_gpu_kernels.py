@@ -623,6 +623,34 @@ def test_conv2d_forward_output_channel_tiles(hip, oracle, rng, shape):
     assert np.array_equal(y.numpy(), oracle.conv2d_forward(x, wt, b, stride, pad))
 
 
+CONV_MFMA_SHAPES = [  # batch, ic, h, w, oc, k(=3), stride, pad: ragged channel counts, odd channel counts, strides, two LDS stages
+    (2, 3, 7, 6, 4, 3, 1, 1), (3, 1, 8, 8, 5, 3, 1, 0), (2, 3, 10, 10, 2, 3, 3, 0), (1, 5, 3, 3, 70, 3, 1, 1),
+    (8, 32, 14, 14, 64, 3, 1, 1), (64, 32, 14, 14, 64, 3, 1, 1), (3, 33, 9, 11, 65, 3, 2, 1), (2, 70, 6, 6, 40, 3, 1, 2),
+]
+
+
+@pytest.mark.parametrize("shape", CONV_MFMA_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_conv2d_forward_on_the_matrix_cores(hip, oracle, rng, shape):
+    """The opt-in forward (one contraction on the fp32 matrix cores) against the oracle in the reference's order
+    (src/layers/conv.c:326-437): equal to fp32 rounding -- the bound is the one only full fp32 accumulation meets."""
+    B, ic, h, w, oc, k, stride, pad = shape
+    ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    x = rng.standard_normal((B, ic, h, w)).astype(np.float32)
+    wt = (0.3 * rng.standard_normal((oc, ic, k, k))).astype(np.float32)
+    b = rng.standard_normal(oc).astype(np.float32)
+    dx_, dw_, db_ = dev(hip, x), dev(hip, wt), dev(hip, b)
+    for bias, bias_np in ((db_.ptr, b), (None, None)):
+        y = hip.to_device(np.full((B, oc, ho, wo), np.nan, np.float32))
+        hip.check(hip.bh_conv2d_forward_mfma(dx_.ptr, dw_.ptr, bias, y.ptr, B, ic, h, w, oc, k, stride, pad))
+        want = oracle.conv2d_forward(x, wt, bias_np, stride, pad)
+        got = y.numpy()
+        assert np.isfinite(got).all()
+        assert np.linalg.norm(got - want) <= fp32_gemm_bound(ic * k * k) * np.linalg.norm(want)
+        assert np.max(np.abs(got - want)) <= 1e-5 * max(1.0, np.abs(want).max())
+    with pytest.raises(RuntimeError):
+        hip.check(hip.bh_conv2d_forward_mfma(dx_.ptr, dw_.ptr, None, y.ptr, B, ic, h, w, oc, 5, stride, pad))
+
+
 def test_conv2d_refuses_bad_shapes(hip):
     p = hip.empty(16)
     assert hip.bh_conv2d_forward(p.ptr, p.ptr, None, p.ptr, 1, 1, 2, 2, 1, 3, 1, 0) == -1       # kernel larger than image

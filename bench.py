@@ -263,7 +263,22 @@ def bench_sdpa(hip, steps, warmup):
     flops = 4 * 2.0 * bh_ * S * S * D
     tf = flops / (ms * 1e-3) / 1e12
     out["sdpa_bwd_B8h16S1024D64"] = {"ms": round(ms, 4), "bound": "mfma", "achieved_TFLOPs": round(tf, 2),
-                                     "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "credited_flops": flops}
+                                     "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "credited_flops": flops,
+                                     "note": "recomputes Q.K^T (a fifth contraction that is not credited); no [S, S] matrix in memory"}
+    # the pair an attention layer uses when the scores fit its cache limit: the forward pass also leaves the scaled
+    # scores (bh*S*S*4 bytes, what the reference keeps as attention weights), the backward pass reads them
+    cache = hip.empty((bh_, S, S))
+    ms_f = time_steps(hip, lambda: hip.check(hip.bh_sdpa_forward_cached(q.ptr, k.ptr, vv.ptr, scale, 0, o.ptr, lse.ptr, cache.ptr,
+                                                                        bh_, S, D)), steps, warmup)
+    ms_b = time_steps(hip, lambda: hip.check(hip.bh_sdpa_backward_cached(q.ptr, k.ptr, vv.ptr, o.ptr, lse.ptr, cache.ptr, go.ptr, scale,
+                                                                         0, dq.ptr, dk.ptr, dv.ptr, bh_, S, D)), steps, warmup)
+    tf_f, tf_b = flops / 2 / (ms_f * 1e-3) / 1e12, flops / (ms_b * 1e-3) / 1e12
+    out["sdpa_with_score_cache_B8h16S1024D64"] = {
+        "fwd_ms": round(ms_f, 4), "fwd_frac": round(tf_f / PEAK_FP32_MFMA_TFLOPS, 4),
+        "bwd_ms": round(ms_b, 4), "bwd_achieved_TFLOPs": round(tf_b, 2), "bwd_frac": round(tf_b / PEAK_FP32_MFMA_TFLOPS, 4),
+        "bound": "mfma", "cache_bytes": int(bh_) * S * S * 4,
+        "fwd_plus_bwd_ms": round(ms_f + ms_b, 4),
+        "fwd_plus_bwd_ms_without_cache": round(out["sdpa_fwd_B8h16S1024D64"]["ms"] + out["sdpa_bwd_B8h16S1024D64"]["ms"], 4)}
     return out
 
 

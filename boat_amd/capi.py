@@ -252,6 +252,7 @@ _EXT_SIGS = {
     "boat_hip_optimizer_add_conv": (None, [P, P]),
     "boat_hip_conv_reference_input_grad": (None, [C.c_int]),
     "boat_hip_conv_forward_matrix_cores": (None, [C.c_int]),
+    "boat_hip_set_attention_score_cache_limit": (None, [C.c_size_t]),
     "boat_hip_optimizer_add_attention": (None, [P, P]),
     "boat_hip_optimizer_add_layernorm": (None, [P, P]),
     "boat_layernorm_update": (None, [P, C.c_float]),

@@ -317,10 +317,11 @@ using namespace bh;
 namespace bh {
 // MFMA path (defined in bh_sdpa_mfma.hip); returns BH_EINVAL-free "not applicable" as 1
 int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
-                      int64_t bh_count, int64_t s, int64_t d);
+                      float* scores_t, int64_t bh_count, int64_t s, int64_t d);
 int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
-                       const float* d_out, float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count,
-                       int64_t s, int64_t d);
+                       const float* d_out, const float* scores_t, float scale, int causal, float* dq, float* dk, float* dv,
+                       int64_t bh_count, int64_t s, int64_t d);
+bool sdpa_scores_shape(int64_t s, int64_t d);
 static int g_sdpa_force_general = 0;
 }  // namespace bh
 
@@ -340,7 +341,7 @@ int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale,
     BH_CHECK_ARG(q && k && v && out, "null pointer");
     ProfScope prof(BH_PROF_SDPA_FWD, 4.0 * (double)bh_count * (double)s * (double)s * (double)d);
     if (!g_sdpa_force_general && !attn_out && lse) {
-        int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, bh_count, s, d);
+        int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, nullptr, bh_count, s, d);
         if (rc <= 0) return rc;   // 0 done, <0 error, 1 shape not covered
     }
     // from 64 keys on the six products are worth a trip through the matrix cores
@@ -369,7 +370,7 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
     if (rc == BH_OK) {
         int done = 1;
         if (!g_sdpa_force_general)
-            done = sdpa_backward_mfma(q, k, v, lse, delta, d_out, scale, causal, dq, dk, dv, bh_count, s, d);
+            done = sdpa_backward_mfma(q, k, v, lse, delta, d_out, nullptr, scale, causal, dq, dk, dv, bh_count, s, d);
         // the matrix-core kernel's dQ workspace grows with s^2: when it cannot be had, the GEMM-based path, whose
         // [s, s] matrices are held for a bounded chunk of heads at a time, takes the shape
         if (done == BH_ENOMEM && s >= 64 && s <= 16384) done = 1;
@@ -391,6 +392,48 @@ int bh_sdpa_backward(const float* q, const float* k, const float* v, const float
                                dk, dv, s, d);
             rc = BH_LAUNCH_CHECK("sdpa_bwd_row_kernels");
         }
+    }
+    bh_free(delta);
+    return rc;
+}
+
+// ---- score cache: the forward pass leaves the scaled scores for the backward pass, as the reference keeps its
+// attention weights (src/layers/attention.c:424-431, 1046-1050 cache the [B, nh, S, S] softmax; :584-598 hand it to attention_backward) ----
+size_t bh_sdpa_score_cache_bytes(int64_t bh_count, int64_t s, int64_t d) {
+    if (bh_count <= 0 || s <= 0 || !sdpa_scores_shape(s, d)) return 0;
+    return sizeof(float) * (size_t)bh_count * (size_t)s * (size_t)s;
+}
+
+int bh_sdpa_forward_cached(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
+                           float* scores, int64_t bh_count, int64_t s, int64_t d) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
+    if (bh_count == 0 || s == 0) return BH_OK;
+    BH_CHECK_ARG(q && k && v && out && lse && scores, "null pointer");
+    BH_CHECK_ARG(bh_sdpa_score_cache_bytes(bh_count, s, d) != 0, "bh_sdpa_forward_cached: head_dim 64 and a sequence length that is a multiple of 128 only");
+    ProfScope prof(BH_PROF_SDPA_FWD, 4.0 * (double)bh_count * (double)s * (double)s * (double)d);
+    int rc = sdpa_forward_mfma(q, k, v, scale, causal, out, lse, scores, bh_count, s, d);
+    if (rc == 1) return set_error(BH_EINVAL, "bh_sdpa_forward_cached: pointers must be 16-byte aligned");
+    return rc;
+}
+
+int bh_sdpa_backward_cached(const float* q, const float* k, const float* v, const float* out, const float* lse,
+                            const float* scores, const float* d_out, float scale, int causal, float* dq, float* dk, float* dv,
+                            int64_t bh_count, int64_t s, int64_t d) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(bh_count >= 0 && s >= 0 && d > 0, "bad shape");
+    if (bh_count == 0 || s == 0) return BH_OK;
+    BH_CHECK_ARG(q && k && v && out && lse && scores && d_out && dq && dk && dv, "null pointer");
+    BH_CHECK_ARG(bh_sdpa_score_cache_bytes(bh_count, s, d) != 0, "bh_sdpa_backward_cached: head_dim 64 and a sequence length that is a multiple of 128 only");
+    ProfScope prof(BH_PROF_SDPA_BWD, 8.0 * (double)bh_count * (double)s * (double)s * (double)d);
+    const int64_t rows = bh_count * s;
+    float* delta = (float*)bh_malloc(sizeof(float) * (size_t)rows);
+    if (!delta) return BH_ENOMEM;
+    launch_delta(out, d_out, delta, rows, d);
+    int rc = BH_LAUNCH_CHECK("sdpa_delta_kernel");
+    if (rc == BH_OK) {
+        rc = sdpa_backward_mfma(q, k, v, lse, delta, d_out, scores, scale, causal, dq, dk, dv, bh_count, s, d);
+        if (rc == 1) rc = set_error(BH_EINVAL, "bh_sdpa_backward_cached: pointers must be 16-byte aligned");
     }
     bh_free(delta);
     return rc;

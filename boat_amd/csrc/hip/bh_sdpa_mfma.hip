@@ -47,10 +47,14 @@ __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + 
 
 // ------------------------------------------------------------------ forward
 // grid (s/128, bh); 4 wavefronts, each owns 32 queries; key/value tiles of 64 rows double-buffered in LDS.
-template <bool CAUSAL, bool RAGGED>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
+// EMIT: the scaled scores (log2 units, masked pairs -inf) are also written, transposed ([head][key][query]: a key's row
+// is what a lane of the backward kernel reads), so that the backward pass can skip the Q.K^T recompute.  Under a causal
+// mask the tiles past the diagonal are never visited and their part of the cache stays unwritten.
+template <bool CAUSAL, bool RAGGED, bool EMIT = false>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
 __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ out,
-                                                            float* __restrict__ lse, int s, int n_heads, float scale_log2e) {
+                                                            float* __restrict__ lse, int s, int n_heads, float scale_log2e,
+                                                            float* __restrict__ scores_t) {
     extern __shared__ __align__(16) float smem[];
     constexpr int KT = 64;                       // keys per tile
     constexpr int TILE = KT * kLd;               // floats per K or V tile in LDS
@@ -141,6 +145,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
                         if ((CAUSAL && key > my_q) || (RAGGED && key >= s)) acc_s[t][e] = -INFINITY;
                     }
                     mx = fmaxf(mx, acc_s[t][e]);
+                    if (EMIT) __builtin_nontemporal_store(acc_s[t][e], scores_t + ((int64_t)head * s + jt * KT + t * 32 + acc_row(e, half)) * s + my_q);
                 }
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m_run, mx);      // finite: key 0 is never masked and tiles are visited in order
@@ -229,28 +234,34 @@ struct BwdSmem {
 
 // RAGGED: rows past s are clamped on load; padding keys are masked, padding queries contribute nothing because their
 // dO rows and delta are staged as zeros; stores are guarded
-template <bool CAUSAL, bool RAGGED>
+// CACHED: the forward pass left the scaled scores (log2 units, [head][key][query]); S = Q.K^T is read instead of recomputed
+template <bool CAUSAL, bool RAGGED, bool CACHED = false>
 __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                const float* __restrict__ v, const float* __restrict__ lse,
                                                                const float* __restrict__ delta, const float* __restrict__ d_out,
                                                                float* __restrict__ dq_partial, float* __restrict__ dk,
-                                                               float* __restrict__ dv, int s, int n_heads, float scale) {
+                                                               float* __restrict__ dv, int s, int n_heads, float scale,
+                                                               int mirror, const float* __restrict__ scores_t) {
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
     // tile-major reading of the linear workgroup id, as in the forward kernel: key tile 0, which meets every query tile
     // under a causal mask, is handed out first for all heads
+    // mirror: the second of two launches that share one set of dQ partials.  Workgroup px of the first launch takes key
+    // tile px, workgroup px of the second takes key tile tiles-1-px and adds its dQ contribution to the rows its
+    // counterpart stored (the stream orders the launches; a partial is read and written by one workgroup per launch).
     const int lin = blockIdx.x;
     const int64_t head = lin % n_heads;
-    const int bx = lin / n_heads;
+    const int px = lin / n_heads;
+    const int bx = mirror ? (s + 127) / 128 - 1 - px : px;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
     const float* vh = v + head * s * kD;
     const float* gh = d_out + head * s * kD;
     const float* lh = lse + head * s;
     const float* dh = delta + head * s;
-    // partial dQ of this key tile: [key tile][bh][s][64]
-    float* dqh = dq_partial + ((int64_t)bx * n_heads + head) * s * kD;
+    // partial dQ of this workgroup: [px][bh][s][64]
+    float* dqh = dq_partial + ((int64_t)px * n_heads + head) * s * kD;
     const int kv_wg = bx * 128;          // first key of the workgroup
     const int kv0 = kv_wg + w * 32;              // first key of this wavefront
     const float c1 = scale * kLog2e;
@@ -279,9 +290,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
 
     const int n_qt = RAGGED ? (s + 31) / 32 : s / 32;
     const int first_qt = CAUSAL ? kv_wg / 32 : 0;   // earlier query tiles see none of this workgroup's keys
-    // their partial dQ rows are zero
-    for (int i = tid; i < first_qt * 32 * (kD / 4); i += 256)
-        reinterpret_cast<float4*>(dqh)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    // their partial dQ rows are zero (a mirror launch leaves them as its counterpart wrote them)
+    if (!mirror)
+        for (int i = tid; i < first_qt * 32 * (kD / 4); i += 256)
+            reinterpret_cast<float4*>(dqh)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     // staging: a Q tile and a dO tile are 512 float4 each, 2 per lane and operand
     float4 qst0, qst1, gst0, gst1;
     float stat = 0.f;
@@ -322,54 +334,84 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
 
     const int my_key = kv0 + r;
     const bool key_pad = RAGGED && my_key >= s;
+    // cached scores of this lane's key: row my_key of the head's [key][query] matrix
+    const float* sc_row = CACHED ? scores_t + ((int64_t)head * s + my_key) * s : nullptr;
+    // cached scores of the tile in work and of the next one (fetched a whole iteration ahead: a trip to HBM takes longer
+    // than the dP chain that could hide it inside one iteration)
+    float4 sc_cur[4], sc_next[4];
+    if (CACHED) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) sc_cur[j] = sc_next[j] = *reinterpret_cast<const float4*>(sc_row + first_qt * 32 + 8 * j + 4 * half);
+    }
     for (int qt = first_qt; qt < n_qt; qt++) {
         const bool more = qt + 1 < n_qt;
         if (more) BWD_STAGE_LOAD(qt + 1)
+        if (CACHED && more) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) sc_next[j] = *reinterpret_cast<const float4*>(sc_row + (qt + 1) * 32 + 8 * j + 4 * half);
+        }
         const int q0 = qt * 32;
         if (!CAUSAL || q0 + 31 >= kv0) {
             // S = Q.K^T and dP = dO.V^T : query = row (acc_row), key = lane
             floatx16 acc_s = zero16(), acc_dp = zero16();
+            if (CACHED) {
+                // registers 4j .. 4j+3 are query rows 8j + 4*half .. +3: the four 16-byte pieces fetched an iteration ago
 #pragma unroll
-            for (int g = 0; g < 8; g++) {
-                const int off = r * kLd + 8 * g + 4 * half;
-                const float4 aq = *reinterpret_cast<const float4*>(qs + off);
-                const float4 bk = *reinterpret_cast<const float4*>(ks + off);
-                const float4 ag = *reinterpret_cast<const float4*>(gs + off);
-                const float4 bv = vreg[g];
-                acc_s = MFMA(aq.x, bk.x, acc_s);
-                acc_dp = MFMA(ag.x, bv.x, acc_dp);
-                acc_s = MFMA(aq.y, bk.y, acc_s);
-                acc_dp = MFMA(ag.y, bv.y, acc_dp);
-                acc_s = MFMA(aq.z, bk.z, acc_s);
-                acc_dp = MFMA(ag.z, bv.z, acc_dp);
-                acc_s = MFMA(aq.w, bk.w, acc_s);
-                acc_dp = MFMA(ag.w, bv.w, acc_dp);
+                for (int j = 0; j < 4; j++) {
+                    acc_s[4 * j + 0] = sc_cur[j].x;
+                    acc_s[4 * j + 1] = sc_cur[j].y;
+                    acc_s[4 * j + 2] = sc_cur[j].z;
+                    acc_s[4 * j + 3] = sc_cur[j].w;
+                }
+                floatx16 acc_dp2 = zero16();     // two chains, so that a product never waits for its predecessor
+#pragma unroll
+                for (int g = 0; g < 8; g++) {
+                    const float4 ag = *reinterpret_cast<const float4*>(gs + r * kLd + 8 * g + 4 * half);
+                    const float4 bv = vreg[g];
+                    acc_dp = MFMA(ag.x, bv.x, acc_dp);
+                    acc_dp2 = MFMA(ag.y, bv.y, acc_dp2);
+                    acc_dp = MFMA(ag.z, bv.z, acc_dp);
+                    acc_dp2 = MFMA(ag.w, bv.w, acc_dp2);
+                }
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc_dp[e] += acc_dp2[e];
+            } else {
+#pragma unroll
+                for (int g = 0; g < 8; g++) {
+                    const int off = r * kLd + 8 * g + 4 * half;
+                    const float4 aq = *reinterpret_cast<const float4*>(qs + off);
+                    const float4 bk = *reinterpret_cast<const float4*>(ks + off);
+                    const float4 ag = *reinterpret_cast<const float4*>(gs + off);
+                    const float4 bv = vreg[g];
+                    acc_s = MFMA(aq.x, bk.x, acc_s);
+                    acc_dp = MFMA(ag.x, bv.x, acc_dp);
+                    acc_s = MFMA(aq.y, bk.y, acc_s);
+                    acc_dp = MFMA(ag.y, bv.y, acc_dp);
+                    acc_s = MFMA(aq.z, bk.z, acc_s);
+                    acc_dp = MFMA(ag.z, bv.z, acc_dp);
+                    acc_s = MFMA(aq.w, bk.w, acc_s);
+                    acc_dp = MFMA(ag.w, bv.w, acc_dp);
+                }
             }
-            // P and dS in place
+            // Row by row: P and dS of query row acc_row(e, half), dS published for the dQ product, then the row's four
+            // products dV += P^T.dO, dK += dS^T.Q (step e contracts that query row).  The exponential and the
+            // arithmetic of row e + 1 are issued while the matrix core still works on row e.
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int row = acc_row(e, half);
-                float p = __builtin_amdgcn_exp2f(acc_s[e] * c1 - st[row]);
+                float p = __builtin_amdgcn_exp2f(CACHED ? acc_s[e] - st[row] : acc_s[e] * c1 - st[row]);
                 // masked pairs and padding keys carry no probability (padding queries need no mask: their dO rows
                 // and delta were staged as zeros, so everything they contribute below is zero)
                 if ((CAUSAL && my_key > q0 + row) || key_pad) p = 0.f;
-                acc_s[e] = p;
-                acc_dp[e] = p * (acc_dp[e] - st[32 + row]) * scale;
-            }
-            // dV += P^T.dO ; dK += dS^T.Q : step e contracts query row acc_row(e, half)
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int row = acc_row(e, half);
+                const float ds = p * (acc_dp[e] - st[32 + row]) * scale;
+                dsb[row * BwdSmem::kDsLd + w * 32 + r] = ds;
                 const float2 bg = *reinterpret_cast<const float2*>(gs + row * kLd + 2 * r);
                 const float2 bq = *reinterpret_cast<const float2*>(qs + row * kLd + 2 * r);
-                acc_dv[0] = MFMA(acc_s[e], bg.x, acc_dv[0]);
-                acc_dv[1] = MFMA(acc_s[e], bg.y, acc_dv[1]);
-                acc_dk[0] = MFMA(acc_dp[e], bq.x, acc_dk[0]);
-                acc_dk[1] = MFMA(acc_dp[e], bq.y, acc_dk[1]);
+                acc_dv[0] = MFMA(p, bg.x, acc_dv[0]);
+                acc_dv[1] = MFMA(p, bg.y, acc_dv[1]);
+                acc_dk[0] = MFMA(ds, bq.x, acc_dk[0]);
+                acc_dk[1] = MFMA(ds, bq.y, acc_dk[1]);
             }
-            // publish dS[query][key] for the dQ product
-#pragma unroll
-            for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * BwdSmem::kDsLd + w * 32 + r] = acc_dp[e];
         } else {
 #pragma unroll
             for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * BwdSmem::kDsLd + w * 32 + r] = 0.f;
@@ -380,6 +422,14 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
         // consecutive keys of its dS row at once and feeds them to four successive products (the order
         // of the contraction index is free as long as both operands use the same one)
         floatx4 acc_dq0 = {0.f, 0.f, 0.f, 0.f}, acc_dq1 = {0.f, 0.f, 0.f, 0.f};
+        float* dq_row0 = dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk;
+        float* dq_row1 = dq_row0 + 16 * kD;
+        // mirror launch: what the first launch stored here, in flight while the products below run
+        float4 old0 = make_float4(0.f, 0.f, 0.f, 0.f), old1 = old0;
+        if (mirror) {
+            if (!RAGGED || q0 + i16 < s) old0 = *reinterpret_cast<const float4*>(dq_row0);
+            if (!RAGGED || q0 + 16 + i16 < s) old1 = *reinterpret_cast<const float4*>(dq_row1);
+        }
         const int g_lim = CAUSAL ? min(8, (q0 + 32 - kv_wg + 15) / 16) : 8;   // keys past the tile's last query are masked
         for (int g = 0; g < g_lim; g++) {
             const float4 a0 = *reinterpret_cast<const float4*>(dsb + i16 * BwdSmem::kDsLd + 16 * g + 4 * kk);
@@ -399,12 +449,16 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
         }
         // accumulator register e of lane (i16, kk) is head-dim column 16w + 4*kk + e of query row i16 of the 16-row tile
         if (!RAGGED || q0 + i16 < s)
-            *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk) =
-                make_float4(acc_dq0[0], acc_dq0[1], acc_dq0[2], acc_dq0[3]);
+            *reinterpret_cast<float4*>(dq_row0) =
+                make_float4(acc_dq0[0] + old0.x, acc_dq0[1] + old0.y, acc_dq0[2] + old0.z, acc_dq0[3] + old0.w);
         if (!RAGGED || q0 + 16 + i16 < s)
-            *reinterpret_cast<float4*>(dqh + (int64_t)(q0 + 16 + i16) * kD + 16 * w + 4 * kk) =
-                make_float4(acc_dq1[0], acc_dq1[1], acc_dq1[2], acc_dq1[3]);
+            *reinterpret_cast<float4*>(dq_row1) =
+                make_float4(acc_dq1[0] + old1.x, acc_dq1[1] + old1.y, acc_dq1[2] + old1.z, acc_dq1[3] + old1.w);
         __syncthreads();   // dS tile free again; the next Q and dO tiles are in place
+        if (CACHED) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) sc_cur[j] = sc_next[j];
+        }
     }
 #undef BWD_LD
 #undef BWD_ST
@@ -438,18 +492,24 @@ static bool mfma_shape(int64_t s, int64_t d) { return d == kD && s >= 32 && s <=
 // the grids are one-dimensional (tiles * heads workgroups): no 65535 limit on the number of heads
 static bool grid_fits(int64_t s, int64_t bh_count) { return ceil_div(s, 128) * bh_count <= 0x7fffffff && bh_count <= 0x7fffffff; }
 
+// shapes whose scaled scores the forward pass can leave for the backward pass: whole 128-row tiles
+bool sdpa_scores_shape(int64_t s, int64_t d) { return mfma_shape(s, d) && s % 128 == 0; }
+
 int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
-                      int64_t bh_count, int64_t s, int64_t d) {
+                      float* scores_t, int64_t bh_count, int64_t s, int64_t d) {
     if (!mfma_shape(s, d) || !grid_fits(s, bh_count)) return 1;
+    if (scores_t && !sdpa_scores_shape(s, d)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(out)) return 1;
     constexpr size_t lds = sizeof(float) * 2 * 2 * 64 * kLd;
     static bool attr = false;
     if (!attr) {
-        const void* fns[4] = {reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, false>),
+        const void* fns[6] = {reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, false>),
                               reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, false>),
                               reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, true>),
-                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, true>)};
+                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, true>),
+                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, false, true>),
+                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, false, true>)};
         for (const void* fn : fns) {
             int rc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
             if (rc) return rc;
@@ -459,8 +519,10 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
     dim3 grid((unsigned)(ceil_div(s, 128) * bh_count));
     const bool ragged = s % 128 != 0;
     const float sl = scale * kLog2e;
-#define FWD_LAUNCH(C, R) hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, (int)bh_count, sl)
-    if (causal && ragged) FWD_LAUNCH(true, true);
+#define FWD_LAUNCH(...) hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<__VA_ARGS__>), grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, (int)bh_count, sl, scores_t)
+    if (scores_t && causal) FWD_LAUNCH(true, false, true);
+    else if (scores_t) FWD_LAUNCH(false, false, true);
+    else if (causal && ragged) FWD_LAUNCH(true, true);
     else if (causal) FWD_LAUNCH(true, false);
     else if (ragged) FWD_LAUNCH(false, true);
     else FWD_LAUNCH(false, false);
@@ -469,39 +531,53 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
 }
 
 int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
-                       const float* d_out, float scale, int causal, float* dq, float* dk, float* dv, int64_t bh_count,
-                       int64_t s, int64_t d) {
+                       const float* d_out, const float* scores_t, float scale, int causal, float* dq, float* dk, float* dv,
+                       int64_t bh_count, int64_t s, int64_t d) {
     if (!mfma_shape(s, d) || !grid_fits(s, bh_count)) return 1;
+    if (scores_t && !sdpa_scores_shape(s, d)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(d_out) || !al(dq) || !al(dk) || !al(dv)) return 1;
     constexpr size_t lds = sizeof(float) * BwdSmem::TOTAL;
     static bool attr = false;
     if (!attr) {
-        const void* fns[4] = {reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, false>),
+        const void* fns[6] = {reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, false>),
                               reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, false>),
                               reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, true>),
-                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, true>)};
+                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, true>),
+                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, false, true>),
+                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, false, true>)};
         for (const void* fn : fns) {
             int arc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
             if (arc) return arc;
         }
         attr = true;
     }
-    const int tiles = (int)ceil_div(s, 128);
+    const int key_tiles = (int)ceil_div(s, 128);
+    // Two launches that share one set of dQ partials (the second takes the key tiles in mirrored order and adds to what
+    // the first stored) when each launch still puts two workgroups on every compute unit: half as many partials to
+    // write and fold, and each launch is a single round of workgroups that start and finish together instead of two
+    // rounds whose second runs out unevenly.  Not under a causal mask, where a launch would hold tiles of unequal work.
+    const bool two_launches = !causal && key_tiles >= 2 && (int64_t)(key_tiles / 2) * bh_count >= 2 * (int64_t)bh_device_cu_count();
+    const int tiles = two_launches ? (key_tiles + 1) / 2 : key_tiles;      // dQ partials per head
     const bool ragged = s % 128 != 0;
     const int64_t n = bh_count * s * d;
-    float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one key tile: dq itself
+    float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one partial: dq itself
     if (!partial) return BH_ENOMEM;
-    dim3 grid((unsigned)(tiles * bh_count));
-#define BWD_LAUNCH(C, R)                                                                                                   \
-    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<C, R>), grid, dim3(256), lds, stream(), q, k, v, lse, delta, d_out, partial, dk, dv, \
-                       (int)s, (int)bh_count, scale)
-    if (causal && ragged) BWD_LAUNCH(true, true);
-    else if (causal) BWD_LAUNCH(true, false);
-    else if (ragged) BWD_LAUNCH(false, true);
-    else BWD_LAUNCH(false, false);
+#define BWD_LAUNCH(GRID, MIRROR, ...)                                                                                      \
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<__VA_ARGS__>), dim3((unsigned)(GRID)), dim3(256), lds, stream(), q, k, v, lse, delta, \
+                       d_out, partial, dk, dv, (int)s, (int)bh_count, scale, MIRROR, scores_t)
+    int rc = BH_OK;
+    for (int pass = 0; pass < (two_launches ? 2 : 1) && rc == BH_OK; pass++) {
+        const int64_t grid = (pass == 0 ? tiles : key_tiles / 2) * bh_count;
+        if (scores_t && causal) BWD_LAUNCH(grid, pass, true, false, true);
+        else if (scores_t) BWD_LAUNCH(grid, pass, false, false, true);
+        else if (causal && ragged) BWD_LAUNCH(grid, pass, true, true);
+        else if (causal) BWD_LAUNCH(grid, pass, true, false);
+        else if (ragged) BWD_LAUNCH(grid, pass, false, true);
+        else BWD_LAUNCH(grid, pass, false, false);
+        rc = BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
+    }
 #undef BWD_LAUNCH
-    int rc = BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
     if (tiles > 1) {
         if (rc == BH_OK) {
             const int64_t n4 = n / 4;

@@ -111,6 +111,8 @@ struct boat_attention_t {
     boat_tensor_t *cache_q_proj, *cache_k_proj, *cache_v_proj;
     boat_tensor_t* cache_lse;                /* [B*nh, S] row log-sum-exp, replaces the [B,nh,S,S] weights cache */
     boat_tensor_t* cache_attention_output;   /* [B,S,H] before the output projection */
+    boat_tensor_t* cache_scores;             /* [B*nh, S, S] scaled scores for the backward pass, or NULL (shape without the
+                                                cached path, or larger than the score-cache limit) */
 };
 
 /* boat_attention_backward for a layer whose query, key and value were one tensor: *grad_input = dq + dk + dv, the sums

@@ -547,13 +547,28 @@ boat_attention_t* boat_attention_create(const boat_attention_config_t* config) {
     return a;
 }
 
+/* largest [B*nh, S, S] score matrix (bytes) an attention layer keeps from its forward pass for its backward pass; 0 = never.
+ * BOAT_HIP_ATTENTION_SCORE_CACHE (bytes) in the environment sets the initial value. */
+static size_t g_score_cache_limit = (size_t)1 << 30;
+static int g_score_cache_env_read = 0;
+static void score_cache_env(void) {
+    if (g_score_cache_env_read) return;
+    g_score_cache_env_read = 1;
+    const char* e = getenv("BOAT_HIP_ATTENTION_SCORE_CACHE");
+    if (e && *e) g_score_cache_limit = (size_t)strtoull(e, NULL, 10);
+}
+void boat_hip_set_attention_score_cache_limit(size_t bytes) {
+    g_score_cache_env_read = 1;
+    g_score_cache_limit = bytes;
+}
+
 void boat_attention_free(boat_attention_t* a) {
     if (!a) return;
     boat_tensor_t** all[] = {&a->weight_q, &a->weight_k, &a->weight_v, &a->weight_o, &a->bias_q, &a->bias_k, &a->bias_v,
                              &a->bias_o, &a->grad_weight_q, &a->grad_weight_k, &a->grad_weight_v, &a->grad_weight_o,
                              &a->grad_bias_q, &a->grad_bias_k, &a->grad_bias_v, &a->grad_bias_o, &a->cache_query,
                              &a->cache_key, &a->cache_value, &a->cache_q_proj, &a->cache_k_proj, &a->cache_v_proj,
-                             &a->cache_lse, &a->cache_attention_output};
+                             &a->cache_lse, &a->cache_attention_output, &a->cache_scores};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++) boat_tensor_free(*all[i]);
     free(a);
 }
@@ -588,8 +603,9 @@ boat_tensor_t* boat_attention_forward(boat_attention_t* a, const boat_tensor_t* 
     swap_tensor(&a->cache_query, (boat_tensor_t*)query);
     swap_tensor(&a->cache_key, (boat_tensor_t*)key);
     swap_tensor(&a->cache_value, (boat_tensor_t*)value);
-    boat_tensor_t** stale[] = {&a->cache_q_proj, &a->cache_k_proj, &a->cache_v_proj, &a->cache_lse, &a->cache_attention_output};
-    for (size_t i = 0; i < 5; i++) {
+    boat_tensor_t** stale[] = {&a->cache_q_proj, &a->cache_k_proj, &a->cache_v_proj, &a->cache_lse, &a->cache_attention_output,
+                               &a->cache_scores};
+    for (size_t i = 0; i < 6; i++) {
         boat_tensor_free(*stale[i]);
         *stale[i] = NULL;
     }
@@ -606,11 +622,23 @@ boat_tensor_t* boat_attention_forward(boat_attention_t* a, const boat_tensor_t* 
     a->cache_attention_output = bt_new_like_uninit(query);
     if (!a->cache_lse || !a->cache_attention_output) return NULL;
     const float scale = 1.0f / sqrtf((float)hd);
-    if (!boat_hip_ok(bh_sdpa_forward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj), scale,
-                                     a->config.causal_mask ? 1 : 0, bt_dev_write(a->cache_attention_output),
-                                     bt_dev_write(a->cache_lse), NULL, batch * nh, seq, hd),
-                     "attention core forward"))
-        return NULL;
+    /* The reference keeps the [B, nh, S, S] attention weights for its backward pass (attention.c:424-431, 584-598).  Here
+     * the forward kernel can leave the scaled scores instead, which saves the backward kernel one of its five contractions;
+     * kept when the shape has that path and the matrix fits the score-cache limit, otherwise the backward pass recomputes. */
+    score_cache_env();
+    const size_t score_bytes = bh_sdpa_score_cache_bytes(batch * nh, seq, hd);
+    if (score_bytes && score_bytes <= g_score_cache_limit) {
+        const int64_t sshape[] = {batch * nh, seq, seq};
+        a->cache_scores = bt_new_uninit(sshape, 3, query->device);     /* no room: fall back to recomputing */
+    }
+    float* scores = a->cache_scores ? bt_dev_write(a->cache_scores) : NULL;
+    const int rc = scores ? bh_sdpa_forward_cached(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
+                                                   scale, a->config.causal_mask ? 1 : 0, bt_dev_write(a->cache_attention_output),
+                                                   bt_dev_write(a->cache_lse), scores, batch * nh, seq, hd)
+                          : bh_sdpa_forward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj), scale,
+                                            a->config.causal_mask ? 1 : 0, bt_dev_write(a->cache_attention_output),
+                                            bt_dev_write(a->cache_lse), NULL, batch * nh, seq, hd);
+    if (!boat_hip_ok(rc, "attention core forward")) return NULL;
     return project(a->cache_attention_output, a->weight_o, a->bias_o, rows, h);
 }
 
@@ -759,12 +787,18 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
     boat_tensor_t* dkp = bt_new_like_uninit(q);
     boat_tensor_t* dvp = bt_new_like_uninit(q);
     const float scale = 1.0f / sqrtf((float)hd);
-    bool ok = dqp && dkp && dvp &&
-              boat_hip_ok(bh_sdpa_backward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
-                                           bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(d_ao), scale,
-                                           a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp),
-                                           batch * nh, seq, hd),
-                          "attention core backward");
+    bool ok = dqp && dkp && dvp;
+    if (ok) {
+        const int rc = a->cache_scores
+            ? bh_sdpa_backward_cached(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
+                                      bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(a->cache_scores),
+                                      bt_dev_read(d_ao), scale, a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp),
+                                      bt_dev_write(dvp), batch * nh, seq, hd)
+            : bh_sdpa_backward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
+                               bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(d_ao), scale,
+                               a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
+        ok = boat_hip_ok(rc, "attention core backward");
+    }
     boat_tensor_free(d_ao);
     /* 3. input projections */
     boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;

@@ -66,6 +66,9 @@ _SIGS = {
     "bh_sdpa_forward": (I, [P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_backward": (I, [P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_force_general": (I, [I]),
+    "bh_sdpa_score_cache_bytes": (C.c_size_t, [L, L, L]),
+    "bh_sdpa_forward_cached": (I, [P, P, P, F, I, P, P, P, L, L, L]),
+    "bh_sdpa_backward_cached": (I, [P, P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
     "bh_adam_update": (I, [P, P, P, P, L, F, F, F, F, L]),
     "bh_conv2d_forward": (I, [P, P, P, P] + [L] * 8),
     "bh_conv2d_forward_mfma": (I, [P, P, P, P] + [L] * 8),

@@ -511,6 +511,11 @@ BOAT_API void boat_hip_conv_reference_input_grad(int enable);
  * sums in MFMA order: equal to the reference to fp32 rounding, not bit for bit).  Default 0, or BOAT_HIP_CONV_FORWARD_MFMA. */
 BOAT_API void boat_hip_conv_forward_matrix_cores(int enable);
 BOAT_API void boat_hip_optimizer_add_attention(boat_optimizer_t* opt, boat_attention_t* attention);
+/* An attention layer keeps the scaled scores [batch*heads, seq, seq] of its forward pass for its backward pass (as the
+ * reference keeps its attention weights, src/layers/attention.c:424-431) when head_size is 64, seq a multiple of 128 and
+ * the matrix is no larger than this many bytes: the backward pass then skips recomputing Q.K^T.  Default 1 GiB, or
+ * BOAT_HIP_ATTENTION_SCORE_CACHE; 0 = always recompute (no [seq, seq] matrix is ever stored). */
+BOAT_API void boat_hip_set_attention_score_cache_limit(size_t bytes);
 BOAT_API void boat_hip_optimizer_add_layernorm(boat_optimizer_t* opt, boat_layernorm_t* norm);
 
 #ifdef __cplusplus

@@ -203,6 +203,17 @@ int bh_sdpa_forward(const float* q, const float* k, const float* v, float scale,
 int bh_sdpa_backward(const float* q, const float* k, const float* v, const float* out, const float* lse,
                      const float* d_out, float scale, int causal,
                      float* dq, float* dk, float* dv, int64_t bh, int64_t s, int64_t d);
+/* The same pair with a score cache: the forward pass also leaves the scaled scores ([bh, s(key), s(query)] floats, an
+ * opaque layout) and the backward pass reads them instead of recomputing Q.K^T -- the trade the reference makes when it
+ * keeps its [B, nh, S, S] attention weights for attention_backward (attention.c:424-431 and 1046-1050 store them, :584-598 hand them to attention_backward).  One contraction
+ * of five less in the backward pass for bh*s*s*4 bytes of HBM.  head_dim 64 and s a multiple of 128 only:
+ * bh_sdpa_score_cache_bytes returns the size of the cache, 0 for shapes without this path. */
+size_t bh_sdpa_score_cache_bytes(int64_t bh, int64_t s, int64_t d);
+int bh_sdpa_forward_cached(const float* q, const float* k, const float* v, float scale, int causal,
+                           float* out, float* lse, float* scores, int64_t bh, int64_t s, int64_t d);
+int bh_sdpa_backward_cached(const float* q, const float* k, const float* v, const float* out, const float* lse,
+                            const float* scores, const float* d_out, float scale, int causal,
+                            float* dq, float* dk, float* dv, int64_t bh, int64_t s, int64_t d);
 
 /* ---- 2-D convolution and max pooling, NCHW, square kernel/window (src/layers/conv.c:46-201,326-437; src/layers/pool.c:63-218) ----
  * x [batch, in_channels, height, width]; w [out_channels, in_channels, kernel, kernel]; bias [out_channels] or NULL;

@@ -371,6 +371,33 @@ def test_attention_layer(boat, oracle, case):
                 assert rel_fro(rec["gb" + n], g["gb" + n]) <= TOL_GEMM, n
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_layer_with_and_without_score_cache(boat, oracle, causal):
+    """Head size 64, 128 keys: the layer keeps the scaled scores of its forward pass and its backward kernel reads them
+    (the reference keeps its attention weights, src/layers/attention.c:424-431, 584-598); with the limit at 0 the
+    backward kernel recomputes Q.K^T.  Both against the oracle, and against each other to fp32 rounding."""
+    case = dict(B=2, S=128, H=128, heads=2, causal=causal, bias=True)
+    xs, w, b, dys = make_attention_inputs(case, 5)
+    o_out, cache = oracle.attention_forward(*xs, w, b, 2, causal)
+    runs = []
+    for limit in (1 << 30, 0):
+        boat.boat_hip_set_attention_score_cache_limit(limit)
+        try:
+            runs.append(bc.attention(boat, *xs, w, b, 2, causal, dys))
+        finally:
+            boat.boat_hip_set_attention_score_cache_limit(1 << 30)
+    for out, results in runs:
+        assert rel_fro(out, o_out) <= TOL_GEMM
+        for dy, rec in zip(dys, results):
+            g = oracle.attention_backward(*xs, w, True, cache, dy, 2)
+            for got, want in ((rec["dq"], g["d_query"]), (rec["dk"], g["d_key"]), (rec["dv"], g["d_value"])):
+                assert rel_fro(got, want) <= TOL_GEMM
+    assert np.array_equal(runs[0][0], runs[1][0])                      # the forward arithmetic is the same
+    for a, c in zip(runs[0][1], runs[1][1]):
+        for key in ("dq", "dk", "dv", "gwq", "gwk", "gwv", "gwo"):
+            assert rel_fro(a[key], c[key]) <= 2e-5, key
+
+
 def test_attention_through_the_tape_self_attention(boat, oracle):
     """boat_var_attention(x, x, x): the three input gradients land in the same leaf (autodiff.c:2458-2532)."""
     case = dict(B=2, S=8, H=32, heads=4, causal=False, bias=True)

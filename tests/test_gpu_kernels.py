@@ -573,6 +573,72 @@ def test_sdpa_more_head_blocks_than_a_grid_dimension_holds(hip, oracle, rng):
             assert rel_fro(g[sl], w) <= TOL_GEMM
 
 
+@pytest.mark.parametrize("causal", [0, 1])
+@pytest.mark.parametrize("bh,s", [(3, 128), (2, 384), (1, 1024), (520, 256)])
+def test_sdpa_with_score_cache(hip, oracle, rng, bh, s, causal):
+    """bh_sdpa_forward_cached leaves the scaled scores, bh_sdpa_backward_cached reads them instead of recomputing Q.K^T:
+    same outputs as the plain pair to fp32 rounding, against the oracle's attention backward
+    (src/layers/attention.c:1417-1520) at the bound only fp32 accumulation meets; (520, 256) also takes the mirrored
+    second launch.  Shapes without the path are refused."""
+    d = 64
+    q, k, v, go = (rng.standard_normal((bh, s, d), dtype=np.float32) for _ in range(4))
+    dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)
+    scale = 0.125
+    assert hip.bh_sdpa_score_cache_bytes(bh, s, d) == 4 * bh * s * s
+    o, lse, cache = hip.empty((bh, s, d)), hip.empty((bh, s)), hip.to_device(np.full((bh, s, s), np.nan, np.float32))
+    hip.check(hip.bh_sdpa_forward_cached(dq_.ptr, dk_.ptr, dv_.ptr, scale, causal, o.ptr, lse.ptr, cache.ptr, bh, s, d))
+    o2, lse2 = hip.empty((bh, s, d)), hip.empty((bh, s))
+    hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, causal, o2.ptr, lse2.ptr, None, bh, s, d))
+    assert np.array_equal(o.numpy(), o2.numpy()) and np.array_equal(lse.numpy(), lse2.numpy())   # same arithmetic, one more store
+    gq, gk, gv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
+    hip.check(hip.bh_sdpa_backward_cached(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, cache.ptr, dgo.ptr, scale, causal,
+                                          gq.ptr, gk.ptr, gv.ptr, bh, s, d))
+    got = [x.numpy() for x in (gq, gk, gv)]
+    assert all(np.isfinite(g).all() for g in got)
+    for sl in (slice(0, 2), slice(bh - 1, bh)):
+        _, _, wattn = oracle.sdpa_forward(q[sl], k[sl], v[sl], scale, causal)
+        for g, w in zip(got, oracle.sdpa_backward(q[sl], k[sl], v[sl], wattn, go[sl], scale)):
+            assert rel_fro(g[sl], w) <= FP32_ATTENTION_BOUND
+    rq, rk, rv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
+    hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, dgo.ptr, scale, causal, rq.ptr, rk.ptr, rv.ptr, bh, s, d))
+    for g, x in zip(got, (rq, rk, rv)):
+        assert rel_fro(g, x.numpy()) <= FP32_ATTENTION_BOUND
+
+
+def test_sdpa_score_cache_refuses_other_shapes(hip):
+    assert hip.bh_sdpa_score_cache_bytes(4, 100, 64) == 0 and hip.bh_sdpa_score_cache_bytes(4, 128, 32) == 0
+    buf = hip.empty(4 * 128 * 64)
+    with pytest.raises(RuntimeError):
+        hip.check(hip.bh_sdpa_forward_cached(buf.ptr, buf.ptr, buf.ptr, 0.1, 0, buf.ptr, buf.ptr, buf.ptr, 4, 100, 64))
+    with pytest.raises(RuntimeError):
+        hip.check(hip.bh_sdpa_backward_cached(buf.ptr, buf.ptr, buf.ptr, buf.ptr, buf.ptr, buf.ptr, buf.ptr, 0.1, 0,
+                                              buf.ptr, buf.ptr, buf.ptr, 4, 128, 32))
+
+
+@pytest.mark.parametrize("bh,s", [(512, 384), (512, 300), (256, 512), (600, 256)])
+def test_sdpa_backward_mirrored_second_launch(hip, oracle, rng, bh, s):
+    """Enough heads for the unmasked backward to run as two launches that share one set of dQ partials (the second
+    takes the key tiles in mirrored order and adds to what the first stored): odd tile counts (the middle tile belongs
+    to the first launch), a ragged length, an even count; sampled heads against float64, a second call gives the same
+    bits (nothing of the first call's partials survives into it)."""
+    d = 64
+    q, k, v, go = (rng.standard_normal((bh, s, d), dtype=np.float32) for _ in range(4))
+    dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)
+    o, lse = hip.empty((bh, s, d)), hip.empty((bh, s))
+    scale = 0.125
+    hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, 0, o.ptr, lse.ptr, None, bh, s, d))
+    gq, gk, gv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
+    hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, dgo.ptr, scale, 0, gq.ptr, gk.ptr, gv.ptr, bh, s, d))
+    got = [x.numpy() for x in (gq, gk, gv)]
+    for sl in (slice(0, 2), slice(bh // 2, bh // 2 + 2), slice(bh - 2, bh)):
+        _, _, wattn = oracle.sdpa_forward(q[sl], k[sl], v[sl], scale, 0)
+        for g, w in zip(got, oracle.sdpa_backward(q[sl], k[sl], v[sl], wattn, go[sl], scale)):
+            assert rel_fro(g[sl], w) <= FP32_ATTENTION_BOUND
+    hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, dgo.ptr, scale, 0, gq.ptr, gk.ptr, gv.ptr, bh, s, d))
+    for g, x in zip(got, (gq, gk, gv)):
+        assert np.array_equal(g, x.numpy())
+
+
 # ------------------------------------------------------------------ convolution / max pooling
 
 CONV_SHAPES = [  # batch, ic, h, w, oc, k, stride, pad

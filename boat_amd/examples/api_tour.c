@@ -327,6 +327,122 @@ static void tour_attention_and_conv(void) {
     boat_tensor_unref(logits);
 }
 
+/* ---- RMSNorm, the stateless norms, the public attention core, arithmetic on other element types, the opt-in paths ---- */
+static void tour_norms_attention_core_and_types(void) {
+    const int64_t xs[2] = {6, 32}, ns[1] = {32};
+    boat_tensor_t* x = random_tensor(xs, 2, 1.0f);
+    boat_rmsnorm_config_t rc;
+    memset(&rc, 0, sizeof(rc));
+    rc.normalized_shape = 32;
+    rc.eps = 1e-6f;
+    rc.elementwise_affine = true;
+    boat_rmsnorm_t* rms = boat_rmsnorm_create(&rc);
+    boat_tensor_t* y = boat_rmsnorm_forward(rms, x);
+    boat_tensor_t* gx = y ? boat_rmsnorm_backward(rms, y) : NULL;
+    CHECK(rms && y && gx && boat_tensor_nelements(gx) == 6 * 32);
+    CHECK(boat_hip_rmsnorm_get_grad_weight(rms) && sum_abs(boat_hip_rmsnorm_get_grad_weight(rms)) > 0.0f);
+    boat_rmsnorm_update(rms, 1e-3f);
+    boat_tensor_t* ln = boat_layer_norm(x, ns, 1, 1e-5f);
+    boat_tensor_t* rn = boat_rms_norm(x, ns, 1, 1e-6f);
+    boat_tensor_t* rg = rn ? boat_rms_norm_grad(rn, x, rn, ns, 1, 1e-6f) : NULL;
+    CHECK(ln && rn && rg);
+    boat_tensor_t* owned[] = {rg, rn, ln, gx, y, x};
+    for (size_t i = 0; i < sizeof(owned) / sizeof(owned[0]); i++) boat_tensor_unref(owned[i]);
+    boat_rmsnorm_free(rms);
+
+    /* attention core on [batch, heads, seq, head_size]; self-attention through a throw-away layer */
+    const int64_t qs[4] = {2, 3, 10, 16};
+    boat_tensor_t* q = random_tensor(qs, 4, 1.0f);
+    boat_tensor_t* core = boat_scaled_dot_product_attention(q, q, q, 0.25f, NULL, true, 0.0f);
+    CHECK(core && boat_tensor_nelements(core) == 2 * 3 * 10 * 16);
+    const int64_t hs[3] = {2, 10, 48};
+    boat_tensor_t* h = random_tensor(hs, 3, 1.0f);
+    boat_tensor_t* mh = boat_multihead_attention(h, 3, 0.0f, false, NULL);
+    CHECK(mh && boat_tensor_shape(mh)[2] == 48);
+    boat_tensor_unref(mh);
+    boat_tensor_unref(h);
+    boat_tensor_unref(core);
+    boat_tensor_unref(q);
+
+    /* an attention layer whose forward pass keeps the scores for its backward pass (head size 64, 128 keys), then the
+     * same with the cache switched off */
+    for (int pass = 0; pass < 2; pass++) {
+        boat_hip_set_attention_score_cache_limit(pass == 0 ? (size_t)1 << 30 : 0);
+        boat_attention_config_t cfg;
+        memset(&cfg, 0, sizeof(cfg));
+        cfg.hidden_size = 128;
+        cfg.num_heads = 2;
+        cfg.head_size = 64;
+        cfg.use_bias = true;
+        boat_attention_t* att = boat_attention_create(&cfg);
+        const int64_t as[3] = {1, 128, 128};
+        boat_tensor_t* ax = random_tensor(as, 3, 1.0f);
+        boat_tensor_t* ay = boat_attention_forward(att, ax, ax, ax, NULL);
+        boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
+        CHECK(att && ay && boat_attention_backward(att, ay, &gq, &gk, &gv) && gq && gk && gv && sum_abs(gq) > 0.0f);
+        boat_tensor_t* at[] = {gq, gk, gv, ay, ax};
+        for (size_t i = 0; i < sizeof(at) / sizeof(at[0]); i++) boat_tensor_unref(at[i]);
+        boat_attention_free(att);
+    }
+    boat_hip_set_attention_score_cache_limit((size_t)1 << 30);
+
+    /* elementwise arithmetic on float64 and integers, with broadcasting */
+    const int64_t ds[2] = {3, 4}, bs[2] = {1, 4};
+    boat_tensor_t* a64 = boat_tensor_create(ds, 2, BOAT_DTYPE_FLOAT64, BOAT_DEVICE_CPU);
+    boat_tensor_t* b64 = boat_tensor_create(bs, 2, BOAT_DTYPE_FLOAT64, BOAT_DEVICE_CPU);
+    for (int i = 0; i < 12; i++) ((double*)boat_tensor_data(a64))[i] = 1.0 + i;
+    for (int i = 0; i < 4; i++) ((double*)boat_tensor_data(b64))[i] = 2.0 + i;
+    boat_tensor_t* s64 = boat_add(a64, b64);
+    boat_tensor_t* m64 = boat_mod(a64, b64);
+    boat_tensor_t* p64 = boat_pow_scalar(a64, 2.0);
+    CHECK(s64 && ((const double*)boat_tensor_const_data(s64))[5] == 6.0 + 3.0);
+    CHECK(m64 && ((const double*)boat_tensor_const_data(m64))[5] == fmod(6.0, 3.0));
+    CHECK(p64 && ((const double*)boat_tensor_const_data(p64))[3] == 16.0);
+    boat_tensor_t* i32 = boat_tensor_create(ds, 2, BOAT_DTYPE_INT32, BOAT_DEVICE_CPU);
+    for (int i = 0; i < 12; i++) ((int32_t*)boat_tensor_data(i32))[i] = 10 * i;
+    boat_tensor_t* d32 = boat_div_scalar(i32, 3.0);
+    boat_mul_scalar_(i32, 2.0);
+    CHECK(d32 && ((const int32_t*)boat_tensor_const_data(d32))[4] == 13 && ((const int32_t*)boat_tensor_const_data(i32))[4] == 80);
+    boat_tensor_t* tt[] = {d32, i32, p64, m64, s64, b64, a64};
+    for (size_t i = 0; i < sizeof(tt) / sizeof(tt[0]); i++) boat_tensor_unref(tt[i]);
+
+    /* a 3x3 convolution with enough input channels for the matrix-core forward, switched on and off again */
+    const int64_t is[4] = {2, 8, 6, 6};
+    boat_tensor_t* img = random_tensor(is, 4, 1.0f);
+    boat_conv_layer_t* conv = boat_conv_layer_create(8, 5, 3, 1, 1);
+    boat_tensor_t* direct = boat_conv_layer_forward(conv, img);
+    boat_hip_conv_forward_matrix_cores(1);
+    boat_tensor_t* mfma = boat_conv_layer_forward(conv, img);
+    boat_hip_conv_forward_matrix_cores(0);
+    CHECK(direct && mfma && fabsf(sum_abs(direct) - sum_abs(mfma)) <= 1e-3f * sum_abs(direct));
+    boat_tensor_unref(mfma);
+    boat_tensor_unref(direct);
+    boat_conv_layer_free(conv);
+    boat_tensor_unref(img);
+
+    /* reference-exact mode: the fan-out of a non-leaf counts once per consumer, as in the reference */
+    const int64_t one[1] = {1};
+    for (int mode = 0; mode < 2; mode++) {
+        boat_hip_set_reference_exact(mode);
+        boat_tensor_t* ta = random_tensor(one, 1, 1.0f);
+        boat_tensor_t* tb = random_tensor(one, 1, 1.0f);
+        boat_variable_t* va = boat_variable_create(ta, true);
+        boat_variable_t* vb = boat_variable_create(tb, true);
+        boat_variable_t* vy = boat_var_mul(va, vb);
+        boat_variable_t* vz = boat_var_add(vy, vy);
+        boat_variable_backward_full(vz);
+        const float want = (mode ? 4.0f : 2.0f) * first_value(tb);
+        CHECK(boat_variable_grad(va) && fabsf(first_value(boat_variable_grad(va)) - want) <= 1e-6f * fabsf(want));
+        boat_variable_free(vz);
+        boat_variable_free(vy);
+        boat_variable_free(vb);
+        boat_variable_free(va);
+        boat_tensor_unref(tb);
+        boat_tensor_unref(ta);
+    }
+    boat_hip_set_reference_exact(0);
+}
+
 int main(void) {
     boat_init();
     if (boat_has_error()) {
@@ -337,6 +453,7 @@ int main(void) {
     tour_tape();
     tour_layers();
     tour_attention_and_conv();
+    tour_norms_attention_core_and_types();
     boat_hip_synchronize();
     CHECK(!boat_has_error());
     const boat_memory_stats_t st = boat_memory_get_stats();

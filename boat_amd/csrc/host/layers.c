@@ -632,6 +632,11 @@ boat_tensor_t* boat_attention_forward(boat_attention_t* a, const boat_tensor_t* 
         a->cache_scores = bt_new_uninit(sshape, 3, query->device);     /* no room: fall back to recomputing */
     }
     float* scores = a->cache_scores ? bt_dev_write(a->cache_scores) : NULL;
+    if (a->cache_scores && !scores) {           /* no HBM for it: the backward pass recomputes */
+        boat_tensor_free(a->cache_scores);
+        a->cache_scores = NULL;
+        boat_reset_error();
+    }
     const int rc = scores ? bh_sdpa_forward_cached(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
                                                    scale, a->config.causal_mask ? 1 : 0, bt_dev_write(a->cache_attention_output),
                                                    bt_dev_write(a->cache_lse), scores, batch * nh, seq, hd)

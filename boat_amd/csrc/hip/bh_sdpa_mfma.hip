@@ -83,6 +83,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
         qreg[4 * g + 2] = t.z * scale_log2e;
         qreg[4 * g + 3] = t.w * scale_log2e;
     }
+    float* sc_base = EMIT ? scores_t + ((int64_t)head * s + half * 4) * s + my_q : nullptr;
     floatx16 acc_o[2] = {zero16(), zero16()};    // O^T: [d tile][...]; d = 2*row + tile, query = lane
     float m_run = -INFINITY, l_run = 0.f;
 
@@ -145,7 +146,6 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
                         if ((CAUSAL && key > my_q) || (RAGGED && key >= s)) acc_s[t][e] = -INFINITY;
                     }
                     mx = fmaxf(mx, acc_s[t][e]);
-                    if (EMIT) __builtin_nontemporal_store(acc_s[t][e], scores_t + ((int64_t)head * s + jt * KT + t * 32 + acc_row(e, half)) * s + my_q);
                 }
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m_run, mx);      // finite: key 0 is never masked and tiles are visited in order
@@ -155,6 +155,9 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
+                    // the score goes to the cache between the exponentials: row (tile's first key + t*32 + 8*(e/4) + e%4) of
+                    // the lane's base, which already holds the lane-dependent part (half, query)
+                    if (EMIT) __builtin_nontemporal_store(acc_s[t][e], sc_base + (int64_t)(jt * KT + t * 32 + (e >> 2) * 8 + (e & 3)) * s);
                     const float p = __builtin_amdgcn_exp2f(acc_s[t][e] - m_new);
                     acc_s[t][e] = p;
                     psum += p;

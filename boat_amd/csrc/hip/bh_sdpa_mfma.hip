@@ -123,6 +123,10 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
         // a wavefront whose queries all precede this tile's keys has nothing to add
         if (!CAUSAL || jt * KT <= q0 + 31) {
             floatx16 acc_s[2] = {zero16(), zero16()};   // S^T: key = row (tile*32 + acc_row), query = lane
+            // the wavefront's priority rises with its progress through the tile (scores 1, softmax 2, O^T 3, 0 around the
+            // staging and the barrier): of the two wavefronts that share a SIMD the one nearer to its barrier goes first
+            // (measured: 287 -> 273 us unmasked, 175 -> 162 us causal at B8 h16 S1024)
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int g = 0; g < 8; g++) {
                 const float4 a0 = *reinterpret_cast<const float4*>(ks + r * kLd + 8 * g + 4 * half);
@@ -136,6 +140,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
                 acc_s[0] = MFMA(a0.w, qreg[4 * g + 3], acc_s[0]);
                 acc_s[1] = MFMA(a1.w, qreg[4 * g + 3], acc_s[1]);
             }
+            __builtin_amdgcn_s_setprio(2);
             float mx = -INFINITY;
 #pragma unroll
             for (int t = 0; t < 2; t++)
@@ -169,6 +174,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc_o[t][e] *= alpha;
+            __builtin_amdgcn_s_setprio(3);
             // O^T += V^T . P^T : step e of key tile t uses key row t*32 + acc_row(e, half)
 #pragma unroll
             for (int t = 0; t < 2; t++)
@@ -180,6 +186,7 @@ __global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restr
                     acc_o[1] = MFMA(a.y, acc_s[t][e], acc_o[1]);
                 }
         }
+        __builtin_amdgcn_s_setprio(0);
         if (more) FWD_STAGE_STORE(cur ^ 1)
         __syncthreads();
     }
@@ -357,6 +364,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
         if (!CAUSAL || q0 + 31 >= kv0) {
             // S = Q.K^T and dP = dO.V^T : query = row (acc_row), key = lane
             floatx16 acc_s = zero16(), acc_dp = zero16();
+            // The wavefront's priority rises with its progress through the iteration (1 here, 2 in the row loop, 3 in
+            // the dQ product, 0 around the barriers and the staging): of the two wavefronts that share a matrix core the
+            // one nearer to its barrier goes first, so its workgroup's other wavefronts wait less.  Measured: 1 % on the
+            // recomputing kernel, 3 % on the one that reads the score cache.
+            __builtin_amdgcn_s_setprio(1);
             if (CACHED) {
                 // registers 4j .. 4j+3 are query rows 8j + 4*half .. +3: the four 16-byte pieces fetched an iteration ago
 #pragma unroll
@@ -396,6 +408,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                     acc_dp = MFMA(ag.w, bv.w, acc_dp);
                 }
             }
+            __builtin_amdgcn_s_setprio(2);
             // Row by row: P and dS of query row acc_row(e, half), dS published for the dQ product, then the row's four
             // products dV += P^T.dO, dK += dS^T.Q (step e contracts that query row).  The exponential and the
             // arithmetic of row e + 1 are issued while the matrix core still works on row e.
@@ -415,6 +428,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                 acc_dk[0] = MFMA(ds, bq.x, acc_dk[0]);
                 acc_dk[1] = MFMA(ds, bq.y, acc_dk[1]);
             }
+            __builtin_amdgcn_s_setprio(0);
         } else {
 #pragma unroll
             for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * BwdSmem::kDsLd + w * 32 + r] = 0.f;
@@ -425,6 +439,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
         // consecutive keys of its dS row at once and feeds them to four successive products (the order
         // of the contraction index is free as long as both operands use the same one)
         floatx4 acc_dq0 = {0.f, 0.f, 0.f, 0.f}, acc_dq1 = {0.f, 0.f, 0.f, 0.f};
+        __builtin_amdgcn_s_setprio(3);
         float* dq_row0 = dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk;
         float* dq_row1 = dq_row0 + 16 * kD;
         // mirror launch: what the first launch stored here, in flight while the products below run
@@ -450,6 +465,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
             acc_dq0 = MFMA16(b3, a0.w, acc_dq0);
             acc_dq1 = MFMA16(b3, a1.w, acc_dq1);
         }
+        __builtin_amdgcn_s_setprio(0);
         // accumulator register e of lane (i16, kk) is head-dim column 16w + 4*kk + e of query row i16 of the 16-row tile
         if (!RAGGED || q0 + i16 < s)
             *reinterpret_cast<float4*>(dq_row0) =

@@ -794,7 +794,7 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
     const float scale = 1.0f / sqrtf((float)hd);
     bool ok = dqp && dkp && dvp;
     if (ok) {
-        const int rc = a->cache_scores
+        int rc = a->cache_scores
             ? bh_sdpa_backward_cached(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
                                       bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(a->cache_scores),
                                       bt_dev_read(d_ao), scale, a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp),
@@ -802,6 +802,11 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
             : bh_sdpa_backward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
                                bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(d_ao), scale,
                                a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
+        /* no room for the cached kernel's dQ workspace: the plain entry point can fall back to its bounded GEMM path */
+        if (rc == BH_ENOMEM && a->cache_scores)
+            rc = bh_sdpa_backward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
+                                  bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(d_ao), scale,
+                                  a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
         ok = boat_hip_ok(rc, "attention core backward");
     }
     boat_tensor_free(d_ao);

@@ -50,8 +50,12 @@ __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + 
 // EMIT: the scaled scores (log2 units, masked pairs -inf) are also written, transposed ([head][key][query]: a key's row
 // is what a lane of the backward kernel reads), so that the backward pass can skip the Q.K^T recompute.  Under a causal
 // mask the tiles past the diagonal are never visited and their part of the cache stays unwritten.
+// The second launch-bounds figure is the least number of wavefronts per SIMD the register allocation must allow: two,
+// i.e. two workgroups per compute unit (the LDS allows no more).  Left to itself the compiler gave the causal
+// cache-writing form 244 registers and one wavefront per SIMD; the unmasked cache-writing form is the one that runs faster
+// with its own allocation (300 against 313 us).
 template <bool CAUSAL, bool RAGGED, bool EMIT = false>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
-__global__ __launch_bounds__(256) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
+__global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ out,
                                                             float* __restrict__ lse, int s, int n_heads, float scale_log2e,
                                                             float* __restrict__ scores_t) {

@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="all",
-                    help="comma list of step,dense,adam,ln_gelu,sdpa,mlp,cnn (default all); for profiling one workload at a time. "
+                    help="comma list of step,dense,adam,ln_gelu,sdpa,mlp,cnn,conv (default all); for profiling one workload at a time. "
                          "Without the step leg the line carries no value/roofline.")
     return ap.parse_args()
 
@@ -391,7 +391,7 @@ def bench_cnn_step(steps, warmup):
     api.boat_hip_conv_forward_matrix_cores(0)
     conv_flops = 2.0 * B * (32 * 1 * 9 * 28 * 28 + 64 * 32 * 9 * 14 * 14) * 3       # forward + dX + dW of both conv layers
     return {"ms": round(ms, 4), "bound": "launch latency / small kernels", "conv_flops": conv_flops,
-            "ms_conv_forward_on_matrix_cores": round(ms_mfma, 4), "conv_forward_kernels": bench_conv_forward_kernels(),
+            "ms_conv_forward_on_matrix_cores": round(ms_mfma, 4),
             "loss_first_last": [round(l, 6) for l in losses],
             "note": "MNIST CNN B64 (conv 1->32, conv 32->64, dense 3136->128->10): fwd + bwd + Adam + zero_grad through the "
                     "C API from Python, wall clock"}
@@ -732,7 +732,7 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build (the path has no inter-GPU work)",
               file=sys.stderr)
         sys.exit(2)
-    all_legs = ["step", "dense", "adam", "ln_gelu", "sdpa", "mlp", "cnn"]
+    all_legs = ["step", "dense", "adam", "ln_gelu", "sdpa", "mlp", "cnn", "conv"]
     legs = all_legs if args.legs == "all" else [l.strip() for l in args.legs.split(",") if l.strip()]
     unknown = [l for l in legs if l not in all_legs]
     if unknown:
@@ -774,6 +774,8 @@ def main():
         extra.update(bench_sdpa(hip, args.steps, args.warmup))
     if "mlp" in legs:
         extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20) * 25, max(args.warmup, 1) * 100)
+    if "conv" in legs:
+        extra["conv_forward_kernels"] = bench_conv_forward_kernels()
     if "cnn" in legs:
         extra["mnist_cnn_step"] = bench_cnn_step(max(args.steps, 20), max(args.warmup, 3))
     if extra:

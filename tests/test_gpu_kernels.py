@@ -717,6 +717,31 @@ def test_conv2d_forward_on_the_matrix_cores(hip, oracle, rng, shape):
         hip.check(hip.bh_conv2d_forward_mfma(dx_.ptr, dw_.ptr, None, y.ptr, B, ic, h, w, oc, 5, stride, pad))
 
 
+def test_conv2d_forward_on_the_matrix_cores_random_shapes(hip, oracle):
+    """Forty seeded random shapes (channel counts on both sides of the 32-channel LDS stage and the 64-channel tile, odd
+    counts, strides 1-3, paddings 0-2, images from 3x3 up, position counts that are no multiple of the 64-position tile)
+    against the oracle at the fp32 bound."""
+    shapes = np.random.default_rng(20250109)
+    for case in range(40):
+        B = int(shapes.integers(1, 5))
+        ic = int(shapes.choice([1, 2, 3, 7, 8, 16, 31, 32, 33, 48, 65, 70]))
+        oc = int(shapes.choice([1, 3, 16, 31, 32, 33, 63, 64, 65, 100, 130]))
+        h, w = int(shapes.integers(3, 20)), int(shapes.integers(3, 20))
+        stride, pad = int(shapes.integers(1, 4)), int(shapes.integers(0, 3))
+        data = np.random.default_rng(1000 + case)
+        x = data.standard_normal((B, ic, h, w)).astype(np.float32)
+        wt = (0.3 * data.standard_normal((oc, ic, 3, 3))).astype(np.float32)
+        b = data.standard_normal(oc).astype(np.float32)
+        ho, wo = (h + 2 * pad - 3) // stride + 1, (w + 2 * pad - 3) // stride + 1
+        y = hip.to_device(np.full((B, oc, ho, wo), np.nan, np.float32))
+        hip.check(hip.bh_conv2d_forward_mfma(dev(hip, x).ptr, dev(hip, wt).ptr, dev(hip, b).ptr, y.ptr, B, ic, h, w, oc, 3, stride, pad))
+        want = oracle.conv2d_forward(x, wt, b, stride, pad)
+        got = y.numpy()
+        shape = (B, ic, h, w, oc, stride, pad)
+        assert np.isfinite(got).all(), shape
+        assert np.max(np.abs(got - want)) <= 1e-5 * max(1.0, np.abs(want).max()), shape
+
+
 def test_conv2d_refuses_bad_shapes(hip):
     p = hip.empty(16)
     assert hip.bh_conv2d_forward(p.ptr, p.ptr, None, p.ptr, 1, 1, 2, 2, 1, 3, 1, 0) == -1       # kernel larger than image

@@ -151,20 +151,24 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_generic_kernel(const float
 // needs nine patch values and, per 32 output channels, nine weights.  The weights of the workgroup's 64 output channels
 // and of up to 32 input channels sit in LDS, split by kk parity ([oc][kk & 1][kk >> 1], row stride odd: conflict free
 // 4-byte reads).
-// Workgroup: 8 wavefronts = 64 channels x 64 positions; a wavefront owns 32 positions, both 32-channel halves (a patch
-// value feeds two products) and every fourth pair of input channels: small layers are bound by the latency of the
-// patch loads, and four wavefronts per position tile have four times the loads in flight.  The four partial sums are
-// added in a fixed order through LDS.  grid (ceil(P/64), ceil(oc/64)).
+// Workgroup: 2 * SPLIT wavefronts = 64 channels x 64 positions; a wavefront owns 32 positions, both 32-channel halves
+// (a patch value feeds two products) and every SPLIT-th pair of input channels; the SPLIT partial sums are added in a
+// fixed order through LDS.  SPLIT = 4 (512 lanes, one workgroup per CU) for small layers: they are bound by the latency
+// of the patch loads, and four wavefronts per position tile have four times the loads in flight.  SPLIT = 2 (256 lanes,
+// two workgroups per CU) for layers with many workgroups: one workgroup's staging, reduction and stores run under the
+// other's products.  grid (ceil(P/64), ceil(oc/64)).
 constexpr int kFmCi = 32;                       // input channels per LDS stage
 constexpr int kFmKk = kFmCi * 9;                // 288 contraction indices per stage
 constexpr int kFmRow = kFmKk + 1;               // LDS row stride in floats
-constexpr int kFmSplit = 4;                     // wavefronts that share a position tile
+constexpr int64_t kFmBlocksSplit2 = 257;        // from this many workgroups on (more than the part has CUs) a layer runs with SPLIT = 2
 
-__global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wt,
+template <int SPLIT>                            // wavefronts that share a position tile: 2 or 4
+__global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wt,
                                                                  const float* __restrict__ bias, float* __restrict__ y,
                                                                  ConvShape c, int positions) {
     extern __shared__ __align__(16) float wl[];          // [64][kFmRow] + bias[64]; the weights' part holds the partial sums afterwards
-    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, half = lane >> 5;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: what follows from it is the same for the whole wavefront
     const int wn = wv & 1, kg = wv >> 1;
     const int oc0 = blockIdx.y * 64;
     const int per = c.ho * c.wo, plane = c.h * c.w;
@@ -173,19 +177,21 @@ __global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __
     const int b = n / per, p = n - b * per;
     const int oh = p / c.wo, ow = p - oh * c.wo;
     const int ih0 = oh * c.stride - c.pad, iw0 = ow * c.stride - c.pad;
-    // the nine contraction indices 2j + half of a channel pair: which of the two channels, pixel offset, inside the image?
-    int off[9];
-    unsigned inside = 0, second_bits = 0;
+    // the nine contraction indices 2j + half of a channel pair: byte offset of the lane's patch value from the first
+    // channel's plane in image 0 (the second channel lies one plane further; byte offsets fit 32 bits, a tensor has fewer
+    // than 2^30 elements), and whether the tap lies inside the image.  The nine conditions live as wavefront masks in
+    // scalar registers, so that a turn costs one vector instruction per load and one per select: anything more per
+    // patch value competes with the matrix instructions for issue slots.
+    unsigned offb[9];
+    bool in[9];
 #pragma unroll
     for (int j = 0; j < 9; j++) {
         const int kk = 2 * j + half, cp = kk >= 9 ? 1 : 0, tap = kk - 9 * cp;
         const int kh = tap / 3, kw = tap - 3 * kh;
         const int ih = ih0 + kh, iw = iw0 + kw;
-        if (ih >= 0 && ih < c.h && iw >= 0 && iw < c.w) inside |= 1u << j;
-        second_bits |= (unsigned)cp << j;
-        off[j] = min(max(ih, 0), c.h - 1) * c.w + min(max(iw, 0), c.w - 1);
+        in[j] = ih >= 0 && ih < c.h && iw >= 0 && iw < c.w;
+        offb[j] = 4u * (unsigned)((b * c.ic + cp) * plane + min(max(ih, 0), c.h - 1) * c.w + min(max(iw, 0), c.w - 1));
     }
-    const float* xp = x + (int64_t)b * c.ic * plane;      // 32-bit offsets from here on: a tensor has fewer than 2^30 elements
     const float* wrow = wl + r * kFmRow + half * (kFmKk / 2);
     floatx16 acc[2];
 #pragma unroll
@@ -194,37 +200,47 @@ __global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __
     // patch values of channels ci, ci + 1: the loads go to clamped (valid) addresses and nothing looks at their results
     // until mask() runs three turns later -- a select right behind a load would make the wavefront wait for it there
     const auto fetch = [&](int ci, float (&v)[9]) {
+        const char* xc = reinterpret_cast<const char*>(x + (int64_t)ci * plane);     // the same for every lane
 #pragma unroll
-        for (int j = 0; j < 9; j++) v[j] = xp[min(ci + (int)((second_bits >> j) & 1u), c.ic - 1) * plane + off[j]];
+        for (int j = 0; j < 9; j++) {
+            // the empty statement keeps the offset's widening next to the load, where it folds into the load's
+            // scalar-base-plus-32-bit-offset form; hoisted out of the loop it would hold nine register pairs
+            unsigned o = offb[j];
+            asm volatile("" : "+v"(o));
+            v[j] = *reinterpret_cast<const float*>(xc + o);
+        }
     };
-    const auto mask = [&](int ci, float (&v)[9]) {         // taps outside the image and channels past the last count as zero
+    const auto mask = [&](float (&v)[9]) {                 // taps outside the image count as zero
 #pragma unroll
-        for (int j = 0; j < 9; j++) v[j] = (((inside >> j) & 1u) && ci + (int)((second_bits >> j) & 1u) < c.ic) ? v[j] : 0.f;
+        for (int j = 0; j < 9; j++) v[j] = in[j] ? v[j] : 0.f;
     };
-    const int l16 = tid & 15, rg = tid >> 4;               // weight staging: 16 lanes per row, 32 rows per pass
+    const int l16 = tid & 15, rg = tid >> 4;               // weight staging: 16 lanes per row, 8 * SPLIT rows per pass
     // the bias of the 64 channels travels with the first stage's weights and waits in LDS behind them: fetched at the end
     // it would cost a trip to memory of its own
     float* bl = wl + 64 * kFmRow;
     float bias_in = 0.f;
     if (tid < 64 && bias && oc0 + tid < c.oc) bias_in = bias[oc0 + tid];
+    // this wavefront's pairs of input channels are kg, kg + SPLIT, ... over the whole layer: a multiple of four to a full
+    // stage, so the four patch buffers take turns in step with the stages (a register copy would have to wait for the
+    // loads it copies) and the patch values run three turns ahead, across stage boundaries too (a turn's 18 products
+    // take a quarter of a trip to memory)
+    const int all_pairs = c.ic / 2;                        // an odd channel count's last channel follows behind its stage
+    float x0[9], x1[9], x2[9], x3[9];
+    if (kg < all_pairs) fetch(2 * kg, x0);
+    if (kg + SPLIT < all_pairs) fetch(2 * (kg + SPLIT), x1);
+    if (kg + 2 * SPLIT < all_pairs) fetch(2 * (kg + 2 * SPLIT), x2);
     for (int ci0 = 0; ci0 < c.ic; ci0 += kFmCi) {
         if (ci0) __syncthreads();                          // every wavefront is done with the previous stage's weights
-        const int chunk = min(kFmCi, c.ic - ci0);
-        const int pairs = (chunk + 1) / 2, real = chunk * 9;
-        // this wavefront's pairs are kg, kg + 4, ...; their patch values run three turns ahead (a turn's 18 products take
-        // a quarter of a trip to memory), the first three fetches of a stage are in flight while its weights are staged
-        float x0[9], x1[9], x2[9], x3[9];
-        fetch(ci0 + 2 * kg, x0);
-        fetch(ci0 + 2 * (kg + kFmSplit), x1);
-        fetch(ci0 + 2 * (kg + 2 * kFmSplit), x2);
+        const int real = min(kFmCi, c.ic - ci0) * 9;
         // weights of the stage: row oc of w holds its ic*9 values contiguously, so a stage's run of chunk*9 is contiguous;
-        // what lies past it (an odd channel count's partner, a short last stage) is zero.  A lane's 36 loads are in flight
+        // what lies past it (an odd channel count's partner, a short last stage) is zero.  36 loads of a lane are in flight
         // together before their LDS stores.
-        {
+#pragma unroll
+        for (int q0 = 0; q0 < 8 / SPLIT; q0 += 2) {
             float v[2][18];
 #pragma unroll
             for (int q = 0; q < 2; q++) {
-                const int o = rg + 32 * q;
+                const int o = rg + 8 * SPLIT * (q0 + q);
                 const float* src = wt + ((int64_t)min(oc0 + o, c.oc - 1) * c.ic + ci0) * 9;
 #pragma unroll
                 for (int i = 0; i < 18; i++) {
@@ -234,7 +250,7 @@ __global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __
             }
 #pragma unroll
             for (int q = 0; q < 2; q++) {
-                float* dst = wl + (rg + 32 * q) * kFmRow;
+                float* dst = wl + (rg + 8 * SPLIT * (q0 + q)) * kFmRow;
 #pragma unroll
                 for (int i = 0; i < 18; i++) {
                     const int kk = l16 + 16 * i;
@@ -244,22 +260,38 @@ __global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __
         }
         if (ci0 == 0 && tid < 64) bl[tid] = bias_in;
         __syncthreads();
-        // the four buffers take turns (a register copy would have to wait for the loads it copies)
-        const auto products = [&](int cp, float (&cur)[9], float (&ahead)[9]) {
-            if (cp + 3 * kFmSplit < pairs) fetch(ci0 + 2 * (cp + 3 * kFmSplit), ahead);
-            mask(ci0 + 2 * cp, cur);
-            const float* wp = wrow + cp * 9;
+        const int first = ci0 / 2 + kg;                    // this wavefront's first pair of the stage
+        const auto products = [&](int turn, float (&cur)[9], float (&ahead)[9]) {
+            const int gp = first + turn * SPLIT;
+            if (gp + 3 * SPLIT < all_pairs) fetch(2 * (gp + 3 * SPLIT), ahead);
+            mask(cur);
+            const float* wp = wrow + (kg + turn * SPLIT) * 9;
 #pragma unroll
             for (int j = 0; j < 9; j++) {
                 acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], cur[j], acc[0], 0, 0, 0);
                 acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * kFmRow + j], cur[j], acc[1], 0, 0, 0);
             }
         };
-        for (int cp = kg; cp < pairs; cp += 4 * kFmSplit) {
-            products(cp, x0, x3);
-            if (cp + kFmSplit < pairs) products(cp + kFmSplit, x1, x0);
-            if (cp + 2 * kFmSplit < pairs) products(cp + 2 * kFmSplit, x2, x1);
-            if (cp + 3 * kFmSplit < pairs) products(cp + 3 * kFmSplit, x3, x2);
+        for (int turn = 0; turn < kFmCi / 2 / SPLIT && first + turn * SPLIT < all_pairs; turn += 4) {
+            products(turn, x0, x3);
+            if (first + (turn + 1) * SPLIT < all_pairs) products(turn + 1, x1, x0);
+            if (first + (turn + 2) * SPLIT < all_pairs) products(turn + 2, x2, x1);
+            if (first + (turn + 3) * SPLIT < all_pairs) products(turn + 3, x3, x2);
+        }
+        // the single last channel of an odd count: one wavefront per position half takes it with its lanes of the
+        // pair's second channel reading the first and counting as zero (the weights past the last channel are zero too)
+        const int single = c.ic / 2 - ci0 / 2;            // its pair's index within this stage
+        if ((c.ic & 1) && ci0 + kFmCi >= c.ic && kg == single % SPLIT) {
+            const char* xc = reinterpret_cast<const char*>(x + (int64_t)(c.ic - 1) * plane);
+            const float* wp = wrow + single * 9;
+#pragma unroll
+            for (int j = 0; j < 9; j++) {
+                const bool other = 2 * j + half >= 9;
+                float v = *reinterpret_cast<const float*>(xc + (offb[j] - (other ? 4u * (unsigned)plane : 0u)));
+                v = (in[j] && !other) ? v : 0.f;
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], v, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * kFmRow + j], v, acc[1], 0, 0, 0);
+            }
         }
     }
     __syncthreads();                                       // the weights are no longer needed: their LDS holds the partial sums
@@ -273,7 +305,7 @@ __global__ __launch_bounds__(512, 2) void conv2d_fwd_mfma_kernel(const float* __
     __syncthreads();
     if (kg > 0 || n_raw >= positions) return;
 #pragma unroll
-    for (int g = 0; g < kFmSplit - 1; g++) {
+    for (int g = 0; g < SPLIT - 1; g++) {
         const float* src = wl + ((g * 2 + wn) * 32) * 64 + lane;
 #pragma unroll
         for (int t = 0; t < 2; t++)
@@ -514,13 +546,20 @@ int bh_conv2d_forward_mfma(const float* x, const float* w, const float* bias, fl
     constexpr size_t lds = sizeof(float) * (64 * kFmRow + 64);      // weights + bias
     static bool attr = false;
     if (!attr) {
-        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel),
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<4>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<2>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
         if (rc) return rc;
         attr = true;
     }
     const dim3 grid((unsigned)ceil_div(positions, 64), (unsigned)ceil_div(c.oc, 64));
-    hipLaunchKernelGGL(conv2d_fwd_mfma_kernel, grid, dim3(512), lds, stream(), x, w, bias, y, c, (int)positions);
+    // the split follows the shape alone, not the device: a layer's sums always run in the same order
+    if ((int64_t)grid.x * grid.y >= kFmBlocksSplit2)
+        hipLaunchKernelGGL(conv2d_fwd_mfma_kernel<2>, grid, dim3(256), lds, stream(), x, w, bias, y, c, (int)positions);
+    else
+        hipLaunchKernelGGL(conv2d_fwd_mfma_kernel<4>, grid, dim3(512), lds, stream(), x, w, bias, y, c, (int)positions);
     return BH_LAUNCH_CHECK("conv2d_fwd_mfma_kernel");
 }
 

@@ -22,11 +22,18 @@
 static int g_reference_input_grad = -1;   /* -1: not set by a call, follow reference-exact mode */
 
 void boat_hip_conv_reference_input_grad(int enable) { g_reference_input_grad = enable < 0 ? -1 : enable != 0; }
-/* forward on the matrix cores (3x3 kernels with at least 8 input channels); off by default because the direct kernel's
- * output is bit-identical to the reference's and the MFMA order is not.  BOAT_HIP_CONV_FORWARD_MFMA=1 in the
- * environment sets the initial value. */
+/* forward on the matrix cores (3x3 kernels of layers wide enough for it to win, see conv_forward_wants_mfma); off by
+ * default because the direct kernel's output is bit-identical to the reference's and the MFMA order is not.
+ * BOAT_HIP_CONV_FORWARD_MFMA=1 in the environment sets the initial value. */
 static int g_forward_mfma = -1;
 void boat_hip_conv_forward_matrix_cores(int enable) { g_forward_mfma = enable != 0; }
+/* The matrix-core kernel works on tiles of 64 output channels and pairs of input channels, and a workgroup of it costs
+ * a weight staging and a reduction whatever the layer: measured against the direct kernel over batch 16-256, images
+ * 14x14 and 28x28, it wins (1.3x to 3.6x) from 32 output channels on with at least 8 input channels (a tie at 8 -> 32)
+ * and from 16 output channels on with at least 32 input channels; narrower layers lose up to 2x. */
+static int conv_forward_wants_mfma(size_t in_channels, size_t out_channels) {
+    return (in_channels >= 8 && out_channels >= 32) || (in_channels >= 32 && out_channels >= 16);
+}
 static int forward_mfma(void) {
     if (g_forward_mfma < 0) {
         const char* e = getenv("BOAT_HIP_CONV_FORWARD_MFMA");
@@ -112,7 +119,7 @@ boat_tensor_t* boat_conv_layer_forward(boat_conv_layer_t* l, const boat_tensor_t
     const float* pw = bt_dev_read(l->weight);
     const float* pb = (l->use_bias && l->bias) ? bt_dev_read(l->bias) : NULL;
     float* py = bt_dev_write(out);
-    const int mfma = forward_mfma() && k == 3 && l->in_channels >= 8;
+    const int mfma = forward_mfma() && k == 3 && conv_forward_wants_mfma(l->in_channels, l->out_channels);
     if (!px || !pw || !py ||
         !boat_hip_ok((mfma ? bh_conv2d_forward_mfma : bh_conv2d_forward)(px, pw, pb, py, batch, (int64_t)l->in_channels, h, w,
                                                                          (int64_t)l->out_channels, k, s, p),

@@ -544,11 +544,12 @@ def test_conv_known_answer_and_hooks(boat):
 
 def test_conv_forward_on_the_matrix_cores_is_opt_in(boat, oracle, rng):
     """boat_conv_layer_forward is bit-identical to the reference's loop order by default (src/layers/conv.c:326-437); after
-    boat_hip_conv_forward_matrix_cores(1) a 3x3 layer with at least 8 input channels runs as one MFMA contraction and
-    agrees to fp32 rounding; layers the switch does not cover (few channels, other kernel sizes) stay bit-identical."""
+    boat_hip_conv_forward_matrix_cores(1) a 3x3 layer wide enough to gain (here 16 -> 32 channels) runs as one MFMA
+    contraction and agrees to fp32 rounding; layers the switch does not cover (few channels, other kernel sizes) stay
+    bit-identical."""
     x = rng.standard_normal((4, 16, 10, 9)).astype(np.float32)
-    w = (0.2 * rng.standard_normal((24, 16, 3, 3))).astype(np.float32)
-    b = rng.standard_normal(24).astype(np.float32)
+    w = (0.2 * rng.standard_normal((32, 16, 3, 3))).astype(np.float32)
+    b = rng.standard_normal(32).astype(np.float32)
     want = oracle.conv2d_forward(x, w, b, 1, 1)
     y_default, _ = bc.conv_layer(boat, x, w, b, 1, 1, [])
     assert np.array_equal(y_default, want)
@@ -562,7 +563,8 @@ def test_conv_forward_on_the_matrix_cores_is_opt_in(boat, oracle, rng):
     finally:
         boat.boat_hip_conv_forward_matrix_cores(0)
     assert np.max(np.abs(y_mfma - want)) <= 1e-5 * np.abs(want).max()
-    assert grads[0][2].tolist() == [4.0 * 10 * 9] * 24                      # the backward hooks are untouched
+    assert grads[0][2].tolist() == [4.0 * 10 * 9] * 32                      # the backward hooks are untouched
+    assert not np.array_equal(y_mfma, want)                                # it did take the other kernel
     assert np.array_equal(y_small, oracle.conv2d_forward(x_small, w_small, b_small, 1, 1))
     y_again, _ = bc.conv_layer(boat, x, w, b, 1, 1, [])
     assert np.array_equal(y_again, want)

@@ -692,6 +692,9 @@ def test_conv2d_forward_output_channel_tiles(hip, oracle, rng, shape):
 CONV_MFMA_SHAPES = [  # batch, ic, h, w, oc, k(=3), stride, pad: ragged channel counts, odd channel counts, strides, two LDS stages
     (2, 3, 7, 6, 4, 3, 1, 1), (3, 1, 8, 8, 5, 3, 1, 0), (2, 3, 10, 10, 2, 3, 3, 0), (1, 5, 3, 3, 70, 3, 1, 1),
     (8, 32, 14, 14, 64, 3, 1, 1), (64, 32, 14, 14, 64, 3, 1, 1), (3, 33, 9, 11, 65, 3, 2, 1), (2, 70, 6, 6, 40, 3, 1, 2),
+    # more than 256 workgroups: the kernel's two-wavefronts-per-position-tile form
+    (40, 33, 20, 21, 65, 3, 1, 1), (64, 64, 28, 28, 64, 3, 1, 1), (30, 70, 31, 29, 130, 3, 2, 1), (40, 5, 21, 20, 10, 3, 1, 1),
+    (33, 8, 30, 30, 3, 3, 1, 2),
 ]
 
 

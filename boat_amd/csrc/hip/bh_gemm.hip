@@ -309,6 +309,12 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             fa0.load(smem, wm * Cfg::WM, 0, r, half);
             fb0.load(smem + A_FLOATS, wn * Cfg::WN, 0, r, half);
         }
+        // A wavefront whose load cannot be queued issues nothing else, matrix instructions included, and eight
+        // wavefronts that issue their 64 KB of loads at the same point queue behind each other for about a thousand
+        // cycles per pair.  So only half of them issue right after the barrier; the other half issue the same pair one
+        // group of products later, into the stage that barrier freed (8192x4096x4096: 1.94 -> 1.89 ms, the same bits).
+        // More than two issue points were measured and are slower.
+        const bool late = NW >= 8 && __builtin_amdgcn_readfirstlane(wave) >= NW / 2;
         int cur = 0;
         for (int64_t p = 0; p < pairs; p++) {
             const float* sa0 = smem + cur * 2 * STAGE;     // first k-tile of the pair: A, then B
@@ -316,15 +322,16 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             fa1.load(sa0, wm * Cfg::WM, 8, r, half);
             fb1.load(sa0 + A_FLOATS, wn * Cfg::WN, 8, r, half);
             products(fa0, fb0);
+            if (late && p >= 1 && p + 1 < pairs) issue_pair((unsigned)(cur ^ 1));     // pair p+1; pairs 0 and 1 were issued up front
             fa0.load(sa1, wm * Cfg::WM, 0, r, half);
             fb0.load(sa1 + A_FLOATS, wn * Cfg::WN, 0, r, half);
             products(fa1, fb1);
             fa1.load(sa1, wm * Cfg::WM, 8, r, half);
             fb1.load(sa1 + A_FLOATS, wn * Cfg::WN, 8, r, half);
             products(fa0, fb0);
-            wait_direct_loads();       // pair p+1, issued a whole pair ago
+            wait_direct_loads();       // pair p+1, issued a whole pair (or, by the late half, two groups of products) ago
             __syncthreads();           // ... is visible to everyone, and everyone has the last fragments of stage cur in registers
-            if (p + 2 < pairs) issue_pair((unsigned)cur);
+            if (!late && p + 2 < pairs) issue_pair((unsigned)cur);
             if (p + 1 < pairs) {
                 const float* na = smem + (cur ^ 1) * 2 * STAGE;
                 fa0.load(na, wm * Cfg::WM, 0, r, half);
@@ -1011,19 +1018,18 @@ static int launch_mfma_layout2(const GemmArgs& g, int64_t batch, bool a_kc, bool
     return launch_mfma<Cfg, false, false, DIRECT>(g, batch);
 }
 
-// the big tile with two k-tiles per barrier (direct loads, contraction a multiple of 32, no split)
-static int launch_mfma_big_pairs(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc);
+// an eight-wavefront tile with two k-tiles per barrier (direct loads, every workgroup's contraction range a multiple of 32)
+template <typename Cfg>
+static int launch_mfma_pairs(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc) {
+    if (a_kc && b_kc) return launch_mfma<Cfg, true, true, true, 2>(g, batch);
+    if (a_kc && !b_kc) return launch_mfma<Cfg, true, false, true, 2>(g, batch);
+    if (!a_kc && b_kc) return launch_mfma<Cfg, false, true, true, 2>(g, batch);
+    return launch_mfma<Cfg, false, false, true, 2>(g, batch);
+}
 
 template <typename Cfg>
 static int launch_mfma_layout(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc, bool direct) {
     return direct ? launch_mfma_layout2<Cfg, true>(g, batch, a_kc, b_kc) : launch_mfma_layout2<Cfg, false>(g, batch, a_kc, b_kc);
-}
-
-static int launch_mfma_big_pairs(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc) {
-    if (a_kc && b_kc) return launch_mfma<CfgBig, true, true, true, 2>(g, batch);
-    if (a_kc && !b_kc) return launch_mfma<CfgBig, true, false, true, 2>(g, batch);
-    if (!a_kc && b_kc) return launch_mfma<CfgBig, false, true, true, 2>(g, batch);
-    return launch_mfma<CfgBig, false, false, true, 2>(g, batch);
 }
 
 template <bool A_KFAST, bool B_KFAST, int KCH>
@@ -1067,7 +1073,7 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
 }
 
 static int g_force_splits = 0;    // test hook: > 0 = this many k-splits for the MFMA tiles
-static int g_pairs = 1;           // test hook: 0 = the big tile keeps one k-tile per barrier
+static int g_pairs = 1;           // test hook: 0 = every tile keeps one k-tile per barrier
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
 static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, 6 = tiny, -1 = heuristic
 
@@ -1091,7 +1097,7 @@ int bh_gemm_force_splits(int splits) {
 
 // test/benchmark hook: 0 stages operand tiles through registers even where the direct-to-LDS loader applies
 int bh_gemm_force_direct(int mode) {
-    g_pairs = !(mode & 2);       // bit 1 set: one k-tile per barrier also for the big tile
+    g_pairs = !(mode & 2);       // bit 1 set: one k-tile per barrier also for the eight-wavefront tiles
     g_force_direct = mode < 0 ? -1 : (mode & 1);
     return BH_OK;
 }
@@ -1293,7 +1299,9 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         if (plan_splits > 0 && g_force_cfg < 0) splits = plan_splits;
         if (g_force_splits > 0 && g_force_splits <= k / kBK) splits = g_force_splits;
         if (splits > 1) {
-            g.k_per_split = ceil_div(ceil_div(k, splits), kBK) * kBK;
+            // whole pairs of k-tiles per workgroup where the contraction allows it (the paired main loop needs them)
+            const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
+            g.k_per_split = ceil_div(ceil_div(k, splits), unit) * unit;
             g.k_splits = (int)ceil_div(k, g.k_per_split);
         }
     }
@@ -1308,13 +1316,13 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     // the direct-to-LDS loader cannot zero-fill a k tail, and its edge clamps need 4 valid floats in a row
     const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4);
     int rc;
+    // the eight-wavefront tiles take two k-tiles per barrier whenever every workgroup's contraction range is whole pairs
+    // (measured at the block's shapes with the staggered loads: 1.5-3 % faster than one tile per barrier on all three)
+    const bool pairs = direct && g_pairs && k % (2 * kBK) == 0 && (g.k_splits == 1 || g.k_per_split % (2 * kBK) == 0);
     switch (cfg) {
-        case 2:
-            if (direct && g_pairs && g.k_splits == 1 && k % (2 * kBK) == 0) rc = launch_mfma_big_pairs(run, batch, a_kc, b_kc);
-            else rc = launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct);
-            break;
-        case 3: rc = launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc, direct); break;
-        case 4: rc = launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc, direct); break;
+        case 2: rc = pairs ? launch_mfma_pairs<CfgBig>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct); break;
+        case 3: rc = pairs ? launch_mfma_pairs<CfgTall>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc, direct); break;
+        case 4: rc = pairs ? launch_mfma_pairs<CfgWide>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc, direct); break;
         default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc, direct); break;
     }
     if (rc == BH_OK && g.k_splits > 1) rc = launch_fold(ws, c, bias, m, n, ldc, g.k_splits, batch, g.stride_c, accumulate);

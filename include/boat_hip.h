@@ -263,9 +263,9 @@ int bh_zero_multi(float* const* p, const int64_t* n, int count);
  * 5 = small-problem kernel (whole k-chunk in LDS, one trip to memory), 6 = tiny-problem kernel (operands straight
  * into the MFMA registers, contraction split among a workgroup's wavefronts), -1 = heuristic (default).
  * bh_gemm_force_direct: 0 = MFMA tiles stage their operands through registers; 1 or -1 (default) = operands go
- * straight to LDS (global_load_lds) whenever the contraction length is a multiple of 16, and the 256x256 tile keeps
- * two k-tiles per LDS stage (one barrier per 32 k) when it is a multiple of 32; 3 = straight to LDS with one k-tile per
- * stage everywhere.
+ * straight to LDS (global_load_lds) whenever the contraction length is a multiple of 16, and the eight-wavefront
+ * tiles keep two k-tiles per LDS stage (one barrier per 32 k) when every workgroup's share of it is a multiple of 32;
+ * 3 = straight to LDS with one k-tile per stage everywhere.
  * bh_sdpa_force_general: 0 = heuristic (default); 1 = always the row kernels; 2 = always the GEMM-based path (batched
  * bh_gemm products with row kernels for softmax and dS in between, what shapes other than head_dim 64 use from 64 keys on). */
 int bh_gemm_force_config(int cfg);

@@ -468,7 +468,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     }
     // accumulate: the old values of one 32-row slab are fetched by loads that depend on nothing, then added; a load
     // placed between the stores below would have to wait for them (the compiler cannot tell the rows apart)
-    // (wavefront tiles of 128x64 have no registers to spare for this and keep the load next to its store)
+    // (with wavefront tiles of 128x64 the addresses, which the stores need again, would not fit the register file
+    // next to the accumulators: those tiles take the pipelined groups further down)
     constexpr bool kPrefetchC = TM * TN <= 4;
     if (kPrefetchC && add_c) {
 #pragma unroll
@@ -494,6 +495,46 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             }
         }
     }
+    if (!kPrefetchC && add_c) {
+        // the larger wavefront tiles: groups of four rows, the old values of the next group fetched before the current
+        // group is stored (a load behind a store has to stay there: the compiler cannot tell the rows apart), so that
+        // one trip to memory is exposed per wavefront instead of one per group, and a group's addresses die with it
+        constexpr int NG = TM * 4;
+        float prev[2][4][TN];
+        const auto fetch = [&](int G, float (&pv)[4][TN]) {
+            const int i = G >> 2, eq = G & 3;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int ri = eq * 8 + half * 4 + e4;
+                const int64_t row = m0 + wm * Cfg::WM + (A_KC ? i * 32 + ri : TM * ri + i);
+                const float* crow = C + row * g.ldc;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
+                    pv[e4][j] = (row < g.m && col < g.n) ? __builtin_nontemporal_load(crow + col) : 0.f;
+                }
+            }
+        };
+        fetch(0, prev[0]);
+#pragma unroll
+        for (int G = 0; G < NG; G++) {
+            if (G + 1 < NG) fetch(G + 1, prev[(G + 1) & 1]);
+            const int i = G >> 2, eq = G & 3;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int ri = eq * 8 + half * 4 + e4;
+                const int64_t row = m0 + wm * Cfg::WM + (A_KC ? i * 32 + ri : TM * ri + i);
+                if (row >= g.m) continue;
+                float* crow = C + row * g.ldc;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
+                    if (col < g.n) crow[col] = acc[i][j][eq * 4 + e4] + bias_v[j] + prev[G & 1][e4][j];
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -506,9 +547,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             for (int j = 0; j < TN; j++) {
                 const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
                 if (col < g.n) {
-                    float v = acc[i][j][e] + bias_v[j];
-                    if (!kPrefetchC && add_c) v += crow[col];
-                    crow[col] = v;
+                    crow[col] = acc[i][j][e] + bias_v[j];
                 }
             }
         }

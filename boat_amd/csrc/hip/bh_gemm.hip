@@ -30,6 +30,7 @@
 #include "bh_common.h"
 
 #include <stdint.h>
+#include <type_traits>
 
 namespace bh {
 
@@ -157,10 +158,14 @@ template <bool KC, int R> struct DirectTile {
     static constexpr int floats = blocks * block_stride;
 };
 
-__device__ __forceinline__ void load_block_to_lds(const float* src, unsigned lds_byte_addr) {
+__device__ __forceinline__ void load_block_to_lds(const float* base, unsigned lane_byte_offset, unsigned lds_byte_addr) {
     // M0 carries the LDS address of the block.  It is a reserved register that the compiler neither allocates nor keeps
     // live in these kernels (no s_movrel / s_sendmsg / GWS), so nothing of its own is disturbed.
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_byte_addr) : "memory");
+    // The address is a scalar base (the same for the whole workgroup, advanced from k-tile to k-tile by scalar
+    // instructions) plus a 32-bit byte offset per lane that never changes: the main loop spends no vector instruction
+    // on addresses -- it has no issue slot to spare between two matrix instructions.
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(lane_byte_offset), "s"(base), "s"(lds_byte_addr) : "memory");
 }
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -168,13 +173,15 @@ template <bool KC, int R, int NW>
 struct DirectLoader {
     static constexpr int PER = DirectTile<KC, R>::blocks / NW;   // blocks per wavefront and k-tile
     static_assert(DirectTile<KC, R>::blocks % NW == 0, "blocks must divide among the wavefronts");
-    const float* src[PER];
+    const float* base;      // the workgroup's tile at the next k-tile to issue (the same for every lane)
+    unsigned off[PER];      // this lane's byte offset from base (the host keeps leading dimensions below 2^22, so 256 rows fit)
     unsigned dst[PER];      // LDS byte address inside stage 0
     int64_t step;           // floats from one k-tile to the next
 
-    __device__ __forceinline__ void init(const float* base, int64_t ld, int64_t row0, int64_t row_lim, int64_t k_begin,
+    __device__ __forceinline__ void init(const float* mat, int64_t ld, int64_t row0, int64_t row_lim, int64_t k_begin,
                                          const float* lds_tile, int wave, int lane) {
         step = KC ? kBK : kBK * ld;
+        base = KC ? mat + row0 * ld + k_begin : mat + k_begin * ld;
 #pragma unroll
         for (int j = 0; j < PER; j++) {
             const int blk = wave + j * NW;
@@ -182,12 +189,12 @@ struct DirectLoader {
                 int64_t row = row0 + 16 * blk + (lane >> 2);
                 if (row > row_lim - 1) row = row_lim - 1;
                 const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
-                src[j] = base + row * ld + k_begin + 4 * chunk;
+                off[j] = (unsigned)(((row - row0) * ld + 4 * chunk) * (int64_t)sizeof(float));
             } else {
                 const int krow = R == 256 ? blk : 2 * blk + (lane >> 5);
                 int64_t col = row0 + 4 * (R == 256 ? lane : (lane & 31));
                 if (col > row_lim - 4) col = row_lim - 4;
-                src[j] = base + (k_begin + krow) * ld + col;
+                off[j] = (unsigned)((krow * ld + col) * (int64_t)sizeof(float));
             }
             const unsigned addr = (unsigned)(uintptr_t)(lds_ptr_t)(lds_tile + blk * DirectTile<KC, R>::block_stride);
             dst[j] = __builtin_amdgcn_readfirstlane(addr);
@@ -196,10 +203,8 @@ struct DirectLoader {
     // issue this wavefront's blocks of the next k-tile into the stage at byte offset stage_bytes
     __device__ __forceinline__ void issue(unsigned stage_bytes) {
 #pragma unroll
-        for (int j = 0; j < PER; j++) {
-            load_block_to_lds(src[j], dst[j] + stage_bytes);
-            src[j] += step;
-        }
+        for (int j = 0; j < PER; j++) load_block_to_lds(base, off[j], dst[j] + stage_bytes);
+        base += step;
     }
 };
 
@@ -281,7 +286,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         DirectLoader<B_KC, BN, NW> db;
         da.init(A, g.lda, m0, g.m, k_begin, smem, wave, lane);
         db.init(B, g.ldb, n0, g.n, k_begin, smem + A_FLOATS, wave, lane);
-        const int64_t pairs = (k_end - k_begin) / (2 * kBK);
+        const int pairs = (int)((k_end - k_begin) / (2 * kBK));
         DirectFrags<A_KC, BM, TM> fa0, fa1;
         DirectFrags<B_KC, BN, TN> fb0, fb1;
         auto products = [&](const DirectFrags<A_KC, BM, TM>& fa, const DirectFrags<B_KC, BN, TN>& fb) {
@@ -315,8 +320,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         // group of products later, into the stage that barrier freed (8192x4096x4096: 1.94 -> 1.89 ms, the same bits).
         // More than two issue points were measured and are slower.
         const bool late = NW >= 8 && __builtin_amdgcn_readfirstlane(wave) >= NW / 2;
-        int cur = 0;
-        for (int64_t p = 0; p < pairs; p++) {
+        // The stage a pair sits in is a compile-time constant of its iteration (two iterations per trip of the loop), so
+        // every fragment address is one of a few per-lane registers plus an immediate offset: no vector instruction for
+        // addresses between the matrix instructions.
+        const auto iteration = [&](auto stage_const, int p) {
+            constexpr int cur = decltype(stage_const)::value;
             const float* sa0 = smem + cur * 2 * STAGE;     // first k-tile of the pair: A, then B
             const float* sa1 = sa0 + STAGE;                // second k-tile
             fa1.load(sa0, wm * Cfg::WM, 8, r, half);
@@ -338,8 +346,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                 fb0.load(na + A_FLOATS, wn * Cfg::WN, 0, r, half);
             }
             products(fa1, fb1);
-            cur ^= 1;
+        };
+        int p = 0;
+        for (; p + 1 < pairs; p += 2) {
+            iteration(std::integral_constant<int, 0>{}, p);
+            iteration(std::integral_constant<int, 1>{}, p + 1);
         }
+        if (p < pairs) iteration(std::integral_constant<int, 0>{}, p);
     } else if constexpr (DIRECT) {
         // tile kt+1 streams straight into the other LDS stage while tile kt feeds the MFMAs; the wait for this
         // wavefront's own loads and the barrier at the end of the k-tile publish it to the workgroup
@@ -348,7 +361,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         DirectLoader<B_KC, BN, NW> db;
         da.init(A, g.lda, m0, g.m, k_begin, smem, wave, lane);
         db.init(B, g.ldb, n0, g.n, k_begin, smem + A_FLOATS, wave, lane);
-        const int64_t kt_count = (k_end - k_begin) / kBK;
+        const int kt_count = (int)((k_end - k_begin) / kBK);
         // Two tiles are in flight ahead of the arithmetic and the fragments are software pipelined across the one
         // barrier of a k-tile, which sits between its two halves: the fragments of the second half are read while the
         // first half's products run, those of the next tile's first half right after the barrier while the second
@@ -369,8 +382,10 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             fa0.load(smem, wm * Cfg::WM, 0, r, half);
             fb0.load(smem + A_FLOATS, wn * Cfg::WN, 0, r, half);
         }
-        int cur = 0;
-        for (int64_t kt = 0; kt < kt_count; kt++) {
+        // the stage is a compile-time constant of the iteration (two per trip of the loop): fragment addresses are
+        // per-lane registers plus immediates, no vector instruction for addresses between the matrix instructions
+        const auto iteration = [&](auto stage_const, int kt) {
+            constexpr int cur = decltype(stage_const)::value;
             const float* sa = smem + cur * STAGE;
             const float* sb = sa + A_FLOATS;
             fa1.load(sa, wm * Cfg::WM, 8, r, half);
@@ -387,7 +402,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             wait_direct_loads();       // tile kt+1, issued a whole tile ago
             __syncthreads();           // ... is visible to everyone, and everyone has its fragments of stage cur in registers
             if (kt + 2 < kt_count) {
-                const unsigned stage_bytes = (unsigned)(cur * STAGE * sizeof(float));
+                constexpr unsigned stage_bytes = (unsigned)(cur * STAGE * sizeof(float));
                 da.issue(stage_bytes);
                 db.issue(stage_bytes);
             }
@@ -405,8 +420,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                     for (int j = 0; j < TN; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1.v[s][i], fb1.v[s][j], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            cur ^= 1;
+        };
+        int kt = 0;
+        for (; kt + 1 < kt_count; kt += 2) {
+            iteration(std::integral_constant<int, 0>{}, kt);
+            iteration(std::integral_constant<int, 1>{}, kt + 1);
         }
+        if (kt < kt_count) iteration(std::integral_constant<int, 0>{}, kt);
     } else {
         TileLoader<A_KC, BM, NT> la;
         TileLoader<B_KC, BN, NT> lb;
@@ -1353,7 +1373,9 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         run.stride_c = m * n;
     }
     // the direct-to-LDS loader cannot zero-fill a k tail, and its edge clamps need 4 valid floats in a row
-    const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4);
+    // (and it addresses a tile with 32-bit byte offsets from the tile's first row: leading dimensions below 2^22)
+    const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4) &&
+                        lda < ((int64_t)1 << 22) && ldb < ((int64_t)1 << 22);
     int rc;
     // the eight-wavefront tiles take two k-tiles per barrier whenever every workgroup's contraction range is whole pairs
     // (measured at the block's shapes with the staggered loads: 1.5-3 % faster than one tile per barrier on all three)

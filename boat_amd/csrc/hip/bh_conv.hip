@@ -26,6 +26,7 @@
 // flip_taps == 0 computes the true gradient dx[ih,iw] = sum w[oc,ic,kh,kw]*dy[oh,ow]; flip_taps != 0 reproduces
 // the reference's pairing (the weights are mirrored into a scratch copy first), so that its numbers can be checked.
 #include "bh_common.h"
+#include <type_traits>
 
 #include <math.h>
 
@@ -193,6 +194,11 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
         offb[j] = 4u * (unsigned)((b * c.ic + cp) * plane + min(max(ih, 0), c.h - 1) * c.w + min(max(iw, 0), c.w - 1));
     }
     const float* wrow = wl + r * kFmRow + half * (kFmKk / 2);
+    // the second 32 channels' rows lie beyond the reach of a paired LDS read's offsets from wrow: their own base, kept
+    // in a register of its own (the empty statement hides that it is wrow plus a constant, which the compiler would
+    // otherwise add again in every turn)
+    int far_row = (r + 32) * kFmRow + half * (kFmKk / 2);
+    asm volatile("" : "+v"(far_row));
     floatx16 acc[2];
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[0][e] = acc[1][e] = 0.f;
@@ -203,11 +209,11 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
         const char* xc = reinterpret_cast<const char*>(x + (int64_t)ci * plane);     // the same for every lane
 #pragma unroll
         for (int j = 0; j < 9; j++) {
-            // the empty statement keeps the offset's widening next to the load, where it folds into the load's
-            // scalar-base-plus-32-bit-offset form; hoisted out of the loop it would hold nine register pairs
-            unsigned o = offb[j];
-            asm volatile("" : "+v"(o));
-            v[j] = *reinterpret_cast<const float*>(xc + o);
+            // the empty statement (it leaves the offset as it is) keeps the offset's widening next to the load, where it
+            // folds into the load's scalar-base-plus-32-bit-offset form; hoisted out of the loop it would hold nine
+            // register pairs
+            asm volatile("" : "+v"(offb[j]));
+            v[j] = *reinterpret_cast<const float*>(xc + offb[j]);
         }
     };
     const auto mask = [&](float (&v)[9]) {                 // taps outside the image count as zero
@@ -226,10 +232,18 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
     // take a quarter of a trip to memory)
     const int all_pairs = c.ic / 2;                        // an odd channel count's last channel follows behind its stage
     float x0[9], x1[9], x2[9], x3[9];
-    if (kg < all_pairs) fetch(2 * kg, x0);
-    if (kg + SPLIT < all_pairs) fetch(2 * (kg + SPLIT), x1);
-    if (kg + 2 * SPLIT < all_pairs) fetch(2 * (kg + 2 * SPLIT), x2);
-    for (int ci0 = 0; ci0 < c.ic; ci0 += kFmCi) {
+    // a fetch past the last pair re-reads the last pair (valid memory, never used): with the same number of loads on
+    // every path the waits the compiler places in front of a turn's selects count exactly the three turns in flight
+    // (a fetch under a condition makes it wait for everything but the current turn's loads)
+    const auto fetch_pair = [&](int pair, float (&v)[9]) { fetch(2 * min(pair, all_pairs - 1), v); };
+    if (all_pairs > 0) {
+        fetch_pair(kg, x0);
+        fetch_pair(kg + SPLIT, x1);
+        fetch_pair(kg + 2 * SPLIT, x2);
+    }
+    // a stage of the layer; FULL: all its 16 pairs of channels exist, so every turn runs unconditionally
+    const auto stage = [&](int ci0, auto full_const) {
+        constexpr bool FULL = decltype(full_const)::value;
         if (ci0) __syncthreads();                          // every wavefront is done with the previous stage's weights
         const int real = min(kFmCi, c.ic - ci0) * 9;
         // weights of the stage: row oc of w holds its ic*9 values contiguously, so a stage's run of chunk*9 is contiguous;
@@ -245,16 +259,17 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
 #pragma unroll
                 for (int i = 0; i < 18; i++) {
                     const int kk = l16 + 16 * i;
-                    v[q][i] = (oc0 + o < c.oc && kk < real) ? src[kk] : 0.f;
+                    v[q][i] = src[FULL ? kk : min(kk, real - 1)];     // a valid address in any case; what does not exist becomes zero below
                 }
             }
 #pragma unroll
             for (int q = 0; q < 2; q++) {
-                float* dst = wl + (rg + 8 * SPLIT * (q0 + q)) * kFmRow;
+                const int o = rg + 8 * SPLIT * (q0 + q);
+                float* dst = wl + o * kFmRow;
 #pragma unroll
                 for (int i = 0; i < 18; i++) {
                     const int kk = l16 + 16 * i;
-                    dst[(kk & 1) * (kFmKk / 2) + (kk >> 1)] = v[q][i];
+                    dst[(kk & 1) * (kFmKk / 2) + (kk >> 1)] = (oc0 + o < c.oc && (FULL || kk < real)) ? v[q][i] : 0.f;
                 }
             }
         }
@@ -263,20 +278,35 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
         const int first = ci0 / 2 + kg;                    // this wavefront's first pair of the stage
         const auto products = [&](int turn, float (&cur)[9], float (&ahead)[9]) {
             const int gp = first + turn * SPLIT;
-            if (gp + 3 * SPLIT < all_pairs) fetch(2 * (gp + 3 * SPLIT), ahead);
+            if (FULL) fetch_pair(gp + 3 * SPLIT, ahead);
+            else if (gp + 3 * SPLIT < all_pairs) fetch(2 * (gp + 3 * SPLIT), ahead);
+            // nothing moves across this line: left to itself the scheduler lifts the selects of a later turn up to their
+            // loads, three turns early, and the wavefront waits for those loads there
+            __builtin_amdgcn_sched_barrier(0);
             mask(cur);
             const float* wp = wrow + (kg + turn * SPLIT) * 9;
+            const float* wq = wl + far_row + (kg + turn * SPLIT) * 9;
 #pragma unroll
             for (int j = 0; j < 9; j++) {
                 acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], cur[j], acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * kFmRow + j], cur[j], acc[1], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wq[j], cur[j], acc[1], 0, 0, 0);
             }
         };
-        for (int turn = 0; turn < kFmCi / 2 / SPLIT && first + turn * SPLIT < all_pairs; turn += 4) {
-            products(turn, x0, x3);
-            if (first + (turn + 1) * SPLIT < all_pairs) products(turn + 1, x1, x0);
-            if (first + (turn + 2) * SPLIT < all_pairs) products(turn + 2, x2, x1);
-            if (first + (turn + 3) * SPLIT < all_pairs) products(turn + 3, x3, x2);
+        if (FULL) {
+#pragma unroll
+            for (int turn = 0; turn < kFmCi / 2 / SPLIT; turn += 4) {
+                products(turn, x0, x3);
+                products(turn + 1, x1, x0);
+                products(turn + 2, x2, x1);
+                products(turn + 3, x3, x2);
+            }
+        } else {
+            for (int turn = 0; turn < kFmCi / 2 / SPLIT && first + turn * SPLIT < all_pairs; turn += 4) {
+                products(turn, x0, x3);
+                if (first + (turn + 1) * SPLIT < all_pairs) products(turn + 1, x1, x0);
+                if (first + (turn + 2) * SPLIT < all_pairs) products(turn + 2, x2, x1);
+                if (first + (turn + 3) * SPLIT < all_pairs) products(turn + 3, x3, x2);
+            }
         }
         // the single last channel of an odd count: one wavefront per position half takes it with its lanes of the
         // pair's second channel reading the first and counting as zero (the weights past the last channel are zero too)
@@ -293,7 +323,10 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
                 acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * kFmRow + j], v, acc[1], 0, 0, 0);
             }
         }
-    }
+    };
+    int ci0_run = 0;
+    for (; ci0_run + kFmCi <= 2 * all_pairs; ci0_run += kFmCi) stage(ci0_run, std::true_type{});
+    if (ci0_run < c.ic) stage(ci0_run, std::false_type{});   // a short last stage (at most one: it holds fewer than 32 channels)
     __syncthreads();                                       // the weights are no longer needed: their LDS holds the partial sums
     if (kg > 0) {
         float* red = wl + (((kg - 1) * 2 + wn) * 32) * 64 + lane;  // [kg - 1][wn][t * 16 + e][lane]

@@ -29,7 +29,7 @@ static int g_forward_mfma = -1;
 void boat_hip_conv_forward_matrix_cores(int enable) { g_forward_mfma = enable != 0; }
 /* The matrix-core kernel works on tiles of 64 output channels and pairs of input channels, and a workgroup of it costs
  * a weight staging and a reduction whatever the layer: measured against the direct kernel over batch 16-256, images
- * 14x14 and 28x28, it wins (1.3x to 3.6x) from 32 output channels on with at least 8 input channels (a tie at 8 -> 32)
+ * 14x14 and 28x28, it wins (1.3x to 4x) from 32 output channels on with at least 8 input channels (a tie at 8 -> 32)
  * and from 16 output channels on with at least 32 input channels; narrower layers lose up to 2x. */
 static int conv_forward_wants_mfma(size_t in_channels, size_t out_channels) {
     return (in_channels >= 8 && out_channels >= 32) || (in_channels >= 32 && out_channels >= 16);

@@ -811,6 +811,34 @@ def test_device_to_device_copy(hip, rng, n, offset):
     assert np.array_equal(d_dst.numpy().view(np.uint8)[1:7], src.view(np.uint8)[1:7])
 
 
+def test_gemm_with_very_wide_leading_dimensions(hip):
+    """The MFMA tiles address an operand tile with 32-bit byte offsets from the tile's first row when they stream it
+    straight to LDS; a leading dimension of 2^22 or more does not fit that and takes the register-staged loader.  Both
+    sides of the limit, operands that are windows of much wider rows, against float64."""
+    rng = np.random.default_rng(77)
+    for ld, (ta, tb, m, n, k) in (((1 << 22) - 4, (0, 1, 8, 8, 64)), (1 << 22, (0, 1, 8, 8, 64)), ((1 << 22) + 8, (0, 0, 4, 128, 32)),
+                                  (1 << 22, (1, 0, 128, 64, 4))):
+        ra = k if ta else m
+        rb = n if tb else k
+        ca, cb = (m if ta else k), (k if tb else n)
+        lda = ld if ra * ld * 4 <= (1 << 28) else ca
+        ldb = ld if lda == ca else cb                      # one wide operand per case keeps the buffers small
+        a = rng.standard_normal((ra, lda)).astype(np.float32)
+        b = rng.standard_normal((rb, ldb)).astype(np.float32)
+        A = a[:, :ca].T if ta else a[:, :ca]
+        B = b[:, :cb].T if tb else b[:, :cb]
+        want = A.astype(np.float64) @ B.astype(np.float64)
+        dc = hip.zeros((m, n))
+        for cfg in (-1, 1, 4):                             # the heuristic, and the MFMA tiles pinned
+            hip.bh_gemm_force_config(cfg)
+            try:
+                hip.check(hip.bh_gemm(ta, tb, m, n, k, dev(hip, a).ptr, lda, dev(hip, b).ptr, ldb, dc.ptr, n, None, 0, 1))
+            finally:
+                hip.bh_gemm_force_config(-1)
+            assert rel_fro(dc.numpy(), want) <= TOL_GEMM, (ld, ta, tb, m, n, k, cfg)
+        _KEEP.clear()
+
+
 def test_gemm_random_sweep_with_padded_leading_dimensions(hip):
     """Seeded sweep over shapes, layouts, epilogues and leading dimensions wider than the rows (every kernel behind
     bh_gemm must honour lda / ldb / ldc), against float64."""

@@ -1197,7 +1197,14 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         // eight-wavefront 128x256 / 256x128 tiles (same operand reuse per wavefront, twice the workgroups) beat both
         // it and the 128x128 tile; narrow outputs keep the small tile
         const int64_t big_tiles = ceil_div(m, 256) * ceil_div(n, 256);
-        if (big_tiles >= 256) cfg = 2;
+        // (a tile shape pays for the rows and columns it pads: 288 rows are two 256-row tiles, 56 % full, but three
+        // 128-row ones, 75 % full -- 288x50176x64, the input gradient's product of a 32-channel 3x3 convolution, takes
+        // 68 us on 256x256 tiles and 53 us on 128x256 ones; the big tile keeps a problem it fills to within 15 % of the others)
+        const auto filled = [&](int64_t bm_, int64_t bn_) {
+            return (double)(m * n) / (double)(ceil_div(m, bm_) * bm_ * ceil_div(n, bn_) * bn_);
+        };
+        const double fill_big = filled(256, 256), fill_other = filled(128, 256) > filled(128, 128) ? filled(128, 256) : filled(128, 128);
+        if (big_tiles >= 256 && fill_big >= 0.85 * fill_other) cfg = 2;
         else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096 && (256 / big_tiles) * 2048 <= k) {
             // a mid-sized output under a long contraction (the weight gradient of a wide layer): 256x256 tiles with the
             // contraction cut so that the tiles fill the chip once, at least 2048 k each (4096x1024x8192: 512 us with
@@ -1218,6 +1225,9 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     }
     // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
     if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
+    // so is a contraction of at most 64 under an output of a few million elements, where the tiles above spend their
+    // time filling and draining their pipeline (288x12544x64: 15.7 against 20.0 us; 4096x4096x64 is past it: 56 against 37)
+    if (k > 0 && k <= 64 && m * n <= ((int64_t)1 << 22)) cfg = 5;
     // A few million multiply-adds in at most a few hundred 32x32 tiles: the kernels without workgroup-wide staging.
     // Measured against the staged small-problem kernel plus its fold (11-14 us beyond k = 128): two row-fast operands
     // 6-10 us up to k = 1024; one k-fast operand 7.5-8 us up to k = 512 (one trip) and 12 us up to 1024 (two trips);

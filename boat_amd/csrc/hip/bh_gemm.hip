@@ -1205,7 +1205,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         };
         const double fill_big = filled(256, 256), fill_other = filled(128, 256) > filled(128, 128) ? filled(128, 256) : filled(128, 128);
         if (big_tiles >= 256 && fill_big >= 0.85 * fill_other) cfg = 2;
-        else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096 && (256 / big_tiles) * 2048 <= k) {
+        else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096 && big_tiles < 256 && (256 / big_tiles) * 2048 <= k) {
             // a mid-sized output under a long contraction (the weight gradient of a wide layer): 256x256 tiles with the
             // contraction cut so that the tiles fill the chip once, at least 2048 k each (4096x1024x8192: 512 us with
             // the fold against 530 for two-way split 128x256 tiles)

@@ -323,6 +323,21 @@ def main():
               "dw": w.grad.numpy(), "eps": np.float64(eps)}
         save(f"rmsnorm_bwd_ref64_{tag}", **rm)
 
+    # One batch element of benchmark configuration 5's block at its real sizes (d_model 1024, 16 heads, seq 512, FFN 4096)
+    # in float64 autograd: sampled rows of y and dx, sampled entries of every parameter gradient, the loss.  The inputs
+    # are regenerated from the seed by tests/test_block.py::make_block, the sample positions by block_ref64_sample().
+    if not ONLY or "block_config5_ref64" in ONLY:
+        from test_block import BLOCK_REF64, block_ref64_sample, make_block, torch_block_grads
+        c = BLOCK_REF64
+        x, target, params = make_block(c["seed"], 1, c["S"], c["H"], c["ffn"])
+        want = torch_block_grads(x, target, params, c["heads"])
+        rows, picks = block_ref64_sample(params)
+        blk = {"loss": np.float64(want["loss"]), "y_rows": want["y"][0][rows].astype(np.float32),
+               "dx_rows": want["dx"][0][rows].astype(np.float32)}
+        for name in bc.BLOCK_PARAM_ORDER:
+            blk["g_" + name] = want["g_" + name].reshape(-1)[picks[name]].astype(np.float32)
+        save("block_config5_ref64", **blk)
+
 
 if __name__ == "__main__":
     main()

@@ -154,3 +154,45 @@ def test_block_training_steps(boat, oracle, B, S, H, heads, ffn):
                 gref = w["g_" + k]
                 resolved = np.abs(gref) > 1e-3 * np.abs(gref).max()
                 assert np.max(np.abs(got[0]["p_" + k] - want[0]["p_" + k])[resolved]) <= 2e-5, k
+
+
+# One batch element of benchmark configuration 5's block at its real sizes, pinned by float64 autograd
+# (tests/golden/make_golden.py writes tests/golden/block_config5_ref64.npz from torch_block_grads above).
+BLOCK_REF64 = {"seed": 11, "S": 512, "H": 1024, "ffn": 4096, "heads": 16}
+
+
+def block_ref64_sample(params, n_rows=12, n_picks=512):
+    """Rows of y / dx and flat positions inside every parameter gradient that the fixture holds (seeded)."""
+    rng = np.random.default_rng(20251125)
+    rows = np.sort(rng.choice(BLOCK_REF64["S"], n_rows, replace=False))
+    picks = {}
+    for name in bc.BLOCK_PARAM_ORDER:
+        size = params[name].size
+        picks[name] = np.sort(rng.choice(size, min(n_picks, size), replace=False))
+    return rows, picks
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("score_cache", [True, False])
+def test_config5_block_one_element_against_float64(boat, score_cache):
+    """d_model 1024, 16 heads, seq 512, FFN 4096, batch 1: the shapes that pick the split-K weight-gradient GEMMs, the
+    head_dim-64 matrix-core attention kernels (with and without the score cache) and the grouped self-attention
+    projections, against float64 autograd on sampled rows and entries.  The batch-independence test of
+    test_full_size.py carries this to batch 16."""
+    from pathlib import Path
+    c = BLOCK_REF64
+    with np.load(Path(__file__).resolve().parent / "golden" / "block_config5_ref64.npz", allow_pickle=False) as z:
+        want = {k: z[k] for k in z.files}
+    x, target, params = make_block(c["seed"], 1, c["S"], c["H"], c["ffn"])
+    rows, picks = block_ref64_sample(params)
+    boat.boat_hip_set_attention_score_cache_limit((1 << 30) if score_cache else 0)
+    try:
+        got = bc.transformer_block_steps(boat, x, target, params, c["heads"], steps=1)[0]
+    finally:
+        boat.boat_hip_set_attention_score_cache_limit(1 << 30)
+    assert abs(got["loss"] - float(want["loss"])) <= TOL_RED * abs(float(want["loss"]))
+    assert rel_fro(got["y"][0][rows], want["y_rows"]) <= TOL_GEMM
+    assert rel_fro(got["dx"][0][rows], want["dx_rows"]) <= TOL_GEMM
+    for name in bc.BLOCK_PARAM_ORDER:
+        tol = TOL_RED if name.startswith("ln") else TOL_GEMM
+        assert rel_fro(got["g_" + name].reshape(-1)[picks[name]], want["g_" + name]) <= tol, name

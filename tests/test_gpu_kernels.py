@@ -574,12 +574,13 @@ def test_sdpa_more_head_blocks_than_a_grid_dimension_holds(hip, oracle, rng):
 
 
 @pytest.mark.parametrize("causal", [0, 1])
-@pytest.mark.parametrize("bh,s", [(3, 128), (2, 384), (1, 1024), (520, 256)])
+@pytest.mark.parametrize("bh,s", [(3, 128), (2, 384), (1, 1024), (520, 256), (128, 1024)])
 def test_sdpa_with_score_cache(hip, oracle, rng, bh, s, causal):
     """bh_sdpa_forward_cached leaves the scaled scores, bh_sdpa_backward_cached reads them instead of recomputing Q.K^T:
     same outputs as the plain pair to fp32 rounding, against the oracle's attention backward
     (src/layers/attention.c:1417-1520) at the bound only fp32 accumulation meets; (520, 256) also takes the mirrored
-    second launch.  Shapes without the path are refused."""
+    second launch, (128, 1024) is benchmark configuration 4 (a 537 MB cache, sampled heads against the oracle).  Shapes
+    without the path are refused."""
     d = 64
     q, k, v, go = (rng.standard_normal((bh, s, d), dtype=np.float32) for _ in range(4))
     dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)

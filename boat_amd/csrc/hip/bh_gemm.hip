@@ -69,6 +69,22 @@ struct GemmArgs {
     int tiles_m, tiles_n;
 };
 
+// Operand tables of a grouped launch (up to kMaxGroups problems of one shape).  Two forms:
+//   k_segments == 1: blockIdx.y picks the group: c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g])
+//   k_segments  > 1: ONE product whose contraction runs over the operand pairs in turn,
+//                    c[0] (+)= sum_s op(a[s]) . op(b[s]) (+ bias[0]), seg_k of the contraction per pair
+// (the three input projections of self-attention: one launch for the forward products, one for the three weight
+// gradients, one contraction for the summed input gradient dQ.Wq^T + dK.Wk^T + dV.Wv^T)
+constexpr int kMaxGroups = 3;
+struct GemmTab {
+    const float* a[kMaxGroups];
+    const float* b[kMaxGroups];
+    float* c[kMaxGroups];
+    const float* bias[kMaxGroups];
+    int k_segments;
+    int64_t seg_k;       // multiple of 2 * kBK
+};
+
 // Global -> registers for one operand tile.  KC: tile is [R rows][kBK], row r at base + r*ld.
 // !KC: tile is [kBK k-rows][R], k-row kk at base + kk*ld.
 template <bool KC, int R, int NT>
@@ -200,6 +216,8 @@ struct DirectLoader {
             dst[j] = __builtin_amdgcn_readfirstlane(addr);
         }
     }
+    // continue at the start (k = 0) of another matrix of the same shape: the lane offsets stay what they are
+    __device__ __forceinline__ void rebase(const float* mat, int64_t ld, int64_t row0) { base = KC ? mat + row0 * ld : mat; }
     // issue this wavefront's blocks of the next k-tile into the stage at byte offset stage_bytes
     __device__ __forceinline__ void issue(unsigned stage_bytes) {
 #pragma unroll
@@ -233,8 +251,9 @@ struct DirectFrags {
     }
 };
 
-template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1>   // KT: k-tiles per LDS stage (and per barrier)
-__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
+template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1, bool TAB = false>   // KT: k-tiles per LDS stage (and per barrier); TAB: operands from tables
+__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g, GemmTab t) {
+    static_assert(!TAB || DIRECT, "grouped launches use the direct-to-LDS loaders");
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int A_FLOATS = DIRECT ? DirectTile<A_KC, BM>::floats : TileShape<A_KC, BM>::floats;
     constexpr int B_FLOATS = DIRECT ? DirectTile<B_KC, BN>::floats : TileShape<B_KC, BN>::floats;
@@ -259,9 +278,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     int64_t k_end = g.k_splits > 1 ? k_begin + g.k_per_split : g.k;
     if (k_end > g.k) k_end = g.k;
 
-    const float* A = g.a + (int64_t)batch * g.stride_a;
-    const float* B = g.b + (int64_t)batch * g.stride_b;
+    const float* A = TAB ? t.a[batch] : g.a + (int64_t)batch * g.stride_a;
+    const float* B = TAB ? t.b[batch] : g.b + (int64_t)batch * g.stride_b;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    // a segmented contraction: the operand pairs that follow the first, picked by scalar selects when the issue stream
+    // crosses into the next segment (blockIdx.y is 0 then)
+    const float* A1 = TAB ? t.a[1] : nullptr;
+    const float* A2 = TAB ? t.a[2] : nullptr;
+    const float* B1 = TAB ? t.b[1] : nullptr;
+    const float* B2 = TAB ? t.b[2] : nullptr;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -300,11 +325,20 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.v[s][i], fb.v[s][j], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         };
+        int seg = 0, seg_left = TAB && t.k_segments > 1 ? (int)(t.seg_k / (2 * kBK)) : 0x7fffffff;   // pairs to issue before the next segment
         auto issue_pair = [&](unsigned stage) {     // the next two k-tiles of this wavefront's blocks into stage `stage`
             da.issue(stage * 2 * TILE_BYTES);
             db.issue(stage * 2 * TILE_BYTES);
             da.issue(stage * 2 * TILE_BYTES + TILE_BYTES);
             db.issue(stage * 2 * TILE_BYTES + TILE_BYTES);
+            if constexpr (TAB) {
+                if (--seg_left == 0) {
+                    seg++;
+                    seg_left = (int)(t.seg_k / (2 * kBK));
+                    da.rebase(seg == 1 ? A1 : A2, g.lda, m0);
+                    db.rebase(seg == 1 ? B1 : B2, g.ldb, n0);
+                }
+            }
         };
         if (pairs > 0) issue_pair(0);
         if (pairs > 1) issue_pair(1);
@@ -368,14 +402,21 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
         // half's products run, so no product ever waits for an LDS read it has just issued.
         DirectFrags<A_KC, BM, TM> fa0, fa1;
         DirectFrags<B_KC, BN, TN> fb0, fb1;
-        if (kt_count > 0) {
-            da.issue(0);
-            db.issue(0);
-        }
-        if (kt_count > 1) {
-            da.issue((unsigned)(STAGE * sizeof(float)));
-            db.issue((unsigned)(STAGE * sizeof(float)));
-        }
+        int seg = 0, seg_left = TAB && t.k_segments > 1 ? (int)(t.seg_k / kBK) : 0x7fffffff;   // k-tiles to issue before the next segment
+        const auto issue_tile = [&](unsigned stage_bytes) {
+            da.issue(stage_bytes);
+            db.issue(stage_bytes);
+            if constexpr (TAB) {
+                if (--seg_left == 0) {
+                    seg++;
+                    seg_left = (int)(t.seg_k / kBK);
+                    da.rebase(seg == 1 ? A1 : A2, g.lda, m0);
+                    db.rebase(seg == 1 ? B1 : B2, g.ldb, n0);
+                }
+            }
+        };
+        if (kt_count > 0) issue_tile(0);
+        if (kt_count > 1) issue_tile((unsigned)(STAGE * sizeof(float)));
         wait_direct_loads();
         __syncthreads();
         if (kt_count > 0) {
@@ -403,8 +444,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
             __syncthreads();           // ... is visible to everyone, and everyone has its fragments of stage cur in registers
             if (kt + 2 < kt_count) {
                 constexpr unsigned stage_bytes = (unsigned)(cur * STAGE * sizeof(float));
-                da.issue(stage_bytes);
-                db.issue(stage_bytes);
+                issue_tile(stage_bytes);
             }
             if (kt + 1 < kt_count) {
                 const float* na = smem + (cur ^ 1) * STAGE;
@@ -475,10 +515,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g) {
     }
 
     // ---- epilogue ----
-    float* C = g.c + (int64_t)batch * g.stride_c;
+    // (a split launch writes partials to the workspace in g.c, [split][group][m][n], tables or not)
+    float* C = TAB && g.k_splits <= 1 ? t.c[batch] : g.c + (int64_t)batch * g.stride_c;
     if (g.k_splits > 1) C += (int64_t)split * gridDim.y * g.stride_c;
     const bool add_c = g.accumulate && g.k_splits <= 1;
-    const float* bias = g.k_splits <= 1 ? g.bias : nullptr;
+    const float* bias = g.k_splits <= 1 ? (TAB ? t.bias[batch] : g.bias) : nullptr;
     // a lane's TN columns are the same for every row it stores: their bias values are fetched once, not once per element
     float bias_v[TN];
 #pragma unroll
@@ -620,6 +661,34 @@ __global__ __launch_bounds__(64) void splitk_fold_vec_kernel(const float* __rest
         acc += *reinterpret_cast<const fold_f32x4*>(bias + col);
     }
     fold_f32x4* dst = reinterpret_cast<fold_f32x4*>(c) + i;
+    if (accumulate) acc = __builtin_nontemporal_load(dst) + acc;
+    __builtin_nontemporal_store(acc, dst);
+}
+
+// the same for a grouped launch: blockIdx.y picks the group, whose partials sit at [split][group][m*n] in the workspace
+__global__ __launch_bounds__(64) void splitk_fold_vec_tab_kernel(const float* __restrict__ ws, GemmTab t, int64_t per4, int64_t n,
+                                                                 int splits, int accumulate) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= per4) return;
+    const int grp = blockIdx.y;
+    const int64_t split_stride = per4 * gridDim.y;
+    const fold_f32x4* w4 = reinterpret_cast<const fold_f32x4*>(ws) + grp * per4 + i;
+    fold_f32x4 acc = __builtin_nontemporal_load(w4);
+    int sp = 1;
+    for (; sp + 3 < splits; sp += 4) {
+        const fold_f32x4 a = __builtin_nontemporal_load(w4 + (int64_t)sp * split_stride);
+        const fold_f32x4 b = __builtin_nontemporal_load(w4 + (int64_t)(sp + 1) * split_stride);
+        const fold_f32x4 d = __builtin_nontemporal_load(w4 + (int64_t)(sp + 2) * split_stride);
+        const fold_f32x4 e = __builtin_nontemporal_load(w4 + (int64_t)(sp + 3) * split_stride);
+        acc += a;
+        acc += b;
+        acc += d;
+        acc += e;
+    }
+    for (; sp < splits; sp++) acc += __builtin_nontemporal_load(w4 + (int64_t)sp * split_stride);
+    const float* bias = t.bias[grp];
+    if (bias) acc += *reinterpret_cast<const fold_f32x4*>(bias + (i * 4) % n);
+    fold_f32x4* dst = reinterpret_cast<fold_f32x4*>(t.c[grp]) + i;
     if (accumulate) acc = __builtin_nontemporal_load(dst) + acc;
     __builtin_nontemporal_store(acc, dst);
 }
@@ -1051,21 +1120,22 @@ __global__ __launch_bounds__(256) void swap_dims_kernel(const T* __restrict__ in
     }
 }
 
-template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1>
-static int launch_mfma(const GemmArgs& g, int64_t batch) {
+template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1, bool TAB = false>
+static int launch_mfma(const GemmArgs& g, int64_t batch, const GemmTab* tab = nullptr) {
     constexpr size_t lds = KT * 2 * sizeof(float) *
         (DIRECT ? DirectTile<A_KC, Cfg::BM>::floats + DirectTile<B_KC, Cfg::BN>::floats
                 : TileShape<A_KC, Cfg::BM>::floats + TileShape<B_KC, Cfg::BN>::floats);
     static bool attr_set = false;
     if (!attr_set) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT, KT>),
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT, KT, TAB>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                            "hipFuncSetAttribute");
         if (rc) return rc;
         attr_set = true;
     }
     dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch, (unsigned)(g.k_splits > 1 ? g.k_splits : 1));
-    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT, KT>), grid, dim3(Cfg::NT), lds, stream(), g);
+    GemmTab none = {};
+    hipLaunchKernelGGL((gemm_mfma_kernel<Cfg, A_KC, B_KC, DIRECT, KT, TAB>), grid, dim3(Cfg::NT), lds, stream(), g, tab ? *tab : none);
     return BH_LAUNCH_CHECK("gemm_mfma_kernel");
 }
 
@@ -1084,6 +1154,15 @@ static int launch_mfma_pairs(const GemmArgs& g, int64_t batch, bool a_kc, bool b
     if (a_kc && !b_kc) return launch_mfma<Cfg, true, false, true, 2>(g, batch);
     if (!a_kc && b_kc) return launch_mfma<Cfg, false, true, true, 2>(g, batch);
     return launch_mfma<Cfg, false, false, true, 2>(g, batch);
+}
+
+// the same tiles with their operands taken from tables (grouped launches); KT as the tile would have it ungrouped
+template <typename Cfg, int KT>
+static int launch_mfma_tab(const GemmArgs& g, int64_t batch, bool a_kc, bool b_kc, const GemmTab* tab) {
+    if (a_kc && b_kc) return launch_mfma<Cfg, true, true, true, KT, true>(g, batch, tab);
+    if (a_kc && !b_kc) return launch_mfma<Cfg, true, false, true, KT, true>(g, batch, tab);
+    if (!a_kc && b_kc) return launch_mfma<Cfg, false, true, true, KT, true>(g, batch, tab);
+    return launch_mfma<Cfg, false, false, true, KT, true>(g, batch, tab);
 }
 
 template <typename Cfg>
@@ -1134,6 +1213,7 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
 static int g_force_splits = 0;    // test hook: > 0 = this many k-splits for the MFMA tiles
 static int g_pairs = 1;           // test hook: 0 = every tile keeps one k-tile per barrier
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
+static int g_no_tables = 0;       // test hook: 1 = grouped launches fall back to one launch per group
 static int g_force_cfg = -1;   // test hook: 0 = fallback, 1..4 = MFMA tile shapes, 5 = small-problem kernel, 6 = tiny, -1 = heuristic
 
 }  // namespace bh
@@ -1161,15 +1241,13 @@ int bh_gemm_force_direct(int mode) {
     return BH_OK;
 }
 
-int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const float* a, int64_t lda, const float* b,
-            int64_t ldb, float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch) {
-    BH_REQUIRE_INIT();
-    BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && batch >= 0, "negative dimension");
-    if (m == 0 || n == 0 || batch == 0) return BH_OK;
-    BH_CHECK_ARG(a && b && c, "null pointer");
-    BH_CHECK_ARG(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "leading dimension too small");
-    BH_CHECK_ARG(batch <= 65535, "batch too large");
-    ProfScope prof(BH_PROF_GEMM, 2.0 * (double)m * (double)n * (double)k * (double)batch);
+}  // extern "C"
+
+// `tab` != NULL: a grouped launch (operands from the tables, a/b/c/bias unused; k is the whole contraction of a segmented
+// product).  Returns kTabUnsupported, having launched nothing, when the shape does not take one of the table kernels.
+constexpr int kTabUnsupported = -1000;
+static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const float* a, int64_t lda, const float* b,
+                     int64_t ldb, float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch, const GemmTab* tab) {
 
     GemmArgs g;
     g.a = a; g.b = b; g.c = c; g.bias = bias;
@@ -1184,6 +1262,15 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
 
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (tab) {
+        const int count = tab->k_segments > 1 ? tab->k_segments : (int)batch;
+        a = tab->a[0];
+        b = tab->b[0];
+        for (int i = 1; i < count; i++)
+            if (!al16(tab->a[i]) || !al16(tab->b[i])) return kTabUnsupported;
+        for (int i = 0; i < (tab->k_segments > 1 ? 1 : count); i++)
+            if (!al16(tab->c[i]) || !al16(tab->bias[i])) return kTabUnsupported;
+    }
     // float4 global loads need: 16 B aligned bases, leading dimensions and the contiguous extent % 4
     bool vec_ok = al16(a) && al16(b) && (lda % 4 == 0) && (ldb % 4 == 0) && k > 0;
     vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
@@ -1205,18 +1292,26 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         };
         const double fill_big = filled(256, 256), fill_other = filled(128, 256) > filled(128, 128) ? filled(128, 256) : filled(128, 128);
         if (big_tiles >= 256 && fill_big >= 0.85 * fill_other) cfg = 2;
-        else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096 && big_tiles < 256 && (256 / big_tiles) * 2048 <= k) {
+        else if ((batch == 1 || tab) && m >= 512 && n >= 512 && k >= 4096 && big_tiles * batch < 256 && (256 / (big_tiles * batch)) * 2048 <= k) {
             // a mid-sized output under a long contraction (the weight gradient of a wide layer): 256x256 tiles with the
             // contraction cut so that the tiles fill the chip once, at least 2048 k each (4096x1024x8192: 512 us with
             // the fold against 530 for two-way split 128x256 tiles)
             cfg = 2;
-            plan_splits = (int)(256 / big_tiles);
-        } else if (batch == 1 && m >= 512 && n >= 512 && k >= 4096) {
+            plan_splits = (int)(256 / (big_tiles * batch));
+        } else if ((batch == 1 || tab) && m >= 512 && n >= 512 && k >= 4096 && !(tab && tab->k_segments > 1)) {
             // smaller still (1024x1024x8192): 128x128 tiles, two workgroups per compute unit, 1024 k each where that
             // fills the chip (145 us with the fold against 155 for sixteen-way split 128x256 tiles)
             cfg = 1;
-            const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128);
+            const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
             plan_splits = (int)ceil_div(512, t128);
+            // two of these workgroups share a compute unit, so what counts is an even load per compute unit: the first
+            // count from there on that is a multiple of 256 workgroups (three grouped 1024x1024x8192 products: 4 splits,
+            // 768 workgroups, 388 us with the fold against 402-500 for 3, 5, 6 or 8)
+            for (int s2 = plan_splits; s2 <= 2 * plan_splits && k / s2 >= 1024; s2++)
+                if ((t128 * s2) % 256 == 0) {
+                    plan_splits = s2;
+                    break;
+                }
             while (plan_splits > 1 && k / plan_splits < 1024) plan_splits--;
         }
         else if (n >= 192 && m >= 96) cfg = 4;
@@ -1246,6 +1341,7 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     if (g_force_cfg >= 0 && g_force_cfg <= 6 && (vec_ok || g_force_cfg == 0 || g_force_cfg >= 5)) cfg = g_force_cfg;
     if (cfg == 6 && k == 0) cfg = 5;
     if (cfg != 6) tiny_split = false;
+    if (tab && (cfg == 0 || cfg >= 5)) return kTabUnsupported;
 
     if (cfg == 6) {
         g.tiles_m = (int)ceil_div(m, 32);
@@ -1360,7 +1456,8 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     float* ws = nullptr;
     // (a handful of tiles with a contraction of a few hundred is latency bound per k-tile: split it finer)
     const bool few_tiles = tiles <= 8 && k >= 256;
-    if ((tiles < 256 && k >= 1024) || few_tiles) {
+    const bool segmented = tab && tab->k_segments > 1;     // one product over several operand pairs: never split
+    if (((tiles < 256 && k >= 1024) || few_tiles) && !segmented) {
         const int64_t min_k = few_tiles && k < 2048 ? 128 : 256;
         int64_t splits = ceil_div(512, tiles);
         if (splits > k / min_k) splits = k / min_k;
@@ -1374,6 +1471,20 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
             g.k_splits = (int)ceil_div(k, g.k_per_split);
         }
     }
+    // the direct-to-LDS loader cannot zero-fill a k tail, and its edge clamps need 4 valid floats in a row
+    // (and it addresses a tile with 32-bit byte offsets from the tile's first row: leading dimensions below 2^22)
+    const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4) &&
+                        lda < ((int64_t)1 << 22) && ldb < ((int64_t)1 << 22);
+    // the eight-wavefront tiles take two k-tiles per barrier whenever every workgroup's contraction range is whole pairs
+    // (measured at the block's shapes with the staggered loads: 1.5-3 % faster than one tile per barrier on all three)
+    const bool pairs = direct && g_pairs && k % (2 * kBK) == 0 && (g.k_splits == 1 || g.k_per_split % (2 * kBK) == 0);
+    if (tab) {
+        // table kernels exist for the direct loaders only: paired k-tiles on the eight-wavefront tiles, single ones on 128x128;
+        // a split launch folds with 16-byte pieces into dense outputs
+        if (!direct || (cfg != 1 && !pairs)) return kTabUnsupported;
+        if (g.k_splits > 1 && (ldc != n || n % 4 != 0 || ceil_div(m * n / 4, 64) > 0x7fffffff)) return kTabUnsupported;
+        if (segmented && tab->seg_k % (2 * kBK) != 0) return kTabUnsupported;
+    }
     GemmArgs run = g;
     if (g.k_splits > 1) {
         ws = (float*)bh_malloc(sizeof(float) * (size_t)(g.k_splits * batch * m * n));
@@ -1382,14 +1493,23 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
         run.ldc = n;
         run.stride_c = m * n;
     }
-    // the direct-to-LDS loader cannot zero-fill a k tail, and its edge clamps need 4 valid floats in a row
-    // (and it addresses a tile with 32-bit byte offsets from the tile's first row: leading dimensions below 2^22)
-    const bool direct = g_force_direct != 0 && k % kBK == 0 && k >= kBK && (a_kc || m >= 4) && (b_kc || n >= 4) &&
-                        lda < ((int64_t)1 << 22) && ldb < ((int64_t)1 << 22);
     int rc;
-    // the eight-wavefront tiles take two k-tiles per barrier whenever every workgroup's contraction range is whole pairs
-    // (measured at the block's shapes with the staggered loads: 1.5-3 % faster than one tile per barrier on all three)
-    const bool pairs = direct && g_pairs && k % (2 * kBK) == 0 && (g.k_splits == 1 || g.k_per_split % (2 * kBK) == 0);
+    if (tab) {
+        switch (cfg) {
+            case 2: rc = launch_mfma_tab<CfgBig, 2>(run, batch, a_kc, b_kc, tab); break;
+            case 3: rc = launch_mfma_tab<CfgTall, 2>(run, batch, a_kc, b_kc, tab); break;
+            case 4: rc = launch_mfma_tab<CfgWide, 2>(run, batch, a_kc, b_kc, tab); break;
+            default: rc = launch_mfma_tab<CfgMid, 1>(run, batch, a_kc, b_kc, tab); break;
+        }
+        if (rc == BH_OK && g.k_splits > 1) {
+            const int64_t per4 = m * n / 4;
+            hipLaunchKernelGGL(splitk_fold_vec_tab_kernel, dim3((unsigned)ceil_div(per4, 64), (unsigned)batch), dim3(64), 0, stream(),
+                               ws, *tab, per4, n, g.k_splits, accumulate);
+            rc = BH_LAUNCH_CHECK("splitk_fold_vec_tab_kernel");
+        }
+        if (ws) bh_free(ws);
+        return rc;
+    }
     switch (cfg) {
         case 2: rc = pairs ? launch_mfma_pairs<CfgBig>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct); break;
         case 3: rc = pairs ? launch_mfma_pairs<CfgTall>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc, direct); break;
@@ -1399,6 +1519,88 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
     if (rc == BH_OK && g.k_splits > 1) rc = launch_fold(ws, c, bias, m, n, ldc, g.k_splits, batch, g.stride_c, accumulate);
     if (ws) bh_free(ws);
     return rc;
+}
+
+extern "C" {
+
+int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const float* a, int64_t lda, const float* b,
+            int64_t ldb, float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && batch >= 0, "negative dimension");
+    if (m == 0 || n == 0 || batch == 0) return BH_OK;
+    BH_CHECK_ARG(a && b && c, "null pointer");
+    BH_CHECK_ARG(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "leading dimension too small");
+    BH_CHECK_ARG(batch <= 65535, "batch too large");
+    ProfScope prof(BH_PROF_GEMM, 2.0 * (double)m * (double)n * (double)k * (double)batch);
+    return gemm_core(trans_a, trans_b, m, n, k, a, lda, b, ldb, c, ldc, bias, accumulate, batch, nullptr);
+}
+
+// c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g]) for `groups` problems of one shape: one launch where the shape takes the
+// matrix-core tiles with direct loads, the same kernels one after the other otherwise (the same arithmetic either way)
+int bh_gemm_grouped(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int groups, const float* const* a, int64_t lda,
+                    const float* const* b, int64_t ldb, float* const* c, int64_t ldc, const float* const* bias, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0, "negative dimension");
+    BH_CHECK_ARG(groups >= 1 && groups <= kMaxGroups, "1 to 3 groups");
+    BH_CHECK_ARG(a && b && c, "null table");
+    if (m == 0 || n == 0) return BH_OK;
+    for (int i = 0; i < groups; i++) BH_CHECK_ARG(a[i] && b[i] && c[i], "null pointer");
+    BH_CHECK_ARG(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "leading dimension too small");
+    ProfScope prof(BH_PROF_GEMM, 2.0 * (double)m * (double)n * (double)k * (double)groups);   // the launches below nest inside it
+    if (groups > 1 && !g_no_tables) {
+        GemmTab t = {};
+        for (int i = 0; i < groups; i++) {
+            t.a[i] = a[i]; t.b[i] = b[i]; t.c[i] = c[i];
+            t.bias[i] = bias ? bias[i] : nullptr;
+        }
+        t.k_segments = 1;
+        const int rc = gemm_core(trans_a, trans_b, m, n, k, nullptr, lda, nullptr, ldb, nullptr, ldc, nullptr, accumulate, groups, &t);
+        if (rc != kTabUnsupported) return rc;
+    }
+    for (int i = 0; i < groups; i++) {
+        const int rc = bh_gemm(trans_a, trans_b, m, n, k, a[i], lda, b[i], ldb, c[i], ldc, bias ? bias[i] : nullptr, accumulate, 1);
+        if (rc != BH_OK) return rc;
+    }
+    return BH_OK;
+}
+
+// c (+)= sum_s op(a[s]) . op(b[s]) (+ bias): one product whose contraction runs over `segments` operand pairs of k each.
+// One launch where the shape takes the matrix-core tiles with direct loads; otherwise the pairs one after the other,
+// each adding into c.  The two forms add the segments' products in different orders (one long chain against partial
+// sums), so they agree to fp32 rounding, not bit for bit; which form runs depends on the shape only.
+int bh_gemm_ksegments(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int segments, const float* const* a, int64_t lda,
+                      const float* const* b, int64_t ldb, float* c, int64_t ldc, const float* bias, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0, "negative dimension");
+    BH_CHECK_ARG(segments >= 1 && segments <= kMaxGroups, "1 to 3 segments");
+    BH_CHECK_ARG(a && b && c, "null pointer");
+    if (m == 0 || n == 0) return BH_OK;
+    for (int i = 0; i < segments; i++) BH_CHECK_ARG(a[i] && b[i], "null pointer");
+    BH_CHECK_ARG(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "leading dimension too small");
+    ProfScope prof(BH_PROF_GEMM, 2.0 * (double)m * (double)n * (double)k * (double)segments);
+    if (segments > 1 && k > 0 && !g_no_tables) {
+        GemmTab t = {};
+        for (int i = 0; i < segments; i++) {
+            t.a[i] = a[i]; t.b[i] = b[i];
+        }
+        t.c[0] = c;
+        t.bias[0] = bias;
+        t.k_segments = segments;
+        t.seg_k = k;
+        const int rc = gemm_core(trans_a, trans_b, m, n, k * segments, nullptr, lda, nullptr, ldb, nullptr, ldc, nullptr, accumulate, 1, &t);
+        if (rc != kTabUnsupported) return rc;
+    }
+    for (int i = 0; i < segments; i++) {
+        const int rc = bh_gemm(trans_a, trans_b, m, n, k, a[i], lda, b[i], ldb, c, ldc, i == 0 ? bias : nullptr, i == 0 ? accumulate : 1, 1);
+        if (rc != BH_OK) return rc;
+    }
+    return BH_OK;
+}
+
+// test/benchmark hook: 1 = grouped entry points always run their problems one after the other
+int bh_gemm_no_tables(int off) {
+    g_no_tables = off != 0;
+    return BH_OK;
 }
 
 int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, int64_t cols) {

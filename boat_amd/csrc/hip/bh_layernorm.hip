@@ -186,12 +186,14 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_generic_kernel(const float* _
 // RMS: backward of y = x*s*w with s = 1/(r+eps), r = sqrtf(mean(x^2)) (`rstd` holds s, `mean` is not read).  With
 // xhat = x*s and g = dy*w:  dx = s*(g - xhat*mean_h(g*xhat)/c), c = r*s = 1 - eps*s (a row of zeros has c = 0 and
 // xhat = 0: the second term is dropped); dweight = sum_rows dy*xhat.  The dbeta half of a partial is then unused.
-template <int TPR, int VPT, bool RMS>
-__global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
-                                                          const float* __restrict__ dy, const float* __restrict__ mean,
-                                                          const float* __restrict__ rstd, float* __restrict__ dx,
-                                                          float* __restrict__ partial, int64_t rows, int hidden,
-                                                          int64_t iters, float eps) {
+// ADD: dx = (the gradient above) + add, the residual branch's gradient that a pre-LN block would otherwise add in a
+// pass of its own; the row of `add` is fetched at the top of the row's iteration and lands under the row sums.
+template <int TPR, int VPT, bool RMS, bool ADD>
+__device__ __forceinline__ void ln_bwd_body(const float* __restrict__ x, const float* __restrict__ gamma,
+                                            const float* __restrict__ dy, const float* __restrict__ mean,
+                                            const float* __restrict__ rstd, const float* __restrict__ add,
+                                            float* __restrict__ dx, float* __restrict__ partial, int64_t rows, int hidden,
+                                            int64_t iters, float eps) {
     constexpr int GROUPS = kLnBlock / TPR;
     extern __shared__ float dyn_lds[];           // GROUPS>1: [GROUPS][2][hidden] for the cross-group fold
     __shared__ float lds[GROUPS * (TPR / 64) * 2 + 2];
@@ -223,8 +225,15 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
     // `iters` is the same for every group, so the barriers below are reached uniformly; rows past the
     // end are masked (they contribute zeros and store nothing).
     for (int64_t it = 0; it < iters; it++) {
-        float4 xh[VPT], g[VPT];
+        float4 xh[VPT], g[VPT], av[ADD ? VPT : 1];
         float s1 = 0.f, s2 = 0.f;
+        if constexpr (ADD) {
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                const int c4 = t + i * TPR;
+                av[i] = (live && c4 < h4) ? ld4_stream(add + row * hidden, c4) : make_float4(0, 0, 0, 0);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
             xh[i].x = (xv[i].x - mu) * rs; xh[i].y = (xv[i].y - mu) * rs; xh[i].z = (xv[i].z - mu) * rs; xh[i].w = (xv[i].w - mu) * rs;
@@ -267,6 +276,9 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
                     o.y = cur_rs * (g[i].y - s1 - xh[i].y * s2);
                     o.z = cur_rs * (g[i].z - s1 - xh[i].z * s2);
                     o.w = cur_rs * (g[i].w - s1 - xh[i].w * s2);
+                    if constexpr (ADD) {
+                        o.x += av[i].x; o.y += av[i].y; o.z += av[i].z; o.w += av[i].w;
+                    }
                     st4_stream(dx + cur_row * hidden, c4, o);
                 }
             }
@@ -303,10 +315,28 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restric
     }
 }
 
+template <int TPR, int VPT, bool RMS>
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                          const float* __restrict__ dy, const float* __restrict__ mean,
+                                                          const float* __restrict__ rstd, const float* __restrict__ add,
+                                                          float* __restrict__ dx, float* __restrict__ partial, int64_t rows,
+                                                          int hidden, int64_t iters, float eps) {
+    ln_bwd_body<TPR, VPT, RMS, false>(x, gamma, dy, mean, rstd, nullptr, dx, partial, rows, hidden, iters, eps);
+}
+template <int TPR, int VPT, bool RMS>
+__global__ __launch_bounds__(kLnBlock) void ln_bwd_add_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                              const float* __restrict__ dy, const float* __restrict__ mean,
+                                                              const float* __restrict__ rstd, const float* __restrict__ add,
+                                                              float* __restrict__ dx, float* __restrict__ partial, int64_t rows,
+                                                              int hidden, int64_t iters, float eps) {
+    ln_bwd_body<TPR, VPT, RMS, true>(x, gamma, dy, mean, rstd, add, dx, partial, rows, hidden, iters, eps);
+}
+
 // generic backward: one block per row, partial per row-chunk accumulated by columns
 __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_generic_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                                      const float* __restrict__ dy, const float* __restrict__ mean,
-                                                                     const float* __restrict__ rstd, float* __restrict__ dx,
+                                                                     const float* __restrict__ rstd, const float* __restrict__ add,
+                                                                     float* __restrict__ dx,
                                                                      int64_t rows, int64_t hidden, int rms, float eps) {
     __shared__ float red[kLnBlock / 64];
     const int64_t r = blockIdx.x;
@@ -328,7 +358,8 @@ __global__ __launch_bounds__(kLnBlock) void ln_bwd_dx_generic_kernel(const float
     for (int64_t c = threadIdx.x; c < hidden; c += kLnBlock) {
         float xh = (x[r * hidden + c] - mu) * rs;
         float g = dy[r * hidden + c] * (gamma ? gamma[c] : 1.0f);
-        dx[r * hidden + c] = rs * (g - s1 - xh * s2);
+        const float o = rs * (g - s1 - xh * s2);
+        dx[r * hidden + c] = add ? o + add[r * hidden + c] : o;
     }
 }
 __global__ __launch_bounds__(kLnBlock) void ln_bwd_param_generic_kernel(const float* __restrict__ x, const float* __restrict__ dy,
@@ -468,11 +499,16 @@ int bh_rmsnorm_forward(const float* x, const float* weight, float* y, float* inv
 // (blocks x 2 x hidden floats), fold_rows_kernel sums them.
 static int ln_backward_vector(bool rms, float eps, const LnPlan& plan, size_t shmem, int64_t blocks, float* partial,
                               const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
-                              float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
+                              const float* add, float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden,
+                              int accumulate) {
     const int groups = kLnBlock / plan.tpr;
     const int64_t iters = ceil_div(rows, blocks * groups);
-    BH_LN_DISPATCH(ln_bwd_kernel, rms, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, dx, partial, rows,
-                   (int)hidden, iters, eps);
+    if (add)
+        BH_LN_DISPATCH(ln_bwd_add_kernel, rms, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, add, dx, partial,
+                       rows, (int)hidden, iters, eps);
+    else
+        BH_LN_DISPATCH(ln_bwd_kernel, rms, plan, dim3((unsigned)blocks), shmem, x, gamma, dy, mean, rstd, add, dx, partial, rows,
+                       (int)hidden, iters, eps);
     if (dgamma || dbeta)
         hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(2 * hidden, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
                            stream(), partial, blocks, 2 * hidden, dgamma, dbeta, hidden, accumulate);
@@ -502,12 +538,13 @@ static bool ln_backward_plan(LnPlan& plan, size_t& shmem, const float* x, const 
 }
 
 static int norm_backward(bool rms, float eps, const float* x, const float* gamma, const float* dy, const float* mean,
-                         const float* rstd, float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden,
-                         int accumulate) {
-    ProfScope prof(BH_PROF_NORM, 12.0 * (double)rows * (double)hidden);
+                         const float* rstd, const float* add, float* dx, float* dgamma, float* dbeta, int64_t rows,
+                         int64_t hidden, int accumulate) {
+    ProfScope prof(BH_PROF_NORM, (add ? 16.0 : 12.0) * (double)rows * (double)hidden);
     LnPlan plan;
     size_t shmem;
     ln_backward_plan(plan, shmem, x, gamma, dy, dx, hidden);
+    if (plan.vector && add && (reinterpret_cast<uintptr_t>(add) & 15)) plan.vector = false;
 
     int rc;
     if (plan.vector) {
@@ -517,12 +554,12 @@ static int norm_backward(bool rms, float eps, const float* x, const float* gamma
         if (blocks > cap) blocks = cap;
         float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(blocks * 2 * hidden));
         if (!partial) return BH_ENOMEM;
-        rc = ln_backward_vector(rms, eps, plan, shmem, blocks, partial, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows,
+        rc = ln_backward_vector(rms, eps, plan, shmem, blocks, partial, x, gamma, dy, mean, rstd, add, dx, dgamma, dbeta, rows,
                                 hidden, accumulate);
         bh_free(partial);
     } else {
         hipLaunchKernelGGL(ln_bwd_dx_generic_kernel, dim3((unsigned)rows), dim3(kLnBlock), 0, stream(), x, gamma, dy, mean,
-                           rstd, dx, rows, hidden, rms ? 1 : 0, eps);
+                           rstd, add, dx, rows, hidden, rms ? 1 : 0, eps);
         rc = BH_LAUNCH_CHECK("norm backward dx");
         if (rc == BH_OK && (dgamma || dbeta)) {
             int64_t chunks = ceil_div(rows, 64);
@@ -555,7 +592,20 @@ int bh_layernorm_backward(const float* x, const float* gamma, const float* dy, c
         return BH_OK;
     }
     BH_CHECK_ARG(x && dy && mean && rstd && dx, "null pointer");
-    return norm_backward(false, 0.f, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden, accumulate);
+    return norm_backward(false, 0.f, x, gamma, dy, mean, rstd, nullptr, dx, dgamma, dbeta, rows, hidden, accumulate);
+}
+
+// dx = (LayerNorm input gradient) + add: the same kernel with the other gradient of a variable that feeds both a
+// LayerNorm and a residual connection added on the way out (add must not overlap dx)
+int bh_layernorm_backward_add(const float* x, const float* gamma, const float* dy, const float* mean, const float* rstd,
+                              const float* add, float* dx, float* dgamma, float* dbeta, int64_t rows, int64_t hidden, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && hidden > 0, "bad shape");
+    BH_CHECK_ARG(hidden < (int64_t(1) << 30), "hidden too large");
+    if (rows == 0) return bh_layernorm_backward(x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows, hidden, accumulate);
+    BH_CHECK_ARG(x && dy && mean && rstd && dx && add, "null pointer");
+    BH_CHECK_ARG(add + rows * hidden <= dx || dx + rows * hidden <= add, "add overlaps dx");
+    return norm_backward(false, 0.f, x, gamma, dy, mean, rstd, add, dx, dgamma, dbeta, rows, hidden, accumulate);
 }
 
 int bh_rmsnorm_backward(const float* x, const float* weight, const float* dy, const float* inv_rms, float* dx, float* dweight,
@@ -568,7 +618,7 @@ int bh_rmsnorm_backward(const float* x, const float* weight, const float* dy, co
         return BH_OK;
     }
     BH_CHECK_ARG(x && dy && inv_rms && dx, "null pointer");
-    return norm_backward(true, eps, x, weight, dy, nullptr, inv_rms, dx, dweight, nullptr, rows, hidden, accumulate);
+    return norm_backward(true, eps, x, weight, dy, nullptr, inv_rms, nullptr, dx, dweight, nullptr, rows, hidden, accumulate);
 }
 
 // bh_layernorm_backward for callers that may not allocate: same kernels, the partials live in ln_scratch.
@@ -605,7 +655,7 @@ int bh_layernorm_backward_noalloc(const float* x, const float* gamma, const floa
     if (cap > fit) cap = fit;
     if (blocks > cap) blocks = cap;
     // every partial the fold reads is written by this call's ln_bwd_kernel first: nothing to clear
-    return ln_backward_vector(false, 0.f, plan, shmem, blocks, scratch, x, gamma, dy, mean, rstd, dx, dgamma, dbeta, rows,
+    return ln_backward_vector(false, 0.f, plan, shmem, blocks, scratch, x, gamma, dy, mean, rstd, nullptr, dx, dgamma, dbeta, rows,
                               hidden, accumulate);
 }
 

@@ -173,6 +173,7 @@ int bh_sum_all(const float* x, float* out1, int64_t n) {
 }
 
 int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n);  // defined below
+int bh_mse_grad(const float* pred, const float* target, float* grad, int64_t n);
 
 int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumulate) {
     BH_REQUIRE_INIT();
@@ -268,6 +269,26 @@ __global__ __launch_bounds__(kRBlock) void sse_partial_kernel(const float* p, co
     float s = block_sum<kRBlock / 64>(acc, red);
     if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
+// the same sum with the gradient 2*(p - t)/n written on the way (one read of p and t for both): 16-byte pieces
+typedef float red_f32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(kRBlock) void sse_grad_partial_kernel(const float* __restrict__ p, const float* __restrict__ t,
+                                                                   float* __restrict__ grad, float* __restrict__ partial,
+                                                                   int64_t n4, float nf) {
+    __shared__ float red[kRBlock / 64];
+    float acc = 0.f;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const red_f32x4* p4 = reinterpret_cast<const red_f32x4*>(p);
+    const red_f32x4* t4 = reinterpret_cast<const red_f32x4*>(t);
+    red_f32x4* g4 = reinterpret_cast<red_f32x4*>(grad);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        const red_f32x4 d = __builtin_nontemporal_load(p4 + i) - __builtin_nontemporal_load(t4 + i);
+        acc += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+        const red_f32x4 g = {2.0f * d.x / nf, 2.0f * d.y / nf, 2.0f * d.z / nf, 2.0f * d.w / nf};   // as FMseGrad: 2*(p-t)/n
+        __builtin_nontemporal_store(g, g4 + i);
+    }
+    float s = block_sum<kRBlock / 64>(acc, red);
+    if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
 // per-element loss terms of the reference's loss objects, summed: kind 0 (p-t)^2 (src/loss/mse.c:72-76),
 // 1 t*logf(clip(p, 1e-7, 1-1e-7)) (src/loss/cross_entropy.c:35-44, 91-95), 2 Huber with threshold delta (src/loss/huber.c)
 __global__ __launch_bounds__(kRBlock) void loss_terms_partial_kernel(int kind, const float* p, const float* t, float* partial,
@@ -306,6 +327,29 @@ extern "C" int bh_loss_terms_sum(int kind, const float* pred, const float* targe
     hipLaunchKernelGGL(bh::sum_final_kernel, dim3(1), dim3(bh::kRBlock), 0, bh::stream(), partial, sum_out, blocks, 1.0f);
     bh_free(partial);
     return BH_LAUNCH_CHECK("bh_loss_terms_sum");
+}
+
+// loss = mean((p-t)^2) and grad = 2*(p-t)/n in one pass over p and t (what a training loop asks for together);
+// the gradient is bit for bit bh_mse_grad's, the loss sums in another order than bh_mse_loss
+extern "C" int bh_mse_loss_grad(const float* pred, const float* target, float* loss_out, float* grad, int64_t n) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(n > 0 && pred && target && loss_out && grad, "bad argument");
+    const bool vec = n % 4 == 0 && ((reinterpret_cast<uintptr_t>(pred) | reinterpret_cast<uintptr_t>(target) | reinterpret_cast<uintptr_t>(grad)) & 15) == 0;
+    if (!vec) {
+        const int rc = bh_mse_loss(pred, target, loss_out, n);
+        return rc != BH_OK ? rc : bh_mse_grad(pred, target, grad, n);
+    }
+    const int64_t n4 = n / 4;
+    int blocks = (int)ceil_div(n4, (int64_t)kRBlock * 2);
+    if (blocks > 2048) blocks = 2048;
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);
+    if (!partial) return BH_ENOMEM;
+    hipLaunchKernelGGL(bh::sse_grad_partial_kernel, dim3(blocks), dim3(bh::kRBlock), 0, bh::stream(), pred, target, grad, partial, n4,
+                       (float)(size_t)n);
+    hipLaunchKernelGGL(bh::sum_final_kernel, dim3(1), dim3(bh::kRBlock), 0, bh::stream(), partial, loss_out, blocks,
+                       1.0f / (float)(size_t)n);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK("bh_mse_loss_grad");
 }
 
 extern "C" int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n) {

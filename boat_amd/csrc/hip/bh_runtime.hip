@@ -48,8 +48,9 @@ int check_hip(hipError_t e, const char* what) {
 }
 
 // ---- profiling: one start/stop event pair per instrumented call, taken from a pool created when profiling is
-// switched on (nothing is created inside a timed region); a nested scope (bh_dense_backward calling bh_gemm) is
-// recorded for the innermost call only
+// switched on (nothing is created inside a timed region); of nested scopes (bh_dense_backward calling bh_gemm) only
+// the outermost is recorded.  A benchmark hook for ONE host thread: this state is not guarded by the library's
+// mutex, so while profiling is on no second thread may call into the library.
 struct ProfRec {
     int cls;
     double work;
@@ -70,7 +71,11 @@ void prof_open(int cls, double work, int* slot) {
     g_prof_pool.pop_back();
     r.b = g_prof_pool.back();
     g_prof_pool.pop_back();
-    if (hipEventRecord(r.a, g_stream) != hipSuccess) return;
+    if (hipEventRecord(r.a, g_stream) != hipSuccess) {   // not recorded: the pair goes back to the pool
+        g_prof_pool.push_back(r.b);
+        g_prof_pool.push_back(r.a);
+        return;
+    }
     g_prof.push_back(r);
     *slot = (int)g_prof.size() - 1;
 }

@@ -161,6 +161,14 @@ void boat_variable_zero_grad(boat_variable_t* v) {
 
 boat_tensor_t* boat_hip_variable_ensure_grad(boat_variable_t* v) {
     if (!v) return NULL;
+    if (v->grad && (v->grad_shared || v->grad->ref_count > 1)) {
+        /* a tensor other holders read too cannot become this variable's own, lasting buffer: take a copy */
+        boat_tensor_t* own = boat_tensor_clone(v->grad);
+        if (!own) return NULL;
+        boat_tensor_unref(v->grad);
+        v->grad = own;
+        v->grad_shared = false;
+    }
     if (!v->grad) v->grad = boat_tensor_create_like(v->data);
     v->persistent_grad = v->grad != NULL;
     return v->grad;
@@ -370,6 +378,9 @@ boat_variable_t* boat_hip_var_layernorm(const boat_variable_t* a, boat_layernorm
 
 /* v->grad += g ; takes ownership of g when `own` (it may become the gradient tensor itself,
  * as the reference does with freshly computed gradients, autodiff.c:1128-1135) */
+static const boat_tensor_t* g_walk_seed = NULL;   /* the caller's grad_output during a backward walk */
+static boat_variable_t* g_lender = NULL;          /* the variable whose gradient the current op hands on (its output) */
+
 static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
     if (!g) return;
     if (!v->grad) {
@@ -383,10 +394,18 @@ static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
          * handed on, so nobody adds into it afterwards, and this variable replaces it (below) instead of adding into it
          * if a second contribution comes.  Leaves keep a buffer of their own, which outlives the walk.  The
          * reference-exact walk hands on gradients that are still growing, so it copies. */
-        if (v->producer && !bt_reference_exact() && bt_is_f32(g) && bt_same_shape(g, v->data)) {
+        /* A leaf shares as well when the tensor is one the walk made itself (a non-leaf's finished gradient handed on
+         * by an add): whoever holds a tensor with other holders replaces it instead of writing into it (below), so the
+         * leaf's gradient stays what it is.  The caller's own grad_output is never a leaf's gradient: the caller may
+         * reuse that buffer. */
+        const bool lent = g_lender && g_lender->grad && g_lender->grad->st == g->st;
+        if ((v->producer || g != g_walk_seed) && !bt_reference_exact() && bt_is_f32(g) && bt_same_shape(g, v->data) &&
+            !(lent && g_lender->persistent_grad)) {
             if (!own) boat_tensor_ref(g);
             v->grad = g;
             v->grad_shared = true;
+            /* the variable it came from must not add into it later either (a second backward over a kept graph) */
+            if (lent) g_lender->grad_shared = true;
             return;
         }
         if (bt_is_f32(g) && bt_is_f32(v->data) && g->nelements == v->data->nelements && g->nelements > 0) {
@@ -415,6 +434,7 @@ static void accumulate(boat_variable_t* v, boat_tensor_t* g, bool own) {
             v->grad_shared = false;
         } else {
             boat_tensor_free(sum);
+            boat_add_(v->grad, g);      /* shapes the out-of-place kernel does not take: the reference's in-place add */
         }
     } else if (v->grad) {
         boat_add_(v->grad, g);
@@ -596,9 +616,22 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
             break;
         }
         case OP_LAYERNORM: {
-            boat_tensor_t* dx = boat_layernorm_backward_impl((boat_layernorm_t*)op->layer, op->saved[0], op->saved[1], op->saved[2], dy);
-            if (dx && a->requires_grad) accumulate(a, dx, true);
-            else boat_tensor_free(dx);
+            /* A gradient that reached the input earlier in the walk (the residual connection around a pre-LN branch) is
+             * added by the LayerNorm kernel's own store: dx = LN'(dy) + pending replaces the pending tensor. */
+            const boat_tensor_t* pending = NULL;
+            if (a->requires_grad && a->grad && !a->persistent_grad && !bt_reference_exact() && bt_is_f32(a->grad) &&
+                bt_same_shape(a->grad, a->data) && a->data == op->saved[0])
+                pending = a->grad;
+            boat_tensor_t* dx = boat_layernorm_backward_add_impl((boat_layernorm_t*)op->layer, op->saved[0], op->saved[1], op->saved[2], dy, pending);
+            if (dx && pending) {
+                boat_tensor_unref(a->grad);
+                a->grad = dx;
+                a->grad_shared = false;
+            } else if (dx && a->requires_grad) {
+                accumulate(a, dx, true);
+            } else {
+                boat_tensor_free(dx);
+            }
             break;
         }
         case OP_ATTENTION: {   /* :2458-2532 */
@@ -648,7 +681,13 @@ static void backward_depth_first(boat_variable_t* v, const boat_tensor_t* dy) {
     }
 }
 
+static void backward_walk(boat_variable_t* variable, boat_tensor_t* grad_output);
 static void boat_variable_backward_unflushed(boat_variable_t* variable, boat_tensor_t* grad_output) {
+    g_walk_seed = grad_output;
+    backward_walk(variable, grad_output);
+    g_walk_seed = NULL;
+}
+static void backward_walk(boat_variable_t* variable, boat_tensor_t* grad_output) {
     if (!variable || !variable->requires_grad) return;
     boat_tensor_t* seed = grad_output;
     if (!seed) {
@@ -696,8 +735,10 @@ static void boat_variable_backward_unflushed(boat_variable_t* variable, boat_ten
     for (size_t i = 0; i < n; i++) {
         boat_op_t* op = ops[i];
         const boat_tensor_t* dy = op == variable->producer ? seed : op->output->grad;
+        g_lender = op == variable->producer ? NULL : op->output;
         if (dy) backward_op(op, dy);
     }
+    g_lender = NULL;
     free(ops);
     if (!grad_output) boat_tensor_unref(seed);
 }

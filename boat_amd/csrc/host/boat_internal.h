@@ -112,7 +112,10 @@ struct boat_attention_t {
     boat_tensor_t* cache_lse;                /* [B*nh, S] row log-sum-exp, replaces the [B,nh,S,S] weights cache */
     boat_tensor_t* cache_attention_output;   /* [B,S,H] before the output projection */
     boat_tensor_t* cache_scores;             /* [B*nh, S, S] scaled scores for the backward pass, or NULL (shape without the
-                                                cached path, or larger than the score-cache limit) */
+                                                cached path, or larger than the score-cache limit); released by the
+                                                backward pass that reads it */
+    bool cache_causal;                       /* the mask the forward pass ran with: what its backward pass must use
+                                                (the reference's backward works from the cached weights) */
 };
 
 /* boat_attention_backward for a layer whose query, key and value were one tensor: *grad_input = dq + dk + dv, the sums
@@ -122,5 +125,8 @@ bool boat_attention_backward_self(boat_attention_t* attention, const boat_tensor
 /* layernorm backward used by both the layer hook and the tape */
 boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
                                             const boat_tensor_t* rstd, const boat_tensor_t* grad_output);
+/* the same with `add` (may be NULL; same shape as x) added to the returned input gradient by the kernel's own store */
+boat_tensor_t* boat_layernorm_backward_add_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
+                                                const boat_tensor_t* rstd, const boat_tensor_t* grad_output, const boat_tensor_t* add);
 
 #endif

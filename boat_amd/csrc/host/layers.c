@@ -299,7 +299,12 @@ boat_tensor_t* boat_layernorm_forward(boat_layernorm_t* norm, const boat_tensor_
 
 boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
                                             const boat_tensor_t* rstd, const boat_tensor_t* grad_output) {
+    return boat_layernorm_backward_add_impl(norm, x, mean, rstd, grad_output, NULL);
+}
+boat_tensor_t* boat_layernorm_backward_add_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
+                                                const boat_tensor_t* rstd, const boat_tensor_t* grad_output, const boat_tensor_t* add) {
     if (!norm || !x || !mean || !rstd || !grad_output) return NULL;
+    if (add && (!bt_is_f32(add) || add->nelements != x->nelements)) return NULL;
     if (!bt_is_f32(grad_output) || grad_output->nelements != x->nelements) {
         fprintf(stderr, "Error: LayerNorm backward shape mismatch\n");
         return NULL;
@@ -307,19 +312,35 @@ boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_t
     const int64_t hidden = (int64_t)norm->config.normalized_shape;
     const int64_t rows = (int64_t)mean->nelements;
     const bool covers_all = rows * hidden == (int64_t)x->nelements;
+    if (add && (!covers_all || rows == 0)) {
+        /* rows the kernel does not visit keep the other gradient alone: start from a copy of it */
+        boat_tensor_t* base = boat_tensor_clone(add);
+        boat_tensor_t* part = base ? boat_layernorm_backward_add_impl(norm, x, mean, rstd, grad_output, NULL) : NULL;
+        if (part) boat_add_(base, part);
+        else {
+            boat_tensor_free(base);
+            base = NULL;
+        }
+        boat_tensor_free(part);
+        return base;
+    }
     boat_tensor_t* dx = covers_all ? bt_new_like_uninit(x) : boat_tensor_create_like(x);
     if (!dx) return NULL;
     if (rows == 0) return dx;
     const float* px = bt_dev_read(x);
     const float* pdy = bt_dev_read(grad_output);
     const float* pg = norm->weight ? bt_dev_read(norm->weight) : NULL;
+    const float* padd = add ? bt_dev_read(add) : NULL;
     float* pdx = covers_all ? bt_dev_write(dx) : bt_dev_rw(dx);
     float* pgw = norm->grad_weight ? bt_dev_rw(norm->grad_weight) : NULL;
     float* pgb = norm->grad_bias ? bt_dev_rw(norm->grad_bias) : NULL;
     /* parameter gradients accumulate across calls like the dense layer's (dense.c:255-291) */
-    if (!px || !pdy || !pdx ||
-        !boat_hip_ok(bh_layernorm_backward(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), pdx, pgw, pgb, rows, hidden, 1),
-                     "layernorm backward")) {
+    bool ok = px && pdy && pdx && (padd || !add);
+    if (ok && add) ok = boat_hip_ok(bh_layernorm_backward_add(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), padd, pdx, pgw, pgb, rows, hidden, 1),
+                                    "layernorm backward");
+    else if (ok) ok = boat_hip_ok(bh_layernorm_backward(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), pdx, pgw, pgb, rows, hidden, 1),
+                                  "layernorm backward");
+    if (!ok) {
         boat_tensor_free(dx);
         return NULL;
     }
@@ -611,10 +632,21 @@ boat_tensor_t* boat_attention_forward(boat_attention_t* a, const boat_tensor_t* 
     }
     if (rows == 0) return bt_new_like_uninit(query);
 
-    a->cache_q_proj = project(query, a->weight_q, a->bias_q, rows, h);
-    a->cache_k_proj = project(key, a->weight_k, a->bias_k, rows, h);
-    a->cache_v_proj = project(value, a->weight_v, a->bias_v, rows, h);
+    /* the three input projections (attention.c:363-365) as one grouped launch */
+    a->cache_q_proj = bt_new_like_uninit(query);
+    a->cache_k_proj = bt_new_like_uninit(query);
+    a->cache_v_proj = bt_new_like_uninit(query);
     if (!a->cache_q_proj || !a->cache_k_proj || !a->cache_v_proj) return NULL;
+    {
+        const float* px[3] = {bt_dev_read(query), bt_dev_read(key), bt_dev_read(value)};
+        const float* pw[3] = {bt_dev_read(a->weight_q), bt_dev_read(a->weight_k), bt_dev_read(a->weight_v)};
+        const float* pb[3] = {a->bias_q ? bt_dev_read(a->bias_q) : NULL, a->bias_k ? bt_dev_read(a->bias_k) : NULL,
+                              a->bias_v ? bt_dev_read(a->bias_v) : NULL};
+        float* py[3] = {bt_dev_write(a->cache_q_proj), bt_dev_write(a->cache_k_proj), bt_dev_write(a->cache_v_proj)};
+        for (int i = 0; i < 3; i++)
+            if (!px[i] || !pw[i] || !py[i]) return NULL;
+        if (!boat_hip_ok(bh_gemm_grouped(0, 0, rows, h, h, 3, px, h, pw, h, py, h, pb, 0), "attention input projections")) return NULL;
+    }
 
     /* [B,S,H] viewed as [B*nh, S, hd]: block (b,h) is the h-th run of S*hd floats of batch b */
     const int64_t lshape[] = {batch * nh, seq};
@@ -631,17 +663,19 @@ boat_tensor_t* boat_attention_forward(boat_attention_t* a, const boat_tensor_t* 
         const int64_t sshape[] = {batch * nh, seq, seq};
         a->cache_scores = bt_new_uninit(sshape, 3, query->device);     /* no room: fall back to recomputing */
     }
+    const boat_error_t err_before = boat_get_last_error();
     float* scores = a->cache_scores ? bt_dev_write(a->cache_scores) : NULL;
     if (a->cache_scores && !scores) {           /* no HBM for it: the backward pass recomputes */
         boat_tensor_free(a->cache_scores);
         a->cache_scores = NULL;
-        boat_reset_error();
+        if (err_before == BOAT_SUCCESS) boat_reset_error();   /* only the error this attempt raised */
     }
+    a->cache_causal = a->config.causal_mask;
     const int rc = scores ? bh_sdpa_forward_cached(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
-                                                   scale, a->config.causal_mask ? 1 : 0, bt_dev_write(a->cache_attention_output),
+                                                   scale, a->cache_causal ? 1 : 0, bt_dev_write(a->cache_attention_output),
                                                    bt_dev_write(a->cache_lse), scores, batch * nh, seq, hd)
                           : bh_sdpa_forward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj), scale,
-                                            a->config.causal_mask ? 1 : 0, bt_dev_write(a->cache_attention_output),
+                                            a->cache_causal ? 1 : 0, bt_dev_write(a->cache_attention_output),
                                             bt_dev_write(a->cache_lse), NULL, batch * nh, seq, hd);
     if (!boat_hip_ok(rc, "attention core forward")) return NULL;
     return project(a->cache_attention_output, a->weight_o, a->bias_o, rows, h);
@@ -733,6 +767,58 @@ static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor
     return dx;
 }
 
+/* the backward of the three input projections; sum: *gq = dq.Wq^T + dk.Wk^T + dv.Wv^T and *gk, *gv are further
+ * references to it */
+static bool project_backward3(boat_attention_t* a, const boat_tensor_t* dqp, const boat_tensor_t* dkp, const boat_tensor_t* dvp,
+                              int64_t rows, int64_t h, bool sum, boat_tensor_t** gq, boat_tensor_t** gk, boat_tensor_t** gv) {
+    const boat_tensor_t* x[3] = {a->cache_query, a->cache_key, a->cache_value};
+    const boat_tensor_t* w[3] = {a->weight_q, a->weight_k, a->weight_v};
+    const boat_tensor_t* bias[3] = {a->bias_q, a->bias_k, a->bias_v};
+    const boat_tensor_t* dy[3] = {dqp, dkp, dvp};
+    boat_tensor_t** gw[3] = {&a->grad_weight_q, &a->grad_weight_k, &a->grad_weight_v};
+    boat_tensor_t** gb[3] = {&a->grad_bias_q, &a->grad_bias_k, &a->grad_bias_v};
+    boat_tensor_t* dx[3] = {NULL, NULL, NULL};
+    const float *px[3], *pw[3], *pdy[3];
+    float *pgw[3], *pdx[3];
+    bool ok = true;
+    for (int i = 0; i < 3 && ok; i++) {
+        if (!*gw[i]) *gw[i] = boat_tensor_create_like(w[i]);
+        if (bias[i] && !*gb[i]) *gb[i] = boat_tensor_create_like(bias[i]);
+        if (i == 0 || !sum) dx[i] = bt_new_like_uninit(x[i]);
+        ok = *gw[i] && (!bias[i] || *gb[i]) && (dx[i] || (sum && i > 0));
+        if (!ok) break;
+        px[i] = bt_dev_read(x[i]);
+        pw[i] = bt_dev_read(w[i]);
+        pdy[i] = bt_dev_read(dy[i]);
+        pgw[i] = bt_dev_write(*gw[i]);
+        pdx[i] = dx[i] ? bt_dev_write(dx[i]) : NULL;
+        ok = px[i] && pw[i] && pdy[i] && pgw[i] && (pdx[i] || !dx[i]);
+    }
+    /* dx = dy.w^T */
+    if (ok && sum) ok = boat_hip_ok(bh_gemm_ksegments(0, 1, rows, h, h, 3, pdy, h, pw, h, pdx[0], h, NULL, 0), "attention input gradient");
+    else if (ok) ok = boat_hip_ok(bh_gemm_grouped(0, 1, rows, h, h, 3, pdy, h, pw, h, pdx, h, NULL, 0), "attention input gradients");
+    /* gw = x^T.dy (overwritten per call, attention.c:1262-1279) */
+    if (ok) ok = boat_hip_ok(bh_gemm_grouped(1, 0, h, h, rows, 3, px, h, pdy, h, pgw, h, NULL, 0), "attention weight gradients");
+    /* gb = colsum(dy) */
+    for (int i = 0; i < 3 && ok; i++) {
+        float* pgb = bias[i] ? bt_dev_write(*gb[i]) : NULL;
+        if (bias[i]) ok = pgb && boat_hip_ok(bh_colsum(pdy[i], pgb, rows, h, 0), "attention bias gradient");
+    }
+    if (!ok) {
+        for (int i = 0; i < 3; i++) boat_tensor_free(dx[i]);
+        return false;
+    }
+    if (sum) {
+        boat_tensor_ref(dx[0]);
+        boat_tensor_ref(dx[0]);
+        dx[1] = dx[2] = dx[0];
+    }
+    *gq = dx[0];
+    *gk = dx[1];
+    *gv = dx[2];
+    return true;
+}
+
 static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_t* grad_output, boat_tensor_t** grad_query,
                                          boat_tensor_t** grad_key, boat_tensor_t** grad_value);
 static boat_tensor_t* g_sum_into = NULL;   /* set by boat_attention_backward_self for the duration of one call */
@@ -797,26 +883,29 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
         int rc = a->cache_scores
             ? bh_sdpa_backward_cached(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
                                       bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(a->cache_scores),
-                                      bt_dev_read(d_ao), scale, a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp),
+                                      bt_dev_read(d_ao), scale, a->cache_causal ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp),
                                       bt_dev_write(dvp), batch * nh, seq, hd)
             : bh_sdpa_backward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
                                bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(d_ao), scale,
-                               a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
+                               a->cache_causal ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
         /* no room for the cached kernel's dQ workspace: the plain entry point can fall back to its bounded GEMM path */
         if (rc == BH_ENOMEM && a->cache_scores)
             rc = bh_sdpa_backward(bt_dev_read(a->cache_q_proj), bt_dev_read(a->cache_k_proj), bt_dev_read(a->cache_v_proj),
                                   bt_dev_read(a->cache_attention_output), bt_dev_read(a->cache_lse), bt_dev_read(d_ao), scale,
-                                  a->config.causal_mask ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
+                                  a->cache_causal ? 1 : 0, bt_dev_write(dqp), bt_dev_write(dkp), bt_dev_write(dvp), batch * nh, seq, hd);
         ok = boat_hip_ok(rc, "attention core backward");
     }
     boat_tensor_free(d_ao);
-    /* 3. input projections */
+    /* the score matrix has served its one backward pass: a repeated backward call recomputes Q.K^T from the projections,
+     * and a model of many layers holds no score matrices between steps */
+    boat_tensor_free(a->cache_scores);
+    a->cache_scores = NULL;
+    /* 3. input projections (linear_projection_backward three times, attention.c:1186-1285): the three weight gradients
+     * as one grouped launch, the three column sums, and the input gradients either as one grouped launch or, for
+     * self-attention through the tape, as ONE product whose contraction runs over the three (dY, W) pairs */
     boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
-    /* self-attention through the tape: the key and value projections add their input gradients into the query's */
     const bool sum = g_sum_into != NULL;
-    if (ok) gq = project_backward(a->cache_query, a->weight_q, a->bias_q, dqp, &a->grad_weight_q, &a->grad_bias_q, rows, h, NULL);
-    if (ok && gq) gk = project_backward(a->cache_key, a->weight_k, a->bias_k, dkp, &a->grad_weight_k, &a->grad_bias_k, rows, h, sum ? gq : NULL);
-    if (ok && gk) gv = project_backward(a->cache_value, a->weight_v, a->bias_v, dvp, &a->grad_weight_v, &a->grad_bias_v, rows, h, sum ? gq : NULL);
+    if (ok) ok = project_backward3(a, dqp, dkp, dvp, rows, h, sum, &gq, &gk, &gv);
     boat_tensor_free(dqp);
     boat_tensor_free(dkp);
     boat_tensor_free(dvp);

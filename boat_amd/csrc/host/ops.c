@@ -415,8 +415,8 @@ boat_tensor_t* boat_hip_mse_loss(const boat_tensor_t* pred, const boat_tensor_t*
     const float* pp = bt_dev_read(pred);
     const float* pt = bt_dev_read(target);
     bool ok = loss && pp && pt && (!grad || g);
-    if (ok) ok = boat_hip_ok(bh_mse_loss(pp, pt, bt_dev_write(loss), (int64_t)pred->nelements), "mse loss");
-    if (ok && g) ok = boat_hip_ok(bh_mse_grad(pp, pt, bt_dev_write(g), (int64_t)pred->nelements), "mse grad");
+    if (ok && g) ok = boat_hip_ok(bh_mse_loss_grad(pp, pt, bt_dev_write(loss), bt_dev_write(g), (int64_t)pred->nelements), "mse loss and gradient");
+    else if (ok) ok = boat_hip_ok(bh_mse_loss(pp, pt, bt_dev_write(loss), (int64_t)pred->nelements), "mse loss");
     if (!ok) {
         boat_tensor_free(loss);
         boat_tensor_free(g);

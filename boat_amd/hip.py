@@ -44,7 +44,7 @@ _SIGS = {
     "bh_activation_forward": (I, [I, P, P, L]),
     "bh_activation_backward": (I, [I, P, P, P, L, I]),
     "bh_bias_add_rows": (I, [P, P, L, L]),
-    "bh_mse_grad": (I, [P, P, P, L]), "bh_mse_loss": (I, [P, P, P, L]),
+    "bh_mse_grad": (I, [P, P, P, L]), "bh_mse_loss": (I, [P, P, P, L]), "bh_mse_loss_grad": (I, [P, P, P, P, L]),
     "bh_sgd_update": (I, [P, P, F, L, I]),
     "bh_sum_all": (I, [P, P, L]),
     "bh_colsum": (I, [P, P, L, L, I]),
@@ -53,12 +53,16 @@ _SIGS = {
     "bh_softmax_ce_grad": (I, [P, P, P, P, L, L]),
     "bh_layernorm_forward": (I, [P, P, P, P, P, P, L, L, F]),
     "bh_layernorm_backward": (I, [P, P, P, P, P, P, P, P, L, L, I]),
+    "bh_layernorm_backward_add": (I, [P, P, P, P, P, P, P, P, P, L, L, I]),
     "bh_rmsnorm_forward": (I, [P, P, P, P, L, L, F]),
     "bh_rmsnorm_backward": (I, [P, P, P, P, P, P, L, L, F, I]),
     "bh_binary_typed": (I, [I, I, P, C.POINTER(L), P, C.POINTER(L), P, C.POINTER(L), I]),
     "bh_scalar_op_typed": (I, [I, I, P, C.c_double, P, L]),
     "bh_layernorm_backward_noalloc": (I, [P, P, P, P, P, P, P, P, L, L, I]),
     "bh_gemm": (I, [I, I, L, L, L, P, L, P, L, P, L, P, I, L]),
+    "bh_gemm_grouped": (I, [I, I, L, L, L, I, C.POINTER(P), L, C.POINTER(P), L, C.POINTER(P), L, C.POINTER(P), I]),
+    "bh_gemm_ksegments": (I, [I, I, L, L, L, I, C.POINTER(P), L, C.POINTER(P), L, P, L, P, I]),
+    "bh_gemm_no_tables": (I, [I]),
     "bh_gemm_force_config": (I, [I]), "bh_gemm_force_direct": (I, [I]), "bh_gemm_force_splits": (I, [I]),
     "bh_transpose_last2": (I, [P, P, L, L, L]),
     "bh_dense_backward": (I, [P, P, P, P, P, P, L, L, L, I]),

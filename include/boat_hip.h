@@ -69,7 +69,8 @@ float       bh_event_elapsed_ms(bh_event_t* start, bh_event_t* stop);    /* sync
  * (an entry point called from another instrumented one is not recorded twice); bh_profile_enable(0) stops and frees.
  * Each call to enable starts a fresh recording.  bh_profile_read waits for the stream and sums, for one class, the
  * event-to-event time in ms, the algorithmic work the calls declared (flops for the matrix classes, bytes for the
- * memory-bound ones) and the number of calls.  Calls beyond max_calls are not recorded. */
+ * memory-bound ones) and the number of calls.  Calls beyond max_calls are not recorded.  A hook for single-threaded
+ * benchmarks: while profiling is on, only one host thread may call into the library. */
 #define BH_PROF_GEMM       0   /* bh_gemm: 2*m*n*k*batch flops */
 #define BH_PROF_SDPA_FWD   1   /* bh_sdpa_forward: 2 * 2*bh*s*s*d flops */
 #define BH_PROF_SDPA_BWD   2   /* bh_sdpa_backward: 4 * 2*bh*s*s*d flops (the reference's four contractions) */
@@ -121,6 +122,8 @@ int bh_mse_grad(const float* pred, const float* target, float* grad, int64_t n);
  * kind 0 (p-t)^2, 1 t*logf(clip(p, 1e-7, 1-1e-7)), 2 Huber(|p-t|, delta); sum_out is one float in device memory */
 int bh_loss_terms_sum(int kind, const float* pred, const float* target, float* sum_out, int64_t n, float delta);
 int bh_mse_loss(const float* pred, const float* target, float* loss_out, int64_t n);  /* src/loss/mse.c:70-78 */
+/* both in one pass over pred and target (the loop of tests/test_attention_training.c:28-41 computes them together) */
+int bh_mse_loss_grad(const float* pred, const float* target, float* loss_out, float* grad, int64_t n);
 int bh_sgd_update(float* p, float* g, float lr, int64_t n, int zero_grad);            /* dense.c:297-329 */
 
 /* ---- reductions / softmax (src/ops/arithmetic.c:611-691; src/autodiff.c:1701-2068; dense.c:286-291) ---- */
@@ -153,8 +156,16 @@ int bh_rmsnorm_forward(const float* x, const float* weight, float* y, float* inv
 int bh_rmsnorm_backward(const float* x, const float* weight, const float* dy, const float* inv_rms,
                         float* dx, float* dweight, int64_t rows, int64_t hidden, float eps, int accumulate);
 
-/* bh_layernorm_backward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels and
+/* The same with dx = (the LayerNorm input gradient) + add[rows, hidden]: a variable that feeds a LayerNorm and a residual
+ * connection (x1 in y = x1 + f(LN(x1))) gets both gradients in the LayerNorm kernel's one store instead of in an adding
+ * pass of its own (the sum the reference's tape makes with boat_add_, src/autodiff.c:1002-1061).  add must not overlap dx. */
+int bh_layernorm_backward_add(const float* x, const float* gamma, const float* dy,
+                              const float* mean, const float* rstd, const float* add,
+                              float* dx, float* dgamma, float* dbeta,
+                              int64_t rows, int64_t hidden, int accumulate);
+
+/* bh_layernorm_backward for callers that cannot allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc; it launches on the library's own stream, so it is not for a caller's graph capture).  It has no counterpart in the reference.  Same arguments, same kernels and
  * the same results as bh_layernorm_backward; the per-workgroup dgamma/dbeta partials live in a 16 MiB device array
  * that is part of the library image (one copy per GPU, held until the process ends) instead of coming from bh_malloc.
  * It calls no hipMalloc/hipFree and sets nothing up: bh_init() must have returned BH_OK before.  hidden must be a
@@ -177,6 +188,20 @@ int bh_layernorm_backward_noalloc(const float* x, const float* gamma, const floa
 int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
             const float* a, int64_t lda, const float* b, int64_t ldb,
             float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch);
+/* Up to 3 products of ONE shape whose operands are separate tensors: c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g]), arguments
+ * as bh_gemm with tables of `groups` pointers (bias may be NULL, or hold NULLs).  The three input projections of a
+ * self-attention layer (src/layers/attention.c:363-365: the same input times Wq, Wk, Wv) and their three weight gradients
+ * (:1186-1285 run three times) are one launch each this way; the arithmetic of every product is that of bh_gemm. */
+int bh_gemm_grouped(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int groups,
+                    const float* const* a, int64_t lda, const float* const* b, int64_t ldb,
+                    float* const* c, int64_t ldc, const float* const* bias, int accumulate);
+/* One product whose contraction runs over up to 3 operand pairs of k each: c (+)= sum_s op(a[s]) . op(b[s]) (+ bias).
+ * The summed input gradient of self-attention, dQ.Wq^T + dK.Wk^T + dV.Wv^T (what the reference's caller adds up after
+ * three linear_projection_backward calls, src/autodiff.c:2458-2532), is one launch without read-modify-write this way.
+ * Shapes that do not take the matrix-core tiles run pair by pair, adding into c: the same sum in another order. */
+int bh_gemm_ksegments(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int segments,
+                      const float* const* a, int64_t lda, const float* const* b, int64_t ldb,
+                      float* c, int64_t ldc, const float* bias, int accumulate);
 int bh_transpose_last2(const float* a, float* out, int64_t batch, int64_t rows, int64_t cols); /* linear.c:238-406 */
 /* out[a][d1][b][d0][c] = in[a][d0][b][d1][c]: boat_transpose of any two dimensions of a dense tensor (linear.c:238-406;
  * a, b, c are the products of the extents before, between and after the two) */
@@ -272,6 +297,9 @@ int bh_gemm_force_config(int cfg);
 int bh_gemm_force_direct(int mode);
 /* bh_gemm_force_splits: where the MFMA tiles would split the contraction, split it this many ways (0 = heuristic) */
 int bh_gemm_force_splits(int splits);
+/* bh_gemm_no_tables: 1 = bh_gemm_grouped / bh_gemm_ksegments run their products one launch after the other (0 = one launch
+ * where the shape allows) */
+int bh_gemm_no_tables(int off);
 int bh_sdpa_force_general(int on);
 /* bh_layernorm_tune: cap on the workgroups of the LayerNorm backward (each writes one dgamma/dbeta partial) and of
  * the forward; 0 keeps the current value. */

@@ -130,6 +130,33 @@ def fanout(api, a, b):
     return _grad(api, va), _grad(api, vb)
 
 
+def backward_twice(api, a, b, c, d, g1, g2):
+    """w = (a*b + c) * d, then boat_variable_backward(w, g1) and boat_variable_backward(w, g2) over the same kept graph.
+    Non-leaf gradients are not cleared between the two walks (src/autodiff.c:373-450 adds into what is there), so the
+    second walk hands on u.grad = (g1 + g2)*d: a chain, on which the reference and a walk that visits each op once agree.
+    Returns the gradients of a, b, c, d."""
+    va, vb, vc, vd = (_var(api, t, True) for t in (a, b, c, d))
+    vt = api.boat_var_mul(va, vb)
+    vu = api.boat_var_add(vt, vc)
+    vw = api.boat_var_mul(vu, vd)
+    for g in (g1, g2):
+        tg = api.tensor(np.asarray(g, np.float32))
+        api.boat_variable_backward(vw, tg)
+        api.boat_tensor_unref(tg)
+    return tuple(_grad(api, v) for v in (va, vb, vc, vd))
+
+
+def backward_twice_expected(a, b, c, d, g1, g2):
+    """Closed form of backward_twice in float64."""
+    a, b, c, d, g1, g2 = (np.asarray(t, np.float64) for t in (a, b, c, d, g1, g2))
+    u = a * b + c
+    gu1 = g1 * d                     # after the first walk
+    gu2 = gu1 + g2 * d               # u.grad after the second contribution
+    gt = gu1 + gu2                   # t.grad: first walk's, plus the accumulated u.grad handed on by the add
+    gc = gu1 + gu2
+    return gt * b + gu1 * b, gt * a + gu1 * a, gc, g1 * u + g2 * u
+
+
 def grad_under_disabled_context(api, a, b):
     """y = a*b recorded while the current context has gradients switched off, then backward: the gradient of a, or None
     when the op left no tape entry."""

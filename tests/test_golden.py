@@ -577,6 +577,28 @@ def test_gpu_fanout_is_the_true_gradient_not_the_reference_value(boat):
     assert same(da, 2 * g["b"]) and same(db, 2 * g["a"])      # the reference reports 4b, 4a (see the fixture)
 
 
+def _backward_twice_inputs():
+    rng = np.random.default_rng(77)
+    return [rng.standard_normal((3, 5)).astype(np.float32) for _ in range(6)]
+
+
+def test_reference_backward_twice_over_a_kept_graph(ref):
+    """The compiled reference on bc.backward_twice: non-leaf gradients persist between two backward calls, so the second
+    walk hands on the accumulated gradient (the closed form in bc.backward_twice_expected)."""
+    t = _backward_twice_inputs()
+    for got, want in zip(bc.backward_twice(ref, *t), bc.backward_twice_expected(*t)):
+        assert close_max(got, want, TOL_EW)
+
+
+@pytest.mark.gpu
+def test_gpu_backward_twice_over_a_kept_graph(boat):
+    """The same scenario on this library, whose walk shares gradient tensors between variables instead of copying them:
+    a second backward over the kept graph must not add into a tensor another variable holds."""
+    t = _backward_twice_inputs()
+    for got, want in zip(bc.backward_twice(boat, *t), bc.backward_twice_expected(*t)):
+        assert close_max(got, want, TOL_EW)
+
+
 @pytest.mark.gpu
 def test_gpu_reference_exact_mode(boat):
     """boat_hip_set_reference_exact(1): the three deliberate divergences follow the reference at once -- the depth-first

@@ -291,6 +291,28 @@ def test_layernorm_forward(hip, oracle, rng, rows, hidden):
 
 
 @pytest.mark.parametrize("rows,hidden", LN_SHAPES + [(1000, 1024), (300, 4096)])
+def test_layernorm_backward_with_added_gradient(hip, oracle, rng, rows, hidden):
+    """bh_layernorm_backward_add: dx = LayerNorm input gradient + add, the same kernel's arithmetic plus one fp32 add per
+    element (bit for bit what bh_layernorm_backward followed by an add gives); parameter gradients unchanged."""
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    dy = rng.standard_normal((rows, hidden)).astype(np.float32)
+    add = rng.standard_normal((rows, hidden)).astype(np.float32)
+    _, mean, rstd = oracle.layernorm_forward(x, gamma, None, 1e-5)
+    args = (dev(hip, x).ptr, dev(hip, gamma).ptr, dev(hip, dy).ptr, dev(hip, mean).ptr, dev(hip, rstd).ptr)
+    dx0, dg0, db0 = hip.empty((rows, hidden)), hip.zeros(hidden), hip.zeros(hidden)
+    hip.check(hip.bh_layernorm_backward(*args, dx0.ptr, dg0.ptr, db0.ptr, rows, hidden, 0))
+    dx1, dg1, db1 = hip.empty((rows, hidden)), hip.zeros(hidden), hip.zeros(hidden)
+    hip.check(hip.bh_layernorm_backward_add(*args, dev(hip, add).ptr, dx1.ptr, dg1.ptr, db1.ptr, rows, hidden, 0))
+    assert np.array_equal(dx1.numpy(), dx0.numpy() + add)
+    assert np.array_equal(dg1.numpy(), dg0.numpy()) and np.array_equal(db1.numpy(), db0.numpy())
+    wdx, _, _ = oracle.layernorm_backward_f64(x, gamma, dy, mean, rstd)
+    assert np.max(np.abs(dx1.numpy() - (wdx + add))) <= TOL_RED * np.abs(wdx + add).max()
+    with pytest.raises(RuntimeError):      # in place is refused
+        hip.check(hip.bh_layernorm_backward_add(*args, dx1.ptr, dx1.ptr, dg1.ptr, db1.ptr, rows, hidden, 0))
+
+
+@pytest.mark.parametrize("rows,hidden", LN_SHAPES + [(1000, 1024), (300, 4096)])
 def test_layernorm_backward(hip, oracle, rng, rows, hidden):
     x = rng.standard_normal((rows, hidden)).astype(np.float32)
     gamma = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
@@ -445,6 +467,120 @@ def test_gemm_epilogues_and_batch(hip, rng):
     gemm_case(hip, rng, 0, 0, 5, 4, 6, batch=6)                      # the [2,3,5,4].[2,3,4,6] layout case
     gemm_case(hip, rng, 1, 0, 256, 256, 4096, accumulate=True)       # split-K with accumulation
     gemm_case(hip, rng, 1, 0, 128, 384, 2048, bias=True)             # split-K with bias
+
+
+def _ptr_table(arrays):
+    import ctypes as C
+    return (C.c_void_p * len(arrays))(*[a.ptr if a is not None else None for a in arrays])
+
+
+@pytest.mark.parametrize("force", [None, 1, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k,accumulate,bias,shared_a", [
+    (512, 384, 256, False, True, True),      # the forward projections' form: one input, three weights, three biases
+    (260, 132, 96, True, True, False),       # ragged edge tiles, accumulate
+    (256, 384, 2048, True, False, True),     # split-K: partials of the three groups folded by one launch
+    (40, 24, 12, False, False, False),       # no table kernel for this shape: the groups run one after the other
+])
+def test_gemm_grouped_equals_separate_launches(hip, rng, force, ta, tb, m, n, k, accumulate, bias, shared_a):
+    """bh_gemm_grouped (three products of one shape in one launch, operands from pointer tables) against float64 and,
+    bit for bit, against the same three products through bh_gemm: the grouped kernels walk each product as bh_gemm does."""
+    groups = 3
+    a = [rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32) for _ in range(1 if shared_a else groups)]
+    if shared_a:
+        a = a * groups
+    b = [rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32) for _ in range(groups)]
+    c0 = [rng.standard_normal((m, n)).astype(np.float32) for _ in range(groups)]
+    bv = [rng.standard_normal(n).astype(np.float32) if (bias and g != 1) else None for g in range(groups)]   # one group without bias
+    da = [dev(hip, a[0])] * groups if shared_a else [dev(hip, x) for x in a]
+    db = [dev(hip, x) for x in b]
+    dbias = [dev(hip, x) if x is not None else None for x in bv]
+    lda, ldb = a[0].shape[1], b[0].shape[1]
+    results = []
+    for tables_off in (0, 1):
+        dc = [dev(hip, x) for x in c0]
+        if force is not None:
+            hip.bh_gemm_force_config(force)
+        hip.bh_gemm_no_tables(tables_off)
+        try:
+            hip.check(hip.bh_gemm_grouped(ta, tb, m, n, k, groups, _ptr_table(da), lda, _ptr_table(db), ldb, _ptr_table(dc), n,
+                                          _ptr_table(dbias) if bias else None, int(accumulate)))
+        finally:
+            hip.bh_gemm_force_config(-1)
+            hip.bh_gemm_no_tables(0)
+        results.append([x.numpy() for x in dc])
+    for g in range(groups):
+        A = a[g].T if ta else a[g]
+        B = b[g].T if tb else b[g]
+        want = A.astype(np.float64) @ B.astype(np.float64)
+        if bv[g] is not None:
+            want = want + bv[g]
+        if accumulate:
+            want = want + c0[g]
+        assert rel_fro(results[0][g], want) <= fp32_gemm_bound(k), (g, rel_fro(results[0][g], want))
+        assert np.array_equal(results[0][g], results[1][g]), g
+
+
+@pytest.mark.parametrize("force", [None, 1, 2, 3, 4])
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k,accumulate,bias", [(512, 256, 128, False, False), (300, 260, 64, True, True), (256, 128, 1024, False, True),
+                                                   (48, 40, 20, True, False)])
+def test_gemm_ksegments(hip, rng, force, ta, tb, m, n, k, accumulate, bias):
+    """bh_gemm_ksegments: c (+)= a0.b0 + a1.b1 + a2.b2 as one contraction over three operand pairs (the summed input
+    gradient of self-attention), against float64 at the bound only fp32 accumulation meets, and against the
+    pair-by-pair fallback to fp32 rounding."""
+    segs = 3
+    a = [rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32) for _ in range(segs)]
+    b = [rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32) for _ in range(segs)]
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    bv = rng.standard_normal(n).astype(np.float32) if bias else None
+    want = sum((x.T if ta else x).astype(np.float64) @ (y.T if tb else y).astype(np.float64) for x, y in zip(a, b))
+    if bias:
+        want = want + bv
+    if accumulate:
+        want = want + c0
+    da, db = [dev(hip, x) for x in a], [dev(hip, x) for x in b]
+    dbias = dev(hip, bv) if bias else None
+    got = []
+    for tables_off in (0, 1):
+        dc = dev(hip, c0)
+        if force is not None:
+            hip.bh_gemm_force_config(force)
+        hip.bh_gemm_no_tables(tables_off)
+        try:
+            hip.check(hip.bh_gemm_ksegments(ta, tb, m, n, k, segs, _ptr_table(da), a[0].shape[1], _ptr_table(db), b[0].shape[1], dc.ptr, n,
+                                            dbias.ptr if bias else None, int(accumulate)))
+        finally:
+            hip.bh_gemm_force_config(-1)
+            hip.bh_gemm_no_tables(0)
+        got.append(dc.numpy())
+        assert rel_fro(got[-1], want) <= fp32_gemm_bound(segs * k), (tables_off, rel_fro(got[-1], want))
+    assert rel_fro(got[0], got[1]) <= 2 * fp32_gemm_bound(segs * k)
+
+
+def test_gemm_grouped_at_the_block_shapes(hip, rng):
+    """The three grouped launches of a self-attention layer at d_model 1024 and 8192 rows (forward projections, summed
+    input gradient, weight gradients with split contraction), sampled against float64."""
+    rows, h = 8192, 1024
+    x = rng.standard_normal((rows, h)).astype(np.float32)
+    w = [(0.02 * rng.standard_normal((h, h))).astype(np.float32) for _ in range(3)]
+    bias = [rng.standard_normal(h).astype(np.float32) for _ in range(3)]
+    dy = [rng.standard_normal((rows, h)).astype(np.float32) for _ in range(3)]
+    dx_, dw, db, ddy = dev(hip, x), [dev(hip, t) for t in w], [dev(hip, t) for t in bias], [dev(hip, t) for t in dy]
+    y = [hip.empty((rows, h)) for _ in range(3)]
+    hip.check(hip.bh_gemm_grouped(0, 0, rows, h, h, 3, _ptr_table([dx_] * 3), h, _ptr_table(dw), h, _ptr_table(y), h, _ptr_table(db), 0))
+    gin = hip.empty((rows, h))
+    hip.check(hip.bh_gemm_ksegments(0, 1, rows, h, h, 3, _ptr_table(ddy), h, _ptr_table(dw), h, gin.ptr, h, None, 0))
+    gw = [hip.empty((h, h)) for _ in range(3)]
+    hip.check(hip.bh_gemm_grouped(1, 0, h, h, rows, 3, _ptr_table([dx_] * 3), h, _ptr_table(ddy), h, _ptr_table(gw), h, None, 0))
+    r = np.sort(rng.choice(rows, 24, replace=False))
+    c = np.sort(rng.choice(h, 24, replace=False))
+    x64 = x.astype(np.float64)
+    for g in range(3):
+        assert rel_fro(y[g].numpy()[r], x64[r] @ w[g].astype(np.float64) + bias[g]) <= fp32_gemm_bound(h), g
+        assert rel_fro(gw[g].numpy()[c], x64[:, c].T @ dy[g].astype(np.float64)) <= fp32_gemm_bound(rows), g
+    want = sum(dy[g][r].astype(np.float64) @ w[g].astype(np.float64).T for g in range(3))
+    assert rel_fro(gin.numpy()[r], want) <= fp32_gemm_bound(3 * h)
 
 
 def test_gemm_matches_reference_loop_order_within_tolerance(hip, oracle, rng):

@@ -121,6 +121,25 @@ __global__ __launch_bounds__(kRBlock) void row_softmax_kernel(const float* __res
     }
 }
 
+// Backward of loss = f * sum(w o log_softmax(z)) in one kernel: the chain rule of mul, sum, mul and log-softmax with the
+// operations of the separate kernels in their order (dls = (seed*f) * w ; g = sum_j dls_j ; dz_j = dls_j - expf(y_j) * g),
+// so the result is the chain's bit for bit.  y = log_softmax(z) as the forward pass left it.
+__global__ __launch_bounds__(kRBlock) void log_softmax_weighted_bwd_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                                           const float* __restrict__ seed, const float* __restrict__ f,
+                                                                           float* __restrict__ dz, int64_t rows, int64_t cols) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kRBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float c = (seed ? seed[0] : 1.0f) * f[0];
+    const float* yr = y + row * cols;
+    const float* wr = w + row * cols;
+    float* out = dz + row * cols;
+    float g = 0.f;
+    for (int64_t i = lane; i < cols; i += 64) g += c * wr[i];
+    g = wave_sum(g);
+    for (int64_t i = lane; i < cols; i += 64) out[i] = c * wr[i] - expf(yr[i]) * g;
+}
+
 // fused softmax + cross-entropy gradient; row_ll receives log_softmax(z)[label] per row
 __global__ __launch_bounds__(kRBlock) void softmax_ce_kernel(const float* __restrict__ z, const int32_t* __restrict__ labels,
                                                              float* __restrict__ dz, float* __restrict__ row_ll,
@@ -224,6 +243,17 @@ int bh_log_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols)
 int bh_log_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols) {
     BH_CHECK_ARG(dy || rows * cols == 0, "null dy");
     BH_ROW_LAUNCH(3, y, dy, dx, "bh_log_softmax_backward");
+}
+
+int bh_log_softmax_weighted_backward(const float* y, const float* w, const float* seed, const float* f, float* dz,
+                                     int64_t rows, int64_t cols) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && cols >= 0, "negative shape");
+    if (rows * cols == 0) return BH_OK;
+    BH_CHECK_ARG(y && w && f && dz, "null pointer");
+    hipLaunchKernelGGL(log_softmax_weighted_bwd_kernel, dim3((unsigned)ceil_div(rows, kRBlock / 64)), dim3(kRBlock), 0, stream(),
+                       y, w, seed, f, dz, rows, cols);
+    return BH_LAUNCH_CHECK("bh_log_softmax_weighted_backward");
 }
 
 int bh_softmax_ce_grad(const float* logits, const int32_t* labels, float* dlogits, float* loss_out, int64_t rows,

@@ -34,6 +34,7 @@ typedef struct boat_op {
     boat_tensor_t* saved[3];     /* per-op saved tensors (layernorm: input, mean, rstd) */
     uint64_t seq;                /* recording order == a topological order */
     uint64_t mark;               /* visit epoch of the backward that last collected it */
+    uint64_t skip;               /* visit epoch of a backward in which a fused rule already covered this op */
 } boat_op_t;
 
 struct boat_variable_t {
@@ -44,6 +45,8 @@ struct boat_variable_t {
     bool grad_shared;            /* grad is a tensor other holders read too: replace it, never add into it */
     boat_op_t* producer;
     size_t refs;
+    uint64_t uses_epoch;         /* the backward walk that last counted ... */
+    unsigned walk_uses;          /* ... how many of its ops read this variable */
     struct boat_variable_t *prev, *next;   /* live-variable list of the library */
 };
 
@@ -658,6 +661,48 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
     }
 }
 
+/* The loss chain of the MNIST example (examples/mnist/mnist_autodiff.c:397-522), loss = f * sum(onehot o log_softmax(z))
+ * with f and onehot constants, recognised at the root of a walk: its four gradient rules (mul :1115-1147, sum :1498-1548,
+ * mul, log-softmax :1975-2068) run as one kernel that keeps their operations and order, so z receives the same bits.
+ * Only when nothing else in the walk reads the intermediate variables and none of them holds a gradient yet; their own
+ * gradients are then not materialised.  Returns true when z's gradient has been accumulated and the four ops are done. */
+static bool fuse_log_softmax_loss(boat_variable_t* root, const boat_tensor_t* seed, uint64_t epoch) {
+    boat_op_t* r = root->producer;
+    if (!r || r->type != OP_MUL || root->data->nelements != 1 || (seed && (!bt_is_f32(seed) || seed->nelements < 1))) return false;
+    boat_variable_t* vf = r->inputs[0]->requires_grad ? r->inputs[1] : r->inputs[0];
+    boat_variable_t* s = r->inputs[0]->requires_grad ? r->inputs[0] : r->inputs[1];
+    if (vf == s || vf->requires_grad || !s->requires_grad || !bt_is_f32(vf->data) || vf->data->nelements != 1) return false;
+    boat_op_t* sum = s->producer;
+    if (!sum || sum->type != OP_SUM || s->walk_uses != 1 || s->grad || s->data->nelements != 1) return false;
+    boat_variable_t* m = sum->inputs[0];
+    boat_op_t* mul = m->producer;
+    if (!mul || mul->type != OP_MUL || m->walk_uses != 1 || m->grad || !m->requires_grad) return false;
+    boat_variable_t* w = mul->inputs[0]->requires_grad ? mul->inputs[1] : mul->inputs[0];
+    boat_variable_t* ls = mul->inputs[0]->requires_grad ? mul->inputs[0] : mul->inputs[1];
+    if (w == ls || w->requires_grad || !ls->requires_grad || !bt_is_f32(w->data) || !bt_same_shape(w->data, ls->data) ||
+        !bt_same_shape(m->data, ls->data))
+        return false;
+    boat_op_t* lsm = ls->producer;
+    if (!lsm || lsm->type != OP_LOG_SOFTMAX || ls->walk_uses != 1 || ls->grad || !bt_is_f32(ls->data) || ls->data->ndim < 1) return false;
+    boat_variable_t* z = lsm->inputs[0];
+    if (!z->requires_grad || !bt_same_shape(z->data, ls->data) || ls->data->nelements == 0) return false;
+    const int64_t cols = ls->data->shape[ls->data->ndim - 1];
+    const int64_t rows = (int64_t)ls->data->nelements / cols;
+    boat_tensor_t* dz = bt_new_like_uninit(z->data);
+    const float* py = dz ? bt_dev_read(ls->data) : NULL;
+    const float* pw = py ? bt_dev_read(w->data) : NULL;
+    const float* pf = pw ? bt_dev_read(vf->data) : NULL;
+    const float* ps = (pf && seed) ? bt_dev_read(seed) : NULL;
+    float* pd = pf ? bt_dev_write(dz) : NULL;
+    if (!pd || (seed && !ps) || !boat_hip_ok(bh_log_softmax_weighted_backward(py, pw, ps, pf, pd, rows, cols), "loss chain backward")) {
+        boat_tensor_free(dz);
+        return false;
+    }
+    r->skip = sum->skip = mul->skip = lsm->skip = epoch;
+    accumulate(z, dz, true);
+    return true;
+}
+
 static int by_seq_desc(const void* x, const void* y) {
     const boat_op_t* a = *(boat_op_t* const*)x;
     const boat_op_t* b = *(boat_op_t* const*)y;
@@ -690,8 +735,8 @@ static void boat_variable_backward_unflushed(boat_variable_t* variable, boat_ten
 static void backward_walk(boat_variable_t* variable, boat_tensor_t* grad_output) {
     if (!variable || !variable->requires_grad) return;
     boat_tensor_t* seed = grad_output;
-    if (!seed) {
-        if (!bt_is_f32(variable->data)) return;
+    if (!seed && !bt_is_f32(variable->data)) return;
+    if (!seed && (!variable->producer || bt_reference_exact())) {   /* (the walk below makes its own when it needs one) */
         seed = ones_like(variable->data);   /* autodiff.c:313-338 */
         if (!seed) return;
     }
@@ -709,16 +754,20 @@ static void backward_walk(boat_variable_t* variable, boat_tensor_t* grad_output)
     const uint64_t epoch = ++g_epoch;
     size_t n = 0, cap = 64, head = 0;
     boat_op_t** ops = (boat_op_t**)malloc(cap * sizeof(*ops));
-    if (!ops) {
-        if (!grad_output) boat_tensor_unref(seed);
-        return;
-    }
+    if (!ops) return;
     variable->producer->mark = epoch;
     ops[n++] = variable->producer;
     while (head < n) {
         boat_op_t* op = ops[head++];
         for (size_t i = 0; i < op->num_inputs; i++) {
             boat_variable_t* in = op->inputs[i];
+            if (in) {
+                if (in->uses_epoch != epoch) {
+                    in->uses_epoch = epoch;
+                    in->walk_uses = 0;
+                }
+                in->walk_uses++;
+            }
             if (!in || !in->requires_grad || !in->producer || in->producer->mark == epoch) continue;
             in->producer->mark = epoch;
             if (n == cap) {
@@ -731,16 +780,26 @@ static void backward_walk(boat_variable_t* variable, boat_tensor_t* grad_output)
         }
     }
     qsort(ops, n, sizeof(*ops), by_seq_desc);
+    /* the example's loss chain at the root: one kernel, and without a grad_output not even the tensor of ones */
+    const bool fused_root = fuse_log_softmax_loss(variable, grad_output, epoch);
+    if (!fused_root && !seed) {
+        seed = bt_is_f32(variable->data) ? ones_like(variable->data) : NULL;   /* autodiff.c:313-338 */
+        if (!seed) {
+            free(ops);
+            return;
+        }
+    }
     /* reverse recording order: every consumer of a variable runs before its producer */
     for (size_t i = 0; i < n; i++) {
         boat_op_t* op = ops[i];
+        if (op->skip == epoch) continue;
         const boat_tensor_t* dy = op == variable->producer ? seed : op->output->grad;
         g_lender = op == variable->producer ? NULL : op->output;
         if (dy) backward_op(op, dy);
     }
     g_lender = NULL;
     free(ops);
-    if (!grad_output) boat_tensor_unref(seed);
+    if (!grad_output && seed) boat_tensor_unref(seed);
 }
 void boat_variable_backward(boat_variable_t* variable, boat_tensor_t* grad_output) {
     boat_variable_backward_unflushed(variable, grad_output);

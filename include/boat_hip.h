@@ -133,6 +133,12 @@ int bh_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);
 int bh_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols);
 int bh_log_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);
 int bh_log_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols);
+/* Backward of the loss chain loss = f * sum(w o log_softmax(z)) as the MNIST example writes it (w = one-hot labels, f = -1/B;
+ * examples/mnist/mnist_autodiff.c:397-522) in one launch: dz_j = c*w_j - expf(y_j) * sum_j c*w_j with c = seed[0]*f[0]
+ * (seed NULL = 1), y = log_softmax(z) from the forward pass.  The operations and their order are those of the four
+ * separate gradient rules (src/autodiff.c:1115-1147, 1498-1548, 1975-2068), so the result is theirs bit for bit. */
+int bh_log_softmax_weighted_backward(const float* y, const float* w, const float* seed, const float* f, float* dz,
+                                     int64_t rows, int64_t cols);
 /* fused replacement of the chain log_softmax -> mul(onehot) -> sum -> mul(-1/B) and its backward
  * (examples/mnist/mnist_autodiff.c:397-522): loss_out[0] = -(1/B) sum onehot*log_softmax(z),
  * dlogits = (softmax(z) - onehot)/B.  labels are class indices. */

@@ -144,6 +144,28 @@ def test_dense_error_paths(boat):
     boat.boat_dense_layer_free(layer)
 
 
+def test_loss_chain_recognised_on_the_tape_gives_the_op_by_op_bits(boat):
+    """The example's loss chain (log_softmax, mul by the one-hot matrix, sum, mul by -1/B) at the root of a backward walk
+    runs as one kernel that keeps the four gradient rules' operations: every gradient and updated parameter of the MLP step
+    equals, bit for bit, what the op-by-op walk gives (reference-exact mode walks op by op; on a chain its results are the
+    default walk's)."""
+    rng = np.random.default_rng(99)
+    x = rng.random((64, 784), dtype=np.float32)
+    labels = rng.integers(0, 10, 64)
+    w1 = rng.uniform(-0.08, 0.08, (784, 128)).astype(np.float32)
+    w2 = rng.uniform(-0.2, 0.2, (128, 10)).astype(np.float32)
+    b1, b2 = np.zeros(128, np.float32), np.zeros(10, np.float32)
+    fused = bc.mlp_ce_adam(boat, x, labels, w1, b1, w2, b2, steps=2)
+    boat.boat_hip_set_reference_exact(1)
+    try:
+        plain = bc.mlp_ce_adam(boat, x, labels, w1, b1, w2, b2, steps=2)
+    finally:
+        boat.boat_hip_set_reference_exact(0)
+    for a, b in zip(fused, plain):
+        for key in a:
+            assert np.array_equal(a[key], b[key]), key
+
+
 @pytest.mark.parametrize("dims,batch,steps", [((20, 16, 10), 8, 3), ((784, 128, 10), 64, 2)])
 def test_mlp_ce_adam_training_steps(boat, oracle, dims, batch, steps):
     """Config 1: MLP 784->128->10, batch 64, forward + boat_variable_backward_full + Adam."""

@@ -249,6 +249,30 @@ def test_softmax_family(hip, oracle, rng, rows, cols):
         assert np.max(np.abs(g.numpy() - gw)) <= TOL_RED * max(1.0, np.abs(gw).max())
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 10), (3, 33), (5, 1), (7, 1000)])
+def test_loss_chain_backward_kernel(hip, oracle, rng, rows, cols):
+    """bh_log_softmax_weighted_backward against the oracle's log-softmax backward of dls = (seed*f)*w and, bit for bit,
+    against the separate kernel on the same dls (the fused kernel keeps the rules' operations), with and without a seed."""
+    z = (3 * rng.standard_normal((rows, cols))).astype(np.float32)
+    y = oracle.log_softmax_forward(z)
+    w = np.zeros((rows, cols), np.float32)
+    w[np.arange(rows), rng.integers(0, cols, rows)] = 1.0
+    w[0] = rng.standard_normal(cols).astype(np.float32)          # any weights, not only one-hot rows
+    f, seed = np.array([-1.0 / rows], np.float32), np.array([0.75], np.float32)
+    dz = hip.empty((rows, cols))
+    for s in (None, seed):
+        c = np.float32((np.float32(1.0) if s is None else s[0]) * f[0])
+        hip.check(hip.bh_log_softmax_weighted_backward(dev(hip, y).ptr, dev(hip, w).ptr, dev(hip, s).ptr if s is not None else None,
+                                                       dev(hip, f).ptr, dz.ptr, rows, cols))
+        dls = (c * w).astype(np.float32)
+        want = oracle.log_softmax_backward(y, dls)
+        got = dz.numpy()
+        assert np.max(np.abs(got - want)) <= TOL_RED * max(1e-6, np.abs(want).max())
+        dchain = hip.empty((rows, cols))
+        hip.check(hip.bh_log_softmax_backward(dev(hip, y).ptr, dev(hip, dls).ptr, dchain.ptr, rows, cols))
+        assert np.array_equal(got, dchain.numpy())
+
+
 @pytest.mark.parametrize("rows,cols", [(64, 10), (8, 10), (5, 130)])
 def test_fused_softmax_ce_matches_tape_chain(hip, oracle, rng, rows, cols):
     z = (2 * rng.standard_normal((rows, cols))).astype(np.float32)

@@ -250,6 +250,30 @@ int bh_memcpy_d2h(void* dst, const void* src, size_t nbytes) {
     if (rc) return rc;
     return check_hip(hipStreamSynchronize(g_stream), "memcpy d2h sync");
 }
+void* bh_host_alloc(size_t nbytes) {
+    if (!ready() && bh_init() != BH_OK) return nullptr;
+    void* p = nullptr;
+    if (hipHostMalloc(&p, nbytes ? nbytes : 1, hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();   /* the caller falls back to pageable memory: not an error of the library */
+        return nullptr;
+    }
+    return p;
+}
+void bh_host_free(void* p) {
+    if (p) (void)hipHostFree(p);
+}
+int bh_memcpy_h2d_async(void* dst, const void* src, size_t nbytes) {
+    BH_REQUIRE_INIT();
+    if (nbytes == 0) return BH_OK;
+    BH_CHECK_ARG(dst && src, "null pointer");
+    return check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, g_stream), "memcpy h2d (queued)");
+}
+int bh_memcpy_d2h_async(void* dst, const void* src, size_t nbytes) {
+    BH_REQUIRE_INIT();
+    if (nbytes == 0) return BH_OK;
+    BH_CHECK_ARG(dst && src, "null pointer");
+    return check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, g_stream), "memcpy d2h (queued)");
+}
 int bh_memcpy_d2d(void* dst, const void* src, size_t nbytes) {
     BH_REQUIRE_INIT();
     if (nbytes == 0) return BH_OK;

@@ -16,6 +16,11 @@ typedef struct boat_storage {
     size_t refs;
     bool exposed;          /* coherent-pointer mode: the caller holds the host pointer and may use it at any time */
     bool pending;          /* coherent-pointer mode: written on the device since the last write-back to the host */
+    void* shadow;          /* coherent-pointer mode: page-locked copy of what host mirror and device buffer both held
+                              at their last transfer; a host mirror that still equals it was not written by the caller,
+                              so the device copy is current without an upload; transfers are staged through it */
+    bool shadow_valid;
+    uint64_t upload_ticket;   /* the queued upload from `shadow` that must have run before shadow is written again */
 } boat_storage_t;
 
 struct boat_tensor_t {

@@ -334,8 +334,10 @@ static boat_tensor_t* tensor_alloc(const int64_t* shape, size_t ndim, boat_dtype
     return t;
 }
 
+static void shadow_release(boat_storage_t* st);
 static void storage_unref(boat_storage_t* st) {
     if (--st->refs > 0) return;
+    shadow_release(st);
     free(st->host);
     if (st->dev) bh_buffer_unref(st->dev);
     stats_free(st->nbytes);
@@ -394,7 +396,36 @@ void boat_hip_set_coherent_pointers(int enable) {
     g_coherent = enable != 0;
 }
 
+/* ---- the shadow of an exposed storage ----
+ * Without it every device read of an exposed tensor has to upload the host mirror (the caller may have written) and wait,
+ * and every write-back waits per tensor.  With it a read costs one memcmp of the mirror against the shadow (equal: the
+ * device copy is current), an upload is a memcpy into the shadow plus a queued copy that nobody waits for, and the
+ * write-backs of one call share one wait.  Page-locked memory is finite: storages above kShadowLimit keep the plain path. */
+static const size_t kShadowLimit = (size_t)256 << 20;
+static uint64_t g_ticket = 0, g_synced_ticket = 0;   /* queued uploads issued / known to have completed */
+
+static void stream_synced(void) { g_synced_ticket = g_ticket; }
+static bool shadow_ensure(boat_storage_t* st) {
+    if (st->shadow) return true;
+    if (!st->exposed || st->nbytes == 0 || st->nbytes > kShadowLimit) return false;
+    st->shadow = bh_host_alloc(st->nbytes);
+    st->shadow_valid = false;
+    return st->shadow != NULL;
+}
+/* the shadow is about to be written (or freed): a queued upload out of it must have run */
+static void shadow_settle(boat_storage_t* st) {
+    if (st->shadow && st->upload_ticket > g_synced_ticket && bh_synchronize() == BH_OK) stream_synced();
+}
+static void shadow_release(boat_storage_t* st) {
+    if (!st->shadow) return;
+    shadow_settle(st);
+    bh_host_free(st->shadow);
+    st->shadow = NULL;
+    st->shadow_valid = false;
+}
+
 static void mark_device_write(boat_storage_t* st) {
+    st->shadow_valid = false;
     if (!st->exposed || st->pending) return;
     if (g_pending_n == g_pending_cap) {
         const size_t cap = g_pending_cap ? 2 * g_pending_cap : 64;
@@ -409,12 +440,37 @@ static void mark_device_write(boat_storage_t* st) {
 }
 
 void bt_flush_exposed(void) {
+    if (g_pending_n == 0) return;
+    /* storages with a shadow: all copies queued, one wait, then shadow -> mirror; the others one waiting copy each */
+    size_t queued = 0;
+    for (size_t i = 0; i < g_pending_n; i++) {
+        boat_storage_t* st = g_pending[i];
+        st->pending = false;
+        if (!(st->refs > 1 && st->host && st->dev && st->dev_valid && !st->host_valid)) continue;
+        if (shadow_ensure(st)) {
+            shadow_settle(st);
+            if (boat_hip_ok(bh_memcpy_d2h_async(st->shadow, bh_buffer_ptr(st->dev), st->nbytes), "write-back of an exposed tensor")) {
+                st->pending = true;   /* marks: copy queued */
+                queued++;
+                continue;
+            }
+        }
+        if (boat_hip_ok(bh_memcpy_d2h(st->host, bh_buffer_ptr(st->dev), st->nbytes), "write-back of an exposed tensor")) {
+            st->host_valid = true;
+            stream_synced();
+        }
+    }
+    const bool landed = queued > 0 && boat_hip_ok(bh_synchronize(), "write-back of exposed tensors");
+    if (landed) stream_synced();
     while (g_pending_n > 0) {
         boat_storage_t* st = g_pending[--g_pending_n];
-        st->pending = false;
-        if (st->refs > 1 && st->host && st->dev && st->dev_valid && !st->host_valid) {
-            if (boat_hip_ok(bh_memcpy_d2h(st->host, bh_buffer_ptr(st->dev), st->nbytes), "write-back of an exposed tensor"))
+        if (st->pending) {
+            st->pending = false;
+            if (landed) {
+                memcpy(st->host, st->shadow, st->nbytes);
                 st->host_valid = true;
+                st->shadow_valid = true;
+            }
         }
         storage_unref(st);
     }
@@ -429,6 +485,11 @@ static bool storage_host_ready(boat_storage_t* st) {
     if (!st->host_valid) {
         if (st->dev_valid) {
             if (!boat_hip_ok(bh_memcpy_d2h(st->host, bh_buffer_ptr(st->dev), st->nbytes), "tensor download")) return false;
+            stream_synced();
+            if (st->shadow) {          /* mirror and device agree again: so does the shadow */
+                memcpy(st->shadow, st->host, st->nbytes);
+                st->shadow_valid = true;
+            }
         } else {
             memset(st->host, 0, st->nbytes);
         }
@@ -447,11 +508,22 @@ static bool storage_dev_ready(boat_storage_t* st, bool need_contents) {
         }
         if (zero) st->dev_valid = true;
     }
-    /* an exposed tensor may have been written through the caller's pointer since the last upload */
-    if (need_contents && st->exposed && !st->pending && st->host_valid) st->dev_valid = false;
+    /* an exposed tensor may have been written through the caller's pointer since the last upload: it was not if the
+     * mirror still equals the shadow, the copy of what was uploaded or written back last */
+    if (need_contents && st->exposed && !st->pending && st->host_valid &&
+        !(st->dev_valid && st->shadow && st->shadow_valid && memcmp(st->host, st->shadow, st->nbytes) == 0))
+        st->dev_valid = false;
     if (need_contents && !st->dev_valid) {
-        if (st->host_valid) {
+        if (st->host_valid && shadow_ensure(st)) {
+            /* staged: the caller may overwrite the mirror as soon as this call returns, the queued copy reads the shadow */
+            shadow_settle(st);
+            memcpy(st->shadow, st->host, st->nbytes);
+            if (!boat_hip_ok(bh_memcpy_h2d_async(bh_buffer_ptr(st->dev), st->shadow, st->nbytes), "tensor upload")) return false;
+            st->upload_ticket = ++g_ticket;
+            st->shadow_valid = true;
+        } else if (st->host_valid) {
             if (!boat_hip_ok(bh_memcpy_h2d(bh_buffer_ptr(st->dev), st->host, st->nbytes), "tensor upload")) return false;
+            stream_synced();
         } else {
             if (!boat_hip_ok(bh_memset_zero(bh_buffer_ptr(st->dev), st->nbytes), "tensor zero fill")) return false;
         }
@@ -522,7 +594,8 @@ void* bt_host_rw(boat_tensor_t* tensor) {
     boat_storage_t* st = tensor->st;
     if (tensor->device == BOAT_DEVICE_HIP) return bt_dev_rw(tensor);
     if (!storage_host_ready(st)) return NULL;
-    st->dev_valid = false;   /* written through the pointer */
+    /* written through the pointer -- unless a shadow will tell whether it really was */
+    if (!(st->exposed && st->shadow && st->shadow_valid)) st->dev_valid = false;
     return (char*)st->host + tensor->offset;
 }
 void* boat_tensor_data(const boat_tensor_t* tensor) {

@@ -29,6 +29,7 @@ _SIGS = {
     "bh_bytes_in_use": (Z, []), "bh_bytes_cached": (Z, []),
     "bh_buffer_create": (P, [Z, I]), "bh_buffer_ref": (None, [P]), "bh_buffer_unref": (None, [P]),
     "bh_buffer_ptr": (P, [P]), "bh_buffer_nbytes": (Z, [P]), "bh_buffer_refcount": (I, [P]),
+    "bh_host_alloc": (P, [Z]), "bh_host_free": (None, [P]), "bh_memcpy_h2d_async": (I, [P, P, Z]), "bh_memcpy_d2h_async": (I, [P, P, Z]),
     "bh_memcpy_h2d": (I, [P, P, Z]), "bh_memcpy_d2h": (I, [P, P, Z]), "bh_memcpy_d2d": (I, [P, P, Z]),
     "bh_memset_zero": (I, [P, Z]),
     "bh_event_create": (P, []), "bh_event_destroy": (None, [P]), "bh_event_record": (I, [P]),

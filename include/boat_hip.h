@@ -55,6 +55,13 @@ int bh_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes);
 int bh_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes);   /* waits for the stream */
 int bh_memcpy_d2d(void* dst_dev, const void* src_dev, size_t nbytes);
 int bh_memset_zero(void* dst_dev, size_t nbytes);
+/* page-locked host memory (hipHostMalloc) and copies to and from it that are queued on the stream and do NOT wait: the
+ * host side of a transfer the library stages itself (src/core/memory.c:46-247 is the reference's allocator seam; it has
+ * no device).  The memory must stay untouched until the stream has passed the copy (bh_synchronize). */
+void* bh_host_alloc(size_t nbytes);
+void  bh_host_free(void* p);
+int bh_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t nbytes);
+int bh_memcpy_d2h_async(void* dst_pinned, const void* src_dev, size_t nbytes);
 
 /* events on the library stream, for timing */
 typedef struct bh_event bh_event_t;

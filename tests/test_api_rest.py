@@ -427,6 +427,48 @@ def test_gpu_kept_pointers_in_the_default_configuration(boat):
     boat.boat_tensor_unref(g)
 
 
+@pytest.mark.gpu
+def test_gpu_kept_pointer_batches_are_staged(boat):
+    """The input batch lives behind a kept pointer and is overwritten the moment a forward call returns, while the
+    device may not have run that call yet: each forward must have used the values the mirror held when it was called
+    (uploads are staged through a page-locked copy before the call returns), a mirror that was not touched is not
+    uploaded again, and results written by the device are in the mirror when the writing call returns."""
+    import ctypes as C
+    rng = np.random.default_rng(31)
+    rows, d_in, d_out = 512, 784, 128
+    layer = boat.boat_dense_layer_create(d_in, d_out, True)
+    w = rng.standard_normal((d_in, d_out)).astype(F)
+    boat.write(boat.boat_dense_layer_get_weight(layer), w)
+    x = boat.tensor(np.zeros((rows, d_in), F))
+    xp = np.ctypeslib.as_array(C.cast(boat.boat_tensor_data(x), C.POINTER(C.c_float)), shape=(rows, d_in))
+    batches = [rng.standard_normal((rows, d_in)).astype(F) for _ in range(6)]
+    outs = []
+    for b in batches:
+        xp[:] = b                                          # through the pointer taken once
+        outs.append(boat.boat_dense_layer_forward(layer, x))
+        xp[:] = -7.0                                       # scribbled over before the device has to have run
+    outs.append(boat.boat_dense_layer_forward(layer, x))   # the scribble itself
+    outs.append(boat.boat_dense_layer_forward(layer, x))   # an untouched mirror
+    for b, t in zip(batches, outs):
+        want = b.astype(np.float64) @ w.astype(np.float64)
+        assert np.linalg.norm(boat.numpy(t) - want) <= 1e-5 * np.linalg.norm(want)
+    want = np.full((rows, d_in), -7.0) @ w.astype(np.float64)
+    assert np.linalg.norm(boat.numpy(outs[-2]) - want) <= 1e-5 * np.linalg.norm(want)
+    assert np.array_equal(boat.numpy(outs[-1]), boat.numpy(outs[-2]))
+    # a device write into a tensor behind a kept pointer: in the mirror when boat_add_ returns, and the next read of
+    # the mirror's owner sees a host write made after that
+    a = boat.tensor(np.ones((rows, d_in), F))
+    ap = np.ctypeslib.as_array(C.cast(boat.boat_tensor_data(a), C.POINTER(C.c_float)), shape=(rows, d_in))
+    boat.boat_add_(a, x)                                   # a += x on the device (x holds -7)
+    assert np.all(ap == -6.0)
+    ap[0, 0] = 100.0
+    boat.boat_add_(a, x)
+    assert ap[0, 0] == 93.0 and np.all(ap[1:] == -13.0)
+    for t in outs + [a, x]:
+        boat.boat_tensor_unref(t)
+    boat.boat_dense_layer_free(layer)
+
+
 SLICE_FACTS = {
     "shape": (3, 4), "values": [[8.0, 9.0, 10.0, 11.0], [12.0, 13.0, 14.0, 15.0], [16.0, 17.0, 18.0, 19.0]],
     "is_contiguous": False, "pointer_offset": 32, "nbytes": 48,

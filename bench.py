@@ -279,6 +279,23 @@ def bench_sdpa(hip, steps, warmup):
         "bound": "mfma", "cache_bytes": int(bh_) * S * S * 4,
         "fwd_plus_bwd_ms": round(ms_f + ms_b, 4),
         "fwd_plus_bwd_ms_without_cache": round(out["sdpa_fwd_B8h16S1024D64"]["ms"] + out["sdpa_bwd_B8h16S1024D64"]["ms"], 4)}
+    del cache, q, k, vv, go, o, lse, dq, dk, dv
+    # the other head sizes of the matrix-core kernels at the same sequence length and 8192 floats per token
+    for heads, D in ((64, 128), (256, 32)):
+        q, k, vv, go = (hip.to_device(rng.standard_normal((heads, S, D), dtype=np.float32)) for _ in range(4))
+        o, lse = hip.empty((heads, S, D)), hip.empty((heads, S))
+        dq, dk, dv = hip.empty((heads, S, D)), hip.empty((heads, S, D)), hip.empty((heads, S, D))
+        scale = float(1.0 / np.sqrt(D))
+        ms_f = time_steps(hip, lambda: hip.check(hip.bh_sdpa_forward(q.ptr, k.ptr, vv.ptr, scale, 0, o.ptr, lse.ptr, None, heads, S, D)),
+                          steps, warmup)
+        ms_b = time_steps(hip, lambda: hip.check(hip.bh_sdpa_backward(q.ptr, k.ptr, vv.ptr, o.ptr, lse.ptr, go.ptr, scale, 0, dq.ptr,
+                                                                      dk.ptr, dv.ptr, heads, S, D)), steps, warmup)
+        f_fwd = 2 * 2.0 * heads * S * S * D
+        tf_f, tf_b = f_fwd / (ms_f * 1e-3) / 1e12, 2 * f_fwd / (ms_b * 1e-3) / 1e12
+        out[f"sdpa_heads{heads}_S{S}_D{D}"] = {
+            "fwd_ms": round(ms_f, 4), "fwd_achieved_TFLOPs": round(tf_f, 2), "fwd_frac": round(tf_f / PEAK_FP32_MFMA_TFLOPS, 4),
+            "bwd_ms": round(ms_b, 4), "bwd_achieved_TFLOPs": round(tf_b, 2), "bwd_frac": round(tf_b / PEAK_FP32_MFMA_TFLOPS, 4),
+            "bound": "mfma", "fwd_flops": f_fwd, "bwd_credited_flops": 2 * f_fwd}
     return out
 
 

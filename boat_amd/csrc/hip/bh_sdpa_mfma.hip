@@ -1,4 +1,4 @@
-// bh_sdpa_mfma.hip - attention core on the fp32 matrix cores for head_dim 64, any sequence length from 32 up.
+// bh_sdpa_mfma.hip - attention core on the fp32 matrix cores for head_dim 32, 64 and 128, any sequence length from 32 up.
 //
 // Same mathematics as the reference's scaled_dot_product_attention_impl / attention_backward
 // (src/layers/attention.c:997-1073, 1417-1520) on one [s, 64] block per (batch, head):
@@ -23,14 +23,24 @@
 // Any order of the contraction index is a valid sum, so the index order inside a chain is whatever the
 // register layout gives; operands fetched from LDS use 16-byte reads along head_dim (row stride 68
 // floats, conflict free) or 8-byte reads that hand one lane two interleaved output columns.
+// The kernels are templates on the head size D: rows of D + 4 floats in LDS, D / 8 groups of four head-dim values per
+// half-wavefront in every chain over head_dim, D / 32 interleaved 32-column accumulator tiles wherever head_dim is an
+// output index (a lane owns columns NT*lane .. NT*lane + NT - 1).  The reference takes any head_size = hidden / heads
+// (src/layers/attention.c:145-146, 393-397); other sizes than these three use the kernels of bh_sdpa.hip.
 #include "bh_common.h"
 
 namespace bh {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int kD = 64;         // head_dim
-constexpr int kLd = 68;        // LDS row stride in floats (64 + 4 pad)
+// N consecutive floats from LDS (the N interleaved head-dim columns a lane owns)
+template <int N> struct FloatN;
+template <> struct FloatN<1> { float v[1]; __device__ __forceinline__ void load(const float* p) { v[0] = p[0]; }
+                               __device__ __forceinline__ void store(float* p) const { p[0] = v[0]; } };
+template <> struct FloatN<2> { float v[2]; __device__ __forceinline__ void load(const float* p) { const float2 t = *reinterpret_cast<const float2*>(p); v[0] = t.x; v[1] = t.y; }
+                               __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); } };
+template <> struct FloatN<4> { float v[4]; __device__ __forceinline__ void load(const float* p) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+                               __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); } };
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -46,7 +56,8 @@ __device__ __forceinline__ floatx16 zero16() {
 __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + half * 4 + (e & 3); }
 
 // ------------------------------------------------------------------ forward
-// grid (s/128, bh); 4 wavefronts, each owns 32 queries; key/value tiles of 64 rows double-buffered in LDS.
+// grid (s/128, bh); 4 wavefronts, each owns 32 queries; key/value tiles of KT rows double-buffered in LDS (64 rows; 32
+// for head_dim 128, whose 64-row tiles would leave room for one workgroup per compute unit only).
 // EMIT: the scaled scores (log2 units, masked pairs -inf) are also written, transposed ([head][key][query]: a key's row
 // is what a lane of the backward kernel reads), so that the backward pass can skip the Q.K^T recompute.  Under a causal
 // mask the tiles past the diagonal are never visited and their part of the cache stays unwritten.
@@ -54,13 +65,17 @@ __device__ __forceinline__ int acc_row(int e, int half) { return (e >> 2) * 8 + 
 // i.e. two workgroups per compute unit (the LDS allows no more).  Left to itself the compiler gave the causal
 // cache-writing form 244 registers and one wavefront per SIMD; the unmasked cache-writing form is the one that runs faster
 // with its own allocation (300 against 313 us).
-template <bool CAUSAL, bool RAGGED, bool EMIT = false>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
+template <int D, int KT, bool CAUSAL, bool RAGGED, bool EMIT = false>   // RAGGED: s is not a multiple of 128; rows past s are clamped on load, masked, never stored
 __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                             const float* __restrict__ v, float* __restrict__ out,
                                                             float* __restrict__ lse, int s, int n_heads, float scale_log2e,
                                                             float* __restrict__ scores_t) {
+    static_assert(!EMIT || (D == 64 && KT == 64), "the score cache exists for head_dim 64");
     extern __shared__ __align__(16) float smem[];
-    constexpr int KT = 64;                       // keys per tile
+    constexpr int kD = D, kLd = D + 4;           // LDS row stride in floats (4 pad)
+    constexpr int NT = D / 32;                   // 32-row tiles of O^T; a lane's A operand rows are d = NT*lane + tile
+    constexpr int G = D / 8;                     // groups of four head-dim values per half-wavefront
+    constexpr int ST = KT / 32;                  // 32-key tiles of S^T per key/value tile
     constexpr int TILE = KT * kLd;               // floats per K or V tile in LDS
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     // Workgroups are handed out in the order of their linear id.  Read it tile-major: all heads' workgroups of one query
@@ -78,9 +93,9 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
     const int ld_q = RAGGED ? min(my_q, s - 1) : my_q;
 
     // this lane's query row, pre-scaled so that scores come out in log2 units: step (g, e) <-> d = 8g + 4*half + e
-    float qreg[32];
+    float qreg[4 * G];
 #pragma unroll
-    for (int g = 0; g < 8; g++) {
+    for (int g = 0; g < G; g++) {
         const float4 t = *reinterpret_cast<const float4*>(qh + (int64_t)ld_q * kD + 8 * g + 4 * half);
         qreg[4 * g + 0] = t.x * scale_log2e;
         qreg[4 * g + 1] = t.y * scale_log2e;
@@ -88,7 +103,9 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
         qreg[4 * g + 3] = t.w * scale_log2e;
     }
     float* sc_base = EMIT ? scores_t + ((int64_t)head * s + half * 4) * s + my_q : nullptr;
-    floatx16 acc_o[2] = {zero16(), zero16()};    // O^T: [d tile][...]; d = 2*row + tile, query = lane
+    floatx16 acc_o[NT];                          // O^T: [d tile][...]; d = NT*row + tile, query = lane
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc_o[t] = zero16();
     float m_run = -INFINITY, l_run = 0.f;
 
     int n_tiles = RAGGED ? (s + KT - 1) / KT : s / KT;
@@ -96,19 +113,20 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
         const int last = (bx * 128 + 127) / KT + 1;   // tiles that hold a key <= the last query of the workgroup
         if (last < n_tiles) n_tiles = last;
     }
-    // global -> register staging: 1024 float4 per tile and operand, 4 per lane (macros, not lambdas:
+    // global -> register staging: KT * D / 4 float4 per tile and operand, PER per lane (macros, not lambdas:
     // the staging registers must stay registers)
+    constexpr int PER = KT * D / 4 / 256, C4 = D / 4;      // PER is 2 or 4
     float4 kst0, kst1, kst2, kst3, vst0, vst1, vst2, vst3;
 #define FWD_LD(i, K, V)                                                                                   \
-    {                                                                                                     \
-        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+    if constexpr (PER > (i)) {                                                                            \
+        const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
         const int grow = RAGGED ? min(jt_ld * KT + row, s - 1) : jt_ld * KT + row;                        \
         K = *reinterpret_cast<const float4*>(kh + (int64_t)grow * kD + c4 * 4);                           \
         V = *reinterpret_cast<const float4*>(vh + (int64_t)grow * kD + c4 * 4);                           \
     }
 #define FWD_ST(i, K, V)                                                                                   \
-    {                                                                                                     \
-        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+    if constexpr (PER > (i)) {                                                                            \
+        const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
         *reinterpret_cast<float4*>(st_base + row * kLd + c4 * 4) = K;                                     \
         *reinterpret_cast<float4*>(st_base + TILE + row * kLd + c4 * 4) = V;                              \
     }
@@ -126,28 +144,31 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
         const float* vs = ks + TILE;
         // a wavefront whose queries all precede this tile's keys has nothing to add
         if (!CAUSAL || jt * KT <= q0 + 31) {
-            floatx16 acc_s[2] = {zero16(), zero16()};   // S^T: key = row (tile*32 + acc_row), query = lane
+            floatx16 acc_s[ST];                         // S^T: key = row (tile*32 + acc_row), query = lane
+#pragma unroll
+            for (int t = 0; t < ST; t++) acc_s[t] = zero16();
             // the wavefront's priority rises with its progress through the tile (scores 1, softmax 2, O^T 3, 0 around the
             // staging and the barrier): of the two wavefronts that share a SIMD the one nearer to its barrier goes first
             // (measured: 287 -> 273 us unmasked, 175 -> 162 us causal at B8 h16 S1024)
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-            for (int g = 0; g < 8; g++) {
-                const float4 a0 = *reinterpret_cast<const float4*>(ks + r * kLd + 8 * g + 4 * half);
-                const float4 a1 = *reinterpret_cast<const float4*>(ks + (32 + r) * kLd + 8 * g + 4 * half);
-                acc_s[0] = MFMA(a0.x, qreg[4 * g + 0], acc_s[0]);
-                acc_s[1] = MFMA(a1.x, qreg[4 * g + 0], acc_s[1]);
-                acc_s[0] = MFMA(a0.y, qreg[4 * g + 1], acc_s[0]);
-                acc_s[1] = MFMA(a1.y, qreg[4 * g + 1], acc_s[1]);
-                acc_s[0] = MFMA(a0.z, qreg[4 * g + 2], acc_s[0]);
-                acc_s[1] = MFMA(a1.z, qreg[4 * g + 2], acc_s[1]);
-                acc_s[0] = MFMA(a0.w, qreg[4 * g + 3], acc_s[0]);
-                acc_s[1] = MFMA(a1.w, qreg[4 * g + 3], acc_s[1]);
+            for (int g = 0; g < G; g++) {
+                float4 a[ST];
+#pragma unroll
+                for (int t = 0; t < ST; t++) a[t] = *reinterpret_cast<const float4*>(ks + (t * 32 + r) * kLd + 8 * g + 4 * half);
+#pragma unroll
+                for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].x, qreg[4 * g + 0], acc_s[t]);
+#pragma unroll
+                for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].y, qreg[4 * g + 1], acc_s[t]);
+#pragma unroll
+                for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].z, qreg[4 * g + 2], acc_s[t]);
+#pragma unroll
+                for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].w, qreg[4 * g + 3], acc_s[t]);
             }
             __builtin_amdgcn_s_setprio(2);
             float mx = -INFINITY;
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < ST; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
                     if (CAUSAL || RAGGED) {
@@ -161,7 +182,7 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
             const float alpha = exp2f(m_run - m_new);
             float psum = 0.f;
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < ST; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
                     // the score goes to the cache between the exponentials: row (tile's first key + t*32 + 8*(e/4) + e%4) of
@@ -175,19 +196,20 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
             l_run = l_run * alpha + psum;
             m_run = m_new;
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < NT; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc_o[t][e] *= alpha;
             __builtin_amdgcn_s_setprio(3);
             // O^T += V^T . P^T : step e of key tile t uses key row t*32 + acc_row(e, half)
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < ST; t++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) {
                     const int key = t * 32 + acc_row(e, half);
-                    const float2 a = *reinterpret_cast<const float2*>(vs + key * kLd + 2 * r);
-                    acc_o[0] = MFMA(a.x, acc_s[t][e], acc_o[0]);
-                    acc_o[1] = MFMA(a.y, acc_s[t][e], acc_o[1]);
+                    FloatN<NT> a;
+                    a.load(vs + key * kLd + NT * r);
+#pragma unroll
+                    for (int n = 0; n < NT; n++) acc_o[n] = MFMA(a.v[n], acc_s[t][e], acc_o[n]);
                 }
         }
         __builtin_amdgcn_s_setprio(0);
@@ -201,18 +223,19 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
 
     // O = O^T / l, transposed through LDS so that rows are written whole
     const float inv_l = 1.0f / l_run;
-    float* os = smem + w * 32 * kLd;             // 32 x 68 floats per wavefront, tiles are no longer needed
+    float* os = smem + w * 32 * kLd;             // 32 x (D + 4) floats per wavefront, tiles are no longer needed
 #pragma unroll
-    for (int t = 0; t < 2; t++)
+    for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) os[r * kLd + 2 * acc_row(e, half) + t] = acc_o[t][e] * inv_l;
+        for (int e = 0; e < 16; e++) os[r * kLd + NT * acc_row(e, half) + t] = acc_o[t][e] * inv_l;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     float* oh = out + head * s * kD;
+    constexpr int RPI = 64 / C4;                 // rows one pass of the wavefront stores (C4 lanes per row)
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
-        const int row = it * 4 + (lane >> 4), c4 = lane & 15;
+    for (int it = 0; it < 32 / RPI; it++) {
+        const int row = it * RPI + lane / C4, c4 = lane % C4;
         const float4 val = *reinterpret_cast<const float4*>(os + row * kLd + c4 * 4);
         if (!RAGGED || q0 + row < s) *reinterpret_cast<float4*>(oh + (int64_t)(q0 + row) * kD + c4 * 4) = val;
     }
@@ -221,20 +244,23 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
 
 // ----------------------------------------------------------------- backward
 // grid (s/128, bh); 4 wavefronts, each owns 32 keys (dK, dV rows) and loops over query tiles of 32.
-// Two workgroups fit a CU (69 KB of LDS, <= 256 registers per lane), so a SIMD always has a second
-// wavefront to run while one waits at a barrier or on LDS.
+// Two workgroups fit a CU at head_dim 32 and 64 (69 KB of LDS, <= 256 registers per lane), so a SIMD always has a second
+// wavefront to run while one waits at a barrier or on LDS; head_dim 128 (119 KB of LDS, 128 accumulator registers for
+// dK and dV alone) runs one workgroup per compute unit.
 // LDS per workgroup: the 128 K rows, one Q tile and one dO tile (refilled through registers between the
 // two barriers of an iteration), a [32 queries][128 keys] dS tile, and the tile's lse/delta.
 // V never enters LDS: a lane keeps the 32 values of V it feeds to dP = dO.V^T in registers for the
 // whole kernel.
 // dQ = dS.K of a query tile contracts over all 128 keys of the workgroup, so the four wavefronts first
-// publish their dS blocks in LDS and then each computes a [32 queries][16 head-dim columns] slice with
+// publish their dS blocks in LDS and then each computes a [32 queries][D/4 head-dim columns] slice (head_dim 32: a
+// [16 queries][16 columns] quarter) with
 // v_mfma_f32_16x16x4_f32 (as the transposed product, so that a lane holds four consecutive head-dim columns of a query
 // row) and stores it straight to the key tile's partial dQ with 16-byte stores: no cross-wavefront sum.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
 
-struct BwdSmem {
+template <int D> struct BwdSmem {
+    static constexpr int kLd = D + 4;
     static constexpr int K = 128 * kLd;                 // K rows of the workgroup
     static constexpr int QT = 32 * kLd;                 // one Q (or dO) tile
     static constexpr int kDsLd = 132;                   // dS row stride: 128 keys + 4 pad
@@ -249,14 +275,17 @@ struct BwdSmem {
 // RAGGED: rows past s are clamped on load; padding keys are masked, padding queries contribute nothing because their
 // dO rows and delta are staged as zeros; stores are guarded
 // CACHED: the forward pass left the scaled scores (log2 units, [head][key][query]); S = Q.K^T is read instead of recomputed
-template <bool CAUSAL, bool RAGGED, bool CACHED = false>
-__global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
+template <int D, bool CAUSAL, bool RAGGED, bool CACHED = false>
+__global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                const float* __restrict__ v, const float* __restrict__ lse,
                                                                const float* __restrict__ delta, const float* __restrict__ d_out,
                                                                float* __restrict__ dq_partial, float* __restrict__ dk,
                                                                float* __restrict__ dv, int s, int n_heads, float scale,
                                                                int mirror, const float* __restrict__ scores_t) {
+    static_assert(!CACHED || D == 64, "the score cache exists for head_dim 64");
     extern __shared__ __align__(16) float smem[];
+    using Smem = BwdSmem<D>;
+    constexpr int kD = D, kLd = D + 4, NT = D / 32, G = D / 8, C4 = D / 4;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
     // tile-major reading of the linear workgroup id, as in the forward kernel: key tile 0, which meets every query tile
@@ -280,27 +309,28 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     const int kv0 = kv_wg + w * 32;              // first key of this wavefront
     const float c1 = scale * kLog2e;
 
-    float* kall = smem + BwdSmem::OFF_K;         // all 128 K rows
+    float* kall = smem + Smem::OFF_K;         // all 128 K rows
     float* ks = kall + w * 32 * kLd;             // this wavefront's 32
-    float* qs = smem + BwdSmem::OFF_Q;
-    float* gs = smem + BwdSmem::OFF_DO;
-    float* dsb = smem + BwdSmem::OFF_DS;
-    float* st = smem + BwdSmem::OFF_STAT;
-    // this wavefront's K rows -> LDS (each lane: 8 float4)
+    float* qs = smem + Smem::OFF_Q;
+    float* gs = smem + Smem::OFF_DO;
+    float* dsb = smem + Smem::OFF_DS;
+    float* st = smem + Smem::OFF_STAT;
+    // this wavefront's K rows -> LDS (each lane: D/8 float4)
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int idx = lane + i * 64, row = idx >> 4, c4 = idx & 15;
+    for (int i = 0; i < G; i++) {
+        const int idx = lane + i * 64, row = idx / C4, c4 = idx % C4;
         const int grow = RAGGED ? min(kv0 + row, s - 1) : kv0 + row;
         *reinterpret_cast<float4*>(ks + row * kLd + c4 * 4) = *reinterpret_cast<const float4*>(kh + (int64_t)grow * kD + c4 * 4);
     }
-    // this lane's slice of V: key kv0 + r, head-dim 8g + 4*half .. +3 for g = 0..7
-    float4 vreg[8];
+    // this lane's slice of V: key kv0 + r, head-dim 8g + 4*half .. +3 for g = 0..G-1
+    float4 vreg[G];
 #pragma unroll
-    for (int g = 0; g < 8; g++)
+    for (int g = 0; g < G; g++)
         vreg[g] = *reinterpret_cast<const float4*>(vh + (int64_t)(RAGGED ? min(kv0 + r, s - 1) : kv0 + r) * kD + 8 * g + 4 * half);
 
-    floatx16 acc_dk[2] = {zero16(), zero16()};   // [d tile]: key = acc_row, d = 2*lane + tile
-    floatx16 acc_dv[2] = {zero16(), zero16()};
+    floatx16 acc_dk[NT], acc_dv[NT];             // [d tile]: key = acc_row, d = NT*lane + tile
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc_dk[t] = acc_dv[t] = zero16();
 
     const int n_qt = RAGGED ? (s + 31) / 32 : s / 32;
     const int first_qt = CAUSAL ? kv_wg / 32 : 0;   // earlier query tiles see none of this workgroup's keys
@@ -308,27 +338,28 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     if (!mirror)
         for (int i = tid; i < first_qt * 32 * (kD / 4); i += 256)
             reinterpret_cast<float4*>(dqh)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    // staging: a Q tile and a dO tile are 512 float4 each, 2 per lane and operand
-    float4 qst0, qst1, gst0, gst1;
+    // staging: a Q tile and a dO tile are 8 * D float4 each, D / 32 per lane and operand
+    constexpr int PERQ = D / 32;       // 1, 2 or 4
+    float4 qst0, qst1, qst2, qst3, gst0, gst1, gst2, gst3;
     float stat = 0.f;
-#define BWD_LD(i, Q, G)                                                                                   \
-    {                                                                                                     \
-        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+#define BWD_LD(i, Q, G_)                                                                                  \
+    if constexpr (PERQ > (i)) {                                                                           \
+        const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
         const int grow = RAGGED ? min(qt_ld * 32 + row, s - 1) : qt_ld * 32 + row;                        \
         Q = *reinterpret_cast<const float4*>(qh + (int64_t)grow * kD + c4 * 4);                           \
-        G = *reinterpret_cast<const float4*>(gh + (int64_t)grow * kD + c4 * 4);                           \
-        if (RAGGED && qt_ld * 32 + row >= s) G = make_float4(0.f, 0.f, 0.f, 0.f);                         \
+        G_ = *reinterpret_cast<const float4*>(gh + (int64_t)grow * kD + c4 * 4);                          \
+        if (RAGGED && qt_ld * 32 + row >= s) G_ = make_float4(0.f, 0.f, 0.f, 0.f);                        \
     }
-#define BWD_ST(i, Q, G)                                                                                   \
-    {                                                                                                     \
-        const int idx = tid + (i) * 256, row = idx >> 4, c4 = idx & 15;                                   \
+#define BWD_ST(i, Q, G_)                                                                                  \
+    if constexpr (PERQ > (i)) {                                                                           \
+        const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
         *reinterpret_cast<float4*>(qs + row * kLd + c4 * 4) = Q;                                          \
-        *reinterpret_cast<float4*>(gs + row * kLd + c4 * 4) = G;                                          \
+        *reinterpret_cast<float4*>(gs + row * kLd + c4 * 4) = G_;                                         \
     }
 #define BWD_STAGE_LOAD(QT)                                                 \
     {                                                                      \
         const int qt_ld = (QT);                                            \
-        BWD_LD(0, qst0, gst0) BWD_LD(1, qst1, gst1)                        \
+        BWD_LD(0, qst0, gst0) BWD_LD(1, qst1, gst1) BWD_LD(2, qst2, gst2) BWD_LD(3, qst3, gst3)                    \
         if (tid < 32) stat = lh[RAGGED ? min(qt_ld * 32 + tid, s - 1) : qt_ld * 32 + tid] * kLog2e;                \
         else if (tid < 64) {                                                                                       \
             stat = dh[RAGGED ? min(qt_ld * 32 + tid - 32, s - 1) : qt_ld * 32 + tid - 32];                         \
@@ -337,7 +368,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     }
 #define BWD_STAGE_STORE()                                                  \
     {                                                                      \
-        BWD_ST(0, qst0, gst0) BWD_ST(1, qst1, gst1)                        \
+        BWD_ST(0, qst0, gst0) BWD_ST(1, qst1, gst1) BWD_ST(2, qst2, gst2) BWD_ST(3, qst3, gst3)                    \
         if (tid < 64) st[tid] = stat;                                      \
     }
     if (first_qt < n_qt) {
@@ -365,7 +396,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
             for (int j = 0; j < 4; j++) sc_next[j] = *reinterpret_cast<const float4*>(sc_row + (qt + 1) * 32 + 8 * j + 4 * half);
         }
         const int q0 = qt * 32;
-        if (!CAUSAL || q0 + 31 >= kv0) {
+        // (head_dim 128 takes no branch here: with 128 accumulator registers flowing around it the kernel would not fit
+        // the register file; the masked pairs of the few tiles it would skip contribute exact zeros)
+        if (D == 128 || !CAUSAL || q0 + 31 >= kv0) {
             // S = Q.K^T and dP = dO.V^T : query = row (acc_row), key = lane
             floatx16 acc_s = zero16(), acc_dp = zero16();
             // The wavefront's priority rises with its progress through the iteration (1 here, 2 in the row loop, 3 in
@@ -384,7 +417,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                 }
                 floatx16 acc_dp2 = zero16();     // two chains, so that a product never waits for its predecessor
 #pragma unroll
-                for (int g = 0; g < 8; g++) {
+                for (int g = 0; g < G; g++) {
                     const float4 ag = *reinterpret_cast<const float4*>(gs + r * kLd + 8 * g + 4 * half);
                     const float4 bv = vreg[g];
                     acc_dp = MFMA(ag.x, bv.x, acc_dp);
@@ -396,7 +429,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                 for (int e = 0; e < 16; e++) acc_dp[e] += acc_dp2[e];
             } else {
 #pragma unroll
-                for (int g = 0; g < 8; g++) {
+                for (int g = 0; g < G; g++) {
                     const int off = r * kLd + 8 * g + 4 * half;
                     const float4 aq = *reinterpret_cast<const float4*>(qs + off);
                     const float4 bk = *reinterpret_cast<const float4*>(ks + off);
@@ -424,59 +457,90 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
                 // and delta were staged as zeros, so everything they contribute below is zero)
                 if ((CAUSAL && my_key > q0 + row) || key_pad) p = 0.f;
                 const float ds = p * (acc_dp[e] - st[32 + row]) * scale;
-                dsb[row * BwdSmem::kDsLd + w * 32 + r] = ds;
-                const float2 bg = *reinterpret_cast<const float2*>(gs + row * kLd + 2 * r);
-                const float2 bq = *reinterpret_cast<const float2*>(qs + row * kLd + 2 * r);
-                acc_dv[0] = MFMA(p, bg.x, acc_dv[0]);
-                acc_dv[1] = MFMA(p, bg.y, acc_dv[1]);
-                acc_dk[0] = MFMA(ds, bq.x, acc_dk[0]);
-                acc_dk[1] = MFMA(ds, bq.y, acc_dk[1]);
+                dsb[row * Smem::kDsLd + w * 32 + r] = ds;
+                FloatN<NT> bg, bq;
+                bg.load(gs + row * kLd + NT * r);
+                bq.load(qs + row * kLd + NT * r);
+#pragma unroll
+                for (int t = 0; t < NT; t++) acc_dv[t] = MFMA(p, bg.v[t], acc_dv[t]);
+#pragma unroll
+                for (int t = 0; t < NT; t++) acc_dk[t] = MFMA(ds, bq.v[t], acc_dk[t]);
             }
             __builtin_amdgcn_s_setprio(0);
         } else {
 #pragma unroll
-            for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * BwdSmem::kDsLd + w * 32 + r] = 0.f;
+            for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * Smem::kDsLd + w * 32 + r] = 0.f;
         }
         __syncthreads();   // dS complete; every wavefront is done with the Q and dO tiles
         if (more) BWD_STAGE_STORE()
-        // dQ[32 queries][16w .. 16w+15] = dS[32][128 keys] . K[128][16w ..]; lane (i16, kk) reads four
+        // dQ[32 queries][D] = dS[32][128 keys] . K[128][D] in 16x16 output tiles: a wavefront owns column tiles
+        // ct0 .. ct0+NCT-1 of both 16-row tiles (head_dim 32: one column tile of one row tile); lane (i16, kk) reads four
         // consecutive keys of its dS row at once and feeds them to four successive products (the order
         // of the contraction index is free as long as both operands use the same one)
-        floatx4 acc_dq0 = {0.f, 0.f, 0.f, 0.f}, acc_dq1 = {0.f, 0.f, 0.f, 0.f};
+        constexpr int NCT = D >= 64 ? D / 64 : 1, NRT = D >= 64 ? 2 : 1;
+        const int ct0 = D >= 64 ? w * NCT : (w & 1), rt0 = D >= 64 ? 0 : (w >> 1);
+        floatx4 acc_dq[NCT][NRT];
+#pragma unroll
+        for (int c = 0; c < NCT; c++)
+#pragma unroll
+            for (int t = 0; t < NRT; t++) acc_dq[c][t] = floatx4{0.f, 0.f, 0.f, 0.f};
         __builtin_amdgcn_s_setprio(3);
-        float* dq_row0 = dqh + (int64_t)(q0 + i16) * kD + 16 * w + 4 * kk;
-        float* dq_row1 = dq_row0 + 16 * kD;
-        // mirror launch: what the first launch stored here, in flight while the products below run
-        float4 old0 = make_float4(0.f, 0.f, 0.f, 0.f), old1 = old0;
-        if (mirror) {
-            if (!RAGGED || q0 + i16 < s) old0 = *reinterpret_cast<const float4*>(dq_row0);
-            if (!RAGGED || q0 + 16 + i16 < s) old1 = *reinterpret_cast<const float4*>(dq_row1);
+        float* dq_row0 = dqh + (int64_t)(q0 + 16 * rt0 + i16) * kD + 16 * ct0 + 4 * kk;   // tile (c, t) at + 16*t rows, + 16*c columns
+        // mirror launch (never under a causal mask): what the first launch stored here, in flight while the products below run
+        float4 old[CAUSAL ? 1 : NCT][CAUSAL ? 1 : NRT];
+        if constexpr (!CAUSAL) {
+#pragma unroll
+            for (int c = 0; c < NCT; c++)
+#pragma unroll
+                for (int t = 0; t < NRT; t++) {
+                    old[c][t] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (mirror && (!RAGGED || q0 + 16 * (rt0 + t) + i16 < s))
+                        old[c][t] = *reinterpret_cast<const float4*>(dq_row0 + (int64_t)16 * t * kD + 16 * c);
+                }
         }
         const int g_lim = CAUSAL ? min(8, (q0 + 32 - kv_wg + 15) / 16) : 8;   // keys past the tile's last query are masked
         for (int g = 0; g < g_lim; g++) {
-            const float4 a0 = *reinterpret_cast<const float4*>(dsb + i16 * BwdSmem::kDsLd + 16 * g + 4 * kk);
-            const float4 a1 = *reinterpret_cast<const float4*>(dsb + (16 + i16) * BwdSmem::kDsLd + 16 * g + 4 * kk);
-            const float* kb = kall + (16 * g + 4 * kk) * kLd + 16 * w + i16;
-            const float b0 = kb[0], b1 = kb[kLd], b2 = kb[2 * kLd], b3 = kb[3 * kLd];
+            float4 a[NRT];
+#pragma unroll
+            for (int t = 0; t < NRT; t++) a[t] = *reinterpret_cast<const float4*>(dsb + (16 * (rt0 + t) + i16) * Smem::kDsLd + 16 * g + 4 * kk);
+            float b[NCT][4];
+#pragma unroll
+            for (int c = 0; c < NCT; c++) {
+                const float* kb = kall + (16 * g + 4 * kk) * kLd + 16 * (ct0 + c) + i16;
+                b[c][0] = kb[0]; b[c][1] = kb[kLd]; b[c][2] = kb[2 * kLd]; b[c][3] = kb[3 * kLd];
+            }
             // operands swapped: the product is the transpose dQ^T[d][query], so a lane ends up with four consecutive
             // head-dim columns of one query row and stores them as one 16-byte piece
-            acc_dq0 = MFMA16(b0, a0.x, acc_dq0);
-            acc_dq1 = MFMA16(b0, a1.x, acc_dq1);
-            acc_dq0 = MFMA16(b1, a0.y, acc_dq0);
-            acc_dq1 = MFMA16(b1, a1.y, acc_dq1);
-            acc_dq0 = MFMA16(b2, a0.z, acc_dq0);
-            acc_dq1 = MFMA16(b2, a1.z, acc_dq1);
-            acc_dq0 = MFMA16(b3, a0.w, acc_dq0);
-            acc_dq1 = MFMA16(b3, a1.w, acc_dq1);
+#pragma unroll
+            for (int c = 0; c < NCT; c++)
+#pragma unroll
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][0], a[t].x, acc_dq[c][t]);
+#pragma unroll
+            for (int c = 0; c < NCT; c++)
+#pragma unroll
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][1], a[t].y, acc_dq[c][t]);
+#pragma unroll
+            for (int c = 0; c < NCT; c++)
+#pragma unroll
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][2], a[t].z, acc_dq[c][t]);
+#pragma unroll
+            for (int c = 0; c < NCT; c++)
+#pragma unroll
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][3], a[t].w, acc_dq[c][t]);
         }
         __builtin_amdgcn_s_setprio(0);
-        // accumulator register e of lane (i16, kk) is head-dim column 16w + 4*kk + e of query row i16 of the 16-row tile
-        if (!RAGGED || q0 + i16 < s)
-            *reinterpret_cast<float4*>(dq_row0) =
-                make_float4(acc_dq0[0] + old0.x, acc_dq0[1] + old0.y, acc_dq0[2] + old0.z, acc_dq0[3] + old0.w);
-        if (!RAGGED || q0 + 16 + i16 < s)
-            *reinterpret_cast<float4*>(dq_row1) =
-                make_float4(acc_dq1[0] + old1.x, acc_dq1[1] + old1.y, acc_dq1[2] + old1.z, acc_dq1[3] + old1.w);
+        // accumulator register e of lane (i16, kk) is head-dim column 16*ct + 4*kk + e of query row i16 of the 16-row tile
+#pragma unroll
+        for (int c = 0; c < NCT; c++)
+#pragma unroll
+            for (int t = 0; t < NRT; t++)
+                if (!RAGGED || q0 + 16 * (rt0 + t) + i16 < s) {
+                    float4 o = make_float4(acc_dq[c][t][0], acc_dq[c][t][1], acc_dq[c][t][2], acc_dq[c][t][3]);
+                    if constexpr (!CAUSAL) {
+                        o.x += old[c][t].x; o.y += old[c][t].y; o.z += old[c][t].z; o.w += old[c][t].w;
+                    }
+                    *reinterpret_cast<float4*>(dq_row0 + (int64_t)16 * t * kD + 16 * c) = o;
+                }
         __syncthreads();   // dS tile free again; the next Q and dO tiles are in place
         if (CACHED) {
 #pragma unroll
@@ -494,8 +558,14 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_mfma_kernel(const float* __re
     for (int e = 0; e < 16; e++) {
         const int64_t row = kv0 + acc_row(e, half);
         if (RAGGED && row >= s) continue;
-        *reinterpret_cast<float2*>(dkh + row * kD + 2 * r) = make_float2(acc_dk[0][e], acc_dk[1][e]);
-        *reinterpret_cast<float2*>(dvh + row * kD + 2 * r) = make_float2(acc_dv[0][e], acc_dv[1][e]);
+        FloatN<NT> ok, ov;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            ok.v[t] = acc_dk[t][e];
+            ov.v[t] = acc_dv[t][e];
+        }
+        ok.store(dkh + row * kD + NT * r);
+        ov.store(dvh + row * kD + NT * r);
     }
 }
 
@@ -510,13 +580,38 @@ __global__ __launch_bounds__(256) void dq_partial_sum_kernel(const float* __rest
     __builtin_nontemporal_store(acc, reinterpret_cast<f32x4*>(out) + i);
 }
 
-// head_dim 64; any sequence length from 32 up (a length that is not a multiple of 128 takes the kernels' ragged form)
-static bool mfma_shape(int64_t s, int64_t d) { return d == kD && s >= 32 && s <= (1 << 24); }
+// head_dim 32, 64 or 128; any sequence length from 32 up (a length that is not a multiple of 128 takes the kernels' ragged form)
+static bool mfma_shape(int64_t s, int64_t d) { return (d == 32 || d == 64 || d == 128) && s >= 32 && s <= (1 << 24); }
 // the grids are one-dimensional (tiles * heads workgroups): no 65535 limit on the number of heads
 static bool grid_fits(int64_t s, int64_t bh_count) { return ceil_div(s, 128) * bh_count <= 0x7fffffff && bh_count <= 0x7fffffff; }
 
-// shapes whose scaled scores the forward pass can leave for the backward pass: whole 128-row tiles
-bool sdpa_scores_shape(int64_t s, int64_t d) { return mfma_shape(s, d) && s % 128 == 0; }
+// shapes whose scaled scores the forward pass can leave for the backward pass: head_dim 64, whole 128-row tiles
+bool sdpa_scores_shape(int64_t s, int64_t d) { return d == 64 && mfma_shape(s, d) && s % 128 == 0; }
+
+// one launch of one instantiation; the first call raises the kernel's dynamic LDS limit
+template <int D, int KT, bool CAUSAL, bool RAGGED, bool EMIT>
+static int fwd_launch(dim3 grid, const float* q, const float* k, const float* v, float* out, float* lse, int s, int heads, float sl,
+                      float* scores_t) {
+    constexpr size_t lds = sizeof(float) * 2 * 2 * KT * (D + 4);
+    static bool attr = false;
+    if (!attr) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<D, KT, CAUSAL, RAGGED, EMIT>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr = true;
+    }
+    hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<D, KT, CAUSAL, RAGGED, EMIT>), grid, dim3(256), lds, stream(), q, k, v, out, lse, s, heads, sl,
+                       scores_t);
+    return BH_LAUNCH_CHECK("sdpa_fwd_mfma_kernel");
+}
+template <int D, int KT>
+static int fwd_dispatch(dim3 grid, bool causal, bool ragged, const float* q, const float* k, const float* v, float* out, float* lse, int s,
+                        int heads, float sl) {
+    if (causal && ragged) return fwd_launch<D, KT, true, true, false>(grid, q, k, v, out, lse, s, heads, sl, nullptr);
+    if (causal) return fwd_launch<D, KT, true, false, false>(grid, q, k, v, out, lse, s, heads, sl, nullptr);
+    if (ragged) return fwd_launch<D, KT, false, true, false>(grid, q, k, v, out, lse, s, heads, sl, nullptr);
+    return fwd_launch<D, KT, false, false, false>(grid, q, k, v, out, lse, s, heads, sl, nullptr);
+}
 
 int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scale, int causal, float* out, float* lse,
                       float* scores_t, int64_t bh_count, int64_t s, int64_t d) {
@@ -524,33 +619,40 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
     if (scores_t && !sdpa_scores_shape(s, d)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(out)) return 1;
-    constexpr size_t lds = sizeof(float) * 2 * 2 * 64 * kLd;
-    static bool attr = false;
-    if (!attr) {
-        const void* fns[6] = {reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, false>),
-                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, false>),
-                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, true>),
-                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, true>),
-                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<false, false, true>),
-                              reinterpret_cast<const void*>(&sdpa_fwd_mfma_kernel<true, false, true>)};
-        for (const void* fn : fns) {
-            int rc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
-            if (rc) return rc;
-        }
-        attr = true;
-    }
     dim3 grid((unsigned)(ceil_div(s, 128) * bh_count));
     const bool ragged = s % 128 != 0;
     const float sl = scale * kLog2e;
-#define FWD_LAUNCH(...) hipLaunchKernelGGL((sdpa_fwd_mfma_kernel<__VA_ARGS__>), grid, dim3(256), lds, stream(), q, k, v, out, lse, (int)s, (int)bh_count, sl, scores_t)
-    if (scores_t && causal) FWD_LAUNCH(true, false, true);
-    else if (scores_t) FWD_LAUNCH(false, false, true);
-    else if (causal && ragged) FWD_LAUNCH(true, true);
-    else if (causal) FWD_LAUNCH(true, false);
-    else if (ragged) FWD_LAUNCH(false, true);
-    else FWD_LAUNCH(false, false);
-#undef FWD_LAUNCH
-    return BH_LAUNCH_CHECK("sdpa_fwd_mfma_kernel");
+    const int si = (int)s, hi = (int)bh_count;
+    if (scores_t)
+        return causal ? fwd_launch<64, 64, true, false, true>(grid, q, k, v, out, lse, si, hi, sl, scores_t)
+                      : fwd_launch<64, 64, false, false, true>(grid, q, k, v, out, lse, si, hi, sl, scores_t);
+    if (d == 32) return fwd_dispatch<32, 64>(grid, causal != 0, ragged, q, k, v, out, lse, si, hi, sl);
+    if (d == 64) return fwd_dispatch<64, 64>(grid, causal != 0, ragged, q, k, v, out, lse, si, hi, sl);
+    return fwd_dispatch<128, 32>(grid, causal != 0, ragged, q, k, v, out, lse, si, hi, sl);
+}
+
+template <int D, bool CAUSAL, bool RAGGED, bool CACHED>
+static int bwd_launch(int64_t grid, int mirror, const float* q, const float* k, const float* v, const float* lse, const float* delta,
+                      const float* d_out, float* partial, float* dk, float* dv, int s, int heads, float scale, const float* scores_t) {
+    constexpr size_t lds = sizeof(float) * BwdSmem<D>::TOTAL;
+    static bool attr = false;
+    if (!attr) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<D, CAUSAL, RAGGED, CACHED>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        attr = true;
+    }
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<D, CAUSAL, RAGGED, CACHED>), dim3((unsigned)grid), dim3(256), lds, stream(), q, k, v, lse, delta,
+                       d_out, partial, dk, dv, s, heads, scale, mirror, scores_t);
+    return BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
+}
+template <int D>
+static int bwd_dispatch(int64_t grid, int mirror, bool causal, bool ragged, const float* q, const float* k, const float* v, const float* lse,
+                        const float* delta, const float* d_out, float* partial, float* dk, float* dv, int s, int heads, float scale) {
+    if (causal && ragged) return bwd_launch<D, true, true, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    if (causal) return bwd_launch<D, true, false, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    if (ragged) return bwd_launch<D, false, true, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    return bwd_launch<D, false, false, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
 }
 
 int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
@@ -560,47 +662,30 @@ int sdpa_backward_mfma(const float* q, const float* k, const float* v, const flo
     if (scores_t && !sdpa_scores_shape(s, d)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(d_out) || !al(dq) || !al(dk) || !al(dv)) return 1;
-    constexpr size_t lds = sizeof(float) * BwdSmem::TOTAL;
-    static bool attr = false;
-    if (!attr) {
-        const void* fns[6] = {reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, false>),
-                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, false>),
-                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, true>),
-                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, true>),
-                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<false, false, true>),
-                              reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<true, false, true>)};
-        for (const void* fn : fns) {
-            int arc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
-            if (arc) return arc;
-        }
-        attr = true;
-    }
     const int key_tiles = (int)ceil_div(s, 128);
     // Two launches that share one set of dQ partials (the second takes the key tiles in mirrored order and adds to what
-    // the first stored) when each launch still puts two workgroups on every compute unit: half as many partials to
-    // write and fold, and each launch is a single round of workgroups that start and finish together instead of two
-    // rounds whose second runs out unevenly.  Not under a causal mask, where a launch would hold tiles of unequal work.
-    const bool two_launches = !causal && key_tiles >= 2 && (int64_t)(key_tiles / 2) * bh_count >= 2 * (int64_t)bh_device_cu_count();
+    // the first stored) when each launch still fills every compute unit with the workgroups it can hold (two; one at
+    // head_dim 128): half as many partials to write and fold, and each launch is a single round of workgroups that start
+    // and finish together instead of two rounds whose second runs out unevenly.  Not under a causal mask, where a launch
+    // would hold tiles of unequal work.
+    const int64_t resident = (d == 128 ? 1 : 2) * (int64_t)bh_device_cu_count();
+    const bool two_launches = !causal && key_tiles >= 2 && (int64_t)(key_tiles / 2) * bh_count >= resident;
     const int tiles = two_launches ? (key_tiles + 1) / 2 : key_tiles;      // dQ partials per head
     const bool ragged = s % 128 != 0;
     const int64_t n = bh_count * s * d;
     float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one partial: dq itself
     if (!partial) return BH_ENOMEM;
-#define BWD_LAUNCH(GRID, MIRROR, ...)                                                                                      \
-    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<__VA_ARGS__>), dim3((unsigned)(GRID)), dim3(256), lds, stream(), q, k, v, lse, delta, \
-                       d_out, partial, dk, dv, (int)s, (int)bh_count, scale, MIRROR, scores_t)
+    const int si = (int)s, hi = (int)bh_count;
     int rc = BH_OK;
     for (int pass = 0; pass < (two_launches ? 2 : 1) && rc == BH_OK; pass++) {
         const int64_t grid = (pass == 0 ? tiles : key_tiles / 2) * bh_count;
-        if (scores_t && causal) BWD_LAUNCH(grid, pass, true, false, true);
-        else if (scores_t) BWD_LAUNCH(grid, pass, false, false, true);
-        else if (causal && ragged) BWD_LAUNCH(grid, pass, true, true);
-        else if (causal) BWD_LAUNCH(grid, pass, true, false);
-        else if (ragged) BWD_LAUNCH(grid, pass, false, true);
-        else BWD_LAUNCH(grid, pass, false, false);
-        rc = BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
+        if (scores_t)
+            rc = causal ? bwd_launch<64, true, false, true>(grid, pass, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale, scores_t)
+                        : bwd_launch<64, false, false, true>(grid, pass, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale, scores_t);
+        else if (d == 32) rc = bwd_dispatch<32>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
+        else if (d == 64) rc = bwd_dispatch<64>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
+        else rc = bwd_dispatch<128>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
     }
-#undef BWD_LAUNCH
     if (tiles > 1) {
         if (rc == BH_OK) {
             const int64_t n4 = n / 4;

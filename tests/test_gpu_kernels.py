@@ -642,7 +642,10 @@ def test_transpose(hip, oracle, rng):
 # ---------------------------------------------------------------- attention
 
 SDPA_SHAPES = [(8, 4, 8), (4, 16, 16), (2, 8, 8), (3, 33, 20), (2, 64, 64), (3, 130, 32), (2, 200, 128), (2, 96, 20), (4, 128, 64), (2, 256, 64), (3, 100, 64),
-               (2, 512, 64), (1, 1024, 64), (2, 32, 64), (2, 77, 64), (1, 129, 64), (2, 191, 64), (1, 1000, 64)]
+               (2, 512, 64), (1, 1024, 64), (2, 32, 64), (2, 77, 64), (1, 129, 64), (2, 191, 64), (1, 1000, 64),
+               # the matrix-core kernels' other head sizes: whole tiles, ragged lengths, the shortest sequence
+               (2, 128, 32), (2, 256, 32), (1, 1024, 32), (3, 77, 32), (2, 32, 32), (1, 513, 32),
+               (2, 128, 128), (2, 384, 128), (1, 1024, 128), (2, 100, 128), (2, 32, 128), (1, 257, 128)]
 
 
 @pytest.mark.parametrize("causal", [0, 1])
@@ -776,17 +779,17 @@ def test_sdpa_score_cache_refuses_other_shapes(hip):
                                               buf.ptr, buf.ptr, buf.ptr, 4, 128, 32))
 
 
-@pytest.mark.parametrize("bh,s", [(512, 384), (512, 300), (256, 512), (600, 256)])
-def test_sdpa_backward_mirrored_second_launch(hip, oracle, rng, bh, s):
+@pytest.mark.parametrize("bh,s,d", [(512, 384, 64), (512, 300, 64), (256, 512, 64), (600, 256, 64), (512, 384, 32), (600, 300, 32),
+                                    (256, 384, 128), (300, 300, 128)])
+def test_sdpa_backward_mirrored_second_launch(hip, oracle, rng, bh, s, d):
     """Enough heads for the unmasked backward to run as two launches that share one set of dQ partials (the second
     takes the key tiles in mirrored order and adds to what the first stored): odd tile counts (the middle tile belongs
     to the first launch), a ragged length, an even count; sampled heads against float64, a second call gives the same
-    bits (nothing of the first call's partials survives into it)."""
-    d = 64
+    bits (nothing of the first call's partials survives into it).  All three head sizes of the matrix-core kernels."""
     q, k, v, go = (rng.standard_normal((bh, s, d), dtype=np.float32) for _ in range(4))
     dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)
     o, lse = hip.empty((bh, s, d)), hip.empty((bh, s))
-    scale = 0.125
+    scale = float(1.0 / np.sqrt(d))
     hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, 0, o.ptr, lse.ptr, None, bh, s, d))
     gq, gk, gv = hip.empty((bh, s, d)), hip.empty((bh, s, d)), hip.empty((bh, s, d))
     hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, dgo.ptr, scale, 0, gq.ptr, gk.ptr, gv.ptr, bh, s, d))

@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="all",
-                    help="comma list of step,dense,adam,ln_gelu,sdpa,mlp,cnn,conv (default all); for profiling one workload at a time. "
+                    help="comma list of step,dense,adam,ln_gelu,sdpa,gemm,mlp,cnn,conv (default all); for profiling one workload at a time. "
                          "Without the step leg the line carries no value/roofline.")
     return ap.parse_args()
 
@@ -297,6 +297,63 @@ def bench_sdpa(hip, steps, warmup):
             "bwd_ms": round(ms_b, 4), "bwd_achieved_TFLOPs": round(tf_b, 2), "bwd_frac": round(tf_b / PEAK_FP32_MFMA_TFLOPS, 4),
             "bound": "mfma", "fwd_flops": f_fwd, "bwd_credited_flops": 2 * f_fwd}
     return out
+
+
+def bench_gemm_choice(hip):
+    """The tile / split choice of bh_gemm away from the headline block's shapes: the nine GEMMs of a pre-LN block with
+    8192 rows at d_model 512 and at d_model 2048 (projection and both FFN layers: forward, dX, dW), each timed as the
+    library chooses and with every tile shape forced at 1, 2, 4, 8 and 16 cuts of the contraction; `ratio` is chosen / best
+    forced (1.0 = the cost model found the fastest tile)."""
+    rng = np.random.default_rng(20250110)
+    rows = 8192
+    nmax = rows * 4 * 2048
+    A = hip.to_device(rng.standard_normal((nmax,), dtype=np.float32))
+    B = hip.to_device(rng.standard_normal((nmax,), dtype=np.float32))
+    Cc = hip.empty((nmax,))
+
+    def timed(fn, n=10):
+        warm_clocks(hip.synchronize, fn, 3)
+        t = hip.Timer()
+        with t:
+            for _ in range(n):
+                fn()
+        hip.synchronize()
+        return t.ms / n
+
+    out = {}
+    worst = 0.0
+    for d in (512, 2048):
+        cases = [("proj_fwd", 0, 0, rows, d, d), ("proj_dx", 0, 1, rows, d, d), ("proj_dw", 1, 0, d, d, rows),
+                 ("ffn1_fwd", 0, 0, rows, 4 * d, d), ("ffn1_dx", 0, 1, rows, d, 4 * d), ("ffn1_dw", 1, 0, d, 4 * d, rows),
+                 ("ffn2_fwd", 0, 0, rows, d, 4 * d), ("ffn2_dx", 0, 1, rows, 4 * d, d), ("ffn2_dw", 1, 0, 4 * d, d, rows)]
+        for name, ta, tb, m, n, k in cases:
+            def run():
+                hip.check(hip.bh_gemm(ta, tb, m, n, k, A.ptr, m if ta else k, B.ptr, k if tb else n, Cc.ptr, n, None, 0, 1))
+            chosen = timed(run)
+            best, best_cfg = 1e9, None
+            try:
+                for cfg in (1, 2, 3, 4):
+                    hip.bh_gemm_force_config(cfg)
+                    tiles = -(-m // (256 if cfg in (2, 3) else 128)) * -(-n // (256 if cfg in (2, 4) else 128))
+                    for sp in (1, 2, 4, 8, 16):
+                        if sp > 1 and (tiles * sp > 2048 or k // sp < 128):
+                            continue
+                        hip.bh_gemm_force_splits(sp)
+                        t = timed(run, 6)
+                        if t < best:
+                            best, best_cfg = t, f"tile{cfg}x{sp}"
+            finally:
+                hip.bh_gemm_force_config(-1)
+                hip.bh_gemm_force_splits(0)
+            chosen = min(chosen, timed(run))
+            tf = 2.0 * m * n * k / (chosen * 1e-3) / 1e12
+            ratio = chosen / best
+            worst = max(worst, ratio)
+            out[f"d{d}_{name}"] = {"m": m, "n": n, "k": k, "ms": round(chosen, 4), "TFLOPs": round(tf, 1),
+                                   "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4), "best_forced": best_cfg, "best_forced_ms": round(best, 4),
+                                   "ratio": round(ratio, 3)}
+    out["worst_ratio"] = round(worst, 3)
+    return {"gemm_choice_blocks_d512_d2048": out}
 
 
 def bench_mlp_step(steps, warmup):
@@ -749,7 +806,7 @@ def main():
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build (the path has no inter-GPU work)",
               file=sys.stderr)
         sys.exit(2)
-    all_legs = ["step", "dense", "adam", "ln_gelu", "sdpa", "mlp", "cnn", "conv"]
+    all_legs = ["step", "dense", "adam", "ln_gelu", "sdpa", "gemm", "mlp", "cnn", "conv"]
     legs = all_legs if args.legs == "all" else [l.strip() for l in args.legs.split(",") if l.strip()]
     unknown = [l for l in legs if l not in all_legs]
     if unknown:
@@ -789,6 +846,8 @@ def main():
         extra.update(bench_ln_gelu(hip, args.steps, args.warmup))
     if "sdpa" in legs:
         extra.update(bench_sdpa(hip, args.steps, args.warmup))
+    if "gemm" in legs:
+        extra.update(bench_gemm_choice(hip))
     if "mlp" in legs:
         extra["mlp_784_128_10_step"] = bench_mlp_step(max(args.steps, 20) * 25, max(args.warmup, 1) * 100)
     if "conv" in legs:

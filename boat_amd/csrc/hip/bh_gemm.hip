@@ -1210,6 +1210,87 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
     return BH_LAUNCH_CHECK("splitk_fold_kernel");
 }
 
+// ---- which tile, and how many cuts of the contraction: a cost model instead of a table of shapes ----
+// A workgroup's time is (its share of k) x (us per k of its tile) + a fixed part (launch of the round, first trip to
+// memory, pipeline fill, the store of its tile); a launch takes as many such rounds as the busiest compute unit gets
+// workgroups; a split contraction pays a fold that streams its partials once.  The constants are measured on MI355X
+// (least-squares fit of these constants to a sweep of every tile at 1..32 cuts over 120 shapes from 256 to 8192 in each
+// dimension, two operand layouts: the three eight-wavefront tiles are predicted to 2-3 %, the 128x128 one to 5-8 %):
+//   256x256 (8 wavefronts, one workgroup per CU)   0.2194 us per k, 19.6 us per round
+//   256x128 / 128x256 (8 wavefronts, one per CU)   0.1126 us per k (half the products at 2.6 % less than the big tile's
+//                                                  rate), 10.7 us per round
+//   128x128 (4 wavefronts, two per CU)             two resident workgroups take turns on the matrix cores: 0.0534 us per k
+//                                                  each while they share, 0.0581 for one that has the unit to itself (one
+//                                                  wavefront per SIMD hides less), 10-11 us fixed; workgroups left over
+//                                                  after a full round of 512 are handed to the first units that fall
+//                                                  free, two at a time, so they run at the shared rate on half the chip
+//                                                  (measured so with A stored [k][m]; not with a k-contiguous A)
+//   fold of a cut contraction                      5 us + (cuts + 1) x output bytes at 6.2 TB/s (the partials mostly
+//                                                  still sit in the last-level cache)
+// Padding is paid automatically (a tile costs the same full or not), and so is the quantisation of rounds: 384 big
+// tiles are two rounds, the second half empty, where 768 tiles of half the size are three full ones.
+struct TilePlan {
+    int cfg, splits;
+    double us;
+};
+static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, int64_t splits, bool accumulate, int cus, bool a_kc) {
+    static const int bms[5] = {0, 128, 256, 256, 128}, bns[5] = {0, 128, 256, 128, 256};
+    const int64_t tiles = ceil_div(m, bms[cfg]) * ceil_div(n, bns[cfg]) * batch;
+    const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
+    const int64_t ks = splits > 1 ? ceil_div(ceil_div(k, splits), unit) * unit : k;
+    const int64_t real_splits = splits > 1 ? ceil_div(k, ks) : 1;
+    const int64_t wgs = tiles * real_splits;
+    double us;
+    if (cfg == 1) {
+        const double alone = 0.0581, shared = 0.0534, fixed_alone = 10.9, fixed_shared = 10.3;
+        const int64_t full = wgs / (2 * cus), rest = wgs - full * 2 * cus;
+        us = full * (2 * ks * shared + fixed_shared);
+        // (with a k-contiguous A operand the left-over workgroups were measured spread one per unit after all: 8192x1536x1536,
+        // 768 workgroups, 277-281 us against 367 us with A stored [k][m])
+        if (rest > 0) us += (rest <= cus && (full == 0 || a_kc)) ? ks * alone + fixed_alone : 2 * ks * shared + fixed_shared;
+    } else {
+        const double per_k = cfg == 2 ? 0.2194 : 0.1126, fixed = cfg == 2 ? 19.6 : 10.7;
+        us = ceil_div(wgs, cus) * (ks * per_k + fixed);
+    }
+    if (real_splits > 1) {
+        const double bytes = (double)(real_splits + 1 + (accumulate ? 1 : 0)) * (double)(m * n * batch) * 4.0;
+        us += 5.1 + bytes / 6.2e6;
+    }
+    return us;
+}
+static TilePlan plan_tiles(int64_t m, int64_t n, int64_t k, int64_t batch, bool segmented, bool accumulate, bool a_kc) {
+    int cus = bh_device_cu_count();
+    if (cus <= 0) cus = 256;
+    TilePlan best{1, 1, 1e30};
+    for (int cfg = 1; cfg <= 4; cfg++) {
+        if (cfg == 3 && m < 192) continue;      // a 256-row tile over fewer rows than that is mostly padding ...
+        if (cfg == 4 && n < 192) continue;      // ... and the model's fixed part does not shrink with it
+        if (cfg == 2 && (m < 192 || n < 192)) continue;
+        const int64_t max_splits = segmented ? 1 : (k / 128 < 32 ? (k / 128 < 1 ? 1 : k / 128) : 32);
+        for (int64_t sp = 1; sp <= max_splits; sp++) {
+            const double us = tile_us(cfg, m, n, k, batch, sp, accumulate, cus, a_kc);
+            if (us < best.us * 0.995) best = TilePlan{cfg, (int)sp, us};   // ties go to the earlier (smaller) choice
+        }
+    }
+    return best;
+}
+// the number of cuts the model would choose for a tile shape somebody forced (test hook)
+static int64_t default_splits(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, bool a_kc) {
+    int cus = bh_device_cu_count();
+    if (cus <= 0) cus = 256;
+    double best = 1e30;
+    int64_t best_sp = 1;
+    const int64_t max_splits = k / 128 < 32 ? (k / 128 < 1 ? 1 : k / 128) : 32;
+    for (int64_t sp = 1; sp <= max_splits; sp++) {
+        const double us = tile_us(cfg, m, n, k, batch, sp, false, cus, a_kc);
+        if (us < best * 0.995) {
+            best = us;
+            best_sp = sp;
+        }
+    }
+    return best_sp;
+}
+
 static int g_force_splits = 0;    // test hook: > 0 = this many k-splits for the MFMA tiles
 static int g_pairs = 1;           // test hook: 0 = every tile keeps one k-tile per barrier
 static int g_force_direct = -1;   // test hook: 0 = staged through registers, 1 / -1 = direct to LDS whenever eligible
@@ -1275,48 +1356,14 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     bool vec_ok = al16(a) && al16(b) && (lda % 4 == 0) && (ldb % 4 == 0) && k > 0;
     vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
     int cfg;   // 0 fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256
-    int plan_splits = 0;   // > 0: the tile choice below came with its own number of k-splits
+    int plan_splits = 1;   // k-splits that come with the tile choice
+    const bool segmented = tab && tab->k_segments > 1;     // one product over several operand pairs: never split
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
-        // measured on MI355X (forced-config sweep over the dense, block and attention-projection shapes, operands
-        // streamed straight to LDS): the 256x256 tile wins as soon as it fills the chip once; below that the
-        // eight-wavefront 128x256 / 256x128 tiles (same operand reuse per wavefront, twice the workgroups) beat both
-        // it and the 128x128 tile; narrow outputs keep the small tile
-        const int64_t big_tiles = ceil_div(m, 256) * ceil_div(n, 256);
-        // (a tile shape pays for the rows and columns it pads: 288 rows are two 256-row tiles, 56 % full, but three
-        // 128-row ones, 75 % full -- 288x50176x64, the input gradient's product of a 32-channel 3x3 convolution, takes
-        // 68 us on 256x256 tiles and 53 us on 128x256 ones; the big tile keeps a problem it fills to within 15 % of the others)
-        const auto filled = [&](int64_t bm_, int64_t bn_) {
-            return (double)(m * n) / (double)(ceil_div(m, bm_) * bm_ * ceil_div(n, bn_) * bn_);
-        };
-        const double fill_big = filled(256, 256), fill_other = filled(128, 256) > filled(128, 128) ? filled(128, 256) : filled(128, 128);
-        if (big_tiles >= 256 && fill_big >= 0.85 * fill_other) cfg = 2;
-        else if ((batch == 1 || tab) && m >= 512 && n >= 512 && k >= 4096 && big_tiles * batch < 256 && (256 / (big_tiles * batch)) * 2048 <= k) {
-            // a mid-sized output under a long contraction (the weight gradient of a wide layer): 256x256 tiles with the
-            // contraction cut so that the tiles fill the chip once, at least 2048 k each (4096x1024x8192: 512 us with
-            // the fold against 530 for two-way split 128x256 tiles)
-            cfg = 2;
-            plan_splits = (int)(256 / (big_tiles * batch));
-        } else if ((batch == 1 || tab) && m >= 512 && n >= 512 && k >= 4096 && !(tab && tab->k_segments > 1)) {
-            // smaller still (1024x1024x8192): 128x128 tiles, two workgroups per compute unit, 1024 k each where that
-            // fills the chip (145 us with the fold against 155 for sixteen-way split 128x256 tiles)
-            cfg = 1;
-            const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
-            plan_splits = (int)ceil_div(512, t128);
-            // two of these workgroups share a compute unit, so what counts is an even load per compute unit: the first
-            // count from there on that is a multiple of 256 workgroups (three grouped 1024x1024x8192 products: 4 splits,
-            // 768 workgroups, 388 us with the fold against 402-500 for 3, 5, 6 or 8)
-            for (int s2 = plan_splits; s2 <= 2 * plan_splits && k / s2 >= 1024; s2++)
-                if ((t128 * s2) % 256 == 0) {
-                    plan_splits = s2;
-                    break;
-                }
-            while (plan_splits > 1 && k / plan_splits < 1024) plan_splits--;
-        }
-        else if (n >= 192 && m >= 96) cfg = 4;
-        else if (m >= 192 && n >= 96) cfg = 3;
-        else cfg = 1;
+        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0, a_kc);
+        cfg = plan.cfg;
+        plan_splits = plan.splits;
     }
     // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
     if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
@@ -1338,6 +1385,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
         cfg = 6;
         tiny_split = true;
     }
+    const int cfg_planned = cfg;
     if (g_force_cfg >= 0 && g_force_cfg <= 6 && (vec_ok || g_force_cfg == 0 || g_force_cfg >= 5)) cfg = g_force_cfg;
     if (cfg == 6 && k == 0) cfg = 5;
     if (cfg != 6) tiny_split = false;
@@ -1451,19 +1499,11 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     const int bm = (cfg == 2 || cfg == 3) ? 256 : 128, bn = (cfg == 2 || cfg == 4) ? 256 : 128;
     g.tiles_m = (int)ceil_div(m, bm);
     g.tiles_n = (int)ceil_div(n, bn);
-    // split K when the output alone cannot fill the chip
-    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * batch;
     float* ws = nullptr;
-    // (a handful of tiles with a contraction of a few hundred is latency bound per k-tile: split it finer)
-    const bool few_tiles = tiles <= 8 && k >= 256;
-    const bool segmented = tab && tab->k_segments > 1;     // one product over several operand pairs: never split
-    if (((tiles < 256 && k >= 1024) || few_tiles) && !segmented) {
-        const int64_t min_k = few_tiles && k < 2048 ? 128 : 256;
-        int64_t splits = ceil_div(512, tiles);
-        if (splits > k / min_k) splits = k / min_k;
-        if (splits > 32) splits = 32;
-        if (plan_splits > 0 && g_force_cfg < 0) splits = plan_splits;
+    {
+        int64_t splits = (g_force_cfg >= 1 && g_force_cfg <= 4 && g_force_cfg != cfg_planned) ? default_splits(cfg, m, n, k, batch, a_kc) : plan_splits;
         if (g_force_splits > 0 && g_force_splits <= k / kBK) splits = g_force_splits;
+        if (segmented) splits = 1;
         if (splits > 1) {
             // whole pairs of k-tiles per workgroup where the contraction allows it (the paired main loop needs them)
             const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
@@ -1536,7 +1576,8 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, const flo
 }
 
 // c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g]) for `groups` problems of one shape: one launch where the shape takes the
-// matrix-core tiles with direct loads, the same kernels one after the other otherwise (the same arithmetic either way)
+// matrix-core tiles with direct loads, the same kernels one after the other otherwise (the same products; a long
+// contraction may be cut differently for the group than for a single product)
 int bh_gemm_grouped(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int groups, const float* const* a, int64_t lda,
                     const float* const* b, int64_t ldb, float* const* c, int64_t ldc, const float* const* bias, int accumulate) {
     BH_REQUIRE_INIT();

@@ -204,7 +204,8 @@ int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
 /* Up to 3 products of ONE shape whose operands are separate tensors: c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g]), arguments
  * as bh_gemm with tables of `groups` pointers (bias may be NULL, or hold NULLs).  The three input projections of a
  * self-attention layer (src/layers/attention.c:363-365: the same input times Wq, Wk, Wv) and their three weight gradients
- * (:1186-1285 run three times) are one launch each this way; the arithmetic of every product is that of bh_gemm. */
+ * (:1186-1285 run three times) are one launch each this way, with the kernels of bh_gemm; the number of cuts of a long
+ * contraction is chosen for the group as a whole, so a product agrees with a separate bh_gemm call to fp32 rounding. */
 int bh_gemm_grouped(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int groups,
                     const float* const* a, int64_t lda, const float* const* b, int64_t ldb,
                     float* const* c, int64_t ldc, const float* const* bias, int accumulate);

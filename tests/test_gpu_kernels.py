@@ -507,8 +507,10 @@ def _ptr_table(arrays):
     (40, 24, 12, False, False, False),       # no table kernel for this shape: the groups run one after the other
 ])
 def test_gemm_grouped_equals_separate_launches(hip, rng, force, ta, tb, m, n, k, accumulate, bias, shared_a):
-    """bh_gemm_grouped (three products of one shape in one launch, operands from pointer tables) against float64 and,
-    bit for bit, against the same three products through bh_gemm: the grouped kernels walk each product as bh_gemm does."""
+    """bh_gemm_grouped (three products of one shape in one launch, operands from pointer tables) against float64 and
+    against the same three products through bh_gemm: bit for bit where the contraction is too short to be cut (the grouped
+    kernels walk a product as bh_gemm does), to fp32 rounding otherwise (the number of cuts is chosen for the group as a
+    whole, and partial sums are added in another order)."""
     groups = 3
     a = [rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32) for _ in range(1 if shared_a else groups)]
     if shared_a:
@@ -542,7 +544,10 @@ def test_gemm_grouped_equals_separate_launches(hip, rng, force, ta, tb, m, n, k,
         if accumulate:
             want = want + c0[g]
         assert rel_fro(results[0][g], want) <= fp32_gemm_bound(k), (g, rel_fro(results[0][g], want))
-        assert np.array_equal(results[0][g], results[1][g]), g
+        if k < 256:
+            assert np.array_equal(results[0][g], results[1][g]), g
+        else:
+            assert rel_fro(results[0][g], results[1][g]) <= 2 * fp32_gemm_bound(k), g
 
 
 @pytest.mark.parametrize("force", [None, 1, 2, 3, 4])

@@ -185,6 +185,14 @@ def bench_adam(hip, steps, warmup):
     gbs = 28.0 * n / (ms * 1e-3) / 1e9
     out["adam_flat_268M"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4),
                              "bytes": 28 * n}
+    # the same four read and three written streams with one add each instead of Adam's arithmetic: this memory
+    # pattern's own ceiling on this part (a read-write mix pays for turning the bus around; a plain copy reaches more)
+    ms_probe = time_steps(hip, lambda: hip.check(hip.bh_stream_probe_4r3w(p.ptr, g.ptr, m.ptr, v.ptr, n)), steps, warmup)
+    gbs_probe = 28.0 * n / (ms_probe * 1e-3) / 1e9
+    out["adam_flat_268M"].update(same_pattern_ceiling_ms=round(ms_probe, 4), same_pattern_ceiling_frac=round(gbs_probe / PEAK_HBM_GBS, 4),
+                                 frac_of_same_pattern_ceiling=round(ms_probe / ms, 4))
+    hip.check(hip.bh_memset_zero(m.ptr, 4 * n))
+    hip.check(hip.bh_memset_zero(v.ptr, 4 * n))
     # RMSprop and Adagrad over the same flat arrays (one state tensor: read p, g, state; write p, state = 20 B/param)
     for name, fn in (("rmsprop_flat_268M", lambda: hip.bh_rmsprop_update(p.ptr, g.ptr, m.ptr, n, 1e-3, 0.99, 1e-8)),
                      ("adagrad_flat_268M", lambda: hip.bh_adagrad_update(p.ptr, g.ptr, v.ptr, n, 1e-3, 1e-10))):
@@ -214,6 +222,12 @@ def bench_ln_gelu(hip, steps, warmup):
     gbs = nbytes / (ms * 1e-3) / 1e9
     out["layernorm_bwd_16384x4096"] = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBps": round(gbs, 1),
                                        "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+    # LayerNorm backward's three streams (x and dy read, dx written) without its row structure and arithmetic: an
+    # elementwise add over the same buffers is this pattern's own ceiling
+    ms_probe = time_steps(hip, lambda: hip.check(hip.bh_binary(0, x.ptr, dy.ptr, dx.ptr, R * H)), steps, warmup)
+    out["layernorm_bwd_16384x4096"].update(same_pattern_ceiling_ms=round(ms_probe, 4),
+                                           same_pattern_ceiling_frac=round(3 * 4 * R * H / (ms_probe * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                           frac_of_same_pattern_ceiling=round(ms_probe / ms, 4))
     ms = time_steps(hip, lambda: hip.check(hip.bh_activation_backward(hip.ACT_GELU, x.ptr, dy.ptr, dx.ptr, R * H, 0)), steps, warmup)
     nbytes = 3 * 4 * R * H
     gbs = nbytes / (ms * 1e-3) / 1e9

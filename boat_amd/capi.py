@@ -107,6 +107,7 @@ _SIGS = {
     "boat_relu": (P, [P]),
     "boat_softmax": (P, [P, C.c_int]), "boat_log_softmax": (P, [P, C.c_int]),
     "boat_sum": (P, [P, C.POINTER(C.c_int64), C.c_size_t, C.c_bool]),
+    "boat_can_broadcast": (C.c_bool, [P, P]), "boat_broadcast_to": (P, [P, C.POINTER(C.c_int64), C.c_size_t]),
     "boat_mod": (P, [P, P]), "boat_pow_scalar": (P, [P, C.c_double]),
     "boat_add_scalar_": (None, [P, C.c_double]), "boat_sub_scalar_": (None, [P, C.c_double]),
     "boat_mul_scalar_": (None, [P, C.c_double]), "boat_div_scalar_": (None, [P, C.c_double]),

@@ -120,6 +120,24 @@ __global__ __launch_bounds__(kAdamBlock) void adam_flat_kernel(float* p, const f
     adam_group(p, g, m, v, n, s, (int64_t)blockIdx.x * kAdamBlock + threadIdx.x);
 }
 
+// Adam's memory pattern without Adam's arithmetic (four streams read, three written, one add each): what the same
+// grid of the same workgroups reaches when nothing but the memory system is in the way (benchmark hook)
+__global__ __launch_bounds__(kAdamBlock) void stream_4r3w_kernel(float* __restrict__ p, const float* __restrict__ g,
+                                                                 float* __restrict__ m, float* __restrict__ v, int64_t n4) {
+    const int64_t idx = (int64_t)blockIdx.x * kAdamBlock + threadIdx.x;
+    if (idx >= n4) return;
+    f32x4 pp = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(p) + idx);
+    const f32x4 gg = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(g) + idx);
+    f32x4 mm = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(m) + idx);
+    f32x4 vv = __builtin_nontemporal_load(reinterpret_cast<f32x4*>(v) + idx);
+    pp += gg;
+    mm += gg;
+    vv += gg;
+    __builtin_nontemporal_store(pp, reinterpret_cast<f32x4*>(p) + idx);
+    __builtin_nontemporal_store(mm, reinterpret_cast<f32x4*>(m) + idx);
+    __builtin_nontemporal_store(vv, reinterpret_cast<f32x4*>(v) + idx);
+}
+
 __global__ __launch_bounds__(kAdamBlock) void adam_flat_scalar_kernel(float* p, const float* g, float* m, float* v,
                                                                       int64_t n, AdamScalars s) {
     const int64_t i = (int64_t)blockIdx.x * kAdamBlock + threadIdx.x;
@@ -269,6 +287,20 @@ int bh_adam_update(float* p, const float* g, float* m, float* v, int64_t n, floa
     else
         hipLaunchKernelGGL(adam_flat_scalar_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), p, g, m, v, n, s);
     return BH_LAUNCH_CHECK("bh_adam_update");
+}
+
+// benchmark hook: p += g, m += g, v += g over n floats (n % 4 == 0, 16-byte aligned) with Adam's grid and access pattern
+int bh_stream_probe_4r3w(float* p, const float* g, float* m, float* v, int64_t n) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(n >= 0 && n % 4 == 0, "n must be a multiple of 4");
+    if (n == 0) return BH_OK;
+    BH_CHECK_ARG(p && g && m && v, "null pointer");
+    BH_CHECK_ARG(((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
+                   reinterpret_cast<uintptr_t>(v)) & 15) == 0, "pointers must be 16-byte aligned");
+    const int64_t blocks = blocks_for(n);
+    BH_CHECK_ARG(blocks <= 0x7fffffff, "tensor too large");
+    hipLaunchKernelGGL(stream_4r3w_kernel, dim3((unsigned)blocks), dim3(kAdamBlock), 0, stream(), p, g, m, v, n / 4);
+    return BH_LAUNCH_CHECK("bh_stream_probe_4r3w");
 }
 
 int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m, float* const* v, const int64_t* n,

@@ -425,3 +425,36 @@ boat_tensor_t* boat_hip_mse_loss(const boat_tensor_t* pred, const boat_tensor_t*
     if (grad) *grad = g;
     return loss;
 }
+
+/* arithmetic.c:575-581: whether the two shapes broadcast under the right-aligned rule of :78-104 */
+bool boat_can_broadcast(const boat_tensor_t* a, const boat_tensor_t* b) {
+    if (!a || !b) return false;
+    int64_t shape[BOAT_MAX_DIMS];
+    size_t ndim = 0;
+    return broadcast_shape(a, b, shape, &ndim);
+}
+
+/* arithmetic.c:583-608: the reference does no broadcasting here either -- a new dense tensor of the target shape holding
+ * a's values, and NULL unless the element counts agree */
+boat_tensor_t* boat_broadcast_to(const boat_tensor_t* a, const int64_t* shape, size_t ndim) {
+    if (!a || !shape) return NULL;
+    boat_tensor_t* out = boat_tensor_create(shape, ndim, a->dtype, a->device);
+    if (!out) return NULL;
+    if (out->nelements != a->nelements) {
+        boat_tensor_free(out);
+        return NULL;
+    }
+    if (a->nbytes == 0) return out;
+    boat_tensor_t* copy = boat_tensor_clone(a);
+    if (!copy) {
+        boat_tensor_free(out);
+        return NULL;
+    }
+    /* the clone is dense and owns its payload: hand that payload to the tensor of the new shape */
+    boat_storage_t* st = out->st;
+    out->st = copy->st;
+    copy->st = st;
+    boat_tensor_free(copy);
+    return out;
+}
+

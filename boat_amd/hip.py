@@ -76,6 +76,7 @@ _SIGS = {
     "bh_sdpa_forward_cached": (I, [P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_backward_cached": (I, [P, P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
     "bh_adam_update": (I, [P, P, P, P, L, F, F, F, F, L]),
+    "bh_stream_probe_4r3w": (I, [P, P, P, P, L]),
     "bh_conv2d_forward": (I, [P, P, P, P] + [L] * 8),
     "bh_conv2d_forward_mfma": (I, [P, P, P, P] + [L] * 8),
     "bh_conv2d_backward": (I, [P, P, P, P, P, P] + [L] * 8 + [I, I]),

@@ -154,6 +154,9 @@ BOAT_API boat_tensor_t* boat_gelu(const boat_tensor_t* a);                      
 BOAT_API boat_tensor_t* boat_selu(const boat_tensor_t* a);                          /* returns NULL, as the reference's stub (activation.c:304-308) */
 BOAT_API boat_tensor_t* boat_sum(const boat_tensor_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
 BOAT_API boat_tensor_t* boat_mean(const boat_tensor_t* a, const int64_t* dims, size_t n_dims, bool keepdim);
+/* ---- include/boat/ops.h:107-108 (the shape rule of the elementwise ops, arithmetic.c:575-608) ---- */
+BOAT_API bool boat_can_broadcast(const boat_tensor_t* a, const boat_tensor_t* b);
+BOAT_API boat_tensor_t* boat_broadcast_to(const boat_tensor_t* a, const int64_t* shape, size_t ndim);   /* as the reference: a dense copy under the new shape, equal element counts only */
 
 /* ---- include/boat/autodiff.h:15-98 ---- */
 typedef struct boat_variable_t boat_variable_t;

@@ -280,6 +280,9 @@ int bh_maxpool2d_backward(const float* dy, const int32_t* argmax, float* dx, int
  * timestep is the pre-increment value the reference passes to powf(beta, (float)(t+1)). */
 int bh_adam_update(float* p, const float* g, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, int64_t timestep);
+/* benchmark hook: Adam's four read and three written streams with one add each instead of Adam's arithmetic (p += g,
+ * m += g, v += g; n % 4 == 0, 16-byte aligned pointers): the rate the same grid reaches on this memory pattern */
+int bh_stream_probe_4r3w(float* p, const float* g, float* m, float* v, int64_t n);
 /* one launch over a table of tensors (host arrays of device pointers and element counts) */
 int bh_adam_update_multi(float* const* p, const float* const* g, float* const* m, float* const* v,
                          const int64_t* n, int count,

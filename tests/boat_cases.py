@@ -804,6 +804,13 @@ def tensor_ops(api, a, b, row, col, v1, v2):
         take(name, getattr(api, "boat_" + name)(ta))
     take("softmax", api.boat_softmax(ta, -1))
     take("log_softmax", api.boat_log_softmax(ta, -1))
+    # arithmetic.c:575-608: the shape rule, and boat_broadcast_to (a dense copy under a new shape of equal element count)
+    m, n = np.asarray(a).shape
+    tm = api.tensor(np.zeros(m, np.float32))            # [m] against [m, n]: the last dimensions differ
+    out["can_broadcast"] = [bool(api.boat_can_broadcast(ta, trow)), bool(api.boat_can_broadcast(tcol, ta)), bool(api.boat_can_broadcast(ta, tm))]
+    api.boat_tensor_unref(tm)
+    take("broadcast_to_same_count", api.boat_broadcast_to(ta, (C.c_int64 * 3)(1, n, m), 3))
+    out["broadcast_to_other_count_is_null"] = not api.boat_broadcast_to(trow, (C.c_int64 * 2)(m, n), 2)
     out["is_contiguous"] = bool(api.boat_tensor_is_contiguous(ta))
     out["dtype_names"] = [api.boat_dtype_name(d).decode() for d in (0, 1, 5, 6, 10, 77)]
     out["dtype_sizes"] = [int(api.boat_dtype_size(d)) for d in (0, 1, 5, 6)]

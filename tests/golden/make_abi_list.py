@@ -137,7 +137,9 @@ def main() -> None:
         for line, name, proto in declarations(path.read_text()):
             if any(a <= line <= b for a, b in spans):
                 entries.append({"header": header, "line": line, "name": name, "prototype": proto, "defined": name in defined})
-    OUT.write_text(json.dumps({"cited_ranges": {h: s for h, s in sorted(ranges.items())}, "functions": entries}, indent=1) + "\n")
+    exports = sorted(n for n in defined if n.startswith("boat_"))      # every boat_* function the reference's library defines
+    OUT.write_text(json.dumps({"cited_ranges": {h: s for h, s in sorted(ranges.items())}, "functions": entries, "exports": exports},
+                              indent=1) + "\n")
     print(f"{len(entries)} functions ({sum(e['defined'] for e in entries)} defined by the reference) in {len(ranges)} headers -> {OUT}")
 
 

@@ -46,6 +46,9 @@ def check_tensor_ops(out, stubs_return_null):
     e = np.exp(a64 - a64.max(1, keepdims=True))
     assert np.max(np.abs(out["softmax"] - e / e.sum(1, keepdims=True))) <= 1e-6
     assert np.max(np.abs(out["log_softmax"] - np.log(e / e.sum(1, keepdims=True)))) <= 1e-5
+    assert out["can_broadcast"] == [True, True, False]                      # [5,8] with [8], [5,1] with [5,8], but not [5,8] with [5]
+    assert out["broadcast_to_same_count"].shape == (1, 8, 5) and np.array_equal(out["broadcast_to_same_count"].reshape(-1), a.reshape(-1))
+    assert out["broadcast_to_other_count_is_null"]
     assert out["is_contiguous"] is True
     assert out["dtype_names"] == ["float64", "float32", "int64", "int32", "bool", "unknown"]
     assert out["dtype_sizes"] == [8, 4, 8, 4]

@@ -42,9 +42,14 @@ METRIC = "backward+Adam step ms; GB/s & TFLOP/s as % of MI355X roofline (1 GPU)"
 # FETCH_SIZE 409,880 KiB x 2.000 + WRITE_SIZE 98,304 KiB x 1.000, the factors being what the same counters read for
 # a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).  A constant taken from that profile, not a
 # measurement of this run.
-GEMM_TRAFFIC_BYTES_CONFIG2 = int((2.0 * 409880.2 + 98304.0) * 1024)
+GEMM_TRAFFIC_BYTES_CONFIG2 = int(((2.0 * 779903.4 + 131072.0) + (2.0 * 557368.4 + 65536.0)) / 2 * 1024)
+# the bytes the same two launches need at least: dX reads dY and W and writes dX (335.5 MB), dW reads X and dY, reads and
+# writes dW (402.7 MB)
+GEMM_ALGORITHMIC_BYTES_CONFIG2 = int((335.5e6 + 402.7e6) / 2)
 # HBM bytes per GEMM launch of the block training step, averaged over the step's 18 launches (same file, same counters)
-GEMM_TRAFFIC_BYTES_STEP = 268_700_000
+GEMM_TRAFFIC_BYTES_STEP = 383_400_000
+# what the step's 12 GEMM launches need at least (each operand read once, each output written once): 1,929 MB
+GEMM_ALGORITHMIC_BYTES_STEP = 1_929_000_000 // 12
 
 
 def parse_args():
@@ -136,11 +141,12 @@ def bench_dense_backward(hip, steps, warmup):
         "ms_per_step": ms_per_step,
         "wall_ms_per_step": wall_ms,
         "roofline": {
-            "bound": "mfma", "kernel": "gemm_mfma_kernel (fp32 v_mfma_f32_32x32x2_f32, 256x256 tile, operands direct to LDS)",
+            "bound": "mfma", "kernel": "gemm_mfma_kernel (fp32 v_mfma_f32_32x32x2_f32, tile chosen by the cost model, operands direct to LDS)",
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(gemm_launch_ms, 4), "flops_per_launch": flops_per_launch,
-            "traffic": GEMM_TRAFFIC_BYTES_CONFIG2, "traffic_source": "profile constant (profiles/pmc_hbm_traffic_and_mfma.md), not measured in this run",
+            "traffic": GEMM_TRAFFIC_BYTES_CONFIG2, "algorithmic_bytes": GEMM_ALGORITHMIC_BYTES_CONFIG2,
+            "traffic_source": "profile constant (profiles/pmc_hbm_traffic_and_mfma.md), not measured in this run",
         },
         "step_tflops": round(2 * flops_per_launch / (ms_per_step * 1e-3) / 1e12, 2),
     }
@@ -612,6 +618,7 @@ def bench_training_step(hip, steps, warmup):
     GEMM, attention, LayerNorm, column-sum and optimizer launch inside the timed region is bracketed by its own event
     pair (bh_profile_enable), which gives the dominant kernel family's duration live."""
     block, flat = Block(), FlatAdam(hip)
+    block_probe = hip.zeros(64)
     block.step(keep_loss=True)
     for _ in range(warmup):
         block.step()
@@ -643,10 +650,22 @@ def bench_training_step(hip, steps, warmup):
             flat.step()
     hip.synchronize()
     profiled_ms = profiled.ms / steps
+    # what an event pair reads with nothing between its two events: that much of every recorded call is the measurement
+    empty = [hip.bh_event_create() for _ in range(40)]
+    for i in range(0, 40, 2):
+        hip.check(hip.bh_fill(block_probe.ptr, 0.0, 64))          # something before the pair, as in the step
+        hip.check(hip.bh_event_record(empty[i]))
+        hip.check(hip.bh_event_record(empty[i + 1]))
+    hip.synchronize()
+    pair_ms = float(np.median([hip.bh_event_elapsed_ms(empty[i], empty[i + 1]) for i in range(0, 40, 2)]))
+    for e in empty:
+        hip.bh_event_destroy(e)
     classes = {}
     for name, cls in (("gemm", hip.PROF_GEMM), ("attention_core_fwd", hip.PROF_SDPA_FWD), ("attention_core_bwd", hip.PROF_SDPA_BWD),
                       ("layernorm", hip.PROF_NORM), ("adam", hip.PROF_OPTIMIZER), ("colsum", hip.PROF_COLSUM)):
         ms, work, calls = hip.profile_read(cls)
+        if name != "gemm":          # short kernels: the pair's own reading is a visible share; the headline family keeps the raw sum
+            ms = max(ms - calls * pair_ms, 0.0)
         classes[name] = (ms / steps, work / steps, calls // steps)
     hip.check(hip.bh_profile_enable(0))
     block.step(keep_loss=True)
@@ -667,6 +686,9 @@ def bench_training_step(hip, steps, warmup):
     accounted = sum(ms for ms, _, _ in classes.values())
     breakdown["other_kernels_and_gaps_ms"] = round(ms_per_step - accounted, 4)
     breakdown["ms_per_step_with_launch_events"] = round(profiled_ms, 4)
+    breakdown["empty_event_pair_ms"] = round(pair_ms, 5)
+    breakdown["note"] = ("per-class times are sums over HIP event pairs around each call, minus the reading of an empty pair per call for every "
+                         "class but gemm; profiles/kernel_trace_block.md has the per-kernel medians of a kernel trace")
     flat_gbs = 28.0 * flat.n / (flat_ms * 1e-3) / 1e9
     return {
         "ms_per_step": ms_per_step, "wall_ms_per_step": wall_ms,
@@ -676,7 +698,7 @@ def bench_training_step(hip, steps, warmup):
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(g_ms / max(g_calls, 1), 4), "flops_per_launch": g_flops / max(g_calls, 1),
-            "launches_per_step": g_calls, "traffic": GEMM_TRAFFIC_BYTES_STEP,
+            "launches_per_step": g_calls, "traffic": GEMM_TRAFFIC_BYTES_STEP, "algorithmic_bytes": GEMM_ALGORITHMIC_BYTES_STEP,
             "traffic_source": "profile constant (profiles/pmc_hbm_traffic_and_mfma.md: 2.0 x FETCH_SIZE + WRITE_SIZE per launch, averaged "
                               "over the step's launches), not measured in this run",
             "measured": "HIP event pairs around each bh_gemm launch of K further steps run right after the timed K (the events "

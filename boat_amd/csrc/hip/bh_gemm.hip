@@ -1233,7 +1233,7 @@ struct TilePlan {
     int cfg, splits;
     double us;
 };
-static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, int64_t splits, bool accumulate, int cus, bool a_kc) {
+static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, int64_t splits, bool accumulate, int cus, bool spread_rest) {
     static const int bms[5] = {0, 128, 256, 256, 128}, bns[5] = {0, 128, 256, 128, 256};
     const int64_t tiles = ceil_div(m, bms[cfg]) * ceil_div(n, bns[cfg]) * batch;
     const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
@@ -1246,8 +1246,9 @@ static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, i
         const int64_t full = wgs / (2 * cus), rest = wgs - full * 2 * cus;
         us = full * (2 * ks * shared + fixed_shared);
         // (with a k-contiguous A operand the left-over workgroups were measured spread one per unit after all: 8192x1536x1536,
-        // 768 workgroups, 277-281 us against 367 us with A stored [k][m])
-        if (rest > 0) us += (rest <= cus && (full == 0 || a_kc)) ? ks * alone + fixed_alone : 2 * ks * shared + fixed_shared;
+        // 768 workgroups, 277-281 us against 367 us with A stored [k][m]; and so were those of a grouped launch: three
+        // 1024x1024x8192 weight gradients with A stored [k][m], 768 workgroups at 4 cuts 388 us against 402 at 8)
+        if (rest > 0) us += (rest <= cus && (full == 0 || spread_rest)) ? ks * alone + fixed_alone : 2 * ks * shared + fixed_shared;
     } else {
         const double per_k = cfg == 2 ? 0.2194 : 0.1126, fixed = cfg == 2 ? 19.6 : 10.7;
         us = ceil_div(wgs, cus) * (ks * per_k + fixed);
@@ -1361,7 +1362,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
-        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0, a_kc);
+        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0, a_kc || (tab && batch > 1));
         cfg = plan.cfg;
         plan_splits = plan.splits;
     }

@@ -80,6 +80,57 @@ __global__ __launch_bounds__(kRBlock) void colsum_partial_kernel(const float* __
     partial[(int64_t)blockIdx.y * cols + c] = (a0 + a1) + (a2 + a3);
 }
 
+// the same for up to three matrices of one shape in one launch (blockIdx.z picks the matrix): partial[rb][g*cols + c]
+struct ColsumTab {
+    const float* x[3];
+    float* out[3];
+};
+__global__ __launch_bounds__(kRBlock) void colsum_partial_tab_kernel(ColsumTab t, float* __restrict__ partial, int64_t rows, int64_t cols) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    const float* __restrict__ x = t.x[blockIdx.z];
+    const int64_t step = gridDim.y;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int64_t r = blockIdx.y;
+    for (; r + 3 * step < rows; r += 4 * step) {
+        a0 += x[r * cols + c];
+        a1 += x[(r + step) * cols + c];
+        a2 += x[(r + 2 * step) * cols + c];
+        a3 += x[(r + 3 * step) * cols + c];
+    }
+    for (; r < rows; r += step) a0 += x[r * cols + c];
+    partial[((int64_t)blockIdx.y * gridDim.z + blockIdx.z) * cols + c] = (a0 + a1) + (a2 + a3);
+}
+// folds the row chunks of that launch: column c of matrix g from partial[rb][g][c]; the arithmetic and its order are
+// fold_rows_kernel's (16 row lanes per column, four running sums each, folded through LDS in lane order)
+__global__ __launch_bounds__(kFoldCols * kFoldLanes) void fold_rows_tab_kernel(const float* __restrict__ partial, int64_t nrows, int64_t cols,
+                                                                               int groups, ColsumTab t, int accumulate) {
+    __shared__ float red[kFoldLanes][kFoldCols + 1];
+    const int tx = threadIdx.x % kFoldCols, ty = threadIdx.x / kFoldCols;
+    const int64_t gc = (int64_t)blockIdx.x * kFoldCols + tx;      // column of the [rb][groups * cols] matrix
+    const int64_t ncols = (int64_t)groups * cols;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (gc < ncols) {
+        int64_t r = ty;
+        for (; r + 3 * kFoldLanes < nrows; r += 4 * kFoldLanes) {
+            a0 += partial[r * ncols + gc];
+            a1 += partial[(r + kFoldLanes) * ncols + gc];
+            a2 += partial[(r + 2 * kFoldLanes) * ncols + gc];
+            a3 += partial[(r + 3 * kFoldLanes) * ncols + gc];
+        }
+        for (; r < nrows; r += kFoldLanes) a0 += partial[r * ncols + gc];
+    }
+    red[ty][tx] = (a0 + a1) + (a2 + a3);
+    __syncthreads();
+    if (ty == 0 && gc < ncols) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < kFoldLanes; i++) acc += red[i][tx];
+        float* dst = t.out[gc / cols] + gc % cols;
+        *dst = accumulate ? *dst + acc : acc;
+    }
+}
+
 // ---- row kernels: one wavefront per row, 4 rows per block ----
 // MODE 0 softmax fwd, 1 softmax bwd, 2 log-softmax fwd, 3 log-softmax bwd
 template <int MODE>
@@ -229,6 +280,40 @@ int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumu
                            0, stream(), a, b, out, rows, cols);                                                \
         return BH_LAUNCH_CHECK(name);                                                                          \
     } while (0)
+
+// out[g][c] (+)= sum_r x[g][r][c] for up to three matrices of one shape: one partial launch and one fold where bh_colsum
+// takes two per matrix; the sums and their order are bh_colsum's, so the results are the same bits
+int bh_colsum_grouped(const float* const* x, float* const* out, int groups, int64_t rows, int64_t cols, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(groups >= 1 && groups <= 3 && rows >= 0 && cols >= 0 && x && out, "bad argument");
+    if (cols == 0) return BH_OK;
+    for (int g = 0; g < groups; g++) BH_CHECK_ARG(out[g] && (x[g] || rows == 0), "null pointer");
+    if (groups == 1 || rows <= 256) {
+        for (int g = 0; g < groups; g++) {
+            const int rc = bh_colsum(x[g], out[g], rows, cols, accumulate);
+            if (rc != BH_OK) return rc;
+        }
+        return BH_OK;
+    }
+    ProfScope prof(BH_PROF_COLSUM, 4.0 * (double)rows * (double)cols * groups);
+    const int col_blocks = (int)ceil_div(cols, kRBlock);
+    int64_t chunks = ceil_div(2048, col_blocks);          // per matrix, as bh_colsum cuts it
+    if (chunks > ceil_div(rows, 32)) chunks = ceil_div(rows, 32);
+    if (chunks < 1) chunks = 1;
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * groups * cols));
+    if (!partial) return BH_ENOMEM;
+    ColsumTab t = {};
+    for (int g = 0; g < groups; g++) {
+        t.x[g] = x[g];
+        t.out[g] = out[g];
+    }
+    hipLaunchKernelGGL(colsum_partial_tab_kernel, dim3(col_blocks, (unsigned)chunks, (unsigned)groups), dim3(kRBlock), 0, stream(), t, partial,
+                       rows, cols);
+    hipLaunchKernelGGL(fold_rows_tab_kernel, dim3((unsigned)ceil_div((int64_t)groups * cols, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0, stream(),
+                       partial, chunks, cols, groups, t, accumulate);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK("bh_colsum_grouped");
+}
 
 int bh_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols) {
     BH_ROW_LAUNCH(0, x, (const float*)nullptr, y, "bh_softmax_forward");

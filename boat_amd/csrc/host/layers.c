@@ -799,10 +799,15 @@ static bool project_backward3(boat_attention_t* a, const boat_tensor_t* dqp, con
     else if (ok) ok = boat_hip_ok(bh_gemm_grouped(0, 1, rows, h, h, 3, pdy, h, pw, h, pdx, h, NULL, 0), "attention input gradients");
     /* gw = x^T.dy (overwritten per call, attention.c:1262-1279) */
     if (ok) ok = boat_hip_ok(bh_gemm_grouped(1, 0, h, h, rows, 3, px, h, pdy, h, pgw, h, NULL, 0), "attention weight gradients");
-    /* gb = colsum(dy) */
-    for (int i = 0; i < 3 && ok; i++) {
-        float* pgb = bias[i] ? bt_dev_write(*gb[i]) : NULL;
-        if (bias[i]) ok = pgb && boat_hip_ok(bh_colsum(pdy[i], pgb, rows, h, 0), "attention bias gradient");
+    /* gb = colsum(dy): the three in one pair of launches when all three projections have a bias */
+    if (ok && bias[0] && bias[1] && bias[2]) {
+        float* pgb[3] = {bt_dev_write(*gb[0]), bt_dev_write(*gb[1]), bt_dev_write(*gb[2])};
+        ok = pgb[0] && pgb[1] && pgb[2] && boat_hip_ok(bh_colsum_grouped(pdy, pgb, 3, rows, h, 0), "attention bias gradients");
+    } else {
+        for (int i = 0; i < 3 && ok; i++) {
+            float* pgb = bias[i] ? bt_dev_write(*gb[i]) : NULL;
+            if (bias[i]) ok = pgb && boat_hip_ok(bh_colsum(pdy[i], pgb, rows, h, 0), "attention bias gradient");
+        }
     }
     if (!ok) {
         for (int i = 0; i < 3; i++) boat_tensor_free(dx[i]);

@@ -48,7 +48,7 @@ _SIGS = {
     "bh_mse_grad": (I, [P, P, P, L]), "bh_mse_loss": (I, [P, P, P, L]), "bh_mse_loss_grad": (I, [P, P, P, P, L]),
     "bh_sgd_update": (I, [P, P, F, L, I]),
     "bh_sum_all": (I, [P, P, L]),
-    "bh_colsum": (I, [P, P, L, L, I]),
+    "bh_colsum": (I, [P, P, L, L, I]), "bh_colsum_grouped": (I, [C.POINTER(P), C.POINTER(P), I, L, L, I]),
     "bh_softmax_forward": (I, [P, P, L, L]), "bh_softmax_backward": (I, [P, P, P, L, L]),
     "bh_log_softmax_forward": (I, [P, P, L, L]), "bh_log_softmax_backward": (I, [P, P, P, L, L]),
     "bh_softmax_ce_grad": (I, [P, P, P, P, L, L]),

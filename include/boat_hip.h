@@ -135,7 +135,10 @@ int bh_sgd_update(float* p, float* g, float lr, int64_t n, int zero_grad);      
 
 /* ---- reductions / softmax (src/ops/arithmetic.c:611-691; src/autodiff.c:1701-2068; dense.c:286-291) ---- */
 int bh_sum_all(const float* x, float* out1, int64_t n);
-int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumulate); /* db (+)= sum_rows dY */
+int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumulate);
+/* the same for up to 3 matrices of one shape in one pair of launches (the bias gradients of a self-attention layer's three
+ * input projections, src/layers/attention.c:1262-1279 three times); the same sums in the same order as bh_colsum */
+int bh_colsum_grouped(const float* const* x, float* const* out, int groups, int64_t rows, int64_t cols, int accumulate); /* db (+)= sum_rows dY */
 int bh_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);
 int bh_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols);
 int bh_log_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);

@@ -233,6 +233,25 @@ def test_colsum(hip, rng, rows, cols):
     assert np.max(np.abs(out.numpy() - 2 * want)) <= 2 * TOL_RED * np.abs(x).sum(0).max()
 
 
+@pytest.mark.parametrize("rows,cols", [(8192, 1024), (1000, 37), (300, 4096), (64, 10)])
+def test_colsum_grouped(hip, rng, rows, cols):
+    """bh_colsum_grouped: three matrices in one pair of launches give bh_colsum's bits for each, with and without
+    accumulation (few rows fall back to bh_colsum itself)."""
+    import ctypes as C
+    xs = [rng.standard_normal((rows, cols)).astype(np.float32) for _ in range(3)]
+    dxs = [dev(hip, x) for x in xs]
+    outs = [hip.zeros(cols) for _ in range(3)]
+    singles = [hip.zeros(cols) for _ in range(3)]
+    tab = lambda arrs: (C.c_void_p * 3)(*[a.ptr for a in arrs])
+    for acc in (0, 1):
+        hip.check(hip.bh_colsum_grouped(tab(dxs), tab(outs), 3, rows, cols, acc))
+        for g in range(3):
+            hip.check(hip.bh_colsum(dxs[g].ptr, singles[g].ptr, rows, cols, acc))
+            assert np.array_equal(outs[g].numpy(), singles[g].numpy()), (acc, g)
+            want = (1 + acc) * xs[g].sum(0, dtype=np.float64)
+            assert np.max(np.abs(outs[g].numpy() - want)) <= TOL_RED * max(1.0, np.abs(want).max())
+
+
 @pytest.mark.parametrize("rows,cols", [(64, 10), (3, 33), (5, 1), (7, 1000)])
 def test_softmax_family(hip, oracle, rng, rows, cols):
     x = (3 * rng.standard_normal((rows, cols))).astype(np.float32)

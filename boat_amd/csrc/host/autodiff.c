@@ -153,8 +153,10 @@ bool boat_variable_reset_data(boat_variable_t* v, boat_tensor_t* new_tensor) {
 void boat_variable_zero_grad(boat_variable_t* v) {
     if (!v || !v->grad) return;
     if (v->persistent_grad) {
-        float* g = bt_dev_write(v->grad);
-        if (g) boat_hip_ok(bh_memset_zero(g, v->grad->nbytes), "boat_variable_zero_grad");
+        if (!bt_set_zero(v->grad)) {
+            float* g = bt_dev_write(v->grad);
+            if (g) boat_hip_ok(bh_memset_zero(g, v->grad->nbytes), "boat_variable_zero_grad");
+        }
         bt_flush_exposed();
     } else {
         boat_tensor_unref(v->grad);   /* the reference drops the tensor (autodiff.c:285-292) */

@@ -60,6 +60,14 @@ const float* bt_dev_read(const boat_tensor_t* t);
 float* bt_dev_write(boat_tensor_t* t);
 /* device pointer for read-modify-write */
 float* bt_dev_rw(boat_tensor_t* t);
+/* A storage with no valid copy on either side is all zeros by definition (a new tensor, tensor.c:132 zero-fills) and
+ * is filled in only when somebody reads it.  bt_set_zero puts a whole tensor back into that state without touching
+ * memory when it can (not a slice, pointer not held by the caller) and returns whether it did; bt_dev_accumulate is the
+ * pointer for `t += contribution`: while t is in the zero state the kernel may overwrite instead (*accumulate = 0), so
+ * the zeros are never written and never read back. */
+bool bt_set_zero(boat_tensor_t* t);
+bool bt_is_zero(const boat_tensor_t* t);
+float* bt_dev_accumulate(boat_tensor_t* t, int* accumulate);
 /* what boat_tensor_data() returns, for the library's own host-side writes (initial weights): the pointer does not
  * leave the library, so the tensor does not become "exposed" in coherent-pointer mode */
 void* bt_host_rw(boat_tensor_t* t);

@@ -554,6 +554,27 @@ float* bt_dev_rw(boat_tensor_t* t) {
     return (float*)((char*)bh_buffer_ptr(t->st->dev) + t->offset);
 }
 
+bool bt_is_zero(const boat_tensor_t* t) {
+    return t && t->st && !t->st->host_valid && !t->st->dev_valid && !t->st->exposed && t->nbytes == t->st->nbytes;
+}
+bool bt_set_zero(boat_tensor_t* t) {
+    if (!t || !t->st) return false;
+    boat_storage_t* st = t->st;
+    if (t->nbytes != st->nbytes || st->exposed || st->pending) return false;
+    st->host_valid = false;
+    st->dev_valid = false;
+    st->shadow_valid = false;
+    return true;
+}
+float* bt_dev_accumulate(boat_tensor_t* t, int* accumulate) {
+    if (bt_is_zero(t)) {
+        *accumulate = 0;
+        return bt_dev_write(t);
+    }
+    *accumulate = 1;
+    return bt_dev_rw(t);
+}
+
 boat_tensor_t* boat_tensor_from_data(const int64_t* shape, size_t ndim, boat_dtype_t dtype, const void* data) {
     boat_tensor_t* t = boat_tensor_create(shape, ndim, dtype, BOAT_DEVICE_CPU);
     if (!t) return NULL;

@@ -119,10 +119,14 @@ static boat_tensor_t* boat_dense_layer_backward_unflushed(boat_dense_layer_t* la
     const float* pw = bt_dev_read(layer->weight);
     const float* pg = bt_dev_read(grad_output);
     float* pdx = bt_dev_write(dx);
-    float* pgw = layer->grad_weight ? bt_dev_rw(layer->grad_weight) : NULL;
-    float* pgb = (with_bias && layer->grad_bias) ? bt_dev_rw(layer->grad_bias) : NULL;
+    /* the parameter gradients accumulate (dense.c:255-291); into gradients that are still the zeros of a zero_grad
+     * nobody has looked at since, the kernels write instead of adding */
+    boat_tensor_t* gb = (with_bias && layer->grad_bias) ? layer->grad_bias : NULL;
+    const bool fresh = bt_is_zero(layer->grad_weight) && (!gb || bt_is_zero(gb));
+    float* pgw = !layer->grad_weight ? NULL : fresh ? bt_dev_write(layer->grad_weight) : bt_dev_rw(layer->grad_weight);
+    float* pgb = !gb ? NULL : fresh ? bt_dev_write(gb) : bt_dev_rw(gb);
     if (!px || !pw || !pg || !pdx || !pgw ||
-        !boat_hip_ok(bh_dense_backward(px, pw, pg, pdx, pgw, pgb, m, k, n, 1), "dense backward")) {
+        !boat_hip_ok(bh_dense_backward(px, pw, pg, pdx, pgw, pgb, m, k, n, fresh ? 0 : 1), "dense backward")) {
         boat_tensor_free(dx);
         return NULL;
     }
@@ -332,13 +336,16 @@ boat_tensor_t* boat_layernorm_backward_add_impl(boat_layernorm_t* norm, const bo
     const float* pg = norm->weight ? bt_dev_read(norm->weight) : NULL;
     const float* padd = add ? bt_dev_read(add) : NULL;
     float* pdx = covers_all ? bt_dev_write(dx) : bt_dev_rw(dx);
-    float* pgw = norm->grad_weight ? bt_dev_rw(norm->grad_weight) : NULL;
-    float* pgb = norm->grad_bias ? bt_dev_rw(norm->grad_bias) : NULL;
-    /* parameter gradients accumulate across calls like the dense layer's (dense.c:255-291) */
+    /* parameter gradients accumulate across calls like the dense layer's (dense.c:255-291), or are written when they
+     * are still the untouched zeros of a zero_grad */
+    const bool fresh = (!norm->grad_weight || bt_is_zero(norm->grad_weight)) && (!norm->grad_bias || bt_is_zero(norm->grad_bias));
+    float* pgw = !norm->grad_weight ? NULL : fresh ? bt_dev_write(norm->grad_weight) : bt_dev_rw(norm->grad_weight);
+    float* pgb = !norm->grad_bias ? NULL : fresh ? bt_dev_write(norm->grad_bias) : bt_dev_rw(norm->grad_bias);
+    const int acc = fresh ? 0 : 1;
     bool ok = px && pdy && pdx && (padd || !add);
-    if (ok && add) ok = boat_hip_ok(bh_layernorm_backward_add(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), padd, pdx, pgw, pgb, rows, hidden, 1),
+    if (ok && add) ok = boat_hip_ok(bh_layernorm_backward_add(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), padd, pdx, pgw, pgb, rows, hidden, acc),
                                     "layernorm backward");
-    else if (ok) ok = boat_hip_ok(bh_layernorm_backward(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), pdx, pgw, pgb, rows, hidden, 1),
+    else if (ok) ok = boat_hip_ok(bh_layernorm_backward(px, pg, pdy, bt_dev_read(mean), bt_dev_read(rstd), pdx, pgw, pgb, rows, hidden, acc),
                                   "layernorm backward");
     if (!ok) {
         boat_tensor_free(dx);
@@ -486,10 +493,11 @@ boat_tensor_t* boat_rmsnorm_backward(boat_rmsnorm_t* norm, const boat_tensor_t* 
     const float* pdy = bt_dev_read(grad_output);
     const float* pw = norm->weight ? bt_dev_read(norm->weight) : NULL;
     float* pdx = covers_all ? bt_dev_write(dx) : bt_dev_rw(dx);
-    float* pgw = norm->grad_weight ? bt_dev_rw(norm->grad_weight) : NULL;
     /* the parameter gradient accumulates across calls like the dense layer's (dense.c:255-291) */
+    int acc = 1;
+    float* pgw = norm->grad_weight ? bt_dev_accumulate(norm->grad_weight, &acc) : NULL;
     if (!px || !pdy || !pdx ||
-        !boat_hip_ok(bh_rmsnorm_backward(px, pw, pdy, bt_dev_read(norm->cache_inv_rms), pdx, pgw, rows, hidden, norm->config.eps, 1),
+        !boat_hip_ok(bh_rmsnorm_backward(px, pw, pdy, bt_dev_read(norm->cache_inv_rms), pdx, pgw, rows, hidden, norm->config.eps, acc),
                      "rmsnorm backward")) {
         boat_tensor_free(dx);
         dx = NULL;

@@ -122,6 +122,12 @@ static void inplace_op(int op, boat_tensor_t* a, const boat_tensor_t* b) {
         return;
     }
     const float* pb = bt_dev_read(b);
+    if (op == 0 && pb && bt_is_zero(a) && a != b && a->st != b->st) {   /* 0 + b: a copy, the zeros are never written */
+        float* pz = bt_dev_write(a);
+        if (pz) boat_hip_ok(bh_memcpy_d2d(pz, pb, a->nbytes), "boat_add_");
+        bt_flush_exposed();
+        return;
+    }
     float* pa = bt_dev_rw(a);
     if (!pa || !pb) return;
     if (op == 0) boat_hip_ok(bh_add_inplace(pa, pb, (int64_t)a->nelements), "boat_add_");

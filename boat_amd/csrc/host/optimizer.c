@@ -162,11 +162,14 @@ void boat_optimizer_zero_grad(boat_optimizer_t* optimizer) {
     if (!optimizer) return;
     adam_state_t* s = (adam_state_t*)optimizer;
     if (!known_type(s)) return;
-    /* one launch over all gradient tensors (the table arrays are sized for num_params) */
+    /* A gradient nobody holds a pointer to becomes zero by losing its contents (the next backward writes it instead of
+     * adding to it, a reader in between gets zeros filled in); the others are cleared by one launch over all of them
+     * (the table arrays are sized for num_params) */
     int count = 0;
     for (size_t i = 0; i < s->num_params; i++) {
         boat_tensor_t* g = s->grads[i];
         if (!g || g->nelements == 0 || !bt_is_f32(g)) continue;
+        if (bt_set_zero(g)) continue;
         float* p = bt_dev_write(g);
         if (!p) continue;
         s->tp[count] = p;

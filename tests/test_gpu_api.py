@@ -127,6 +127,60 @@ def test_dense_backward_accumulates(boat, oracle, rng):
         assert rel_fro(got, want) <= TOL_GEMM
 
 
+def test_zero_grad_keeps_its_meaning_when_the_zeros_are_never_written(boat, oracle, rng):
+    """With pointers not kept, boat_optimizer_zero_grad clears a gradient by dropping its contents: the next backward
+    writes it (the same numbers as adding to zeros, dense.c:255-291), a second backward adds, a reader in between sees
+    zeros, and an optimizer step right after zero_grad uses zero gradients (adam.c:203-222)."""
+    m, k, n = 12, 20, 7
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    dy = rng.standard_normal((m, n)).astype(np.float32)
+    _, gw, gb = oracle.dense_backward(x, w, dy)
+    boat.boat_hip_set_coherent_pointers(0)
+    try:
+        layer = bc._make_dense(boat, w, b)
+        opt = boat.boat_adam_optimizer_create(1e-2, 0.9, 0.999, 1e-8)
+        tgw, tgb = boat.boat_dense_layer_get_grad_weight(layer), boat.boat_dense_layer_get_grad_bias(layer)
+        boat.boat_optimizer_add_parameter(opt, boat.boat_dense_layer_get_weight(layer), tgw)
+        boat.boat_optimizer_add_parameter(opt, boat.boat_dense_layer_get_bias(layer), tgb)
+        tx, tdy = boat.tensor(x), boat.tensor(dy)
+
+        def backward():
+            ty = boat.boat_dense_layer_forward(layer, tx)
+            tdx = boat.boat_dense_layer_backward(layer, tdy)
+            boat.boat_tensor_unref(ty)
+            boat.boat_tensor_unref(tdx)
+
+        backward()
+        boat.boat_optimizer_zero_grad(opt)
+        backward()                                             # written, not added to stale contents
+        assert rel_fro(boat.numpy(tgw), gw) <= TOL_GEMM and rel_fro(boat.numpy(tgb), gb) <= TOL_GEMM
+        once_w, once_b = boat.numpy(tgw).copy(), boat.numpy(tgb).copy()
+        backward()                                             # no zero_grad in between: accumulates
+        assert np.array_equal(boat.numpy(tgw), once_w + once_w) and np.array_equal(boat.numpy(tgb), once_b + once_b)
+        boat.boat_optimizer_zero_grad(opt)
+        assert not boat.numpy(tgw).any() and not boat.numpy(tgb).any()      # a reader in between sees zeros
+        backward()
+        assert np.array_equal(boat.numpy(tgw), once_w) and np.array_equal(boat.numpy(tgb), once_b)
+        boat.boat_optimizer_zero_grad(opt)
+        before = boat.numpy(boat.boat_dense_layer_get_weight(layer)).copy()
+        boat.boat_optimizer_step(opt)                          # a step on cleared gradients: m, v decay, the update is m/(sqrt(v)+eps)
+        after = boat.numpy(boat.boat_dense_layer_get_weight(layer))
+        assert np.isfinite(after).all() and np.abs(after - before).max() <= 1e-2 * 1.0001
+        boat.boat_optimizer_zero_grad(opt)
+        only_b = boat.numpy(tgb)                                # one of the pair looked at, the other still dropped
+        assert not only_b.any()
+        backward()
+        assert np.array_equal(boat.numpy(tgw), once_w) and np.array_equal(boat.numpy(tgb), once_b)
+        boat.boat_optimizer_free(opt)
+        boat.boat_dense_layer_free(layer)
+        boat.boat_tensor_unref(tx)
+        boat.boat_tensor_unref(tdy)
+    finally:
+        boat.boat_hip_set_coherent_pointers(1)
+
+
 def test_dense_error_paths(boat):
     layer = boat.boat_dense_layer_create(4, 3, True)
     bad = boat.tensor(np.zeros((2, 3), np.float32))

@@ -203,6 +203,148 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* p, float* g, float l
     }
 }
 
+// ---- activation backward that also sums its result over the rows (see launch_act_bwd_colsum) ----
+// Row chunk y of Y takes rows y, y+Y, ...; a lane owns one column (VEC: four neighbouring ones); per column four running
+// sums, exactly the sums of colsum_partial_kernel on the stored dx.
+template <typename F, bool VEC>
+__global__ __launch_bounds__(VEC ? 64 : 256) void act_bwd_colsum_partial_kernel(F f, const float* __restrict__ saved,
+                                                                                 const float* __restrict__ dy, float* __restrict__ dx,
+                                                                                 float* __restrict__ partial, int64_t rows, int64_t cols) {
+    const int64_t step = gridDim.y;
+    if constexpr (VEC) {
+        const int64_t c = ((int64_t)blockIdx.x * 64 + threadIdx.x) * 4;
+        if (c >= cols) return;
+        f32x4 acc[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        int64_t r = blockIdx.y;
+        for (; r + 3 * step < rows; r += 4 * step) {
+            f32x4 a[4], g[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                a[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(saved + (r + j * step) * cols + c));
+                g[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + (r + j * step) * cols + c));
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                f32x4 v;
+                v.x = f(a[j].x, g[j].x, 0.f, 0.f);
+                v.y = f(a[j].y, g[j].y, 0.f, 0.f);
+                v.z = f(a[j].z, g[j].z, 0.f, 0.f);
+                v.w = f(a[j].w, g[j].w, 0.f, 0.f);
+                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dx + (r + j * step) * cols + c));
+                acc[j].x += v.x; acc[j].y += v.y; acc[j].z += v.z; acc[j].w += v.w;
+            }
+        }
+        for (; r < rows; r += step) {
+            const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(saved + r * cols + c));
+            const f32x4 g = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + r * cols + c));
+            f32x4 v;
+            v.x = f(a.x, g.x, 0.f, 0.f);
+            v.y = f(a.y, g.y, 0.f, 0.f);
+            v.z = f(a.z, g.z, 0.f, 0.f);
+            v.w = f(a.w, g.w, 0.f, 0.f);
+            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dx + r * cols + c));
+            acc[0].x += v.x; acc[0].y += v.y; acc[0].z += v.z; acc[0].w += v.w;
+        }
+        f32x4 t;
+        t.x = (acc[0].x + acc[1].x) + (acc[2].x + acc[3].x);
+        t.y = (acc[0].y + acc[1].y) + (acc[2].y + acc[3].y);
+        t.z = (acc[0].z + acc[1].z) + (acc[2].z + acc[3].z);
+        t.w = (acc[0].w + acc[1].w) + (acc[2].w + acc[3].w);
+        *reinterpret_cast<f32x4*>(partial + (int64_t)blockIdx.y * cols + c) = t;
+    } else {
+        const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (c >= cols) return;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int64_t r = blockIdx.y;
+        for (; r + 3 * step < rows; r += 4 * step) {
+            const float v0 = f(saved[r * cols + c], dy[r * cols + c], 0.f, 0.f);
+            const float v1 = f(saved[(r + step) * cols + c], dy[(r + step) * cols + c], 0.f, 0.f);
+            const float v2 = f(saved[(r + 2 * step) * cols + c], dy[(r + 2 * step) * cols + c], 0.f, 0.f);
+            const float v3 = f(saved[(r + 3 * step) * cols + c], dy[(r + 3 * step) * cols + c], 0.f, 0.f);
+            dx[r * cols + c] = v0;
+            dx[(r + step) * cols + c] = v1;
+            dx[(r + 2 * step) * cols + c] = v2;
+            dx[(r + 3 * step) * cols + c] = v3;
+            a0 += v0; a1 += v1; a2 += v2; a3 += v3;
+        }
+        for (; r < rows; r += step) {
+            const float v = f(saved[r * cols + c], dy[r * cols + c], 0.f, 0.f);
+            dx[r * cols + c] = v;
+            a0 += v;
+        }
+        partial[(int64_t)blockIdx.y * cols + c] = (a0 + a1) + (a2 + a3);
+    }
+}
+// few rows: fold_rows_kernel's shape (64 columns x 16 row lanes, folded through LDS in lane order) on values computed here
+template <typename F>
+__global__ __launch_bounds__(kFoldCols * kFoldLanes) void act_bwd_colsum_small_kernel(F f, const float* __restrict__ saved,
+                                                                                      const float* __restrict__ dy, float* __restrict__ dx,
+                                                                                      int64_t rows, int64_t cols, float* __restrict__ out,
+                                                                                      int accumulate) {
+    __shared__ float red[kFoldLanes][kFoldCols + 1];
+    const int tx = threadIdx.x % kFoldCols, ty = threadIdx.x / kFoldCols;
+    const int64_t c = (int64_t)blockIdx.x * kFoldCols + tx;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (c < cols) {
+        int64_t r = ty;
+        for (; r + 3 * kFoldLanes < rows; r += 4 * kFoldLanes) {
+            const float v0 = f(saved[r * cols + c], dy[r * cols + c], 0.f, 0.f);
+            const float v1 = f(saved[(r + kFoldLanes) * cols + c], dy[(r + kFoldLanes) * cols + c], 0.f, 0.f);
+            const float v2 = f(saved[(r + 2 * kFoldLanes) * cols + c], dy[(r + 2 * kFoldLanes) * cols + c], 0.f, 0.f);
+            const float v3 = f(saved[(r + 3 * kFoldLanes) * cols + c], dy[(r + 3 * kFoldLanes) * cols + c], 0.f, 0.f);
+            dx[r * cols + c] = v0;
+            dx[(r + kFoldLanes) * cols + c] = v1;
+            dx[(r + 2 * kFoldLanes) * cols + c] = v2;
+            dx[(r + 3 * kFoldLanes) * cols + c] = v3;
+            a0 += v0; a1 += v1; a2 += v2; a3 += v3;
+        }
+        for (; r < rows; r += kFoldLanes) {
+            const float v = f(saved[r * cols + c], dy[r * cols + c], 0.f, 0.f);
+            dx[r * cols + c] = v;
+            a0 += v;
+        }
+    }
+    red[ty][tx] = (a0 + a1) + (a2 + a3);
+    __syncthreads();
+    if (ty == 0 && c < cols) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < kFoldLanes; i++) acc += red[i][tx];
+        out[c] = accumulate ? out[c] + acc : acc;
+    }
+}
+
+// dx = dy * f'(saved) and, in the same pass, the column sums of dx (the bias gradient of the dense layer whose output the
+// activation took): out[c] (+)= sum_r dx[r][c].  The sums are bh_colsum's, in its order: rows <= 256 take the one-launch
+// fold (64 columns x 16 row lanes), larger matrices the same row chunks, four running sums per lane and fold_rows_kernel.
+template <typename F>
+static int launch_act_bwd_colsum(const char* name, F f, const float* saved, const float* dy, float* dx, float* out, int64_t rows,
+                                 int64_t cols, int accumulate) {
+    if (rows <= 256) {
+        hipLaunchKernelGGL((act_bwd_colsum_small_kernel<F>), dim3((unsigned)ceil_div(cols, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0,
+                           stream(), f, saved, dy, dx, rows, cols, out, accumulate);
+        return BH_LAUNCH_CHECK(name);
+    }
+    const int col_blocks = (int)ceil_div(cols, 256);
+    int64_t chunks = ceil_div(2048, col_blocks);          // as bh_colsum cuts the rows
+    if (chunks > ceil_div(rows, 32)) chunks = ceil_div(rows, 32);
+    if (chunks < 1) chunks = 1;
+    float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * cols));
+    if (!partial) return BH_ENOMEM;
+    if (cols % 4 == 0 && aligned16(saved) && aligned16(dy) && aligned16(dx))
+        hipLaunchKernelGGL((act_bwd_colsum_partial_kernel<F, true>), dim3(col_blocks, (unsigned)chunks), dim3(64), 0, stream(), f, saved, dy,
+                           dx, partial, rows, cols);
+    else
+        hipLaunchKernelGGL((act_bwd_colsum_partial_kernel<F, false>), dim3(col_blocks, (unsigned)chunks), dim3(256), 0, stream(), f, saved,
+                           dy, dx, partial, rows, cols);
+    hipLaunchKernelGGL(fold_rows_kernel, dim3((unsigned)ceil_div(cols, kFoldCols)), dim3(kFoldCols * kFoldLanes), 0, stream(), partial,
+                       chunks, cols, out, (float*)nullptr, cols, accumulate);
+    bh_free(partial);
+    return BH_LAUNCH_CHECK(name);
+}
+
 }  // namespace bh
 
 using namespace bh;
@@ -317,6 +459,21 @@ int bh_activation_forward(int act, const float* x, float* y, int64_t n) {
         case BH_ACT_GELU: return launch_ew<1, false>("gelu fwd", FGelu{}, y, x, nullptr, nullptr, n);
     }
     return set_error(BH_EINVAL, "bh_activation_forward: unknown activation %d", act);
+}
+
+int bh_activation_backward_colsum(int act, const float* saved, const float* dy, float* dx, float* colsum, int64_t rows, int64_t cols,
+                                  int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && cols >= 0 && (colsum || cols == 0) && ((saved && dy && dx) || rows * cols == 0), "bad argument");
+    if (cols == 0) return BH_OK;
+    if (rows == 0) return accumulate ? BH_OK : bh_memset_zero(colsum, sizeof(float) * (size_t)cols);
+    switch (act) {
+        case BH_ACT_RELU: return launch_act_bwd_colsum("relu bwd + colsum", FReluBwd<false>{}, saved, dy, dx, colsum, rows, cols, accumulate);
+        case BH_ACT_SIGMOID: return launch_act_bwd_colsum("sigmoid bwd + colsum", FSigmoidBwd<false>{}, saved, dy, dx, colsum, rows, cols, accumulate);
+        case BH_ACT_TANH: return launch_act_bwd_colsum("tanh bwd + colsum", FTanhBwd<false>{}, saved, dy, dx, colsum, rows, cols, accumulate);
+        case BH_ACT_GELU: return launch_act_bwd_colsum("gelu bwd + colsum", FGeluBwd<false>{}, saved, dy, dx, colsum, rows, cols, accumulate);
+    }
+    return set_error(BH_EINVAL, "bh_activation_backward_colsum: unknown activation %d", act);
 }
 
 int bh_activation_backward(int act, const float* saved, const float* dy, float* dx, int64_t n, int accumulate) {

@@ -35,6 +35,7 @@ typedef struct boat_op {
     uint64_t seq;                /* recording order == a topological order */
     uint64_t mark;               /* visit epoch of the backward that last collected it */
     uint64_t skip;               /* visit epoch of a backward in which a fused rule already covered this op */
+    uint64_t bias_done;          /* dense: visit epoch of a backward in which the consumer's rule already added the bias gradient */
 } boat_op_t;
 
 struct boat_variable_t {
@@ -505,6 +506,22 @@ static boat_tensor_t* scaled_by_first(const boat_tensor_t* shape_of, const boat_
     return g;
 }
 
+/* dx of an activation.  When the activation's input is the output of a dense layer with a bias, read by nothing else in
+ * this walk and without a gradient so far, dx is all of that layer's grad_output: its column sums, the layer's bias
+ * gradient (dense.c:286-291), are taken in the same pass and the dense rule is told so. */
+static boat_tensor_t* activation_grad_of(int act, boat_variable_t* in, const boat_tensor_t* saved, const boat_tensor_t* dy) {
+    boat_op_t* p = in->producer;
+    if (p && p->type == OP_DENSE && p->mark == g_epoch && in->uses_epoch == g_epoch && in->walk_uses == 1 && !in->grad &&
+        !bt_reference_exact()) {
+        boat_tensor_t* dx = bt_activation_backward_with_dense_bias(act, saved, dy, (boat_dense_layer_t*)p->layer);
+        if (dx) {
+            p->bias_done = g_epoch;
+            return dx;
+        }
+    }
+    return activation_grad(act, saved, dy);
+}
+
 static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
     boat_variable_t* a = op->inputs[0];
     boat_variable_t* b = op->num_inputs > 1 ? op->inputs[1] : NULL;
@@ -547,16 +564,16 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
             if (b->requires_grad) accumulate(b, scaled_by_first(a->data, a->data, dy), true);
             break;
         case OP_RELU:      /* :1244-1296, mask from the op input */
-            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_RELU, a->data, dy), true);
+            if (a->requires_grad) accumulate(a, activation_grad_of(BH_ACT_RELU, a, a->data, dy), true);
             break;
         case OP_GELU:
-            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_GELU, a->data, dy), true);
+            if (a->requires_grad) accumulate(a, activation_grad_of(BH_ACT_GELU, a, a->data, dy), true);
             break;
         case OP_SIGMOID:   /* :1298-1353, from the saved output */
-            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_SIGMOID, op->output->data, dy), true);
+            if (a->requires_grad) accumulate(a, activation_grad_of(BH_ACT_SIGMOID, a, op->output->data, dy), true);
             break;
         case OP_TANH:      /* :1355-1452 */
-            if (a->requires_grad) accumulate(a, activation_grad(BH_ACT_TANH, op->output->data, dy), true);
+            if (a->requires_grad) accumulate(a, activation_grad_of(BH_ACT_TANH, a, op->output->data, dy), true);
             break;
         case OP_MATMUL: {  /* :1454-1496, 2-D operands */
             const boat_tensor_t *A = a->data, *B = b->data;
@@ -603,7 +620,9 @@ static void backward_op(boat_op_t* op, const boat_tensor_t* dy) {
             if (a->requires_grad) accumulate(a, boat_tensor_reshape(dy, a->data->shape, a->data->ndim), true);
             break;
         case OP_DENSE: {       /* :2640-2672 */
-            boat_tensor_t* dx = boat_dense_layer_backward((boat_dense_layer_t*)op->layer, dy);
+            boat_tensor_t* dx = (op->bias_done == g_epoch && !bt_reference_exact())
+                                    ? bt_dense_layer_backward_bias_done((boat_dense_layer_t*)op->layer, dy)
+                                    : boat_dense_layer_backward((boat_dense_layer_t*)op->layer, dy);
             if (dx && a->requires_grad) accumulate(a, dx, true);
             else boat_tensor_free(dx);
             break;

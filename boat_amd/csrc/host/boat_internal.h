@@ -139,6 +139,12 @@ bool boat_attention_backward_self(boat_attention_t* attention, const boat_tensor
 boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
                                             const boat_tensor_t* rstd, const boat_tensor_t* grad_output);
 /* the same with `add` (may be NULL; same shape as x) added to the returned input gradient by the kernel's own store */
+/* The tape's rule for an activation that sat directly behind a dense layer: dx = dy * f'(saved) together with that layer's
+ * bias gradient (the column sums of dx, dense.c:286-291) in one pass; NULL when the shapes do not allow it (nothing done).
+ * The dense layer's own backward is then run with bias_done, which leaves grad_bias alone. */
+boat_tensor_t* bt_activation_backward_with_dense_bias(int act, const boat_tensor_t* saved, const boat_tensor_t* dy,
+                                                      boat_dense_layer_t* layer);
+boat_tensor_t* bt_dense_layer_backward_bias_done(boat_dense_layer_t* layer, const boat_tensor_t* grad_output);
 boat_tensor_t* boat_layernorm_backward_add_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
                                                 const boat_tensor_t* rstd, const boat_tensor_t* grad_output, const boat_tensor_t* add);
 

@@ -96,7 +96,7 @@ boat_tensor_t* boat_dense_layer_forward(boat_dense_layer_t* layer, const boat_te
     return out;
 }
 
-static boat_tensor_t* boat_dense_layer_backward_unflushed(boat_dense_layer_t* layer, const boat_tensor_t* grad_output) {
+static boat_tensor_t* dense_backward_impl(boat_dense_layer_t* layer, const boat_tensor_t* grad_output, bool bias_done) {
     if (!layer || !grad_output || !layer->cache_input) return NULL;
     const boat_tensor_t* input = layer->cache_input;
     if (input->ndim != 2 || grad_output->ndim != 2) {
@@ -113,7 +113,7 @@ static boat_tensor_t* boat_dense_layer_backward_unflushed(boat_dense_layer_t* la
     boat_tensor_t* dx = bt_new_uninit(shape, 2, grad_output->device);
     if (!dx) return NULL;
     if (!layer->grad_weight) layer->grad_weight = boat_tensor_create_like(layer->weight);
-    const bool with_bias = layer->use_bias && layer->bias;
+    const bool with_bias = layer->use_bias && layer->bias && !bias_done;   /* (done: the caller has already added this call's column sums) */
     if (with_bias && !layer->grad_bias) layer->grad_bias = boat_tensor_create_like(layer->bias);
     const float* px = bt_dev_read(input);
     const float* pw = bt_dev_read(layer->weight);
@@ -132,8 +132,33 @@ static boat_tensor_t* boat_dense_layer_backward_unflushed(boat_dense_layer_t* la
     }
     return dx;
 }
+boat_tensor_t* bt_dense_layer_backward_bias_done(boat_dense_layer_t* layer, const boat_tensor_t* grad_output) {
+    boat_tensor_t* result = dense_backward_impl(layer, grad_output, true);
+    bt_flush_exposed();
+    return result;
+}
+boat_tensor_t* bt_activation_backward_with_dense_bias(int act, const boat_tensor_t* saved, const boat_tensor_t* dy,
+                                                      boat_dense_layer_t* layer) {
+    if (!layer || !saved || !dy || !(layer->use_bias && layer->bias) || !bt_is_f32(saved) || !bt_is_f32(dy) || dy->ndim != 2 ||
+        !bt_same_shape(saved, dy) || dy->shape[1] != (int64_t)layer->output_features || dy->nelements == 0)
+        return NULL;
+    if (!layer->grad_bias) layer->grad_bias = boat_tensor_create_like(layer->bias);
+    boat_tensor_t* dx = layer->grad_bias ? bt_new_like_uninit(saved) : NULL;
+    if (!dx) return NULL;
+    const float* ps = bt_dev_read(saved);
+    const float* pg = bt_dev_read(dy);
+    float* pd = bt_dev_write(dx);
+    int acc = 1;
+    float* pgb = (ps && pg && pd) ? bt_dev_accumulate(layer->grad_bias, &acc) : NULL;
+    if (!pgb || !boat_hip_ok(bh_activation_backward_colsum(act, ps, pg, pd, pgb, dy->shape[0], dy->shape[1], acc),
+                             "activation backward with the bias gradient")) {
+        boat_tensor_free(dx);
+        return NULL;
+    }
+    return dx;
+}
 boat_tensor_t* boat_dense_layer_backward(boat_dense_layer_t* layer, const boat_tensor_t* grad_output) {
-    boat_tensor_t* result = boat_dense_layer_backward_unflushed(layer, grad_output);
+    boat_tensor_t* result = dense_backward_impl(layer, grad_output, false);
     bt_flush_exposed();
     return result;
 }

@@ -44,6 +44,7 @@ _SIGS = {
     "bh_div_backward_b": (I, [P, P, P, P, L]),
     "bh_activation_forward": (I, [I, P, P, L]),
     "bh_activation_backward": (I, [I, P, P, P, L, I]),
+    "bh_activation_backward_colsum": (I, [I, P, P, P, P, L, L, I]),
     "bh_bias_add_rows": (I, [P, P, L, L]),
     "bh_mse_grad": (I, [P, P, P, L]), "bh_mse_loss": (I, [P, P, P, L]), "bh_mse_loss_grad": (I, [P, P, P, P, L]),
     "bh_sgd_update": (I, [P, P, F, L, I]),

@@ -111,6 +111,11 @@ int bh_activation_forward(int act, const float* x, float* y, int64_t n);        
 /* saved = op input for RELU/GELU, op output for SIGMOID/TANH (autodiff.c:1244-1452).
  * accumulate!=0 adds into dx instead of assigning. */
 int bh_activation_backward(int act, const float* saved, const float* dy, float* dx, int64_t n, int accumulate);
+/* The same on a [rows, cols] matrix, and in the same pass colsum[c] (+)= sum_r dx[r][c]: the activation sat behind a dense
+ * layer, so dx is that layer's grad_output and its column sums are the bias gradient (src/layers/dense.c:286-291), which
+ * would otherwise read dx once more.  dx and the sums are bit for bit those of bh_activation_backward followed by bh_colsum. */
+int bh_activation_backward_colsum(int act, const float* saved, const float* dy, float* dx, float* colsum, int64_t rows,
+                                  int64_t cols, int accumulate);
 
 /* the reference's elementwise arithmetic on its other element types (src/ops/arithmetic.c:157-360 with boat_mod,
  * :425-560 scalar ops and boat_pow_scalar): op 0 add, 1 sub, 2 mul, 3 div, 4 mod (fmodf / fmod / %), 5 pow (scalar form,

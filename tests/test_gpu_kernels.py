@@ -252,6 +252,27 @@ def test_colsum_grouped(hip, rng, rows, cols):
             assert np.max(np.abs(outs[g].numpy() - want)) <= TOL_RED * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 128), (1, 5), (256, 33), (257, 64), (1000, 37), (300, 4096), (8192, 1024), (1030, 516)])
+def test_activation_backward_with_column_sums(hip, rng, rows, cols):
+    """bh_activation_backward_colsum: dx and the column sums of dx in one pass are, bit for bit, bh_activation_backward
+    followed by bh_colsum (few rows, the vector and the scalar form of the partial kernel), with and without accumulation."""
+    saved = (2 * rng.standard_normal((rows, cols))).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    ds, ddy = dev(hip, saved), dev(hip, dy)
+    for act in (hip.ACT_RELU, hip.ACT_GELU, hip.ACT_SIGMOID, hip.ACT_TANH):
+        sv = dev(hip, 1 / (1 + np.exp(-saved))) if act in (hip.ACT_SIGMOID, hip.ACT_TANH) else ds   # those two save the output
+        base = rng.standard_normal(cols).astype(np.float32)
+        dx_a, dx_b, sum_a, sum_b = hip.empty((rows, cols)), hip.empty((rows, cols)), dev(hip, base), dev(hip, base)
+        for acc in (0, 1):
+            hip.check(hip.bh_activation_backward_colsum(act, sv.ptr, ddy.ptr, dx_a.ptr, sum_a.ptr, rows, cols, acc))
+            hip.check(hip.bh_activation_backward(act, sv.ptr, ddy.ptr, dx_b.ptr, rows * cols, 0))
+            hip.check(hip.bh_colsum(dx_b.ptr, sum_b.ptr, rows, cols, acc))
+            assert np.array_equal(dx_a.numpy(), dx_b.numpy()), (act, acc)
+            assert np.array_equal(sum_a.numpy(), sum_b.numpy()), (act, acc)
+        want = 2 * dx_b.numpy().astype(np.float64).sum(0)
+        assert np.max(np.abs(sum_a.numpy() - want)) <= TOL_RED * max(1.0, np.abs(dx_b.numpy()).sum(0).max())
+
+
 @pytest.mark.parametrize("rows,cols", [(64, 10), (3, 33), (5, 1), (7, 1000)])
 def test_softmax_family(hip, oracle, rng, rows, cols):
     x = (3 * rng.standard_normal((rows, cols))).astype(np.float32)

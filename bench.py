@@ -493,19 +493,23 @@ def bench_cnn_step(steps, warmup):
 
 def bench_conv_forward_kernels():
     """bh_conv2d_forward (direct, the reference's operation order) against bh_conv2d_forward_mfma (one contraction on the
-    fp32 matrix cores) on the MNIST network's 32->64 layer at batch 64 and on a layer with many channels; HIP events."""
+    fp32 matrix cores) on the MNIST network's 32->64 layer at batch 64, on a layer with many channels and on two 5x5 layers (one
+    with stride 2); HIP events."""
     from boat_amd import hip
     rng = np.random.default_rng(20250108)
     out = {}
-    for name, (B, ic, h, w, oc) in (("64x32x14x14_to_64", (64, 32, 14, 14, 64)), ("32x128x28x28_to_256", (32, 128, 28, 28, 256))):
+    cases = (("64x32x14x14_to_64", (64, 32, 14, 14, 64, 3, 1, 1)), ("32x128x28x28_to_256", (32, 128, 28, 28, 256, 3, 1, 1)),
+             ("64x32x28x28_to_64_k5", (64, 32, 28, 28, 64, 5, 1, 2)), ("32x64x56x56_to_128_k5_stride2", (32, 64, 56, 56, 128, 5, 2, 2)))
+    for name, (B, ic, h, w, oc, k, stride, pad) in cases:
+        ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
         x = hip.to_device(rng.standard_normal((B, ic, h, w), dtype=np.float32))
-        wt = hip.to_device((0.1 * rng.standard_normal((oc, ic, 3, 3), dtype=np.float32)).astype(np.float32))
+        wt = hip.to_device((0.1 * rng.standard_normal((oc, ic, k, k), dtype=np.float32)).astype(np.float32))
         b = hip.to_device(rng.standard_normal(oc, dtype=np.float32))
-        y = hip.empty((B, oc, h, w))
-        flops = 2.0 * B * oc * h * w * ic * 9
+        y = hip.empty((B, oc, ho, wo))
+        flops = 2.0 * B * oc * ho * wo * ic * k * k
         res = {}
         for label, fn in (("direct", hip.bh_conv2d_forward), ("matrix_cores", hip.bh_conv2d_forward_mfma)):
-            call = lambda: hip.check(fn(x.ptr, wt.ptr, b.ptr, y.ptr, B, ic, h, w, oc, 3, 1, 1))
+            call = lambda: hip.check(fn(x.ptr, wt.ptr, b.ptr, y.ptr, B, ic, h, w, oc, k, stride, pad))
             warm_clocks(hip.synchronize, call, 10)
             timer = hip.Timer()
             with timer:

@@ -158,16 +158,32 @@ __global__ __launch_bounds__(kCBlock) void conv2d_fwd_generic_kernel(const float
 // of the patch loads, and four wavefronts per position tile have four times the loads in flight.  SPLIT = 2 (256 lanes,
 // two workgroups per CU) for layers with many workgroups: one workgroup's staging, reduction and stores run under the
 // other's products.  grid (ceil(P/64), ceil(oc/64)).
-constexpr int kFmCi = 32;                       // input channels per LDS stage
-constexpr int kFmKk = kFmCi * 9;                // 288 contraction indices per stage
-constexpr int kFmRow = kFmKk + 1;               // LDS row stride in floats
-constexpr int64_t kFmBlocksSplit2 = 257;        // from this many workgroups on (more than the part has CUs) a layer runs with SPLIT = 2
+// Kernel sizes 3 and 5 (template parameter K, T = K*K taps): a lane holds four buffers of T patch values, and a 7x7
+// kernel's 196 would not leave room for anything else.  The weights of 32 input channels x 64 output channels x 25 taps
+// do not fit LDS, so a 32-channel stage is staged in NSUB parts of CI channels (3x3: one of 32, 5x5: two of 16).
+constexpr int kFmStage = 32;                    // input channels per stage (the unit in which the patch buffers rotate)
+template <int K> struct FmGeom {
+    static constexpr int T = K * K;                          // taps per channel
+    static constexpr int CI = K == 3 ? 32 : 16;              // input channels per LDS part
+    static constexpr int NSUB = kFmStage / CI;               // parts per stage
+    static constexpr int KK = CI * T;                        // contraction indices per part (a multiple of 16)
+    static constexpr int ROW = KK + 1;                       // LDS row stride in floats (odd: conflict-free 4-byte reads)
+    static constexpr size_t kLds = sizeof(float) * (64 * ROW + 64);      // weights + bias
+};
+constexpr int64_t kFmBlocksSplit2 = 257;        // from this many workgroups on (more than the part has CUs) a 3x3 layer runs with SPLIT = 2
 
-template <int SPLIT>                            // wavefronts that share a position tile: 2 or 4
+template <int SPLIT, int K>                     // wavefronts that share a position tile: 2 or 4; kernel size 3 or 5
 __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wt,
                                                                  const float* __restrict__ bias, float* __restrict__ y,
                                                                  ConvShape c, int positions) {
-    extern __shared__ __align__(16) float wl[];          // [64][kFmRow] + bias[64]; the weights' part holds the partial sums afterwards
+    using Geo = FmGeom<K>;
+    constexpr int T = Geo::T, CI = Geo::CI, NSUB = Geo::NSUB, KK = Geo::KK, ROW = Geo::ROW;
+    constexpr int TPS = CI / 2 / SPLIT;                    // turns (pairs of channels) of a wavefront per part: 2, 4 or 8
+    // how many turns ahead the patch values are fetched.  3x3: three (four buffers of 9 that rotate in fours); 5x5: one (two
+    // buffers of 25 -- four would not fit the register file, and one turn is 50 matrix instructions, longer than a trip to memory)
+    constexpr int AHEAD = K == 3 ? 3 : 1;
+    static_assert(KK % 16 == 0 && TPS % (AHEAD + 1) == 0, "the patch buffers rotate in step with the parts");
+    extern __shared__ __align__(16) float wl[];          // [64][ROW] + bias[64]; the weights' part holds the partial sums afterwards
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: what follows from it is the same for the whole wavefront
     const int wn = wv & 1, kg = wv >> 1;
@@ -178,26 +194,26 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
     const int b = n / per, p = n - b * per;
     const int oh = p / c.wo, ow = p - oh * c.wo;
     const int ih0 = oh * c.stride - c.pad, iw0 = ow * c.stride - c.pad;
-    // the nine contraction indices 2j + half of a channel pair: byte offset of the lane's patch value from the first
+    // the T contraction indices 2j + half of a channel pair: byte offset of the lane's patch value from the first
     // channel's plane in image 0 (the second channel lies one plane further; byte offsets fit 32 bits, a tensor has fewer
-    // than 2^30 elements), and whether the tap lies inside the image.  The nine conditions live as wavefront masks in
+    // than 2^30 elements), and whether the tap lies inside the image.  The T conditions live as wavefront masks in
     // scalar registers, so that a turn costs one vector instruction per load and one per select: anything more per
     // patch value competes with the matrix instructions for issue slots.
-    unsigned offb[9];
-    bool in[9];
+    unsigned offb[T];
+    bool in[T];
 #pragma unroll
-    for (int j = 0; j < 9; j++) {
-        const int kk = 2 * j + half, cp = kk >= 9 ? 1 : 0, tap = kk - 9 * cp;
-        const int kh = tap / 3, kw = tap - 3 * kh;
+    for (int j = 0; j < T; j++) {
+        const int kk = 2 * j + half, cp = kk >= T ? 1 : 0, tap = kk - T * cp;
+        const int kh = tap / K, kw = tap - K * kh;
         const int ih = ih0 + kh, iw = iw0 + kw;
         in[j] = ih >= 0 && ih < c.h && iw >= 0 && iw < c.w;
         offb[j] = 4u * (unsigned)((b * c.ic + cp) * plane + min(max(ih, 0), c.h - 1) * c.w + min(max(iw, 0), c.w - 1));
     }
-    const float* wrow = wl + r * kFmRow + half * (kFmKk / 2);
+    const float* wrow = wl + r * ROW + half * (KK / 2);
     // the second 32 channels' rows lie beyond the reach of a paired LDS read's offsets from wrow: their own base, kept
     // in a register of its own (the empty statement hides that it is wrow plus a constant, which the compiler would
     // otherwise add again in every turn)
-    int far_row = (r + 32) * kFmRow + half * (kFmKk / 2);
+    int far_row = (r + 32) * ROW + half * (KK / 2);
     asm volatile("" : "+v"(far_row));
     floatx16 acc[2];
 #pragma unroll
@@ -205,128 +221,202 @@ __global__ __launch_bounds__(128 * SPLIT, 2) void conv2d_fwd_mfma_kernel(const f
 
     // patch values of channels ci, ci + 1: the loads go to clamped (valid) addresses and nothing looks at their results
     // until mask() runs three turns later -- a select right behind a load would make the wavefront wait for it there
-    const auto fetch = [&](int ci, float (&v)[9]) {
+    const auto fetch = [&](int ci, float (&v)[T]) {
         const char* xc = reinterpret_cast<const char*>(x + (int64_t)ci * plane);     // the same for every lane
 #pragma unroll
-        for (int j = 0; j < 9; j++) {
+        for (int j = 0; j < T; j++) {
             // the empty statement (it leaves the offset as it is) keeps the offset's widening next to the load, where it
-            // folds into the load's scalar-base-plus-32-bit-offset form; hoisted out of the loop it would hold nine
+            // folds into the load's scalar-base-plus-32-bit-offset form; hoisted out of the loop it would hold T
             // register pairs
             asm volatile("" : "+v"(offb[j]));
             v[j] = *reinterpret_cast<const float*>(xc + offb[j]);
         }
     };
-    const auto mask = [&](float (&v)[9]) {                 // taps outside the image count as zero
+    const auto mask = [&](float (&v)[T]) {                 // taps outside the image count as zero
 #pragma unroll
-        for (int j = 0; j < 9; j++) v[j] = in[j] ? v[j] : 0.f;
+        for (int j = 0; j < T; j++) v[j] = in[j] ? v[j] : 0.f;
     };
     const int l16 = tid & 15, rg = tid >> 4;               // weight staging: 16 lanes per row, 8 * SPLIT rows per pass
-    // the bias of the 64 channels travels with the first stage's weights and waits in LDS behind them: fetched at the end
+    // the bias of the 64 channels travels with the first part's weights and waits in LDS behind them: fetched at the end
     // it would cost a trip to memory of its own
-    float* bl = wl + 64 * kFmRow;
+    float* bl = wl + 64 * ROW;
     float bias_in = 0.f;
     if (tid < 64 && bias && oc0 + tid < c.oc) bias_in = bias[oc0 + tid];
-    // this wavefront's pairs of input channels are kg, kg + SPLIT, ... over the whole layer: a multiple of four to a full
-    // stage, so the four patch buffers take turns in step with the stages (a register copy would have to wait for the
-    // loads it copies) and the patch values run three turns ahead, across stage boundaries too (a turn's 18 products
+    // this wavefront's pairs of input channels are kg, kg + SPLIT, ... over the whole layer: a multiple of the number of
+    // patch buffers to a part, so the buffers take turns in step with the parts (a register copy would have to wait for the
+    // loads it copies) and the patch values run AHEAD turns ahead, across part boundaries too (a 3x3 turn's 18 products
     // take a quarter of a trip to memory)
-    const int all_pairs = c.ic / 2;                        // an odd channel count's last channel follows behind its stage
-    float x0[9], x1[9], x2[9], x3[9];
+    const int all_pairs = c.ic / 2;                        // an odd channel count's last channel follows behind its part
+    float x0[T], x1[T], x2[T], x3[T];
     // a fetch past the last pair re-reads the last pair (valid memory, never used): with the same number of loads on
     // every path the waits the compiler places in front of a turn's selects count exactly the three turns in flight
     // (a fetch under a condition makes it wait for everything but the current turn's loads)
-    const auto fetch_pair = [&](int pair, float (&v)[9]) { fetch(2 * min(pair, all_pairs - 1), v); };
+    const auto fetch_pair = [&](int pair, float (&v)[T]) { fetch(2 * min(pair, all_pairs - 1), v); };
     if (all_pairs > 0) {
         fetch_pair(kg, x0);
-        fetch_pair(kg + SPLIT, x1);
-        fetch_pair(kg + 2 * SPLIT, x2);
+        if constexpr (AHEAD == 3) {
+            fetch_pair(kg + SPLIT, x1);
+            fetch_pair(kg + 2 * SPLIT, x2);
+        }
     }
-    // a stage of the layer; FULL: all its 16 pairs of channels exist, so every turn runs unconditionally
-    const auto stage = [&](int ci0, auto full_const) {
+    bool first_part = true;
+    // one part of a stage: CI channels from cs on; FULL: all its pairs of channels exist, so every turn runs unconditionally
+    const auto part = [&](int cs, auto full_const) {
         constexpr bool FULL = decltype(full_const)::value;
-        if (ci0) __syncthreads();                          // every wavefront is done with the previous stage's weights
-        const int real = min(kFmCi, c.ic - ci0) * 9;
-        // weights of the stage: row oc of w holds its ic*9 values contiguously, so a stage's run of chunk*9 is contiguous;
-        // what lies past it (an odd channel count's partner, a short last stage) is zero.  36 loads of a lane are in flight
-        // together before their LDS stores.
+        if (!first_part) __syncthreads();                  // every wavefront is done with the previous part's weights
+        const int real = min(CI, c.ic - cs) * T;
+        // weights of the part: row oc of w holds its ic*T values contiguously, so a part's run of chunk*T is contiguous;
+        // what lies past it (an odd channel count's partner, a short last part) is zero.  A lane's loads of RQ rows are
+        // in flight together before their LDS stores.
+        constexpr int RQ = K == 3 ? 2 : 1;                  // rows a lane has in flight (5x5: a row is 25 loads, and registers are short)
 #pragma unroll
-        for (int q0 = 0; q0 < 8 / SPLIT; q0 += 2) {
-            float v[2][18];
+        for (int q0 = 0; q0 < 8 / SPLIT; q0 += RQ) {
+            float v[RQ][KK / 16];
 #pragma unroll
-            for (int q = 0; q < 2; q++) {
+            for (int q = 0; q < RQ; q++) {
                 const int o = rg + 8 * SPLIT * (q0 + q);
-                const float* src = wt + ((int64_t)min(oc0 + o, c.oc - 1) * c.ic + ci0) * 9;
+                const float* src = wt + ((int64_t)min(oc0 + o, c.oc - 1) * c.ic + cs) * T;
+                if constexpr (K == 3) {
 #pragma unroll
-                for (int i = 0; i < 18; i++) {
-                    const int kk = l16 + 16 * i;
-                    v[q][i] = src[FULL ? kk : min(kk, real - 1)];     // a valid address in any case; what does not exist becomes zero below
+                    for (int i = 0; i < KK / 16; i++) {
+                        const int kk = l16 + 16 * i;
+                        v[q][i] = src[FULL ? kk : min(kk, real - 1)];     // a valid address in any case; what does not exist becomes zero below
+                    }
+                } else {
+                    // 25 clamped addresses would take 50 registers: a short part reads on into the next rows of w, whose values
+                    // become zeros below like everything past the part; only where that would leave the tensor (its last
+                    // rows) are the indices clamped, a few at a time
+                    if (FULL || src + KK <= wt + (int64_t)c.oc * c.ic * T) {
+#pragma unroll
+                        for (int i = 0; i < KK / 16; i++) v[q][i] = src[l16 + 16 * i];
+                    } else {
+#pragma unroll
+                        for (int i0 = 0; i0 < KK / 16; i0 += 5) {
+#pragma unroll
+                            for (int i = i0; i < i0 + 5; i++) v[q][i] = src[min(l16 + 16 * i, real - 1)];
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
                 }
             }
 #pragma unroll
-            for (int q = 0; q < 2; q++) {
+            for (int q = 0; q < RQ; q++) {
                 const int o = rg + 8 * SPLIT * (q0 + q);
-                float* dst = wl + o * kFmRow;
+                float* dst = wl + o * ROW;
+                // kk = l16 + 16 i lands at [kk & 1][kk >> 1]: the parity is the lane's, the rest a constant step of 8
+                const int lbase = (l16 & 1) * (KK / 2) + (l16 >> 1);
 #pragma unroll
-                for (int i = 0; i < 18; i++) {
+                for (int i = 0; i < KK / 16; i++) {
                     const int kk = l16 + 16 * i;
-                    dst[(kk & 1) * (kFmKk / 2) + (kk >> 1)] = (oc0 + o < c.oc && (FULL || kk < real)) ? v[q][i] : 0.f;
+                    dst[lbase + 8 * i] = (oc0 + o < c.oc && (FULL || kk < real)) ? v[q][i] : 0.f;
                 }
             }
         }
-        if (ci0 == 0 && tid < 64) bl[tid] = bias_in;
+        if (first_part && tid < 64) bl[tid] = bias_in;
+        first_part = false;
         __syncthreads();
-        const int first = ci0 / 2 + kg;                    // this wavefront's first pair of the stage
-        const auto products = [&](int turn, float (&cur)[9], float (&ahead)[9]) {
+        const int first = cs / 2 + kg;                     // this wavefront's first pair of the part
+        const auto products = [&](int turn, float (&cur)[T], float (&ahead)[T]) {
             const int gp = first + turn * SPLIT;
-            if (FULL) fetch_pair(gp + 3 * SPLIT, ahead);
-            else if (gp + 3 * SPLIT < all_pairs) fetch(2 * (gp + 3 * SPLIT), ahead);
+            if (FULL) fetch_pair(gp + AHEAD * SPLIT, ahead);
+            else if (gp + AHEAD * SPLIT < all_pairs) fetch(2 * (gp + AHEAD * SPLIT), ahead);
             // nothing moves across this line: left to itself the scheduler lifts the selects of a later turn up to their
             // loads, three turns early, and the wavefront waits for those loads there
             __builtin_amdgcn_sched_barrier(0);
             mask(cur);
-            const float* wp = wrow + (kg + turn * SPLIT) * 9;
-            const float* wq = wl + far_row + (kg + turn * SPLIT) * 9;
+            const float* wp = wrow + (kg + turn * SPLIT) * T;
+            const float* wq = wl + far_row + (kg + turn * SPLIT) * T;
+            if constexpr (K == 3) {
 #pragma unroll
-            for (int j = 0; j < 9; j++) {
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], cur[j], acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wq[j], cur[j], acc[1], 0, 0, 0);
+                for (int j = 0; j < T; j++) {
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], cur[j], acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wq[j], cur[j], acc[1], 0, 0, 0);
+                }
+            } else {
+                // K taps at a time, the next K taps' weights read from LDS while these run: left alone the compiler reads all
+                // 2T weights of the turn first, and they do not fit beside the patch buffers
+                float wa[K], wb[K];
+#pragma unroll
+                for (int i = 0; i < K; i++) {
+                    wa[i] = wp[i];
+                    wb[i] = wq[i];
+                }
+#pragma unroll
+                for (int ch = 0; ch < K; ch++) {
+                    float na[K], nb[K];
+                    if (ch + 1 < K) {
+#pragma unroll
+                        for (int i = 0; i < K; i++) {
+                            na[i] = wp[(ch + 1) * K + i];
+                            nb[i] = wq[(ch + 1) * K + i];
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < K; i++) {
+                        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[i], cur[ch * K + i], acc[0], 0, 0, 0);
+                        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wb[i], cur[ch * K + i], acc[1], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (ch + 1 < K) {
+#pragma unroll
+                        for (int i = 0; i < K; i++) {
+                            wa[i] = na[i];
+                            wb[i] = nb[i];
+                        }
+                    }
+                }
             }
         };
-        if (FULL) {
+        const auto have = [&](int turn) { return FULL || first + turn * SPLIT < all_pairs; };
+        if constexpr (AHEAD == 1) {
 #pragma unroll
-            for (int turn = 0; turn < kFmCi / 2 / SPLIT; turn += 4) {
+            for (int turn = 0; turn < TPS; turn += 2) {
+                if (have(turn)) products(turn, x0, x1);
+                if (have(turn + 1)) products(turn + 1, x1, x0);
+            }
+        } else if (FULL) {
+#pragma unroll
+            for (int turn = 0; turn < TPS; turn += 4) {
                 products(turn, x0, x3);
                 products(turn + 1, x1, x0);
                 products(turn + 2, x2, x1);
                 products(turn + 3, x3, x2);
             }
         } else {
-            for (int turn = 0; turn < kFmCi / 2 / SPLIT && first + turn * SPLIT < all_pairs; turn += 4) {
+            for (int turn = 0; turn < TPS && have(turn); turn += 4) {
                 products(turn, x0, x3);
-                if (first + (turn + 1) * SPLIT < all_pairs) products(turn + 1, x1, x0);
-                if (first + (turn + 2) * SPLIT < all_pairs) products(turn + 2, x2, x1);
-                if (first + (turn + 3) * SPLIT < all_pairs) products(turn + 3, x3, x2);
+                if (have(turn + 1)) products(turn + 1, x1, x0);
+                if (have(turn + 2)) products(turn + 2, x2, x1);
+                if (have(turn + 3)) products(turn + 3, x3, x2);
             }
         }
         // the single last channel of an odd count: one wavefront per position half takes it with its lanes of the
         // pair's second channel reading the first and counting as zero (the weights past the last channel are zero too)
-        const int single = c.ic / 2 - ci0 / 2;            // its pair's index within this stage
-        if ((c.ic & 1) && ci0 + kFmCi >= c.ic && kg == single % SPLIT) {
+        const int single = c.ic / 2 - cs / 2;             // its pair's index within this part
+        if ((c.ic & 1) && cs + CI >= c.ic && kg == single % SPLIT) {
             const char* xc = reinterpret_cast<const char*>(x + (int64_t)(c.ic - 1) * plane);
-            const float* wp = wrow + single * 9;
+            const float* wp = wrow + single * T;
 #pragma unroll
-            for (int j = 0; j < 9; j++) {
-                const bool other = 2 * j + half >= 9;
+            for (int j = 0; j < T; j++) {
+                const bool other = 2 * j + half >= T;
                 float v = *reinterpret_cast<const float*>(xc + (offb[j] - (other ? 4u * (unsigned)plane : 0u)));
                 v = (in[j] && !other) ? v : 0.f;
                 acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], v, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * kFmRow + j], v, acc[1], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[32 * ROW + j], v, acc[1], 0, 0, 0);
             }
         }
     };
-    int ci0_run = 0;
-    for (; ci0_run + kFmCi <= 2 * all_pairs; ci0_run += kFmCi) stage(ci0_run, std::true_type{});
-    if (ci0_run < c.ic) stage(ci0_run, std::false_type{});   // a short last stage (at most one: it holds fewer than 32 channels)
+    int cs_run = 0;
+    for (; cs_run + kFmStage <= 2 * all_pairs; cs_run += kFmStage) {       // full stages
+        part(cs_run, std::true_type{});
+        if constexpr (NSUB == 2) part(cs_run + CI, std::true_type{});
+    }
+    // a short last stage (at most one: it holds fewer than 32 channels); its parts as far as they hold channels
+    if (cs_run < c.ic) {
+        part(cs_run, std::false_type{});
+        if constexpr (NSUB == 2)
+            if (cs_run + CI < c.ic) part(cs_run + CI, std::false_type{});
+    }
     __syncthreads();                                       // the weights are no longer needed: their LDS holds the partial sums
     if (kg > 0) {
         float* red = wl + (((kg - 1) * 2 + wn) * 32) * 64 + lane;  // [kg - 1][wn][t * 16 + e][lane]
@@ -571,28 +661,33 @@ int bh_conv2d_forward_mfma(const float* x, const float* w, const float* bias, fl
     ConvShape c;
     int rc = make_conv_shape(c, batch, in_channels, height, width, out_channels, kernel, stride, pad);
     if (rc) return rc;
-    BH_CHECK_ARG(kernel == 3, "conv2d on the matrix cores: 3x3 kernels only");
+    BH_CHECK_ARG(kernel == 3 || kernel == 5, "conv2d on the matrix cores: 3x3 and 5x5 kernels only");
     if (batch == 0) return BH_OK;
     BH_CHECK_ARG(x && w && y, "null pointer");
     const int64_t positions = (int64_t)c.batch * c.ho * c.wo;
     BH_CHECK_ARG(ceil_div(c.oc, 64) <= 65535, "conv2d on the matrix cores: too many output channels");
-    constexpr size_t lds = sizeof(float) * (64 * kFmRow + 64);      // weights + bias
     static bool attr = false;
     if (!attr) {
-        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<4>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<4, 3>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)FmGeom<3>::kLds), "hipFuncSetAttribute");
         if (rc) return rc;
-        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<2>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<2, 3>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)FmGeom<3>::kLds), "hipFuncSetAttribute");
+        if (rc) return rc;
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_fwd_mfma_kernel<4, 5>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)FmGeom<5>::kLds), "hipFuncSetAttribute");
         if (rc) return rc;
         attr = true;
     }
     const dim3 grid((unsigned)ceil_div(positions, 64), (unsigned)ceil_div(c.oc, 64));
-    // the split follows the shape alone, not the device: a layer's sums always run in the same order
-    if ((int64_t)grid.x * grid.y >= kFmBlocksSplit2)
-        hipLaunchKernelGGL(conv2d_fwd_mfma_kernel<2>, grid, dim3(256), lds, stream(), x, w, bias, y, c, (int)positions);
+    // the split follows the shape alone, not the device: a layer's sums always run in the same order.  (5x5: the weights of a
+    // part fill more than half of a compute unit's LDS, so a second workgroup would not fit beside the first whatever the split.)
+    if (kernel == 5)
+        hipLaunchKernelGGL((conv2d_fwd_mfma_kernel<4, 5>), grid, dim3(512), FmGeom<5>::kLds, stream(), x, w, bias, y, c, (int)positions);
+    else if ((int64_t)grid.x * grid.y >= kFmBlocksSplit2)
+        hipLaunchKernelGGL((conv2d_fwd_mfma_kernel<2, 3>), grid, dim3(256), FmGeom<3>::kLds, stream(), x, w, bias, y, c, (int)positions);
     else
-        hipLaunchKernelGGL(conv2d_fwd_mfma_kernel<4>, grid, dim3(512), lds, stream(), x, w, bias, y, c, (int)positions);
+        hipLaunchKernelGGL((conv2d_fwd_mfma_kernel<4, 3>), grid, dim3(512), FmGeom<3>::kLds, stream(), x, w, bias, y, c, (int)positions);
     return BH_LAUNCH_CHECK("conv2d_fwd_mfma_kernel");
 }
 

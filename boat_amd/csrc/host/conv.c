@@ -22,7 +22,7 @@
 static int g_reference_input_grad = -1;   /* -1: not set by a call, follow reference-exact mode */
 
 void boat_hip_conv_reference_input_grad(int enable) { g_reference_input_grad = enable < 0 ? -1 : enable != 0; }
-/* forward on the matrix cores (3x3 kernels of layers wide enough for it to win, see conv_forward_wants_mfma); off by
+/* forward on the matrix cores (3x3 and 5x5 kernels of layers wide enough for it to win, see conv_forward_wants_mfma); off by
  * default because the direct kernel's output is bit-identical to the reference's and the MFMA order is not.
  * BOAT_HIP_CONV_FORWARD_MFMA=1 in the environment sets the initial value. */
 static int g_forward_mfma = -1;
@@ -119,7 +119,7 @@ boat_tensor_t* boat_conv_layer_forward(boat_conv_layer_t* l, const boat_tensor_t
     const float* pw = bt_dev_read(l->weight);
     const float* pb = (l->use_bias && l->bias) ? bt_dev_read(l->bias) : NULL;
     float* py = bt_dev_write(out);
-    const int mfma = forward_mfma() && k == 3 && conv_forward_wants_mfma(l->in_channels, l->out_channels);
+    const int mfma = forward_mfma() && (k == 3 || k == 5) && conv_forward_wants_mfma(l->in_channels, l->out_channels);
     if (!px || !pw || !py ||
         !boat_hip_ok((mfma ? bh_conv2d_forward_mfma : bh_conv2d_forward)(px, pw, pb, py, batch, (int64_t)l->in_channels, h, w,
                                                                          (int64_t)l->out_channels, k, s, p),

@@ -510,8 +510,8 @@ BOAT_API void boat_hip_optimizer_add_conv(boat_optimizer_t* opt, boat_conv_layer
  * weight, src/layers/conv.c:86-88) instead of the true one; 0: the true one; < 0 (the initial state): whatever
  * reference-exact mode says.  Process-wide. */
 BOAT_API void boat_hip_conv_reference_input_grad(int enable);
-/* 1: boat_conv_layer_forward runs 3x3 layers that are wide enough to gain from it (at least 8 input and 32 output
- * channels, or at least 32 and 16) on the matrix cores: 1.3x to 4x faster; sums in MFMA order: equal to the reference to
+/* 1: boat_conv_layer_forward runs 3x3 and 5x5 layers that are wide enough to gain from it (at least 8 input and 32 output
+ * channels, or at least 32 and 16) on the matrix cores: 1.3x to 6x faster; sums in MFMA order: equal to the reference to
  * fp32 rounding, not bit for bit.  Default 0, or BOAT_HIP_CONV_FORWARD_MFMA. */
 BOAT_API void boat_hip_conv_forward_matrix_cores(int enable);
 BOAT_API void boat_hip_optimizer_add_attention(boat_optimizer_t* opt, boat_attention_t* attention);

@@ -269,7 +269,7 @@ int bh_sdpa_backward_cached(const float* q, const float* k, const float* v, cons
  * true input gradient; flip_taps != 0 pairs each tap with the mirrored weight as conv.c:86-88 does. */
 int bh_conv2d_forward(const float* x, const float* w, const float* bias, float* y, int64_t batch, int64_t in_channels,
                       int64_t height, int64_t width, int64_t out_channels, int64_t kernel, int64_t stride, int64_t pad);
-/* the same forward (conv.c:326-437) as one contraction on the matrix cores, 3x3 kernels only: sums in MFMA order, so it
+/* the same forward (conv.c:326-437) as one contraction on the matrix cores, 3x3 and 5x5 kernels (any stride and padding): sums in MFMA order, so it
  * agrees with the reference to fp32 rounding instead of bit for bit (a max-pooling layer behind it may then pick the other
  * of two nearly equal maxima); several times faster on layers with many channels */
 int bh_conv2d_forward_mfma(const float* x, const float* w, const float* bias, float* y, int64_t batch, int64_t in_channels,

@@ -898,12 +898,17 @@ def test_conv2d_forward_output_channel_tiles(hip, oracle, rng, shape):
     assert np.array_equal(y.numpy(), oracle.conv2d_forward(x, wt, b, stride, pad))
 
 
-CONV_MFMA_SHAPES = [  # batch, ic, h, w, oc, k(=3), stride, pad: ragged channel counts, odd channel counts, strides, two LDS stages
+CONV_MFMA_SHAPES = [  # batch, ic, h, w, oc, k (3 or 5), stride, pad: ragged channel counts, odd channel counts, strides, two LDS stages
     (2, 3, 7, 6, 4, 3, 1, 1), (3, 1, 8, 8, 5, 3, 1, 0), (2, 3, 10, 10, 2, 3, 3, 0), (1, 5, 3, 3, 70, 3, 1, 1),
     (8, 32, 14, 14, 64, 3, 1, 1), (64, 32, 14, 14, 64, 3, 1, 1), (3, 33, 9, 11, 65, 3, 2, 1), (2, 70, 6, 6, 40, 3, 1, 2),
     # more than 256 workgroups: the kernel's two-wavefronts-per-position-tile form
     (40, 33, 20, 21, 65, 3, 1, 1), (64, 64, 28, 28, 64, 3, 1, 1), (30, 70, 31, 29, 130, 3, 2, 1), (40, 5, 21, 20, 10, 3, 1, 1),
     (33, 8, 30, 30, 3, 3, 1, 2),
+    # 5x5 kernels (two 16-channel parts per 32-channel stage): one part, a short second part, an odd count behind a full
+    # part and behind a full stage, several stages, stride 2, more than 256 workgroups
+    (2, 3, 9, 8, 4, 5, 1, 2), (3, 1, 8, 8, 5, 5, 1, 0), (2, 16, 12, 12, 64, 5, 2, 2), (2, 17, 10, 11, 33, 5, 1, 2),
+    (4, 20, 14, 14, 70, 5, 2, 1), (2, 33, 9, 9, 65, 5, 1, 2), (8, 32, 28, 28, 64, 5, 2, 2), (3, 70, 13, 12, 40, 5, 1, 0),
+    (40, 48, 24, 24, 96, 5, 1, 2), (2, 15, 7, 7, 130, 5, 3, 2),
 ]
 
 
@@ -926,30 +931,31 @@ def test_conv2d_forward_on_the_matrix_cores(hip, oracle, rng, shape):
         assert np.linalg.norm(got - want) <= fp32_gemm_bound(ic * k * k) * np.linalg.norm(want)
         assert np.max(np.abs(got - want)) <= 1e-5 * max(1.0, np.abs(want).max())
     with pytest.raises(RuntimeError):
-        hip.check(hip.bh_conv2d_forward_mfma(dx_.ptr, dw_.ptr, None, y.ptr, B, ic, h, w, oc, 5, stride, pad))
+        hip.check(hip.bh_conv2d_forward_mfma(dx_.ptr, dw_.ptr, None, y.ptr, B, ic, h + 4, w + 4, oc, 7, stride, pad))   # 3x3 and 5x5 only
 
 
 def test_conv2d_forward_on_the_matrix_cores_random_shapes(hip, oracle):
-    """Forty seeded random shapes (channel counts on both sides of the 32-channel LDS stage and the 64-channel tile, odd
-    counts, strides 1-3, paddings 0-2, images from 3x3 up, position counts that are no multiple of the 64-position tile)
-    against the oracle at the fp32 bound."""
+    """Eighty seeded random shapes (3x3 and 5x5 kernels, channel counts on both sides of the 16- and 32-channel LDS stages and
+    the 64-channel tile, odd counts, strides 1-3, paddings 0-2, images from the kernel's size up, position counts that are
+    no multiple of the 64-position tile) against the oracle at the fp32 bound."""
     shapes = np.random.default_rng(20250109)
-    for case in range(40):
+    for case in range(80):
+        k = 3 if case < 40 else 5
         B = int(shapes.integers(1, 5))
         ic = int(shapes.choice([1, 2, 3, 7, 8, 16, 31, 32, 33, 48, 65, 70]))
         oc = int(shapes.choice([1, 3, 16, 31, 32, 33, 63, 64, 65, 100, 130]))
-        h, w = int(shapes.integers(3, 20)), int(shapes.integers(3, 20))
+        h, w = int(shapes.integers(k, 20)), int(shapes.integers(k, 20))
         stride, pad = int(shapes.integers(1, 4)), int(shapes.integers(0, 3))
         data = np.random.default_rng(1000 + case)
         x = data.standard_normal((B, ic, h, w)).astype(np.float32)
-        wt = (0.3 * data.standard_normal((oc, ic, 3, 3))).astype(np.float32)
+        wt = (0.3 * data.standard_normal((oc, ic, k, k))).astype(np.float32)
         b = data.standard_normal(oc).astype(np.float32)
-        ho, wo = (h + 2 * pad - 3) // stride + 1, (w + 2 * pad - 3) // stride + 1
+        ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
         y = hip.to_device(np.full((B, oc, ho, wo), np.nan, np.float32))
-        hip.check(hip.bh_conv2d_forward_mfma(dev(hip, x).ptr, dev(hip, wt).ptr, dev(hip, b).ptr, y.ptr, B, ic, h, w, oc, 3, stride, pad))
+        hip.check(hip.bh_conv2d_forward_mfma(dev(hip, x).ptr, dev(hip, wt).ptr, dev(hip, b).ptr, y.ptr, B, ic, h, w, oc, k, stride, pad))
         want = oracle.conv2d_forward(x, wt, b, stride, pad)
         got = y.numpy()
-        shape = (B, ic, h, w, oc, stride, pad)
+        shape = (B, ic, h, w, oc, k, stride, pad)
         assert np.isfinite(got).all(), shape
         assert np.max(np.abs(got - want)) <= 1e-5 * max(1.0, np.abs(want).max()), shape
 

@@ -191,6 +191,57 @@ __global__ __launch_bounds__(kRBlock) void log_softmax_weighted_bwd_kernel(const
     for (int64_t i = lane; i < cols; i += 64) out[i] = c * wr[i] - expf(yr[i]) * g;
 }
 
+// The same for a small matrix, followed in the same launch by the column sums of dz (the bias gradient of the dense layer that
+// produced z): one workgroup, rows dealt to its 16 wavefronts, dz kept in LDS, then fold_rows_kernel's own summation (64
+// columns x 16 row lanes, four running sums each, folded in lane order), so the sums are bh_colsum's bit for bit.
+constexpr int kLswTile = 8192;                  // rows * cols the LDS copy of dz holds
+__global__ __launch_bounds__(kFoldCols * kFoldLanes) void lsw_bwd_colsum_small_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                                                      const float* __restrict__ seed, const float* __restrict__ f,
+                                                                                      float* __restrict__ dz, float* __restrict__ colsum,
+                                                                                      int rows, int cols, int accumulate) {
+    __shared__ float tile[kLswTile];
+    __shared__ float red[kFoldLanes][kFoldCols + 1];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float c = (seed ? seed[0] : 1.0f) * f[0];
+    for (int row = wave; row < rows; row += kFoldCols * kFoldLanes / 64) {
+        const float* yr = y + (int64_t)row * cols;
+        const float* wr = w + (int64_t)row * cols;
+        float g = 0.f;
+        for (int i = lane; i < cols; i += 64) g += c * wr[i];
+        g = wave_sum(g);
+        for (int i = lane; i < cols; i += 64) {
+            const float v = c * wr[i] - expf(yr[i]) * g;
+            dz[(int64_t)row * cols + i] = v;
+            tile[row * cols + i] = v;
+        }
+    }
+    __syncthreads();
+    const int tx = threadIdx.x % kFoldCols, ty = threadIdx.x / kFoldCols;
+    for (int cb = 0; cb < cols; cb += kFoldCols) {
+        const int col = cb + tx;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        if (col < cols) {
+            int r = ty;
+            for (; r + 3 * kFoldLanes < rows; r += 4 * kFoldLanes) {
+                a0 += tile[r * cols + col];
+                a1 += tile[(r + kFoldLanes) * cols + col];
+                a2 += tile[(r + 2 * kFoldLanes) * cols + col];
+                a3 += tile[(r + 3 * kFoldLanes) * cols + col];
+            }
+            for (; r < rows; r += kFoldLanes) a0 += tile[r * cols + col];
+        }
+        red[ty][tx] = (a0 + a1) + (a2 + a3);
+        __syncthreads();
+        if (ty == 0 && col < cols) {
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < kFoldLanes; i++) acc += red[i][tx];
+            colsum[col] = accumulate ? colsum[col] + acc : acc;
+        }
+        __syncthreads();
+    }
+}
+
 // fused softmax + cross-entropy gradient; row_ll receives log_softmax(z)[label] per row
 __global__ __launch_bounds__(kRBlock) void softmax_ce_kernel(const float* __restrict__ z, const int32_t* __restrict__ labels,
                                                              float* __restrict__ dz, float* __restrict__ row_ll,
@@ -341,6 +392,22 @@ int bh_log_softmax_weighted_backward(const float* y, const float* w, const float
     return BH_LAUNCH_CHECK("bh_log_softmax_weighted_backward");
 }
 
+int bh_log_softmax_weighted_backward_colsum(const float* y, const float* w, const float* seed, const float* f, float* dz,
+                                            float* colsum, int64_t rows, int64_t cols, int accumulate) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(rows >= 0 && cols >= 0 && (colsum || cols == 0), "bad argument");
+    if (cols == 0) return BH_OK;
+    if (rows == 0) return accumulate ? BH_OK : bh_memset_zero(colsum, sizeof(float) * (size_t)cols);
+    BH_CHECK_ARG(y && w && f && dz, "null pointer");
+    if (rows <= 256 && rows * cols <= kLswTile) {
+        hipLaunchKernelGGL(lsw_bwd_colsum_small_kernel, dim3(1), dim3(kFoldCols * kFoldLanes), 0, stream(), y, w, seed, f, dz, colsum,
+                           (int)rows, (int)cols, accumulate);
+        return BH_LAUNCH_CHECK("bh_log_softmax_weighted_backward_colsum");
+    }
+    const int rc = bh_log_softmax_weighted_backward(y, w, seed, f, dz, rows, cols);
+    return rc != BH_OK ? rc : bh_colsum(dz, colsum, rows, cols, accumulate);
+}
+
 int bh_softmax_ce_grad(const float* logits, const int32_t* labels, float* dlogits, float* loss_out, int64_t rows,
                        int64_t cols) {
     BH_REQUIRE_INIT();
@@ -353,7 +420,10 @@ int bh_softmax_ce_grad(const float* logits, const int32_t* labels, float* dlogit
     const float f = -1.0f / (float)(size_t)rows;
     hipLaunchKernelGGL(softmax_ce_kernel, dim3((unsigned)ceil_div(rows, kRBlock / 64)), dim3(kRBlock), 0, stream(),
                        logits, labels, dlogits, row_ll, rows, cols, f);
-    if (loss_out) {
+    if (loss_out && rows <= 16 * kRBlock) {   // a few values per lane: the final stage alone sums them (in double)
+        hipLaunchKernelGGL(sum_final_kernel, dim3(1), dim3(kRBlock), 0, stream(), row_ll, loss_out, (int)rows, f);
+        bh_free(row_ll);
+    } else if (loss_out) {
         int blocks = (int)ceil_div(rows, (int64_t)kRBlock * 8);
         if (blocks > 1024) blocks = 1024;
         float* partial = (float*)bh_malloc(sizeof(float) * (size_t)blocks);

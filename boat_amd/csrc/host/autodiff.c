@@ -715,10 +715,22 @@ static bool fuse_log_softmax_loss(boat_variable_t* root, const boat_tensor_t* se
     const float* pf = pw ? bt_dev_read(vf->data) : NULL;
     const float* ps = (pf && seed) ? bt_dev_read(seed) : NULL;
     float* pd = pf ? bt_dev_write(dz) : NULL;
-    if (!pd || (seed && !ps) || !boat_hip_ok(bh_log_softmax_weighted_backward(py, pw, ps, pf, pd, rows, cols), "loss chain backward")) {
+    /* z straight out of a dense layer and read by nothing else: dz is that layer's whole grad_output, and its bias gradient
+     * (the column sums, dense.c:286-291) comes out of the same launch */
+    boat_op_t* zp = z->producer;
+    int acc = 1;
+    float* pgb = (pd && (!seed || ps) && zp && zp->type == OP_DENSE && zp->mark == epoch && z->uses_epoch == epoch && z->walk_uses == 1 &&
+                  !z->grad && z->data->ndim == 2)
+                     ? bt_dense_bias_grad_target((boat_dense_layer_t*)zp->layer, cols, &acc)
+                     : NULL;
+    if (!pd || (seed && !ps) ||
+        !boat_hip_ok(pgb ? bh_log_softmax_weighted_backward_colsum(py, pw, ps, pf, pd, pgb, rows, cols, acc)
+                         : bh_log_softmax_weighted_backward(py, pw, ps, pf, pd, rows, cols),
+                     "loss chain backward")) {
         boat_tensor_free(dz);
         return false;
     }
+    if (pgb) zp->bias_done = epoch;
     r->skip = sum->skip = mul->skip = lsm->skip = epoch;
     accumulate(z, dz, true);
     return true;

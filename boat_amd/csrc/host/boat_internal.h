@@ -145,6 +145,9 @@ boat_tensor_t* boat_layernorm_backward_impl(boat_layernorm_t* norm, const boat_t
 boat_tensor_t* bt_activation_backward_with_dense_bias(int act, const boat_tensor_t* saved, const boat_tensor_t* dy,
                                                       boat_dense_layer_t* layer);
 boat_tensor_t* bt_dense_layer_backward_bias_done(boat_dense_layer_t* layer, const boat_tensor_t* grad_output);
+/* where a rule that computes this layer's grad_output [rows, cols] may add that call's bias gradient itself: the device
+ * pointer of grad_bias and whether to add or to write (NULL: the layer has no bias of that width; nothing is touched) */
+float* bt_dense_bias_grad_target(boat_dense_layer_t* layer, int64_t cols, int* accumulate);
 boat_tensor_t* boat_layernorm_backward_add_impl(boat_layernorm_t* norm, const boat_tensor_t* x, const boat_tensor_t* mean,
                                                 const boat_tensor_t* rstd, const boat_tensor_t* grad_output, const boat_tensor_t* add);
 

@@ -137,6 +137,11 @@ boat_tensor_t* bt_dense_layer_backward_bias_done(boat_dense_layer_t* layer, cons
     bt_flush_exposed();
     return result;
 }
+float* bt_dense_bias_grad_target(boat_dense_layer_t* layer, int64_t cols, int* accumulate) {
+    if (!layer || !(layer->use_bias && layer->bias) || cols != (int64_t)layer->output_features) return NULL;
+    if (!layer->grad_bias) layer->grad_bias = boat_tensor_create_like(layer->bias);
+    return layer->grad_bias ? bt_dev_accumulate(layer->grad_bias, accumulate) : NULL;
+}
 boat_tensor_t* bt_activation_backward_with_dense_bias(int act, const boat_tensor_t* saved, const boat_tensor_t* dy,
                                                       boat_dense_layer_t* layer) {
     if (!layer || !saved || !dy || !(layer->use_bias && layer->bias) || !bt_is_f32(saved) || !bt_is_f32(dy) || dy->ndim != 2 ||

@@ -54,6 +54,7 @@ _SIGS = {
     "bh_log_softmax_forward": (I, [P, P, L, L]), "bh_log_softmax_backward": (I, [P, P, P, L, L]),
     "bh_softmax_ce_grad": (I, [P, P, P, P, L, L]),
     "bh_log_softmax_weighted_backward": (I, [P, P, P, P, P, L, L]),
+    "bh_log_softmax_weighted_backward_colsum": (I, [P, P, P, P, P, P, L, L, I]),
     "bh_layernorm_forward": (I, [P, P, P, P, P, P, L, L, F]),
     "bh_layernorm_backward": (I, [P, P, P, P, P, P, P, P, L, L, I]),
     "bh_layernorm_backward_add": (I, [P, P, P, P, P, P, P, P, P, L, L, I]),

@@ -154,6 +154,11 @@ int bh_log_softmax_backward(const float* y, const float* dy, float* dx, int64_t 
  * separate gradient rules (src/autodiff.c:1115-1147, 1498-1548, 1975-2068), so the result is theirs bit for bit. */
 int bh_log_softmax_weighted_backward(const float* y, const float* w, const float* seed, const float* f, float* dz,
                                      int64_t rows, int64_t cols);
+/* The same, and colsum[c] (+)= sum_r dz[r][c] with it: z came out of a dense layer, so dz is that layer's grad_output and its
+ * column sums are the bias gradient (src/layers/dense.c:286-291).  A small batch (at most 256 rows, 8192 elements) takes one
+ * launch for both; dz and the sums are those of bh_log_softmax_weighted_backward followed by bh_colsum, bit for bit. */
+int bh_log_softmax_weighted_backward_colsum(const float* y, const float* w, const float* seed, const float* f, float* dz,
+                                            float* colsum, int64_t rows, int64_t cols, int accumulate);
 /* fused replacement of the chain log_softmax -> mul(onehot) -> sum -> mul(-1/B) and its backward
  * (examples/mnist/mnist_autodiff.c:397-522): loss_out[0] = -(1/B) sum onehot*log_softmax(z),
  * dlogits = (softmax(z) - onehot)/B.  labels are class indices. */

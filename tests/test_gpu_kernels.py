@@ -313,6 +313,26 @@ def test_loss_chain_backward_kernel(hip, oracle, rng, rows, cols):
         assert np.array_equal(got, dchain.numpy())
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 10), (1, 3), (256, 32), (17, 130), (100, 81), (257, 10), (300, 100)])
+def test_loss_chain_backward_kernel_with_column_sums(hip, oracle, rng, rows, cols):
+    """bh_log_softmax_weighted_backward_colsum: dz and its column sums in one launch (small batches) are, bit for bit,
+    bh_log_softmax_weighted_backward followed by bh_colsum; larger matrices take those two."""
+    z = (3 * rng.standard_normal((rows, cols))).astype(np.float32)
+    y = dev(hip, oracle.log_softmax_forward(z))
+    w = dev(hip, rng.standard_normal((rows, cols)).astype(np.float32))
+    f, seed = dev(hip, np.array([-1.0 / rows], np.float32)), dev(hip, np.array([0.75], np.float32))
+    base = rng.standard_normal(cols).astype(np.float32)
+    dz_a, dz_b, sum_a, sum_b = hip.empty((rows, cols)), hip.empty((rows, cols)), dev(hip, base), dev(hip, base)
+    for acc in (0, 1):
+        hip.check(hip.bh_log_softmax_weighted_backward_colsum(y.ptr, w.ptr, seed.ptr, f.ptr, dz_a.ptr, sum_a.ptr, rows, cols, acc))
+        hip.check(hip.bh_log_softmax_weighted_backward(y.ptr, w.ptr, seed.ptr, f.ptr, dz_b.ptr, rows, cols))
+        hip.check(hip.bh_colsum(dz_b.ptr, sum_b.ptr, rows, cols, acc))
+        assert np.array_equal(dz_a.numpy(), dz_b.numpy()), acc
+        assert np.array_equal(sum_a.numpy(), sum_b.numpy()), acc
+    want = 2 * dz_b.numpy().astype(np.float64).sum(0)
+    assert np.max(np.abs(sum_a.numpy() - want)) <= TOL_RED * max(1e-6, np.abs(dz_b.numpy()).sum(0).max())
+
+
 @pytest.mark.parametrize("rows,cols", [(64, 10), (8, 10), (5, 130)])
 def test_fused_softmax_ce_matches_tape_chain(hip, oracle, rng, rows, cols):
     z = (2 * rng.standard_normal((rows, cols))).astype(np.float32)

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
 
 // ----------------------------------------------------------------- backward
 // grid (s/128, bh); 4 wavefronts, each owns 32 keys (dK, dV rows) and loops over query tiles of 32.
-// Two workgroups fit a CU at head_dim 32 and 64 (69 KB of LDS, <= 256 registers per lane), so a SIMD always has a second
+// Two workgroups fit a CU at head_dim 32 and 64 (71 and 69 KB of LDS, <= 256 registers per lane), so a SIMD always has a second
 // wavefront to run while one waits at a barrier or on LDS; head_dim 128 (119 KB of LDS, 128 accumulator registers for
 // dK and dV alone) runs one workgroup per compute unit.
 // LDS per workgroup: the 128 K rows, one Q tile and one dO tile (refilled through registers between the
@@ -261,15 +261,19 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 template <int D> struct BwdSmem {
     static constexpr int kLd = D + 4;
+    // queries per turn of the loop: 32, or two sub-tiles of 32 at head_dim 32, where a 32-query turn holds half the matrix
+    // work of head_dim 64 for the same two barriers, the same staging and the same dQ store
+    static constexpr int QSUB = D == 32 ? 2 : 1;
+    static constexpr int QROWS = 32 * QSUB;
     static constexpr int K = 128 * kLd;                 // K rows of the workgroup
-    static constexpr int QT = 32 * kLd;                 // one Q (or dO) tile
+    static constexpr int QT = QROWS * kLd;              // one Q (or dO) tile
     static constexpr int kDsLd = 132;                   // dS row stride: 128 keys + 4 pad
     static constexpr int OFF_K = 0;
     static constexpr int OFF_Q = OFF_K + K;
     static constexpr int OFF_DO = OFF_Q + QT;
-    static constexpr int OFF_DS = OFF_DO + QT;          // [32][kDsLd]
-    static constexpr int OFF_STAT = OFF_DS + 32 * kDsLd; // [2][32]: lse*log2e, delta
-    static constexpr int TOTAL = OFF_STAT + 64;
+    static constexpr int OFF_DS = OFF_DO + QT;          // [QROWS][kDsLd]
+    static constexpr int OFF_STAT = OFF_DS + QROWS * kDsLd; // [2][QROWS]: lse*log2e, delta
+    static constexpr int TOTAL = OFF_STAT + 2 * QROWS;
 };
 
 // RAGGED: rows past s are clamped on load; padding keys are masked, padding queries contribute nothing because their
@@ -286,6 +290,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
     extern __shared__ __align__(16) float smem[];
     using Smem = BwdSmem<D>;
     constexpr int kD = D, kLd = D + 4, NT = D / 32, G = D / 8, C4 = D / 4;
+    constexpr int QSUB = Smem::QSUB, QROWS = Smem::QROWS;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
     // tile-major reading of the linear workgroup id, as in the forward kernel: key tile 0, which meets every query tile
@@ -332,23 +337,23 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
     for (int t = 0; t < NT; t++) acc_dk[t] = acc_dv[t] = zero16();
 
-    const int n_qt = RAGGED ? (s + 31) / 32 : s / 32;
-    const int first_qt = CAUSAL ? kv_wg / 32 : 0;   // earlier query tiles see none of this workgroup's keys
+    const int n_qt = RAGGED ? (s + QROWS - 1) / QROWS : s / QROWS;
+    const int first_qt = CAUSAL ? kv_wg / QROWS : 0;   // earlier query tiles see none of this workgroup's keys
     // their partial dQ rows are zero (a mirror launch leaves them as its counterpart wrote them)
     if (!mirror)
-        for (int i = tid; i < first_qt * 32 * (kD / 4); i += 256)
+        for (int i = tid; i < first_qt * QROWS * (kD / 4); i += 256)
             reinterpret_cast<float4*>(dqh)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    // staging: a Q tile and a dO tile are 8 * D float4 each, D / 32 per lane and operand
-    constexpr int PERQ = D / 32;       // 1, 2 or 4
+    // staging: a Q tile and a dO tile are QROWS * D / 4 float4 each, 2 or 4 per lane and operand
+    constexpr int PERQ = QROWS * D / 1024;       // 2, 2 or 4
     float4 qst0, qst1, qst2, qst3, gst0, gst1, gst2, gst3;
     float stat = 0.f;
 #define BWD_LD(i, Q, G_)                                                                                  \
     if constexpr (PERQ > (i)) {                                                                           \
         const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
-        const int grow = RAGGED ? min(qt_ld * 32 + row, s - 1) : qt_ld * 32 + row;                        \
+        const int grow = RAGGED ? min(qt_ld * QROWS + row, s - 1) : qt_ld * QROWS + row;                  \
         Q = *reinterpret_cast<const float4*>(qh + (int64_t)grow * kD + c4 * 4);                           \
         G_ = *reinterpret_cast<const float4*>(gh + (int64_t)grow * kD + c4 * 4);                          \
-        if (RAGGED && qt_ld * 32 + row >= s) G_ = make_float4(0.f, 0.f, 0.f, 0.f);                        \
+        if (RAGGED && qt_ld * QROWS + row >= s) G_ = make_float4(0.f, 0.f, 0.f, 0.f);                     \
     }
 #define BWD_ST(i, Q, G_)                                                                                  \
     if constexpr (PERQ > (i)) {                                                                           \
@@ -360,16 +365,16 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
     {                                                                      \
         const int qt_ld = (QT);                                            \
         BWD_LD(0, qst0, gst0) BWD_LD(1, qst1, gst1) BWD_LD(2, qst2, gst2) BWD_LD(3, qst3, gst3)                    \
-        if (tid < 32) stat = lh[RAGGED ? min(qt_ld * 32 + tid, s - 1) : qt_ld * 32 + tid] * kLog2e;                \
-        else if (tid < 64) {                                                                                       \
-            stat = dh[RAGGED ? min(qt_ld * 32 + tid - 32, s - 1) : qt_ld * 32 + tid - 32];                         \
-            if (RAGGED && qt_ld * 32 + tid - 32 >= s) stat = 0.f;                                                  \
+        if (tid < QROWS) stat = lh[RAGGED ? min(qt_ld * QROWS + tid, s - 1) : qt_ld * QROWS + tid] * kLog2e;       \
+        else if (tid < 2 * QROWS) {                                                                                \
+            stat = dh[RAGGED ? min(qt_ld * QROWS + tid - QROWS, s - 1) : qt_ld * QROWS + tid - QROWS];             \
+            if (RAGGED && qt_ld * QROWS + tid - QROWS >= s) stat = 0.f;                                            \
         }                                                                                                          \
     }
 #define BWD_STAGE_STORE()                                                  \
     {                                                                      \
         BWD_ST(0, qst0, gst0) BWD_ST(1, qst1, gst1) BWD_ST(2, qst2, gst2) BWD_ST(3, qst3, gst3)                    \
-        if (tid < 64) st[tid] = stat;                                      \
+        if (tid < 2 * QROWS) st[tid] = stat;                               \
     }
     if (first_qt < n_qt) {
         BWD_STAGE_LOAD(first_qt)
@@ -395,10 +400,17 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
             for (int j = 0; j < 4; j++) sc_next[j] = *reinterpret_cast<const float4*>(sc_row + (qt + 1) * 32 + 8 * j + 4 * half);
         }
-        const int q0 = qt * 32;
+        const int q0 = qt * QROWS;
+#pragma unroll
+        for (int u = 0; u < QSUB; u++) {                 // the turn's sub-tiles of 32 queries, one after the other
+        const int qu = q0 + 32 * u;
+        const float* qsu = qs + 32 * u * kLd;
+        const float* gsu = gs + 32 * u * kLd;
+        const float* stu = st + 32 * u;
+        float* dsu = dsb + 32 * u * Smem::kDsLd;
         // (head_dim 128 takes no branch here: with 128 accumulator registers flowing around it the kernel would not fit
         // the register file; the masked pairs of the few tiles it would skip contribute exact zeros)
-        if (D == 128 || !CAUSAL || q0 + 31 >= kv0) {
+        if (D == 128 || !CAUSAL || qu + 31 >= kv0) {
             // S = Q.K^T and dP = dO.V^T : query = row (acc_row), key = lane
             floatx16 acc_s = zero16(), acc_dp = zero16();
             // The wavefront's priority rises with its progress through the iteration (1 here, 2 in the row loop, 3 in
@@ -418,7 +430,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
                 floatx16 acc_dp2 = zero16();     // two chains, so that a product never waits for its predecessor
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    const float4 ag = *reinterpret_cast<const float4*>(gs + r * kLd + 8 * g + 4 * half);
+                    const float4 ag = *reinterpret_cast<const float4*>(gsu + r * kLd + 8 * g + 4 * half);
                     const float4 bv = vreg[g];
                     acc_dp = MFMA(ag.x, bv.x, acc_dp);
                     acc_dp2 = MFMA(ag.y, bv.y, acc_dp2);
@@ -431,9 +443,9 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
                 for (int g = 0; g < G; g++) {
                     const int off = r * kLd + 8 * g + 4 * half;
-                    const float4 aq = *reinterpret_cast<const float4*>(qs + off);
+                    const float4 aq = *reinterpret_cast<const float4*>(qsu + off);
                     const float4 bk = *reinterpret_cast<const float4*>(ks + off);
-                    const float4 ag = *reinterpret_cast<const float4*>(gs + off);
+                    const float4 ag = *reinterpret_cast<const float4*>(gsu + off);
                     const float4 bv = vreg[g];
                     acc_s = MFMA(aq.x, bk.x, acc_s);
                     acc_dp = MFMA(ag.x, bv.x, acc_dp);
@@ -452,15 +464,15 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int row = acc_row(e, half);
-                float p = __builtin_amdgcn_exp2f(CACHED ? acc_s[e] - st[row] : acc_s[e] * c1 - st[row]);
+                float p = __builtin_amdgcn_exp2f(CACHED ? acc_s[e] - stu[row] : acc_s[e] * c1 - stu[row]);
                 // masked pairs and padding keys carry no probability (padding queries need no mask: their dO rows
                 // and delta were staged as zeros, so everything they contribute below is zero)
-                if ((CAUSAL && my_key > q0 + row) || key_pad) p = 0.f;
-                const float ds = p * (acc_dp[e] - st[32 + row]) * scale;
-                dsb[row * Smem::kDsLd + w * 32 + r] = ds;
+                if ((CAUSAL && my_key > qu + row) || key_pad) p = 0.f;
+                const float ds = p * (acc_dp[e] - stu[QROWS + row]) * scale;
+                dsu[row * Smem::kDsLd + w * 32 + r] = ds;
                 FloatN<NT> bg, bq;
-                bg.load(gs + row * kLd + NT * r);
-                bq.load(qs + row * kLd + NT * r);
+                bg.load(gsu + row * kLd + NT * r);
+                bq.load(qsu + row * kLd + NT * r);
 #pragma unroll
                 for (int t = 0; t < NT; t++) acc_dv[t] = MFMA(p, bg.v[t], acc_dv[t]);
 #pragma unroll
@@ -469,7 +481,8 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
             __builtin_amdgcn_s_setprio(0);
         } else {
 #pragma unroll
-            for (int e = 0; e < 16; e++) dsb[acc_row(e, half) * Smem::kDsLd + w * 32 + r] = 0.f;
+            for (int e = 0; e < 16; e++) dsu[acc_row(e, half) * Smem::kDsLd + w * 32 + r] = 0.f;
+        }
         }
         __syncthreads();   // dS complete; every wavefront is done with the Q and dO tiles
         if (more) BWD_STAGE_STORE()
@@ -477,7 +490,8 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
         // ct0 .. ct0+NCT-1 of both 16-row tiles (head_dim 32: one column tile of one row tile); lane (i16, kk) reads four
         // consecutive keys of its dS row at once and feeds them to four successive products (the order
         // of the contraction index is free as long as both operands use the same one)
-        constexpr int NCT = D >= 64 ? D / 64 : 1, NRT = D >= 64 ? 2 : 1;
+        // (head_dim 32 with its 64-query turns: column tile w & 1 of row tiles w >> 1 and (w >> 1) + 2)
+        constexpr int NCT = D >= 64 ? D / 64 : 1, NRT = 2, RSTEP = D >= 64 ? 1 : 2;
         const int ct0 = D >= 64 ? w * NCT : (w & 1), rt0 = D >= 64 ? 0 : (w >> 1);
         floatx4 acc_dq[NCT][NRT];
 #pragma unroll
@@ -485,7 +499,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
             for (int t = 0; t < NRT; t++) acc_dq[c][t] = floatx4{0.f, 0.f, 0.f, 0.f};
         __builtin_amdgcn_s_setprio(3);
-        float* dq_row0 = dqh + (int64_t)(q0 + 16 * rt0 + i16) * kD + 16 * ct0 + 4 * kk;   // tile (c, t) at + 16*t rows, + 16*c columns
+        float* dq_row0 = dqh + (int64_t)(q0 + 16 * rt0 + i16) * kD + 16 * ct0 + 4 * kk;   // tile (c, t) at + 16*RSTEP*t rows, + 16*c columns
         // mirror launch (never under a causal mask): what the first launch stored here, in flight while the products below run
         float4 old[CAUSAL ? 1 : NCT][CAUSAL ? 1 : NRT];
         if constexpr (!CAUSAL) {
@@ -494,15 +508,15 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
                 for (int t = 0; t < NRT; t++) {
                     old[c][t] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (mirror && (!RAGGED || q0 + 16 * (rt0 + t) + i16 < s))
-                        old[c][t] = *reinterpret_cast<const float4*>(dq_row0 + (int64_t)16 * t * kD + 16 * c);
+                    if (mirror && (!RAGGED || q0 + 16 * (rt0 + RSTEP * t) + i16 < s))
+                        old[c][t] = *reinterpret_cast<const float4*>(dq_row0 + (int64_t)16 * RSTEP * t * kD + 16 * c);
                 }
         }
-        const int g_lim = CAUSAL ? min(8, (q0 + 32 - kv_wg + 15) / 16) : 8;   // keys past the tile's last query are masked
+        const int g_lim = CAUSAL ? min(8, (q0 + QROWS - kv_wg + 15) / 16) : 8;   // keys past the tile's last query are masked
         for (int g = 0; g < g_lim; g++) {
             float4 a[NRT];
 #pragma unroll
-            for (int t = 0; t < NRT; t++) a[t] = *reinterpret_cast<const float4*>(dsb + (16 * (rt0 + t) + i16) * Smem::kDsLd + 16 * g + 4 * kk);
+            for (int t = 0; t < NRT; t++) a[t] = *reinterpret_cast<const float4*>(dsb + (16 * (rt0 + RSTEP * t) + i16) * Smem::kDsLd + 16 * g + 4 * kk);
             float b[NCT][4];
 #pragma unroll
             for (int c = 0; c < NCT; c++) {
@@ -534,12 +548,12 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
         for (int c = 0; c < NCT; c++)
 #pragma unroll
             for (int t = 0; t < NRT; t++)
-                if (!RAGGED || q0 + 16 * (rt0 + t) + i16 < s) {
+                if (!RAGGED || q0 + 16 * (rt0 + RSTEP * t) + i16 < s) {
                     float4 o = make_float4(acc_dq[c][t][0], acc_dq[c][t][1], acc_dq[c][t][2], acc_dq[c][t][3]);
                     if constexpr (!CAUSAL) {
                         o.x += old[c][t].x; o.y += old[c][t].y; o.z += old[c][t].z; o.w += old[c][t].w;
                     }
-                    *reinterpret_cast<float4*>(dq_row0 + (int64_t)16 * t * kD + 16 * c) = o;
+                    *reinterpret_cast<float4*>(dq_row0 + (int64_t)16 * RSTEP * t * kD + 16 * c) = o;
                 }
         __syncthreads();   // dS tile free again; the next Q and dO tiles are in place
         if (CACHED) {

@@ -1358,6 +1358,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
     int cfg;   // 0 fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256
     int plan_splits = 1;   // k-splits that come with the tile choice
+    double plan_us = 1e30; // what the cost model expects of that choice
     const bool segmented = tab && tab->k_segments > 1;     // one product over several operand pairs: never split
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
@@ -1365,6 +1366,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
         const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0, a_kc || (tab && batch > 1));
         cfg = plan.cfg;
         plan_splits = plan.splits;
+        plan_us = plan.us;
     }
     // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
     if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
@@ -1381,8 +1383,13 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
         cfg = 6;
     // A small output with a very long contraction over k-fast operands (the weight gradient of a convolution: 64 x 288
     // outputs, k = 12544): chunks of 512 k per workgroup of the same kernel, partials folded afterwards.
+    // Its 32x32 tiles read every operand value once per tile row or column, k*m*n/4 bytes in all, at 3.2 TB/s when both
+    // operands are k-fast and 4.3 TB/s with one (measured from 64x288 to 256x256 outputs, k 2048 to 32768); the 128x128
+    // tiles with a cut contraction read a quarter of that and win from about 128x256x12544 on, which the cost model's figure
+    // for them shows (256x256x8192: 43 us here against 31 us there).
     bool tiny_split = false;
-    if (k >= 2048 && tiles32 <= 64 && (a_kc || b_kc) && ceil_div(k, 512) <= 65535) {
+    if (k >= 2048 && tiles32 <= 64 && (a_kc || b_kc) && ceil_div(k, 512) <= 65535 &&
+        8.0 + 0.25 * (double)k * (double)m * (double)n * (double)batch / ((a_kc && b_kc) ? 3.2e6 : 4.3e6) <= plan_us) {
         cfg = 6;
         tiny_split = true;
     }

@@ -405,6 +405,29 @@ def bench_mlp_step(steps, warmup):
                     "mul(onehot), sum, mul(-1/B) and their backward by boat_hip_softmax_cross_entropy"}
 
 
+def bench_block_step_c_caller(steps, warmup):
+    """Config 5a from a C program (boat_amd/examples/block_train_step.c, built beside the library): the same block step as
+    the headline's, written against Boat's C API only, wall ms measured inside the program between two device
+    synchronisations; once with pointers not kept and once in the library's default configuration (the program took the
+    data pointers of its weights, input and target during set-up, so the default keeps those coherent with the host on
+    every call)."""
+    import subprocess
+    exe = ROOT / "boat_amd" / "lib" / "block_train_step"
+    if not exe.exists():
+        raise FileNotFoundError(f"{exe} not found: build it first (python -m boat_amd.build)")
+    out = {}
+    for key, coherent in (("ms", "0"), ("ms_default_coherent_pointers", "1")):
+        env = dict(os.environ, BOAT_HIP_COHERENT_POINTERS=coherent)
+        text = subprocess.run([str(exe), str(steps), str(warmup)], check=True, capture_output=True, text=True, env=env).stdout
+        rec = json.loads(text.strip().splitlines()[-1])
+        assert rec["loss_last"] < rec["loss_first"], f"block training does not reduce the loss: {rec}"
+        out[key] = round(rec["ms_per_step"], 4)
+        out["loss_first_last"] = [rec["loss_first"], rec["loss_last"]]
+    out["note"] = ("the block step (d_model 1024, 16 heads, FFN 4096, seq 512, batch 16: forward, boat_variable_backward, Adam, "
+                   "zero_grad) from a C caller linked against libboat_amd.so, wall clock, flat Adam not included")
+    return out
+
+
 def bench_cnn_step(steps, warmup):
     """The MNIST CNN of examples/mnist/mnist_autodiff.c:536-557 through Boat's C API, batch 64: conv(1->32, 3x3, pad 1),
     relu, maxpool 2, conv(32->64), relu, maxpool 2, flatten, dense 3136->128, relu, dense 128->10, cross-entropy chain;
@@ -874,6 +897,8 @@ def main():
         extra["step_breakdown"] = res["breakdown"]
         extra["transformer_block_step"] = res["block"]
         extra["adam_flat_268M_in_step"] = res["flat_adam"]
+        if not args.no_extra:
+            extra["transformer_block_step"]["c_caller"] = bench_block_step_c_caller(args.steps, args.warmup)
     if "dense" in legs:
         d = bench_dense_backward(hip, args.steps, args.warmup)
         extra["dense_backward_config2"] = {"ms": round(d["ms_per_step"], 4), "bound": "mfma", "step_TFLOPs": d["step_tflops"],

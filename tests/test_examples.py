@@ -35,3 +35,11 @@ def test_mlp_train_step_program_trains():
     assert proc.returncode == 0, proc.stderr[-2000:]
     rec = json.loads(proc.stdout.strip().splitlines()[-1])
     assert rec["steps"] == 50 and rec["loss_last"] < rec["loss_first"]
+
+
+def test_block_train_step_program_trains():
+    """The pre-LN transformer block step of the benchmark as a C program against Boat's API, at a small size."""
+    proc = run_example("block_train_step", 4, 1, 2, 128, 256, 4, 512)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert rec["steps"] == 4 and rec["d_model"] == 256 and 0 < rec["loss_last"] < rec["loss_first"]

@@ -75,7 +75,8 @@ struct GemmArgs {
 //                    c[0] (+)= sum_s op(a[s]) . op(b[s]) (+ bias[0]), seg_k of the contraction per pair
 // (the three input projections of self-attention: one launch for the forward products, one for the three weight
 // gradients, one contraction for the summed input gradient dQ.Wq^T + dK.Wk^T + dV.Wv^T)
-constexpr int kMaxGroups = 3;
+constexpr int kMaxGroups = 4;
+constexpr int kMaxSegments = 3;
 struct GemmTab {
     const float* a[kMaxGroups];
     const float* b[kMaxGroups];
@@ -1590,7 +1591,7 @@ int bh_gemm_grouped(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, i
                     const float* const* b, int64_t ldb, float* const* c, int64_t ldc, const float* const* bias, int accumulate) {
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0, "negative dimension");
-    BH_CHECK_ARG(groups >= 1 && groups <= kMaxGroups, "1 to 3 groups");
+    BH_CHECK_ARG(groups >= 1 && groups <= kMaxGroups, "1 to 4 groups");
     BH_CHECK_ARG(a && b && c, "null table");
     if (m == 0 || n == 0) return BH_OK;
     for (int i = 0; i < groups; i++) BH_CHECK_ARG(a[i] && b[i] && c[i], "null pointer");
@@ -1621,7 +1622,7 @@ int bh_gemm_ksegments(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
                       const float* const* b, int64_t ldb, float* c, int64_t ldc, const float* bias, int accumulate) {
     BH_REQUIRE_INIT();
     BH_CHECK_ARG(m >= 0 && n >= 0 && k >= 0, "negative dimension");
-    BH_CHECK_ARG(segments >= 1 && segments <= kMaxGroups, "1 to 3 segments");
+    BH_CHECK_ARG(segments >= 1 && segments <= kMaxSegments, "1 to 3 segments");
     BH_CHECK_ARG(a && b && c, "null pointer");
     if (m == 0 || n == 0) return BH_OK;
     for (int i = 0; i < segments; i++) BH_CHECK_ARG(a[i] && b[i], "null pointer");

@@ -80,10 +80,10 @@ __global__ __launch_bounds__(kRBlock) void colsum_partial_kernel(const float* __
     partial[(int64_t)blockIdx.y * cols + c] = (a0 + a1) + (a2 + a3);
 }
 
-// the same for up to three matrices of one shape in one launch (blockIdx.z picks the matrix): partial[rb][g*cols + c]
+// the same for up to four matrices of one shape in one launch (blockIdx.z picks the matrix): partial[rb][g*cols + c]
 struct ColsumTab {
-    const float* x[3];
-    float* out[3];
+    const float* x[4];
+    float* out[4];
 };
 __global__ __launch_bounds__(kRBlock) void colsum_partial_tab_kernel(ColsumTab t, float* __restrict__ partial, int64_t rows, int64_t cols) {
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -332,11 +332,11 @@ int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumu
         return BH_LAUNCH_CHECK(name);                                                                          \
     } while (0)
 
-// out[g][c] (+)= sum_r x[g][r][c] for up to three matrices of one shape: one partial launch and one fold where bh_colsum
+// out[g][c] (+)= sum_r x[g][r][c] for up to four matrices of one shape: one partial launch and one fold where bh_colsum
 // takes two per matrix; the sums and their order are bh_colsum's, so the results are the same bits
 int bh_colsum_grouped(const float* const* x, float* const* out, int groups, int64_t rows, int64_t cols, int accumulate) {
     BH_REQUIRE_INIT();
-    BH_CHECK_ARG(groups >= 1 && groups <= 3 && rows >= 0 && cols >= 0 && x && out, "bad argument");
+    BH_CHECK_ARG(groups >= 1 && groups <= 4 && rows >= 0 && cols >= 0 && x && out, "bad argument");
     if (cols == 0) return BH_OK;
     for (int g = 0; g < groups; g++) BH_CHECK_ARG(out[g] && (x[g] || rows == 0), "null pointer");
     if (groups == 1 || rows <= 256) {

@@ -775,74 +775,48 @@ void boat_apply_rotary_embedding(boat_tensor_t* query, boat_tensor_t* key, size_
     (void)query; (void)key; (void)seq_len; (void)head_size; (void)theta;
 }
 
-/* linear_projection_backward, attention.c:1186-1285: dx = dy.w^T ; *gw = x^T.dy ; *gb = colsum(dy), all overwritten */
-/* `into` non-NULL: dx is added into that tensor by the GEMM's epilogue (and a new reference to it is returned) instead of
- * being written to a new one */
-static boat_tensor_t* project_backward(const boat_tensor_t* x, const boat_tensor_t* w, const boat_tensor_t* bias,
-                                       const boat_tensor_t* dy, boat_tensor_t** gw, boat_tensor_t** gb, int64_t rows, int64_t h,
-                                       boat_tensor_t* into) {
-    boat_tensor_t* dx = into ? into : bt_new_like_uninit(x);
-    if (into) boat_tensor_ref(into);
-    if (!*gw) *gw = boat_tensor_create_like(w);
-    if (bias && !*gb) *gb = boat_tensor_create_like(bias);
-    if (!dx || !*gw || (bias && !*gb)) {
-        boat_tensor_free(dx);
-        return NULL;
-    }
-    const float* px = bt_dev_read(x);
-    const float* pw = bt_dev_read(w);
-    const float* pdy = bt_dev_read(dy);
-    float* pdx = into ? bt_dev_rw(dx) : bt_dev_write(dx);
-    float* pgw = bt_dev_write(*gw);
-    float* pgb = bias ? bt_dev_write(*gb) : NULL;
-    bool ok = px && pw && pdy && pdx && pgw;
-    /* dx (+)= dy.w^T ; gw = x^T.dy ; gb = colsum(dy) */
-    if (ok) ok = boat_hip_ok(bh_dense_backward_into(px, pw, pdy, pdx, pgw, pgb, rows, h, h, 0, into ? 1 : 0), "attention projection backward");
-    if (!ok) {
-        boat_tensor_free(dx);
-        return NULL;
-    }
-    return dx;
-}
-
+/* linear_projection_backward, attention.c:1186-1285, for the four projections: dx = dy.w^T ; *gw = x^T.dy ; *gb = colsum(dy),
+ * all overwritten */
 /* the backward of the three input projections; sum: *gq = dq.Wq^T + dk.Wk^T + dv.Wv^T and *gk, *gv are further
- * references to it */
+ * references to it.  The parameter gradients of the output projection (x^T.dy and colsum(dy) of attention output and
+ * grad_output) have the same shapes and depend on nothing computed in between, so they ride along as a fourth group. */
 static bool project_backward3(boat_attention_t* a, const boat_tensor_t* dqp, const boat_tensor_t* dkp, const boat_tensor_t* dvp,
-                              int64_t rows, int64_t h, bool sum, boat_tensor_t** gq, boat_tensor_t** gk, boat_tensor_t** gv) {
-    const boat_tensor_t* x[3] = {a->cache_query, a->cache_key, a->cache_value};
-    const boat_tensor_t* w[3] = {a->weight_q, a->weight_k, a->weight_v};
-    const boat_tensor_t* bias[3] = {a->bias_q, a->bias_k, a->bias_v};
-    const boat_tensor_t* dy[3] = {dqp, dkp, dvp};
-    boat_tensor_t** gw[3] = {&a->grad_weight_q, &a->grad_weight_k, &a->grad_weight_v};
-    boat_tensor_t** gb[3] = {&a->grad_bias_q, &a->grad_bias_k, &a->grad_bias_v};
+                              const boat_tensor_t* grad_output, int64_t rows, int64_t h, bool sum, boat_tensor_t** gq,
+                              boat_tensor_t** gk, boat_tensor_t** gv) {
+    const boat_tensor_t* x[4] = {a->cache_query, a->cache_key, a->cache_value, a->cache_attention_output};
+    const boat_tensor_t* w[4] = {a->weight_q, a->weight_k, a->weight_v, a->weight_o};
+    const boat_tensor_t* bias[4] = {a->bias_q, a->bias_k, a->bias_v, a->bias_o};
+    const boat_tensor_t* dy[4] = {dqp, dkp, dvp, grad_output};
+    boat_tensor_t** gw[4] = {&a->grad_weight_q, &a->grad_weight_k, &a->grad_weight_v, &a->grad_weight_o};
+    boat_tensor_t** gb[4] = {&a->grad_bias_q, &a->grad_bias_k, &a->grad_bias_v, &a->grad_bias_o};
     boat_tensor_t* dx[3] = {NULL, NULL, NULL};
-    const float *px[3], *pw[3], *pdy[3];
-    float *pgw[3], *pdx[3];
+    const float *px[4], *pw[4], *pdy[4];
+    float *pgw[4], *pdx[3];
     bool ok = true;
-    for (int i = 0; i < 3 && ok; i++) {
+    for (int i = 0; i < 4 && ok; i++) {
         if (!*gw[i]) *gw[i] = boat_tensor_create_like(w[i]);
         if (bias[i] && !*gb[i]) *gb[i] = boat_tensor_create_like(bias[i]);
-        if (i == 0 || !sum) dx[i] = bt_new_like_uninit(x[i]);
-        ok = *gw[i] && (!bias[i] || *gb[i]) && (dx[i] || (sum && i > 0));
+        if (i < 3 && (i == 0 || !sum)) dx[i] = bt_new_like_uninit(x[i]);
+        ok = *gw[i] && (!bias[i] || *gb[i]) && (i == 3 || dx[i] || (sum && i > 0));
         if (!ok) break;
         px[i] = bt_dev_read(x[i]);
         pw[i] = bt_dev_read(w[i]);
         pdy[i] = bt_dev_read(dy[i]);
         pgw[i] = bt_dev_write(*gw[i]);
-        pdx[i] = dx[i] ? bt_dev_write(dx[i]) : NULL;
-        ok = px[i] && pw[i] && pdy[i] && pgw[i] && (pdx[i] || !dx[i]);
+        if (i < 3) pdx[i] = dx[i] ? bt_dev_write(dx[i]) : NULL;
+        ok = px[i] && pw[i] && pdy[i] && pgw[i] && (i == 3 || pdx[i] || !dx[i]);
     }
     /* dx = dy.w^T */
     if (ok && sum) ok = boat_hip_ok(bh_gemm_ksegments(0, 1, rows, h, h, 3, pdy, h, pw, h, pdx[0], h, NULL, 0), "attention input gradient");
     else if (ok) ok = boat_hip_ok(bh_gemm_grouped(0, 1, rows, h, h, 3, pdy, h, pw, h, pdx, h, NULL, 0), "attention input gradients");
-    /* gw = x^T.dy (overwritten per call, attention.c:1262-1279) */
-    if (ok) ok = boat_hip_ok(bh_gemm_grouped(1, 0, h, h, rows, 3, px, h, pdy, h, pgw, h, NULL, 0), "attention weight gradients");
-    /* gb = colsum(dy): the three in one pair of launches when all three projections have a bias */
-    if (ok && bias[0] && bias[1] && bias[2]) {
-        float* pgb[3] = {bt_dev_write(*gb[0]), bt_dev_write(*gb[1]), bt_dev_write(*gb[2])};
-        ok = pgb[0] && pgb[1] && pgb[2] && boat_hip_ok(bh_colsum_grouped(pdy, pgb, 3, rows, h, 0), "attention bias gradients");
+    /* gw = x^T.dy (overwritten per call, attention.c:1262-1279): the four in one launch */
+    if (ok) ok = boat_hip_ok(bh_gemm_grouped(1, 0, h, h, rows, 4, px, h, pdy, h, pgw, h, NULL, 0), "attention weight gradients");
+    /* gb = colsum(dy): the four in one pair of launches when all projections have a bias */
+    if (ok && bias[0] && bias[1] && bias[2] && bias[3]) {
+        float* pgb[4] = {bt_dev_write(*gb[0]), bt_dev_write(*gb[1]), bt_dev_write(*gb[2]), bt_dev_write(*gb[3])};
+        ok = pgb[0] && pgb[1] && pgb[2] && pgb[3] && boat_hip_ok(bh_colsum_grouped(pdy, pgb, 4, rows, h, 0), "attention bias gradients");
     } else {
-        for (int i = 0; i < 3 && ok; i++) {
+        for (int i = 0; i < 4 && ok; i++) {
             float* pgb = bias[i] ? bt_dev_write(*gb[i]) : NULL;
             if (bias[i]) ok = pgb && boat_hip_ok(bh_colsum(pdy[i], pgb, rows, h, 0), "attention bias gradient");
         }
@@ -912,10 +886,17 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
         fprintf(stderr, "[ERROR] boat_attention_backward: grad_output shape mismatch\n");
         return false;
     }
-    /* 1. output projection */
-    boat_tensor_t* d_ao = project_backward(a->cache_attention_output, a->weight_o, a->bias_o, grad_output, &a->grad_weight_o,
-                                           &a->grad_bias_o, rows, h, NULL);
-    if (!d_ao) return false;
+    /* 1. output projection: its input gradient now, its parameter gradients with those of the input projections (step 3) */
+    boat_tensor_t* d_ao = bt_new_like_uninit(a->cache_attention_output);
+    {
+        const float* pdy = bt_dev_read(grad_output);
+        const float* pwo = bt_dev_read(a->weight_o);
+        float* pd = d_ao ? bt_dev_write(d_ao) : NULL;
+        if (!pdy || !pwo || !pd || !boat_hip_ok(bh_gemm(0, 1, rows, h, h, pdy, h, pwo, h, pd, h, NULL, 0, 1), "attention output projection backward")) {
+            boat_tensor_free(d_ao);
+            return false;
+        }
+    }
     /* 2. attention core on [B*nh, S, hd] blocks */
     boat_tensor_t* dqp = bt_new_like_uninit(q);
     boat_tensor_t* dkp = bt_new_like_uninit(q);
@@ -948,7 +929,7 @@ static bool attention_backward_unflushed(boat_attention_t* a, const boat_tensor_
      * self-attention through the tape, as ONE product whose contraction runs over the three (dY, W) pairs */
     boat_tensor_t *gq = NULL, *gk = NULL, *gv = NULL;
     const bool sum = g_sum_into != NULL;
-    if (ok) ok = project_backward3(a, dqp, dkp, dvp, rows, h, sum, &gq, &gk, &gv);
+    if (ok) ok = project_backward3(a, dqp, dkp, dvp, grad_output, rows, h, sum, &gq, &gk, &gv);
     boat_tensor_free(dqp);
     boat_tensor_free(dkp);
     boat_tensor_free(dvp);

@@ -141,8 +141,8 @@ int bh_sgd_update(float* p, float* g, float lr, int64_t n, int zero_grad);      
 /* ---- reductions / softmax (src/ops/arithmetic.c:611-691; src/autodiff.c:1701-2068; dense.c:286-291) ---- */
 int bh_sum_all(const float* x, float* out1, int64_t n);
 int bh_colsum(const float* x, float* out, int64_t rows, int64_t cols, int accumulate);
-/* the same for up to 3 matrices of one shape in one pair of launches (the bias gradients of a self-attention layer's three
- * input projections, src/layers/attention.c:1262-1279 three times); the same sums in the same order as bh_colsum */
+/* the same for up to 4 matrices of one shape in one pair of launches (the bias gradients of an attention layer's four
+ * projections, src/layers/attention.c:1262-1279 four times); the same sums in the same order as bh_colsum */
 int bh_colsum_grouped(const float* const* x, float* const* out, int groups, int64_t rows, int64_t cols, int accumulate); /* db (+)= sum_rows dY */
 int bh_softmax_forward(const float* x, float* y, int64_t rows, int64_t cols);
 int bh_softmax_backward(const float* y, const float* dy, float* dx, int64_t rows, int64_t cols);
@@ -214,10 +214,10 @@ int bh_layernorm_backward_noalloc(const float* x, const float* gamma, const floa
 int bh_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
             const float* a, int64_t lda, const float* b, int64_t ldb,
             float* c, int64_t ldc, const float* bias, int accumulate, int64_t batch);
-/* Up to 3 products of ONE shape whose operands are separate tensors: c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g]), arguments
+/* Up to 4 products of ONE shape whose operands are separate tensors: c[g] (+)= op(a[g]) . op(b[g]) (+ bias[g]), arguments
  * as bh_gemm with tables of `groups` pointers (bias may be NULL, or hold NULLs).  The three input projections of a
- * self-attention layer (src/layers/attention.c:363-365: the same input times Wq, Wk, Wv) and their three weight gradients
- * (:1186-1285 run three times) are one launch each this way, with the kernels of bh_gemm; the number of cuts of a long
+ * self-attention layer (src/layers/attention.c:363-365: the same input times Wq, Wk, Wv) and the weight gradients of its
+ * four projections (:1186-1285 run four times) are one launch each this way, with the kernels of bh_gemm; the number of cuts of a long
  * contraction is chosen for the group as a whole, so a product agrees with a separate bh_gemm call to fp32 rounding. */
 int bh_gemm_grouped(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int groups,
                     const float* const* a, int64_t lda, const float* const* b, int64_t ldb,

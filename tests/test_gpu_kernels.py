@@ -233,19 +233,20 @@ def test_colsum(hip, rng, rows, cols):
     assert np.max(np.abs(out.numpy() - 2 * want)) <= 2 * TOL_RED * np.abs(x).sum(0).max()
 
 
+@pytest.mark.parametrize("groups", [3, 4])
 @pytest.mark.parametrize("rows,cols", [(8192, 1024), (1000, 37), (300, 4096), (64, 10)])
-def test_colsum_grouped(hip, rng, rows, cols):
-    """bh_colsum_grouped: three matrices in one pair of launches give bh_colsum's bits for each, with and without
+def test_colsum_grouped(hip, rng, rows, cols, groups):
+    """bh_colsum_grouped: three or four matrices in one pair of launches give bh_colsum's bits for each, with and without
     accumulation (few rows fall back to bh_colsum itself)."""
     import ctypes as C
-    xs = [rng.standard_normal((rows, cols)).astype(np.float32) for _ in range(3)]
+    xs = [rng.standard_normal((rows, cols)).astype(np.float32) for _ in range(groups)]
     dxs = [dev(hip, x) for x in xs]
-    outs = [hip.zeros(cols) for _ in range(3)]
-    singles = [hip.zeros(cols) for _ in range(3)]
-    tab = lambda arrs: (C.c_void_p * 3)(*[a.ptr for a in arrs])
+    outs = [hip.zeros(cols) for _ in range(groups)]
+    singles = [hip.zeros(cols) for _ in range(groups)]
+    tab = lambda arrs: (C.c_void_p * groups)(*[a.ptr for a in arrs])
     for acc in (0, 1):
-        hip.check(hip.bh_colsum_grouped(tab(dxs), tab(outs), 3, rows, cols, acc))
-        for g in range(3):
+        hip.check(hip.bh_colsum_grouped(tab(dxs), tab(outs), groups, rows, cols, acc))
+        for g in range(groups):
             hip.check(hip.bh_colsum(dxs[g].ptr, singles[g].ptr, rows, cols, acc))
             assert np.array_equal(outs[g].numpy(), singles[g].numpy()), (acc, g)
             want = (1 + acc) * xs[g].sum(0, dtype=np.float64)
@@ -560,18 +561,20 @@ def _ptr_table(arrays):
 
 @pytest.mark.parametrize("force", [None, 1, 2, 3, 4])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
-@pytest.mark.parametrize("m,n,k,accumulate,bias,shared_a", [
-    (512, 384, 256, False, True, True),      # the forward projections' form: one input, three weights, three biases
-    (260, 132, 96, True, True, False),       # ragged edge tiles, accumulate
-    (256, 384, 2048, True, False, True),     # split-K: partials of the three groups folded by one launch
-    (40, 24, 12, False, False, False),       # no table kernel for this shape: the groups run one after the other
+@pytest.mark.parametrize("m,n,k,accumulate,bias,shared_a,groups", [
+    (512, 384, 256, False, True, True, 3),   # the forward projections' form: one input, three weights, three biases
+    (260, 132, 96, True, True, False, 3),    # ragged edge tiles, accumulate
+    (256, 384, 2048, True, False, True, 3),  # split-K: partials of the three groups folded by one launch
+    (40, 24, 12, False, False, False, 3),    # no table kernel for this shape: the groups run one after the other
+    (256, 256, 2048, False, False, False, 4),   # four groups (the weight gradients of an attention layer's four projections), split-K
+    (260, 132, 96, True, True, False, 4),
+    (384, 256, 64, False, True, False, 2),
 ])
-def test_gemm_grouped_equals_separate_launches(hip, rng, force, ta, tb, m, n, k, accumulate, bias, shared_a):
-    """bh_gemm_grouped (three products of one shape in one launch, operands from pointer tables) against float64 and
-    against the same three products through bh_gemm: bit for bit where the contraction is too short to be cut (the grouped
+def test_gemm_grouped_equals_separate_launches(hip, rng, force, ta, tb, m, n, k, accumulate, bias, shared_a, groups):
+    """bh_gemm_grouped (two to four products of one shape in one launch, operands from pointer tables) against float64 and
+    against the same products through bh_gemm: bit for bit where the contraction is too short to be cut (the grouped
     kernels walk a product as bh_gemm does), to fp32 rounding otherwise (the number of cuts is chosen for the group as a
     whole, and partial sums are added in another order)."""
-    groups = 3
     a = [rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32) for _ in range(1 if shared_a else groups)]
     if shared_a:
         a = a * groups

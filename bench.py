@@ -46,10 +46,10 @@ GEMM_TRAFFIC_BYTES_CONFIG2 = int(((2.0 * 779903.4 + 131072.0) + (2.0 * 557368.4 
 # the bytes the same two launches need at least: dX reads dY and W and writes dX (335.5 MB), dW reads X and dY, reads and
 # writes dW (402.7 MB)
 GEMM_ALGORITHMIC_BYTES_CONFIG2 = int((335.5e6 + 402.7e6) / 2)
-# HBM bytes per GEMM launch of the block training step, averaged over the step's 12 launches (same file, same counters)
-GEMM_TRAFFIC_BYTES_STEP = 379_300_000
-# what the step's 12 GEMM launches need at least (each operand read once, each output written once): 1,929 MB
-GEMM_ALGORITHMIC_BYTES_STEP = 1_929_000_000 // 12
+# HBM bytes per GEMM launch of the block training step, averaged over the step's 11 launches (same file, same counters)
+GEMM_TRAFFIC_BYTES_STEP = 398_000_000
+# what the step's 11 GEMM launches need at least (each operand read once, each output written once): 1,929 MB
+GEMM_ALGORITHMIC_BYTES_STEP = 1_929_000_000 // 11
 
 
 def parse_args():

@@ -467,7 +467,7 @@ void bt_flush_exposed(void) {
         if (st->pending) {
             st->pending = false;
             if (landed) {
-                memcpy(st->host, st->shadow, st->nbytes);
+                bt_bytes_copy(st->host, st->shadow, st->nbytes);
                 st->host_valid = true;
                 st->shadow_valid = true;
             }
@@ -487,7 +487,7 @@ static bool storage_host_ready(boat_storage_t* st) {
             if (!boat_hip_ok(bh_memcpy_d2h(st->host, bh_buffer_ptr(st->dev), st->nbytes), "tensor download")) return false;
             stream_synced();
             if (st->shadow) {          /* mirror and device agree again: so does the shadow */
-                memcpy(st->shadow, st->host, st->nbytes);
+                bt_bytes_copy(st->shadow, st->host, st->nbytes);
                 st->shadow_valid = true;
             }
         } else {
@@ -511,13 +511,13 @@ static bool storage_dev_ready(boat_storage_t* st, bool need_contents) {
     /* an exposed tensor may have been written through the caller's pointer since the last upload: it was not if the
      * mirror still equals the shadow, the copy of what was uploaded or written back last */
     if (need_contents && st->exposed && !st->pending && st->host_valid &&
-        !(st->dev_valid && st->shadow && st->shadow_valid && memcmp(st->host, st->shadow, st->nbytes) == 0))
+        !(st->dev_valid && st->shadow && st->shadow_valid && bt_bytes_equal(st->host, st->shadow, st->nbytes)))
         st->dev_valid = false;
     if (need_contents && !st->dev_valid) {
         if (st->host_valid && shadow_ensure(st)) {
             /* staged: the caller may overwrite the mirror as soon as this call returns, the queued copy reads the shadow */
             shadow_settle(st);
-            memcpy(st->shadow, st->host, st->nbytes);
+            bt_bytes_copy(st->shadow, st->host, st->nbytes);
             if (!boat_hip_ok(bh_memcpy_h2d_async(bh_buffer_ptr(st->dev), st->shadow, st->nbytes), "tensor upload")) return false;
             st->upload_ticket = ++g_ticket;
             st->shadow_valid = true;

@@ -43,3 +43,23 @@ def test_block_train_step_program_trains():
     assert proc.returncode == 0, proc.stderr[-2000:]
     rec = json.loads(proc.stdout.strip().splitlines()[-1])
     assert rec["steps"] == 4 and rec["d_model"] == 256 and 0 < rec["loss_last"] < rec["loss_first"]
+
+
+def test_block_train_step_with_kept_pointers_and_large_tensors():
+    """The same program in the default configuration (pointers to the weights, the input and the target stay valid, so
+    the library compares and copies their buffers around every call) at a size where those buffers are large enough
+    for the helper threads (FFN weights and activations of 8 MiB and more): the losses must be the ones of the run in
+    which nothing is kept coherent."""
+    import os
+    args = ("block_train_step", 3, 1, 8, 512, 1024, 16, 2048)
+    exe = LIB_DIR / args[0]
+    if not exe.exists():
+        pytest.fail(f"{exe} is missing: build it first (python -m boat_amd.build)")
+    recs = []
+    for mode in ("1", "0"):
+        env = dict(os.environ, BOAT_HIP_COHERENT_POINTERS=mode)
+        proc = subprocess.run([str(exe), *map(str, args[1:])], capture_output=True, text=True, timeout=110, env=env)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        recs.append(json.loads(proc.stdout.strip().splitlines()[-1]))
+    assert recs[0]["loss_first"] == recs[1]["loss_first"] and recs[0]["loss_last"] == recs[1]["loss_last"]
+    assert 0 < recs[0]["loss_last"] < recs[0]["loss_first"]

@@ -354,6 +354,11 @@ int bh_event_record(bh_event_t* e) {
     BH_CHECK_ARG(e, "null event");
     return check_hip(hipEventRecord(e->ev, g_stream), "hipEventRecord");
 }
+int bh_event_wait(bh_event_t* e) {
+    BH_REQUIRE_INIT();
+    BH_CHECK_ARG(e, "null event");
+    return check_hip(hipEventSynchronize(e->ev), "hipEventSynchronize");
+}
 float bh_event_elapsed_ms(bh_event_t* a, bh_event_t* b) {
     if (!a || !b) return -1.f;
     if (hipEventSynchronize(b->ev) != hipSuccess) return -1.f;

@@ -66,7 +66,7 @@ float* bt_dev_rw(boat_tensor_t* t);
  * pointer for `t += contribution`: while t is in the zero state the kernel may overwrite instead (*accumulate = 0), so
  * the zeros are never written and never read back. */
 bool bt_set_zero(boat_tensor_t* t);
-/* memcmp(a, b, n) == 0 and memcpy for the buffers of exposed tensors: on a few threads from 8 MiB on (parbytes.c) */
+/* memcmp(a, b, n) == 0 and memcpy for the buffers of exposed tensors: on a few threads from 2 MiB on (parbytes.c) */
 bool bt_bytes_equal(const void* a, const void* b, size_t n);
 void bt_bytes_copy(void* dst, const void* src, size_t n);
 bool bt_is_zero(const boat_tensor_t* t);

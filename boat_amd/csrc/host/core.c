@@ -439,18 +439,45 @@ static void mark_device_write(boat_storage_t* st) {
     g_pending[g_pending_n++] = st;
 }
 
+/* One event per queued write-back when a call writes back several large tensors: the copy shadow -> mirror of one tensor
+ * then runs while the next tensors are still crossing PCIe, instead of after a wait for all of them. */
+static const size_t kPipelinedFlushMin = (size_t)8 << 20;
+static bh_event_t** g_flush_events = NULL;
+static size_t g_flush_events_n = 0;
+static bool flush_events_ensure(size_t n) {
+    if (n <= g_flush_events_n) return true;
+    bh_event_t** grown = (bh_event_t**)realloc(g_flush_events, n * sizeof(*grown));
+    if (!grown) return false;
+    g_flush_events = grown;
+    while (g_flush_events_n < n) {
+        bh_event_t* e = bh_event_create();
+        if (!e) return false;
+        g_flush_events[g_flush_events_n++] = e;
+    }
+    return true;
+}
+
 void bt_flush_exposed(void) {
     if (g_pending_n == 0) return;
-    /* storages with a shadow: all copies queued, one wait, then shadow -> mirror; the others one waiting copy each */
-    size_t queued = 0;
+    /* storages with a shadow: all copies queued, then shadow -> mirror as they land; the others one waiting copy each */
+    size_t queued = 0, queued_bytes = 0, shadowed = 0;
+    for (size_t i = 0; i < g_pending_n; i++) {
+        boat_storage_t* st = g_pending[i];
+        if (st->refs > 1 && st->host && st->dev && st->dev_valid && !st->host_valid && st->exposed && st->nbytes && st->nbytes <= kShadowLimit) {
+            shadowed++;
+            queued_bytes += st->nbytes;
+        }
+    }
+    const bool pipelined = shadowed > 1 && queued_bytes >= kPipelinedFlushMin && flush_events_ensure(shadowed);
     for (size_t i = 0; i < g_pending_n; i++) {
         boat_storage_t* st = g_pending[i];
         st->pending = false;
         if (!(st->refs > 1 && st->host && st->dev && st->dev_valid && !st->host_valid)) continue;
         if (shadow_ensure(st)) {
             shadow_settle(st);
-            if (boat_hip_ok(bh_memcpy_d2h_async(st->shadow, bh_buffer_ptr(st->dev), st->nbytes), "write-back of an exposed tensor")) {
-                st->pending = true;   /* marks: copy queued */
+            if (boat_hip_ok(bh_memcpy_d2h_async(st->shadow, bh_buffer_ptr(st->dev), st->nbytes), "write-back of an exposed tensor") &&
+                (!pipelined || queued >= g_flush_events_n || boat_hip_ok(bh_event_record(g_flush_events[queued]), "write-back of an exposed tensor"))) {
+                st->pending = true;   /* marks: copy queued (the queued-th of this call) */
                 queued++;
                 continue;
             }
@@ -460,20 +487,28 @@ void bt_flush_exposed(void) {
             stream_synced();
         }
     }
-    const bool landed = queued > 0 && boat_hip_ok(bh_synchronize(), "write-back of exposed tensors");
+    const bool per_copy = pipelined && queued <= g_flush_events_n;
+    bool landed = queued > 0 && !per_copy && boat_hip_ok(bh_synchronize(), "write-back of exposed tensors");
     if (landed) stream_synced();
-    while (g_pending_n > 0) {
-        boat_storage_t* st = g_pending[--g_pending_n];
+    size_t nth = 0;
+    for (size_t i = 0; i < g_pending_n; i++) {
+        boat_storage_t* st = g_pending[i];
         if (st->pending) {
             st->pending = false;
+            if (per_copy) landed = boat_hip_ok(bh_event_wait(g_flush_events[nth]), "write-back of exposed tensors");
+            nth++;
             if (landed) {
                 bt_bytes_copy(st->host, st->shadow, st->nbytes);
                 st->host_valid = true;
                 st->shadow_valid = true;
             }
         }
-        storage_unref(st);
     }
+    if (per_copy && landed && nth > 0) stream_synced();   /* the last event is behind everything queued before it */
+    /* (a storage freed by the unref below may wait for the stream itself: only after every copy of this call was handled) */
+    const size_t n = g_pending_n;
+    g_pending_n = 0;
+    for (size_t i = 0; i < n; i++) storage_unref(g_pending[i]);
 }
 
 static bool storage_host_ready(boat_storage_t* st) {

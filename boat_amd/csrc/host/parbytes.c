@@ -14,7 +14,7 @@
 #include <unistd.h>
 
 enum { kHelpers = 3 };
-static const size_t kParallelMin = (size_t)8 << 20;
+static const size_t kParallelMin = (size_t)2 << 20;
 
 typedef struct {
     const char* a;      /* compare: first operand; copy: source */

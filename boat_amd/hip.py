@@ -32,7 +32,7 @@ _SIGS = {
     "bh_host_alloc": (P, [Z]), "bh_host_free": (None, [P]), "bh_memcpy_h2d_async": (I, [P, P, Z]), "bh_memcpy_d2h_async": (I, [P, P, Z]),
     "bh_memcpy_h2d": (I, [P, P, Z]), "bh_memcpy_d2h": (I, [P, P, Z]), "bh_memcpy_d2d": (I, [P, P, Z]),
     "bh_memset_zero": (I, [P, Z]),
-    "bh_event_create": (P, []), "bh_event_destroy": (None, [P]), "bh_event_record": (I, [P]),
+    "bh_event_create": (P, []), "bh_event_destroy": (None, [P]), "bh_event_record": (I, [P]), "bh_event_wait": (I, [P]),
     "bh_event_elapsed_ms": (F, [P, P]),
     "bh_profile_enable": (I, [I]),
     "bh_profile_read": (I, [I, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(L)]),

@@ -63,11 +63,12 @@ void  bh_host_free(void* p);
 int bh_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t nbytes);
 int bh_memcpy_d2h_async(void* dst_pinned, const void* src_dev, size_t nbytes);
 
-/* events on the library stream, for timing */
+/* events on the library stream: for timing, and for waiting until the stream has passed one queued copy among several */
 typedef struct bh_event bh_event_t;
 bh_event_t* bh_event_create(void);
 void        bh_event_destroy(bh_event_t* e);
 int         bh_event_record(bh_event_t* e);
+int         bh_event_wait(bh_event_t* e);                                /* returns when the stream has passed the record */
 float       bh_event_elapsed_ms(bh_event_t* start, bh_event_t* stop);    /* synchronises on stop */
 
 /* ---- per-class timing of the library's own launches, for benchmarks that drive whole training steps through Boat's API

@@ -46,7 +46,7 @@ static int check(size_t n) {
 }
 
 int main(void) {
-    const size_t sizes[] = {0, 1, 4095, 4096, (size_t)1 << 20, ((size_t)8 << 20) - 1, (size_t)8 << 20, ((size_t)8 << 20) + 4097,
+    const size_t sizes[] = {0, 1, 4095, 4096, (size_t)1 << 20, ((size_t)2 << 20) - 1, (size_t)2 << 20, ((size_t)2 << 20) + 4097, ((size_t)8 << 20) + 1,
                             ((size_t)33 << 20) + 12345};
     for (size_t i = 0; i < sizeof(sizes) / sizeof(sizes[0]); i++) {
         const int rc = check(sizes[i]);
@@ -54,7 +54,7 @@ int main(void) {
     }
     /* many calls in a row (the helpers are reused) */
     for (int rep = 0; rep < 40; rep++)
-        if (check(((size_t)8 << 20) + 4096 * (size_t)rep)) { printf("repeat %d failed\n", rep); return 1; }
+        if (check(((size_t)2 << 20) + 40960 * (size_t)rep + (size_t)rep)) { printf("repeat %d failed\n", rep); return 1; }
     /* a child of a process whose helpers exist has none: it must still get the right answers */
     const pid_t pid = fork();
     if (pid == 0) _exit(check((size_t)16 << 20) || check((size_t)9 << 20) ? 9 : 0);

@@ -259,15 +259,16 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
 
-template <int D> struct BwdSmem {
+template <int D, int KW = 4> struct BwdSmem {          // KW: wavefronts (32 keys each) per workgroup
     static constexpr int kLd = D + 4;
     // queries per turn of the loop: 32, or two sub-tiles of 32 at head_dim 32, where a 32-query turn holds half the matrix
     // work of head_dim 64 for the same two barriers, the same staging and the same dQ store
     static constexpr int QSUB = D == 32 ? 2 : 1;
     static constexpr int QROWS = 32 * QSUB;
-    static constexpr int K = 128 * kLd;                 // K rows of the workgroup
+    static constexpr int KEYS = 32 * KW;                // keys per workgroup
+    static constexpr int K = KEYS * kLd;                // K rows of the workgroup
     static constexpr int QT = QROWS * kLd;              // one Q (or dO) tile
-    static constexpr int kDsLd = 132;                   // dS row stride: 128 keys + 4 pad
+    static constexpr int kDsLd = KEYS + 4;              // dS row stride: the workgroup's keys + 4 pad
     static constexpr int OFF_K = 0;
     static constexpr int OFF_Q = OFF_K + K;
     static constexpr int OFF_DO = OFF_Q + QT;
@@ -279,8 +280,8 @@ template <int D> struct BwdSmem {
 // RAGGED: rows past s are clamped on load; padding keys are masked, padding queries contribute nothing because their
 // dO rows and delta are staged as zeros; stores are guarded
 // CACHED: the forward pass left the scaled scores (log2 units, [head][key][query]); S = Q.K^T is read instead of recomputed
-template <int D, bool CAUSAL, bool RAGGED, bool CACHED = false>
-__global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
+template <int D, bool CAUSAL, bool RAGGED, bool CACHED = false, int KW = 4>
+__global__ __launch_bounds__(64 * KW, (D == 128 || KW == 8) ? 1 : 2) void sdpa_bwd_mfma_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                const float* __restrict__ v, const float* __restrict__ lse,
                                                                const float* __restrict__ delta, const float* __restrict__ d_out,
                                                                float* __restrict__ dq_partial, float* __restrict__ dk,
@@ -288,8 +289,8 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
                                                                int mirror, const float* __restrict__ scores_t) {
     static_assert(!CACHED || D == 64, "the score cache exists for head_dim 64");
     extern __shared__ __align__(16) float smem[];
-    using Smem = BwdSmem<D>;
-    constexpr int kD = D, kLd = D + 4, NT = D / 32, G = D / 8, C4 = D / 4;
+    using Smem = BwdSmem<D, KW>;
+    constexpr int kD = D, kLd = D + 4, NT = D / 32, G = D / 8, C4 = D / 4, NTHR = 64 * KW, KEYS = 32 * KW;
     constexpr int QSUB = Smem::QSUB, QROWS = Smem::QROWS;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane & 31, half = lane >> 5;
     const int i16 = lane & 15, kk = lane >> 4;   // operand coordinates of the 16x16x4 products
@@ -301,7 +302,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
     const int lin = blockIdx.x;
     const int64_t head = lin % n_heads;
     const int px = lin / n_heads;
-    const int bx = mirror ? (s + 127) / 128 - 1 - px : px;
+    const int bx = mirror ? (s + KEYS - 1) / KEYS - 1 - px : px;
     const float* qh = q + head * s * kD;
     const float* kh = k + head * s * kD;
     const float* vh = v + head * s * kD;
@@ -310,7 +311,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
     const float* dh = delta + head * s;
     // partial dQ of this workgroup: [px][bh][s][64]
     float* dqh = dq_partial + ((int64_t)px * n_heads + head) * s * kD;
-    const int kv_wg = bx * 128;          // first key of the workgroup
+    const int kv_wg = bx * KEYS;         // first key of the workgroup
     const int kv0 = kv_wg + w * 32;              // first key of this wavefront
     const float c1 = scale * kLog2e;
 
@@ -341,15 +342,15 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
     const int first_qt = CAUSAL ? kv_wg / QROWS : 0;   // earlier query tiles see none of this workgroup's keys
     // their partial dQ rows are zero (a mirror launch leaves them as its counterpart wrote them)
     if (!mirror)
-        for (int i = tid; i < first_qt * QROWS * (kD / 4); i += 256)
+        for (int i = tid; i < first_qt * QROWS * (kD / 4); i += NTHR)
             reinterpret_cast<float4*>(dqh)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     // staging: a Q tile and a dO tile are QROWS * D / 4 float4 each, 2 or 4 per lane and operand
-    constexpr int PERQ = QROWS * D / 1024;       // 2, 2 or 4
+    constexpr int PERQ = QROWS * D / (4 * NTHR);  // 2, 2 or 4 (1, 1 or 2 with eight wavefronts)
     float4 qst0, qst1, qst2, qst3, gst0, gst1, gst2, gst3;
     float stat = 0.f;
 #define BWD_LD(i, Q, G_)                                                                                  \
     if constexpr (PERQ > (i)) {                                                                           \
-        const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
+        const int idx = tid + (i) * NTHR, row = idx / C4, c4 = idx % C4;                                  \
         const int grow = RAGGED ? min(qt_ld * QROWS + row, s - 1) : qt_ld * QROWS + row;                  \
         Q = *reinterpret_cast<const float4*>(qh + (int64_t)grow * kD + c4 * 4);                           \
         G_ = *reinterpret_cast<const float4*>(gh + (int64_t)grow * kD + c4 * 4);                          \
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
     }
 #define BWD_ST(i, Q, G_)                                                                                  \
     if constexpr (PERQ > (i)) {                                                                           \
-        const int idx = tid + (i) * 256, row = idx / C4, c4 = idx % C4;                                   \
+        const int idx = tid + (i) * NTHR, row = idx / C4, c4 = idx % C4;                                  \
         *reinterpret_cast<float4*>(qs + row * kLd + c4 * 4) = Q;                                          \
         *reinterpret_cast<float4*>(gs + row * kLd + c4 * 4) = G_;                                         \
     }
@@ -491,8 +492,13 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
         // consecutive keys of its dS row at once and feeds them to four successive products (the order
         // of the contraction index is free as long as both operands use the same one)
         // (head_dim 32 with its 64-query turns: column tile w & 1 of row tiles w >> 1 and (w >> 1) + 2)
-        constexpr int NCT = D >= 64 ? D / 64 : 1, NRT = 2, RSTEP = D >= 64 ? 1 : 2;
-        const int ct0 = D >= 64 ? w * NCT : (w & 1), rt0 = D >= 64 ? 0 : (w >> 1);
+        // (eight wavefronts, head_dim 32 or 64: the turn's eight 16x16 tiles, one each -- column tile w % (D/16) of row
+        // tile w / (D/16) -- over 256 keys, as two chains of products over alternate key groups so that a product never
+        // waits for its predecessor)
+        constexpr bool WIDE = KW == 8;
+        static_assert(!WIDE || D == 64 || D == 32, "eight wavefronts per workgroup exist for head_dim 32 and 64");
+        constexpr int NCT = WIDE ? 1 : (D >= 64 ? D / 64 : 1), NRT = 2, RSTEP = WIDE ? 0 : (D >= 64 ? 1 : 2);
+        const int ct0 = WIDE ? (w % (D / 16)) : (D >= 64 ? w * NCT : (w & 1)), rt0 = WIDE ? (w / (D / 16)) : (D >= 64 ? 0 : (w >> 1));
         floatx4 acc_dq[NCT][NRT];
 #pragma unroll
         for (int c = 0; c < NCT; c++)
@@ -501,26 +507,34 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
         __builtin_amdgcn_s_setprio(3);
         float* dq_row0 = dqh + (int64_t)(q0 + 16 * rt0 + i16) * kD + 16 * ct0 + 4 * kk;   // tile (c, t) at + 16*RSTEP*t rows, + 16*c columns
         // mirror launch (never under a causal mask): what the first launch stored here, in flight while the products below run
-        float4 old[CAUSAL ? 1 : NCT][CAUSAL ? 1 : NRT];
+        constexpr int NST = WIDE ? 1 : NRT;     // row tiles this wavefront stores (the two chains of the wide form are one tile)
+        float4 old[CAUSAL ? 1 : NCT][CAUSAL ? 1 : NST];
         if constexpr (!CAUSAL) {
 #pragma unroll
             for (int c = 0; c < NCT; c++)
 #pragma unroll
-                for (int t = 0; t < NRT; t++) {
+                for (int t = 0; t < NST; t++) {
                     old[c][t] = make_float4(0.f, 0.f, 0.f, 0.f);
                     if (mirror && (!RAGGED || q0 + 16 * (rt0 + RSTEP * t) + i16 < s))
                         old[c][t] = *reinterpret_cast<const float4*>(dq_row0 + (int64_t)16 * RSTEP * t * kD + 16 * c);
                 }
         }
-        const int g_lim = CAUSAL ? min(8, (q0 + QROWS - kv_wg + 15) / 16) : 8;   // keys past the tile's last query are masked
-        for (int g = 0; g < g_lim; g++) {
+        constexpr int GN = KEYS / 16;           // groups of 16 keys
+        const int g_lim = CAUSAL ? min(GN, (q0 + QROWS - kv_wg + 15) / 16) : GN;   // keys past the tile's last query are masked
+        for (int g0 = 0; g0 < g_lim; g0 += (WIDE ? 2 : 1)) {
             float4 a[NRT];
 #pragma unroll
-            for (int t = 0; t < NRT; t++) a[t] = *reinterpret_cast<const float4*>(dsb + (16 * (rt0 + RSTEP * t) + i16) * Smem::kDsLd + 16 * g + 4 * kk);
-            float b[NCT][4];
+            for (int t = 0; t < NRT; t++) {
+                // the wide form's second chain takes the next key group of the same rows (an odd g_lim: its last turn adds zeros)
+                const int g = WIDE ? min(g0 + t, g_lim - 1) : g0;
+                a[t] = *reinterpret_cast<const float4*>(dsb + (16 * (rt0 + RSTEP * t) + i16) * Smem::kDsLd + 16 * g + 4 * kk);
+                if (WIDE && g0 + t >= g_lim) a[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            float b[WIDE ? 2 : NCT][4];
 #pragma unroll
-            for (int c = 0; c < NCT; c++) {
-                const float* kb = kall + (16 * g + 4 * kk) * kLd + 16 * (ct0 + c) + i16;
+            for (int c = 0; c < (WIDE ? 2 : NCT); c++) {
+                const int g = WIDE ? min(g0 + c, g_lim - 1) : g0;
+                const float* kb = kall + (16 * g + 4 * kk) * kLd + 16 * (ct0 + (WIDE ? 0 : c)) + i16;
                 b[c][0] = kb[0]; b[c][1] = kb[kLd]; b[c][2] = kb[2 * kLd]; b[c][3] = kb[3 * kLd];
             }
             // operands swapped: the product is the transpose dQ^T[d][query], so a lane ends up with four consecutive
@@ -528,26 +542,30 @@ __global__ __launch_bounds__(256, D == 128 ? 1 : 2) void sdpa_bwd_mfma_kernel(co
 #pragma unroll
             for (int c = 0; c < NCT; c++)
 #pragma unroll
-                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][0], a[t].x, acc_dq[c][t]);
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[WIDE ? t : c][0], a[t].x, acc_dq[c][t]);
 #pragma unroll
             for (int c = 0; c < NCT; c++)
 #pragma unroll
-                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][1], a[t].y, acc_dq[c][t]);
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[WIDE ? t : c][1], a[t].y, acc_dq[c][t]);
 #pragma unroll
             for (int c = 0; c < NCT; c++)
 #pragma unroll
-                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][2], a[t].z, acc_dq[c][t]);
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[WIDE ? t : c][2], a[t].z, acc_dq[c][t]);
 #pragma unroll
             for (int c = 0; c < NCT; c++)
 #pragma unroll
-                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[c][3], a[t].w, acc_dq[c][t]);
+                for (int t = 0; t < NRT; t++) acc_dq[c][t] = MFMA16(b[WIDE ? t : c][3], a[t].w, acc_dq[c][t]);
         }
         __builtin_amdgcn_s_setprio(0);
+        if constexpr (WIDE) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc_dq[0][0][e] += acc_dq[0][1][e];
+        }
         // accumulator register e of lane (i16, kk) is head-dim column 16*ct + 4*kk + e of query row i16 of the 16-row tile
 #pragma unroll
         for (int c = 0; c < NCT; c++)
 #pragma unroll
-            for (int t = 0; t < NRT; t++)
+            for (int t = 0; t < NST; t++)
                 if (!RAGGED || q0 + 16 * (rt0 + RSTEP * t) + i16 < s) {
                     float4 o = make_float4(acc_dq[c][t][0], acc_dq[c][t][1], acc_dq[c][t][2], acc_dq[c][t][3]);
                     if constexpr (!CAUSAL) {
@@ -602,6 +620,8 @@ static bool grid_fits(int64_t s, int64_t bh_count) { return ceil_div(s, 128) * b
 // shapes whose scaled scores the forward pass can leave for the backward pass: head_dim 64, whole 128-row tiles
 bool sdpa_scores_shape(int64_t s, int64_t d) { return d == 64 && mfma_shape(s, d) && s % 128 == 0; }
 
+int g_sdpa_wide = -1;   // test hook: 1 = the backward kernel's 256-key workgroups wherever they exist, 0 = never, -1 = by shape
+
 // one launch of one instantiation; the first call raises the kernel's dynamic LDS limit
 template <int D, int KT, bool CAUSAL, bool RAGGED, bool EMIT>
 static int fwd_launch(dim3 grid, const float* q, const float* k, const float* v, float* out, float* lse, int s, int heads, float sl,
@@ -645,28 +665,28 @@ int sdpa_forward_mfma(const float* q, const float* k, const float* v, float scal
     return fwd_dispatch<128, 32>(grid, causal != 0, ragged, q, k, v, out, lse, si, hi, sl);
 }
 
-template <int D, bool CAUSAL, bool RAGGED, bool CACHED>
+template <int D, bool CAUSAL, bool RAGGED, bool CACHED, int KW = 4>
 static int bwd_launch(int64_t grid, int mirror, const float* q, const float* k, const float* v, const float* lse, const float* delta,
                       const float* d_out, float* partial, float* dk, float* dv, int s, int heads, float scale, const float* scores_t) {
-    constexpr size_t lds = sizeof(float) * BwdSmem<D>::TOTAL;
+    constexpr size_t lds = sizeof(float) * BwdSmem<D, KW>::TOTAL;
     static bool attr = false;
     if (!attr) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<D, CAUSAL, RAGGED, CACHED>),
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_bwd_mfma_kernel<D, CAUSAL, RAGGED, CACHED, KW>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "hipFuncSetAttribute");
         if (rc) return rc;
         attr = true;
     }
-    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<D, CAUSAL, RAGGED, CACHED>), dim3((unsigned)grid), dim3(256), lds, stream(), q, k, v, lse, delta,
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<D, CAUSAL, RAGGED, CACHED, KW>), dim3((unsigned)grid), dim3(64 * KW), lds, stream(), q, k, v, lse, delta,
                        d_out, partial, dk, dv, s, heads, scale, mirror, scores_t);
     return BH_LAUNCH_CHECK("sdpa_bwd_mfma_kernel");
 }
-template <int D>
+template <int D, int KW = 4>
 static int bwd_dispatch(int64_t grid, int mirror, bool causal, bool ragged, const float* q, const float* k, const float* v, const float* lse,
                         const float* delta, const float* d_out, float* partial, float* dk, float* dv, int s, int heads, float scale) {
-    if (causal && ragged) return bwd_launch<D, true, true, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
-    if (causal) return bwd_launch<D, true, false, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
-    if (ragged) return bwd_launch<D, false, true, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
-    return bwd_launch<D, false, false, false>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    if (causal && ragged) return bwd_launch<D, true, true, false, KW>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    if (causal) return bwd_launch<D, true, false, false, KW>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    if (ragged) return bwd_launch<D, false, true, false, KW>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
+    return bwd_launch<D, false, false, false, KW>(grid, mirror, q, k, v, lse, delta, d_out, partial, dk, dv, s, heads, scale, nullptr);
 }
 
 int sdpa_backward_mfma(const float* q, const float* k, const float* v, const float* lse, const float* delta,
@@ -676,16 +696,25 @@ int sdpa_backward_mfma(const float* q, const float* k, const float* v, const flo
     if (scores_t && !sdpa_scores_shape(s, d)) return 1;
     const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     if (!al(q) || !al(k) || !al(v) || !al(d_out) || !al(dq) || !al(dk) || !al(dv)) return 1;
-    const int key_tiles = (int)ceil_div(s, 128);
+    // Eight wavefronts and 256 keys per workgroup, one workgroup per compute unit (head_dim 32 and 64; the score-cache
+    // kernel only unmasked and over whole 256-key tiles): half as many dQ partials to write, add to and fold -- none at
+    // all when two mirrored launches cover the sequence, as at 512 keys -- and one dQ tile per wavefront and turn.  It
+    // pays when the launch still fills the chip twice over (B8 h16 S1024 D64: 0.684 against 0.699 ms; 256 heads of
+    // S512 with the score cache: 0.319 against 0.336 ms); with fewer workgroups the 128-key form's finer grain wins (32
+    // heads of S1024: 0.217 against 0.333 ms).
+    const bool wide_exists = (d == 64 || d == 32) && (!scores_t || (s % 256 == 0 && !causal));
+    const bool wide = wide_exists && (g_sdpa_wide > 0 || (g_sdpa_wide < 0 && ceil_div(s, 256) * bh_count >= 2 * (int64_t)bh_device_cu_count()));
+    const int keys = wide ? 256 : 128;
+    const int key_tiles = (int)ceil_div(s, keys);
     // Two launches that share one set of dQ partials (the second takes the key tiles in mirrored order and adds to what
     // the first stored) when each launch still fills every compute unit with the workgroups it can hold (two; one at
     // head_dim 128): half as many partials to write and fold, and each launch is a single round of workgroups that start
     // and finish together instead of two rounds whose second runs out unevenly.  Not under a causal mask, where a launch
     // would hold tiles of unequal work.
-    const int64_t resident = (d == 128 ? 1 : 2) * (int64_t)bh_device_cu_count();
+    const int64_t resident = ((d == 128 || wide) ? 1 : 2) * (int64_t)bh_device_cu_count();
     const bool two_launches = !causal && key_tiles >= 2 && (int64_t)(key_tiles / 2) * bh_count >= resident;
     const int tiles = two_launches ? (key_tiles + 1) / 2 : key_tiles;      // dQ partials per head
-    const bool ragged = s % 128 != 0;
+    const bool ragged = s % keys != 0;
     const int64_t n = bh_count * s * d;
     float* partial = tiles > 1 ? (float*)bh_malloc(sizeof(float) * (size_t)(tiles * n)) : dq;   // one partial: dq itself
     if (!partial) return BH_ENOMEM;
@@ -693,9 +722,13 @@ int sdpa_backward_mfma(const float* q, const float* k, const float* v, const flo
     int rc = BH_OK;
     for (int pass = 0; pass < (two_launches ? 2 : 1) && rc == BH_OK; pass++) {
         const int64_t grid = (pass == 0 ? tiles : key_tiles / 2) * bh_count;
-        if (scores_t)
+        if (scores_t && wide)
+            rc = bwd_launch<64, false, false, true, 8>(grid, pass, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale, scores_t);
+        else if (scores_t)
             rc = causal ? bwd_launch<64, true, false, true>(grid, pass, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale, scores_t)
                         : bwd_launch<64, false, false, true>(grid, pass, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale, scores_t);
+        else if (wide && d == 32) rc = bwd_dispatch<32, 8>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
+        else if (wide) rc = bwd_dispatch<64, 8>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
         else if (d == 32) rc = bwd_dispatch<32>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
         else if (d == 64) rc = bwd_dispatch<64>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
         else rc = bwd_dispatch<128>(grid, pass, causal != 0, ragged, q, k, v, lse, delta, d_out, partial, dk, dv, si, hi, scale);
@@ -712,3 +745,9 @@ int sdpa_backward_mfma(const float* q, const float* k, const float* v, const flo
 }
 
 }  // namespace bh
+
+// test/benchmark hook: 1 = 256-key workgroups in the attention backward wherever that form exists, 0 = never, -1 = by shape
+extern "C" int bh_sdpa_force_wide(int mode) {
+    bh::g_sdpa_wide = mode;
+    return BH_OK;
+}

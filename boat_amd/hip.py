@@ -73,7 +73,7 @@ _SIGS = {
     "bh_dense_backward_into": (I, [P, P, P, P, P, P, L, L, L, I, I]),
     "bh_sdpa_forward": (I, [P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_backward": (I, [P, P, P, P, P, P, F, I, P, P, P, L, L, L]),
-    "bh_sdpa_force_general": (I, [I]),
+    "bh_sdpa_force_general": (I, [I]), "bh_sdpa_force_wide": (I, [I]),
     "bh_sdpa_score_cache_bytes": (C.c_size_t, [L, L, L]),
     "bh_sdpa_forward_cached": (I, [P, P, P, F, I, P, P, P, L, L, L]),
     "bh_sdpa_backward_cached": (I, [P, P, P, P, P, P, P, F, I, P, P, P, L, L, L]),

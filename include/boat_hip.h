@@ -332,6 +332,9 @@ int bh_gemm_force_splits(int splits);
  * where the shape allows) */
 int bh_gemm_no_tables(int off);
 int bh_sdpa_force_general(int on);
+/* bh_sdpa_force_wide: 1 = the attention backward's 256-key workgroups (eight wavefronts) wherever that form exists
+ * (head_dim 32 and 64), 0 = never, -1 = chosen by shape (the default) */
+int bh_sdpa_force_wide(int mode);
 /* bh_layernorm_tune: cap on the workgroups of the LayerNorm backward (each writes one dgamma/dbeta partial) and of
  * the forward; 0 keeps the current value. */
 int bh_layernorm_tune(int bwd_blocks, int fwd_blocks);

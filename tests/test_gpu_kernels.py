@@ -837,6 +837,64 @@ def test_sdpa_with_score_cache(hip, oracle, rng, bh, s, causal):
         assert rel_fro(g, x.numpy()) <= FP32_ATTENTION_BOUND
 
 
+@pytest.mark.parametrize("causal", [0, 1])
+@pytest.mark.parametrize("bh,s,d", [(2, 256, 64), (3, 512, 64), (2, 300, 64), (1, 1000, 64), (2, 77, 64), (2, 32, 64), (1, 1024, 64),
+                                    (2, 256, 32), (3, 520, 32), (1, 1024, 32), (2, 77, 32), (2, 32, 32)])
+def test_sdpa_backward_with_256_key_workgroups(hip, oracle, rng, bh, s, d, causal):
+    """The backward kernel's form with eight wavefronts and 256 keys per workgroup, which the library picks for launches
+    that fill the chip twice over, forced on small shapes (whole tiles, ragged lengths, a sequence shorter than one
+    tile): the oracle's attention backward (src/layers/attention.c:1417-1520) at the bound only fp32 accumulation meets,
+    dK and dV bit for bit those of the 128-key form (the same products in the same order), dQ to rounding (its
+    contraction over the keys is cut differently)."""
+    q, k, v, go = (rng.standard_normal((bh, s, d)).astype(np.float32) for _ in range(4))
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(d)))
+    _, _, wattn = oracle.sdpa_forward(q, k, v, scale, causal)
+    want = oracle.sdpa_backward(q, k, v, wattn, go, scale)
+    dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)
+    out, lse = hip.empty((bh, s, d)), hip.empty((bh, s))
+    hip.check(hip.bh_sdpa_forward(dq_.ptr, dk_.ptr, dv_.ptr, scale, causal, out.ptr, lse.ptr, None, bh, s, d))
+    got = {}
+    try:
+        for mode in (0, 1):
+            hip.check(hip.bh_sdpa_force_wide(mode))
+            g = [hip.to_device(np.full((bh, s, d), np.nan, np.float32)) for _ in range(3)]
+            hip.check(hip.bh_sdpa_backward(dq_.ptr, dk_.ptr, dv_.ptr, out.ptr, lse.ptr, dgo.ptr, scale, causal,
+                                           g[0].ptr, g[1].ptr, g[2].ptr, bh, s, d))
+            got[mode] = [x.numpy() for x in g]
+    finally:
+        hip.check(hip.bh_sdpa_force_wide(-1))
+    for g, w in zip(got[1], want):
+        assert rel_fro(g, w) <= FP32_ATTENTION_BOUND
+    assert np.array_equal(got[0][1], got[1][1]) and np.array_equal(got[0][2], got[1][2])
+    assert rel_fro(got[1][0], got[0][0]) <= 1e-6
+
+
+@pytest.mark.parametrize("bh,s", [(3, 256), (2, 512), (1, 1024)])
+def test_sdpa_score_cache_with_256_key_workgroups(hip, oracle, rng, bh, s):
+    """The score-cache backward in its 256-key form (unmasked, whole 256-key tiles), forced: against the oracle and the
+    128-key form."""
+    d, scale = 64, 0.125
+    q, k, v, go = (rng.standard_normal((bh, s, d), dtype=np.float32) for _ in range(4))
+    dq_, dk_, dv_, dgo = dev(hip, q), dev(hip, k), dev(hip, v), dev(hip, go)
+    o, lse, cache = hip.empty((bh, s, d)), hip.empty((bh, s)), hip.empty((bh, s, s))
+    hip.check(hip.bh_sdpa_forward_cached(dq_.ptr, dk_.ptr, dv_.ptr, scale, 0, o.ptr, lse.ptr, cache.ptr, bh, s, d))
+    got = {}
+    try:
+        for mode in (0, 1):
+            hip.check(hip.bh_sdpa_force_wide(mode))
+            g = [hip.to_device(np.full((bh, s, d), np.nan, np.float32)) for _ in range(3)]
+            hip.check(hip.bh_sdpa_backward_cached(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, cache.ptr, dgo.ptr, scale, 0,
+                                                  g[0].ptr, g[1].ptr, g[2].ptr, bh, s, d))
+            got[mode] = [x.numpy() for x in g]
+    finally:
+        hip.check(hip.bh_sdpa_force_wide(-1))
+    _, _, wattn = oracle.sdpa_forward(q, k, v, scale, 0)
+    for g, w in zip(got[1], oracle.sdpa_backward(q, k, v, wattn, go, scale)):
+        assert rel_fro(g, w) <= FP32_ATTENTION_BOUND
+    assert np.array_equal(got[0][1], got[1][1]) and np.array_equal(got[0][2], got[1][2])
+    assert rel_fro(got[1][0], got[0][0]) <= 1e-6
+
+
 def test_sdpa_score_cache_refuses_other_shapes(hip):
     assert hip.bh_sdpa_score_cache_bytes(4, 100, 64) == 0 and hip.bh_sdpa_score_cache_bytes(4, 128, 32) == 0
     buf = hip.empty(4 * 128 * 64)

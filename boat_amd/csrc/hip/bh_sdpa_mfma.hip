@@ -269,12 +269,15 @@ template <int D, int KW = 4> struct BwdSmem {          // KW: wavefronts (32 key
     static constexpr int K = KEYS * kLd;                // K rows of the workgroup
     static constexpr int QT = QROWS * kLd;              // one Q (or dO) tile
     static constexpr int kDsLd = KEYS + 4;              // dS row stride: the workgroup's keys + 4 pad
-    static constexpr int OFF_K = 0;
-    static constexpr int OFF_Q = OFF_K + K;
+    // The tiles that are read row by row with constant steps come first: an LDS instruction's immediate offset reaches
+    // 64 KB, and whatever lies beyond costs an address register per access (with K first, the 256-key form spent some forty
+    // registers on the addresses of its Q and dO rows).
+    static constexpr int OFF_Q = 0;
     static constexpr int OFF_DO = OFF_Q + QT;
     static constexpr int OFF_DS = OFF_DO + QT;          // [QROWS][kDsLd]
     static constexpr int OFF_STAT = OFF_DS + QROWS * kDsLd; // [2][QROWS]: lse*log2e, delta
-    static constexpr int TOTAL = OFF_STAT + 2 * QROWS;
+    static constexpr int OFF_K = OFF_STAT + 2 * QROWS;
+    static constexpr int TOTAL = OFF_K + K;
 };
 
 // RAGGED: rows past s are clamped on load; padding keys are masked, padding queries contribute nothing because their
@@ -429,25 +432,40 @@ __global__ __launch_bounds__(64 * KW, (D == 128 || KW == 8) ? 1 : 2) void sdpa_b
                     acc_s[4 * j + 3] = sc_cur[j].w;
                 }
                 floatx16 acc_dp2 = zero16();     // two chains, so that a product never waits for its predecessor
+                // (the operands of group g + 1 are read from LDS before the products of group g are issued: left to
+                // itself the compiler places a read right in front of its first use and the wavefront waits out the
+                // LDS latency once per group)
+                float4 ag_next = *reinterpret_cast<const float4*>(gsu + r * kLd + 4 * half);
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    const float4 ag = *reinterpret_cast<const float4*>(gsu + r * kLd + 8 * g + 4 * half);
+                    const float4 ag = ag_next;
+                    if (g + 1 < G) ag_next = *reinterpret_cast<const float4*>(gsu + r * kLd + 8 * (g + 1) + 4 * half);
                     const float4 bv = vreg[g];
+                    __builtin_amdgcn_sched_barrier(0);
                     acc_dp = MFMA(ag.x, bv.x, acc_dp);
                     acc_dp2 = MFMA(ag.y, bv.y, acc_dp2);
                     acc_dp = MFMA(ag.z, bv.z, acc_dp);
                     acc_dp2 = MFMA(ag.w, bv.w, acc_dp2);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc_dp[e] += acc_dp2[e];
             } else {
+                const int off0 = r * kLd + 4 * half;
+                float4 aq_next = *reinterpret_cast<const float4*>(qsu + off0);
+                float4 bk_next = *reinterpret_cast<const float4*>(ks + off0);
+                float4 ag_next = *reinterpret_cast<const float4*>(gsu + off0);
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    const int off = r * kLd + 8 * g + 4 * half;
-                    const float4 aq = *reinterpret_cast<const float4*>(qsu + off);
-                    const float4 bk = *reinterpret_cast<const float4*>(ks + off);
-                    const float4 ag = *reinterpret_cast<const float4*>(gsu + off);
+                    const float4 aq = aq_next, bk = bk_next, ag = ag_next;
+                    if (g + 1 < G) {             // group g + 1's operands, read before group g's products are issued
+                        const int off = off0 + 8 * (g + 1);
+                        aq_next = *reinterpret_cast<const float4*>(qsu + off);
+                        bk_next = *reinterpret_cast<const float4*>(ks + off);
+                        ag_next = *reinterpret_cast<const float4*>(gsu + off);
+                    }
                     const float4 bv = vreg[g];
+                    __builtin_amdgcn_sched_barrier(0);
                     acc_s = MFMA(aq.x, bk.x, acc_s);
                     acc_dp = MFMA(ag.x, bv.x, acc_dp);
                     acc_s = MFMA(aq.y, bk.y, acc_s);
@@ -456,28 +474,70 @@ __global__ __launch_bounds__(64 * KW, (D == 128 || KW == 8) ? 1 : 2) void sdpa_b
                     acc_dp = MFMA(ag.z, bv.z, acc_dp);
                     acc_s = MFMA(aq.w, bk.w, acc_s);
                     acc_dp = MFMA(ag.w, bv.w, acc_dp);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
             __builtin_amdgcn_s_setprio(2);
             // Row by row: P and dS of query row acc_row(e, half), dS published for the dQ product, then the row's four
             // products dV += P^T.dO, dK += dS^T.Q (step e contracts that query row).  The exponential and the
             // arithmetic of row e + 1 are issued while the matrix core still works on row e.
+            // Software pipelined by hand, two rows deep: while the matrix core works on row e, the vector unit computes
+            // P and dS of row e + 1 (between the products, not after them) and LDS delivers the operands of row e + 2.
+            // In the compiler's own order a row's exponential chain sits in front of its products, and the two
+            // wavefronts of a SIMD, which run in step, leave the matrix core idle for that long once per row.
+            FloatN<NT> bg_buf[2], bq_buf[2];
+            float lse_buf[2], delta_buf[2];
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int row = acc_row(e, half);
-                float p = __builtin_amdgcn_exp2f(CACHED ? acc_s[e] - stu[row] : acc_s[e] * c1 - stu[row]);
+            for (int i = 0; i < 2; i++) {
+                const int row_i = acc_row(i, half);
+                bg_buf[i].load(gsu + row_i * kLd + NT * r);
+                bq_buf[i].load(qsu + row_i * kLd + NT * r);
+                lse_buf[i] = stu[row_i];
+                delta_buf[i] = stu[QROWS + row_i];
+            }
+            float p_cur, ds_cur;
+            {
+                const int row0 = acc_row(0, half);
+                p_cur = __builtin_amdgcn_exp2f(CACHED ? acc_s[0] - lse_buf[0] : acc_s[0] * c1 - lse_buf[0]);
                 // masked pairs and padding keys carry no probability (padding queries need no mask: their dO rows
                 // and delta were staged as zeros, so everything they contribute below is zero)
-                if ((CAUSAL && my_key > qu + row) || key_pad) p = 0.f;
-                const float ds = p * (acc_dp[e] - stu[QROWS + row]) * scale;
-                dsu[row * Smem::kDsLd + w * 32 + r] = ds;
-                FloatN<NT> bg, bq;
-                bg.load(gsu + row * kLd + NT * r);
-                bq.load(qsu + row * kLd + NT * r);
+                if ((CAUSAL && my_key > qu + row0) || key_pad) p_cur = 0.f;
+                ds_cur = p_cur * (acc_dp[0] - delta_buf[0]) * scale;
+                dsu[row0 * Smem::kDsLd + w * 32 + r] = ds_cur;
+            }
 #pragma unroll
-                for (int t = 0; t < NT; t++) acc_dv[t] = MFMA(p, bg.v[t], acc_dv[t]);
+            for (int e = 0; e < 16; e++) {
+                const FloatN<NT> bg = bg_buf[e & 1], bq = bq_buf[e & 1];
+                const float p = p_cur, ds = ds_cur;
+                __builtin_amdgcn_sched_barrier(0);
+                acc_dv[0] = MFMA(p, bg.v[0], acc_dv[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (e + 1 < 16) {
+                    const int nrow = acc_row(e + 1, half);
+                    p_cur = __builtin_amdgcn_exp2f(CACHED ? acc_s[e + 1] - lse_buf[(e + 1) & 1] : acc_s[e + 1] * c1 - lse_buf[(e + 1) & 1]);
+                    if ((CAUSAL && my_key > qu + nrow) || key_pad) p_cur = 0.f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < NT; t++) acc_dk[t] = MFMA(ds, bq.v[t], acc_dk[t]);
+                for (int t = 1; t < NT; t++) acc_dv[t] = MFMA(p, bg.v[t], acc_dv[t]);
+                acc_dk[0] = MFMA(ds, bq.v[0], acc_dk[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (e + 1 < 16) {
+                    const int nrow = acc_row(e + 1, half);
+                    ds_cur = p_cur * (acc_dp[e + 1] - delta_buf[(e + 1) & 1]) * scale;
+                    dsu[nrow * Smem::kDsLd + w * 32 + r] = ds_cur;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 1; t < NT; t++) acc_dk[t] = MFMA(ds, bq.v[t], acc_dk[t]);
+                if (e + 2 < 16) {                // row e + 2 into the buffers row e has just left
+                    const int row2 = acc_row(e + 2, half);
+                    bg_buf[e & 1].load(gsu + row2 * kLd + NT * r);
+                    bq_buf[e & 1].load(qsu + row2 * kLd + NT * r);
+                    lse_buf[e & 1] = stu[row2];
+                    delta_buf[e & 1] = stu[QROWS + row2];
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_setprio(0);
         } else {

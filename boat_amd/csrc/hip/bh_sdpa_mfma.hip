@@ -151,11 +151,22 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
             // staging and the barrier): of the two wavefronts that share a SIMD the one nearer to its barrier goes first
             // (measured: 287 -> 273 us unmasked, 175 -> 162 us causal at B8 h16 S1024)
             __builtin_amdgcn_s_setprio(1);
+            // (the K fragments of group g + 1 are read from LDS before the products of group g are issued, and further down
+            // the V rows two steps ahead of the step in work: left to itself the compiler puts a read right in front of its
+            // first use, and the wavefront waits out the LDS latency every few products)
+            float4 a_next[ST];
+#pragma unroll
+            for (int t = 0; t < ST; t++) a_next[t] = *reinterpret_cast<const float4*>(ks + (t * 32 + r) * kLd + 4 * half);
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 float4 a[ST];
 #pragma unroll
-                for (int t = 0; t < ST; t++) a[t] = *reinterpret_cast<const float4*>(ks + (t * 32 + r) * kLd + 8 * g + 4 * half);
+                for (int t = 0; t < ST; t++) a[t] = a_next[t];
+                if (g + 1 < G) {
+#pragma unroll
+                    for (int t = 0; t < ST; t++) a_next[t] = *reinterpret_cast<const float4*>(ks + (t * 32 + r) * kLd + 8 * (g + 1) + 4 * half);
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].x, qreg[4 * g + 0], acc_s[t]);
 #pragma unroll
@@ -164,8 +175,14 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
                 for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].z, qreg[4 * g + 2], acc_s[t]);
 #pragma unroll
                 for (int t = 0; t < ST; t++) acc_s[t] = MFMA(a[t].w, qreg[4 * g + 3], acc_s[t]);
+                __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_setprio(2);
+            // the first two V rows of the O^T products are on their way while the softmax runs
+            constexpr int NSTEP = ST * 16;
+            FloatN<NT> v_buf[3];
+#pragma unroll
+            for (int i = 0; i < 2; i++) v_buf[i].load(vs + ((i / 16) * 32 + acc_row(i % 16, half)) * kLd + NT * r);
             float mx = -INFINITY;
 #pragma unroll
             for (int t = 0; t < ST; t++)
@@ -202,15 +219,14 @@ __global__ __launch_bounds__(256, (EMIT && !CAUSAL) ? 1 : 2) void sdpa_fwd_mfma_
             __builtin_amdgcn_s_setprio(3);
             // O^T += V^T . P^T : step e of key tile t uses key row t*32 + acc_row(e, half)
 #pragma unroll
-            for (int t = 0; t < ST; t++)
+            for (int i = 0; i < NSTEP; i++) {
+                if (i + 2 < NSTEP) v_buf[(i + 2) % 3].load(vs + (((i + 2) / 16) * 32 + acc_row((i + 2) % 16, half)) * kLd + NT * r);
+                __builtin_amdgcn_sched_barrier(0);
+                const FloatN<NT> a = v_buf[i % 3];
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const int key = t * 32 + acc_row(e, half);
-                    FloatN<NT> a;
-                    a.load(vs + key * kLd + NT * r);
-#pragma unroll
-                    for (int n = 0; n < NT; n++) acc_o[n] = MFMA(a.v[n], acc_s[t][e], acc_o[n]);
-                }
+                for (int n = 0; n < NT; n++) acc_o[n] = MFMA(a.v[n], acc_s[i / 16][i % 16], acc_o[n]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         __builtin_amdgcn_s_setprio(0);
         if (more) FWD_STAGE_STORE(cur ^ 1)
@@ -422,6 +438,17 @@ __global__ __launch_bounds__(64 * KW, (D == 128 || KW == 8) ? 1 : 2) void sdpa_b
             // one nearer to its barrier goes first, so its workgroup's other wavefronts wait less.  Measured: 1 % on the
             // recomputing kernel, 3 % on the one that reads the score cache.
             __builtin_amdgcn_s_setprio(1);
+            // what the first two rows of the row loop need from LDS is on its way while the score and dP products run
+            FloatN<NT> bg_buf[2], bq_buf[2];
+            float lse_buf[2], delta_buf[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int row_i = acc_row(i, half);
+                bg_buf[i].load(gsu + row_i * kLd + NT * r);
+                bq_buf[i].load(qsu + row_i * kLd + NT * r);
+                lse_buf[i] = stu[row_i];
+                delta_buf[i] = stu[QROWS + row_i];
+            }
             if (CACHED) {
                 // registers 4j .. 4j+3 are query rows 8j + 4*half .. +3: the four 16-byte pieces fetched an iteration ago
 #pragma unroll
@@ -485,16 +512,6 @@ __global__ __launch_bounds__(64 * KW, (D == 128 || KW == 8) ? 1 : 2) void sdpa_b
             // P and dS of row e + 1 (between the products, not after them) and LDS delivers the operands of row e + 2.
             // In the compiler's own order a row's exponential chain sits in front of its products, and the two
             // wavefronts of a SIMD, which run in step, leave the matrix core idle for that long once per row.
-            FloatN<NT> bg_buf[2], bq_buf[2];
-            float lse_buf[2], delta_buf[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const int row_i = acc_row(i, half);
-                bg_buf[i].load(gsu + row_i * kLd + NT * r);
-                bq_buf[i].load(qsu + row_i * kLd + NT * r);
-                lse_buf[i] = stu[row_i];
-                delta_buf[i] = stu[QROWS + row_i];
-            }
             float p_cur, ds_cur;
             {
                 const int row0 = acc_row(0, half);

@@ -906,7 +906,8 @@ def test_sdpa_score_cache_refuses_other_shapes(hip):
 
 
 @pytest.mark.parametrize("bh,s,d", [(512, 384, 64), (512, 300, 64), (256, 512, 64), (600, 256, 64), (512, 384, 32), (600, 300, 32),
-                                    (256, 384, 128), (300, 300, 128)])
+                                    (256, 384, 128), (300, 300, 128),
+                                    (512, 700, 64), (512, 768, 32)])     # three 256-key tiles: the middle one belongs to the first launch
 def test_sdpa_backward_mirrored_second_launch(hip, oracle, rng, bh, s, d):
     """Enough heads for the unmasked backward to run as two launches that share one set of dQ partials (the second
     takes the key tiles in mirrored order and adds to what the first stored): odd tile counts (the middle tile belongs

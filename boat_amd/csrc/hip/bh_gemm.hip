@@ -528,6 +528,52 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g, GemmTab 
         const int64_t col = B_KC ? n0 + wn * Cfg::WN + j * 32 + r : n0 + wn * Cfg::WN + TN * r + j;
         bias_v[j] = (bias && col < g.n) ? bias[col] : 0.f;
     }
+    // A tile that lies wholly inside the matrix (every tile of a shape that is a multiple of the tile) needs no bounds
+    // checks, and its addresses are one per-lane pointer plus row and column steps that are the same for every lane: the
+    // row step goes through the scalar unit, the column step into the store's immediate offset.  The general code below
+    // spends about fifteen vector instructions per stored element on indices, comparisons and 64-bit address arithmetic,
+    // a thousand per wavefront, in the one phase of the kernel in which no matrix instruction is in flight.
+    if (m0 + BM <= g.m && n0 + BN <= g.n) {
+        const int64_t ldc = g.ldc;
+        float* lp = C + (m0 + wm * Cfg::WM + (A_KC ? half * 4 : TM * half * 4)) * ldc + n0 + wn * Cfg::WN + (B_KC ? r : TN * r);
+        constexpr int GR = TM * TN <= 4 ? 8 : 4;      // rows whose old values are fetched together when accumulating
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int eg = 0; eg < 16; eg += GR) {
+                if (add_c) {       // the same sums in the same order as the general code: (acc + bias) + old
+                    float prev[GR][TN];
+#pragma unroll
+                    for (int e = 0; e < GR; e++) {
+                        const int ec = eg + e;
+                        const int rc = A_KC ? i * 32 + (ec >> 2) * 8 + (ec & 3) : TM * ((ec >> 2) * 8 + (ec & 3)) + i;
+                        const float* rp = lp + rc * ldc;
+#pragma unroll
+                        for (int j = 0; j < TN; j++) prev[e][j] = __builtin_nontemporal_load(rp + (B_KC ? j * 32 : j));
+                    }
+#pragma unroll
+                    for (int e = 0; e < GR; e++) {
+                        const int ec = eg + e;
+                        const int rc = A_KC ? i * 32 + (ec >> 2) * 8 + (ec & 3) : TM * ((ec >> 2) * 8 + (ec & 3)) + i;
+                        float* rp = lp + rc * ldc;
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            rp[B_KC ? j * 32 : j] = GR == 8 ? (acc[i][j][ec] + prev[e][j]) + bias_v[j] : (acc[i][j][ec] + bias_v[j]) + prev[e][j];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < GR; e++) {
+                        const int ec = eg + e;
+                        const int rc = A_KC ? i * 32 + (ec >> 2) * 8 + (ec & 3) : TM * ((ec >> 2) * 8 + (ec & 3)) + i;
+                        float* rp = lp + rc * ldc;
+#pragma unroll
+                        for (int j = 0; j < TN; j++) rp[B_KC ? j * 32 : j] = acc[i][j][ec] + bias_v[j];
+                    }
+                }
+            }
+        }
+        return;
+    }
     // accumulate: the old values of one 32-row slab are fetched by loads that depend on nothing, then added; a load
     // placed between the stores below would have to wait for them (the compiler cannot tell the rows apart)
     // (with wavefront tiles of 128x64 the addresses, which the stores need again, would not fit the register file

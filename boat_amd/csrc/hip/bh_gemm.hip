@@ -252,8 +252,10 @@ struct DirectFrags {
     }
 };
 
+// (the four-wavefront tile is held to the registers of three workgroups per compute unit -- 146, its accumulators among
+// them -- which its 33 KB of LDS allow as well: a third resident workgroup is worth 0.3-0.9 % on the block's shapes)
 template <typename Cfg, bool A_KC, bool B_KC, bool DIRECT, int KT = 1, bool TAB = false>   // KT: k-tiles per LDS stage (and per barrier); TAB: operands from tables
-__global__ __launch_bounds__(Cfg::NT) void gemm_mfma_kernel(GemmArgs g, GemmTab t) {
+__global__ __launch_bounds__(Cfg::NT, Cfg::NT == 256 ? 3 : 1) void gemm_mfma_kernel(GemmArgs g, GemmTab t) {
     static_assert(!TAB || DIRECT, "grouped launches use the direct-to-LDS loaders");
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int A_FLOATS = DIRECT ? DirectTile<A_KC, BM>::floats : TileShape<A_KC, BM>::floats;

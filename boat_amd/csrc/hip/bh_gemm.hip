@@ -1268,7 +1268,7 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
 //   256x256 (8 wavefronts, one workgroup per CU)   0.2194 us per k, 19.6 us per round
 //   256x128 / 128x256 (8 wavefronts, one per CU)   0.1126 us per k (half the products at 2.6 % less than the big tile's
 //                                                  rate), 10.7 us per round
-//   128x128 (4 wavefronts, two per CU)             two resident workgroups take turns on the matrix cores: 0.0534 us per k
+//   128x128 (4 wavefronts, two per CU when fitted; three fit since)  two resident workgroups take turns on the matrix cores: 0.0534 us per k
 //                                                  each while they share, 0.0581 for one that has the unit to itself (one
 //                                                  wavefront per SIMD hides less), 10-11 us fixed; workgroups left over
 //                                                  after a full round of 512 are handed to the first units that fall

@@ -1263,17 +1263,18 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
 // A workgroup's time is (its share of k) x (us per k of its tile) + a fixed part (launch of the round, first trip to
 // memory, pipeline fill, the store of its tile); a launch takes as many such rounds as the busiest compute unit gets
 // workgroups; a split contraction pays a fold that streams its partials once.  The constants are measured on MI355X
-// (least-squares fit of these constants to a sweep of every tile at 1..32 cuts over 120 shapes from 256 to 8192 in each
-// dimension, two operand layouts: the three eight-wavefront tiles are predicted to 2-3 %, the 128x128 one to 5-8 %):
-//   256x256 (8 wavefronts, one workgroup per CU)   0.2194 us per k, 19.6 us per round
+// (first a least-squares fit to a sweep of every tile at 1..32 cuts over 120 shapes from 256 to 8192 in each dimension,
+// two operand layouts; then, after the epilogue lost its index arithmetic and the 128x128 tile took a third resident
+// workgroup, straight lines through one-round launches at k = 512 .. 4096):
+//   256x256 (8 wavefronts, one workgroup per CU)   0.2192 us per k, 14.6 us per round
 //   256x128 / 128x256 (8 wavefronts, one per CU)   0.1126 us per k (half the products at 2.6 % less than the big tile's
-//                                                  rate), 10.7 us per round
-//   128x128 (4 wavefronts, two per CU when fitted; three fit since)  two resident workgroups take turns on the matrix cores: 0.0534 us per k
-//                                                  each while they share, 0.0581 for one that has the unit to itself (one
-//                                                  wavefront per SIMD hides less), 10-11 us fixed; workgroups left over
-//                                                  after a full round of 512 are handed to the first units that fall
-//                                                  free, two at a time, so they run at the shared rate on half the chip
-//                                                  (measured so with A stored [k][m]; not with a k-contiguous A)
+//                                                  rate), 9.0 us per round
+//   128x128 (4 wavefronts, up to three per CU)     resident workgroups take turns on the matrix cores: 0.0559 us per k
+//                                                  each while two share a unit, 0.0558 with three, 0.0585 for one that has
+//                                                  the unit to itself (one wavefront per SIMD hides less); fixed part
+//                                                  6.5, 8.0 and 8.8 us.  A launch hands its workgroups round the units
+//                                                  in turn, so what is left after whole rounds of three per unit runs
+//                                                  one, two or three to a unit
 //   fold of a cut contraction                      5 us + (cuts + 1) x output bytes at 6.2 TB/s (the partials mostly
 //                                                  still sit in the last-level cache)
 // Padding is paid automatically (a tile costs the same full or not), and so is the quantisation of rounds: 384 big
@@ -1282,7 +1283,7 @@ struct TilePlan {
     int cfg, splits;
     double us;
 };
-static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, int64_t splits, bool accumulate, int cus, bool spread_rest) {
+static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, int64_t splits, bool accumulate, int cus) {
     static const int bms[5] = {0, 128, 256, 256, 128}, bns[5] = {0, 128, 256, 128, 256};
     const int64_t tiles = ceil_div(m, bms[cfg]) * ceil_div(n, bns[cfg]) * batch;
     const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
@@ -1291,15 +1292,17 @@ static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, i
     const int64_t wgs = tiles * real_splits;
     double us;
     if (cfg == 1) {
-        const double alone = 0.0581, shared = 0.0534, fixed_alone = 10.9, fixed_shared = 10.3;
-        const int64_t full = wgs / (2 * cus), rest = wgs - full * 2 * cus;
-        us = full * (2 * ks * shared + fixed_shared);
-        // (with a k-contiguous A operand the left-over workgroups were measured spread one per unit after all: 8192x1536x1536,
-        // 768 workgroups, 277-281 us against 367 us with A stored [k][m]; and so were those of a grouped launch: three
-        // 1024x1024x8192 weight gradients with A stored [k][m], 768 workgroups at 4 cuts 388 us against 402 at 8)
-        if (rest > 0) us += (rest <= cus && (full == 0 || spread_rest)) ? ks * alone + fixed_alone : 2 * ks * shared + fixed_shared;
+        // us per k and workgroup, and the fixed part of a round, when one, two or three workgroups share a compute unit
+        // (the tile's registers and LDS let three be resident; a launch hands its workgroups round the units in turn)
+        static const double rate[4] = {0.0, 0.0585, 0.0559, 0.0558}, fixed[4] = {0.0, 6.5, 8.0, 8.8};
+        const int64_t full = wgs / (3 * cus), rest = wgs - full * 3 * cus;
+        us = full * (3 * ks * rate[3] + fixed[3]);
+        if (rest > 0) {
+            const int64_t share = ceil_div(rest, cus);
+            us += share * ks * rate[share] + fixed[share];
+        }
     } else {
-        const double per_k = cfg == 2 ? 0.2194 : 0.1126, fixed = cfg == 2 ? 19.6 : 10.7;
+        const double per_k = cfg == 2 ? 0.2192 : 0.1126, fixed = cfg == 2 ? 14.6 : 9.0;
         us = ceil_div(wgs, cus) * (ks * per_k + fixed);
     }
     if (real_splits > 1) {
@@ -1308,7 +1311,7 @@ static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, i
     }
     return us;
 }
-static TilePlan plan_tiles(int64_t m, int64_t n, int64_t k, int64_t batch, bool segmented, bool accumulate, bool a_kc) {
+static TilePlan plan_tiles(int64_t m, int64_t n, int64_t k, int64_t batch, bool segmented, bool accumulate) {
     int cus = bh_device_cu_count();
     if (cus <= 0) cus = 256;
     TilePlan best{1, 1, 1e30};
@@ -1318,21 +1321,21 @@ static TilePlan plan_tiles(int64_t m, int64_t n, int64_t k, int64_t batch, bool 
         if (cfg == 2 && (m < 192 || n < 192)) continue;
         const int64_t max_splits = segmented ? 1 : (k / 128 < 32 ? (k / 128 < 1 ? 1 : k / 128) : 32);
         for (int64_t sp = 1; sp <= max_splits; sp++) {
-            const double us = tile_us(cfg, m, n, k, batch, sp, accumulate, cus, a_kc);
+            const double us = tile_us(cfg, m, n, k, batch, sp, accumulate, cus);
             if (us < best.us * 0.995) best = TilePlan{cfg, (int)sp, us};   // ties go to the earlier (smaller) choice
         }
     }
     return best;
 }
 // the number of cuts the model would choose for a tile shape somebody forced (test hook)
-static int64_t default_splits(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, bool a_kc) {
+static int64_t default_splits(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch) {
     int cus = bh_device_cu_count();
     if (cus <= 0) cus = 256;
     double best = 1e30;
     int64_t best_sp = 1;
     const int64_t max_splits = k / 128 < 32 ? (k / 128 < 1 ? 1 : k / 128) : 32;
     for (int64_t sp = 1; sp <= max_splits; sp++) {
-        const double us = tile_us(cfg, m, n, k, batch, sp, false, cus, a_kc);
+        const double us = tile_us(cfg, m, n, k, batch, sp, false, cus);
         if (us < best * 0.995) {
             best = us;
             best_sp = sp;
@@ -1412,7 +1415,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
-        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0, a_kc || (tab && batch > 1));
+        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0);
         cfg = plan.cfg;
         plan_splits = plan.splits;
         plan_us = plan.us;
@@ -1558,7 +1561,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     g.tiles_n = (int)ceil_div(n, bn);
     float* ws = nullptr;
     {
-        int64_t splits = (g_force_cfg >= 1 && g_force_cfg <= 4 && g_force_cfg != cfg_planned) ? default_splits(cfg, m, n, k, batch, a_kc) : plan_splits;
+        int64_t splits = (g_force_cfg >= 1 && g_force_cfg <= 4 && g_force_cfg != cfg_planned) ? default_splits(cfg, m, n, k, batch) : plan_splits;
         if (g_force_splits > 0 && g_force_splits <= k / kBK) splits = g_force_splits;
         if (segmented) splits = 1;
         if (splits > 1) {

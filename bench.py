@@ -39,15 +39,15 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 METRIC = "backward+Adam step ms; GB/s & TFLOP/s as % of MI355X roofline (1 GPU)"
 
 # HBM bytes per GEMM launch of configuration 2 (average of its dX and dW launches) measured with rocprofv3 --pmc:
-# FETCH_SIZE 409,880 KiB x 2.000 + WRITE_SIZE 98,304 KiB x 1.000, the factors being what the same counters read for
-# a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).  A constant taken from that profile, not a
-# measurement of this run.
-GEMM_TRAFFIC_BYTES_CONFIG2 = int(((2.0 * 779903.4 + 131072.0) + (2.0 * 557368.4 + 65536.0)) / 2 * 1024)
+# 2.000 x FETCH_SIZE (393,392 and 426,101 KiB) + 1.000 x WRITE_SIZE (131,072 and 65,536 KiB), the factors being what the
+# same counters read for a streaming copy of known size (profiles/pmc_hbm_traffic_and_mfma.md).  A constant taken from
+# that profile, not a measurement of this run.
+GEMM_TRAFFIC_BYTES_CONFIG2 = int(((2.0 * 393392.3 + 131072.0) + (2.0 * 426101.2 + 65536.0)) / 2 * 1024)
 # the bytes the same two launches need at least: dX reads dY and W and writes dX (335.5 MB), dW reads X and dY, reads and
 # writes dW (402.7 MB)
 GEMM_ALGORITHMIC_BYTES_CONFIG2 = int((335.5e6 + 402.7e6) / 2)
 # HBM bytes per GEMM launch of the block training step, averaged over the step's 11 launches (same file, same counters)
-GEMM_TRAFFIC_BYTES_STEP = 398_000_000
+GEMM_TRAFFIC_BYTES_STEP = 364_800_000
 # what the step's 11 GEMM launches need at least (each operand read once, each output written once): 1,929 MB
 GEMM_ALGORITHMIC_BYTES_STEP = 1_929_000_000 // 11
 

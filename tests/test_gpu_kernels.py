@@ -1168,3 +1168,35 @@ def test_gemm_random_sweep_with_padded_leading_dimensions(hip):
         assert rel_fro(got[:, :n], want) <= TOL_GEMM, tag
         assert np.array_equal(got[:, n:], c0[:, n:]), tag            # the padding of C is never written
         _KEEP.clear()
+
+
+@pytest.mark.parametrize("force", [-1, 1, 2, 3, 4])
+def test_gemm_tiles_inside_and_on_the_edge_of_odd_outputs(hip, force):
+    """Outputs whose row length is odd or padded, large enough to hold tiles that lie wholly inside them (which store
+    through one pointer per lane and immediate offsets) next to tiles cut by the edge (which keep the bounds-checked
+    code): every layout, with and without bias and accumulation, on every tile shape, against float64 at the bound only
+    fp32 accumulation meets; the padding behind a row of C is never written."""
+    rng = np.random.default_rng(97)
+    hip.bh_gemm_force_config(force)
+    try:
+        for (m, n, k) in ((300, 257, 64), (513, 385, 48), (260, 1001, 32)):
+            for ta, tb in ((0, 0), (0, 1), (1, 0)):
+                for accumulate, bias, pad in ((0, 0, 0), (1, 0, 3), (0, 1, 3), (1, 1, 0)):
+                    a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+                    b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+                    c0 = rng.standard_normal((m, n + pad)).astype(np.float32)
+                    bv = rng.standard_normal(n).astype(np.float32)
+                    dc = dev(hip, c0)
+                    rc = hip.bh_gemm(ta, tb, m, n, k, dev(hip, a).ptr, m if ta else k, dev(hip, b).ptr, k if tb else n, dc.ptr, n + pad,
+                                     dev(hip, bv).ptr if bias else None, accumulate, 1)
+                    hip.check(rc)
+                    A = a.T if ta else a
+                    B = b.T if tb else b
+                    want = A.astype(np.float64) @ B.astype(np.float64) + (bv if bias else 0) + (c0[:, :n] if accumulate else 0)
+                    got = dc.numpy()
+                    tag = (force, m, n, k, ta, tb, accumulate, bias, pad)
+                    assert np.abs(got[:, :n] - want).max() <= 2e-6 * np.abs(want).max(), tag
+                    assert np.array_equal(got[:, n:], c0[:, n:]), tag
+                    _KEEP.clear()
+    finally:
+        hip.bh_gemm_force_config(-1)

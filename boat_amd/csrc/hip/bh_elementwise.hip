@@ -302,6 +302,73 @@ __global__ __launch_bounds__(VEC ? 64 : 256) void act_bwd_colsum_partial_kernel(
         partial[(int64_t)blockIdx.y * cols + c] = (a0 + a1) + (a2 + a3);
     }
 }
+// The same sums from four wavefronts per row chunk, for matrices too small to fill the chip with one wavefront per
+// chunk and column group (the chunks are bh_colsum's, so their number is given): wavefront w keeps running sum w, i.e.
+// rows w, w+4, ... of the chunk's whole trips of four, two of them in flight; the first wavefront also takes the rows
+// after the last whole trip, as the first running sum does above; the four sums meet in LDS and are added in the order
+// above.  4096x1024 GELU: 15 us against 26, the same bits.
+template <typename F>
+__global__ __launch_bounds__(256) void act_bwd_colsum_partial4_kernel(F f, const float* __restrict__ saved, const float* __restrict__ dy,
+                                                                      float* __restrict__ dx, float* __restrict__ partial, int64_t rows,
+                                                                      int64_t cols) {
+    __shared__ f32x4 red[4][64];
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t step = gridDim.y;
+    const int64_t c = ((int64_t)blockIdx.x * 64 + lane) * 4;
+    const bool live = c < cols;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const auto one_row = [&](int64_t r) {
+        const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(saved + r * cols + c));
+        const f32x4 g = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + r * cols + c));
+        f32x4 v;
+        v.x = f(a.x, g.x, 0.f, 0.f);
+        v.y = f(a.y, g.y, 0.f, 0.f);
+        v.z = f(a.z, g.z, 0.f, 0.f);
+        v.w = f(a.w, g.w, 0.f, 0.f);
+        __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dx + r * cols + c));
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    };
+    if (live) {
+        const int64_t in_chunk = (rows - blockIdx.y + step - 1) / step;    // rows blockIdx.y, blockIdx.y + step, ... (gridDim.y <= rows)
+        const int64_t trips = in_chunk / 4;
+        const int64_t first = blockIdx.y + w * step;                       // this wavefront's row of trip 0
+        int64_t t = 0;
+        for (; t + 2 <= trips; t += 2) {
+            const int64_t r0 = first + t * 4 * step, r1 = r0 + 4 * step;
+            const f32x4 a0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(saved + r0 * cols + c));
+            const f32x4 g0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + r0 * cols + c));
+            const f32x4 a1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(saved + r1 * cols + c));
+            const f32x4 g1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(dy + r1 * cols + c));
+            f32x4 v;
+            v.x = f(a0.x, g0.x, 0.f, 0.f);
+            v.y = f(a0.y, g0.y, 0.f, 0.f);
+            v.z = f(a0.z, g0.z, 0.f, 0.f);
+            v.w = f(a0.w, g0.w, 0.f, 0.f);
+            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dx + r0 * cols + c));
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+            v.x = f(a1.x, g1.x, 0.f, 0.f);
+            v.y = f(a1.y, g1.y, 0.f, 0.f);
+            v.z = f(a1.z, g1.z, 0.f, 0.f);
+            v.w = f(a1.w, g1.w, 0.f, 0.f);
+            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dx + r1 * cols + c));
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+        if (t < trips) one_row(first + t * 4 * step);
+        if (w == 0)
+            for (int64_t q = trips * 4; q < in_chunk; q++) one_row(blockIdx.y + q * step);
+    }
+    red[w][lane] = acc;
+    __syncthreads();
+    if (w == 0 && live) {
+        const f32x4 s1 = red[1][lane], s2 = red[2][lane], s3 = red[3][lane];
+        f32x4 t;
+        t.x = (acc.x + s1.x) + (s2.x + s3.x);
+        t.y = (acc.y + s1.y) + (s2.y + s3.y);
+        t.z = (acc.z + s1.z) + (s2.z + s3.z);
+        t.w = (acc.w + s1.w) + (s2.w + s3.w);
+        *reinterpret_cast<f32x4*>(partial + (int64_t)blockIdx.y * cols + c) = t;
+    }
+}
 // few rows: fold_rows_kernel's shape (64 columns x 16 row lanes, folded through LDS in lane order) on values computed here
 template <typename F>
 __global__ __launch_bounds__(kFoldCols * kFoldLanes) void act_bwd_colsum_small_kernel(F f, const float* __restrict__ saved,
@@ -344,6 +411,9 @@ __global__ __launch_bounds__(kFoldCols * kFoldLanes) void act_bwd_colsum_small_k
 // dx = dy * f'(saved) and, in the same pass, the column sums of dx (the bias gradient of the dense layer whose output the
 // activation took): out[c] (+)= sum_r dx[r][c].  The sums are bh_colsum's, in its order: rows <= 256 take the one-launch
 // fold (64 columns x 16 row lanes), larger matrices the same row chunks, four running sums per lane and fold_rows_kernel.
+// up to this many elements the partial kernel runs four wavefronts per row chunk (measured: faster up to 8M elements, level at 16M, slower at 32M)
+constexpr int64_t kActFourWaveMax = (int64_t)1 << 23;
+
 template <typename F>
 static int launch_act_bwd_colsum(const char* name, F f, const float* saved, const float* dy, float* dx, float* out, int64_t rows,
                                  int64_t cols, int accumulate) {
@@ -358,7 +428,11 @@ static int launch_act_bwd_colsum(const char* name, F f, const float* saved, cons
     if (chunks < 1) chunks = 1;
     float* partial = (float*)bh_malloc(sizeof(float) * (size_t)(chunks * cols));
     if (!partial) return BH_ENOMEM;
-    if (cols % 4 == 0 && aligned16(saved) && aligned16(dy) && aligned16(dx))
+    const bool vec = cols % 4 == 0 && aligned16(saved) && aligned16(dy) && aligned16(dx);
+    if (vec && rows * cols <= kActFourWaveMax)
+        hipLaunchKernelGGL((act_bwd_colsum_partial4_kernel<F>), dim3(col_blocks, (unsigned)chunks), dim3(256), 0, stream(), f, saved, dy,
+                           dx, partial, rows, cols);
+    else if (vec)
         hipLaunchKernelGGL((act_bwd_colsum_partial_kernel<F, true>), dim3(col_blocks, (unsigned)chunks), dim3(64), 0, stream(), f, saved, dy,
                            dx, partial, rows, cols);
     else

@@ -274,7 +274,7 @@ def test_activation_backward_with_column_sums(hip, rng, rows, cols):
         assert np.max(np.abs(sum_a.numpy() - want)) <= TOL_RED * max(1.0, np.abs(dx_b.numpy()).sum(0).max())
 
 
-@pytest.mark.parametrize("rows,cols", [(64, 10), (3, 33), (5, 1), (7, 1000)])
+@pytest.mark.parametrize("rows,cols", [(64, 10), (3, 33), (5, 1), (7, 1000), (300, 257), (129, 1025), (40, 2049)])
 def test_softmax_family(hip, oracle, rng, rows, cols):
     x = (3 * rng.standard_normal((rows, cols))).astype(np.float32)
     dy = rng.standard_normal((rows, cols)).astype(np.float32)

@@ -253,10 +253,11 @@ def test_colsum_grouped(hip, rng, rows, cols, groups):
             assert np.max(np.abs(outs[g].numpy() - want)) <= TOL_RED * max(1.0, np.abs(want).max())
 
 
-@pytest.mark.parametrize("rows,cols", [(64, 128), (1, 5), (256, 33), (257, 64), (1000, 37), (300, 4096), (8192, 1024), (1030, 516)])
+@pytest.mark.parametrize("rows,cols", [(64, 128), (1, 5), (256, 33), (257, 64), (1000, 37), (300, 4096), (8192, 1024), (1030, 516), (4100, 2052)])
 def test_activation_backward_with_column_sums(hip, rng, rows, cols):
     """bh_activation_backward_colsum: dx and the column sums of dx in one pass are, bit for bit, bh_activation_backward
-    followed by bh_colsum (few rows, the vector and the scalar form of the partial kernel), with and without accumulation."""
+    followed by bh_colsum (few rows; the scalar form of the partial kernel; its vector forms with four wavefronts per row
+    chunk, up to 8M elements, and with one, beyond), with and without accumulation."""
     saved = (2 * rng.standard_normal((rows, cols))).astype(np.float32)
     dy = rng.standard_normal((rows, cols)).astype(np.float32)
     ds, ddy = dev(hip, saved), dev(hip, dy)

@@ -91,15 +91,26 @@ __global__ __launch_bounds__(kLnBlock) void ln_fwd_kernel(const float* __restric
     // Group g takes rows g, g+G, g+2G, ...: the resident workgroups read neighbouring rows (one moving
     // window).  rows_per_group is the same for every group, so the loop trip count (and every barrier
     // inside row_sum2) is uniform across the block; out-of-range rows are masked.
+    // The next row of the group is fetched before the current one is reduced, so that its trip to memory runs under the
+    // two reductions and the stores instead of in front of them.
+    float4 xn[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int c4 = t + i * TPR;
+        xn[i] = (g_id < rows && c4 < h4 && rows_per_group > 0) ? ld4_stream(x + g_id * hidden, c4) : make_float4(0, 0, 0, 0);
+    }
     for (int64_t it = 0; it < rows_per_group; it++) {
         const int64_t r = it * total_groups + g_id;
         const bool live = r < rows;
         float4 xv[VPT];
         float s = 0.f, dummy = 0.f;
+        const int64_t rn = r + total_groups;
+        const bool live_n = it + 1 < rows_per_group && rn < rows;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
             const int c4 = t + i * TPR;
-            xv[i] = (live && c4 < h4) ? ld4_stream(x + r * hidden, c4) : make_float4(0, 0, 0, 0);
+            xv[i] = xn[i];
+            xn[i] = (live_n && c4 < h4) ? ld4_stream(x + rn * hidden, c4) : make_float4(0, 0, 0, 0);
             s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
         }
         float mu = 0.f;

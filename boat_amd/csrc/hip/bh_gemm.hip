@@ -163,13 +163,14 @@ struct Frags {
 //   k-contiguous operand   block = 16 rows x 16 k.  Row stride is 16 floats with no room for padding, so the four
 //                          16-byte chunks of a row are swizzled instead: chunk q of row r sits in slot q ^ ((r >> 2) & 3),
 //                          which makes the fragment reads of 16 consecutive rows hit 16 different bank groups.
-//   row-contiguous operand block = 256 consecutive floats of k-rows (one k-row for R = 256, two for R = 128), blocks
+//   row-contiguous operand block = 256 consecutive floats of k-rows (one k-row for R = 256, two for R = 128, four for R = 64), blocks
 //                          padded by 4 floats so that the two half-wavefronts of a fragment read use different banks.
 // Rows or columns past the matrix edge are clamped to the last valid ones (their products are never stored); the
 // contraction range must be a multiple of kBK because nothing zero-fills a k tail.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 template <bool KC, int R> struct DirectTile {
+    static_assert(R == 64 || R == 128 || R == 256, "operand tiles of 64, 128 or 256 rows");
     static constexpr int blocks = R / 16;
     static constexpr int block_stride = KC ? 256 : 260;   // floats
     static constexpr int floats = blocks * block_stride;
@@ -208,8 +209,8 @@ struct DirectLoader {
                 const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
                 off[j] = (unsigned)(((row - row0) * ld + 4 * chunk) * (int64_t)sizeof(float));
             } else {
-                const int krow = R == 256 ? blk : 2 * blk + (lane >> 5);
-                int64_t col = row0 + 4 * (R == 256 ? lane : (lane & 31));
+                const int krow = R == 256 ? blk : R == 128 ? 2 * blk + (lane >> 5) : 4 * blk + (lane >> 4);
+                int64_t col = row0 + 4 * (R == 256 ? lane : R == 128 ? (lane & 31) : (lane & 15));
                 if (col > row_lim - 4) col = row_lim - 4;
                 off[j] = (unsigned)((krow * ld + col) * (int64_t)sizeof(float));
             }
@@ -244,7 +245,7 @@ struct DirectFrags {
             for (int s = 0; s < 4; s++) {
                 const int kk = kb + 4 * half + s;
                 FragT<T> f;
-                f.load(lds + (R == 256 ? kk * 260 : (kk >> 1) * 260 + (kk & 1) * 128) + wave_off + T * r);
+                f.load(lds + (R == 256 ? kk * 260 : R == 128 ? (kk >> 1) * 260 + (kk & 1) * 128 : (kk >> 2) * 260 + (kk & 3) * 64) + wave_off + T * r);
 #pragma unroll
                 for (int t = 0; t < T; t++) v[s][t] = f.v[t];
             }
@@ -1151,6 +1152,7 @@ using CfgBig = GemmCfg<256, 256, 2, 4>;   // 8 waves, 128x64 per wave
 using CfgMid = GemmCfg<128, 128, 2, 2>;   // 4 waves, 64x64 per wave
 using CfgTall = GemmCfg<256, 128, 4, 2>;  // 8 waves, 64x64 per wave
 using CfgWide = GemmCfg<128, 256, 2, 4>;  // 8 waves, 64x64 per wave
+using CfgSmall = GemmCfg<64, 64, 2, 2>;   // 4 waves, 32x32 per wave
 
 // out[a][d1][b][d0][c] = in[a][d0][b][d1][c]: two dimensions of a dense tensor swapped, anything between and after
 // them carried along (the general case of boat_transpose, linear.c:238-406).  One output element per lane and trip;
@@ -1275,6 +1277,13 @@ static int launch_fold(const float* ws, float* c, const float* bias, int64_t m, 
 //                                                  6.5, 8.0 and 8.8 us.  A launch hands its workgroups round the units
 //                                                  in turn, so what is left after whole rounds of three per unit runs
 //                                                  one, two or three to a unit
+//   64x64 (4 wavefronts, eight resident per CU)    4.0 us (11 beyond eight per unit) + k x (0.01432 us x workgroups per
+//                                                  unit + 0.00336 us): 91-93 % of the matrix rate from two per unit on
+//                                                  (one alone: 0.0185 us per k up to k = 1024, 0.0226 beyond), measured
+//                                                  at 1 .. 16 per unit and k = 128 .. 4096; it reads its operands twice as
+//                                                  often as the 128x128 tile and is offered up to sixteen per unit
+//                                                  (1024^3: 20 us against 27; 3072x3072x1024, nine per unit where the
+//                                                  128x128 tile has two and a quarter: 152 against 180)
 //   fold of a cut contraction                      5 us + (cuts + 1) x output bytes at 6.2 TB/s (the partials mostly
 //                                                  still sit in the last-level cache)
 // Padding is paid automatically (a tile costs the same full or not), and so is the quantisation of rounds: 384 big
@@ -1284,9 +1293,9 @@ struct TilePlan {
     double us;
 };
 static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, int64_t splits, bool accumulate, int cus) {
-    static const int bms[5] = {0, 128, 256, 256, 128}, bns[5] = {0, 128, 256, 128, 256};
+    static const int bms[8] = {0, 128, 256, 256, 128, 0, 0, 64}, bns[8] = {0, 128, 256, 128, 256, 0, 0, 64};
     const int64_t tiles = ceil_div(m, bms[cfg]) * ceil_div(n, bns[cfg]) * batch;
-    const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
+    const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1 && cfg != 7) ? 2 * kBK : kBK;
     const int64_t ks = splits > 1 ? ceil_div(ceil_div(k, splits), unit) * unit : k;
     const int64_t real_splits = splits > 1 ? ceil_div(k, ks) : 1;
     const int64_t wgs = tiles * real_splits;
@@ -1301,6 +1310,11 @@ static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, i
             const int64_t share = ceil_div(rest, cus);
             us += share * ks * rate[share] + fixed[share];
         }
+    } else if (cfg == 7) {
+        // the workgroups of a compute unit (the hardware keeps eight resident and refills as they end) take turns
+        const int64_t share = ceil_div(wgs, cus);
+        us = (share <= 8 ? 4.0 : 11.0) + ks * (share == 1 ? (ks <= 1024 ? 0.0185 : 0.0226) : share * 0.01432 + 0.00336);
+        if (share > 8) us *= 1.05;      // past one set of resident workgroups the figure has been up to 10 % low: the larger tiles get the benefit of the doubt
     } else {
         const double per_k = cfg == 2 ? 0.2192 : 0.1126, fixed = cfg == 2 ? 14.6 : 9.0;
         us = ceil_div(wgs, cus) * (ks * per_k + fixed);
@@ -1311,11 +1325,13 @@ static double tile_us(int cfg, int64_t m, int64_t n, int64_t k, int64_t batch, i
     }
     return us;
 }
-static TilePlan plan_tiles(int64_t m, int64_t n, int64_t k, int64_t batch, bool segmented, bool accumulate) {
+static TilePlan plan_tiles(int64_t m, int64_t n, int64_t k, int64_t batch, bool segmented, bool accumulate, bool tables) {
     int cus = bh_device_cu_count();
     if (cus <= 0) cus = 256;
     TilePlan best{1, 1, 1e30};
-    for (int cfg = 1; cfg <= 4; cfg++) {
+    for (int cfg = 1; cfg <= 7; cfg++) {
+        if (cfg == 5 || cfg == 6) continue;     // not tiles of this kernel
+        if (cfg == 7 && (tables || ceil_div(m, 64) * ceil_div(n, 64) * batch > 16 * (int64_t)cus)) continue;
         if (cfg == 3 && m < 192) continue;      // a 256-row tile over fewer rows than that is mostly padding ...
         if (cfg == 4 && n < 192) continue;      // ... and the model's fixed part does not shrink with it
         if (cfg == 2 && (m < 192 || n < 192)) continue;
@@ -1408,48 +1424,70 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
     // float4 global loads need: 16 B aligned bases, leading dimensions and the contiguous extent % 4
     bool vec_ok = al16(a) && al16(b) && (lda % 4 == 0) && (ldb % 4 == 0) && k > 0;
     vec_ok = vec_ok && ((a_kc ? k : m) % 4 == 0) && ((b_kc ? k : n) % 4 == 0);
-    int cfg;   // 0 fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256
+    int cfg;   // 0 fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256, 7 = 64x64
     int plan_splits = 1;   // k-splits that come with the tile choice
     double plan_us = 1e30; // what the cost model expects of that choice
     const bool segmented = tab && tab->k_segments > 1;     // one product over several operand pairs: never split
     if (!vec_ok || m * n < 64 * 64) {
         cfg = 0;
     } else {
-        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0);
+        const TilePlan plan = plan_tiles(m, n, k, batch, segmented, accumulate != 0, tab != nullptr);
         cfg = plan.cfg;
         plan_splits = plan.splits;
         plan_us = plan.us;
     }
-    // up to about 2^25 multiply-adds the problem is latency bound: one load phase per workgroup
-    if (m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1)) cfg = 5;
-    // so is a contraction of at most 64 under an output of a few million elements, where the tiles above spend their
+    // Up to about 2^25 multiply-adds the problem is latency bound.  The 64x64 tile, cut as the cost model says, is the
+    // fastest kernel there wherever its 16-byte loads apply (256x256x512: 8.4 us against 12.6 for the kernel that stages
+    // a whole k-chunk per workgroup, which keeps the shapes the tile cannot load)
+    const bool small_problem = m * n <= ((int64_t)1 << 25) / (k > 0 ? k : 1);
+    if (small_problem) cfg = 5;
+    // so is a contraction of at most 64 under an output of a few million elements, where the larger tiles spend their
     // time filling and draining their pipeline (288x12544x64: 15.7 against 20.0 us; 4096x4096x64 is past it: 56 against 37)
     if (k > 0 && k <= 64 && m * n <= ((int64_t)1 << 22)) cfg = 5;
+    const bool small_tile_ok = vec_ok && m * n >= 64 * 64 && !tab;
+    const auto take_small_tile = [&]() {
+        int cus = bh_device_cu_count();
+        if (cus <= 0) cus = 256;
+        cfg = 7;
+        plan_splits = (int)default_splits(7, m, n, k, batch);
+        plan_us = tile_us(7, m, n, k, batch, plan_splits, accumulate != 0, cus);
+    };
+    if (cfg == 5 && small_tile_ok && small_problem) take_small_tile();
     // A few million multiply-adds in at most a few hundred 32x32 tiles: the kernels without workgroup-wide staging.
     // Measured against the staged small-problem kernel plus its fold (11-14 us beyond k = 128): two row-fast operands
     // 6-10 us up to k = 1024; one k-fast operand 7.5-8 us up to k = 512 (one trip) and 12 us up to 1024 (two trips);
     // two k-fast operands 9-11 us up to k = 512 and slower beyond.
     const int64_t tiles32 = ceil_div(m, 32) * ceil_div(n, 32) * batch;
+    // (with a k-fast operand the 64x64 tile is as fast or faster wherever it applies -- 64x128x1024: 8.3 against 12.5 us --
+    // so the kernel keeps the shapes with two row-fast operands, where it wins -- 512x512x512: 6.9 against 9.4 -- up to
+    // the long contractions under small outputs that the tile cuts -- 64x128x1024: 8.0 against 10.5 --, and those
+    // the tile cannot load)
     if (k > 0 && m * n * k <= ((int64_t)1 << (k <= 128 ? 25 : 24)) && tiles32 <= 512 &&
-        (k <= 512 || (k <= 1024 && !(a_kc && b_kc)) || (!a_kc && !b_kc)))
-        cfg = 6;
+        (k <= 512 || (k <= 1024 && !(a_kc && b_kc)) || (!a_kc && !b_kc))) {
+        if (small_tile_ok && (a_kc || b_kc || (k >= 1024 && m * n <= ((int64_t)1 << 17)))) take_small_tile();
+        else cfg = 6;
+    }
+    // (two row-fast operands over a contraction of 257 .. 512: the tiny kernel's one trip per wavefront beats the tile
+    // up to 256 tiles of 32x32 -- 512x512x512: 6.8 against 9.4 us, 784x128x512: 6.7 against 8.8)
+    if (!a_kc && !b_kc && k > 256 && k <= 512 && tiles32 <= 256) cfg = 6;
     // A small output with a very long contraction over k-fast operands (the weight gradient of a convolution: 64 x 288
     // outputs, k = 12544): chunks of 512 k per workgroup of the same kernel, partials folded afterwards.
     // Its 32x32 tiles read every operand value once per tile row or column, k*m*n/4 bytes in all, at 3.2 TB/s when both
     // operands are k-fast and 4.3 TB/s with one (measured from 64x288 to 256x256 outputs, k 2048 to 32768); the 128x128
     // tiles with a cut contraction read a quarter of that and win from about 128x256x12544 on, which the cost model's figure
-    // for them shows (256x256x8192: 43 us here against 31 us there).
+    // for them shows (256x256x8192: 43 us here against 31 us there).  Where the 64x64 tile was taken it stays: it cuts
+    // such a contraction itself (64x128x2048: 8.7 against 14.1 us).
     bool tiny_split = false;
-    if (k >= 2048 && tiles32 <= 64 && (a_kc || b_kc) && ceil_div(k, 512) <= 65535 &&
+    if (cfg != 7 && k >= 2048 && tiles32 <= 64 && (a_kc || b_kc) && ceil_div(k, 512) <= 65535 &&
         8.0 + 0.25 * (double)k * (double)m * (double)n * (double)batch / ((a_kc && b_kc) ? 3.2e6 : 4.3e6) <= plan_us) {
         cfg = 6;
         tiny_split = true;
     }
     const int cfg_planned = cfg;
-    if (g_force_cfg >= 0 && g_force_cfg <= 6 && (vec_ok || g_force_cfg == 0 || g_force_cfg >= 5)) cfg = g_force_cfg;
+    if (g_force_cfg >= 0 && g_force_cfg <= 7 && (vec_ok || g_force_cfg == 0 || g_force_cfg == 5 || g_force_cfg == 6)) cfg = g_force_cfg;
     if (cfg == 6 && k == 0) cfg = 5;
     if (cfg != 6) tiny_split = false;
-    if (tab && (cfg == 0 || cfg >= 5)) return kTabUnsupported;
+    if (tab && (cfg == 0 || cfg >= 5)) return kTabUnsupported;     // (the 64x64 tile, 7, has no table form either)
 
     if (cfg == 6) {
         g.tiles_m = (int)ceil_div(m, 32);
@@ -1556,17 +1594,17 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
         return BH_LAUNCH_CHECK("gemm_fallback_kernel");
     }
 
-    const int bm = (cfg == 2 || cfg == 3) ? 256 : 128, bn = (cfg == 2 || cfg == 4) ? 256 : 128;
+    const int bm = cfg == 7 ? 64 : (cfg == 2 || cfg == 3) ? 256 : 128, bn = cfg == 7 ? 64 : (cfg == 2 || cfg == 4) ? 256 : 128;
     g.tiles_m = (int)ceil_div(m, bm);
     g.tiles_n = (int)ceil_div(n, bn);
     float* ws = nullptr;
     {
-        int64_t splits = (g_force_cfg >= 1 && g_force_cfg <= 4 && g_force_cfg != cfg_planned) ? default_splits(cfg, m, n, k, batch) : plan_splits;
+        int64_t splits = (((g_force_cfg >= 1 && g_force_cfg <= 4) || g_force_cfg == 7) && g_force_cfg != cfg_planned) ? default_splits(cfg, m, n, k, batch) : plan_splits;
         if (g_force_splits > 0 && g_force_splits <= k / kBK) splits = g_force_splits;
         if (segmented) splits = 1;
         if (splits > 1) {
             // whole pairs of k-tiles per workgroup where the contraction allows it (the paired main loop needs them)
-            const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1) ? 2 * kBK : kBK;
+            const int64_t unit = (k % (2 * kBK) == 0 && cfg != 1 && cfg != 7) ? 2 * kBK : kBK;
             g.k_per_split = ceil_div(ceil_div(k, splits), unit) * unit;
             g.k_splits = (int)ceil_div(k, g.k_per_split);
         }
@@ -1614,6 +1652,7 @@ static int gemm_core(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, 
         case 2: rc = pairs ? launch_mfma_pairs<CfgBig>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgBig>(run, batch, a_kc, b_kc, direct); break;
         case 3: rc = pairs ? launch_mfma_pairs<CfgTall>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgTall>(run, batch, a_kc, b_kc, direct); break;
         case 4: rc = pairs ? launch_mfma_pairs<CfgWide>(run, batch, a_kc, b_kc) : launch_mfma_layout<CfgWide>(run, batch, a_kc, b_kc, direct); break;
+        case 7: rc = launch_mfma_layout<CfgSmall>(run, batch, a_kc, b_kc, direct); break;
         default: rc = launch_mfma_layout<CfgMid>(run, batch, a_kc, b_kc, direct); break;
     }
     if (rc == BH_OK && g.k_splits > 1) rc = launch_fold(ws, c, bias, m, n, ldc, g.k_splits, batch, g.stride_c, accumulate);

@@ -317,7 +317,8 @@ int bh_zero_multi(float* const* p, const int64_t* n, int count);
 /* ---- test hooks (no arithmetic of their own) ----
  * bh_gemm_force_config: 0 = bounds-checked fallback, 1 = 128x128, 2 = 256x256, 3 = 256x128, 4 = 128x256 MFMA tile,
  * 5 = small-problem kernel (whole k-chunk in LDS, one trip to memory), 6 = tiny-problem kernel (operands straight
- * into the MFMA registers, contraction split among a workgroup's wavefronts), -1 = heuristic (default).
+ * into the MFMA registers, contraction split among a workgroup's wavefronts), 7 = 64x64 MFMA tile (mid-sized and
+ * small problems), -1 = heuristic (default).
  * bh_gemm_force_direct: 0 = MFMA tiles stage their operands through registers; 1 or -1 (default) = operands go
  * straight to LDS (global_load_lds) whenever the contraction length is a multiple of 16, and the eight-wavefront
  * tiles keep two k-tiles per LDS stage (one barrier per 32 k) when every workgroup's share of it is a multiple of 32;

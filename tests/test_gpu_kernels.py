@@ -482,7 +482,7 @@ def test_gemm_heuristic_path(hip, rng, ta, tb, m, n, k):
     gemm_case(hip, rng, ta, tb, m, n, k)
 
 
-@pytest.mark.parametrize("force", [1, 2, 3, 4])
+@pytest.mark.parametrize("force", [1, 2, 3, 4, 7])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 16), (256, 512, 64), (128, 128, 8), (260, 132, 36), (512, 768, 100), (1024, 1024, 256)])
 def test_gemm_mfma_tiles(hip, rng, force, ta, tb, m, n, k):
@@ -491,7 +491,7 @@ def test_gemm_mfma_tiles(hip, rng, force, ta, tb, m, n, k):
     gemm_case(hip, rng, ta, tb, m, n, k, force=force, direct=1)
 
 
-@pytest.mark.parametrize("force", [1, 2, 3, 4])
+@pytest.mark.parametrize("force", [1, 2, 3, 4, 7])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_direct_to_lds_edges_epilogues_and_split_k(hip, rng, force, ta, tb):
     gemm_case(hip, rng, ta, tb, 260, 132, 48, force=force, direct=1, accumulate=True, bias=True)   # ragged edge tiles
@@ -1127,7 +1127,7 @@ def test_gemm_with_very_wide_leading_dimensions(hip):
         B = b[:, :cb].T if tb else b[:, :cb]
         want = A.astype(np.float64) @ B.astype(np.float64)
         dc = hip.zeros((m, n))
-        for cfg in (-1, 1, 4):                             # the heuristic, and the MFMA tiles pinned
+        for cfg in (-1, 1, 4, 7):                          # the heuristic, and the MFMA tiles pinned
             hip.bh_gemm_force_config(cfg)
             try:
                 hip.check(hip.bh_gemm(ta, tb, m, n, k, dev(hip, a).ptr, lda, dev(hip, b).ptr, ldb, dc.ptr, n, None, 0, 1))
@@ -1171,7 +1171,7 @@ def test_gemm_random_sweep_with_padded_leading_dimensions(hip):
         _KEEP.clear()
 
 
-@pytest.mark.parametrize("force", [-1, 1, 2, 3, 4])
+@pytest.mark.parametrize("force", [-1, 1, 2, 3, 4, 7])
 def test_gemm_tiles_inside_and_on_the_edge_of_odd_outputs(hip, force):
     """Outputs whose row length is odd or padded, large enough to hold tiles that lie wholly inside them (which store
     through one pointer per lane and immediate offsets) next to tiles cut by the edge (which keep the bounds-checked

@@ -352,9 +352,10 @@ def bench_gemm_choice(hip):
             chosen = timed(run)
             best, best_cfg = 1e9, None
             try:
-                for cfg in (1, 2, 3, 4):
+                for cfg in (1, 2, 3, 4, 7):                 # 128x128, 256x256, 256x128, 128x256 and 64x64 tiles
                     hip.bh_gemm_force_config(cfg)
-                    tiles = -(-m // (256 if cfg in (2, 3) else 128)) * -(-n // (256 if cfg in (2, 4) else 128))
+                    bm, bn = {1: (128, 128), 2: (256, 256), 3: (256, 128), 4: (128, 256), 7: (64, 64)}[cfg]
+                    tiles = -(-m // bm) * -(-n // bn)
                     for sp in (1, 2, 4, 8, 16):
                         if sp > 1 and (tiles * sp > 2048 or k // sp < 128):
                             continue
